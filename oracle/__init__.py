@@ -1,0 +1,191 @@
+"""CPU oracle for the fused-loss path -- TEST INFRASTRUCTURE ONLY.
+
+ctypes front end over ``liboracle.so`` (built from ``plo_oracle.c`` by
+``oracle/build.py``).  Nothing in the shipped package may import this module;
+it is the checker used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py``.
+
+All functions take and return numpy arrays.  The arithmetic type follows the
+dtype of ``logits`` (float32 -> the ``_f32`` restatement, float64 -> ``_f64``).
+Shapes follow the reference: logits ``(N, C, *)``, integer labels ``(N, *)``
+(csrc/lsr_kernel.cu:199-202 flattens to n_size, dimsize, m_size the same way).
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import build as _build
+
+_LIB = None
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = _build.LIB
+        if not os.path.exists(path):
+            path = _build.build()
+        _LIB = ctypes.CDLL(path)
+        assert _LIB.oracle_abi_version() == 1
+    return _LIB
+
+
+def _suffix(a):
+    if a.dtype == np.float32:
+        return "_f32", ctypes.c_float
+    if a.dtype == np.float64:
+        return "_f64", ctypes.c_double
+    raise TypeError("oracle works on float32 or float64 logits, got %s" % a.dtype)
+
+
+def _ptr(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else ctypes.c_void_p(0)
+
+
+def _dims(logits):
+    n_size = int(logits.shape[0])
+    dimsize = int(logits.shape[1])
+    m_size = int(logits.size // max(1, n_size * dimsize)) if logits.size else 0
+    return n_size, dimsize, m_size
+
+
+def _prep(logits, labels):
+    logits = np.ascontiguousarray(logits)
+    labels = np.ascontiguousarray(labels, dtype=np.int64)
+    assert labels.shape == logits.shape[:1] + logits.shape[2:], (labels.shape, logits.shape)
+    return logits, labels
+
+
+def _call(name, *args):
+    fn = getattr(lib(), name)
+    fn.restype = ctypes.c_int
+    return fn(*args)
+
+
+i64 = ctypes.c_int64
+f64 = ctypes.c_double
+
+
+def lsr_forward(logits, labels, ignore_index=-100, smooth=0.1):
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    out = np.zeros(labels.shape, dtype=logits.dtype)
+    if logits.size:
+        _call("oracle_lsr_forward" + sfx, _ptr(logits), _ptr(labels), _ptr(out),
+              i64(n), i64(c), i64(m), i64(ignore_index), f64(smooth))
+    return out
+
+
+def lsr_backward(logits, labels, ignore_index=-100, smooth=0.1, grad_out=None):
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    if grad_out is not None:
+        grad_out = np.ascontiguousarray(np.broadcast_to(grad_out, labels.shape), dtype=logits.dtype)
+    out = np.zeros_like(logits)
+    if logits.size:
+        _call("oracle_lsr_backward" + sfx, _ptr(logits), _ptr(labels), _ptr(grad_out), _ptr(out),
+              i64(n), i64(c), i64(m), i64(ignore_index), f64(smooth))
+    return out
+
+
+def focal_forward(logits, labels, alpha=0.25, gamma=2.0):
+    logits = np.ascontiguousarray(logits)
+    labels = np.ascontiguousarray(labels, dtype=logits.dtype)
+    assert labels.shape == logits.shape
+    sfx, _ = _suffix(logits)
+    out = np.zeros_like(logits)
+    if logits.size:
+        _call("oracle_focal_forward" + sfx, _ptr(logits), _ptr(labels), _ptr(out),
+              i64(logits.size), f64(alpha), f64(gamma))
+    return out
+
+
+def focal_backward(logits, labels, alpha=0.25, gamma=2.0, grad_out=None):
+    logits = np.ascontiguousarray(logits)
+    labels = np.ascontiguousarray(labels, dtype=logits.dtype)
+    sfx, _ = _suffix(logits)
+    if grad_out is not None:
+        grad_out = np.ascontiguousarray(np.broadcast_to(grad_out, logits.shape), dtype=logits.dtype)
+    out = np.zeros_like(logits)
+    if logits.size:
+        _call("oracle_focal_backward" + sfx, _ptr(logits), _ptr(labels), _ptr(grad_out), _ptr(out),
+              i64(logits.size), f64(alpha), f64(gamma))
+    return out
+
+
+def lmargin_forward(logits, labels, lam=0.3, ignore_index=255):
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    out = np.zeros(labels.shape, dtype=logits.dtype)
+    if logits.size:
+        _call("oracle_lmargin_forward" + sfx, _ptr(logits), _ptr(labels), _ptr(out),
+              i64(n), i64(c), i64(m), i64(ignore_index), f64(lam))
+    return out
+
+
+def lmargin_backward(logits, labels, lam=0.3, ignore_index=255, grad_out=None):
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    if grad_out is not None:
+        grad_out = np.ascontiguousarray(np.broadcast_to(grad_out, labels.shape), dtype=logits.dtype)
+    out = np.zeros_like(logits)
+    if logits.size:
+        _call("oracle_lmargin_backward" + sfx, _ptr(logits), _ptr(labels), _ptr(grad_out), _ptr(out),
+              i64(n), i64(c), i64(m), i64(ignore_index), f64(lam))
+    return out
+
+
+def lovasz_forward(logits, labels, ignore_index=-100):
+    """-> (losses[C], jacc[C, P]); jacc holds the Jaccard differences in pixel order."""
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    assert c < 512
+    losses = np.zeros((c,), dtype=logits.dtype)
+    jacc = np.zeros((c, n * m), dtype=logits.dtype)
+    if logits.size:
+        rc = _call("oracle_lovasz_forward" + sfx, _ptr(logits), _ptr(labels), _ptr(losses), _ptr(jacc),
+                   i64(n), i64(c), i64(m), i64(ignore_index))
+        if rc != 0:
+            raise MemoryError("oracle_lovasz_forward ran out of memory")
+    return losses, jacc
+
+
+def lovasz_backward(grad_out, logits, labels, jacc, ignore_index=-100):
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    grad_out = np.ascontiguousarray(np.broadcast_to(grad_out, (c,)), dtype=logits.dtype)
+    jacc = np.ascontiguousarray(jacc, dtype=logits.dtype)
+    out = np.zeros_like(logits)
+    if logits.size:
+        _call("oracle_lovasz_backward" + sfx, _ptr(grad_out), _ptr(logits), _ptr(labels), _ptr(jacc),
+              _ptr(out), i64(n), i64(c), i64(m), i64(ignore_index))
+    return out
+
+
+# ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
+# large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
+
+def reduce_pixels(losses, labels, reduction, ignore_index):
+    """'mean' divides by the count of non-ignored pixels; anything but 'mean'/'sum' is a pass-through."""
+    if reduction == "sum":
+        return losses.sum(dtype=losses.dtype)
+    if reduction == "mean":
+        n_valid = (np.asarray(labels) != ignore_index).sum()
+        with np.errstate(invalid="ignore", divide="ignore"):
+            return losses.sum(dtype=losses.dtype) / losses.dtype.type(n_valid)
+    return losses
+
+
+def reduce_all(losses, reduction):
+    if reduction == "sum":
+        return losses.sum(dtype=losses.dtype)
+    if reduction == "mean":
+        return losses.mean(dtype=losses.dtype)
+    return losses
