@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-loss hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz]
+                    [--no-cpu-baseline] [--no-others]
+
+A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
+already resident in HBM:  loss = criterion(logits, labels); loss.backward().
+The headline workload is LabelSmoothSoftmaxCEV3 on fp32 logits (8, 19, 1024, 1024).
+Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step (GB/s);
+`roofline` prices the dominant kernel (the backward) against the 8 TB/s HBM peak with
+HIP events on the launch stream; `cpu_baseline` times the pure-torch restatement of the
+reference's CPU path on a bounded sample on the host cores.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "pytorch-loss_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (module factory name, logits shape, description)
+    "lsr": dict(shape=(8, 19, 1024, 1024), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8,19,1024,1024), "
+                "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
+    "lmargin": dict(shape=(8, 19, 1024, 1024), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (8,19,1024,1024), "
+                    "int64 labels 5% ignore=255, lam=0.3, mean"),
+    "focal": dict(shape=(16, 80, 128, 128), desc="FocalLossV3 fwd+bwd, fp32 logits/labels (16,80,128,128), "
+                  "Bernoulli(0.02) labels, alpha=0.25 gamma=2, mean"),
+    "lovasz": dict(shape=(4, 19, 512, 1024), desc="LovaszSoftmaxV3 fwd+bwd, fp32 logits (4,19,512,1024), "
+                   "Zipf(1.1) int64 labels 5% ignore=255, mean"),
+}
+
+
+def numel(shape):
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def algorithmic_bytes(name, shape):
+    """Bytes a fwd+bwd pass has to move at the autograd-Function level (fp32 logits, int64 labels):
+    forward reads the inputs and writes the unreduced losses, backward reads the inputs and the
+    upstream gradient and writes the logits gradient."""
+    E = numel(shape)
+    P = E // shape[1]
+    if name in ("lsr", "lmargin"):
+        fwd = 4 * E + 8 * P + 4 * P
+        bwd = 4 * E + 8 * P + 4 * P + 4 * E
+    elif name == "focal":
+        fwd = 3 * 4 * E
+        bwd = 4 * 4 * E
+    else:  # lovasz: compulsory I/O only (logits, labels, saved Jaccard differences, gradient)
+        fwd = 4 * E + 8 * P + 4 * E
+        bwd = 4 * E + 4 * E + 8 * P + 4 * E
+    return fwd, bwd
+
+
+def make_inputs(name, shape, device, seed=15):
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    if name == "focal":
+        logits = torch.randn(shape, device=device, generator=g) * 1.5 - 2.0
+        labels = (torch.rand(shape, device=device, generator=g) < 0.02).float()
+        return logits, labels
+    logits = torch.randn(shape, device=device, generator=g) * 2.0
+    lshape = shape[:1] + shape[2:]
+    if name == "lovasz":
+        p = (torch.arange(19, device=device, dtype=torch.float64) + 1.0) ** -1.1
+        cdf = torch.cumsum(p / p.sum(), 0)
+        u = torch.rand(lshape, device=device, generator=g, dtype=torch.float64)
+        labels = torch.searchsorted(cdf, u).clamp_(max=18)
+    else:
+        labels = torch.randint(0, shape[1], lshape, device=device, generator=g)
+    ignore = torch.rand(lshape, device=device, generator=g) < 0.05
+    labels[ignore] = 255
+    return logits, labels
+
+
+def make_criterion(name):
+    import pytorch_loss as pl
+    if name == "lsr":
+        return pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="mean", ignore_index=255)
+    if name == "lmargin":
+        return pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255)
+    if name == "focal":
+        return pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean")
+    return pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255)
+
+
+def time_steps(crit, logits, labels, steps, warmup):
+    import torch
+    logits.requires_grad_(True)
+
+    def step():
+        logits.grad = None
+        loss = crit(logits, labels)
+        loss.backward()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, float(loss.item())
+
+
+def time_kernel(launch, iters=30, warmup=5):
+    """Average duration (ms) of one launch: HIP events on the stream the kernel runs on."""
+    import torch
+    for _ in range(warmup):
+        launch()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        launch()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def kernel_rooflines(name, logits, labels):
+    """Per-kernel roofline entries for the forward and backward entry points, called directly
+    through the C ABI wrappers with pre-allocated outputs (no allocator, no autograd in the loop)."""
+    import torch
+    from pytorch_loss import _native
+    lib = _native.load()
+    shape = tuple(logits.shape)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(name, shape)
+    x = logits.detach()
+    n, c = shape[0], shape[1]
+    m = numel(shape) // (n * c)
+    st = _native._stream
+    P = _native._ptr
+    out = {}
+    if name in ("lsr", "lmargin"):
+        losses = torch.empty(labels.shape, dtype=torch.float32, device=x.device)
+        grad = torch.empty_like(x)
+        gout = torch.full(labels.shape, 1.0 / labels.numel(), dtype=torch.float32, device=x.device)
+        if name == "lsr":
+            f = lambda: lib.plh_lsr_forward(P(x), P(labels), P(losses), n, c, m, 255, 0.1, st())
+            b = lambda: lib.plh_lsr_backward(P(x), P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.1, st())
+        else:
+            f = lambda: lib.plh_lmargin_forward(P(x), P(labels), P(losses), n, c, m, 255, 0.3, st())
+            b = lambda: lib.plh_lmargin_backward(P(x), P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.3, st())
+    elif name == "focal":
+        losses = torch.empty_like(x)
+        grad = torch.empty_like(x)
+        gout = torch.full(shape, 1.0 / x.numel(), dtype=torch.float32, device=x.device)
+        f = lambda: lib.plh_focal_forward(P(x), P(labels), P(losses), x.numel(), 2.0, 0.25, st())
+        b = lambda: lib.plh_focal_backward(P(x), P(labels), P(gout), 1, P(grad), x.numel(), 2.0, 0.25, st())
+    else:
+        losses = torch.empty(c, dtype=torch.float32, device=x.device)
+        jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
+        grad = torch.empty_like(x)
+        gout = torch.full((c,), 1.0 / c, dtype=torch.float32, device=x.device)
+        ws_bytes = int(lib.plh_lovasz_workspace_bytes(n, c, m))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        f = lambda: lib.plh_lovasz_forward(P(x), P(labels), P(losses), P(jacc), P(ws), ws_bytes, n, c, m, 255, st())
+        b = lambda: lib.plh_lovasz_backward(P(gout), P(x), P(labels), P(jacc), P(grad), n, c, m, 255, st())
+    assert f() == 0 and b() == 0
+    for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
+        ms = time_kernel(fn)
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        out[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "ms": round(ms, 4), "algorithmic_bytes": nbytes}
+    return out
+
+
+def copy_ceiling(device, nbytes=1 << 30):
+    import torch
+    from pytorch_loss import _native
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    ms = time_kernel(lambda: _native.stream_copy(src, dst))
+    return round(2 * nbytes / (ms * 1e-3) / 1e9, 1)
+
+
+def cpu_baseline(name, shape):
+    """Pure-torch restatement of the reference's V2 (V1 for Lovasz) path on the host cores, on a
+    bounded sample: one image of the batch, scaled to the whole batch."""
+    import torch
+    from oracle import synth, torch_ref
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5"}[name]
+    w = synth.workload(cfg, batch=1)
+    logits = torch.from_numpy(w["logits"]).requires_grad_()
+    labels = torch.from_numpy(w["labels"])
+    fn = {"lsr": lambda: torch_ref.lsr(logits, labels, 0.1, "mean", 255),
+          "lmargin": lambda: torch_ref.lmargin(logits, labels, 0.3, "mean", 255),
+          "focal": lambda: torch_ref.focal(logits, labels, 0.25, 2, "mean"),
+          "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255)}[name]
+    times = []
+    for i in range(4):
+        logits.grad = None
+        t0 = time.perf_counter()
+        fn().backward()
+        t1 = time.perf_counter()
+        if i:
+            times.append((t1 - t0) * 1e3)
+    scale = shape[0]
+    ms_full = statistics.median(times) * scale
+    fwd, bwd = algorithmic_bytes(name, shape)
+    return {"value": round((fwd + bwd) / (ms_full * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "ms_per_step": round(ms_full, 2),
+            "sample": "oracle/torch_ref.py (pure-torch restatement of the reference's V2/V1 CPU path) on 1 of %d "
+                      "images of the workload, fwd+bwd, median of 3, time scaled x%d" % (scale, scale)}
+
+
+def run_workload(name, steps, warmup, device):
+    import torch
+    shape = WORKLOADS[name]["shape"]
+    logits, labels = make_inputs(name, shape, device)
+    crit = make_criterion(name)
+    ms, loss = time_steps(crit, logits, labels, steps, warmup)
+    fwd, bwd = algorithmic_bytes(name, shape)
+    gbps = (fwd + bwd) / (ms * 1e-3) / 1e9
+    roof = kernel_rooflines(name, logits, labels)
+    del crit
+    logits.grad = None
+    return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="lsr", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the hot path has no collectives); "
+                 "--gpus %d is not supported, run with --gpus 1" % args.gpus)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from pytorch_loss import _native
+    _native.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    name = args.workload
+    main_res = run_workload(name, args.steps, args.warmup, device)
+    torch.cuda.empty_cache()
+
+    others = {}
+    if not args.no_others:
+        for other in WORKLOADS:
+            if other == name:
+                continue
+            try:
+                r = run_workload(other, max(5, args.steps // 2), max(2, args.warmup // 2), device)
+                others[other] = {"workload": WORKLOADS[other]["desc"], "ms_per_step": round(r["ms_per_step"], 4),
+                                 "GB/s": round(r["gbps"], 1), "frac_of_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
+                                 "kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
+                                             for k, v in r["roofline"].items()}}
+            except Exception as e:  # a secondary workload must not take the headline down
+                others[other] = {"error": "%s: %s" % (type(e).__name__, e)}
+            torch.cuda.empty_cache()
+
+    try:
+        ceiling = copy_ceiling(device)
+    except Exception as e:
+        ceiling = "error: %s" % e
+
+    line = {
+        "metric": "fwd+bwd ms/iter + achieved HBM GB/s (% peak), LSR-CE 8x19x1024^2 fp32",
+        "value": round(main_res["gbps"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_res["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": WORKLOADS[name]["desc"], "algorithmic_bytes_per_step": main_res["bytes"],
+                   "frac_of_hbm_peak": round(main_res["gbps"] / HBM_PEAK_GBPS, 4), "loss": main_res["loss"]},
+        "roofline": dict(main_res["roofline"]["backward"], kernel="backward entry point of the workload"),
+        "roofline_forward": main_res["roofline"]["forward"],
+        "copy_kernel_GBps": ceiling,
+        "other_workloads": others,
+    }
+    if not args.no_cpu_baseline:
+        try:
+            line["cpu_baseline"] = cpu_baseline(name, WORKLOADS[name]["shape"])
+        except Exception as e:
+            line["cpu_baseline"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,143 @@
+/*
+ * C ABI of libpytorch_loss_hip.so: the fused "V3" loss kernels of pytorch-loss,
+ * written for AMD MI355X (gfx950).  This is the boundary that replaces the
+ * reference's four pybind11 extension modules (lsr_cpp, focal_cpp,
+ * large_margin_cpp, lovasz_softmax_cpp).
+ *
+ * Conventions for every entry point
+ *   - plain device pointers, sizes and scalars; no framework types;
+ *   - logits are fp32, laid out (n_size, dimsize, m_size) row-major, i.e. NCHW
+ *     with the spatial dims flattened into m_size (the reference flattens the
+ *     same way, csrc/lsr_kernel.cu:199-202); integer labels are int64 (n_size, m_size);
+ *   - `stream` is a hipStream_t (NULL = the default stream); launches are
+ *     asynchronous and the library never synchronises, allocates or frees
+ *     device memory, and keeps no state between calls (re-entrant);
+ *   - the caller sets the current device to the one that owns the pointers;
+ *   - return value: PLH_OK (0), a negative PLH_ERR_* for rejected arguments
+ *     (nothing was launched), or a positive hipError_t from the launch;
+ *   - sizes of 0 elements return PLH_OK without launching
+ *     (csrc/lsr_kernel.cu:207-210 does the same).
+ *
+ * Upstream gradients: the reference returns dloss/dlogits and lets Python do
+ * `grad.mul_(grad_output...)` in a second pass over the tensor
+ * (pytorch_loss/label_smooth.py:143-144).  Here the multiply is fused:
+ *   grad_output == NULL          -> unit upstream gradient (the reference's raw result)
+ *   grad_output_stride == 0      -> one fp32 scalar in device memory, broadcast
+ *   grad_output_stride == 1      -> one fp32 value per loss element, contiguous
+ */
+#ifndef PYTORCH_LOSS_HIP_H
+#define PYTORCH_LOSS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PLH_ABI_VERSION 1
+
+#define PLH_OK 0
+#define PLH_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
+#define PLH_ERR_BAD_SIZE (-2)       /* negative size, or numel beyond the supported range */
+#define PLH_ERR_BAD_STRIDE (-3)     /* grad_output_stride not 0 or 1 */
+#define PLH_ERR_TOO_MANY_CLASSES (-4) /* Lovasz: dimsize >= 512 (csrc/lovasz_softmax.cu:665) */
+#define PLH_ERR_WORKSPACE (-5)      /* workspace smaller than plh_lovasz_workspace_bytes() */
+#define PLH_ERR_MISALIGNED (-6)     /* a pointer is not aligned to its element size */
+
+int plh_abi_version(void);
+
+/* Text for any value an entry point can return (PLH_ERR_* or hipError_t). */
+const char *plh_error_string(int code);
+
+/* ---- label-smoothed softmax cross entropy -----------------------------------
+ * Replaces lsr_cpp.lsr_forward / lsr_cpp.lsr_backward
+ * (csrc/lsr_kernel.cu:296-305, 307-317; kernels :65-185; host :191-293).
+ * losses: (n_size, m_size) fp32, 0 at ignored pixels.
+ * grad_logits: shape of logits, 0 at ignored pixels.
+ */
+int plh_lsr_forward(const float *logits, const int64_t *labels, float *losses,
+                    int64_t n_size, int64_t dimsize, int64_t m_size,
+                    int64_t ignore_index, float smooth, void *stream);
+
+int plh_lsr_backward(const float *logits, const int64_t *labels,
+                     const float *grad_output, int64_t grad_output_stride,
+                     float *grad_logits,
+                     int64_t n_size, int64_t dimsize, int64_t m_size,
+                     int64_t ignore_index, float smooth, void *stream);
+
+/* ---- sigmoid focal loss -------------------------------------------------------
+ * Replaces focal_cpp.focalloss_forward / focalloss_backward /
+ * focalloss_forward_backward (csrc/focal_kernel.cu:301-335; kernels :29-164).
+ * labels are fp32 with the logits' shape (soft labels allowed).  Argument order
+ * (gamma, alpha) follows the reference's C++ side (csrc/focal_kernel.cu:301-303).
+ */
+int plh_focal_forward(const float *logits, const float *labels, float *losses,
+                      int64_t numel, float gamma, float alpha, void *stream);
+
+int plh_focal_backward(const float *logits, const float *labels,
+                       const float *grad_output, int64_t grad_output_stride,
+                       float *grad_logits,
+                       int64_t numel, float gamma, float alpha, void *stream);
+
+/* One pass producing both the losses and dloss/dlogits under a unit upstream gradient. */
+int plh_focal_forward_backward(const float *logits, const float *labels,
+                               float *losses, float *grad_logits,
+                               int64_t numel, float gamma, float alpha, void *stream);
+
+/* ---- large-margin softmax -------------------------------------------------------
+ * Replaces large_margin_cpp.l_margin_forward / l_margin_backward /
+ * l_margin_forward_backward (csrc/large_margin_kernel.cu:796-831; kernels :140-599).
+ * valid_cnt (forward_backward only): one int64 that receives the number of
+ * non-ignored pixels; the call overwrites it (no need to clear it first).
+ */
+int plh_lmargin_forward(const float *logits, const int64_t *labels, float *losses,
+                        int64_t n_size, int64_t dimsize, int64_t m_size,
+                        int64_t ignore_index, float lam, void *stream);
+
+int plh_lmargin_backward(const float *logits, const int64_t *labels,
+                         const float *grad_output, int64_t grad_output_stride,
+                         float *grad_logits,
+                         int64_t n_size, int64_t dimsize, int64_t m_size,
+                         int64_t ignore_index, float lam, void *stream);
+
+int plh_lmargin_forward_backward(const float *logits, const int64_t *labels,
+                                 float *losses, float *grad_logits, int64_t *valid_cnt,
+                                 int64_t n_size, int64_t dimsize, int64_t m_size,
+                                 int64_t ignore_index, float lam, void *stream);
+
+/* ---- Lovasz-softmax ---------------------------------------------------------------
+ * Replaces lovasz_softmax_cpp.lovasz_softmax_forward / lovasz_softmax_backward
+ * (csrc/lovasz_softmax.cu:778-797; pipeline :495-773; csrc/cumsum.hpp:113-150).
+ * losses: (dimsize) fp32, one Lovasz loss per class.
+ * jacc:   (dimsize, n_size*m_size) fp32, the Jaccard differences scattered back to
+ *         pixel order (pixel i = n*m_size + m); the forward writes every element
+ *         and the backward only reads it.
+ * workspace: scratch device memory of at least plh_lovasz_workspace_bytes() bytes,
+ *         256-byte aligned, owned by the caller; contents are undefined afterwards.
+ * Limits: dimsize < 512 and n_size*dimsize*m_size < 2^31 (csrc/lovasz_softmax.cu:664-665).
+ */
+int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size);
+
+int plh_lovasz_forward(const float *logits, const int64_t *labels,
+                       float *losses, float *jacc,
+                       void *workspace, int64_t workspace_bytes,
+                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                       int64_t ignore_index, void *stream);
+
+int plh_lovasz_backward(const float *grad_output, const float *logits, const int64_t *labels,
+                        const float *jacc, float *grad_logits,
+                        int64_t n_size, int64_t dimsize, int64_t m_size,
+                        int64_t ignore_index, void *stream);
+
+/* ---- measurement aid ----------------------------------------------------------------
+ * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,
+ * 4*numel written), used to calibrate hardware byte counters and to measure the
+ * achievable copy bandwidth.  No counterpart in the reference.
+ */
+int plh_stream_copy(const float *src, float *dst, int64_t numel, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PYTORCH_LOSS_HIP_H */

@@ -1,0 +1,640 @@
+// Lovasz-softmax forward and backward for gfx950.
+//
+// Per class c over all P = n_size*m_size pixels (csrc/lovasz_softmax.cu:71-152,182-239):
+//   e_i   = |1[y_i = c] - softmax(x_i)_c|                   ignored pixels take no part
+//   sort e descending; cs_k = number of positives among the first k+1
+//   J_k   = 1 - (n_pos - cs_k) / (n_pos - cs_k + k + 1),    dJ_k = J_k - J_{k-1}  (dJ_0 = J_0)
+//   loss_c = sum_k e_(k) * dJ_k ;  jacc[c, pixel] = dJ of that pixel (0 when ignored)
+// Backward (csrc/lovasz_softmax.cu:242-278,379-417):
+//   d_ic = (c == y_i ? -1 : +1) * jacc[c,i] * grad_out[c];  g_ic = p_ic * (d_ic - sum_k p_ik d_ik)
+//
+// Pipeline (all launches on the caller's stream, nothing allocated here):
+//   1. build_keys     one pass over the logits: softmax in registers, one 32-bit key per
+//                     (class, pixel):  bit 31 = positive flag, bits 0..30 = 0x3F800000 - bits(e)
+//                     (ascending key order = descending error; e lies in [0,1] so its bit
+//                     pattern is monotone), ignored pixel = 0x7FFFFFFF (sorts last).
+//   2. 4 x (tile_hist, offsets_scan, scatter): stable LSD radix sort, 8 bits per pass, batched
+//                     over classes with blockIdx.y. Ranking inside a tile is done per wavefront
+//                     with ballot-built match masks, tiles are re-ordered in LDS so that the
+//                     global writes are runs of consecutive addresses. The positive flag rides
+//                     along in bit 31 and is masked out of the top digit; the payload (pixel
+//                     index) is generated from the position in the first pass.
+//   3. count_pos + scan_tiles: positives per tile, exclusive scan over tiles, n_pos per class.
+//   4. jaccard        cumulative positives -> J, dJ, per-tile partial of the loss, dJ scattered
+//                     to pixel order.
+//   5. reduce_loss    fixed-order sum of the per-tile partials (no floating-point atomics, so
+//                     results are deterministic).
+// Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
+#include "plh_common.hpp"
+
+namespace plh {
+
+constexpr uint32_t kOne = 0x3F800000u;          // bits of 1.0f
+constexpr uint32_t kIgnoredKey = 0x7FFFFFFFu;
+constexpr uint32_t kHotBit = 0x80000000u;
+
+constexpr int kSortThreads = 256;
+constexpr int kSortItems = 16;
+constexpr int kSortTile = kSortThreads * kSortItems;   // 4096 keys per block
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kRadix = 256;
+
+__device__ __forceinline__ uint32_t make_key(float prob, bool hot, bool ignored) {
+    const float err = hot ? fabsf(1.f - prob) : fabsf(prob);
+    const uint32_t bits = __builtin_bit_cast(uint32_t, err);
+    const uint32_t key = (kOne - (bits > kOne ? kOne : bits)) | (hot ? kHotBit : 0u);
+    return ignored ? kIgnoredKey : key;
+}
+
+__device__ __forceinline__ float key_error(uint32_t key) {
+    return __builtin_bit_cast(float, kOne - (key & 0x7FFFFFFFu));
+}
+
+// ------------------------------------------------------ 1. build keys ----
+
+template <int CP, int V>
+__global__ __launch_bounds__(256) void lov_keys_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
+                                                     uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
+                                                     int64_t ignore) {
+    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+    if (pix >= P) return;
+    const int64_t n = pix / m_size;
+    const float *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
+    float v[CP][V];
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < C) load_vec<V>(xs + (int64_t)j * m_size, v[j]);
+    int64_t lb[V];
+    load_labels<V>(lab + pix, lb);
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float mx = v[0][k];
+#pragma unroll
+        for (int j = 1; j < CP; ++j)
+            if (j < C) mx = fmaxf(mx, v[j][k]);
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < C) {
+                v[j][k] = expf(v[j][k] - mx);
+                s += v[j][k];
+            }
+        const bool ign = (lb[k] == ignore);
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < C) v[j][k] = __builtin_bit_cast(float, make_key(v[j][k] / s, lb[k] == j, ign));
+    }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < C) store_vec<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
+}
+
+// Any channel count: a lane per pixel, three sweeps over the slice (the later ones hit cache).
+__global__ __launch_bounds__(256) void lov_keys_lane(const float *__restrict__ x, const int64_t *__restrict__ lab,
+                                                     uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
+                                                     int64_t ignore) {
+    for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
+        const int64_t n = pix / m_size;
+        const float *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
+        const int64_t lb = lab[pix];
+        float mx = -INFINITY;
+        for (int j = 0; j < C; ++j) mx = fmaxf(mx, xs[(int64_t)j * m_size]);
+        float s = 0.f;
+        for (int j = 0; j < C; ++j) s += expf(xs[(int64_t)j * m_size] - mx);
+        for (int j = 0; j < C; ++j)
+            keys[(int64_t)j * P + pix] = make_key(expf(xs[(int64_t)j * m_size] - mx) / s, lb == j, lb == ignore);
+    }
+}
+
+// --------------------------------------------------- 2. radix sort pass ----
+
+struct SortArgs {
+    const uint32_t *keys_in;
+    const uint32_t *vals_in;     // nullptr in the first pass: payload = position
+    uint32_t *keys_out;
+    uint32_t *vals_out;
+    uint32_t *tile_hist;         // [C][kRadix][tiles]: counts, then exclusive offsets inside the class row
+    int P;                       // keys per class row
+    int tiles;                   // ceil(P / kSortTile)
+    int shift;                   // 0, 8, 16, 24
+    uint32_t digit_mask;         // 0xFF, or 0x7F for the top digit (bit 31 is the positive flag)
+};
+
+// Inclusive scan over the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+    const int lane = __lane_id();
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t up = (uint32_t)__builtin_amdgcn_ds_bpermute(((lane - d) & 63) << 2, (int)v);
+        if (lane >= d) v += up;
+    }
+    return v;
+}
+
+// Exclusive scan of one value per thread over a 256-thread block; `total` = block sum.
+// lds must hold kSortWaves + 1 words. Contains barriers: call from uniform control flow.
+__device__ __forceinline__ uint32_t block_excl_scan_256(uint32_t v, uint32_t *lds, uint32_t &total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t incl = wave_incl_scan(v);
+    if (lane == 63) lds[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) before += (w < wave) ? lds[w] : 0u;
+    total = lds[0] + lds[1] + lds[2] + lds[3];
+    __syncthreads();
+    return before + incl - v;
+}
+
+// Stable rank of every key of the wave's 64-key round among equal digits, accumulated in the
+// wave's private digit counters: returns the number of equal digits seen earlier by this wave.
+__device__ __forceinline__ uint32_t wave_rank(uint32_t digit, bool valid, uint32_t *wave_counts) {
+    const int lane = __lane_id();
+    uint64_t peers = __builtin_amdgcn_ballot_w64(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const bool bit = (digit >> b) & 1u;
+        const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
+        peers &= bit ? vote : ~vote;
+    }
+    const uint32_t lower = __builtin_popcountll(peers & ((1ull << lane) - 1ull));
+    const uint32_t count = __builtin_popcountll(peers);
+    const int leader = peers ? (__builtin_ffsll((long long)peers) - 1) : lane;
+    uint32_t seen = 0;
+    if (valid && lane == leader) {
+        seen = wave_counts[digit];
+        wave_counts[digit] = seen + count;
+    }
+    seen = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen);
+    return seen + lower;
+}
+
+__global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
+    __shared__ uint32_t counts[kSortWaves][kRadix];
+    const int c = blockIdx.y, tile = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    __syncthreads();
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, a.P - begin);
+    const uint32_t *kin = a.keys_in + (int64_t)c * a.P + begin;
+#pragma unroll 4
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        const bool valid = li < count;
+        const uint32_t key = valid ? kin[li] : kIgnoredKey;
+        wave_rank((key >> a.shift) & a.digit_mask, valid, counts[wave]);
+    }
+    __syncthreads();
+    const int d = threadIdx.x;
+    a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile] = counts[0][d] + counts[1][d] + counts[2][d] + counts[3][d];
+}
+
+// Exclusive scan, per class, over the (digit-major, tile-minor) table: entry (d, t) becomes the
+// first output position of tile t's keys with digit d. One 1024-thread block per class.
+__global__ __launch_bounds__(1024) void lov_offsets_scan(uint32_t *tile_hist, int tiles) {
+    __shared__ uint32_t wave_tot[16];
+    const int c = blockIdx.x;
+    uint32_t *row = tile_hist + (int64_t)c * kRadix * tiles;
+    const int total = kRadix * tiles;
+    const int per = (total + 1023) / 1024;
+    const int begin = min(total, (int)threadIdx.x * per);
+    const int end = min(total, begin + per);
+    uint32_t sum = 0;
+    for (int i = begin; i < end; ++i) sum += row[i];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t incl = wave_incl_scan(sum);
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (int w = 0; w < 16; ++w) before += (w < wave) ? wave_tot[w] : 0u;
+    uint32_t run = before + incl - sum;
+    for (int i = begin; i < end; ++i) {
+        const uint32_t t = row[i];
+        row[i] = run;
+        run += t;
+    }
+}
+
+__global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
+    __shared__ uint32_t s_keys[kSortTile];
+    __shared__ uint32_t s_vals[kSortTile];
+    __shared__ uint32_t counts[kSortWaves][kRadix];   // per-wave digit counts, then exclusive over waves
+    __shared__ uint32_t digit_start[kRadix];          // first local position of each digit
+    __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
+    __shared__ uint32_t scan_tmp[kSortWaves + 1];
+
+    const int c = blockIdx.y, tile = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    __syncthreads();
+
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, a.P - begin);
+    const int64_t row = (int64_t)c * a.P;
+    const uint32_t *kin = a.keys_in + row + begin;
+    const uint32_t *vin = a.vals_in ? a.vals_in + row + begin : nullptr;
+
+    uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        const bool valid = li < count;
+        key[r] = valid ? kin[li] : kIgnoredKey;
+        val[r] = vin ? (valid ? vin[li] : 0u) : (uint32_t)(begin + li);
+    }
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        rank[r] = wave_rank((key[r] >> a.shift) & a.digit_mask, li < count, counts[wave]);
+    }
+    __syncthreads();
+
+    {
+        const int d = threadIdx.x;
+        const uint32_t c0 = counts[0][d], c1 = counts[1][d], c2 = counts[2][d], c3 = counts[3][d];
+        counts[0][d] = 0;
+        counts[1][d] = c0;
+        counts[2][d] = c0 + c1;
+        counts[3][d] = c0 + c1 + c2;
+        uint32_t total;
+        digit_start[d] = block_excl_scan_256(c0 + c1 + c2 + c3, scan_tmp, total);
+        out_base[d] = a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        if (li < count) {
+            const uint32_t d = (key[r] >> a.shift) & a.digit_mask;
+            const uint32_t pos = digit_start[d] + counts[wave][d] + rank[r];
+            s_keys[pos] = key[r];
+            s_vals[pos] = val[r];
+        }
+    }
+    __syncthreads();
+
+    uint32_t *kout = a.keys_out + row;
+    uint32_t *vout = a.vals_out + row;
+    for (int i = threadIdx.x; i < count; i += kSortThreads) {
+        const uint32_t k = s_keys[i];
+        const uint32_t d = (k >> a.shift) & a.digit_mask;
+        const uint32_t dst = out_base[d] + ((uint32_t)i - digit_start[d]);
+        kout[dst] = k;
+        vout[dst] = s_vals[i];
+    }
+}
+
+// ------------------------------------------ 3./4./5. Jaccard and loss ----
+
+__global__ __launch_bounds__(kSortThreads) void lov_count_pos(const uint32_t *__restrict__ keys,
+                                                              uint32_t *__restrict__ tile_pos, int P, int tiles) {
+    __shared__ uint32_t wave_cnt[kSortWaves];
+    const int c = blockIdx.y, tile = blockIdx.x;
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, P - begin);
+    const uint32_t *kin = keys + (int64_t)c * P + begin;
+    uint32_t n = 0;
+    for (int i = threadIdx.x; i < count; i += kSortThreads) n += kin[i] >> 31;
+    const uint32_t incl = wave_incl_scan(n);
+    if ((threadIdx.x & 63) == 63) wave_cnt[threadIdx.x >> 6] = incl;
+    __syncthreads();
+    if (threadIdx.x == 0) tile_pos[(int64_t)c * tiles + tile] = wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+}
+
+// Per class: exclusive scan of the positives per tile (in place) and the class total.
+__global__ __launch_bounds__(1024) void lov_scan_tiles(uint32_t *tile_pos, uint32_t *n_pos, int tiles) {
+    __shared__ uint32_t wave_tot[16];
+    const int c = blockIdx.x;
+    uint32_t *row = tile_pos + (int64_t)c * tiles;
+    const int per = (tiles + 1023) / 1024;
+    const int begin = min(tiles, (int)threadIdx.x * per);
+    const int end = min(tiles, begin + per);
+    uint32_t sum = 0;
+    for (int i = begin; i < end; ++i) sum += row[i];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t incl = wave_incl_scan(sum);
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+    for (int w = 0; w < 16; ++w) {
+        before += (w < wave) ? wave_tot[w] : 0u;
+        all += wave_tot[w];
+    }
+    uint32_t run = before + incl - sum;
+    for (int i = begin; i < end; ++i) {
+        const uint32_t t = row[i];
+        row[i] = run;
+        run += t;
+    }
+    if (threadIdx.x == 0) n_pos[c] = all;
+}
+
+// Thread t owns the kSortItems consecutive sorted positions begin + t*kSortItems ...
+__global__ __launch_bounds__(kSortThreads) void lov_jaccard(const uint32_t *__restrict__ keys,
+                                                            const uint32_t *__restrict__ vals,
+                                                            const uint32_t *__restrict__ tile_pos,
+                                                            const uint32_t *__restrict__ n_pos,
+                                                            float *__restrict__ jacc, float *__restrict__ tile_loss,
+                                                            int P, int tiles) {
+    __shared__ uint32_t scan_tmp[kSortWaves + 1];
+    __shared__ float wave_loss[kSortWaves];
+    const int c = blockIdx.y, tile = blockIdx.x;
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, P - begin);
+    const int64_t row = (int64_t)c * P;
+    const int first = threadIdx.x * kSortItems;
+
+    uint32_t key[kSortItems], val[kSortItems];
+    if (first + kSortItems <= count && ((row + begin) & 3) == 0) {
+#pragma unroll
+        for (int q = 0; q < kSortItems / 4; ++q) {
+            const uint4 k4 = *reinterpret_cast<const uint4 *>(keys + row + begin + first + 4 * q);
+            const uint4 v4 = *reinterpret_cast<const uint4 *>(vals + row + begin + first + 4 * q);
+            key[4 * q] = k4.x; key[4 * q + 1] = k4.y; key[4 * q + 2] = k4.z; key[4 * q + 3] = k4.w;
+            val[4 * q] = v4.x; val[4 * q + 1] = v4.y; val[4 * q + 2] = v4.z; val[4 * q + 3] = v4.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < kSortItems; ++r) {
+            const bool valid = first + r < count;
+            key[r] = valid ? keys[row + begin + first + r] : kIgnoredKey;
+            val[r] = valid ? vals[row + begin + first + r] : 0u;
+        }
+    }
+    uint32_t mine = 0;
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) mine += key[r] >> 31;
+    uint32_t total;
+    uint32_t cs = block_excl_scan_256(mine, scan_tmp, total) + tile_pos[(int64_t)c * tiles + tile];
+
+    const float npos = (float)n_pos[c];
+    float part = 0.f;
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        if (first + r < count) {
+            const uint32_t k = key[r];
+            const uint32_t hot = k >> 31;
+            float dj = 0.f;
+            if ((k & 0x7FFFFFFFu) != kIgnoredKey) {
+                const int rank = begin + first + r;                    // position in the descending order
+                const float inter_prev = npos - (float)cs;             // csrc/lovasz_softmax.cu:124-127
+                const float inter = npos - (float)(cs + hot);
+                const float j_now = 1.f - inter / (inter + (float)(rank + 1));
+                const float j_prev = (rank == 0) ? 0.f : 1.f - inter_prev / (inter_prev + (float)rank);
+                dj = j_now - j_prev;                                   // csrc/lovasz_softmax.cu:141-147
+                part += key_error(k) * dj;
+            }
+            cs += hot;
+            jacc[row + val[r]] = dj;
+        }
+    }
+    part = group_reduce<64>(part, OpSum());
+    if ((threadIdx.x & 63) == 0) wave_loss[threadIdx.x >> 6] = part;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        tile_loss[(int64_t)c * tiles + tile] = (wave_loss[0] + wave_loss[1]) + (wave_loss[2] + wave_loss[3]);
+}
+
+__global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__ tile_loss, float *__restrict__ losses,
+                                                       int tiles) {
+    __shared__ float wave_sum[4];
+    const int c = blockIdx.x;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < tiles; i += 256) s += tile_loss[(int64_t)c * tiles + i];
+    s = group_reduce<64>(s, OpSum());
+    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) losses[c] = (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]);
+}
+
+// ------------------------------------------------------------ backward ----
+
+template <int CP, int V>
+__global__ __launch_bounds__(256) void lov_bwd_regs(const float *__restrict__ gout, const float *__restrict__ x,
+                                                    const int64_t *__restrict__ lab, const float *__restrict__ jacc,
+                                                    float *__restrict__ grad, int64_t P, int64_t m_size, int C,
+                                                    int64_t ignore) {
+    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+    if (pix >= P) return;
+    const int64_t n = pix / m_size;
+    const int64_t base = pix + n * (int64_t)(C - 1) * m_size;
+    float v[CP][V], d[CP][V];
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < C) {
+            load_vec<V>(x + base + (int64_t)j * m_size, v[j]);
+            load_vec<V>(jacc + (int64_t)j * P + pix, d[j]);
+        }
+    int64_t lb[V];
+    load_labels<V>(lab + pix, lb);
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float mx = v[0][k];
+#pragma unroll
+        for (int j = 1; j < CP; ++j)
+            if (j < C) mx = fmaxf(mx, v[j][k]);
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < C) {
+                v[j][k] = expf(v[j][k] - mx);
+                s += v[j][k];
+            }
+        float dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < C) {
+                v[j][k] = v[j][k] / s;
+                const float dj = d[j][k] * gout[j];
+                d[j][k] = (lb[k] == j) ? -dj : dj;
+                dot += v[j][k] * d[j][k];
+            }
+        const bool ign = (lb[k] == ignore);
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < C) v[j][k] = ign ? 0.f : v[j][k] * (d[j][k] - dot);
+    }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < C) store_vec<V>(grad + base + (int64_t)j * m_size, v[j]);
+}
+
+__global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ gout, const float *__restrict__ x,
+                                                    const int64_t *__restrict__ lab, const float *__restrict__ jacc,
+                                                    float *__restrict__ grad, int64_t P, int64_t m_size, int C,
+                                                    int64_t ignore) {
+    for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
+        const int64_t n = pix / m_size;
+        const int64_t base = pix + n * (int64_t)(C - 1) * m_size;
+        const float *xs = x + base;
+        const int64_t lb = lab[pix];
+        float mx = -INFINITY;
+        for (int j = 0; j < C; ++j) mx = fmaxf(mx, xs[(int64_t)j * m_size]);
+        float s = 0.f;
+        for (int j = 0; j < C; ++j) s += expf(xs[(int64_t)j * m_size] - mx);
+        float dot = 0.f;
+        for (int j = 0; j < C; ++j) {
+            const float p = expf(xs[(int64_t)j * m_size] - mx) / s;
+            const float dj = jacc[(int64_t)j * P + pix] * gout[j];
+            dot += p * ((lb == j) ? -dj : dj);
+        }
+        const bool ign = (lb == ignore);
+        for (int j = 0; j < C; ++j) {
+            const float p = expf(xs[(int64_t)j * m_size] - mx) / s;
+            const float dj = jacc[(int64_t)j * P + pix] * gout[j];
+            grad[base + (int64_t)j * m_size] = ign ? 0.f : p * (((lb == j) ? -dj : dj) - dot);
+        }
+    }
+}
+
+// ------------------------------------------------------------ host side ----
+
+struct LovaszPlan {
+    int64_t P, E;
+    int tiles;
+    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_tile_pos, off_tile_loss, off_n_pos, bytes;
+};
+
+static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan &pl) {
+    if (n_size < 0 || dimsize < 0 || m_size < 0) return PLH_ERR_BAD_SIZE;
+    if (dimsize >= 512) return PLH_ERR_TOO_MANY_CLASSES;
+    const double numel = (double)n_size * (double)dimsize * (double)m_size;
+    if (numel >= 2147483648.0) return PLH_ERR_BAD_SIZE;
+    pl.P = n_size * m_size;
+    pl.E = pl.P * dimsize;
+    pl.tiles = (int)ceil_div(pl.P, kSortTile);
+    int64_t off = 0;
+    pl.off_keys = off;      off += round_up(4 * pl.E, 256);
+    pl.off_vals_a = off;    off += round_up(4 * pl.E, 256);
+    pl.off_vals_b = off;    off += round_up(4 * pl.E, 256);
+    pl.off_hist = off;      off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
+    pl.off_tile_pos = off;  off += round_up(4 * dimsize * pl.tiles, 256);
+    pl.off_tile_loss = off; off += round_up(4 * dimsize * pl.tiles, 256);
+    pl.off_n_pos = off;     off += round_up(4 * dimsize, 256);
+    pl.bytes = off;
+    return PLH_OK;
+}
+
+}  // namespace plh
+
+using namespace plh;
+
+extern "C" int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size) {
+    LovaszPlan pl;
+    const int rc = make_plan(n_size, dimsize, m_size, pl);
+    return rc == PLH_OK ? pl.bytes : (int64_t)rc;
+}
+
+extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, float *losses, float *jacc,
+                                  void *workspace, int64_t workspace_bytes,
+                                  int64_t n_size, int64_t dimsize, int64_t m_size,
+                                  int64_t ignore_index, void *stream) {
+    LovaszPlan pl;
+    int rc = make_plan(n_size, dimsize, m_size, pl);
+    if (rc != PLH_OK) return rc;
+    if (pl.E == 0) return PLH_OK;
+    if (!logits || !labels || !losses || !jacc) return PLH_ERR_NULL_POINTER;
+    if (misaligned(logits, 4) || misaligned(losses, 4) || misaligned(jacc, 4) || misaligned(labels, 8))
+        return PLH_ERR_MISALIGNED;
+    if (!workspace || misaligned(workspace, 256) || workspace_bytes < pl.bytes) return PLH_ERR_WORKSPACE;
+
+    hipStream_t st = (hipStream_t)stream;
+    char *ws = static_cast<char *>(workspace);
+    uint32_t *keys_a = reinterpret_cast<uint32_t *>(ws + pl.off_keys);
+    uint32_t *keys_b = reinterpret_cast<uint32_t *>(jacc);          // free until the Jaccard pass writes it
+    uint32_t *vals_a = reinterpret_cast<uint32_t *>(ws + pl.off_vals_a);
+    uint32_t *vals_b = reinterpret_cast<uint32_t *>(ws + pl.off_vals_b);
+    uint32_t *hist = reinterpret_cast<uint32_t *>(ws + pl.off_hist);
+    uint32_t *tile_pos = reinterpret_cast<uint32_t *>(ws + pl.off_tile_pos);
+    float *tile_loss = reinterpret_cast<float *>(ws + pl.off_tile_loss);
+    uint32_t *n_pos = reinterpret_cast<uint32_t *>(ws + pl.off_n_pos);
+    const int C = (int)dimsize;
+
+    // 1. keys
+    const Shape shape = pick_shape(dimsize, m_size, logits, keys_a, labels, nullptr, nullptr);
+    if (shape == Shape::Regs4 || shape == Shape::Regs1) {
+        const int V = (shape == Shape::Regs4 && pl.P % 4 == 0) ? 4 : 1;
+        const unsigned grid = (unsigned)ceil_div(ceil_div(pl.P, V), 256);
+        switch ((C + 3) / 4) {
+#define PLH_CASE(K)                                                                                              \
+    case K:                                                                                                      \
+        if (V == 4) hipLaunchKernelGGL((lov_keys_regs<4 * K, 4>), dim3(grid), dim3(256), 0, st, logits, labels,  \
+                                       keys_a, pl.P, m_size, C, ignore_index);                                   \
+        else hipLaunchKernelGGL((lov_keys_regs<4 * K, 1>), dim3(grid), dim3(256), 0, st, logits, labels, keys_a, \
+                                pl.P, m_size, C, ignore_index);                                                  \
+        break;
+            PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+        }
+    } else {
+        hipLaunchKernelGGL(lov_keys_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, logits, labels, keys_a,
+                           pl.P, m_size, C, ignore_index);
+    }
+
+    // 2. four stable radix passes, ping-ponging (keys_a, vals_a) <-> (keys_b, vals_b)
+    const dim3 tile_grid((unsigned)pl.tiles, (unsigned)C);
+    for (int pass = 0; pass < 4; ++pass) {
+        SortArgs a;
+        const bool even = (pass % 2 == 0);
+        a.keys_in = even ? keys_a : keys_b;
+        a.vals_in = (pass == 0) ? nullptr : (even ? vals_a : vals_b);
+        a.keys_out = even ? keys_b : keys_a;
+        a.vals_out = even ? vals_b : vals_a;
+        a.tile_hist = hist;
+        a.P = (int)pl.P;
+        a.tiles = pl.tiles;
+        a.shift = 8 * pass;
+        a.digit_mask = (pass == 3) ? 0x7Fu : 0xFFu;
+        hipLaunchKernelGGL(lov_tile_hist, tile_grid, dim3(kSortThreads), 0, st, a);
+        hipLaunchKernelGGL(lov_offsets_scan, dim3((unsigned)C), dim3(1024), 0, st, hist, pl.tiles);
+        hipLaunchKernelGGL(lov_scatter, tile_grid, dim3(kSortThreads), 0, st, a);
+    }
+
+    // 3.-5. sorted rows are in (keys_a, vals_a); jacc is free again
+    hipLaunchKernelGGL(lov_count_pos, tile_grid, dim3(kSortThreads), 0, st, keys_a, tile_pos, (int)pl.P, pl.tiles);
+    hipLaunchKernelGGL(lov_scan_tiles, dim3((unsigned)C), dim3(1024), 0, st, tile_pos, n_pos, pl.tiles);
+    hipLaunchKernelGGL(lov_jaccard, tile_grid, dim3(kSortThreads), 0, st, keys_a, vals_a, tile_pos, n_pos, jacc,
+                       tile_loss, (int)pl.P, pl.tiles);
+    hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
+    return check_launch();
+}
+
+extern "C" int plh_lovasz_backward(const float *grad_output, const float *logits, const int64_t *labels,
+                                   const float *jacc, float *grad_logits,
+                                   int64_t n_size, int64_t dimsize, int64_t m_size,
+                                   int64_t ignore_index, void *stream) {
+    LovaszPlan pl;
+    const int rc = make_plan(n_size, dimsize, m_size, pl);
+    if (rc != PLH_OK) return rc;
+    if (pl.E == 0) return PLH_OK;
+    if (!grad_output || !logits || !labels || !jacc || !grad_logits) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_output, 4) || misaligned(logits, 4) || misaligned(jacc, 4) || misaligned(grad_logits, 4) ||
+        misaligned(labels, 8))
+        return PLH_ERR_MISALIGNED;
+    hipStream_t st = (hipStream_t)stream;
+    const int C = (int)dimsize;
+    const Shape shape = pick_shape(dimsize, m_size, logits, grad_logits, labels, jacc, nullptr);
+    if (shape == Shape::Regs4 || shape == Shape::Regs1) {
+        const int V = (shape == Shape::Regs4 && pl.P % 4 == 0) ? 4 : 1;
+        const unsigned grid = (unsigned)ceil_div(ceil_div(pl.P, V), 256);
+        switch ((C + 3) / 4) {
+#define PLH_CASE(K)                                                                                               \
+    case K:                                                                                                       \
+        if (V == 4) hipLaunchKernelGGL((lov_bwd_regs<4 * K, 4>), dim3(grid), dim3(256), 0, st, grad_output,       \
+                                       logits, labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);         \
+        else hipLaunchKernelGGL((lov_bwd_regs<4 * K, 1>), dim3(grid), dim3(256), 0, st, grad_output, logits,      \
+                                labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);                        \
+        break;
+            PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+        }
+    } else {
+        hipLaunchKernelGGL(lov_bwd_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, grad_output, logits, labels,
+                           jacc, grad_logits, pl.P, m_size, C, ignore_index);
+    }
+    return check_launch();
+}

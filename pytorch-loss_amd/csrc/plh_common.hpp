@@ -1,0 +1,195 @@
+// Shared device/host helpers for the gfx950 loss kernels.
+//
+// Two execution shapes are used for every channel-dim reduction:
+//   "regs"  : lanes run along consecutive pixels, each thread owns V pixels and
+//             keeps the whole channel slice in VGPRs. Each per-channel load of a
+//             wavefront is one contiguous 64*V*4-byte run, logits are read from
+//             HBM exactly once and no cross-lane traffic is needed.
+//   "group" : G lanes share one pixel and stride over its channels (G = 64: a
+//             wavefront per row, for (N, C) inputs where the channel dim is the
+//             contiguous one; G = 1: a lane per pixel for deep channel dims in
+//             NCHW). Reductions inside a group use DPP/swizzle, the slice is
+//             staged in LDS when it has to be read more than once.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/pytorch_loss_hip.h"
+
+namespace plh {
+
+constexpr int kWave = 64;
+
+// ---- argument checks shared by the entry points -----------------------------
+
+inline bool misaligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+// Largest element count the kernels index (64-bit offsets are used throughout;
+// the bound keeps every intermediate product well inside int64).
+constexpr int64_t kMaxNumel = (int64_t)1 << 40;
+
+inline int check_launch() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? PLH_OK : (int)e;
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Checks for the (n_size, dimsize, m_size) entry points. `out` is the tensor written.
+inline int check_slice_args(const void *logits, const void *labels, const void *out,
+                            int64_t n_size, int64_t dimsize, int64_t m_size) {
+    if (n_size < 0 || dimsize < 0 || m_size < 0) return PLH_ERR_BAD_SIZE;
+    if (n_size > kMaxNumel || dimsize > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    if (dimsize > (int64_t)1 << 30) return PLH_ERR_BAD_SIZE;
+    const double numel = (double)n_size * (double)dimsize * (double)m_size;
+    if (numel > (double)kMaxNumel) return PLH_ERR_BAD_SIZE;
+    if (numel == 0) return PLH_OK;
+    if (!logits || !labels || !out) return PLH_ERR_NULL_POINTER;
+    if (misaligned(logits, 4) || misaligned(out, 4) || misaligned(labels, 8)) return PLH_ERR_MISALIGNED;
+    return PLH_OK;
+}
+
+inline int check_gout(const void *gout, int64_t stride) {
+    if (!gout) return PLH_OK;
+    if (stride != 0 && stride != 1) return PLH_ERR_BAD_STRIDE;
+    if (misaligned(gout, 4)) return PLH_ERR_MISALIGNED;
+    return PLH_OK;
+}
+
+// Which execution shape serves a (dimsize, m_size) problem. The float pointers
+// passed in (nullptr = not used) must all be 16-byte aligned for the 4-pixel
+// vector form, and so must the labels.
+enum class Shape { Regs4, Regs1, Wave, Lane };
+
+constexpr int kMaxRegsChannels = 32;
+
+inline Shape pick_shape(int64_t dimsize, int64_t m_size, const void *f0, const void *f1,
+                        const void *labels, const void *f2, const void *f3) {
+    if (dimsize <= kMaxRegsChannels) {
+        const bool vec = (m_size % 4 == 0) && !(f0 && misaligned(f0, 16)) && !(f1 && misaligned(f1, 16)) &&
+                         !(f2 && misaligned(f2, 16)) && !(f3 && misaligned(f3, 16)) &&
+                         !(labels && misaligned(labels, 16));
+        return vec ? Shape::Regs4 : Shape::Regs1;
+    }
+    return m_size == 1 ? Shape::Wave : Shape::Lane;
+}
+
+// Grid for the group kernels: they loop, so the grid is capped.
+inline unsigned group_grid(int64_t pixels, int pixels_per_block) {
+    const int64_t want = ceil_div(pixels, pixels_per_block);
+    const int64_t cap = 256 * 64;   // 64 resident-or-queued blocks per CU
+    return (unsigned)(want < cap ? (want > 0 ? want : 1) : cap);
+}
+
+// ---- vector access -----------------------------------------------------------
+
+template <int V> struct Vec;
+template <> struct Vec<1> { using type = float; };
+template <> struct Vec<2> { using type = float2; };
+template <> struct Vec<4> { using type = float4; };
+
+template <int V>
+__device__ __forceinline__ void load_vec(const float *p, float (&out)[V]) {
+    if constexpr (V == 1) {
+        out[0] = *p;
+    } else if constexpr (V == 2) {
+        const float2 t = *reinterpret_cast<const float2 *>(p);
+        out[0] = t.x; out[1] = t.y;
+    } else {
+        const float4 t = *reinterpret_cast<const float4 *>(p);
+        out[0] = t.x; out[1] = t.y; out[2] = t.z; out[3] = t.w;
+    }
+}
+
+template <int V>
+__device__ __forceinline__ void store_vec(float *p, const float (&v)[V]) {
+    if constexpr (V == 1) {
+        *p = v[0];
+    } else if constexpr (V == 2) {
+        *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+    } else {
+        *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
+template <int V>
+__device__ __forceinline__ void load_labels(const int64_t *p, int64_t (&out)[V]) {
+    if constexpr (V == 1) {
+        out[0] = *p;
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; k += 2) {
+            const longlong2 t = *reinterpret_cast<const longlong2 *>(p + k);
+            out[k] = t.x; out[k + 1] = t.y;
+        }
+    }
+}
+
+// Upstream gradient for V consecutive loss elements starting at `i`.
+// gout == nullptr: 1; stride 0: broadcast scalar; stride 1: per element.
+template <int V>
+__device__ __forceinline__ void load_gout(const float *gout, int64_t stride, int64_t i, float (&out)[V]) {
+    if (gout == nullptr) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) out[k] = 1.0f;
+    } else if (stride == 0) {
+        const float g = *gout;
+#pragma unroll
+        for (int k = 0; k < V; ++k) out[k] = g;
+    } else {
+        load_vec<V>(gout + i, out);
+    }
+}
+
+// ---- wave64 reductions ---------------------------------------------------------
+// Intra-row steps (16 lanes) are DPP moves folded into the VALU op, the 16<->16
+// step is a ds_swizzle, the 32<->32 step a ds_bpermute. Every lane ends with the
+// full result.
+
+template <int Ctrl>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float swizzle_xor16(float v) {
+    // bit-mode swizzle: and_mask 0x1F, or_mask 0, xor_mask 0x10
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+
+__device__ __forceinline__ float bpermute_xor32(float v) {
+    const int lane = __lane_id();
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), __builtin_bit_cast(int, v)));
+}
+
+struct OpSum { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+
+// Reduce over groups of G consecutive lanes (G = 1, 16 or 64).
+template <int G, class Op>
+__device__ __forceinline__ float group_reduce(float v, Op op) {
+    if constexpr (G >= 16) {
+        v = op(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+        v = op(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+        v = op(v, dpp_move<0x141>(v));   // row_half_mirror
+        v = op(v, dpp_move<0x140>(v));   // row_mirror
+    }
+    if constexpr (G >= 64) {
+        v = op(v, swizzle_xor16(v));
+        v = op(v, bpermute_xor32(v));
+    }
+    return v;
+}
+
+// Block-wide sum for 256-thread blocks (4 waves) through LDS; result valid in thread 0.
+__device__ __forceinline__ float block_sum_256(float v, float *lds4) {
+    v = group_reduce<64>(v, OpSum());
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+    __syncthreads();
+    return lds4[0] + lds4[1] + lds4[2] + lds4[3];
+}
+
+}  // namespace plh

@@ -1,0 +1,18 @@
+"""Drop-in for the fused "V3" losses of pytorch-loss, running on hand-written HIP kernels (MI355X).
+
+    from pytorch_loss import LabelSmoothSoftmaxCEV3, FocalLossV3, LargeMarginSoftmaxV3, LovaszSoftmaxV3
+
+Only this path is provided; the kernels live in libpytorch_loss_hip.so (built by
+``python pytorch-loss_amd/build.py``) and there is no CPU fallback.
+"""
+from .label_smooth import LabelSmoothSoftmaxCEV3, LSRCrossEntropyFunctionV3
+from .focal_loss import FocalLossV3, FocalSigmoidLossFuncV3, FocalSigmoidLossFuncV3FB
+from .large_margin_softmax import LargeMarginSoftmaxV3, LargeMarginSoftmaxFuncV3, LargeMarginSoftmaxFuncV3FB
+from .lovasz_softmax import LovaszSoftmaxV3, LovaszSoftmaxFunctionV3
+
+__all__ = [
+    "LabelSmoothSoftmaxCEV3", "LSRCrossEntropyFunctionV3",
+    "FocalLossV3", "FocalSigmoidLossFuncV3", "FocalSigmoidLossFuncV3FB",
+    "LargeMarginSoftmaxV3", "LargeMarginSoftmaxFuncV3", "LargeMarginSoftmaxFuncV3FB",
+    "LovaszSoftmaxV3", "LovaszSoftmaxFunctionV3",
+]

@@ -1,0 +1,316 @@
+"""ctypes binding of libpytorch_loss_hip.so and the tensor marshalling around it.
+
+The shared library speaks plain pointers and sizes (include/pytorch_loss_hip.h).
+This module owns everything the reference's C++ host wrappers did with ATen:
+device checks, `.contiguous()`, output and workspace allocation (through torch's
+caching allocator, so the library itself never allocates), device guard and
+current-stream lookup, and turning non-zero return codes into RuntimeError.
+
+There is no fallback: if the library is missing or a tensor is not on a GPU the
+call raises, like the reference's AT_ERROR("... only supports gpu mode")
+(csrc/lsr_kernel.cu:300-302).
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpytorch_loss_hip.so")
+ABI_VERSION = 1
+
+_lib = None
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_f32 = ctypes.c_float
+
+_SIGNATURES = {
+    "plh_abi_version": (ctypes.c_int, []),
+    "plh_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "plh_lsr_forward": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_focal_forward": (ctypes.c_int, [_p, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_forward_backward": (ctypes.c_int, [_p, _p, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_lmargin_forward": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "plh_lovasz_forward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
+}
+
+
+def load():
+    """Load the HIP library once; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "pytorch_loss: %s is missing; build it with `python pytorch-loss_amd/build.py` "
+                "(there is no CPU or pure-PyTorch fallback)" % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                raise RuntimeError("pytorch_loss: %s does not export %s; rebuild it" % (LIB_PATH, name))
+            fn.restype = res
+            fn.argtypes = args
+        got = lib.plh_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError("pytorch_loss: library ABI %d, binding expects %d" % (got, ABI_VERSION))
+        _lib = lib
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError("pytorch_loss HIP library: %s (code %d)" % (load().plh_error_string(rc).decode(), rc))
+
+
+def _stream():
+    return _p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return _p(t.data_ptr()) if t is not None else _p(0)
+
+
+def _require_gpu(what, *tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("this %s only supports gpu mode" % what)
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError("%s: all tensors must be on the same device" % what)
+
+
+def _f32c(t):
+    """fp32 contiguous view/copy (fp16/bf16/fp64 inputs are computed in fp32)."""
+    if t.dtype != torch.float32:
+        t = t.float()
+    return t.contiguous()
+
+
+def _labels_i64(labels, logits, what):
+    if labels.dtype != torch.int64:
+        if labels.is_floating_point() or labels.dtype == torch.bool:
+            raise RuntimeError("%s: labels must be an integer tensor (int64)" % what)
+        labels = labels.long()
+    if tuple(labels.shape) != tuple(logits.shape[:1]) + tuple(logits.shape[2:]):
+        raise RuntimeError("%s: labels of shape %s do not match logits of shape %s (expect (N, *) vs (N, C, *))"
+                           % (what, tuple(labels.shape), tuple(logits.shape)))
+    return labels.contiguous()
+
+
+def _dims(logits, what):
+    if logits.dim() < 2:
+        raise RuntimeError("%s: logits must have at least 2 dims (N, C, ...)" % what)
+    n_size, dimsize = int(logits.shape[0]), int(logits.shape[1])
+    m_size = 1
+    for d in logits.shape[2:]:
+        m_size *= int(d)
+    return n_size, dimsize, m_size
+
+
+def _upstream(grad_output, like_shape):
+    """-> (tensor kept alive or None, stride). Expanded scalars are passed as one value."""
+    if grad_output is None:
+        return None, 0
+    if tuple(grad_output.shape) != tuple(like_shape):
+        grad_output = grad_output.expand(like_shape)
+    if grad_output.numel() > 0 and all(s == 0 for s, n in zip(grad_output.stride(), grad_output.shape) if n > 1):
+        # produced by sum()/mean() backward: a single value broadcast over the loss tensor
+        one = grad_output.as_strided((1,), (1,))
+        if one.dtype != torch.float32:
+            one = one.float()
+        return one, 0
+    return _f32c(grad_output), 1
+
+
+def _back_to(t, dtype):
+    return t if dtype == torch.float32 else t.to(dtype)
+
+
+# ------------------------------------------------------------------ LSR ----
+
+def lsr_forward(logits, labels, ignore_index, smooth):
+    _require_gpu("LSR loss", logits, labels)
+    n, c, m = _dims(logits, "lsr_forward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "lsr_forward")
+    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return _back_to(losses.zero_(), logits.dtype)
+    with torch.cuda.device_of(x):
+        _check(load().plh_lsr_forward(_ptr(x), _ptr(lb), _ptr(losses), n, c, m,
+                                      int(ignore_index), float(smooth), _stream()))
+    return _back_to(losses, logits.dtype)
+
+
+def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None):
+    """dloss/dlogits, already multiplied by ``grad_output`` (None = unit upstream gradient)."""
+    _require_gpu("LSR loss", logits, labels)
+    n, c, m = _dims(logits, "lsr_backward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "lsr_backward")
+    grad = torch.empty_like(x)
+    if x.numel() == 0:
+        return _back_to(grad, logits.dtype)
+    go, stride = _upstream(grad_output, lb.shape)
+    with torch.cuda.device_of(x):
+        _check(load().plh_lsr_backward(_ptr(x), _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
+                                       int(ignore_index), float(smooth), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+# ---------------------------------------------------------------- focal ----
+
+def _focal_pair(logits, labels, what):
+    _require_gpu("focal loss", logits, labels)
+    if tuple(labels.shape) != tuple(logits.shape):
+        raise RuntimeError("%s: labels and logits must have the same shape" % what)
+    return _f32c(logits), _f32c(labels)
+
+
+def focal_forward(logits, labels, gamma, alpha):
+    x, y = _focal_pair(logits, labels, "focalloss_forward")
+    losses = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_forward(_ptr(x), _ptr(y), _ptr(losses), x.numel(),
+                                            float(gamma), float(alpha), _stream()))
+    return _back_to(losses, logits.dtype)
+
+
+def focal_backward(logits, labels, gamma, alpha, grad_output=None):
+    x, y = _focal_pair(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(x)
+    if x.numel():
+        go, stride = _upstream(grad_output, x.shape)
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_backward(_ptr(x), _ptr(y), _ptr(go), stride, _ptr(grad), x.numel(),
+                                             float(gamma), float(alpha), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+def focal_forward_backward(logits, labels, gamma, alpha):
+    x, y = _focal_pair(logits, labels, "focalloss_forward_backward")
+    losses = torch.empty_like(x)
+    grad = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_forward_backward(_ptr(x), _ptr(y), _ptr(losses), _ptr(grad), x.numel(),
+                                                     float(gamma), float(alpha), _stream()))
+    return _back_to(losses, logits.dtype), _back_to(grad, logits.dtype)
+
+
+# -------------------------------------------------------------- lmargin ----
+
+def lmargin_forward(logits, labels, lam, ignore_index):
+    _require_gpu("large margin loss", logits, labels)
+    n, c, m = _dims(logits, "l_margin_forward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "l_margin_forward")
+    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return _back_to(losses.zero_(), logits.dtype)
+    with torch.cuda.device_of(x):
+        _check(load().plh_lmargin_forward(_ptr(x), _ptr(lb), _ptr(losses), n, c, m,
+                                          int(ignore_index), float(lam), _stream()))
+    return _back_to(losses, logits.dtype)
+
+
+def lmargin_backward(logits, labels, lam, ignore_index, grad_output=None):
+    _require_gpu("large margin loss", logits, labels)
+    n, c, m = _dims(logits, "l_margin_backward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "l_margin_backward")
+    grad = torch.empty_like(x)
+    if x.numel() == 0:
+        return _back_to(grad, logits.dtype)
+    go, stride = _upstream(grad_output, lb.shape)
+    with torch.cuda.device_of(x):
+        _check(load().plh_lmargin_backward(_ptr(x), _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
+                                           int(ignore_index), float(lam), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+def lmargin_forward_backward(logits, labels, lam, ignore_index):
+    """-> (losses, grad under unit upstream gradient, valid_cnt int64[1])"""
+    _require_gpu("large margin loss", logits, labels)
+    n, c, m = _dims(logits, "l_margin_forward_backward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "l_margin_forward_backward")
+    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
+    grad = torch.empty_like(x)
+    cnt = torch.zeros(1, dtype=torch.int64, device=x.device)
+    if x.numel():
+        with torch.cuda.device_of(x):
+            _check(load().plh_lmargin_forward_backward(_ptr(x), _ptr(lb), _ptr(losses), _ptr(grad), _ptr(cnt),
+                                                       n, c, m, int(ignore_index), float(lam), _stream()))
+    else:
+        losses.zero_()
+    return _back_to(losses, logits.dtype), _back_to(grad, logits.dtype), cnt
+
+
+# --------------------------------------------------------------- lovasz ----
+
+def _lovasz_limits(logits, what):
+    # same limits and wording as csrc/lovasz_softmax.cu:664-665
+    if logits.numel() >= (1 << 31):
+        raise RuntimeError("%s: input tensor too large, int32 type will overflow" % what)
+    if logits.dim() >= 2 and logits.shape[1] >= 512:
+        raise RuntimeError("%s: num of classes should be less than BLOCKSIZE" % what)
+
+
+def lovasz_forward(logits, labels, ignore_index):
+    """-> (losses[C], jacc[C, N*M])"""
+    _require_gpu("lovasz softmax function", logits, labels)
+    _lovasz_limits(logits, "lovasz_softmax_forward")
+    n, c, m = _dims(logits, "lovasz_softmax_forward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "lovasz_softmax_forward")
+    losses = torch.empty((c,), dtype=torch.float32, device=x.device)
+    jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return _back_to(losses.zero_(), logits.dtype), jacc
+    lib = load()
+    ws_bytes = int(lib.plh_lovasz_workspace_bytes(n, c, m))
+    if ws_bytes < 0:
+        _check(ws_bytes)
+    workspace = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device_of(x):
+        _check(lib.plh_lovasz_forward(_ptr(x), _ptr(lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
+                                      n, c, m, int(ignore_index), _stream()))
+    return _back_to(losses, logits.dtype), jacc
+
+
+def lovasz_backward(grad_output, logits, labels, jacc, ignore_index):
+    _require_gpu("lovasz softmax function", logits, labels, grad_output, jacc)
+    n, c, m = _dims(logits, "lovasz_softmax_backward")
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, "lovasz_softmax_backward")
+    grad = torch.empty_like(x)
+    if x.numel() == 0:
+        return _back_to(grad, logits.dtype)
+    go = _f32c(grad_output.expand((c,)) if grad_output.numel() == 1 else grad_output)
+    if go.numel() != c or jacc.numel() != c * n * m or jacc.dtype != torch.float32:
+        raise RuntimeError("lovasz_softmax_backward: grad_output must have C elements and jacc C*N*M fp32 elements")
+    jc = jacc.contiguous()
+    with torch.cuda.device_of(x):
+        _check(load().plh_lovasz_backward(_ptr(go), _ptr(x), _ptr(lb), _ptr(jc), _ptr(grad), n, c, m,
+                                          int(ignore_index), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+def stream_copy(src, dst):
+    _require_gpu("stream copy", src, dst)
+    assert src.dtype == torch.float32 and dst.dtype == torch.float32 and src.numel() == dst.numel()
+    assert src.is_contiguous() and dst.is_contiguous()
+    with torch.cuda.device_of(src):
+        _check(load().plh_stream_copy(_ptr(src), _ptr(dst), src.numel(), _stream()))

@@ -1,0 +1,53 @@
+"""Label-smoothed softmax cross entropy on the HIP kernels.
+
+Same surface as the reference's V3 pair (pytorch_loss/label_smooth.py:126-171):
+``LSRCrossEntropyFunctionV3.apply(logits, labels, lb_smooth, lb_ignore)`` returns the
+per-pixel losses, ``LabelSmoothSoftmaxCEV3(lb_smooth, reduction, ignore_index)`` reduces
+them.  Target weight is ``1 - lb_smooth``, every other class gets ``lb_smooth / C``.
+"""
+import torch
+import torch.amp as amp
+import torch.nn as nn
+
+from . import _native
+
+
+class LSRCrossEntropyFunctionV3(torch.autograd.Function):
+    """forward -> losses of shape ``labels.shape`` (0 at ignored pixels);
+    backward -> d/dlogits, with the upstream gradient folded into the same kernel."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, lb_smooth, lb_ignore):
+        ctx.variables = (logits, labels, lb_ignore, lb_smooth)
+        return _native.lsr_forward(logits, labels, lb_ignore, lb_smooth)
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        logits, labels, lb_ignore, lb_smooth = ctx.variables
+        grad = _native.lsr_backward(logits, labels, lb_ignore, lb_smooth, grad_output)
+        return grad, None, None, None
+
+
+class LabelSmoothSoftmaxCEV3(nn.Module):
+    """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
+
+    reduction: 'mean' divides the summed loss by the number of non-ignored pixels,
+    'sum' sums, anything else returns the per-pixel tensor.
+    """
+
+    def __init__(self, lb_smooth=0.1, reduction="mean", ignore_index=-100):
+        super().__init__()
+        self.lb_smooth = lb_smooth
+        self.reduction = reduction
+        self.lb_ignore = ignore_index
+
+    def forward(self, logits, labels):
+        losses = LSRCrossEntropyFunctionV3.apply(logits, labels, self.lb_smooth, self.lb_ignore)
+        if self.reduction == "sum":
+            return losses.sum()
+        if self.reduction == "mean":
+            n_valid = (labels != self.lb_ignore).sum()
+            return losses.sum() / n_valid
+        return losses

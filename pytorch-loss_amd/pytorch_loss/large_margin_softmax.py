@@ -1,0 +1,77 @@
+"""Large-margin softmax cross entropy (Kobayashi, BMVC 2019) on the HIP kernels.
+
+Same surface as the reference's V3 classes (pytorch_loss/large_margin_softmax.py:149-201
+and the repository root copy large_margin_softmax.py:146-229, which adds the fused
+``LargeMarginSoftmaxFuncV3FB`` and the module's ``fb`` switch).
+"""
+import torch
+import torch.amp as amp
+import torch.nn as nn
+
+from . import _native
+
+
+class LargeMarginSoftmaxFuncV3(torch.autograd.Function):
+    """forward -> per-pixel losses; backward recomputes from the inputs."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
+        ctx.variables = (logits, labels, lam, ignore_index)
+        return _native.lmargin_forward(logits, labels, lam, ignore_index)
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        logits, labels, lam, ignore_index = ctx.variables
+        grads = _native.lmargin_backward(logits, labels, lam, ignore_index, grad_output)
+        return grads, None, None, None
+
+
+class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
+    """forward -> (per-pixel losses, valid_cnt int64[1]); the gradient is produced by the same
+    kernel and kept for backward."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
+        losses, grads, valid_cnt = _native.lmargin_forward_backward(logits, labels, lam, ignore_index)
+        ctx.variables = grads
+        ctx.mark_non_differentiable(valid_cnt)
+        return losses, valid_cnt
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output, grad_cnt):
+        grads = ctx.variables
+        grads.mul_(grad_output.unsqueeze(1))
+        return grads, None, None, None
+
+
+class LargeMarginSoftmaxV3(nn.Module):
+    """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
+
+    fb=True selects the fused forward+backward Function (one kernel, keeps a gradient-sized
+    tensor between forward and backward); the default recomputes in backward, which moves
+    fewer bytes in total.
+    """
+
+    def __init__(self, lam=0.3, reduction="mean", ignore_index=255, fb=False):
+        super().__init__()
+        self.reduction = reduction
+        self.ignore_index = ignore_index
+        self.lam = lam
+        self.fb = fb
+
+    def forward(self, logits, labels):
+        valid_cnt = None
+        if self.fb:
+            losses, valid_cnt = LargeMarginSoftmaxFuncV3FB.apply(logits, labels, self.lam, self.ignore_index)
+        else:
+            losses = LargeMarginSoftmaxFuncV3.apply(logits, labels, self.lam, self.ignore_index)
+        if self.reduction == "mean":
+            n_valid = valid_cnt if valid_cnt is not None else (labels != self.ignore_index).sum()
+            return losses.sum() / n_valid
+        if self.reduction == "sum":
+            return losses.sum()
+        return losses

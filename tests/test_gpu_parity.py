@@ -1,0 +1,351 @@
+"""GPU parity: the HIP path (through the C ABI, via the drop-in Python surface) against the CPU oracle.
+
+Tolerances are the ones the scope states: loss within 1e-5 relative, gradients within
+1e-5 max-abs in fp32, masks exact (zeros at ignored pixels are bit-exact zeros, the valid
+count is an exact integer).  Because a 'mean' over millions of pixels makes the absolute
+gradient bound vacuous, gradients are also held to a relative max-norm bound under unit
+upstream gradient ('sum'/'none').
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+GRAD_ATOL = 1e-5
+GRAD_REL = 2e-5      # max|got - want| / max|want|
+
+
+@pytest.fixture(scope="module")
+def pl():
+    import pytorch_loss
+    from pytorch_loss import _native
+    _native.load()
+    return pytorch_loss
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def close_loss(got, want, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    scale = np.maximum(np.abs(want), 1e-3 if want.ndim else 1e-30)
+    err = np.abs(got - want) / scale
+    assert np.all(err <= LOSS_RTOL), "%s loss rel err %.3e" % (what, err.max())
+
+
+def close_grad(got, want, what=""):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64)).max() if got.size else 0.0
+    assert err <= GRAD_ATOL, "%s grad max-abs err %.3e" % (what, err)
+    ref = np.abs(want).max() if want.size else 0.0
+    if ref > 0:
+        assert err / ref <= GRAD_REL, "%s grad rel err %.3e" % (what, err / ref)
+
+
+SEG_CASES = [
+    # (shape, ignore_index, ignore_frac)            execution shape
+    ((2, 19, 64, 64), 255, 0.05),                   # 4 pixels per thread, channels in registers
+    ((2, 19, 7, 9), 255, 0.1),                      # odd spatial size -> 1 pixel per thread
+    ((3, 2, 5, 8), -100, 0.2),
+    ((4, 32, 4, 4), 255, 0.0),
+    ((2, 3, 1, 1), 255, 0.0),
+    ((37, 10), -100, 0.1),                          # (N, C) classification input, C <= 32
+    ((33, 100), -100, 0.1),                         # (N, C): one wavefront per row
+    ((5, 1000), 255, 0.3),
+    ((3, 4100), 255, 0.0),                          # row longer than the LDS staging buffer
+    ((2, 33, 6, 7), 255, 0.2),                      # deep channel dim in NCHW: one lane per pixel
+    ((2, 227, 5, 5), 255, 0.1),
+    ((1, 64, 2, 3, 4), 0, 0.3),                     # 5-D input, ignore_index inside the class range
+    ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
+]
+
+
+def seg_inputs(seed, shape, ignore, frac):
+    n_cls = shape[1]
+    x = synth.normal(seed, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(seed, shape[:1] + shape[2:], n_cls, ignore, frac)
+    if ignore == 0 and frac < 1.0:
+        y[y == 0] = 1 if n_cls > 1 else 0
+        y[synth.bernoulli(seed, 12, y.shape, frac)] = 0
+    return x, y
+
+
+# ------------------------------------------------------------------ LSR ----
+
+@pytest.mark.parametrize("shape,ignore,frac", SEG_CASES)
+def test_lsr_function_matches_oracle(pl, shape, ignore, frac):
+    x, y = seg_inputs(21, shape, ignore, frac)
+    xt = dev(x).requires_grad_()
+    yt = dev(y)
+    losses = pl.LSRCrossEntropyFunctionV3.apply(xt, yt, 0.1, ignore)
+    want = oracle.lsr_forward(x, y, ignore, 0.1)
+    assert losses.shape == yt.shape and losses.dtype == torch.float32
+    close_loss(losses.detach().cpu().numpy(), want, "lsr")
+    assert (losses.detach().cpu().numpy()[y == ignore] == 0).all()
+    go = synth.normal(5, 3, y.shape, 0.0, 1.0)
+    losses.backward(dev(go))
+    close_grad(xt.grad.cpu().numpy(), oracle.lsr_backward(x, y, ignore, 0.1, go), "lsr")
+    g = xt.grad.cpu().numpy()
+    assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all()
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+@pytest.mark.parametrize("smooth", [0.0, 0.1, 0.4])
+def test_lsr_module_reductions(pl, reduction, smooth):
+    x, y = seg_inputs(22, (2, 19, 32, 32), 255, 0.05)
+    xt = dev(x).requires_grad_()
+    crit = pl.LabelSmoothSoftmaxCEV3(lb_smooth=smooth, reduction=reduction, ignore_index=255)
+    out = crit(xt, dev(y))
+    per = oracle.lsr_forward(x, y, 255, smooth)
+    want = oracle.reduce_pixels(per, y, reduction, 255)
+    close_loss(out.detach().cpu().numpy(), want, "lsr " + reduction)
+    (out.sum() if reduction == "none" else out).backward()
+    scale = 1.0 / (y != 255).sum() if reduction == "mean" else 1.0
+    want_g = oracle.lsr_backward(x, y, 255, smooth, np.float32(scale))
+    close_grad(xt.grad.cpu().numpy(), want_g, "lsr " + reduction)
+    valid_rows = xt.grad.sum(dim=1).cpu().numpy()
+    assert np.abs(valid_rows).max() < 1e-5 * max(1.0, 1.0 if reduction != "mean" else scale * 1e3)
+
+
+def test_lsr_all_ignored_mean_is_nan(pl):
+    x, y = seg_inputs(23, (2, 19, 8, 8), 255, 1.0)
+    out = pl.LabelSmoothSoftmaxCEV3(ignore_index=255)(dev(x), dev(y))
+    assert torch.isnan(out).item()
+
+
+def test_lsr_default_ignore_index_and_noncontiguous(pl):
+    x, y = seg_inputs(24, (2, 8, 8, 19), -100, 0.1)      # channels-last storage
+    xt = dev(x).permute(0, 3, 1, 2)                       # logical (2, 19, 8, 8), non-contiguous
+    y = y[..., 0] % 19
+    y[0, 0, :3] = -100
+    out = pl.LabelSmoothSoftmaxCEV3()(xt, dev(y))
+    per = oracle.lsr_forward(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), y, -100, 0.1)
+    close_loss(out.item(), oracle.reduce_pixels(per, y, "mean", -100), "lsr nc")
+
+
+# ---------------------------------------------------------------- focal ----
+
+FOCAL_SHAPES = [(2, 8, 16, 16), (17, 3, 15, 13), (5,), (1, 1, 1, 3), (3, 1025)]
+
+
+@pytest.mark.parametrize("shape", FOCAL_SHAPES)
+@pytest.mark.parametrize("alpha,gamma", [(0.25, 2), (0.5, 1), (0.75, 3.0), (0.3, 0.5), (0.25, 2.5), (0.25, 0)])
+@pytest.mark.parametrize("soft", [False, True])
+def test_focal_functions_match_oracle(pl, shape, alpha, gamma, soft):
+    x = synth.normal(31, 1, shape, -2.0, 1.5)
+    if soft:
+        y = synth.uniform01(31, 2, int(np.prod(shape))).reshape(shape).astype(np.float32)
+    else:
+        y = synth.bernoulli(31, 2, shape, 0.2).astype(np.float32)
+    want_l = oracle.focal_forward(x, y, alpha, gamma)
+    go = synth.normal(6, 3, shape, 0.0, 1.0)
+    want_g = oracle.focal_backward(x, y, alpha, gamma, go)
+    for fn in (pl.FocalSigmoidLossFuncV3, pl.FocalSigmoidLossFuncV3FB):
+        xt = dev(x).requires_grad_()
+        loss = fn.apply(xt, dev(y), alpha, gamma)
+        got = loss.detach().cpu().numpy()
+        assert np.abs(got - want_l).max() <= 1e-5 * max(1.0, np.abs(want_l).max()), fn.__name__
+        close_loss(got, want_l, fn.__name__)
+        loss.backward(dev(go))
+        close_grad(xt.grad.cpu().numpy(), want_g, fn.__name__)
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+def test_focal_module_reductions(pl, reduction):
+    w = synth.workload("cfg3", scale=0.25, batch=2)
+    x, y = w["logits"], w["labels"]
+    xt = dev(x).requires_grad_()
+    out = pl.FocalLossV3(alpha=0.25, gamma=2, reduction=reduction)(xt, dev(y))
+    per = oracle.focal_forward(x.astype(np.float64), y.astype(np.float64), 0.25, 2.0)
+    close_loss(out.detach().cpu().numpy(), oracle.reduce_all(per, reduction), "focal " + reduction)
+    (out.sum() if reduction == "none" else out).backward()
+    scale = 1.0 / x.size if reduction == "mean" else 1.0
+    close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, 0.25, 2.0, np.float32(scale)), "focal " + reduction)
+
+
+def test_focal_extreme_logits_stay_finite(pl):
+    x = np.array([-120.0, -90.0, -60.0, -30.0, 0.0, 30.0, 60.0, 90.0, 120.0] * 2, dtype=np.float32)
+    y = np.array([0.0] * 9 + [1.0] * 9, dtype=np.float32)
+    xt = dev(x).requires_grad_()
+    loss = pl.FocalSigmoidLossFuncV3.apply(xt, dev(y), 0.25, 2)
+    loss.sum().backward()
+    got, g = loss.detach().cpu().numpy(), xt.grad.cpu().numpy()
+    assert np.isfinite(got).all() and np.isfinite(g).all()
+    close_loss(got, oracle.focal_forward(x.astype(np.float64), y.astype(np.float64), 0.25, 2.0), "focal extreme")
+
+
+# -------------------------------------------------------------- lmargin ----
+
+@pytest.mark.parametrize("shape,ignore,frac", SEG_CASES)
+@pytest.mark.parametrize("fb", [False, True])
+def test_lmargin_functions_match_oracle(pl, shape, ignore, frac, fb):
+    if shape[1] < 2:
+        pytest.skip("needs at least two classes")
+    x, y = seg_inputs(41, shape, ignore, frac)
+    xt = dev(x).requires_grad_()
+    yt = dev(y)
+    if fb:
+        losses, cnt = pl.LargeMarginSoftmaxFuncV3FB.apply(xt, yt, 0.3, ignore)
+        assert cnt.dtype == torch.int64 and cnt.item() == int((y != ignore).sum())
+    else:
+        losses = pl.LargeMarginSoftmaxFuncV3.apply(xt, yt, 0.3, ignore)
+    want = oracle.lmargin_forward(x, y, 0.3, ignore)
+    close_loss(losses.detach().cpu().numpy(), want, "lmargin")
+    assert (losses.detach().cpu().numpy()[y == ignore] == 0).all()
+    go = synth.normal(7, 3, y.shape, 0.0, 1.0)
+    losses.backward(dev(go))
+    g = xt.grad.cpu().numpy()
+    close_grad(g, oracle.lmargin_backward(x, y, 0.3, ignore, go), "lmargin")
+    assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all()
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+@pytest.mark.parametrize("fb", [False, True])
+@pytest.mark.parametrize("lam", [0.0, 0.3, 1.0])
+def test_lmargin_module_reductions(pl, reduction, fb, lam):
+    x, y = seg_inputs(42, (2, 19, 32, 32), 255, 0.05)
+    xt = dev(x).requires_grad_()
+    out = pl.LargeMarginSoftmaxV3(lam=lam, reduction=reduction, ignore_index=255, fb=fb)(xt, dev(y))
+    per = oracle.lmargin_forward(x, y, lam, 255)
+    close_loss(out.detach().cpu().numpy(), oracle.reduce_pixels(per, y, reduction, 255), "lmargin " + reduction)
+    (out.sum() if reduction == "none" else out).backward()
+    scale = 1.0 / (y != 255).sum() if reduction == "mean" else 1.0
+    close_grad(xt.grad.cpu().numpy(), oracle.lmargin_backward(x, y, lam, 255, np.float32(scale)), "lmargin")
+
+
+def test_lmargin_dominant_target_stays_finite(pl):
+    x = np.zeros((1, 4, 1, 4), dtype=np.float32)
+    x[0, 2] = 200.0
+    x[0, 0, 0, 1] = -150.0
+    y = np.full((1, 1, 4), 2, dtype=np.int64)
+    for fb in (False, True):
+        xt = dev(x).requires_grad_()
+        out = pl.LargeMarginSoftmaxV3(reduction="none", fb=fb)(xt, dev(y))
+        out.sum().backward()
+        assert torch.isfinite(out).all() and torch.isfinite(xt.grad).all()
+        close_loss(out.detach().cpu().numpy(), oracle.lmargin_forward(x.astype(np.float64), y, 0.3, 255), "dominant")
+
+
+# --------------------------------------------------------------- lovasz ----
+
+LOVASZ_CASES = [
+    ((2, 19, 64, 64), 255, 0.05),
+    ((2, 19, 7, 9), 255, 0.1),
+    ((3, 2, 5, 8), -100, 0.2),
+    ((1, 4, 70, 64), 255, 0.0),       # a little over one sort tile per class
+    ((2, 5, 100, 100), 255, 0.3),     # several tiles, last one ragged
+    ((37, 10), -100, 0.1),
+    ((2, 33, 6, 7), 255, 0.2),
+    ((2, 227, 5, 5), 255, 0.1),
+    ((1, 8, 4, 4), 0, 0.3),
+    ((2, 19, 16, 16), 255, 1.0),
+]
+
+
+@pytest.mark.parametrize("shape,ignore,frac", LOVASZ_CASES)
+def test_lovasz_function_matches_oracle(pl, shape, ignore, frac):
+    x, y = seg_inputs(51, shape, ignore, frac)
+    xt = dev(x).requires_grad_()
+    losses = pl.LovaszSoftmaxFunctionV3.apply(xt, dev(y), ignore)
+    want, want_jacc = oracle.lovasz_forward(x.astype(np.float64), y, ignore)
+    assert losses.shape == (shape[1],)
+    got = losses.detach().cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-5 * max(1e-30, np.abs(want).max()), np.abs(got - want).max()
+    w = synth.normal(8, 3, (shape[1],), 0.5, 1.0)
+    losses.backward(dev(w))
+    g = xt.grad.cpu().numpy()
+    want_g = oracle.lovasz_backward(w.astype(np.float64), x.astype(np.float64), y, want_jacc, ignore)
+    assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all()
+    # near-ties may be ordered differently in fp32 and fp64; that moves single Jaccard
+    # differences between neighbouring pixels, bounded by the largest difference in the class
+    err = np.abs(g - want_g)
+    assert np.median(err) <= 1e-6
+    assert err.max() <= max(GRAD_ATOL, 2.0 * np.abs(want_jacc).max() * np.abs(w).max() * 1e-3), err.max()
+
+
+def test_lovasz_jacc_is_exact_for_the_computed_order(pl):
+    """Sort, scan and Jaccard differences are integer/rank work: given the fp32 errors the GPU
+    itself computed, the saved differences must equal the fp32 CPU restatement bit for bit."""
+    from pytorch_loss import _native
+    x, y = seg_inputs(52, (2, 5, 100, 100), 255, 0.2)
+    losses, jacc = _native.lovasz_forward(dev(x), dev(y), 255)
+    jacc = jacc.cpu().numpy()
+    l32, j32 = oracle.lovasz_forward(x, y, 255)
+    same = (jacc.view(np.uint32) == j32.view(np.uint32)).mean()
+    assert same > 0.995, same                       # the rest: 1-ulp differences in expf reorder near-ties
+    assert (jacc[:, y.reshape(-1) == 255] == 0).all()
+    np.testing.assert_allclose(jacc.sum(axis=1), 1.0, rtol=1e-4)
+    np.testing.assert_allclose(losses.cpu().numpy(), l32, rtol=1e-5)
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+def test_lovasz_module_reductions(pl, reduction):
+    w = synth.workload("cfg5", scale=1 / 16, batch=2)
+    x, y = w["logits"], w["labels"]
+    xt = dev(x).requires_grad_()
+    out = pl.LovaszSoftmaxV3(reduction=reduction, ignore_index=255)(xt, dev(y))
+    per, jacc = oracle.lovasz_forward(x.astype(np.float64), y, 255)
+    want = oracle.reduce_all(per, reduction)
+    got = out.detach().cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    (out.sum() if reduction == "none" else out).backward()
+    scale = 1.0 / 19 if reduction == "mean" else 1.0
+    want_g = oracle.lovasz_backward(np.full(19, scale), x.astype(np.float64), y, jacc, 255)
+    err = np.abs(xt.grad.cpu().numpy() - want_g)
+    assert err.max() <= GRAD_ATOL and np.median(err) <= 1e-7
+
+
+def test_lovasz_limits_raise(pl):
+    x = torch.zeros(1, 512, 2, 2, device="cuda")
+    y = torch.zeros(1, 2, 2, dtype=torch.long, device="cuda")
+    with pytest.raises(RuntimeError, match="num of classes"):
+        pl.LovaszSoftmaxV3()(x, y)
+
+
+# ------------------------------------------------ shared surface behaviour ----
+
+def test_empty_inputs_return_empty(pl):
+    x = torch.zeros(0, 19, 4, 4, device="cuda", requires_grad=True)
+    y = torch.zeros(0, 4, 4, dtype=torch.long, device="cuda")
+    assert pl.LSRCrossEntropyFunctionV3.apply(x, y, 0.1, 255).numel() == 0
+    assert pl.LargeMarginSoftmaxFuncV3.apply(x, y, 0.3, 255).numel() == 0
+    assert pl.FocalSigmoidLossFuncV3.apply(x, x.detach(), 0.25, 2).numel() == 0
+
+
+def test_half_and_double_inputs_are_computed_in_fp32(pl):
+    x, y = seg_inputs(61, (2, 19, 8, 8), 255, 0.1)
+    for dt in (torch.float16, torch.bfloat16, torch.float64):
+        xt = dev(x).to(dt).requires_grad_()
+        out = pl.LabelSmoothSoftmaxCEV3(ignore_index=255)(xt, dev(y))
+        out.backward()
+        assert xt.grad.dtype == dt and out.dtype == dt
+        xr = xt.detach().float().cpu().numpy()
+        per = oracle.lsr_forward(xr, y, 255, 0.1)
+        assert abs(out.item() - oracle.reduce_pixels(per, y, "mean", 255)) < 2e-2
+
+
+def test_autocast_casts_to_fp32(pl):
+    x, y = seg_inputs(62, (2, 19, 8, 8), 255, 0.1)
+    xt = dev(x).half().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = pl.LabelSmoothSoftmaxCEV3(ignore_index=255)(xt, dev(y))
+    assert out.dtype == torch.float32
+    out.backward()
+    assert xt.grad.dtype == torch.float16
+
+
+def test_runs_on_a_side_stream(pl):
+    x, y = seg_inputs(63, (2, 19, 64, 64), 255, 0.05)
+    xt, yt = dev(x), dev(y)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        out = pl.LSRCrossEntropyFunctionV3.apply(xt, yt, 0.1, 255)
+    side.synchronize()
+    close_loss(out.cpu().numpy(), oracle.lsr_forward(x, y, 255, 0.1), "side stream")
