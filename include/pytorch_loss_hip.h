@@ -65,6 +65,31 @@ int plh_lsr_backward(const float *logits, const int64_t *labels,
                      int64_t n_size, int64_t dimsize, int64_t m_size,
                      int64_t ignore_index, float smooth, void *stream);
 
+/* Module-level reduction fused into the forward (no counterpart in the reference's
+ * extension, which leaves `losses.sum()` and `(labels != ignore).sum()` to ATen,
+ * pytorch_loss/label_smooth.py:165-170).  The forward kernel leaves per-block partial
+ * sums/counts in `workspace`; a one-block kernel adds them in a fixed order.
+ *   losses      per-pixel losses, or NULL to skip writing them
+ *   loss_out    1 fp32: the sum (mean == 0) or sum / n_valid (mean != 0; 0/0 = NaN)
+ *   n_valid_out 1 int64: number of non-ignored pixels, or NULL
+ *   workspace   at least plh_reduce_workspace_bytes(n_size*m_size) bytes, 16-byte aligned
+ * plh_lsr_backward_scaled is the matching backward: the upstream gradient is the scalar
+ * grad_scalar[0] * scale / divide_by[0] (divide_by NULL = 1), all read on the device.
+ */
+int64_t plh_reduce_workspace_bytes(int64_t units);
+
+int plh_lsr_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+                            float *loss_out, int64_t *n_valid_out, int32_t mean,
+                            void *workspace, int64_t workspace_bytes,
+                            int64_t n_size, int64_t dimsize, int64_t m_size,
+                            int64_t ignore_index, float smooth, void *stream);
+
+int plh_lsr_backward_scaled(const float *logits, const int64_t *labels,
+                            const float *grad_scalar, float scale, const int64_t *divide_by,
+                            float *grad_logits,
+                            int64_t n_size, int64_t dimsize, int64_t m_size,
+                            int64_t ignore_index, float smooth, void *stream);
+
 /* ---- sigmoid focal loss -------------------------------------------------------
  * Replaces focal_cpp.focalloss_forward / focalloss_backward /
  * focalloss_forward_backward (csrc/focal_kernel.cu:301-335; kernels :29-164).
@@ -78,6 +103,18 @@ int plh_focal_backward(const float *logits, const float *labels,
                        const float *grad_output, int64_t grad_output_stride,
                        float *grad_logits,
                        int64_t numel, float gamma, float alpha, void *stream);
+
+/* Reduction fused into the forward, as for LSR (replaces `loss.mean()` / `loss.sum()` of
+ * focal_loss.py:196-199): loss_out = sum, or sum / numel when mean != 0; workspace of
+ * plh_reduce_workspace_bytes(numel) bytes. The matching backward takes the upstream
+ * gradient grad_scalar[0] * scale (scale = 1/numel for a mean). */
+int plh_focal_forward_reduced(const float *logits, const float *labels, float *losses,
+                              float *loss_out, int32_t mean, void *workspace, int64_t workspace_bytes,
+                              int64_t numel, float gamma, float alpha, void *stream);
+
+int plh_focal_backward_scaled(const float *logits, const float *labels,
+                              const float *grad_scalar, float scale, float *grad_logits,
+                              int64_t numel, float gamma, float alpha, void *stream);
 
 /* One pass producing both the losses and dloss/dlogits under a unit upstream gradient. */
 int plh_focal_forward_backward(const float *logits, const float *labels,
@@ -99,6 +136,20 @@ int plh_lmargin_backward(const float *logits, const int64_t *labels,
                          float *grad_logits,
                          int64_t n_size, int64_t dimsize, int64_t m_size,
                          int64_t ignore_index, float lam, void *stream);
+
+/* Reduction fused into the forward and the matching backward, as for LSR
+ * (replaces large_margin_softmax.py:169-173 of the packaged copy). */
+int plh_lmargin_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+                                float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                void *workspace, int64_t workspace_bytes,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t ignore_index, float lam, void *stream);
+
+int plh_lmargin_backward_scaled(const float *logits, const int64_t *labels,
+                                const float *grad_scalar, float scale, const int64_t *divide_by,
+                                float *grad_logits,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t ignore_index, float lam, void *stream);
 
 int plh_lmargin_forward_backward(const float *logits, const int64_t *labels,
                                  float *losses, float *grad_logits, int64_t *valid_cnt,

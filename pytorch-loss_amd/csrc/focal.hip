@@ -50,100 +50,155 @@ __device__ __forceinline__ void focal_point(float x, float y, const FocalParams 
     }
 }
 
-// One float4 per thread. gout: nullptr = 1, gstride 0 = broadcast scalar, 1 = per element.
-template <int Mode, bool WantLoss, bool WantGrad>
-__global__ __launch_bounds__(256) void focal_vec4(const float4 *__restrict__ x4, const float4 *__restrict__ y4,
-                                                  const float *__restrict__ gout, int64_t gstride,
-                                                  float4 *__restrict__ loss4, float4 *__restrict__ grad4,
+// One float4 per thread. Reduce: also leave the block's sum of losses in part.sum[slot0 + block].
+template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
+__global__ __launch_bounds__(256) void focal_vec4(const float *__restrict__ x, const float *__restrict__ y,
+                                                  const Upstream up, float *__restrict__ loss,
+                                                  float *__restrict__ grad, float *__restrict__ partial,
                                                   int64_t n4, const FocalParams p) {
+    __shared__ float red[4];
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n4) return;
-    const float4 xv = x4[i];
-    const float4 yv = y4[i];
-    float go[4];
-    if constexpr (WantGrad) load_gout<4>(gout, gstride, i * 4, go);
-    const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
-    const float ys[4] = {yv.x, yv.y, yv.z, yv.w};
-    float l[4], g[4];
+    const bool live = i < n4;
+    if (!Reduce && !live) return;
+    const int64_t at = live ? i * 4 : 0;
+    float xs[4], ys[4], go[4], l[4], g[4];
+    load_vec<4>(x + at, xs);
+    load_vec<4>(y + at, ys);
+    if constexpr (WantGrad) load_upstream<4>(up, at, go);
+    float mine = 0.f;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        focal_point<Mode, WantLoss, WantGrad>(xs[k], ys[k], p, l[k], g[k]);
+        focal_point<Mode, WantLoss || Reduce, WantGrad>(xs[k], ys[k], p, l[k], g[k]);
         if constexpr (WantGrad) g[k] *= go[k];
+        if constexpr (Reduce) mine += live ? l[k] : 0.f;
     }
-    if constexpr (WantLoss) loss4[i] = make_float4(l[0], l[1], l[2], l[3]);
-    if constexpr (WantGrad) grad4[i] = make_float4(g[0], g[1], g[2], g[3]);
+    if (live) {
+        if (WantLoss && loss) store_vec<4>(loss + at, l);
+        if constexpr (WantGrad) store_vec<4>(grad + at, g);
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        if (threadIdx.x == 0) partial[blockIdx.x] = bs;
+    }
 }
 
-template <int Mode, bool WantLoss, bool WantGrad>
+template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
 __global__ __launch_bounds__(256) void focal_scalar(const float *__restrict__ x, const float *__restrict__ y,
-                                                    const float *__restrict__ gout, int64_t gstride,
-                                                    float *__restrict__ loss, float *__restrict__ grad,
+                                                    const Upstream up, float *__restrict__ loss,
+                                                    float *__restrict__ grad, float *__restrict__ partial,
                                                     int64_t first, int64_t numel, const FocalParams p) {
+    __shared__ float red[4];
     const int64_t i = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= numel) return;
-    float l, g;
-    focal_point<Mode, WantLoss, WantGrad>(x[i], y[i], p, l, g);
-    if constexpr (WantLoss) loss[i] = l;
-    if constexpr (WantGrad) {
-        float go[1];
-        load_gout<1>(gout, gstride, i, go);
-        grad[i] = g * go[0];
+    const bool live = i < numel;
+    if (!Reduce && !live) return;
+    const int64_t at = live ? i : first;
+    float l = 0.f, g = 0.f;
+    focal_point<Mode, WantLoss || Reduce, WantGrad>(x[at], y[at], p, l, g);
+    if (live) {
+        if (WantLoss && loss) loss[at] = l;
+        if constexpr (WantGrad) {
+            float go[1];
+            load_upstream<1>(up, at, go);
+            grad[at] = g * go[0];
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(live ? l : 0.f, red);
+        if (threadIdx.x == 0) partial[blockIdx.x] = bs;
     }
 }
 
-template <int Mode, bool WantLoss, bool WantGrad>
-static void launch_mode(const float *x, const float *y, const float *gout, int64_t gstride, float *loss,
-                        float *grad, int64_t numel, const FocalParams &p, hipStream_t st) {
+// Returns the number of partial slots written (0 unless Reduce).
+template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
+static unsigned launch_mode(const float *x, const float *y, const Upstream &up, float *loss, float *grad,
+                            float *partial, int64_t numel, const FocalParams &p, hipStream_t st) {
     int64_t done = 0;
-    const bool aligned = !misaligned(x, 16) && !misaligned(y, 16) && !(WantLoss && misaligned(loss, 16)) &&
+    unsigned slots = 0;
+    const bool aligned = !misaligned(x, 16) && !misaligned(y, 16) && !(loss && misaligned(loss, 16)) &&
                          !(WantGrad && misaligned(grad, 16)) &&
-                         !(WantGrad && gout && gstride == 1 && misaligned(gout, 16));
+                         !(WantGrad && up.gout && up.stride == 1 && misaligned(up.gout, 16));
     if (aligned && numel >= 4) {
         const int64_t n4 = numel / 4;
-        hipLaunchKernelGGL((focal_vec4<Mode, WantLoss, WantGrad>), dim3((unsigned)ceil_div(n4, 256)), dim3(256), 0, st,
-                           reinterpret_cast<const float4 *>(x), reinterpret_cast<const float4 *>(y), gout, gstride,
-                           reinterpret_cast<float4 *>(loss), reinterpret_cast<float4 *>(grad), n4, p);
+        const unsigned grid = (unsigned)ceil_div(n4, 256);
+        hipLaunchKernelGGL((focal_vec4<Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
+                           loss, grad, partial, n4, p);
         done = n4 * 4;
+        slots = grid;
     }
     if (done < numel) {
-        hipLaunchKernelGGL((focal_scalar<Mode, WantLoss, WantGrad>), dim3((unsigned)ceil_div(numel - done, 256)),
-                           dim3(256), 0, st, x, y, gout, gstride, loss, grad, done, numel, p);
+        const unsigned grid = (unsigned)ceil_div(numel - done, 256);
+        hipLaunchKernelGGL((focal_scalar<Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
+                           loss, grad, Reduce ? partial + slots : nullptr, done, numel, p);
+        slots += grid;
     }
+    return Reduce ? slots : 0;
 }
 
-template <bool WantLoss, bool WantGrad>
-static int launch(const float *x, const float *y, const float *gout, int64_t gstride, float *loss, float *grad,
-                  int64_t numel, float gamma, float alpha, void *stream) {
+template <bool WantLoss, bool WantGrad, bool Reduce>
+static int launch(const float *x, const float *y, const Upstream &up, float *loss, float *grad, float *partial,
+                  unsigned *slots_out, int64_t numel, float gamma, float alpha, void *stream) {
+    if (slots_out) *slots_out = 0;
     if (numel < 0 || numel > kMaxNumel) return PLH_ERR_BAD_SIZE;
     if (numel == 0) return PLH_OK;
-    if (!x || !y || (WantLoss && !loss) || (WantGrad && !grad)) return PLH_ERR_NULL_POINTER;
+    if (!x || !y || (WantLoss && !Reduce && !loss) || (WantGrad && !grad)) return PLH_ERR_NULL_POINTER;
     if (misaligned(x, 4) || misaligned(y, 4) || misaligned(loss, 4) || misaligned(grad, 4)) return PLH_ERR_MISALIGNED;
-    const int rc = check_gout(gout, gstride);
-    if (rc != PLH_OK) return rc;
     const FocalParams p{gamma, alpha};
     hipStream_t st = (hipStream_t)stream;
-    if (gamma == 2.f) launch_mode<kGammaTwo, WantLoss, WantGrad>(x, y, gout, gstride, loss, grad, numel, p, st);
-    else if (gamma == 1.f) launch_mode<kGammaOne, WantLoss, WantGrad>(x, y, gout, gstride, loss, grad, numel, p, st);
-    else launch_mode<kGammaAny, WantLoss, WantGrad>(x, y, gout, gstride, loss, grad, numel, p, st);
+    unsigned slots;
+    if (gamma == 2.f) slots = launch_mode<kGammaTwo, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
+    else if (gamma == 1.f) slots = launch_mode<kGammaOne, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
+    else slots = launch_mode<kGammaAny, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
+    if (slots_out) *slots_out = slots;
     return check_launch();
 }
 
 }  // namespace plh
 
+using namespace plh;
+
 extern "C" int plh_focal_forward(const float *logits, const float *labels, float *losses,
                                  int64_t numel, float gamma, float alpha, void *stream) {
-    return plh::launch<true, false>(logits, labels, nullptr, 0, losses, nullptr, numel, gamma, alpha, stream);
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    return launch<true, false, false>(logits, labels, up, losses, nullptr, nullptr, nullptr, numel, gamma, alpha, stream);
+}
+
+extern "C" int plh_focal_forward_reduced(const float *logits, const float *labels, float *losses,
+                                         float *loss_out, int32_t mean, void *workspace, int64_t workspace_bytes,
+                                         int64_t numel, float gamma, float alpha, void *stream) {
+    if (numel < 0 || numel > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    Partials part;
+    int rc = carve_partials(workspace, workspace_bytes, numel, loss_out, nullptr, part);
+    if (rc != PLH_OK) return rc;
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    unsigned slots = 0;
+    rc = launch<true, false, true>(logits, labels, up, losses, nullptr, part.sum, &slots, numel, gamma, alpha, stream);
+    if (rc != PLH_OK) return rc;
+    part.cnt = nullptr;
+    finish_partials(part, slots, loss_out, nullptr, mean ? kFinishMeanOverFixed : kFinishSum, numel, (hipStream_t)stream);
+    return check_launch();
 }
 
 extern "C" int plh_focal_backward(const float *logits, const float *labels,
                                   const float *grad_output, int64_t grad_output_stride, float *grad_logits,
                                   int64_t numel, float gamma, float alpha, void *stream) {
-    return plh::launch<false, true>(logits, labels, grad_output, grad_output_stride, nullptr, grad_logits, numel,
-                                    gamma, alpha, stream);
+    const int rc = check_gout(grad_output, grad_output_stride);
+    if (rc != PLH_OK) return rc;
+    const Upstream up{grad_output, grad_output_stride, nullptr, 1.f};
+    return launch<false, true, false>(logits, labels, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
+}
+
+extern "C" int plh_focal_backward_scaled(const float *logits, const float *labels,
+                                         const float *grad_scalar, float scale, float *grad_logits,
+                                         int64_t numel, float gamma, float alpha, void *stream) {
+    if (numel > 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, nullptr, scale};
+    return launch<false, true, false>(logits, labels, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
 }
 
 extern "C" int plh_focal_forward_backward(const float *logits, const float *labels, float *losses,
                                           float *grad_logits, int64_t numel, float gamma, float alpha,
                                           void *stream) {
-    return plh::launch<true, true>(logits, labels, nullptr, 0, losses, grad_logits, numel, gamma, alpha, stream);
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    return launch<true, true, false>(logits, labels, up, losses, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
 }

@@ -26,13 +26,17 @@ struct LmParams {
 
 // ---------------------------------------------------------------- regs ----
 
-template <int CP, int V, bool WantLoss, bool WantGrad, bool WantCount>
-__global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
-                                               const float *__restrict__ gout, int64_t gstride,
-                                               float *__restrict__ loss, float *__restrict__ grad,
-                                               unsigned long long *__restrict__ valid_cnt, const LmParams p) {
-    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
-    if (pix >= p.P) return;
+template <int CP, int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+__global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
+                                                     const Upstream up,
+                                                     float *__restrict__ loss, float *__restrict__ grad,
+                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
+                                                     const LmParams p) {
+    __shared__ float red[4];
+    const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+    const bool live = want < p.P;
+    if (!Reduce && !live) return;
+    const int64_t pix = live ? want : 0;
     const int64_t n = pix / p.m_size;
     const int64_t base = pix + n * (int64_t)(p.C - 1) * p.m_size;
     const float *xs = x + base;
@@ -44,10 +48,12 @@ __global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, cons
     int64_t lb[V];
     load_labels<V>(lab + pix, lb);
     float go[V];
-    if constexpr (WantGrad) load_gout<V>(gout, gstride, pix, go);
+    if constexpr (WantGrad) load_upstream<V>(up, pix, go);
 
     float out[V];
     unsigned n_valid = 0;
+    float mine = 0.f;
+    int cnt = 0;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         const bool ign = (lb[k] == p.ignore);
@@ -64,12 +70,12 @@ __global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, cons
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
-                const float e = (lb[k] == j) ? 0.f : expf(v[j][k] - m_no);
+                const float e = (lb[k] == j) ? 0.f : fast_exp(v[j][k] - m_no);
                 s_no += e;
                 if constexpr (WantGrad) sum_ex += e * v[j][k];
             }
-        const float t = expf(m_no - m_all);
-        const float e_y = expf(x_y - m_all);
+        const float t = fast_exp(m_no - m_all);
+        const float e_y = fast_exp(x_y - m_all);
         const float s_all = s_no * t + e_y;
         const float inv_no = 1.f / s_no;
         const float inv_all = 1.f / s_all;
@@ -81,7 +87,7 @@ __global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, cons
             if (j < p.C) {
                 const bool hot = (lb[k] == j);
                 const float xv = v[j][k];
-                const float e = expf(xv - m_no);
+                const float e = fast_exp(xv - m_no);
                 const float q = e * inv_no;
                 if constexpr (WantLoss) {
                     const float term = p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
@@ -96,20 +102,32 @@ __global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, cons
             }
         if constexpr (WantLoss) {
             acc += -(x_y - m_all) + logf(s_all);
-            out[k] = ign ? 0.f : acc;
+            out[k] = (ign || !live) ? 0.f : acc;
+            mine += out[k];
+            cnt += (ign || !live) ? 0 : 1;
         }
-        if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(!ign));
+        if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
     }
-    if constexpr (WantLoss) store_vec<V>(loss + pix, out);
-    if constexpr (WantGrad) {
-        float *gs = grad + base;
+    if (live) {
+        if (WantLoss && loss) store_vec<V>(loss + pix, out);
+        if constexpr (WantGrad) {
+            float *gs = grad + base;
 #pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (j < p.C) store_vec<V>(gs + (int64_t)j * p.m_size, v[j]);
+            for (int j = 0; j < CP; ++j)
+                if (j < p.C) store_vec<V>(gs + (int64_t)j * p.m_size, v[j]);
+        }
     }
     if constexpr (WantCount) {
         // lanes leave only at the tail of the grid, so lane 0 of a wave with work is alive
         if ((threadIdx.x & 63) == 0) atomicAdd(valid_cnt, (unsigned long long)n_valid);
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256((float)cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
     }
 }
 
@@ -117,13 +135,16 @@ __global__ __launch_bounds__(256) void lm_regs(const float *__restrict__ x, cons
 
 constexpr int kLmStageCap = 2048;
 
-template <int G, bool WantLoss, bool WantGrad, bool WantCount>
+template <int G, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, const int64_t *__restrict__ lab,
-                                                const float *__restrict__ gout, int64_t gstride,
+                                                const Upstream up,
                                                 float *__restrict__ loss, float *__restrict__ grad,
-                                                unsigned long long *__restrict__ valid_cnt, const LmParams p) {
+                                                unsigned long long *__restrict__ valid_cnt, Partials part,
+                                                const LmParams p) {
     constexpr int kPix = 256 / G;
     __shared__ float stage_mem[(G == 64) ? 4 * kLmStageCap : 1];
+    __shared__ float red[4];
+    float mine = 0.f, cnt = 0.f;
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
     float *stage = stage_mem + ((G == 64) ? grp * kLmStageCap : 0);
@@ -141,7 +162,7 @@ __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, con
         const int64_t lb = lab[pc];
         const bool ign = (lb == p.ignore);
         float go[1] = {1.f};
-        if constexpr (WantGrad) load_gout<1>(gout, gstride, pc, go);
+        if constexpr (WantGrad) load_upstream<1>(up, pc, go);
 
         float m_no = -INFINITY, x_y = -INFINITY;
         for (int j = sub; j < p.C; j += G) {
@@ -155,14 +176,14 @@ __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, con
         float s_no = 0.f, sum_ex = 0.f;
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : xs[(int64_t)j * p.m_size];
-            const float e = (lb == j) ? 0.f : expf(t - m_no);
+            const float e = (lb == j) ? 0.f : fast_exp(t - m_no);
             s_no += e;
             sum_ex += e * t;
         }
         s_no = group_reduce<G>(s_no, OpSum());
         sum_ex = group_reduce<G>(sum_ex, OpSum());
-        const float t_all = expf(m_no - m_all);
-        const float e_y = expf(x_y - m_all);
+        const float t_all = fast_exp(m_no - m_all);
+        const float e_y = fast_exp(x_y - m_all);
         const float s_all = s_no * t_all + e_y;
         const float inv_no = 1.f / s_no, inv_all = 1.f / s_all;
         const float sum_qx = sum_ex * inv_no;
@@ -171,7 +192,7 @@ __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, con
         for (int j = sub; j < p.C; j += G) {
             const float xv = staged ? stage[j] : xs[(int64_t)j * p.m_size];
             const bool hot = (lb == j);
-            const float e = expf(xv - m_no);
+            const float e = fast_exp(xv - m_no);
             const float q = e * inv_no;
             if constexpr (WantLoss) acc += hot ? 0.f : p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
             if constexpr (WantGrad) {
@@ -183,7 +204,11 @@ __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, con
         if constexpr (WantLoss) {
             acc = group_reduce<G>(acc, OpSum());
             acc += -(x_y - m_all) + logf(s_all);
-            if (live && sub == 0) loss[pix] = ign ? 0.f : acc;
+            if (live && sub == 0) {
+                if (loss) loss[pix] = ign ? 0.f : acc;
+                mine += ign ? 0.f : acc;
+                cnt += ign ? 0.f : 1.f;
+            }
         }
         // every lane of the wave is inside the loop, so the ballot sees the whole wave
         if constexpr (WantCount)
@@ -192,41 +217,53 @@ __global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, con
     if constexpr (WantCount) {
         if ((threadIdx.x & 63) == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
 }
 
 __global__ void lm_zero_count(unsigned long long *cnt) { *cnt = 0; }
 
 // ------------------------------------------------------------ dispatch ----
 
-template <int V, bool WantLoss, bool WantGrad, bool WantCount>
-static void launch_regs(const float *x, const int64_t *lab, const float *gout, int64_t gstride, float *loss,
-                        float *grad, unsigned long long *cnt, const LmParams &p, hipStream_t st) {
-    const unsigned grid = (unsigned)ceil_div(ceil_div(p.P, V), 256);
+template <int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+static unsigned launch_regs(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
+                            unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
+    const unsigned grid = regs_grid<V>(p.P);
     switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                                                                                          \
-    case K:                                                                                                  \
-        hipLaunchKernelGGL((lm_regs<4 * K, V, WantLoss, WantGrad, WantCount>), dim3(grid), dim3(256), 0, st, \
-                           x, lab, gout, gstride, loss, grad, cnt, p);                                       \
+#define PLH_CASE(K)                                                                                              \
+    case K:                                                                                                      \
+        hipLaunchKernelGGL((lm_regs<4 * K, V, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), dim3(kRegsBlock), \
+                           0, st, x, lab, up, loss, grad, cnt, part, p);                                         \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
+    return grid;
 }
 
-template <bool WantLoss, bool WantGrad, bool WantCount>
-static int launch(const float *x, const int64_t *lab, const float *gout, int64_t gstride, float *loss, float *grad,
-                  int64_t *valid_cnt, int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float lam,
-                  void *stream) {
-    int rc = check_slice_args(x, lab, WantLoss ? (const void *)loss : (const void *)grad, n_size, dimsize, m_size);
+// Launches one direction (or the fused pair). blocks_out: blocks that wrote partials (Reduce only).
+template <bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+static int launch(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
+                  int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
+                  int64_t m_size, int64_t ignore, float lam, void *stream) {
+    if (blocks_out) *blocks_out = 0;
+    const void *out = (WantLoss && !Reduce) ? (const void *)loss : (WantGrad ? (const void *)grad : (const void *)x);
+    int rc = check_slice_args(x, lab, out, n_size, dimsize, m_size);
     if (rc != PLH_OK) return rc;
-    rc = check_gout(gout, gstride);
-    if (rc != PLH_OK) return rc;
+    if (up.gout && up.stride == 1 && misaligned(up.gout, 4)) return PLH_ERR_MISALIGNED;
     if (WantCount && (!valid_cnt || misaligned(valid_cnt, 8))) return valid_cnt ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
     hipStream_t st = (hipStream_t)stream;
     unsigned long long *cnt = reinterpret_cast<unsigned long long *>(valid_cnt);
     if (WantCount) hipLaunchKernelGGL(lm_zero_count, dim3(1), dim3(1), 0, st, cnt);
     if (n_size * dimsize * m_size == 0) return check_launch();
     if (WantLoss && WantGrad && (!grad || misaligned(grad, 4))) return grad ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
+    if (loss && misaligned(loss, 4)) return PLH_ERR_MISALIGNED;
 
     LmParams p;
     p.P = n_size * m_size;
@@ -235,43 +272,91 @@ static int launch(const float *x, const int64_t *lab, const float *gout, int64_t
     p.ignore = ignore;
     p.half_lam = lam / 2.f;                          // csrc/large_margin_kernel.cu:188
     p.coeff = 1.f / (float)(dimsize - 1);            // csrc/large_margin_kernel.cu:404
-    const float *go_vec = (gout && gstride == 1) ? gout : nullptr;
+    const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    unsigned blocks = 0;
     switch (pick_shape(dimsize, m_size, x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr, go_vec)) {
-        case Shape::Regs4: launch_regs<4, WantLoss, WantGrad, WantCount>(x, lab, gout, gstride, loss, grad, cnt, p, st); break;
-        case Shape::Regs1: launch_regs<1, WantLoss, WantGrad, WantCount>(x, lab, gout, gstride, loss, grad, cnt, p, st); break;
+        case Shape::Regs2:
+            blocks = launch_regs<2, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+            break;
+        case Shape::Regs1:
+            blocks = launch_regs<1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+            break;
         case Shape::Wave:
-            hipLaunchKernelGGL((lm_group<64, WantLoss, WantGrad, WantCount>), dim3(group_grid(p.P, 4)), dim3(256), 0, st,
-                               x, lab, gout, gstride, loss, grad, cnt, p);
+            blocks = group_grid(p.P, 4);
+            hipLaunchKernelGGL((lm_group<64, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
+                               x, lab, up, loss, grad, cnt, part, p);
             break;
         case Shape::Lane:
-            hipLaunchKernelGGL((lm_group<1, WantLoss, WantGrad, WantCount>), dim3(group_grid(p.P, 256)), dim3(256), 0, st,
-                               x, lab, gout, gstride, loss, grad, cnt, p);
+            blocks = group_grid(p.P, 256);
+            hipLaunchKernelGGL((lm_group<1, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
+                               x, lab, up, loss, grad, cnt, part, p);
             break;
     }
+    if (blocks_out) *blocks_out = blocks;
     return check_launch();
 }
 
 }  // namespace plh
 
+using namespace plh;
+
+static const Partials kNoPartials{nullptr, nullptr};
+
 extern "C" int plh_lmargin_forward(const float *logits, const int64_t *labels, float *losses,
                                    int64_t n_size, int64_t dimsize, int64_t m_size,
                                    int64_t ignore_index, float lam, void *stream) {
-    return plh::launch<true, false, false>(logits, labels, nullptr, 0, losses, nullptr, nullptr, n_size, dimsize,
-                                           m_size, ignore_index, lam, stream);
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    return launch<true, false, false, false>(logits, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr,
+                                             n_size, dimsize, m_size, ignore_index, lam, stream);
+}
+
+extern "C" int plh_lmargin_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+                                           float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                           void *workspace, int64_t workspace_bytes,
+                                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                                           int64_t ignore_index, float lam, void *stream) {
+    if (n_size < 0 || m_size < 0 || n_size > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    Partials part;
+    int rc = carve_partials(workspace, workspace_bytes, n_size * m_size, loss_out, n_valid_out, part);
+    if (rc != PLH_OK) return rc;
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    unsigned blocks = 0;
+    rc = launch<true, false, false, true>(logits, labels, up, losses, nullptr, nullptr, part, &blocks, n_size, dimsize,
+                                          m_size, ignore_index, lam, stream);
+    if (rc != PLH_OK) return rc;
+    finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0,
+                    (hipStream_t)stream);
+    return check_launch();
 }
 
 extern "C" int plh_lmargin_backward(const float *logits, const int64_t *labels,
                                     const float *grad_output, int64_t grad_output_stride, float *grad_logits,
                                     int64_t n_size, int64_t dimsize, int64_t m_size,
                                     int64_t ignore_index, float lam, void *stream) {
-    return plh::launch<false, true, false>(logits, labels, grad_output, grad_output_stride, nullptr, grad_logits,
-                                           nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
+    const int rc = check_gout(grad_output, grad_output_stride);
+    if (rc != PLH_OK) return rc;
+    const Upstream up{grad_output, grad_output_stride, nullptr, 1.f};
+    return launch<false, true, false, false>(logits, labels, up, nullptr, grad_logits, nullptr, kNoPartials, nullptr,
+                                             n_size, dimsize, m_size, ignore_index, lam, stream);
+}
+
+extern "C" int plh_lmargin_backward_scaled(const float *logits, const int64_t *labels,
+                                           const float *grad_scalar, float scale, const int64_t *divide_by,
+                                           float *grad_logits,
+                                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                                           int64_t ignore_index, float lam, void *stream) {
+    if (n_size * dimsize * m_size != 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale};
+    return launch<false, true, false, false>(logits, labels, up, nullptr, grad_logits, nullptr, kNoPartials, nullptr,
+                                             n_size, dimsize, m_size, ignore_index, lam, stream);
 }
 
 extern "C" int plh_lmargin_forward_backward(const float *logits, const int64_t *labels, float *losses,
                                             float *grad_logits, int64_t *valid_cnt,
                                             int64_t n_size, int64_t dimsize, int64_t m_size,
                                             int64_t ignore_index, float lam, void *stream) {
-    return plh::launch<true, true, true>(logits, labels, nullptr, 0, losses, grad_logits, valid_cnt, n_size,
-                                         dimsize, m_size, ignore_index, lam, stream);
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    return launch<true, true, true, false>(logits, labels, up, losses, grad_logits, valid_cnt, kNoPartials, nullptr,
+                                           n_size, dimsize, m_size, ignore_index, lam, stream);
 }

@@ -53,10 +53,10 @@ __device__ __forceinline__ float key_error(uint32_t key) {
 // ------------------------------------------------------ 1. build keys ----
 
 template <int CP, int V>
-__global__ __launch_bounds__(256) void lov_keys_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
-                                                     uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
-                                                     int64_t ignore) {
-    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+__global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
+                                                           uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
+                                                           int64_t ignore) {
+    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
     const int64_t n = pix / m_size;
     const float *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
@@ -412,11 +412,11 @@ __global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__
 // ------------------------------------------------------------ backward ----
 
 template <int CP, int V>
-__global__ __launch_bounds__(256) void lov_bwd_regs(const float *__restrict__ gout, const float *__restrict__ x,
-                                                    const int64_t *__restrict__ lab, const float *__restrict__ jacc,
-                                                    float *__restrict__ grad, int64_t P, int64_t m_size, int C,
-                                                    int64_t ignore) {
-    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+__global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restrict__ gout, const float *__restrict__ x,
+                                                          const int64_t *__restrict__ lab, const float *__restrict__ jacc,
+                                                          float *__restrict__ grad, int64_t P, int64_t m_size, int C,
+                                                          int64_t ignore) {
+    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
     const int64_t n = pix / m_size;
     const int64_t base = pix + n * (int64_t)(C - 1) * m_size;
@@ -556,16 +556,16 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
 
     // 1. keys
     const Shape shape = pick_shape(dimsize, m_size, logits, keys_a, labels, nullptr, nullptr);
-    if (shape == Shape::Regs4 || shape == Shape::Regs1) {
-        const int V = (shape == Shape::Regs4 && pl.P % 4 == 0) ? 4 : 1;
-        const unsigned grid = (unsigned)ceil_div(ceil_div(pl.P, V), 256);
+    if (shape == Shape::Regs2 || shape == Shape::Regs1) {
+        const int V = (shape == Shape::Regs2) ? 2 : 1;      // m_size even => P even => rows of [C][P] stay 8-byte aligned
+        const unsigned grid = (V == 2) ? regs_grid<2>(pl.P) : regs_grid<1>(pl.P);
         switch ((C + 3) / 4) {
-#define PLH_CASE(K)                                                                                              \
-    case K:                                                                                                      \
-        if (V == 4) hipLaunchKernelGGL((lov_keys_regs<4 * K, 4>), dim3(grid), dim3(256), 0, st, logits, labels,  \
-                                       keys_a, pl.P, m_size, C, ignore_index);                                   \
-        else hipLaunchKernelGGL((lov_keys_regs<4 * K, 1>), dim3(grid), dim3(256), 0, st, logits, labels, keys_a, \
-                                pl.P, m_size, C, ignore_index);                                                  \
+#define PLH_CASE(K)                                                                                                  \
+    case K:                                                                                                          \
+        if (V == 2) hipLaunchKernelGGL((lov_keys_regs<4 * K, 2>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels, \
+                                       keys_a, pl.P, m_size, C, ignore_index);                                       \
+        else hipLaunchKernelGGL((lov_keys_regs<4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels,      \
+                                keys_a, pl.P, m_size, C, ignore_index);                                              \
         break;
             PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -618,16 +618,16 @@ extern "C" int plh_lovasz_backward(const float *grad_output, const float *logits
     hipStream_t st = (hipStream_t)stream;
     const int C = (int)dimsize;
     const Shape shape = pick_shape(dimsize, m_size, logits, grad_logits, labels, jacc, nullptr);
-    if (shape == Shape::Regs4 || shape == Shape::Regs1) {
-        const int V = (shape == Shape::Regs4 && pl.P % 4 == 0) ? 4 : 1;
-        const unsigned grid = (unsigned)ceil_div(ceil_div(pl.P, V), 256);
+    if (shape == Shape::Regs2 || shape == Shape::Regs1) {
+        const int V = (shape == Shape::Regs2) ? 2 : 1;
+        const unsigned grid = (V == 2) ? regs_grid<2>(pl.P) : regs_grid<1>(pl.P);
         switch ((C + 3) / 4) {
-#define PLH_CASE(K)                                                                                               \
-    case K:                                                                                                       \
-        if (V == 4) hipLaunchKernelGGL((lov_bwd_regs<4 * K, 4>), dim3(grid), dim3(256), 0, st, grad_output,       \
-                                       logits, labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);         \
-        else hipLaunchKernelGGL((lov_bwd_regs<4 * K, 1>), dim3(grid), dim3(256), 0, st, grad_output, logits,      \
-                                labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);                        \
+#define PLH_CASE(K)                                                                                                   \
+    case K:                                                                                                           \
+        if (V == 2) hipLaunchKernelGGL((lov_bwd_regs<4 * K, 2>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output,    \
+                                       logits, labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);             \
+        else hipLaunchKernelGGL((lov_bwd_regs<4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output, logits,   \
+                                labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);                            \
         break;
             PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

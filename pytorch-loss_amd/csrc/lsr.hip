@@ -9,6 +9,9 @@
 // Unlike the reference (ATen log_softmax/softmax into a full-size temporary, a
 // second kernel, then a Python-side multiply) each direction is ONE kernel that
 // reads the logits once: forward 4E + 12P bytes, backward 8E + 12P bytes.
+// The "reduced" forward additionally leaves per-block partial sums and valid-pixel
+// counts behind, which a one-block finishing kernel turns into sum or mean, so the
+// module-level reduction costs no further pass over the pixels.
 #include "plh_common.hpp"
 
 namespace plh {
@@ -23,12 +26,16 @@ struct LsrParams {
 
 // ---------------------------------------------------------------- regs ----
 
-template <int CP, int V>
-__global__ __launch_bounds__(256) void lsr_fwd_regs(const float *__restrict__ x,
-                                                    const int64_t *__restrict__ lab,
-                                                    float *__restrict__ loss, const LsrParams p) {
-    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
-    if (pix >= p.P) return;
+template <int CP, int V, bool Reduce>
+__global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const float *__restrict__ x,
+                                                          const int64_t *__restrict__ lab,
+                                                          float *__restrict__ loss, Partials part,
+                                                          const LsrParams p) {
+    __shared__ float red[4];
+    const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+    const bool live = want < p.P;
+    if (!Reduce && !live) return;
+    const int64_t pix = live ? want : 0;
     const int64_t n = pix / p.m_size;
     const float *xs = x + (pix + n * (int64_t)(p.C - 1) * p.m_size);
 
@@ -40,6 +47,8 @@ __global__ __launch_bounds__(256) void lsr_fwd_regs(const float *__restrict__ x,
     load_labels<V>(lab + pix, lb);
 
     float out[V];
+    float mine = 0.f;
+    int cnt = 0;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         float mx = v[0][k];
@@ -49,7 +58,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_regs(const float *__restrict__ x,
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) s += expf(v[j][k] - mx);
+            if (j < p.C) s += fast_exp(v[j][k] - mx);
         const float lse = logf(s);
         float acc = 0.f;
 #pragma unroll
@@ -58,17 +67,28 @@ __global__ __launch_bounds__(256) void lsr_fwd_regs(const float *__restrict__ x,
                 const float logp = (v[j][k] - mx) - lse;
                 acc -= logp * ((lb[k] == j) ? p.w_pos : p.w_neg);
             }
-        out[k] = (lb[k] == p.ignore) ? 0.f : acc;
+        const bool valid = live && (lb[k] != p.ignore);
+        out[k] = valid ? acc : 0.f;
+        mine += out[k];
+        cnt += valid ? 1 : 0;
     }
-    store_vec<V>(loss + pix, out);
+    if (live && loss) store_vec<V>(loss + pix, out);
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256((float)cnt, red);   // at most 512 per block: exact in fp32
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
 }
 
 template <int CP, int V>
-__global__ __launch_bounds__(256) void lsr_bwd_regs(const float *__restrict__ x,
-                                                    const int64_t *__restrict__ lab,
-                                                    const float *__restrict__ gout, int64_t gstride,
-                                                    float *__restrict__ grad, const LsrParams p) {
-    const int64_t pix = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+__global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const float *__restrict__ x,
+                                                          const int64_t *__restrict__ lab,
+                                                          const Upstream up, float *__restrict__ grad,
+                                                          const LsrParams p) {
+    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
     if (pix >= p.P) return;
     const int64_t n = pix / p.m_size;
     const int64_t base = pix + n * (int64_t)(p.C - 1) * p.m_size;
@@ -82,7 +102,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_regs(const float *__restrict__ x,
     int64_t lb[V];
     load_labels<V>(lab + pix, lb);
     float go[V];
-    load_gout<V>(gout, gstride, pix, go);
+    load_upstream<V>(up, pix, go);
 
 #pragma unroll
     for (int k = 0; k < V; ++k) {
@@ -94,17 +114,14 @@ __global__ __launch_bounds__(256) void lsr_bwd_regs(const float *__restrict__ x,
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
-                v[j][k] = expf(v[j][k] - mx);
+                v[j][k] = fast_exp(v[j][k] - mx);
                 s += v[j][k];
             }
-        const bool ign = (lb[k] == p.ignore);
+        const float gk = (lb[k] == p.ignore) ? 0.f : go[k];
+        const float scale = p.sumw * gk / s;          // one division per pixel
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const float prob = v[j][k] / s;
-                const float g = (p.sumw * prob - ((lb[k] == j) ? p.w_pos : p.w_neg)) * go[k];
-                v[j][k] = ign ? 0.f : g;
-            }
+            if (j < p.C) v[j][k] = v[j][k] * scale - ((lb[k] == j) ? p.w_pos : p.w_neg) * gk;
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
@@ -118,17 +135,20 @@ __global__ __launch_bounds__(256) void lsr_bwd_regs(const float *__restrict__ x,
 
 constexpr int kStageCap = 2048;   // floats per wave -> 32 KiB of LDS per 256-thread block
 
-template <int G>
+template <int G, bool Reduce>
 __global__ __launch_bounds__(256) void lsr_fwd_group(const float *__restrict__ x,
                                                      const int64_t *__restrict__ lab,
-                                                     float *__restrict__ loss, const LsrParams p) {
+                                                     float *__restrict__ loss, Partials part,
+                                                     const LsrParams p) {
     constexpr int kPix = 256 / G;
     __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
+    __shared__ float red[4];
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
     float *stage = stage_mem + ((G == 64) ? grp * kStageCap : 0);
     const bool staged = (G == 64) && (p.C <= kStageCap);
 
+    float mine = 0.f, cnt = 0.f;
     // every lane of a group walks the same pixels, so the loop is group-uniform
     const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
     for (int64_t r = 0; r < rounds; ++r) {
@@ -149,7 +169,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const float *__restrict__ x
         float s = 0.f;
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : xs[(int64_t)j * p.m_size];
-            s += expf(t - mx);
+            s += fast_exp(t - mx);
         }
         s = group_reduce<G>(s, OpSum());
         const float lse = logf(s);
@@ -159,15 +179,28 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const float *__restrict__ x
             acc -= ((t - mx) - lse) * ((lb == j) ? p.w_pos : p.w_neg);
         }
         acc = group_reduce<G>(acc, OpSum());
-        if (live && sub == 0) loss[pix] = (lb == p.ignore) ? 0.f : acc;
+        const bool valid = live && (lb != p.ignore);
+        if (live && sub == 0) {
+            if (loss) loss[pix] = valid ? acc : 0.f;
+            mine += valid ? acc : 0.f;
+            cnt += valid ? 1.f : 0.f;
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);     // exact while a block sees < 2^24 pixels
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
     }
 }
 
 template <int G>
 __global__ __launch_bounds__(256) void lsr_bwd_group(const float *__restrict__ x,
                                                      const int64_t *__restrict__ lab,
-                                                     const float *__restrict__ gout, int64_t gstride,
-                                                     float *__restrict__ grad, const LsrParams p) {
+                                                     const Upstream up, float *__restrict__ grad,
+                                                     const LsrParams p) {
     constexpr int kPix = 256 / G;
     __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
     const int sub = threadIdx.x % G;
@@ -186,7 +219,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const float *__restrict__ x
         float *gs = grad + base;
         const int64_t lb = lab[pc];
         float go[1];
-        load_gout<1>(gout, gstride, pc, go);
+        load_upstream<1>(up, pc, go);
 
         float mx = -INFINITY;
         for (int j = sub; j < p.C; j += G) {
@@ -198,17 +231,17 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const float *__restrict__ x
         float s = 0.f;
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : xs[(int64_t)j * p.m_size];
-            const float e = expf(t - mx);
+            const float e = fast_exp(t - mx);
             if (staged) stage[j] = e;
             s += e;
         }
         s = group_reduce<G>(s, OpSum());
         if (live) {
-            const bool ign = (lb == p.ignore);
+            const float gk = (lb == p.ignore) ? 0.f : go[0];
+            const float scale = p.sumw * gk / s;
             for (int j = sub; j < p.C; j += G) {
-                const float e = staged ? stage[j] : expf(xs[(int64_t)j * p.m_size] - mx);
-                const float g = (p.sumw * (e / s) - ((lb == j) ? p.w_pos : p.w_neg)) * go[0];
-                gs[(int64_t)j * p.m_size] = ign ? 0.f : g;
+                const float e = staged ? stage[j] : fast_exp(xs[(int64_t)j * p.m_size] - mx);
+                gs[(int64_t)j * p.m_size] = e * scale - ((lb == j) ? p.w_pos : p.w_neg) * gk;
             }
         }
     }
@@ -228,25 +261,79 @@ static LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, in
     return p;
 }
 
-template <int V>
-static void launch_fwd_regs(const float *x, const int64_t *lab, float *loss, const LsrParams &p, hipStream_t st) {
-    const unsigned grid = (unsigned)ceil_div(ceil_div(p.P, V), 256);
+template <int V, bool Reduce>
+static unsigned launch_fwd_regs(const float *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
+                                hipStream_t st) {
+    const unsigned grid = regs_grid<V>(p.P);
     switch ((p.C + 3) / 4) {
-#define PLH_CASE(K) case K: hipLaunchKernelGGL((lsr_fwd_regs<4 * K, V>), dim3(grid), dim3(256), 0, st, x, lab, loss, p); break;
+#define PLH_CASE(K)                                                                                         \
+    case K:                                                                                                 \
+        hipLaunchKernelGGL((lsr_fwd_regs<4 * K, V, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, loss, \
+                           part, p);                                                                        \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+    }
+    return grid;
+}
+
+template <int V>
+static void launch_bwd_regs(const float *x, const int64_t *lab, const Upstream &up, float *grad,
+                            const LsrParams &p, hipStream_t st) {
+    const unsigned grid = regs_grid<V>(p.P);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                             \
+    case K:                                                                                                     \
+        hipLaunchKernelGGL((lsr_bwd_regs<4 * K, V>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up, grad, p); \
+        break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
 }
 
-template <int V>
-static void launch_bwd_regs(const float *x, const int64_t *lab, const float *gout, int64_t gstride, float *grad,
-                            const LsrParams &p, hipStream_t st) {
-    const unsigned grid = (unsigned)ceil_div(ceil_div(p.P, V), 256);
-    switch ((p.C + 3) / 4) {
-#define PLH_CASE(K) case K: hipLaunchKernelGGL((lsr_bwd_regs<4 * K, V>), dim3(grid), dim3(256), 0, st, x, lab, gout, gstride, grad, p); break;
-        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
-#undef PLH_CASE
+// Launches the forward; returns the number of blocks that wrote partials.
+template <bool Reduce>
+static unsigned forward(const float *logits, const int64_t *labels, float *losses, Partials part,
+                        const LsrParams &p, hipStream_t st) {
+    switch (pick_shape(p.C, p.m_size, logits, nullptr, labels, losses, nullptr)) {
+        case Shape::Regs2: return launch_fwd_regs<2, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::Regs1: return launch_fwd_regs<1, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::Wave: {
+            const unsigned grid = group_grid(p.P, 4);
+            hipLaunchKernelGGL((lsr_fwd_group<64, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            return grid;
+        }
+        case Shape::Lane: {
+            const unsigned grid = group_grid(p.P, 256);
+            hipLaunchKernelGGL((lsr_fwd_group<1, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            return grid;
+        }
     }
+    return 0;
+}
+
+static int backward(const float *logits, const int64_t *labels, const Upstream &up, float *grad_logits,
+                    int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float smooth,
+                    void *stream) {
+    const int rc = check_slice_args(logits, labels, grad_logits, n_size, dimsize, m_size);
+    if (rc != PLH_OK) return rc;
+    if (n_size * dimsize * m_size == 0) return PLH_OK;
+    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+    hipStream_t st = (hipStream_t)stream;
+    const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    switch (pick_shape(dimsize, m_size, logits, grad_logits, labels, go_vec, nullptr)) {
+        case Shape::Regs2: launch_bwd_regs<2>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::Regs1: launch_bwd_regs<1>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::Wave:
+            hipLaunchKernelGGL((lsr_bwd_group<64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, up,
+                               grad_logits, p);
+            break;
+        case Shape::Lane:
+            hipLaunchKernelGGL((lsr_bwd_group<1>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, logits, labels, up,
+                               grad_logits, p);
+            break;
+    }
+    return check_launch();
 }
 
 }  // namespace plh
@@ -260,17 +347,28 @@ extern "C" int plh_lsr_forward(const float *logits, const int64_t *labels, float
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
     const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+    forward<false>(logits, labels, losses, Partials{nullptr, nullptr}, p, (hipStream_t)stream);
+    return check_launch();
+}
+
+extern "C" int plh_lsr_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+                                       float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                       void *workspace, int64_t workspace_bytes,
+                                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                                       int64_t ignore_index, float smooth, void *stream) {
+    int rc = check_slice_args(logits, labels, loss_out, n_size, dimsize, m_size);
+    if (rc != PLH_OK) return rc;
+    Partials part;
+    rc = carve_partials(workspace, workspace_bytes, n_size * m_size, loss_out, n_valid_out, part);
+    if (rc != PLH_OK) return rc;
+    if (losses && misaligned(losses, 4)) return PLH_ERR_MISALIGNED;
     hipStream_t st = (hipStream_t)stream;
-    switch (pick_shape(dimsize, m_size, logits, nullptr, labels, losses, nullptr)) {
-        case Shape::Regs4: launch_fwd_regs<4>(logits, labels, losses, p, st); break;
-        case Shape::Regs1: launch_fwd_regs<1>(logits, labels, losses, p, st); break;
-        case Shape::Wave:
-            hipLaunchKernelGGL((lsr_fwd_group<64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, losses, p);
-            break;
-        case Shape::Lane:
-            hipLaunchKernelGGL((lsr_fwd_group<1>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, logits, labels, losses, p);
-            break;
+    unsigned blocks = 0;
+    if (n_size * dimsize * m_size != 0) {
+        const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+        blocks = forward<true>(logits, labels, losses, part, p, st);
     }
+    finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
     return check_launch();
 }
 
@@ -279,25 +377,19 @@ extern "C" int plh_lsr_backward(const float *logits, const int64_t *labels,
                                 float *grad_logits,
                                 int64_t n_size, int64_t dimsize, int64_t m_size,
                                 int64_t ignore_index, float smooth, void *stream) {
-    int rc = check_slice_args(logits, labels, grad_logits, n_size, dimsize, m_size);
+    const int rc = check_gout(grad_output, grad_output_stride);
     if (rc != PLH_OK) return rc;
-    rc = check_gout(grad_output, grad_output_stride);
-    if (rc != PLH_OK) return rc;
-    if (n_size * dimsize * m_size == 0) return PLH_OK;
-    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
-    hipStream_t st = (hipStream_t)stream;
-    const float *go_vec = (grad_output && grad_output_stride == 1) ? grad_output : nullptr;
-    switch (pick_shape(dimsize, m_size, logits, grad_logits, labels, go_vec, nullptr)) {
-        case Shape::Regs4: launch_bwd_regs<4>(logits, labels, grad_output, grad_output_stride, grad_logits, p, st); break;
-        case Shape::Regs1: launch_bwd_regs<1>(logits, labels, grad_output, grad_output_stride, grad_logits, p, st); break;
-        case Shape::Wave:
-            hipLaunchKernelGGL((lsr_bwd_group<64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels,
-                               grad_output, grad_output_stride, grad_logits, p);
-            break;
-        case Shape::Lane:
-            hipLaunchKernelGGL((lsr_bwd_group<1>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, logits, labels,
-                               grad_output, grad_output_stride, grad_logits, p);
-            break;
-    }
-    return check_launch();
+    const Upstream up{grad_output, grad_output_stride, nullptr, 1.f};
+    return backward(logits, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream);
+}
+
+extern "C" int plh_lsr_backward_scaled(const float *logits, const int64_t *labels,
+                                       const float *grad_scalar, float scale, const int64_t *divide_by,
+                                       float *grad_logits,
+                                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                                       int64_t ignore_index, float smooth, void *stream) {
+    if (n_size * dimsize * m_size != 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale};
+    return backward(logits, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream);
 }

@@ -30,6 +30,13 @@ _SIGNATURES = {
     "plh_error_string": (ctypes.c_char_p, [ctypes.c_int]),
     "plh_lsr_forward": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lsr_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_reduce_workspace_bytes": (_i64, [_i64]),
+    "plh_lsr_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_focal_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _f32, _f32, _p]),
+    "plh_focal_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _i64, _f32, _f32, _p]),
+    "plh_lmargin_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_focal_forward": (ctypes.c_int, [_p, _p, _p, _i64, _f32, _f32, _p]),
     "plh_focal_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _f32, _f32, _p]),
     "plh_focal_forward_backward": (ctypes.c_int, [_p, _p, _p, _p, _i64, _f32, _f32, _p]),
@@ -168,6 +175,58 @@ def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None):
     return _back_to(grad, logits.dtype)
 
 
+def _reduce_workspace(units, device):
+    nbytes = int(load().plh_reduce_workspace_bytes(int(units)))
+    if nbytes < 0:
+        _check(nbytes)
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device), nbytes
+
+
+def _scalar_f32(t):
+    """A 0-dim upstream gradient as one fp32 value in device memory."""
+    t = t.reshape(-1)[:1]
+    return t if (t.dtype == torch.float32 and t.is_contiguous()) else t.float().contiguous()
+
+
+def _pixel_forward_reduced(entry, what, logits, labels, ignore_index, param, mean):
+    """Shared by LSR and large-margin: -> (loss 0-dim fp32, n_valid 0-dim int64)."""
+    _require_gpu(what, logits, labels)
+    n, c, m = _dims(logits, entry)
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, entry)
+    loss = torch.empty((), dtype=torch.float32, device=x.device)
+    n_valid = torch.empty((), dtype=torch.int64, device=x.device)
+    ws, ws_bytes = _reduce_workspace(n * m, x.device)
+    with torch.cuda.device_of(x):
+        _check(getattr(load(), entry)(_ptr(x), _ptr(lb), None, _ptr(loss), _ptr(n_valid), 1 if mean else 0,
+                                      _ptr(ws), ws_bytes, n, c, m, int(ignore_index), float(param), _stream()))
+    return _back_to(loss, logits.dtype), n_valid
+
+
+def _pixel_backward_scaled(entry, what, logits, labels, ignore_index, param, grad_scalar, divide_by):
+    _require_gpu(what, logits, labels)
+    n, c, m = _dims(logits, entry)
+    x = _f32c(logits)
+    lb = _labels_i64(labels, logits, entry)
+    grad = torch.empty_like(x)
+    if x.numel() == 0:
+        return _back_to(grad, logits.dtype)
+    go = _scalar_f32(grad_scalar)
+    with torch.cuda.device_of(x):
+        _check(getattr(load(), entry)(_ptr(x), _ptr(lb), _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), n, c, m,
+                                      int(ignore_index), float(param), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+def lsr_forward_reduced(logits, labels, ignore_index, smooth, mean):
+    return _pixel_forward_reduced("plh_lsr_forward_reduced", "LSR loss", logits, labels, ignore_index, smooth, mean)
+
+
+def lsr_backward_scaled(logits, labels, ignore_index, smooth, grad_scalar, divide_by=None):
+    return _pixel_backward_scaled("plh_lsr_backward_scaled", "LSR loss", logits, labels, ignore_index, smooth,
+                                  grad_scalar, divide_by)
+
+
 # ---------------------------------------------------------------- focal ----
 
 def _focal_pair(logits, labels, what):
@@ -209,7 +268,38 @@ def focal_forward_backward(logits, labels, gamma, alpha):
     return _back_to(losses, logits.dtype), _back_to(grad, logits.dtype)
 
 
+def focal_forward_reduced(logits, labels, gamma, alpha, mean):
+    x, y = _focal_pair(logits, labels, "focalloss_forward")
+    loss = torch.empty((), dtype=torch.float32, device=x.device)
+    ws, ws_bytes = _reduce_workspace(x.numel(), x.device)
+    with torch.cuda.device_of(x):
+        _check(load().plh_focal_forward_reduced(_ptr(x), _ptr(y), None, _ptr(loss), 1 if mean else 0, _ptr(ws),
+                                                ws_bytes, x.numel(), float(gamma), float(alpha), _stream()))
+    return _back_to(loss, logits.dtype)
+
+
+def focal_backward_scaled(logits, labels, gamma, alpha, grad_scalar, scale):
+    x, y = _focal_pair(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(x)
+    if x.numel():
+        go = _scalar_f32(grad_scalar)
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_backward_scaled(_ptr(x), _ptr(y), _ptr(go), float(scale), _ptr(grad), x.numel(),
+                                                    float(gamma), float(alpha), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
 # -------------------------------------------------------------- lmargin ----
+
+def lmargin_forward_reduced(logits, labels, lam, ignore_index, mean):
+    return _pixel_forward_reduced("plh_lmargin_forward_reduced", "large margin loss", logits, labels, ignore_index,
+                                  lam, mean)
+
+
+def lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_scalar, divide_by=None):
+    return _pixel_backward_scaled("plh_lmargin_backward_scaled", "large margin loss", logits, labels, ignore_index,
+                                  lam, grad_scalar, divide_by)
+
 
 def lmargin_forward(logits, labels, lam, ignore_index):
     _require_gpu("large margin loss", logits, labels)

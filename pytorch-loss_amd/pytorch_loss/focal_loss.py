@@ -49,6 +49,25 @@ class FocalSigmoidLossFuncV3FB(torch.autograd.Function):
         return grads, None, None, None
 
 
+class _FocalReducedFunction(torch.autograd.Function):
+    """'sum' / 'mean' over all elements produced inside the forward kernel (per-block partials,
+    fixed-order finish); backward folds the scalar upstream gradient and 1/numel into its kernel."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, alpha, gamma, mean):
+        ctx.variables = (logits, labels, alpha, gamma, mean)
+        return _native.focal_forward_reduced(logits, labels, gamma, alpha, mean)
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        logits, labels, alpha, gamma, mean = ctx.variables
+        scale = 1.0 / logits.numel() if mean else 1.0
+        grads = _native.focal_backward_scaled(logits, labels, gamma, alpha, grad_output, scale)
+        return grads, None, None, None, None
+
+
 class FocalLossV3(nn.Module):
     """Usage as nn.BCEWithLogitsLoss. reduction 'mean' averages over every element."""
 
@@ -59,6 +78,8 @@ class FocalLossV3(nn.Module):
         self.reduction = reduction
 
     def forward(self, logits, label):
+        if self.reduction in ("mean", "sum") and logits.numel() > 0:
+            return _FocalReducedFunction.apply(logits, label, self.alpha, self.gamma, self.reduction == "mean")
         # the two-kernel Function moves the same bytes as the fused one once the upstream
         # multiply is folded into the backward kernel, and keeps no gradient-sized tensor alive
         loss = FocalSigmoidLossFuncV3.apply(logits, label, self.alpha, self.gamma)

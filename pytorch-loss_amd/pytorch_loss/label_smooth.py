@@ -30,6 +30,27 @@ class LSRCrossEntropyFunctionV3(torch.autograd.Function):
         return grad, None, None, None
 
 
+class _LSRReducedFunction(torch.autograd.Function):
+    """'sum' / 'mean' of the per-pixel losses produced inside the forward kernel (per-block
+    partials, then a fixed-order finishing kernel), so the module needs no ATen pass over the
+    pixels for `losses.sum()` and `(labels != ignore).sum()`; backward folds the scalar
+    upstream gradient and the 1/n_valid of a mean into the gradient kernel."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, lb_smooth, lb_ignore, mean):
+        loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean)
+        ctx.variables = (logits, labels, lb_ignore, lb_smooth, n_valid if mean else None)
+        return loss
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        logits, labels, lb_ignore, lb_smooth, n_valid = ctx.variables
+        grad = _native.lsr_backward_scaled(logits, labels, lb_ignore, lb_smooth, grad_output, n_valid)
+        return grad, None, None, None, None
+
+
 class LabelSmoothSoftmaxCEV3(nn.Module):
     """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
 
@@ -44,6 +65,9 @@ class LabelSmoothSoftmaxCEV3(nn.Module):
         self.lb_ignore = ignore_index
 
     def forward(self, logits, labels):
+        if self.reduction in ("sum", "mean") and logits.numel() > 0:
+            return _LSRReducedFunction.apply(logits, labels, self.lb_smooth, self.lb_ignore,
+                                             self.reduction == "mean")
         losses = LSRCrossEntropyFunctionV3.apply(logits, labels, self.lb_smooth, self.lb_ignore)
         if self.reduction == "sum":
             return losses.sum()

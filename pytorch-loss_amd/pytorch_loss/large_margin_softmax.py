@@ -48,6 +48,24 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
         return grads, None, None, None
 
 
+class _LargeMarginReducedFunction(torch.autograd.Function):
+    """'sum' / 'mean' produced inside the forward kernel; see label_smooth._LSRReducedFunction."""
+
+    @staticmethod
+    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    def forward(ctx, logits, labels, lam, ignore_index, mean):
+        loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean)
+        ctx.variables = (logits, labels, lam, ignore_index, n_valid if mean else None)
+        return loss
+
+    @staticmethod
+    @amp.custom_bwd(device_type="cuda")
+    def backward(ctx, grad_output):
+        logits, labels, lam, ignore_index, n_valid = ctx.variables
+        grads = _native.lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_output, n_valid)
+        return grads, None, None, None, None
+
+
 class LargeMarginSoftmaxV3(nn.Module):
     """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
 
@@ -64,6 +82,9 @@ class LargeMarginSoftmaxV3(nn.Module):
         self.fb = fb
 
     def forward(self, logits, labels):
+        if not self.fb and self.reduction in ("sum", "mean") and logits.numel() > 0:
+            return _LargeMarginReducedFunction.apply(logits, labels, self.lam, self.ignore_index,
+                                                     self.reduction == "mean")
         valid_cnt = None
         if self.fb:
             losses, valid_cnt = LargeMarginSoftmaxFuncV3FB.apply(logits, labels, self.lam, self.ignore_index)
