@@ -2,7 +2,8 @@
 //
 // Per element (x logit, y label in [0,1], csrc/focal_kernel.cu:39-51,65-83):
 //   p      = sigmoid(x)
-//   log p  = min(x,0) - log1p(exp(-|x|)),  log(1-p) = log p - x
+//   log p  = min(x,0) - log1p(exp(-|x|)),  log(1-p) = -max(x,0) - log1p(exp(-|x|))
+//            (focal_loss.py:59-64; the CUDA kernel's log p - x loses digits for x << 0)
 //   ce     = y*alpha*log p + (1-y)*(1-alpha)*log(1-p)
 //   coeff  = -|y-p|^gamma,                  loss = coeff*ce
 //   d_ce   = y*alpha - p*(1 - y - alpha + 2*y*alpha)
@@ -22,11 +23,12 @@ struct FocalParams {
 
 template <int Mode, bool WantLoss, bool WantGrad>
 __device__ __forceinline__ void focal_point(float x, float y, const FocalParams p, float &loss, float &grad) {
-    const float e = expf(-fabsf(x));                 // exp(-|x|) in (0, 1]: one exponential serves p and log p
-    const float inv = 1.f / (1.f + e);
+    const float e = fast_exp(-fabsf(x));             // exp(-|x|) in [0, 1]: one exponential serves p and log p
+    const float inv = __builtin_amdgcn_rcpf(1.f + e);
     const float prob = (x >= 0.f) ? inv : e * inv;
-    const float log_p = fminf(x, 0.f) - log1pf(e);
-    const float log_1p = log_p - x;
+    const float l1p = fast_log1p_unit(e);
+    const float log_p = fminf(x, 0.f) - l1p;
+    const float log_1p = -fmaxf(x, 0.f) - l1p;       // formed directly: log_p - x cancels for x << 0
     const float ce = y * p.alpha * log_p + (1.f - y) * (1.f - p.alpha) * log_1p;
     const float a = fabsf(y - prob);
     float a_pow, a_pow_m1;                           // |y-p|^gamma and |y-p|^(gamma-1)

@@ -56,55 +56,60 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ 
     int cnt = 0;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
-        const bool ign = (lb[k] == p.ignore);
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
         float m_no = -INFINITY, x_y = -INFINITY;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
-                const bool hot = (lb[k] == j);
+                const bool hot = (tgt == j);
                 m_no = hot ? m_no : fmaxf(m_no, v[j][k]);
                 x_y = hot ? v[j][k] : x_y;
             }
         const float m_all = fmaxf(m_no, x_y);
-        float s_no = 0.f, sum_ex = 0.f;
+        // one exponential per channel: with t_j = x_j - m_no and e_j = exp(t_j) over j != y,
+        //   sum_j (q_j - coeff) log q_j = (sum e_j t_j)/s_no - lse_no - coeff * (sum t_j - (C-1) lse_no)
+        float e[WantGrad ? CP : 1];
+        float s_no = 0.f, sum_et = 0.f, sum_t = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
-                const float e = (lb[k] == j) ? 0.f : fast_exp(v[j][k] - m_no);
-                s_no += e;
-                if constexpr (WantGrad) sum_ex += e * v[j][k];
+                const bool hot = (tgt == j);
+                const float t = v[j][k] - m_no;
+                const float ej = hot ? 0.f : fast_exp(t);
+                if constexpr (WantGrad) e[j] = ej;
+                s_no += ej;
+                sum_et += ej * (hot ? 0.f : t);
+                sum_t += hot ? 0.f : t;
             }
-        const float t = fast_exp(m_no - m_all);
+        const float t_all = fast_exp(m_no - m_all);
         const float e_y = fast_exp(x_y - m_all);
-        const float s_all = s_no * t + e_y;
+        const float s_all = s_no * t_all + e_y;
         const float inv_no = 1.f / s_no;
-        const float inv_all = 1.f / s_all;
-        const float sum_qx = sum_ex * inv_no;
-        const float lse_no = logf(s_no);
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const bool hot = (lb[k] == j);
-                const float xv = v[j][k];
-                const float e = fast_exp(xv - m_no);
-                const float q = e * inv_no;
-                if constexpr (WantLoss) {
-                    const float term = p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
-                    acc += hot ? 0.f : term;
-                }
-                if constexpr (WantGrad) {
-                    const float g_hot = e_y * inv_all - 1.f;
-                    const float g_cold = e * t * inv_all + p.half_lam * ((xv + 1.f - sum_qx) * q - p.coeff);
-                    const float g = (hot ? g_hot : g_cold) * go[k];
-                    v[j][k] = ign ? 0.f : g;
-                }
-            }
         if constexpr (WantLoss) {
-            acc += -(x_y - m_all) + logf(s_all);
+            const float lse_no = logf(s_no);
+            const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));   // channels that are not the target
+            const float margin = sum_et * inv_no - lse_no - p.coeff * (sum_t - others * lse_no);
+            const float acc = p.half_lam * margin - (x_y - m_all) + logf(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
             mine += out[k];
             cnt += (ign || !live) ? 0 : 1;
+        }
+        if constexpr (WantGrad) {
+            const float inv_all = 1.f / s_all;
+            // sum_k q_k x_k = (sum e t)/s_no + m_no
+            const float sum_qx = sum_et * inv_no + m_no;
+            const float gk = ign ? 0.f : go[k];
+            const float p_scale = t_all * inv_all;
+            const float g_hot = (e_y * inv_all - 1.f) * gk;
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (j < p.C) {
+                    const float q = e[j] * inv_no;
+                    const float g_cold = e[j] * p_scale + p.half_lam * ((v[j][k] + 1.f - sum_qx) * q - p.coeff);
+                    const float g = (tgt == j) ? g_hot : g_cold * gk;
+                    v[j][k] = ign ? 0.f : g;      // exact zero even for non-finite logits
+                }
         }
         if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
     }

@@ -60,14 +60,16 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const float *__restri
         for (int j = 0; j < CP; ++j)
             if (j < p.C) s += fast_exp(v[j][k] - mx);
         const float lse = logf(s);
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
         float acc = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
                 const float logp = (v[j][k] - mx) - lse;
-                acc -= logp * ((lb[k] == j) ? p.w_pos : p.w_neg);
+                acc -= logp * ((tgt == j) ? p.w_pos : p.w_neg);
             }
-        const bool valid = live && (lb[k] != p.ignore);
+        const bool valid = live && !ign;
         out[k] = valid ? acc : 0.f;
         mine += out[k];
         cnt += valid ? 1 : 0;
@@ -117,11 +119,17 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const float *__restri
                 v[j][k] = fast_exp(v[j][k] - mx);
                 s += v[j][k];
             }
-        const float gk = (lb[k] == p.ignore) ? 0.f : go[k];
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        const float gk = ign ? 0.f : go[k];
         const float scale = p.sumw * gk / s;          // one division per pixel
+        const float g_pos = p.w_pos * gk, g_neg = p.w_neg * gk;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) v[j][k] = v[j][k] * scale - ((lb[k] == j) ? p.w_pos : p.w_neg) * gk;
+            if (j < p.C) {
+                const float g = v[j][k] * scale - ((tgt == j) ? g_pos : g_neg);
+                v[j][k] = ign ? 0.f : g;      // exact zero even for non-finite logits
+            }
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)

@@ -1,0 +1,142 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares with the arity the binding assumes, rejects bad arguments before launching anything,
+and the Python surface mirrors the reference's error behaviour.  No kernel runs here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pytorch_loss_hip.h")
+
+
+def declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|int64_t|const char \*)\s*(plh_\w+)\s*\(([^;{]*)\)\s*;", text):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args in ("", "void") else args.count(",") + 1
+    return out
+
+
+@pytest.fixture(scope="module")
+def native():
+    from pytorch_loss import _native
+    return _native
+
+
+def test_library_exports_every_declared_symbol(native):
+    lib = native.load()
+    decl = declared()
+    assert len(decl) >= 20
+    for name, n_args in decl.items():
+        assert hasattr(lib, name), name
+        assert name in native._SIGNATURES, "binding lacks " + name
+        assert len(native._SIGNATURES[name][1]) == n_args, name
+    assert set(native._SIGNATURES) == set(decl)
+    assert lib.plh_abi_version() == 1
+
+
+def test_error_strings(native):
+    lib = native.load()
+    assert lib.plh_error_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert len(lib.plh_error_string(code)) > 5
+    assert b"512" in lib.plh_error_string(-4)
+    assert lib.plh_error_string(-99) == b"unknown error code"
+
+
+def test_arguments_are_rejected_before_any_launch(native):
+    lib = native.load()
+    buf = (ctypes.c_float * 64)()
+    lab = (ctypes.c_int64 * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    lp = ctypes.cast(lab, ctypes.c_void_p)
+    odd = ctypes.c_void_p(p.value + 2)
+    # zero-sized problems are fine and launch nothing
+    assert lib.plh_lsr_forward(None, None, None, 0, 19, 16, 255, 0.1, None) == 0
+    assert lib.plh_focal_forward(None, None, None, 0, 2.0, 0.25, None) == 0
+    assert lib.plh_lovasz_forward(None, None, None, None, None, 0, 0, 19, 16, 255, None) == 0
+    assert lib.plh_stream_copy(None, None, 0, None) == 0
+    # NULL / negative / misaligned / stride / class-count / workspace
+    assert lib.plh_lsr_forward(None, lp, p, 1, 2, 2, 255, 0.1, None) == -1
+    assert lib.plh_lsr_forward(p, lp, p, -1, 2, 2, 255, 0.1, None) == -2
+    assert lib.plh_lsr_forward(odd, lp, p, 1, 2, 2, 255, 0.1, None) == -6
+    assert lib.plh_lsr_backward(p, lp, p, 2, p, 1, 2, 2, 255, 0.1, None) == -3
+    assert lib.plh_lmargin_backward(p, lp, p, 7, p, 1, 2, 2, 255, 0.3, None) == -3
+    assert lib.plh_focal_backward(p, p, p, 3, p, 4, 2.0, 0.25, None) == -3
+    assert lib.plh_focal_forward(p, None, p, 4, 2.0, 0.25, None) == -1
+    assert lib.plh_lovasz_forward(p, lp, p, p, p, 1 << 20, 1, 512, 2, 255, None) == -4
+    assert lib.plh_lovasz_workspace_bytes(1, 512, 4) == -4
+    assert lib.plh_lovasz_workspace_bytes(1 << 20, 19, 1 << 12) == -2       # numel >= 2^31
+    need = lib.plh_lovasz_workspace_bytes(2, 19, 64)
+    assert need > 3 * 4 * 2 * 19 * 64
+    assert lib.plh_lovasz_forward(p, lp, p, p, None, need, 2, 19, 64, 255, None) == -5
+    assert lib.plh_lsr_forward_reduced(p, lp, None, p, None, 1, None, 0, 1, 2, 2, 255, 0.1, None) == -5
+    assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
+    assert lib.plh_reduce_workspace_bytes(-1) == -2
+
+
+def test_python_surface_refuses_cpu_tensors():
+    import pytorch_loss as pl
+    x = torch.randn(2, 5, 4, 4, requires_grad=True)
+    y = torch.randint(0, 5, (2, 4, 4))
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.LabelSmoothSoftmaxCEV3()(x, y)
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.LargeMarginSoftmaxV3()(x, y)
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.LovaszSoftmaxV3()(x, y)
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.FocalLossV3()(x, torch.rand_like(x))
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.LSRCrossEntropyFunctionV3.apply(x, y, 0.1, -100)
+
+
+def test_constructor_defaults_match_the_reference():
+    # pytorch_loss/label_smooth.py:150, focal_loss.py:177-180, large_margin_softmax.py:151,
+    # lovasz_softmax.py:97
+    import pytorch_loss as pl
+    a = pl.LabelSmoothSoftmaxCEV3()
+    assert (a.lb_smooth, a.reduction, a.lb_ignore) == (0.1, "mean", -100)
+    b = pl.FocalLossV3()
+    assert (b.alpha, b.gamma, b.reduction) == (0.25, 2, "mean")
+    c = pl.LargeMarginSoftmaxV3()
+    assert (c.lam, c.reduction, c.ignore_index) == (0.3, "mean", 255)
+    d = pl.LovaszSoftmaxV3()
+    assert (d.reduction, d.lb_ignore) == ("mean", -100)
+    for name in ("LSRCrossEntropyFunctionV3", "FocalSigmoidLossFuncV3", "FocalSigmoidLossFuncV3FB",
+                 "LargeMarginSoftmaxFuncV3", "LargeMarginSoftmaxFuncV3FB", "LovaszSoftmaxFunctionV3"):
+        assert issubclass(getattr(pl, name), torch.autograd.Function)
+
+
+def test_upstream_gradient_marshalling(native):
+    like = (2, 3, 4)
+    t, stride = native._upstream(None, like)
+    assert t is None and stride == 0
+    scalar = torch.tensor(0.5).expand(like)              # what sum()/mean() backward hands over
+    t, stride = native._upstream(scalar, like)
+    assert stride == 0 and t.numel() == 1 and t.item() == 0.5
+    full = torch.rand(like)
+    t, stride = native._upstream(full, like)
+    assert stride == 1 and t.is_contiguous() and torch.equal(t, full)
+    t, stride = native._upstream(full.double().transpose(1, 2).transpose(1, 2), like)
+    assert stride == 1 and t.dtype == torch.float32
+    assert native._dims(torch.zeros(3, 5), "x") == (3, 5, 1)
+    assert native._dims(torch.zeros(3, 5, 2, 7), "x") == (3, 5, 14)
+    with pytest.raises(RuntimeError):
+        native._dims(torch.zeros(3), "x")
+    with pytest.raises(RuntimeError, match="integer"):
+        native._labels_i64(torch.zeros(3, 2, 7), torch.zeros(3, 5, 2, 7), "x")
+    with pytest.raises(RuntimeError, match="do not match"):
+        native._labels_i64(torch.zeros(3, 7, dtype=torch.long), torch.zeros(3, 5, 2, 7), "x")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)

@@ -1,0 +1,134 @@
+"""The benchmark configurations at full size on the GPU.
+
+The oracle checks one image of each batch (what a CPU finishes in seconds); the rest of the batch
+is held to size-independent properties: gradient rows of valid pixels sum to zero, ignored pixels
+give exact zeros, the valid count is an exact integer, 'mean' equals 'sum' / count, results do
+not depend on where in the batch an image sits, Lovasz Jaccard differences telescope to one and
+the loss does not change under a permutation of the pixels.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pl():
+    import pytorch_loss
+    from pytorch_loss import _native
+    _native.load()
+    return pytorch_loss
+
+
+def _seg_full(name):
+    w = synth.workload(name)            # portable generator: identical bits on every box
+    return w["logits"], w["labels"]
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg4"])
+def test_channel_softmax_losses_full_size(pl, name):
+    x, y = _seg_full(name)
+    assert x.shape == (8, 19, 1024, 1024)
+    xt = torch.from_numpy(x).cuda().requires_grad_()
+    yt = torch.from_numpy(y).cuda()
+    if name == "cfg2":
+        make = lambda red: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=255)
+        o_fwd = lambda a, b: oracle.lsr_forward(a, b, 255, 0.1)
+        o_bwd = lambda a, b, g: oracle.lsr_backward(a, b, 255, 0.1, g)
+    else:
+        make = lambda red: pl.LargeMarginSoftmaxV3(lam=0.3, reduction=red, ignore_index=255)
+        o_fwd = lambda a, b: oracle.lmargin_forward(a, b, 0.3, 255)
+        o_bwd = lambda a, b, g: oracle.lmargin_backward(a, b, 0.3, 255, g)
+
+    n_valid = int((y != 255).sum())
+    mean = make("mean")(xt, yt)
+    mean.backward()
+    g_mean = xt.grad.clone()
+    xt.grad = None
+    total = make("sum")(xt, yt)
+    total.backward()
+    g_sum = xt.grad.clone()
+    xt.grad = None
+    per = make("none")(xt, yt)
+
+    # reductions agree with each other and with the exact integer count
+    assert abs(mean.item() - total.item() / n_valid) <= 1e-6 * abs(mean.item())
+    assert abs(per.double().sum().item() - total.item()) <= 1e-5 * abs(total.item())
+    # masks: exact zeros at ignored pixels, nowhere else
+    ign = yt == 255
+    assert (per[ign] == 0).all() and (per[~ign] > 0).all()
+    assert (g_sum.permute(0, 2, 3, 1)[ign] == 0).all()
+    # softmax-type gradients: rows of valid pixels sum to zero
+    assert g_sum.sum(dim=1).abs().max().item() < 1e-5
+    # mean gradient = sum gradient / n_valid (linearity in the upstream scalar)
+    assert (g_mean * n_valid - g_sum).abs().max().item() < 1e-5
+    # oracle on one image; position in the batch must not matter
+    k = 5
+    want = o_fwd(x[k:k + 1], y[k:k + 1])
+    got = per[k:k + 1].detach().cpu().numpy()
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6)
+    want_g = o_bwd(x[k:k + 1], y[k:k + 1], None)
+    err = np.abs(g_sum[k:k + 1].cpu().numpy() - want_g).max()
+    assert err <= 1e-5, err
+    alone = make("none")(xt[k:k + 1].detach().contiguous(), yt[k:k + 1].contiguous())
+    assert torch.equal(alone, per[k:k + 1].detach())
+    # whole-batch loss against the oracle's per-image sums
+    ref_total = sum(o_fwd(x[i:i + 1], y[i:i + 1]).sum(dtype=np.float64) for i in range(x.shape[0]))
+    assert abs(total.item() - ref_total) <= 1e-5 * abs(ref_total)
+
+
+def test_focal_full_size(pl):
+    w = synth.workload("cfg3")
+    x, y = w["logits"], w["labels"]
+    assert x.shape == (16, 80, 128, 128)
+    xt = torch.from_numpy(x).cuda().requires_grad_()
+    yt = torch.from_numpy(y).cuda()
+    mean = pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean")(xt, yt)
+    mean.backward()
+    per = pl.FocalLossV3(alpha=0.25, gamma=2, reduction="none")(xt.detach(), yt)
+    want = oracle.focal_forward(x.astype(np.float64), y.astype(np.float64), 0.25, 2.0)
+    assert abs(mean.item() - want.mean()) <= 1e-5 * want.mean()
+    got = per.cpu().numpy()
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * want.mean())
+    want_g = oracle.focal_backward(x, y, 0.25, 2.0, np.float32(1.0 / x.size))
+    g = xt.grad.cpu().numpy()
+    assert np.abs(g - want_g).max() <= 1e-5
+    assert np.abs(g - want_g).max() <= 2e-5 * np.abs(want_g).max()      # relative: 'mean' makes 1e-5 absolute vacuous
+    # symmetry loss(x, y; a) == loss(-x, 1-y; 1-a)
+    flipped = pl.FocalLossV3(alpha=0.75, gamma=2, reduction="none")(-xt.detach(), 1.0 - yt)
+    assert (flipped - per).abs().max().item() <= 1e-6
+
+
+def test_lovasz_full_size(pl):
+    from pytorch_loss import _native
+    w = synth.workload("cfg5")
+    x, y = w["logits"], w["labels"]
+    assert x.shape == (4, 19, 512, 1024)
+    xt = torch.from_numpy(x).cuda().requires_grad_()
+    yt = torch.from_numpy(y).cuda()
+    losses = pl.LovaszSoftmaxV3(reduction="none", ignore_index=255)(xt, yt)
+    losses.sum().backward()
+    want, want_jacc = oracle.lovasz_forward(x.astype(np.float64), y, 255)
+    np.testing.assert_allclose(losses.detach().cpu().numpy(), want, rtol=1e-5)
+    # gradient against the fp64 oracle: identical up to re-ordering of near-ties
+    want_g = oracle.lovasz_backward(np.ones(19), x.astype(np.float64), y, want_jacc, 255)
+    err = np.abs(xt.grad.cpu().numpy() - want_g)
+    assert np.median(err) < 1e-9 and err.max() <= 1e-5, (np.median(err), err.max())
+    g = xt.grad
+    assert (g.permute(0, 2, 3, 1)[yt == 255] == 0).all()
+    assert g.sum(dim=1).abs().max().item() < 1e-6            # softmax Jacobian: rows sum to zero
+    # saved Jaccard differences: zero at ignored pixels, each class telescopes to J(all) = 1
+    _, jacc = _native.lovasz_forward(xt.detach(), yt, 255)
+    assert (jacc[:, (yt == 255).reshape(-1)] == 0).all()
+    assert (jacc.double().sum(dim=1) - 1.0).abs().max().item() < 1e-6
+    assert (jacc >= 0).all()        # J is monotone along the sorted order
+    # the loss is a function of the multiset of (error, label) pairs: permuting pixels changes nothing
+    perm = torch.randperm(512 * 1024, device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+    xp = xt.detach().reshape(4, 19, -1)[:, :, perm].reshape(4, 19, 512, 1024).contiguous()
+    yp = yt.reshape(4, -1)[:, perm].reshape(4, 512, 1024).contiguous()
+    lp = pl.LovaszSoftmaxV3(reduction="none", ignore_index=255)(xp, yp)
+    assert (lp - losses.detach()).abs().max().item() <= 2e-6
