@@ -25,6 +25,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by
+# what the same counters read for the plain copy kernel): see profiles/*_hbm_traffic.txt.
+# Only valid for the exact workload shape they were taken on; anything else reports null.
+MEASURED_TRAFFIC = {
+    ("lsr", (8, 19, 1024, 1024)): {"forward": 704.8e6 + 33.6e6, "backward": 735.0e6 + 637.5e6},
+}
+
 WORKLOADS = {
     # name: (module factory name, logits shape, description)
     "lsr": dict(shape=(8, 19, 1024, 1024), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8,19,1024,1024), "
@@ -176,8 +183,9 @@ def kernel_rooflines(name, logits, labels):
     for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
         ms = time_kernel(fn)
         gbps = nbytes / (ms * 1e-3) / 1e9
+        traffic = MEASURED_TRAFFIC.get((name, shape), {}).get(key)
         out[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
                     "ms": round(ms, 4), "algorithmic_bytes": nbytes}
     return out
 
