@@ -113,7 +113,10 @@ struct SortArgs {
     const uint32_t *vals_in;     // nullptr in the first pass: payload = position
     uint32_t *keys_out;
     uint32_t *vals_out;
-    uint32_t *tile_hist;         // [C][kRadix][tiles]: counts, then exclusive offsets inside the class row
+    uint32_t *tile_hist;         // [C][kRadix][tiles]: keys per (digit, tile); row-scanned in place
+    uint32_t *digit_total;       // [C][kRadix]: keys per digit
+    uint32_t *tile_hot;          // last pass only: the same two tables for the positives
+    uint32_t *hot_total;
     int P;                       // keys per class row
     int tiles;                   // ceil(P / kSortTile)
     int shift;                   // 0, 8, 16, 24
@@ -131,25 +134,27 @@ __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
     return v;
 }
 
-// Exclusive scan of one value per thread over a 256-thread block; `total` = block sum.
-// lds must hold kSortWaves + 1 words. Contains barriers: call from uniform control flow.
-__device__ __forceinline__ uint32_t block_excl_scan_256(uint32_t v, uint32_t *lds, uint32_t &total) {
+// Exclusive scan of one value per thread over the whole block (kSortThreads threads);
+// `total` = block sum. lds must hold kSortWaves words. Contains barriers: every thread calls it.
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *lds, uint32_t &total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t incl = wave_incl_scan(v);
     if (lane == 63) lds[wave] = incl;
     __syncthreads();
-    uint32_t before = 0;
+    uint32_t before = 0, all = 0;
 #pragma unroll
-    for (int w = 0; w < kSortWaves; ++w) before += (w < wave) ? lds[w] : 0u;
-    total = lds[0] + lds[1] + lds[2] + lds[3];
+    for (int w = 0; w < kSortWaves; ++w) {
+        const uint32_t t = lds[w];
+        before += (w < wave) ? t : 0u;
+        all += t;
+    }
+    total = all;
     __syncthreads();
     return before + incl - v;
 }
 
-// Stable rank of every key of the wave's 64-key round among equal digits, accumulated in the
-// wave's private digit counters: returns the number of equal digits seen earlier by this wave.
-__device__ __forceinline__ uint32_t wave_rank(uint32_t digit, bool valid, uint32_t *wave_counts) {
-    const int lane = __lane_id();
+// Match mask: the valid lanes of the wave whose digit equals this lane's (8 ballots).
+__device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
     uint64_t peers = __builtin_amdgcn_ballot_w64(valid);
 #pragma unroll
     for (int b = 0; b < 8; ++b) {
@@ -157,23 +162,46 @@ __device__ __forceinline__ uint32_t wave_rank(uint32_t digit, bool valid, uint32
         const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
         peers &= bit ? vote : ~vote;
     }
-    const uint32_t lower = __builtin_popcountll(peers & ((1ull << lane) - 1ull));
-    const uint32_t count = __builtin_popcountll(peers);
-    const int leader = peers ? (__builtin_ffsll((long long)peers) - 1) : lane;
-    uint32_t seen = 0;
-    if (valid && lane == leader) {
-        seen = wave_counts[digit];
-        wave_counts[digit] = seen + count;
-    }
-    seen = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen);
-    return seen + lower;
+    return peers;
 }
 
+// Stable rank of this lane's key among the equal digits the wave has seen so far (earlier rounds
+// through the wave's private counters, this round through the match mask). With Hot, the same for
+// the positives only (hrank = positives with this digit before this key).
+template <bool Hot>
+__device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, uint32_t *counts,
+                                          uint32_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
+    const int lane = __lane_id();
+    const uint64_t peers = wave_peers(digit, valid);
+    const uint64_t below = (1ull << lane) - 1ull;
+    const int leader = peers ? (__builtin_ffsll((long long)peers) - 1) : lane;
+    uint32_t seen = 0, seen_hot = 0;
+    uint64_t hot_peers = 0;
+    if constexpr (Hot) hot_peers = peers & __builtin_amdgcn_ballot_w64(hot && valid);
+    if (valid && lane == leader) {
+        seen = counts[digit];
+        counts[digit] = seen + __builtin_popcountll(peers);
+        if constexpr (Hot) {
+            seen_hot = counts_hot[digit];
+            counts_hot[digit] = seen_hot + __builtin_popcountll(hot_peers);
+        }
+    }
+    rank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen) + __builtin_popcountll(peers & below);
+    if constexpr (Hot)
+        hrank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen_hot) +
+                __builtin_popcountll(hot_peers & below);
+}
+
+template <bool Hot>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];
+    __shared__ uint32_t counts_hot[Hot ? kSortWaves : 1][kRadix];
     const int c = blockIdx.y, tile = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
+        (&counts[0][0])[i] = 0;
+        if constexpr (Hot) (&counts_hot[0][0])[i] = 0;
+    }
     __syncthreads();
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, a.P - begin);
@@ -183,37 +211,57 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         const bool valid = li < count;
         const uint32_t key = valid ? kin[li] : kIgnoredKey;
-        wave_rank((key >> a.shift) & a.digit_mask, valid, counts[wave]);
+        const uint32_t digit = (key >> a.shift) & a.digit_mask;
+        const uint64_t peers = wave_peers(digit, valid);
+        uint64_t hot_peers = 0;
+        if constexpr (Hot) hot_peers = peers & __builtin_amdgcn_ballot_w64(valid && (key >> 31));
+        if (valid && peers && lane == __builtin_ffsll((long long)peers) - 1) {
+            counts[wave][digit] += __builtin_popcountll(peers);
+            if constexpr (Hot) counts_hot[wave][digit] += __builtin_popcountll(hot_peers);
+        }
     }
     __syncthreads();
-    const int d = threadIdx.x;
-    a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile] = counts[0][d] + counts[1][d] + counts[2][d] + counts[3][d];
+    if (threadIdx.x < kRadix) {
+        const int d = threadIdx.x;
+        uint32_t n = 0, nh = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            n += counts[w][d];
+            if constexpr (Hot) nh += counts_hot[w][d];
+        }
+        a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile] = n;
+        if constexpr (Hot) a.tile_hot[((int64_t)c * kRadix + d) * a.tiles + tile] = nh;
+    }
 }
 
-// Exclusive scan, per class, over the (digit-major, tile-minor) table: entry (d, t) becomes the
-// first output position of tile t's keys with digit d. One 1024-thread block per class.
-__global__ __launch_bounds__(1024) void lov_offsets_scan(uint32_t *tile_hist, int tiles) {
-    __shared__ uint32_t wave_tot[16];
-    const int c = blockIdx.x;
-    uint32_t *row = tile_hist + (int64_t)c * kRadix * tiles;
-    const int total = kRadix * tiles;
-    const int per = (total + 1023) / 1024;
-    const int begin = min(total, (int)threadIdx.x * per);
-    const int end = min(total, begin + per);
-    uint32_t sum = 0;
-    for (int i = begin; i < end; ++i) sum += row[i];
+// One block per (digit, class) row of a tile table: exclusive scan over the tiles in place, row
+// total to totals[c][d]. blockIdx.z selects the table (keys / positives).
+__global__ __launch_bounds__(256) void lov_row_scan(uint32_t *table0, uint32_t *totals0, uint32_t *table1,
+                                                    uint32_t *totals1, int tiles) {
+    __shared__ uint32_t wave_tot[4];
+    uint32_t *table = blockIdx.z ? table1 : table0;
+    uint32_t *totals = blockIdx.z ? totals1 : totals0;
+    const int64_t rid = (int64_t)blockIdx.y * kRadix + blockIdx.x;
+    uint32_t *row = table + rid * tiles;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t incl = wave_incl_scan(sum);
-    if (lane == 63) wave_tot[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0;
-    for (int w = 0; w < 16; ++w) before += (w < wave) ? wave_tot[w] : 0u;
-    uint32_t run = before + incl - sum;
-    for (int i = begin; i < end; ++i) {
-        const uint32_t t = row[i];
-        row[i] = run;
-        run += t;
+    uint32_t carry = 0;
+    for (int base = 0; base < tiles; base += 256) {
+        const int i = base + threadIdx.x;
+        const uint32_t v = (i < tiles) ? row[i] : 0u;
+        const uint32_t incl = wave_incl_scan(v);
+        if (lane == 63) wave_tot[wave] = incl;
+        __syncthreads();
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            before += (w < wave) ? wave_tot[w] : 0u;
+            all += wave_tot[w];
+        }
+        if (i < tiles) row[i] = carry + before + incl - v;
+        carry += all;
+        __syncthreads();
     }
+    if (threadIdx.x == 0) totals[rid] = carry;
 }
 
 __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
@@ -222,7 +270,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];   // per-wave digit counts, then exclusive over waves
     __shared__ uint32_t digit_start[kRadix];          // first local position of each digit
     __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
-    __shared__ uint32_t scan_tmp[kSortWaves + 1];
+    __shared__ uint32_t scan_tmp[kSortWaves];
 
     const int c = blockIdx.y, tile = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -246,20 +294,32 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
-        rank[r] = wave_rank((key[r] >> a.shift) & a.digit_mask, li < count, counts[wave]);
+        uint32_t unused;
+        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, li < count, false, counts[wave], nullptr, rank[r], unused);
     }
     __syncthreads();
 
     {
+        uint32_t mine = 0, dtot = 0;
         const int d = threadIdx.x;
-        const uint32_t c0 = counts[0][d], c1 = counts[1][d], c2 = counts[2][d], c3 = counts[3][d];
-        counts[0][d] = 0;
-        counts[1][d] = c0;
-        counts[2][d] = c0 + c1;
-        counts[3][d] = c0 + c1 + c2;
+        if (d < kRadix) {
+            uint32_t run = 0;
+#pragma unroll
+            for (int w = 0; w < kSortWaves; ++w) {
+                const uint32_t t = counts[w][d];
+                counts[w][d] = run;
+                run += t;
+            }
+            mine = run;
+            dtot = a.digit_total[(int64_t)c * kRadix + d];
+        }
         uint32_t total;
-        digit_start[d] = block_excl_scan_256(c0 + c1 + c2 + c3, scan_tmp, total);
-        out_base[d] = a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
+        const uint32_t local_start = block_excl_scan(mine, scan_tmp, total);
+        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, total);
+        if (d < kRadix) {
+            digit_start[d] = local_start;
+            out_base[d] = global_start + a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
+        }
     }
     __syncthreads();
 
@@ -286,115 +346,110 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     }
 }
 
-// ------------------------------------------ 3./4./5. Jaccard and loss ----
+// ----------------------------- 3. last radix pass fused with the Jaccard step ----
+// The last pass knows every key's final position k (its scatter destination) and, with the
+// positives counted the same way as the keys, the number of positives sorted before it. That is
+// all J_k needs, so instead of writing the sorted row the kernel evaluates the Jaccard difference
+// and scatters it straight to pixel order, and leaves the tile's share of sum e_(k) dJ_k behind.
 
-__global__ __launch_bounds__(kSortThreads) void lov_count_pos(const uint32_t *__restrict__ keys,
-                                                              uint32_t *__restrict__ tile_pos, int P, int tiles) {
-    __shared__ uint32_t wave_cnt[kSortWaves];
-    const int c = blockIdx.y, tile = blockIdx.x;
-    const int begin = tile * kSortTile;
-    const int count = min(kSortTile, P - begin);
-    const uint32_t *kin = keys + (int64_t)c * P + begin;
-    uint32_t n = 0;
-    for (int i = threadIdx.x; i < count; i += kSortThreads) n += kin[i] >> 31;
-    const uint32_t incl = wave_incl_scan(n);
-    if ((threadIdx.x & 63) == 63) wave_cnt[threadIdx.x >> 6] = incl;
-    __syncthreads();
-    if (threadIdx.x == 0) tile_pos[(int64_t)c * tiles + tile] = wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
-}
-
-// Per class: exclusive scan of the positives per tile (in place) and the class total.
-__global__ __launch_bounds__(1024) void lov_scan_tiles(uint32_t *tile_pos, uint32_t *n_pos, int tiles) {
-    __shared__ uint32_t wave_tot[16];
-    const int c = blockIdx.x;
-    uint32_t *row = tile_pos + (int64_t)c * tiles;
-    const int per = (tiles + 1023) / 1024;
-    const int begin = min(tiles, (int)threadIdx.x * per);
-    const int end = min(tiles, begin + per);
-    uint32_t sum = 0;
-    for (int i = begin; i < end; ++i) sum += row[i];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t incl = wave_incl_scan(sum);
-    if (lane == 63) wave_tot[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0, all = 0;
-    for (int w = 0; w < 16; ++w) {
-        before += (w < wave) ? wave_tot[w] : 0u;
-        all += wave_tot[w];
-    }
-    uint32_t run = before + incl - sum;
-    for (int i = begin; i < end; ++i) {
-        const uint32_t t = row[i];
-        row[i] = run;
-        run += t;
-    }
-    if (threadIdx.x == 0) n_pos[c] = all;
-}
-
-// Thread t owns the kSortItems consecutive sorted positions begin + t*kSortItems ...
-__global__ __launch_bounds__(kSortThreads) void lov_jaccard(const uint32_t *__restrict__ keys,
-                                                            const uint32_t *__restrict__ vals,
-                                                            const uint32_t *__restrict__ tile_pos,
-                                                            const uint32_t *__restrict__ n_pos,
-                                                            float *__restrict__ jacc, float *__restrict__ tile_loss,
-                                                            int P, int tiles) {
-    __shared__ uint32_t scan_tmp[kSortWaves + 1];
+__global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, float *__restrict__ jacc,
+                                                          float *__restrict__ tile_loss) {
+    __shared__ uint32_t counts[kSortWaves][kRadix];
+    __shared__ uint32_t counts_hot[kSortWaves][kRadix];
+    __shared__ uint32_t out_base[kRadix];     // global position of the tile's first key with digit d
+    __shared__ uint32_t hot_base[kRadix];     // positives sorted before that position
+    __shared__ uint32_t scan_tmp[kSortWaves];
     __shared__ float wave_loss[kSortWaves];
-    const int c = blockIdx.y, tile = blockIdx.x;
-    const int begin = tile * kSortTile;
-    const int count = min(kSortTile, P - begin);
-    const int64_t row = (int64_t)c * P;
-    const int first = threadIdx.x * kSortItems;
 
-    uint32_t key[kSortItems], val[kSortItems];
-    if (first + kSortItems <= count && ((row + begin) & 3) == 0) {
+    const int c = blockIdx.y, tile = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
+        (&counts[0][0])[i] = 0;
+        (&counts_hot[0][0])[i] = 0;
+    }
+    __syncthreads();
+
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, a.P - begin);
+    const int64_t row = (int64_t)c * a.P;
+    const uint32_t *kin = a.keys_in + row + begin;
+    const uint32_t *vin = a.vals_in + row + begin;
+
+    uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], hrank[kSortItems];
 #pragma unroll
-        for (int q = 0; q < kSortItems / 4; ++q) {
-            const uint4 k4 = *reinterpret_cast<const uint4 *>(keys + row + begin + first + 4 * q);
-            const uint4 v4 = *reinterpret_cast<const uint4 *>(vals + row + begin + first + 4 * q);
-            key[4 * q] = k4.x; key[4 * q + 1] = k4.y; key[4 * q + 2] = k4.z; key[4 * q + 3] = k4.w;
-            val[4 * q] = v4.x; val[4 * q + 1] = v4.y; val[4 * q + 2] = v4.z; val[4 * q + 3] = v4.w;
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        const bool valid = li < count;
+        key[r] = valid ? kin[li] : kIgnoredKey;
+        val[r] = valid ? vin[li] : 0u;
+    }
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        wave_rank<true>((key[r] >> a.shift) & a.digit_mask, li < count, key[r] >> 31, counts[wave], counts_hot[wave],
+                        rank[r], hrank[r]);
+    }
+    __syncthreads();
+
+    uint32_t n_pos_u;
+    {
+        uint32_t dtot = 0, htot = 0;
+        const int d = threadIdx.x;
+        if (d < kRadix) {
+            uint32_t run = 0, run_hot = 0;
+#pragma unroll
+            for (int w = 0; w < kSortWaves; ++w) {
+                const uint32_t t = counts[w][d], th = counts_hot[w][d];
+                counts[w][d] = run;
+                counts_hot[w][d] = run_hot;
+                run += t;
+                run_hot += th;
+            }
+            dtot = a.digit_total[(int64_t)c * kRadix + d];
+            htot = a.hot_total[(int64_t)c * kRadix + d];
         }
-    } else {
-#pragma unroll
-        for (int r = 0; r < kSortItems; ++r) {
-            const bool valid = first + r < count;
-            key[r] = valid ? keys[row + begin + first + r] : kIgnoredKey;
-            val[r] = valid ? vals[row + begin + first + r] : 0u;
+        uint32_t total;
+        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, total);
+        const uint32_t hot_start = block_excl_scan(htot, scan_tmp, n_pos_u);
+        if (d < kRadix) {
+            out_base[d] = global_start + a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
+            hot_base[d] = hot_start + a.tile_hot[((int64_t)c * kRadix + d) * a.tiles + tile];
         }
     }
-    uint32_t mine = 0;
-#pragma unroll
-    for (int r = 0; r < kSortItems; ++r) mine += key[r] >> 31;
-    uint32_t total;
-    uint32_t cs = block_excl_scan_256(mine, scan_tmp, total) + tile_pos[(int64_t)c * tiles + tile];
+    __syncthreads();
 
-    const float npos = (float)n_pos[c];
+    const float npos = (float)n_pos_u;
     float part = 0.f;
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
-        if (first + r < count) {
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        if (li < count) {
             const uint32_t k = key[r];
             const uint32_t hot = k >> 31;
+            const uint32_t d = (k >> a.shift) & a.digit_mask;
             float dj = 0.f;
             if ((k & 0x7FFFFFFFu) != kIgnoredKey) {
-                const int rank = begin + first + r;                    // position in the descending order
-                const float inter_prev = npos - (float)cs;             // csrc/lovasz_softmax.cu:124-127
+                const uint32_t pos = out_base[d] + counts[wave][d] + rank[r];            // rank in the descending order
+                const uint32_t cs = hot_base[d] + counts_hot[wave][d] + hrank[r];      // positives before it
+                const float inter_prev = npos - (float)cs;                             // csrc/lovasz_softmax.cu:124-127
                 const float inter = npos - (float)(cs + hot);
-                const float j_now = 1.f - inter / (inter + (float)(rank + 1));
-                const float j_prev = (rank == 0) ? 0.f : 1.f - inter_prev / (inter_prev + (float)rank);
-                dj = j_now - j_prev;                                   // csrc/lovasz_softmax.cu:141-147
+                const float j_now = 1.f - inter / (inter + (float)(pos + 1));
+                const float j_prev = (pos == 0) ? 0.f : 1.f - inter_prev / (inter_prev + (float)pos);
+                dj = j_now - j_prev;                                                   // csrc/lovasz_softmax.cu:141-147
                 part += key_error(k) * dj;
             }
-            cs += hot;
             jacc[row + val[r]] = dj;
         }
     }
     part = group_reduce<64>(part, OpSum());
-    if ((threadIdx.x & 63) == 0) wave_loss[threadIdx.x >> 6] = part;
+    if (lane == 0) wave_loss[wave] = part;
     __syncthreads();
-    if (threadIdx.x == 0)
-        tile_loss[(int64_t)c * tiles + tile] = (wave_loss[0] + wave_loss[1]) + (wave_loss[2] + wave_loss[3]);
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) s += wave_loss[w];
+        tile_loss[(int64_t)c * a.tiles + tile] = s;
+    }
 }
 
 __global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__ tile_loss, float *__restrict__ losses,
@@ -494,7 +549,7 @@ __global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ go
 struct LovaszPlan {
     int64_t P, E;
     int tiles;
-    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_tile_pos, off_tile_loss, off_n_pos, bytes;
+    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss, bytes;
 };
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -508,13 +563,14 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.E = pl.P * dimsize;
     pl.tiles = (int)ceil_div(pl.P, kSortTile);
     int64_t off = 0;
-    pl.off_keys = off;      off += round_up(4 * pl.E, 256);
-    pl.off_vals_a = off;    off += round_up(4 * pl.E, 256);
-    pl.off_vals_b = off;    off += round_up(4 * pl.E, 256);
-    pl.off_hist = off;      off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
-    pl.off_tile_pos = off;  off += round_up(4 * dimsize * pl.tiles, 256);
-    pl.off_tile_loss = off; off += round_up(4 * dimsize * pl.tiles, 256);
-    pl.off_n_pos = off;     off += round_up(4 * dimsize, 256);
+    pl.off_keys = off;        off += round_up(4 * pl.E, 256);
+    pl.off_vals_a = off;      off += round_up(4 * pl.E, 256);
+    pl.off_vals_b = off;      off += round_up(4 * pl.E, 256);
+    pl.off_hist = off;        off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
+    pl.off_hot = off;         off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
+    pl.off_digit_total = off; off += round_up(4 * dimsize * kRadix, 256);
+    pl.off_hot_total = off;   off += round_up(4 * dimsize * kRadix, 256);
+    pl.off_tile_loss = off;   off += round_up(4 * dimsize * pl.tiles, 256);
     pl.bytes = off;
     return PLH_OK;
 }
@@ -549,13 +605,14 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
     uint32_t *vals_a = reinterpret_cast<uint32_t *>(ws + pl.off_vals_a);
     uint32_t *vals_b = reinterpret_cast<uint32_t *>(ws + pl.off_vals_b);
     uint32_t *hist = reinterpret_cast<uint32_t *>(ws + pl.off_hist);
-    uint32_t *tile_pos = reinterpret_cast<uint32_t *>(ws + pl.off_tile_pos);
+    uint32_t *hot = reinterpret_cast<uint32_t *>(ws + pl.off_hot);
+    uint32_t *digit_total = reinterpret_cast<uint32_t *>(ws + pl.off_digit_total);
+    uint32_t *hot_total = reinterpret_cast<uint32_t *>(ws + pl.off_hot_total);
     float *tile_loss = reinterpret_cast<float *>(ws + pl.off_tile_loss);
-    uint32_t *n_pos = reinterpret_cast<uint32_t *>(ws + pl.off_n_pos);
     const int C = (int)dimsize;
 
     // 1. keys
-    const Shape shape = pick_shape(dimsize, m_size, logits, keys_a, labels, nullptr, nullptr);
+    const Shape shape = pick_shape(dimsize, m_size, logits, keys_b, labels, nullptr, nullptr);
     if (shape == Shape::Regs2 || shape == Shape::Regs1) {
         const int V = (shape == Shape::Regs2) ? 2 : 1;      // m_size even => P even => rows of [C][P] stay 8-byte aligned
         const unsigned grid = (V == 2) ? regs_grid<2>(pl.P) : regs_grid<1>(pl.P);
@@ -563,42 +620,54 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
         if (V == 2) hipLaunchKernelGGL((lov_keys_regs<4 * K, 2>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels, \
-                                       keys_a, pl.P, m_size, C, ignore_index);                                       \
+                                       keys_b, pl.P, m_size, C, ignore_index);                                       \
         else hipLaunchKernelGGL((lov_keys_regs<4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels,      \
-                                keys_a, pl.P, m_size, C, ignore_index);                                              \
+                                keys_b, pl.P, m_size, C, ignore_index);                                              \
         break;
             PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
         }
     } else {
-        hipLaunchKernelGGL(lov_keys_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, logits, labels, keys_a,
+        hipLaunchKernelGGL(lov_keys_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, logits, labels, keys_b,
                            pl.P, m_size, C, ignore_index);
     }
 
-    // 2. four stable radix passes, ping-ponging (keys_a, vals_a) <-> (keys_b, vals_b)
+    // 2. three stable radix passes: (keys_b, -) -> (keys_a, vals_a) -> (keys_b, vals_b) -> (keys_a, vals_a).
+    //    keys_b is the jacc output buffer, free until the last pass scatters into it
     const dim3 tile_grid((unsigned)pl.tiles, (unsigned)C);
-    for (int pass = 0; pass < 4; ++pass) {
-        SortArgs a;
+    SortArgs a;
+    a.tile_hist = hist;
+    a.digit_total = digit_total;
+    a.tile_hot = hot;
+    a.hot_total = hot_total;
+    a.P = (int)pl.P;
+    a.tiles = pl.tiles;
+    for (int pass = 0; pass < 3; ++pass) {
         const bool even = (pass % 2 == 0);
-        a.keys_in = even ? keys_a : keys_b;
-        a.vals_in = (pass == 0) ? nullptr : (even ? vals_a : vals_b);
-        a.keys_out = even ? keys_b : keys_a;
-        a.vals_out = even ? vals_b : vals_a;
-        a.tile_hist = hist;
-        a.P = (int)pl.P;
-        a.tiles = pl.tiles;
+        a.keys_in = even ? keys_b : keys_a;
+        a.vals_in = (pass == 0) ? nullptr : (even ? vals_b : vals_a);
+        a.keys_out = even ? keys_a : keys_b;
+        a.vals_out = even ? vals_a : vals_b;
         a.shift = 8 * pass;
-        a.digit_mask = (pass == 3) ? 0x7Fu : 0xFFu;
-        hipLaunchKernelGGL(lov_tile_hist, tile_grid, dim3(kSortThreads), 0, st, a);
-        hipLaunchKernelGGL(lov_offsets_scan, dim3((unsigned)C), dim3(1024), 0, st, hist, pl.tiles);
+        a.digit_mask = 0xFFu;
+        hipLaunchKernelGGL(lov_tile_hist<false>, tile_grid, dim3(kSortThreads), 0, st, a);
+        hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 1), dim3(256), 0, st, hist, digit_total, hot,
+                           hot_total, pl.tiles);
         hipLaunchKernelGGL(lov_scatter, tile_grid, dim3(kSortThreads), 0, st, a);
     }
 
-    // 3.-5. sorted rows are in (keys_a, vals_a); jacc is free again
-    hipLaunchKernelGGL(lov_count_pos, tile_grid, dim3(kSortThreads), 0, st, keys_a, tile_pos, (int)pl.P, pl.tiles);
-    hipLaunchKernelGGL(lov_scan_tiles, dim3((unsigned)C), dim3(1024), 0, st, tile_pos, n_pos, pl.tiles);
-    hipLaunchKernelGGL(lov_jaccard, tile_grid, dim3(kSortThreads), 0, st, keys_a, vals_a, tile_pos, n_pos, jacc,
-                       tile_loss, (int)pl.P, pl.tiles);
+    // 3. last pass (top digit; bit 31 masked out) fused with the Jaccard step: reads the sorted-so-far
+    //    rows from (keys_a, vals_a) and scatters the Jaccard differences into jacc
+    a.keys_in = keys_a;
+    a.vals_in = vals_a;
+    a.keys_out = nullptr;
+    a.vals_out = nullptr;
+    a.shift = 24;
+    a.digit_mask = 0x7Fu;
+    hipLaunchKernelGGL(lov_tile_hist<true>, tile_grid, dim3(kSortThreads), 0, st, a);
+    hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
+                       pl.tiles);
+    hipLaunchKernelGGL(lov_final, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss);
     hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     return check_launch();
 }
