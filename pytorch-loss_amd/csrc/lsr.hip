@@ -26,55 +26,56 @@ struct LsrParams {
 
 // ---------------------------------------------------------------- regs ----
 
-template <int CP, int V, bool Reduce>
+// loss = -sum_j w_j logp_j with logp_j = t_j - lse, t_j = x_j - max:
+//      = -( w_neg * (sum_j t_j - C*lse) + (w_pos - w_neg) * (t_y - lse) )
+// so one pass over the slice gathers max-shifted sum, exp-sum and the target's t.
+template <int CP, int V, bool Uniform, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const float *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           float *__restrict__ loss, Partials part,
                                                           const LsrParams p) {
     __shared__ float red[4];
-    const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
-    const bool live = want < p.P;
-    if (!Reduce && !live) return;
-    const int64_t pix = live ? want : 0;
-    const int64_t n = pix / p.m_size;
-    const float *xs = x + (pix + n * (int64_t)(p.C - 1) * p.m_size);
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    if (!Reduce && !at.live) return;
 
     float v[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(xs + (int64_t)j * p.m_size, v[j]);
+        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
     int64_t lb[V];
-    load_labels<V>(lab + pix, lb);
+    load_labels<V>(lab + at.pix, lb);
 
     float out[V];
     float mine = 0.f;
     int cnt = 0;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
         float mx = v[0][k];
 #pragma unroll
         for (int j = 1; j < CP; ++j)
             if (j < p.C) mx = fmaxf(mx, v[j][k]);
-        float s = 0.f;
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (j < p.C) s += fast_exp(v[j][k] - mx);
-        const float lse = logf(s);
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        float acc = 0.f;
+        float s = 0.f, sum_t = 0.f, t_y = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
-                const float logp = (v[j][k] - mx) - lse;
-                acc -= logp * ((tgt == j) ? p.w_pos : p.w_neg);
+                const float t = v[j][k] - mx;
+                s += fast_exp(t);
+                sum_t += t;
+                t_y = (tgt == j) ? t : t_y;
             }
-        const bool valid = live && !ign;
+        const float lse = fast_log(s);
+        const float all = sum_t - (float)p.C * lse;
+        // no target channel (label outside [0, C)): every weight is w_neg
+        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * (t_y - lse) : 0.f;
+        const float acc = -(p.w_neg * all + hot);
+        const bool valid = at.live && !ign;
         out[k] = valid ? acc : 0.f;
         mine += out[k];
         cnt += valid ? 1 : 0;
     }
-    if (live && loss) store_vec<V>(loss + pix, out);
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
     if constexpr (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);   // at most 512 per block: exact in fp32
@@ -85,26 +86,22 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const float *__restri
     }
 }
 
-template <int CP, int V>
+template <int CP, int V, bool Uniform>
 __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const float *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           const Upstream up, float *__restrict__ grad,
                                                           const LsrParams p) {
-    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
-    if (pix >= p.P) return;
-    const int64_t n = pix / p.m_size;
-    const int64_t base = pix + n * (int64_t)(p.C - 1) * p.m_size;
-    const float *xs = x + base;
-    float *gs = grad + base;
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    if (!at.live) return;
 
     float v[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(xs + (int64_t)j * p.m_size, v[j]);
+        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
     int64_t lb[V];
-    load_labels<V>(lab + pix, lb);
+    load_labels<V>(lab + at.pix, lb);
     float go[V];
-    load_upstream<V>(up, pix, go);
+    load_upstream<V>(up, at.pix, go);
 
 #pragma unroll
     for (int k = 0; k < V; ++k) {
@@ -121,19 +118,19 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const float *__restri
             }
         bool ign;
         const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        const float gk = ign ? 0.f : go[k];
+        const float gk = go[k];
         const float scale = p.sumw * gk / s;          // one division per pixel
         const float g_pos = p.w_pos * gk, g_neg = p.w_neg * gk;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (j < p.C) {
                 const float g = v[j][k] * scale - ((tgt == j) ? g_pos : g_neg);
-                v[j][k] = ign ? 0.f : g;      // exact zero even for non-finite logits
+                v[j][k] = ign ? 0.f : g;              // exact zero even for non-finite logits
             }
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < p.C) store_vec<V>(gs + (int64_t)j * p.m_size, v[j]);
+        if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
 }
 
 // --------------------------------------------------------------- group ----
@@ -273,11 +270,14 @@ template <int V, bool Reduce>
 static unsigned launch_fwd_regs(const float *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                 hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
+    const bool uni = tiles_are_uniform(p.m_size, V);
     switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                                                                                         \
-    case K:                                                                                                 \
-        hipLaunchKernelGGL((lsr_fwd_regs<4 * K, V, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, loss, \
-                           part, p);                                                                        \
+#define PLH_CASE(K)                                                                                              \
+    case K:                                                                                                      \
+        if (uni) hipLaunchKernelGGL((lsr_fwd_regs<4 * K, V, true, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, \
+                                    x, lab, loss, part, p);                                                      \
+        else hipLaunchKernelGGL((lsr_fwd_regs<4 * K, V, false, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
+                                lab, loss, part, p);                                                             \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -289,10 +289,14 @@ template <int V>
 static void launch_bwd_regs(const float *x, const int64_t *lab, const Upstream &up, float *grad,
                             const LsrParams &p, hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
+    const bool uni = tiles_are_uniform(p.m_size, V);
     switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                                                                                             \
-    case K:                                                                                                     \
-        hipLaunchKernelGGL((lsr_bwd_regs<4 * K, V>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up, grad, p); \
+#define PLH_CASE(K)                                                                                               \
+    case K:                                                                                                       \
+        if (uni) hipLaunchKernelGGL((lsr_bwd_regs<4 * K, V, true>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab,  \
+                                    up, grad, p);                                                                 \
+        else hipLaunchKernelGGL((lsr_bwd_regs<4 * K, V, false>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up, \
+                                grad, p);                                                                         \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

@@ -226,6 +226,50 @@ __device__ __forceinline__ int64_t tile_of_block() {
 template <int V>
 inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(pixels, V), kRegsBlock); }
 
+// Where a thread of a regs-shape kernel works. `base` is the element offset of (image n, channel 0,
+// first pixel); channel j of the same pixels sits at base + j*m_size. Two forms:
+//   Uniform  - m_size is a multiple of the tile (kRegsBlock*V pixels), so a tile never straddles two
+//              images and the grid has no ragged end: the image index and the channel base are
+//              block-uniform (one scalar division per block, scalar base + 32-bit lane offset
+//              addressing) and no bounds check is needed. Every BASELINE shape takes this form.
+//   general  - any m_size: per-thread 64-bit index arithmetic and a bounds check.
+template <int V, bool Uniform>
+struct PixelRef {
+    int64_t pix;        // first pixel of this thread (index into labels / losses)
+    int64_t base;       // block-uniform part of the channel-0 offset (Uniform) or the whole of it
+    unsigned lane_off;  // 32-bit per-thread part (Uniform), else 0
+    bool live;
+
+    __device__ __forceinline__ PixelRef(int64_t P, int64_t m_size, int C) {
+        if constexpr (Uniform) {
+            const int64_t start = tile_of_block() * (kRegsBlock * V);
+            const int64_t n = start / m_size;
+            lane_off = threadIdx.x * V;
+            base = start + n * (int64_t)(C - 1) * m_size;
+            pix = start + lane_off;
+            live = true;
+        } else {
+            const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+            live = want < P;
+            pix = live ? want : 0;
+            const int64_t n = pix / m_size;
+            base = pix + n * (int64_t)(C - 1) * m_size;
+            lane_off = 0;
+        }
+    }
+    // address of channel j for this thread's pixels
+    __device__ __forceinline__ const float *chan(const float *t, int j, int64_t m_size) const {
+        return (t + (base + (int64_t)j * m_size)) + lane_off;
+    }
+    __device__ __forceinline__ float *chan(float *t, int j, int64_t m_size) const {
+        return (t + (base + (int64_t)j * m_size)) + lane_off;
+    }
+};
+
+inline bool tiles_are_uniform(int64_t m_size, int V) { return m_size % ((int64_t)kRegsBlock * V) == 0; }
+
+__device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.69314718055994530942f; }
+
 // exp(x) for x <= 0 through the hardware exp2: 2 instructions instead of ~10. Relative
 // error stays below 1e-6 for the arguments a max-subtracted softmax produces.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
