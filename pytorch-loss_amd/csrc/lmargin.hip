@@ -26,25 +26,22 @@ struct LmParams {
 
 // ---------------------------------------------------------------- regs ----
 
-template <int CP, int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <int CP, int V, bool Uniform, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
                                                      const Upstream up,
                                                      float *__restrict__ loss, float *__restrict__ grad,
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
     __shared__ float red[4];
-    const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
-    const bool live = want < p.P;
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    const bool live = at.live;
     if (!Reduce && !live) return;
-    const int64_t pix = live ? want : 0;
-    const int64_t n = pix / p.m_size;
-    const int64_t base = pix + n * (int64_t)(p.C - 1) * p.m_size;
-    const float *xs = x + base;
+    const int64_t pix = at.pix;
 
     float v[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(xs + (int64_t)j * p.m_size, v[j]);
+        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
     int64_t lb[V];
     load_labels<V>(lab + pix, lb);
     float go[V];
@@ -87,10 +84,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ 
         const float s_all = s_no * t_all + e_y;
         const float inv_no = 1.f / s_no;
         if constexpr (WantLoss) {
-            const float lse_no = logf(s_no);
+            const float lse_no = fast_log(s_no);
             const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));   // channels that are not the target
             const float margin = sum_et * inv_no - lse_no - p.coeff * (sum_t - others * lse_no);
-            const float acc = p.half_lam * margin - (x_y - m_all) + logf(s_all);
+            const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
             mine += out[k];
             cnt += (ign || !live) ? 0 : 1;
@@ -116,10 +113,9 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ 
     if (live) {
         if (WantLoss && loss) store_vec<V>(loss + pix, out);
         if constexpr (WantGrad) {
-            float *gs = grad + base;
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (j < p.C) store_vec<V>(gs + (int64_t)j * p.m_size, v[j]);
+                if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
         }
     }
     if constexpr (WantCount) {
@@ -240,11 +236,14 @@ template <int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 static unsigned launch_regs(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
                             unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
+    const bool uni = tiles_are_uniform(p.m_size, V);
     switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                                                                                              \
-    case K:                                                                                                      \
-        hipLaunchKernelGGL((lm_regs<4 * K, V, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), dim3(kRegsBlock), \
-                           0, st, x, lab, up, loss, grad, cnt, part, p);                                         \
+#define PLH_CASE(K)                                                                                               \
+    case K:                                                                                                       \
+        if (uni) hipLaunchKernelGGL((lm_regs<4 * K, V, true, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
+                                    dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);               \
+        else hipLaunchKernelGGL((lm_regs<4 * K, V, false, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),    \
+                                dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                   \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

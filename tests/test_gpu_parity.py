@@ -123,6 +123,35 @@ def test_lsr_module_reductions(pl, reduction, smooth):
     assert np.abs(xt.grad.sum(dim=1).cpu().numpy()).max() < 1e-5     # gradient rows sum to zero
 
 
+@pytest.mark.parametrize("shape,ignore,frac", SEG_CASES)
+@pytest.mark.parametrize("kind", ["lsr", "lmargin"])
+def test_fused_reductions_on_every_execution_shape(pl, kind, shape, ignore, frac):
+    """'mean' / 'sum' come from per-block partials inside the forward kernel: every launch shape
+    (registers, wavefront per row, lane per pixel, ragged tails) must agree with the unreduced path."""
+    if frac >= 1.0:
+        pytest.skip("all ignored: covered by the NaN test")
+    x, y = seg_inputs(25, shape, ignore, frac)
+    yt = dev(y)
+    if kind == "lsr":
+        make = lambda red: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=ignore)
+        per = oracle.lsr_forward(x.astype(np.float64), y, ignore, 0.1)
+        grad_of = lambda g: oracle.lsr_backward(x, y, ignore, 0.1, g)
+    else:
+        make = lambda red: pl.LargeMarginSoftmaxV3(lam=0.3, reduction=red, ignore_index=ignore)
+        per = oracle.lmargin_forward(x.astype(np.float64), y, 0.3, ignore)
+        grad_of = lambda g: oracle.lmargin_backward(x, y, 0.3, ignore, g)
+    n_valid = int((y != ignore).sum())
+    for red in ("sum", "mean"):
+        xt = dev(x).requires_grad_()
+        out = make(red)(xt, yt)
+        assert out.dim() == 0
+        want = per.sum() / (n_valid if red == "mean" else 1)
+        assert abs(out.item() - want) <= 1e-5 * abs(want), (red, out.item(), want)
+        (out * 3.0).backward()                      # a non-unit upstream scalar
+        scale = 3.0 / (n_valid if red == "mean" else 1)
+        close_grad(xt.grad.cpu().numpy(), grad_of(np.float32(scale)), kind + " " + red)
+
+
 def test_lsr_all_ignored_mean_is_nan(pl):
     x, y = seg_inputs(23, (2, 19, 8, 8), 255, 1.0)
     out = pl.LabelSmoothSoftmaxCEV3(ignore_index=255)(dev(x), dev(y))
@@ -180,6 +209,22 @@ def test_focal_module_reductions(pl, reduction):
     (out.sum() if reduction == "none" else out).backward()
     scale = 1.0 / x.size if reduction == "mean" else 1.0
     close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, 0.25, 2.0, np.float32(scale)), "focal " + reduction)
+
+
+@pytest.mark.parametrize("shape", FOCAL_SHAPES)
+@pytest.mark.parametrize("gamma", [2, 1, 1.5])
+def test_focal_fused_reductions(pl, shape, gamma):
+    x = synth.normal(32, 1, shape, -2.0, 1.5)
+    y = synth.bernoulli(32, 2, shape, 0.2).astype(np.float32)
+    per = oracle.focal_forward(x.astype(np.float64), y.astype(np.float64), 0.25, gamma)
+    for red in ("sum", "mean"):
+        xt = dev(x).requires_grad_()
+        out = pl.FocalLossV3(alpha=0.25, gamma=gamma, reduction=red)(xt, dev(y))
+        want = per.sum() / (x.size if red == "mean" else 1)
+        assert abs(out.item() - want) <= 1e-5 * abs(want)
+        (out * -2.0).backward()
+        scale = -2.0 / (x.size if red == "mean" else 1)
+        close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, 0.25, gamma, np.float32(scale)), "focal " + red)
 
 
 def test_focal_extreme_logits_stay_finite(pl):
