@@ -153,16 +153,20 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *lds, u
     return before + incl - v;
 }
 
-// Match mask: the valid lanes of the wave whose digit equals this lane's (8 ballots).
+// Match mask: the valid lanes of the wave whose digit equals this lane's. One ballot per digit bit;
+// each lane ORs up, in two 32-bit halves, the lanes that differ from it in that bit
+// (vote XOR own bit splatted), so a bit costs one field extract, one compare and two 3-input bit ops.
 __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
-    uint64_t peers = __builtin_amdgcn_ballot_w64(valid);
+    uint32_t diff_lo = 0, diff_hi = 0;
 #pragma unroll
     for (int b = 0; b < 8; ++b) {
-        const bool bit = (digit >> b) & 1u;
-        const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
-        peers &= bit ? vote : ~vote;
+        const uint32_t splat = (uint32_t)((int32_t)(digit << (31 - b)) >> 31);   // bit b splatted: 0 or ~0
+        const uint64_t vote = __builtin_amdgcn_ballot_w64((digit & (1u << b)) != 0u);
+        diff_lo |= (uint32_t)vote ^ splat;
+        diff_hi |= (uint32_t)(vote >> 32) ^ splat;
     }
-    return peers;
+    const uint64_t diff = ((uint64_t)diff_hi << 32) | diff_lo;
+    return __builtin_amdgcn_ballot_w64(valid) & ~diff;
 }
 
 // Stable rank of this lane's key among the equal digits the wave has seen so far (earlier rounds
@@ -192,6 +196,9 @@ __device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, 
                 __builtin_popcountll(hot_peers & below);
 }
 
+// Per-tile digit counts (and, for the last pass, the same for the positives). Counting needs no
+// ranks, so it uses LDS atomics on per-wave counters instead of match masks; a round whose keys all
+// share one digit (the rule for the top digit, where errors cluster) is added by a single lane.
 template <bool Hot>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];
@@ -202,22 +209,38 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         (&counts[0][0])[i] = 0;
         if constexpr (Hot) (&counts_hot[0][0])[i] = 0;
     }
-    __syncthreads();
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, a.P - begin);
     const uint32_t *kin = a.keys_in + (int64_t)c * a.P + begin;
-#pragma unroll 4
+    uint32_t key[kSortItems];
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {      // all loads in flight before the first one is used
+        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        key[r] = (li < count) ? kin[li] : kIgnoredKey;
+    }
+    __syncthreads();
+#pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         const bool valid = li < count;
-        const uint32_t key = valid ? kin[li] : kIgnoredKey;
-        const uint32_t digit = (key >> a.shift) & a.digit_mask;
-        const uint64_t peers = wave_peers(digit, valid);
-        uint64_t hot_peers = 0;
-        if constexpr (Hot) hot_peers = peers & __builtin_amdgcn_ballot_w64(valid && (key >> 31));
-        if (valid && peers && lane == __builtin_ffsll((long long)peers) - 1) {
-            counts[wave][digit] += __builtin_popcountll(peers);
-            if constexpr (Hot) counts_hot[wave][digit] += __builtin_popcountll(hot_peers);
+        const uint32_t digit = (key[r] >> a.shift) & a.digit_mask;
+        const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
+        if (vmask == 0) continue;               // wave-uniform
+        const uint32_t first = __builtin_amdgcn_readfirstlane(digit);   // first active lane = lowest valid one here
+        const uint64_t same = __builtin_amdgcn_ballot_w64(valid && digit == first);
+        if (same == vmask) {                    // wave-uniform branch
+            if (lane == 0) atomicAdd(&counts[wave][first], (uint32_t)__builtin_popcountll(vmask));
+        } else if (valid) {
+            atomicAdd(&counts[wave][digit], 1u);
+        }
+        if constexpr (Hot) {
+            const bool hot = valid && (key[r] >> 31);
+            if (same == vmask) {
+                const uint64_t hmask = __builtin_amdgcn_ballot_w64(hot);
+                if (lane == 0 && hmask) atomicAdd(&counts_hot[wave][first], (uint32_t)__builtin_popcountll(hmask));
+            } else if (hot) {
+                atomicAdd(&counts_hot[wave][digit], 1u);
+            }
         }
     }
     __syncthreads();
