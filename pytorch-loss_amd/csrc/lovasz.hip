@@ -375,8 +375,27 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 // all J_k needs, so instead of writing the sorted row the kernel evaluates the Jaccard difference
 // and scatters it straight to pixel order, and leaves the tile's share of sum e_(k) dJ_k behind.
 
+//
+// Scattering 4 bytes per key to a random pixel is the slow part (each store is its own memory
+// transaction). Binned = true splits it in two: pixels are grouped in regions of kRegion; every
+// class row holds each pixel exactly once, so region b of a row receives exactly its own number of
+// values and can be staged in place: the kernel appends (value -> jacc, pixel offset -> idx_stage)
+// at a cursor inside the region's own range [b*kRegion, ...), in runs per (tile, region); a second
+// kernel (lov_unbin) then permutes each region inside LDS and writes it back coalesced.
+constexpr int kRegionBits = 13;
+constexpr int kRegion = 1 << kRegionBits;     // 8192 pixels = 32 KiB of fp32
+constexpr int kMaxRegions = 1024;             // per class row; larger rows take the direct scatter
+
+template <bool Binned>
 __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, float *__restrict__ jacc,
-                                                          float *__restrict__ tile_loss) {
+                                                          float *__restrict__ tile_loss,
+                                                          uint32_t *__restrict__ idx_stage,
+                                                          uint32_t *__restrict__ cursors, int regions) {
+    __shared__ uint32_t region_cnt[Binned ? kMaxRegions : 1];    // keys of this tile per region
+    __shared__ uint32_t region_start[Binned ? kMaxRegions : 1];  // first position of the region in the re-ordered tile
+    __shared__ uint32_t region_base[Binned ? kMaxRegions : 1];   // this tile's run inside the region's staging range
+    __shared__ float s_dj[Binned ? kSortTile : 1];               // tile re-ordered by region, so that the stores
+    __shared__ uint32_t s_val[Binned ? kSortTile : 1];           // of neighbouring threads fall into the same run
     __shared__ uint32_t counts[kSortWaves][kRadix];
     __shared__ uint32_t counts_hot[kSortWaves][kRadix];
     __shared__ uint32_t out_base[kRadix];     // global position of the tile's first key with digit d
@@ -390,6 +409,8 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         (&counts[0][0])[i] = 0;
         (&counts_hot[0][0])[i] = 0;
     }
+    if constexpr (Binned)
+        for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
     __syncthreads();
 
     const int begin = tile * kSortTile;
@@ -399,6 +420,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     const uint32_t *vin = a.vals_in + row + begin;
 
     uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], hrank[kSortItems];
+    uint32_t slot[Binned ? kSortItems : 1];
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
@@ -411,8 +433,28 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         wave_rank<true>((key[r] >> a.shift) & a.digit_mask, li < count, key[r] >> 31, counts[wave], counts_hot[wave],
                         rank[r], hrank[r]);
+        if constexpr (Binned) {
+            // order inside a region's staging range is irrelevant: lov_unbin puts every value at its pixel
+            if (li < count) slot[r] = atomicAdd(&region_cnt[val[r] >> kRegionBits], 1u);
+        }
     }
     __syncthreads();
+    if constexpr (Binned) {
+        // exclusive scan of the per-region counts (each thread owns `per` consecutive regions), and one
+        // cursor reservation per region the tile touches
+        const int per = (regions + kSortThreads - 1) / kSortThreads;
+        const int r0 = threadIdx.x * per;
+        uint32_t mine = 0;
+        for (int i = r0; i < min(regions, r0 + per); ++i) mine += region_cnt[i];
+        uint32_t total;
+        uint32_t run = block_excl_scan(mine, scan_tmp, total);
+        for (int i = r0; i < min(regions, r0 + per); ++i) {
+            const uint32_t n = region_cnt[i];
+            region_start[i] = run;
+            run += n;
+            region_base[i] = n ? atomicAdd(&cursors[(int64_t)c * regions + i], n) : 0u;
+        }
+    }
 
     uint32_t n_pos_u;
     {
@@ -461,7 +503,13 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                 dj = j_now - j_prev;                                                   // csrc/lovasz_softmax.cu:141-147
                 part += key_error(k) * dj;
             }
-            jacc[row + val[r]] = dj;
+            if constexpr (Binned) {
+                const uint32_t lp = region_start[val[r] >> kRegionBits] + slot[r];
+                s_dj[lp] = dj;
+                s_val[lp] = val[r];
+            } else {
+                jacc[row + val[r]] = dj;
+            }
         }
     }
     part = group_reduce<64>(part, OpSum());
@@ -473,6 +521,31 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         for (int w = 0; w < kSortWaves; ++w) s += wave_loss[w];
         tile_loss[(int64_t)c * a.tiles + tile] = s;
     }
+    if constexpr (Binned) {
+        for (int i = threadIdx.x; i < count; i += kSortThreads) {
+            const uint32_t v = s_val[i];
+            const uint32_t region = v >> kRegionBits;
+            const int64_t at = row + ((int64_t)region << kRegionBits) + region_base[region] + ((uint32_t)i - region_start[region]);
+            jacc[at] = s_dj[i];
+            idx_stage[at] = v & (kRegion - 1);
+        }
+    }
+}
+
+// One block per (region, class): the region's staged values are permuted to pixel order inside LDS.
+__global__ __launch_bounds__(256) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
+                                                 int P) {
+    __shared__ float sorted[kRegion];
+    const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
+    const int n = min(kRegion, P - (int)(blockIdx.x << kRegionBits));
+    for (int i = threadIdx.x; i < n; i += 256) sorted[idx_stage[first + i]] = jacc[first + i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 256) jacc[first + i] = sorted[i];
+}
+
+__global__ __launch_bounds__(256) void lov_zero_u32(uint32_t *p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
 }
 
 __global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__ tile_loss, float *__restrict__ losses,
@@ -572,7 +645,9 @@ __global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ go
 struct LovaszPlan {
     int64_t P, E;
     int tiles;
-    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss, bytes;
+    int regions;            // pixel regions per class row (0 = direct scatter)
+    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss,
+        off_cursors, bytes;
 };
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -594,6 +669,9 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.off_digit_total = off; off += round_up(4 * dimsize * kRadix, 256);
     pl.off_hot_total = off;   off += round_up(4 * dimsize * kRadix, 256);
     pl.off_tile_loss = off;   off += round_up(4 * dimsize * pl.tiles, 256);
+    const int64_t regions = ceil_div(pl.P, kRegion);
+    pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
+    pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
     pl.bytes = off;
     return PLH_OK;
 }
@@ -690,7 +768,19 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
     hipLaunchKernelGGL(lov_tile_hist<true>, tile_grid, dim3(kSortThreads), 0, st, a);
     hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
                        pl.tiles);
-    hipLaunchKernelGGL(lov_final, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss);
+    if (pl.regions > 0) {
+        uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);
+        const int n_cur = C * pl.regions;
+        hipLaunchKernelGGL(lov_zero_u32, dim3((unsigned)ceil_div(n_cur, 256)), dim3(256), 0, st, cursors, n_cur);
+        // vals_b is free by now: it receives the pixel offsets that go with the staged values
+        hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
+                           pl.regions);
+        hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(256), 0, st, jacc, vals_b,
+                           (int)pl.P);
+    } else {
+        hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, nullptr,
+                           0);
+    }
     hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     return check_launch();
 }
