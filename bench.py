@@ -124,6 +124,28 @@ def time_steps(crit, logits, labels, steps, warmup):
     return (t1 - t0) * 1e3 / steps, float(loss.item())
 
 
+def step_distribution(crit, inputs, iters=100):
+    """Per-step GPU time (HIP events around each fwd+bwd step): median / p10 / p90 in ms. `inputs` is a
+    list of (logits, labels) sets used round-robin: one set = cache-warm, several sets whose total
+    size exceeds the 256 MB Infinity Cache = cache-cold."""
+    import torch
+    for x, _ in inputs:
+        x.requires_grad_(True)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for i in range(iters + 10):
+        x, y = inputs[i % len(inputs)]
+        x.grad = None
+        if i >= 10:
+            events[i - 10][0].record()
+        crit(x, y).backward()
+        if i >= 10:
+            events[i - 10][1].record()
+    torch.cuda.synchronize()
+    ms = sorted(a.elapsed_time(b) for a, b in events)
+    return {"median": round(ms[len(ms) // 2], 4), "p10": round(ms[len(ms) // 10], 4),
+            "p90": round(ms[(9 * len(ms)) // 10], 4), "iters": iters, "input_sets": len(inputs)}
+
+
 def time_kernel(launch, iters=30, warmup=5):
     """Average duration (ms) of one launch: HIP events on the stream the kernel runs on."""
     import torch
@@ -240,9 +262,17 @@ def run_workload(name, steps, warmup, device):
     fwd, bwd = algorithmic_bytes(name, shape)
     gbps = (fwd + bwd) / (ms * 1e-3) / 1e9
     roof = kernel_rooflines(name, logits, labels)
+    dist = {"warm": step_distribution(crit, [(logits, labels)])}
+    set_bytes = 4 * numel(shape) * (2 if name == "focal" else 1)
+    if set_bytes < (256 << 20):
+        # working set fits the Infinity Cache: also rotate enough input sets to defeat it
+        n_sets = max(4, -(-(768 << 20) // set_bytes))
+        sets = [(logits, labels)] + [make_inputs(name, shape, device, seed=100 + i) for i in range(n_sets - 1)]
+        dist["cold"] = step_distribution(crit, sets)
+        del sets
     del crit
     logits.grad = None
-    return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd)
+    return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist)
 
 
 def main():
@@ -278,6 +308,7 @@ def main():
             try:
                 r = run_workload(other, max(5, args.steps // 2), max(2, args.warmup // 2), device)
                 others[other] = {"workload": WORKLOADS[other]["desc"], "ms_per_step": round(r["ms_per_step"], 4),
+                                 "step_ms": r["step_ms"],
                                  "GB/s": round(r["gbps"], 1), "frac_of_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
                                  "kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
                                              for k, v in r["roofline"].items()}}
@@ -307,6 +338,7 @@ def main():
                    "frac_of_hbm_peak": round(main_res["gbps"] / HBM_PEAK_GBPS, 4), "loss": main_res["loss"]},
         "roofline": dict(main_res["roofline"]["backward"], kernel="backward entry point of the workload"),
         "roofline_forward": main_res["roofline"]["forward"],
+        "step_ms": main_res["step_ms"],
         "copy_kernel_GBps": ceiling,
         "other_workloads": others,
     }
