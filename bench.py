@@ -45,6 +45,10 @@ WORKLOADS = {
 }
 
 
+def describe(name, dtype):
+    return WORKLOADS[name]["desc"].replace("fp32 logits", {"f32": "fp32", "f16": "fp16", "bf16": "bf16"}[dtype] + " logits")
+
+
 def numel(shape):
     n = 1
     for d in shape:
@@ -52,25 +56,42 @@ def numel(shape):
     return n
 
 
-def algorithmic_bytes(name, shape):
-    """Bytes a fwd+bwd pass has to move at the autograd-Function level (fp32 logits, int64 labels):
+ELEM_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
+DTYPE_TAG = {"f32": 0, "f16": 1, "bf16": 2}
+
+
+def algorithmic_bytes(name, shape, dtype="f32"):
+    """Bytes a fwd+bwd pass has to move at the autograd-Function level (logits and their gradient
+    in `dtype`, int64 labels, fp32 losses / upstream gradient / Jaccard differences):
     forward reads the inputs and writes the unreduced losses, backward reads the inputs and the
     upstream gradient and writes the logits gradient."""
     E = numel(shape)
     P = E // shape[1]
+    b = ELEM_BYTES[dtype]
     if name in ("lsr", "lmargin"):
-        fwd = 4 * E + 8 * P + 4 * P
-        bwd = 4 * E + 8 * P + 4 * P + 4 * E
-    elif name == "focal":
-        fwd = 3 * 4 * E
-        bwd = 4 * 4 * E
+        fwd = b * E + 8 * P + 4 * P
+        bwd = b * E + 8 * P + 4 * P + b * E
+    elif name == "focal":   # the labels are floating point and share the logits' type
+        fwd = 2 * b * E + 4 * E
+        bwd = 2 * b * E + 4 * E + b * E
     else:  # lovasz: compulsory I/O only (logits, labels, saved Jaccard differences, gradient)
-        fwd = 4 * E + 8 * P + 4 * E
-        bwd = 4 * E + 4 * E + 8 * P + 4 * E
+        fwd = b * E + 8 * P + 4 * E
+        bwd = b * E + 4 * E + 8 * P + b * E
     return fwd, bwd
 
 
-def make_inputs(name, shape, device, seed=15):
+def make_inputs(name, shape, device, seed=15, dtype="f32"):
+    logits, labels = _make_inputs_f32(name, shape, device, seed)
+    if dtype != "f32":
+        import torch
+        td = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+        logits = logits.to(td)
+        if name == "focal":
+            labels = labels.to(td)
+    return logits, labels
+
+
+def _make_inputs_f32(name, shape, device, seed):
     import torch
     g = torch.Generator(device=device)
     g.manual_seed(seed)
@@ -162,15 +183,16 @@ def time_kernel(launch, iters=30, warmup=5):
     return start.elapsed_time(stop) / iters
 
 
-def kernel_rooflines(name, logits, labels):
+def kernel_rooflines(name, logits, labels, dtype="f32"):
     """Per-kernel roofline entries for the forward and backward entry points, called directly
     through the C ABI wrappers with pre-allocated outputs (no allocator, no autograd in the loop)."""
     import torch
     from pytorch_loss import _native
     lib = _native.load()
     shape = tuple(logits.shape)
-    fwd_bytes, bwd_bytes = algorithmic_bytes(name, shape)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(name, shape, dtype)
     x = logits.detach()
+    tag = DTYPE_TAG[dtype]
     n, c = shape[0], shape[1]
     m = numel(shape) // (n * c)
     st = _native._stream
@@ -181,17 +203,17 @@ def kernel_rooflines(name, logits, labels):
         grad = torch.empty_like(x)
         gout = torch.full(labels.shape, 1.0 / labels.numel(), dtype=torch.float32, device=x.device)
         if name == "lsr":
-            f = lambda: lib.plh_lsr_forward(P(x), P(labels), P(losses), n, c, m, 255, 0.1, st())
-            b = lambda: lib.plh_lsr_backward(P(x), P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.1, st())
+            f = lambda: lib.plh_lsr_forward(P(x), tag, P(labels), P(losses), n, c, m, 255, 0.1, st())
+            b = lambda: lib.plh_lsr_backward(P(x), tag, P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.1, st())
         else:
-            f = lambda: lib.plh_lmargin_forward(P(x), P(labels), P(losses), n, c, m, 255, 0.3, st())
-            b = lambda: lib.plh_lmargin_backward(P(x), P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.3, st())
+            f = lambda: lib.plh_lmargin_forward(P(x), tag, P(labels), P(losses), n, c, m, 255, 0.3, st())
+            b = lambda: lib.plh_lmargin_backward(P(x), tag, P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.3, st())
     elif name == "focal":
-        losses = torch.empty_like(x)
+        losses = torch.empty(shape, dtype=torch.float32, device=x.device)
         grad = torch.empty_like(x)
         gout = torch.full(shape, 1.0 / x.numel(), dtype=torch.float32, device=x.device)
-        f = lambda: lib.plh_focal_forward(P(x), P(labels), P(losses), x.numel(), 2.0, 0.25, st())
-        b = lambda: lib.plh_focal_backward(P(x), P(labels), P(gout), 1, P(grad), x.numel(), 2.0, 0.25, st())
+        f = lambda: lib.plh_focal_forward(P(x), tag, P(labels), P(losses), x.numel(), 2.0, 0.25, st())
+        b = lambda: lib.plh_focal_backward(P(x), tag, P(labels), P(gout), 1, P(grad), x.numel(), 2.0, 0.25, st())
     else:
         losses = torch.empty(c, dtype=torch.float32, device=x.device)
         jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
@@ -199,13 +221,13 @@ def kernel_rooflines(name, logits, labels):
         gout = torch.full((c,), 1.0 / c, dtype=torch.float32, device=x.device)
         ws_bytes = int(lib.plh_lovasz_workspace_bytes(n, c, m))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-        f = lambda: lib.plh_lovasz_forward(P(x), P(labels), P(losses), P(jacc), P(ws), ws_bytes, n, c, m, 255, st())
-        b = lambda: lib.plh_lovasz_backward(P(gout), P(x), P(labels), P(jacc), P(grad), n, c, m, 255, st())
+        f = lambda: lib.plh_lovasz_forward(P(x), tag, P(labels), P(losses), P(jacc), P(ws), ws_bytes, n, c, m, 255, st())
+        b = lambda: lib.plh_lovasz_backward(P(gout), P(x), tag, P(labels), P(jacc), P(grad), n, c, m, 255, st())
     assert f() == 0 and b() == 0
     for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
         ms = time_kernel(fn)
         gbps = nbytes / (ms * 1e-3) / 1e9
-        traffic = MEASURED_TRAFFIC.get((name, shape), {}).get(key)
+        traffic = MEASURED_TRAFFIC.get((name, shape), {}).get(key) if dtype == "f32" else None
         out[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
                     "ms": round(ms, 4), "algorithmic_bytes": nbytes}
@@ -253,21 +275,21 @@ def cpu_baseline(name, shape):
                       "images of the workload, fwd+bwd, median of 3, time scaled x%d" % (scale, scale)}
 
 
-def run_workload(name, steps, warmup, device):
+def run_workload(name, steps, warmup, device, dtype="f32"):
     import torch
     shape = WORKLOADS[name]["shape"]
-    logits, labels = make_inputs(name, shape, device)
+    logits, labels = make_inputs(name, shape, device, dtype=dtype)
     crit = make_criterion(name)
     ms, loss = time_steps(crit, logits, labels, steps, warmup)
-    fwd, bwd = algorithmic_bytes(name, shape)
+    fwd, bwd = algorithmic_bytes(name, shape, dtype)
     gbps = (fwd + bwd) / (ms * 1e-3) / 1e9
-    roof = kernel_rooflines(name, logits, labels)
+    roof = kernel_rooflines(name, logits, labels, dtype)
     dist = {"warm": step_distribution(crit, [(logits, labels)])}
-    set_bytes = 4 * numel(shape) * (2 if name == "focal" else 1)
+    set_bytes = ELEM_BYTES[dtype] * numel(shape) * (2 if name == "focal" else 1)
     if set_bytes < (256 << 20):
         # working set fits the Infinity Cache: also rotate enough input sets to defeat it
         n_sets = max(4, -(-(768 << 20) // set_bytes))
-        sets = [(logits, labels)] + [make_inputs(name, shape, device, seed=100 + i) for i in range(n_sets - 1)]
+        sets = [(logits, labels)] + [make_inputs(name, shape, device, seed=100 + i, dtype=dtype) for i in range(n_sets - 1)]
         dist["cold"] = step_distribution(crit, sets)
         del sets
     del crit
@@ -281,6 +303,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="lsr", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="f32", choices=sorted(ELEM_BYTES),
+                    help="element type of logits and gradients in HBM (the arithmetic is fp32 in every case)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true", help="skip the secondary workloads")
     args = ap.parse_args()
@@ -297,7 +321,7 @@ def main():
     torch.cuda.set_device(device)
 
     name = args.workload
-    main_res = run_workload(name, args.steps, args.warmup, device)
+    main_res = run_workload(name, args.steps, args.warmup, device, args.dtype)
     torch.cuda.empty_cache()
 
     others = {}
@@ -306,8 +330,8 @@ def main():
             if other == name:
                 continue
             try:
-                r = run_workload(other, max(5, args.steps // 2), max(2, args.warmup // 2), device)
-                others[other] = {"workload": WORKLOADS[other]["desc"], "ms_per_step": round(r["ms_per_step"], 4),
+                r = run_workload(other, max(5, args.steps // 2), max(2, args.warmup // 2), device, args.dtype)
+                others[other] = {"workload": describe(other, args.dtype), "ms_per_step": round(r["ms_per_step"], 4),
                                  "step_ms": r["step_ms"],
                                  "GB/s": round(r["gbps"], 1), "frac_of_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
                                  "kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
@@ -334,7 +358,8 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": WORKLOADS[name]["desc"], "algorithmic_bytes_per_step": main_res["bytes"],
+        "config": {"workload": describe(name, args.dtype), "storage_dtype": args.dtype,
+                   "algorithmic_bytes_per_step": main_res["bytes"],
                    "frac_of_hbm_peak": round(main_res["gbps"] / HBM_PEAK_GBPS, 4), "loss": main_res["loss"]},
         "roofline": dict(main_res["roofline"]["backward"], kernel="backward entry point of the workload"),
         "roofline_forward": main_res["roofline"]["forward"],

@@ -6,7 +6,8 @@
  *
  * Conventions for every entry point
  *   - plain device pointers, sizes and scalars; no framework types;
- *   - logits are fp32, laid out (n_size, dimsize, m_size) row-major, i.e. NCHW
+ *   - logits (and the logits gradient) are fp32, fp16 or bf16 as named by `dtype`
+ *     (PLH_DTYPE_*), laid out (n_size, dimsize, m_size) row-major, i.e. NCHW
  *     with the spatial dims flattened into m_size (the reference flattens the
  *     same way, csrc/lsr_kernel.cu:199-202); integer labels are int64 (n_size, m_size);
  *   - `stream` is a hipStream_t (NULL = the default stream); launches are
@@ -34,7 +35,7 @@
 extern "C" {
 #endif
 
-#define PLH_ABI_VERSION 1
+#define PLH_ABI_VERSION 2
 
 #define PLH_OK 0
 #define PLH_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
@@ -43,6 +44,16 @@ extern "C" {
 #define PLH_ERR_TOO_MANY_CLASSES (-4) /* Lovasz: dimsize >= 512 (csrc/lovasz_softmax.cu:665) */
 #define PLH_ERR_WORKSPACE (-5)      /* workspace smaller than plh_lovasz_workspace_bytes() */
 #define PLH_ERR_MISALIGNED (-6)     /* a pointer is not aligned to its element size */
+#define PLH_ERR_BAD_DTYPE (-7)      /* dtype is not one of PLH_DTYPE_* */
+
+/* Element type of the logits and of the logits gradient (`dtype` argument; both tensors of one call
+ * share it). Arithmetic is fp32 whatever the storage type; losses, upstream gradients and the Lovasz
+ * jacc tensor are always fp32. The reference dispatches the same three floating types
+ * (AT_DISPATCH_FLOATING_TYPES_AND_HALF, e.g. csrc/lsr_kernel.cu:215) but computes in the storage
+ * type; computing in fp32 is what its autocast wrapper asks for (custom_fwd(cast_inputs=float32)). */
+#define PLH_DTYPE_F32 0
+#define PLH_DTYPE_F16 1
+#define PLH_DTYPE_BF16 2
 
 int plh_abi_version(void);
 
@@ -55,13 +66,13 @@ const char *plh_error_string(int code);
  * losses: (n_size, m_size) fp32, 0 at ignored pixels.
  * grad_logits: shape of logits, 0 at ignored pixels.
  */
-int plh_lsr_forward(const float *logits, const int64_t *labels, float *losses,
+int plh_lsr_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                     int64_t n_size, int64_t dimsize, int64_t m_size,
                     int64_t ignore_index, float smooth, void *stream);
 
-int plh_lsr_backward(const float *logits, const int64_t *labels,
+int plh_lsr_backward(const void *logits, int32_t dtype, const int64_t *labels,
                      const float *grad_output, int64_t grad_output_stride,
-                     float *grad_logits,
+                     void *grad_logits,
                      int64_t n_size, int64_t dimsize, int64_t m_size,
                      int64_t ignore_index, float smooth, void *stream);
 
@@ -78,47 +89,47 @@ int plh_lsr_backward(const float *logits, const int64_t *labels,
  */
 int64_t plh_reduce_workspace_bytes(int64_t units);
 
-int plh_lsr_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                             float *loss_out, int64_t *n_valid_out, int32_t mean,
                             void *workspace, int64_t workspace_bytes,
                             int64_t n_size, int64_t dimsize, int64_t m_size,
                             int64_t ignore_index, float smooth, void *stream);
 
-int plh_lsr_backward_scaled(const float *logits, const int64_t *labels,
+int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *labels,
                             const float *grad_scalar, float scale, const int64_t *divide_by,
-                            float *grad_logits,
+                            void *grad_logits,
                             int64_t n_size, int64_t dimsize, int64_t m_size,
                             int64_t ignore_index, float smooth, void *stream);
 
 /* ---- sigmoid focal loss -------------------------------------------------------
  * Replaces focal_cpp.focalloss_forward / focalloss_backward /
  * focalloss_forward_backward (csrc/focal_kernel.cu:301-335; kernels :29-164).
- * labels are fp32 with the logits' shape (soft labels allowed).  Argument order
+ * labels have the logits' shape and element type (soft labels allowed).  Argument order
  * (gamma, alpha) follows the reference's C++ side (csrc/focal_kernel.cu:301-303).
  */
-int plh_focal_forward(const float *logits, const float *labels, float *losses,
+int plh_focal_forward(const void *logits, int32_t dtype, const void *labels, float *losses,
                       int64_t numel, float gamma, float alpha, void *stream);
 
-int plh_focal_backward(const float *logits, const float *labels,
+int plh_focal_backward(const void *logits, int32_t dtype, const void *labels,
                        const float *grad_output, int64_t grad_output_stride,
-                       float *grad_logits,
+                       void *grad_logits,
                        int64_t numel, float gamma, float alpha, void *stream);
 
 /* Reduction fused into the forward, as for LSR (replaces `loss.mean()` / `loss.sum()` of
  * focal_loss.py:196-199): loss_out = sum, or sum / numel when mean != 0; workspace of
  * plh_reduce_workspace_bytes(numel) bytes. The matching backward takes the upstream
  * gradient grad_scalar[0] * scale (scale = 1/numel for a mean). */
-int plh_focal_forward_reduced(const float *logits, const float *labels, float *losses,
+int plh_focal_forward_reduced(const void *logits, int32_t dtype, const void *labels, float *losses,
                               float *loss_out, int32_t mean, void *workspace, int64_t workspace_bytes,
                               int64_t numel, float gamma, float alpha, void *stream);
 
-int plh_focal_backward_scaled(const float *logits, const float *labels,
-                              const float *grad_scalar, float scale, float *grad_logits,
+int plh_focal_backward_scaled(const void *logits, int32_t dtype, const void *labels,
+                              const float *grad_scalar, float scale, void *grad_logits,
                               int64_t numel, float gamma, float alpha, void *stream);
 
 /* One pass producing both the losses and dloss/dlogits under a unit upstream gradient. */
-int plh_focal_forward_backward(const float *logits, const float *labels,
-                               float *losses, float *grad_logits,
+int plh_focal_forward_backward(const void *logits, int32_t dtype, const void *labels,
+                               float *losses, void *grad_logits,
                                int64_t numel, float gamma, float alpha, void *stream);
 
 /* ---- large-margin softmax -------------------------------------------------------
@@ -127,32 +138,32 @@ int plh_focal_forward_backward(const float *logits, const float *labels,
  * valid_cnt (forward_backward only): one int64 that receives the number of
  * non-ignored pixels; the call overwrites it (no need to clear it first).
  */
-int plh_lmargin_forward(const float *logits, const int64_t *labels, float *losses,
+int plh_lmargin_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                         int64_t n_size, int64_t dimsize, int64_t m_size,
                         int64_t ignore_index, float lam, void *stream);
 
-int plh_lmargin_backward(const float *logits, const int64_t *labels,
+int plh_lmargin_backward(const void *logits, int32_t dtype, const int64_t *labels,
                          const float *grad_output, int64_t grad_output_stride,
-                         float *grad_logits,
+                         void *grad_logits,
                          int64_t n_size, int64_t dimsize, int64_t m_size,
                          int64_t ignore_index, float lam, void *stream);
 
 /* Reduction fused into the forward and the matching backward, as for LSR
  * (replaces large_margin_softmax.py:169-173 of the packaged copy). */
-int plh_lmargin_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+int plh_lmargin_forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                                 float *loss_out, int64_t *n_valid_out, int32_t mean,
                                 void *workspace, int64_t workspace_bytes,
                                 int64_t n_size, int64_t dimsize, int64_t m_size,
                                 int64_t ignore_index, float lam, void *stream);
 
-int plh_lmargin_backward_scaled(const float *logits, const int64_t *labels,
+int plh_lmargin_backward_scaled(const void *logits, int32_t dtype, const int64_t *labels,
                                 const float *grad_scalar, float scale, const int64_t *divide_by,
-                                float *grad_logits,
+                                void *grad_logits,
                                 int64_t n_size, int64_t dimsize, int64_t m_size,
                                 int64_t ignore_index, float lam, void *stream);
 
-int plh_lmargin_forward_backward(const float *logits, const int64_t *labels,
-                                 float *losses, float *grad_logits, int64_t *valid_cnt,
+int plh_lmargin_forward_backward(const void *logits, int32_t dtype, const int64_t *labels,
+                                 float *losses, void *grad_logits, int64_t *valid_cnt,
                                  int64_t n_size, int64_t dimsize, int64_t m_size,
                                  int64_t ignore_index, float lam, void *stream);
 
@@ -169,14 +180,14 @@ int plh_lmargin_forward_backward(const float *logits, const int64_t *labels,
  */
 int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size);
 
-int plh_lovasz_forward(const float *logits, const int64_t *labels,
+int plh_lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels,
                        float *losses, float *jacc,
                        void *workspace, int64_t workspace_bytes,
                        int64_t n_size, int64_t dimsize, int64_t m_size,
                        int64_t ignore_index, void *stream);
 
-int plh_lovasz_backward(const float *grad_output, const float *logits, const int64_t *labels,
-                        const float *jacc, float *grad_logits,
+int plh_lovasz_backward(const float *grad_output, const void *logits, int32_t dtype, const int64_t *labels,
+                        const float *jacc, void *grad_logits,
                         int64_t n_size, int64_t dimsize, int64_t m_size,
                         int64_t ignore_index, void *stream);
 

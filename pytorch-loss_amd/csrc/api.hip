@@ -31,6 +31,7 @@ extern "C" const char *plh_error_string(int code) {
         case PLH_ERR_TOO_MANY_CLASSES: return "num of classes should be less than 512";
         case PLH_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than plh_lovasz_workspace_bytes()";
         case PLH_ERR_MISALIGNED: return "a pointer is not aligned to its element size";
+        case PLH_ERR_BAD_DTYPE: return "dtype must be PLH_DTYPE_F32, PLH_DTYPE_F16 or PLH_DTYPE_BF16";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

@@ -53,10 +53,10 @@ __device__ __forceinline__ void focal_point(float x, float y, const FocalParams 
 }
 
 // One float4 per thread. Reduce: also leave the block's sum of losses in part.sum[slot0 + block].
-template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
-__global__ __launch_bounds__(256) void focal_vec4(const float *__restrict__ x, const float *__restrict__ y,
+template <class T, int Mode, bool WantLoss, bool WantGrad, bool Reduce>
+__global__ __launch_bounds__(256) void focal_vec4(const T *__restrict__ x, const T *__restrict__ y,
                                                   const Upstream up, float *__restrict__ loss,
-                                                  float *__restrict__ grad, float *__restrict__ partial,
+                                                  T *__restrict__ grad, float *__restrict__ partial,
                                                   int64_t n4, const FocalParams p) {
     __shared__ float red[4];
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -84,10 +84,10 @@ __global__ __launch_bounds__(256) void focal_vec4(const float *__restrict__ x, c
     }
 }
 
-template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
-__global__ __launch_bounds__(256) void focal_scalar(const float *__restrict__ x, const float *__restrict__ y,
+template <class T, int Mode, bool WantLoss, bool WantGrad, bool Reduce>
+__global__ __launch_bounds__(256) void focal_scalar(const T *__restrict__ x, const T *__restrict__ y,
                                                     const Upstream up, float *__restrict__ loss,
-                                                    float *__restrict__ grad, float *__restrict__ partial,
+                                                    T *__restrict__ grad, float *__restrict__ partial,
                                                     int64_t first, int64_t numel, const FocalParams p) {
     __shared__ float red[4];
     const int64_t i = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -95,13 +95,13 @@ __global__ __launch_bounds__(256) void focal_scalar(const float *__restrict__ x,
     if (!Reduce && !live) return;
     const int64_t at = live ? i : first;
     float l = 0.f, g = 0.f;
-    focal_point<Mode, WantLoss || Reduce, WantGrad>(x[at], y[at], p, l, g);
+    focal_point<Mode, WantLoss || Reduce, WantGrad>(load_one(x + at), load_one(y + at), p, l, g);
     if (live) {
         if (WantLoss && loss) loss[at] = l;
         if constexpr (WantGrad) {
             float go[1];
             load_upstream<1>(up, at, go);
-            grad[at] = g * go[0];
+            store_one(grad + at, g * go[0]);
         }
     }
     if constexpr (Reduce) {
@@ -111,25 +111,25 @@ __global__ __launch_bounds__(256) void focal_scalar(const float *__restrict__ x,
 }
 
 // Returns the number of partial slots written (0 unless Reduce).
-template <int Mode, bool WantLoss, bool WantGrad, bool Reduce>
-static unsigned launch_mode(const float *x, const float *y, const Upstream &up, float *loss, float *grad,
-                            float *partial, int64_t numel, const FocalParams &p, hipStream_t st) {
+template <class T, int Mode, bool WantLoss, bool WantGrad, bool Reduce>
+static unsigned launch_mode(const T *x, const T *y, const Upstream &up, float *loss, T *grad, float *partial,
+                            int64_t numel, const FocalParams &p, hipStream_t st) {
     int64_t done = 0;
     unsigned slots = 0;
-    const bool aligned = !misaligned(x, 16) && !misaligned(y, 16) && !(loss && misaligned(loss, 16)) &&
-                         !(WantGrad && misaligned(grad, 16)) &&
+    const bool aligned = !misaligned(x, 4 * sizeof(T)) && !misaligned(y, 4 * sizeof(T)) &&
+                         !(loss && misaligned(loss, 16)) && !(WantGrad && misaligned(grad, 4 * sizeof(T))) &&
                          !(WantGrad && up.gout && up.stride == 1 && misaligned(up.gout, 16));
     if (aligned && numel >= 4) {
         const int64_t n4 = numel / 4;
         const unsigned grid = (unsigned)ceil_div(n4, 256);
-        hipLaunchKernelGGL((focal_vec4<Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
+        hipLaunchKernelGGL((focal_vec4<T, Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
                            loss, grad, partial, n4, p);
         done = n4 * 4;
         slots = grid;
     }
     if (done < numel) {
         const unsigned grid = (unsigned)ceil_div(numel - done, 256);
-        hipLaunchKernelGGL((focal_scalar<Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
+        hipLaunchKernelGGL((focal_scalar<T, Mode, WantLoss, WantGrad, Reduce>), dim3(grid), dim3(256), 0, st, x, y, up,
                            loss, grad, Reduce ? partial + slots : nullptr, done, numel, p);
         slots += grid;
     }
@@ -137,19 +137,26 @@ static unsigned launch_mode(const float *x, const float *y, const Upstream &up, 
 }
 
 template <bool WantLoss, bool WantGrad, bool Reduce>
-static int launch(const float *x, const float *y, const Upstream &up, float *loss, float *grad, float *partial,
-                  unsigned *slots_out, int64_t numel, float gamma, float alpha, void *stream) {
+static int launch(const void *x, const void *y, int32_t dtype, const Upstream &up, float *loss, void *grad,
+                  float *partial, unsigned *slots_out, int64_t numel, float gamma, float alpha, void *stream) {
     if (slots_out) *slots_out = 0;
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     if (numel < 0 || numel > kMaxNumel) return PLH_ERR_BAD_SIZE;
     if (numel == 0) return PLH_OK;
     if (!x || !y || (WantLoss && !Reduce && !loss) || (WantGrad && !grad)) return PLH_ERR_NULL_POINTER;
-    if (misaligned(x, 4) || misaligned(y, 4) || misaligned(loss, 4) || misaligned(grad, 4)) return PLH_ERR_MISALIGNED;
+    const size_t es = dtype_size(dtype);
+    if (misaligned(x, es) || misaligned(y, es) || misaligned(loss, 4) || misaligned(grad, es)) return PLH_ERR_MISALIGNED;
     const FocalParams p{gamma, alpha};
     hipStream_t st = (hipStream_t)stream;
-    unsigned slots;
-    if (gamma == 2.f) slots = launch_mode<kGammaTwo, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
-    else if (gamma == 1.f) slots = launch_mode<kGammaOne, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
-    else slots = launch_mode<kGammaAny, WantLoss, WantGrad, Reduce>(x, y, up, loss, grad, partial, numel, p, st);
+    unsigned slots = 0;
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T *xt = static_cast<const T *>(x), *yt = static_cast<const T *>(y);
+        T *gt = static_cast<T *>(grad);
+        if (gamma == 2.f) slots = launch_mode<T, kGammaTwo, WantLoss, WantGrad, Reduce>(xt, yt, up, loss, gt, partial, numel, p, st);
+        else if (gamma == 1.f) slots = launch_mode<T, kGammaOne, WantLoss, WantGrad, Reduce>(xt, yt, up, loss, gt, partial, numel, p, st);
+        else slots = launch_mode<T, kGammaAny, WantLoss, WantGrad, Reduce>(xt, yt, up, loss, gt, partial, numel, p, st);
+    });
     if (slots_out) *slots_out = slots;
     return check_launch();
 }
@@ -158,13 +165,14 @@ static int launch(const float *x, const float *y, const Upstream &up, float *los
 
 using namespace plh;
 
-extern "C" int plh_focal_forward(const float *logits, const float *labels, float *losses,
+extern "C" int plh_focal_forward(const void *logits, int32_t dtype, const void *labels, float *losses,
                                  int64_t numel, float gamma, float alpha, void *stream) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
-    return launch<true, false, false>(logits, labels, up, losses, nullptr, nullptr, nullptr, numel, gamma, alpha, stream);
+    return launch<true, false, false>(logits, labels, dtype, up, losses, nullptr, nullptr, nullptr, numel, gamma, alpha,
+                                      stream);
 }
 
-extern "C" int plh_focal_forward_reduced(const float *logits, const float *labels, float *losses,
+extern "C" int plh_focal_forward_reduced(const void *logits, int32_t dtype, const void *labels, float *losses,
                                          float *loss_out, int32_t mean, void *workspace, int64_t workspace_bytes,
                                          int64_t numel, float gamma, float alpha, void *stream) {
     if (numel < 0 || numel > kMaxNumel) return PLH_ERR_BAD_SIZE;
@@ -173,34 +181,38 @@ extern "C" int plh_focal_forward_reduced(const float *logits, const float *label
     if (rc != PLH_OK) return rc;
     const Upstream up{nullptr, 0, nullptr, 1.f};
     unsigned slots = 0;
-    rc = launch<true, false, true>(logits, labels, up, losses, nullptr, part.sum, &slots, numel, gamma, alpha, stream);
+    rc = launch<true, false, true>(logits, labels, dtype, up, losses, nullptr, part.sum, &slots, numel, gamma, alpha,
+                                   stream);
     if (rc != PLH_OK) return rc;
     part.cnt = nullptr;
     finish_partials(part, slots, loss_out, nullptr, mean ? kFinishMeanOverFixed : kFinishSum, numel, (hipStream_t)stream);
     return check_launch();
 }
 
-extern "C" int plh_focal_backward(const float *logits, const float *labels,
-                                  const float *grad_output, int64_t grad_output_stride, float *grad_logits,
+extern "C" int plh_focal_backward(const void *logits, int32_t dtype, const void *labels,
+                                  const float *grad_output, int64_t grad_output_stride, void *grad_logits,
                                   int64_t numel, float gamma, float alpha, void *stream) {
     const int rc = check_gout(grad_output, grad_output_stride);
     if (rc != PLH_OK) return rc;
     const Upstream up{grad_output, grad_output_stride, nullptr, 1.f};
-    return launch<false, true, false>(logits, labels, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
+    return launch<false, true, false>(logits, labels, dtype, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma,
+                                      alpha, stream);
 }
 
-extern "C" int plh_focal_backward_scaled(const float *logits, const float *labels,
-                                         const float *grad_scalar, float scale, float *grad_logits,
+extern "C" int plh_focal_backward_scaled(const void *logits, int32_t dtype, const void *labels,
+                                         const float *grad_scalar, float scale, void *grad_logits,
                                          int64_t numel, float gamma, float alpha, void *stream) {
     if (numel > 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_scalar, 4)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, nullptr, scale};
-    return launch<false, true, false>(logits, labels, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
+    return launch<false, true, false>(logits, labels, dtype, up, nullptr, grad_logits, nullptr, nullptr, numel, gamma,
+                                      alpha, stream);
 }
 
-extern "C" int plh_focal_forward_backward(const float *logits, const float *labels, float *losses,
-                                          float *grad_logits, int64_t numel, float gamma, float alpha,
+extern "C" int plh_focal_forward_backward(const void *logits, int32_t dtype, const void *labels, float *losses,
+                                          void *grad_logits, int64_t numel, float gamma, float alpha,
                                           void *stream) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
-    return launch<true, true, false>(logits, labels, up, losses, grad_logits, nullptr, nullptr, numel, gamma, alpha, stream);
+    return launch<true, true, false>(logits, labels, dtype, up, losses, grad_logits, nullptr, nullptr, numel, gamma,
+                                     alpha, stream);
 }

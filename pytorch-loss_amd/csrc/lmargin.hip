@@ -1,264 +1,26 @@
-// Large-margin softmax cross entropy (Kobayashi, BMVC 2019), forward / backward /
-// fused forward+backward, for gfx950.
-//
-// Per valid pixel with target y (csrc/large_margin_kernel.cu:450-475, comment :450-460):
-//   p = softmax(x) over all C channels, q = softmax(x) over the channels j != y,
-//   coeff = 1/(C-1), h = lam/2
-//   loss = -log p_y + h * sum_{j!=y} (q_j - coeff) * log q_j
-//   g_y  = p_y - 1
-//   g_j  = p_j + h * ((x_j + 1 - sum_k q_k x_k) * q_j - coeff)          (j != y)
-//   ignored pixel: loss 0, every grad 0                      (large_margin_kernel.cu:414-421)
-// The two softmaxes keep separate maxima (m_no over j != y, m_all = max(m_no, x_y)),
-// so a dominant target logit cannot underflow the non-target sum; the full sum is
-// rebuilt from the non-target one:  s_all = s_no * exp(m_no - m_all) + exp(x_y - m_all).
-// Each direction is one kernel that reads the logits once.
-#include "plh_common.hpp"
+// Large-margin softmax cross entropy for gfx950: the C entry points. The kernels live in
+// lmargin_kernels.hpp and are compiled once per element type (lmargin_f32.hip, lmargin_f16.hip,
+// lmargin_bf16.hip).
+#include "lmargin_kernels.hpp"
 
 namespace plh {
 
-struct LmParams {
-    int64_t P;
-    int64_t m_size;
-    int C;
-    int64_t ignore;
-    float half_lam, coeff;
-};
-
-// ---------------------------------------------------------------- regs ----
-
-template <int CP, int V, bool Uniform, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-__global__ __launch_bounds__(kRegsBlock) void lm_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
-                                                     const Upstream up,
-                                                     float *__restrict__ loss, float *__restrict__ grad,
-                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
-                                                     const LmParams p) {
-    __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
-    const bool live = at.live;
-    if (!Reduce && !live) return;
-    const int64_t pix = at.pix;
-
-    float v[CP][V];
-#pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
-    int64_t lb[V];
-    load_labels<V>(lab + pix, lb);
-    float go[V];
-    if constexpr (WantGrad) load_upstream<V>(up, pix, go);
-
-    float out[V];
-    unsigned n_valid = 0;
-    float mine = 0.f;
-    int cnt = 0;
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        float m_no = -INFINITY, x_y = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const bool hot = (tgt == j);
-                m_no = hot ? m_no : fmaxf(m_no, v[j][k]);
-                x_y = hot ? v[j][k] : x_y;
-            }
-        const float m_all = fmaxf(m_no, x_y);
-        // one exponential per channel: with t_j = x_j - m_no and e_j = exp(t_j) over j != y,
-        //   sum_j (q_j - coeff) log q_j = (sum e_j t_j)/s_no - lse_no - coeff * (sum t_j - (C-1) lse_no)
-        float e[WantGrad ? CP : 1];
-        float s_no = 0.f, sum_et = 0.f, sum_t = 0.f;
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const bool hot = (tgt == j);
-                const float t = v[j][k] - m_no;
-                const float ej = hot ? 0.f : fast_exp(t);
-                if constexpr (WantGrad) e[j] = ej;
-                s_no += ej;
-                sum_et += ej * (hot ? 0.f : t);
-                sum_t += hot ? 0.f : t;
-            }
-        const float t_all = fast_exp(m_no - m_all);
-        const float e_y = fast_exp(x_y - m_all);
-        const float s_all = s_no * t_all + e_y;
-        const float inv_no = 1.f / s_no;
-        if constexpr (WantLoss) {
-            const float lse_no = fast_log(s_no);
-            const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));   // channels that are not the target
-            const float margin = sum_et * inv_no - lse_no - p.coeff * (sum_t - others * lse_no);
-            const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
-            out[k] = (ign || !live) ? 0.f : acc;
-            mine += out[k];
-            cnt += (ign || !live) ? 0 : 1;
-        }
-        if constexpr (WantGrad) {
-            const float inv_all = 1.f / s_all;
-            // sum_k q_k x_k = (sum e t)/s_no + m_no
-            const float sum_qx = sum_et * inv_no + m_no;
-            const float gk = ign ? 0.f : go[k];
-            const float p_scale = t_all * inv_all;
-            const float g_hot = (e_y * inv_all - 1.f) * gk;
-#pragma unroll
-            for (int j = 0; j < CP; ++j)
-                if (j < p.C) {
-                    const float q = e[j] * inv_no;
-                    const float g_cold = e[j] * p_scale + p.half_lam * ((v[j][k] + 1.f - sum_qx) * q - p.coeff);
-                    const float g = (tgt == j) ? g_hot : g_cold * gk;
-                    v[j][k] = ign ? 0.f : g;      // exact zero even for non-finite logits
-                }
-        }
-        if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
-    }
-    if (live) {
-        if (WantLoss && loss) store_vec<V>(loss + pix, out);
-        if constexpr (WantGrad) {
-#pragma unroll
-            for (int j = 0; j < CP; ++j)
-                if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
-        }
-    }
-    if constexpr (WantCount) {
-        // lanes leave only at the tail of the grid, so lane 0 of a wave with work is alive
-        if ((threadIdx.x & 63) == 0) atomicAdd(valid_cnt, (unsigned long long)n_valid);
-    }
-    if constexpr (Reduce) {
-        const float bs = block_sum_256(mine, red);
-        const float bc = block_sum_256((float)cnt, red);
-        if (threadIdx.x == 0) {
-            part.sum[blockIdx.x] = bs;
-            part.cnt[blockIdx.x] = (int)bc;
-        }
-    }
-}
-
-// --------------------------------------------------------------- group ----
-
-constexpr int kLmStageCap = 2048;
-
-template <int G, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-__global__ __launch_bounds__(256) void lm_group(const float *__restrict__ x, const int64_t *__restrict__ lab,
-                                                const Upstream up,
-                                                float *__restrict__ loss, float *__restrict__ grad,
-                                                unsigned long long *__restrict__ valid_cnt, Partials part,
-                                                const LmParams p) {
-    constexpr int kPix = 256 / G;
-    __shared__ float stage_mem[(G == 64) ? 4 * kLmStageCap : 1];
-    __shared__ float red[4];
-    float mine = 0.f, cnt = 0.f;
-    const int sub = threadIdx.x % G;
-    const int grp = threadIdx.x / G;
-    float *stage = stage_mem + ((G == 64) ? grp * kLmStageCap : 0);
-    const bool staged = (G == 64) && (p.C <= kLmStageCap);
-
-    unsigned long long n_valid = 0;
-    const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
-    for (int64_t r = 0; r < rounds; ++r) {
-        const int64_t pix = (r * gridDim.x + blockIdx.x) * kPix + grp;
-        const bool live = pix < p.P;
-        const int64_t pc = live ? pix : 0;
-        const int64_t n = pc / p.m_size;
-        const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
-        const float *xs = x + base;
-        const int64_t lb = lab[pc];
-        const bool ign = (lb == p.ignore);
-        float go[1] = {1.f};
-        if constexpr (WantGrad) load_upstream<1>(up, pc, go);
-
-        float m_no = -INFINITY, x_y = -INFINITY;
-        for (int j = sub; j < p.C; j += G) {
-            const float t = xs[(int64_t)j * p.m_size];
-            if (staged) stage[j] = t;
-            if (lb == j) x_y = t; else m_no = fmaxf(m_no, t);
-        }
-        m_no = group_reduce<G>(m_no, OpMax());
-        x_y = group_reduce<G>(x_y, OpMax());
-        const float m_all = fmaxf(m_no, x_y);
-        float s_no = 0.f, sum_ex = 0.f;
-        for (int j = sub; j < p.C; j += G) {
-            const float t = staged ? stage[j] : xs[(int64_t)j * p.m_size];
-            const float e = (lb == j) ? 0.f : fast_exp(t - m_no);
-            s_no += e;
-            sum_ex += e * t;
-        }
-        s_no = group_reduce<G>(s_no, OpSum());
-        sum_ex = group_reduce<G>(sum_ex, OpSum());
-        const float t_all = fast_exp(m_no - m_all);
-        const float e_y = fast_exp(x_y - m_all);
-        const float s_all = s_no * t_all + e_y;
-        const float inv_no = 1.f / s_no, inv_all = 1.f / s_all;
-        const float sum_qx = sum_ex * inv_no;
-        const float lse_no = logf(s_no);
-        float acc = 0.f;
-        for (int j = sub; j < p.C; j += G) {
-            const float xv = staged ? stage[j] : xs[(int64_t)j * p.m_size];
-            const bool hot = (lb == j);
-            const float e = fast_exp(xv - m_no);
-            const float q = e * inv_no;
-            if constexpr (WantLoss) acc += hot ? 0.f : p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
-            if constexpr (WantGrad) {
-                const float g_hot = e_y * inv_all - 1.f;
-                const float g_cold = e * t_all * inv_all + p.half_lam * ((xv + 1.f - sum_qx) * q - p.coeff);
-                if (live) grad[base + (int64_t)j * p.m_size] = ign ? 0.f : (hot ? g_hot : g_cold) * go[0];
-            }
-        }
-        if constexpr (WantLoss) {
-            acc = group_reduce<G>(acc, OpSum());
-            acc += -(x_y - m_all) + logf(s_all);
-            if (live && sub == 0) {
-                if (loss) loss[pix] = ign ? 0.f : acc;
-                mine += ign ? 0.f : acc;
-                cnt += ign ? 0.f : 1.f;
-            }
-        }
-        // every lane of the wave is inside the loop, so the ballot sees the whole wave
-        if constexpr (WantCount)
-            n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && sub == 0 && !ign));
-    }
-    if constexpr (WantCount) {
-        if ((threadIdx.x & 63) == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
-    }
-    if constexpr (Reduce) {
-        const float bs = block_sum_256(mine, red);
-        const float bc = block_sum_256(cnt, red);
-        if (threadIdx.x == 0) {
-            part.sum[blockIdx.x] = bs;
-            part.cnt[blockIdx.x] = (int)bc;
-        }
-    }
-}
-
-__global__ void lm_zero_count(unsigned long long *cnt) { *cnt = 0; }
-
-// ------------------------------------------------------------ dispatch ----
-
-template <int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-static unsigned launch_regs(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
-                            unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
-    const unsigned grid = regs_grid<V>(p.P);
-    const bool uni = tiles_are_uniform(p.m_size, V);
-    switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                                                                                               \
-    case K:                                                                                                       \
-        if (uni) hipLaunchKernelGGL((lm_regs<4 * K, V, true, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
-                                    dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);               \
-        else hipLaunchKernelGGL((lm_regs<4 * K, V, false, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),    \
-                                dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                   \
-        break;
-        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
-#undef PLH_CASE
-    }
-    return grid;
-}
+PLH_LM_EXTERN(float)
+PLH_LM_EXTERN(f16)
+PLH_LM_EXTERN(bf16)
 
 // Launches one direction (or the fused pair). blocks_out: blocks that wrote partials (Reduce only).
-template <bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-static int launch(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
+static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,
                   int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
                   int64_t m_size, int64_t ignore, float lam, void *stream) {
+    const bool WantLoss = variant != kLmBackward, WantGrad = variant == kLmBackward || variant == kLmForwardBackwardCount;
+    const bool WantCount = variant == kLmForwardBackwardCount, Reduce = variant == kLmForwardReduced;
     if (blocks_out) *blocks_out = 0;
-    const void *out = (WantLoss && !Reduce) ? (const void *)loss : (WantGrad ? (const void *)grad : (const void *)x);
-    int rc = check_slice_args(x, lab, out, n_size, dimsize, m_size);
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    const size_t es = dtype_size(dtype);
+    const bool out_is_loss = WantLoss && !Reduce;
+    const void *out = out_is_loss ? (const void *)loss : (WantGrad ? (const void *)grad : x);
+    int rc = check_slice_args(x, lab, out, n_size, dimsize, m_size, es, out_is_loss ? 4 : es);
     if (rc != PLH_OK) return rc;
     if (up.gout && up.stride == 1 && misaligned(up.gout, 4)) return PLH_ERR_MISALIGNED;
     if (WantCount && (!valid_cnt || misaligned(valid_cnt, 8))) return valid_cnt ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
@@ -266,7 +28,7 @@ static int launch(const float *x, const int64_t *lab, const Upstream &up, float 
     unsigned long long *cnt = reinterpret_cast<unsigned long long *>(valid_cnt);
     if (WantCount) hipLaunchKernelGGL(lm_zero_count, dim3(1), dim3(1), 0, st, cnt);
     if (n_size * dimsize * m_size == 0) return check_launch();
-    if (WantLoss && WantGrad && (!grad || misaligned(grad, 4))) return grad ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
+    if (WantLoss && WantGrad && (!grad || misaligned(grad, es))) return grad ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
     if (loss && misaligned(loss, 4)) return PLH_ERR_MISALIGNED;
 
     LmParams p;
@@ -276,26 +38,12 @@ static int launch(const float *x, const int64_t *lab, const Upstream &up, float 
     p.ignore = ignore;
     p.half_lam = lam / 2.f;                          // csrc/large_margin_kernel.cu:188
     p.coeff = 1.f / (float)(dimsize - 1);            // csrc/large_margin_kernel.cu:404
-    const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     unsigned blocks = 0;
-    switch (pick_shape(dimsize, m_size, x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr, go_vec)) {
-        case Shape::Regs2:
-            blocks = launch_regs<2, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
-            break;
-        case Shape::Regs1:
-            blocks = launch_regs<1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
-            break;
-        case Shape::Wave:
-            blocks = group_grid(p.P, 4);
-            hipLaunchKernelGGL((lm_group<64, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
-                               x, lab, up, loss, grad, cnt, part, p);
-            break;
-        case Shape::Lane:
-            blocks = group_grid(p.P, 256);
-            hipLaunchKernelGGL((lm_group<1, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
-                               x, lab, up, loss, grad, cnt, part, p);
-            break;
-    }
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        blocks = lmargin_run_typed<T>(variant, static_cast<const T *>(x), lab, up, loss, static_cast<T *>(grad), cnt,
+                                      part, p, st);
+    });
     if (blocks_out) *blocks_out = blocks;
     return check_launch();
 }
@@ -306,15 +54,15 @@ using namespace plh;
 
 static const Partials kNoPartials{nullptr, nullptr};
 
-extern "C" int plh_lmargin_forward(const float *logits, const int64_t *labels, float *losses,
+extern "C" int plh_lmargin_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                                    int64_t n_size, int64_t dimsize, int64_t m_size,
                                    int64_t ignore_index, float lam, void *stream) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
-    return launch<true, false, false, false>(logits, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr,
+    return launch(kLmForward, logits, dtype, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr,
                                              n_size, dimsize, m_size, ignore_index, lam, stream);
 }
 
-extern "C" int plh_lmargin_forward_reduced(const float *logits, const int64_t *labels, float *losses,
+extern "C" int plh_lmargin_forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                                            float *loss_out, int64_t *n_valid_out, int32_t mean,
                                            void *workspace, int64_t workspace_bytes,
                                            int64_t n_size, int64_t dimsize, int64_t m_size,
@@ -325,42 +73,42 @@ extern "C" int plh_lmargin_forward_reduced(const float *logits, const int64_t *l
     if (rc != PLH_OK) return rc;
     const Upstream up{nullptr, 0, nullptr, 1.f};
     unsigned blocks = 0;
-    rc = launch<true, false, false, true>(logits, labels, up, losses, nullptr, nullptr, part, &blocks, n_size, dimsize,
-                                          m_size, ignore_index, lam, stream);
+    rc = launch(kLmForwardReduced, logits, dtype, labels, up, losses, nullptr, nullptr, part, &blocks, n_size,
+                                          dimsize, m_size, ignore_index, lam, stream);
     if (rc != PLH_OK) return rc;
     finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0,
                     (hipStream_t)stream);
     return check_launch();
 }
 
-extern "C" int plh_lmargin_backward(const float *logits, const int64_t *labels,
-                                    const float *grad_output, int64_t grad_output_stride, float *grad_logits,
+extern "C" int plh_lmargin_backward(const void *logits, int32_t dtype, const int64_t *labels,
+                                    const float *grad_output, int64_t grad_output_stride, void *grad_logits,
                                     int64_t n_size, int64_t dimsize, int64_t m_size,
                                     int64_t ignore_index, float lam, void *stream) {
     const int rc = check_gout(grad_output, grad_output_stride);
     if (rc != PLH_OK) return rc;
     const Upstream up{grad_output, grad_output_stride, nullptr, 1.f};
-    return launch<false, true, false, false>(logits, labels, up, nullptr, grad_logits, nullptr, kNoPartials, nullptr,
-                                             n_size, dimsize, m_size, ignore_index, lam, stream);
+    return launch(kLmBackward, logits, dtype, labels, up, nullptr, grad_logits, nullptr, kNoPartials,
+                                             nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
 }
 
-extern "C" int plh_lmargin_backward_scaled(const float *logits, const int64_t *labels,
+extern "C" int plh_lmargin_backward_scaled(const void *logits, int32_t dtype, const int64_t *labels,
                                            const float *grad_scalar, float scale, const int64_t *divide_by,
-                                           float *grad_logits,
+                                           void *grad_logits,
                                            int64_t n_size, int64_t dimsize, int64_t m_size,
                                            int64_t ignore_index, float lam, void *stream) {
     if (n_size * dimsize * m_size != 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, divide_by, scale};
-    return launch<false, true, false, false>(logits, labels, up, nullptr, grad_logits, nullptr, kNoPartials, nullptr,
-                                             n_size, dimsize, m_size, ignore_index, lam, stream);
+    return launch(kLmBackward, logits, dtype, labels, up, nullptr, grad_logits, nullptr, kNoPartials,
+                                             nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
 }
 
-extern "C" int plh_lmargin_forward_backward(const float *logits, const int64_t *labels, float *losses,
-                                            float *grad_logits, int64_t *valid_cnt,
+extern "C" int plh_lmargin_forward_backward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                                            void *grad_logits, int64_t *valid_cnt,
                                             int64_t n_size, int64_t dimsize, int64_t m_size,
                                             int64_t ignore_index, float lam, void *stream) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
-    return launch<true, true, true, false>(logits, labels, up, losses, grad_logits, valid_cnt, kNoPartials, nullptr,
-                                           n_size, dimsize, m_size, ignore_index, lam, stream);
+    return launch(kLmForwardBackwardCount, logits, dtype, labels, up, losses, grad_logits, valid_cnt, kNoPartials,
+                                           nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
 }

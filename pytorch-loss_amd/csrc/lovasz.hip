@@ -52,14 +52,14 @@ __device__ __forceinline__ float key_error(uint32_t key) {
 
 // ------------------------------------------------------ 1. build keys ----
 
-template <int CP, int V>
-__global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const float *__restrict__ x, const int64_t *__restrict__ lab,
+template <class T, int CP, int V>
+__global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
                                                            int64_t ignore) {
     const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
     const int64_t n = pix / m_size;
-    const float *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
+    const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
     float v[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
@@ -90,19 +90,20 @@ __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const float *__restr
 }
 
 // Any channel count: a lane per pixel, three sweeps over the slice (the later ones hit cache).
-__global__ __launch_bounds__(256) void lov_keys_lane(const float *__restrict__ x, const int64_t *__restrict__ lab,
+template <class T>
+__global__ __launch_bounds__(256) void lov_keys_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                      uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
                                                      int64_t ignore) {
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t n = pix / m_size;
-        const float *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
+        const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
         const int64_t lb = lab[pix];
         float mx = -INFINITY;
-        for (int j = 0; j < C; ++j) mx = fmaxf(mx, xs[(int64_t)j * m_size]);
+        for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
-        for (int j = 0; j < C; ++j) s += expf(xs[(int64_t)j * m_size] - mx);
+        for (int j = 0; j < C; ++j) s += expf(load_one(xs + (int64_t)j * m_size) - mx);
         for (int j = 0; j < C; ++j)
-            keys[(int64_t)j * P + pix] = make_key(expf(xs[(int64_t)j * m_size] - mx) / s, lb == j, lb == ignore);
+            keys[(int64_t)j * P + pix] = make_key(expf(load_one(xs + (int64_t)j * m_size) - mx) / s, lb == j, lb == ignore);
     }
 }
 
@@ -562,10 +563,10 @@ __global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__
 
 // ------------------------------------------------------------ backward ----
 
-template <int CP, int V>
-__global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restrict__ gout, const float *__restrict__ x,
+template <class T, int CP, int V>
+__global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restrict__ gout, const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab, const float *__restrict__ jacc,
-                                                          float *__restrict__ grad, int64_t P, int64_t m_size, int C,
+                                                          T *__restrict__ grad, int64_t P, int64_t m_size, int C,
                                                           int64_t ignore) {
     const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
@@ -612,30 +613,31 @@ __global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restri
         if (j < C) store_vec<V>(grad + base + (int64_t)j * m_size, v[j]);
 }
 
-__global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ gout, const float *__restrict__ x,
+template <class T>
+__global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ gout, const T *__restrict__ x,
                                                     const int64_t *__restrict__ lab, const float *__restrict__ jacc,
-                                                    float *__restrict__ grad, int64_t P, int64_t m_size, int C,
+                                                    T *__restrict__ grad, int64_t P, int64_t m_size, int C,
                                                     int64_t ignore) {
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t n = pix / m_size;
         const int64_t base = pix + n * (int64_t)(C - 1) * m_size;
-        const float *xs = x + base;
+        const T *xs = x + base;
         const int64_t lb = lab[pix];
         float mx = -INFINITY;
-        for (int j = 0; j < C; ++j) mx = fmaxf(mx, xs[(int64_t)j * m_size]);
+        for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
-        for (int j = 0; j < C; ++j) s += expf(xs[(int64_t)j * m_size] - mx);
+        for (int j = 0; j < C; ++j) s += expf(load_one(xs + (int64_t)j * m_size) - mx);
         float dot = 0.f;
         for (int j = 0; j < C; ++j) {
-            const float p = expf(xs[(int64_t)j * m_size] - mx) / s;
+            const float p = expf(load_one(xs + (int64_t)j * m_size) - mx) / s;
             const float dj = jacc[(int64_t)j * P + pix] * gout[j];
             dot += p * ((lb == j) ? -dj : dj);
         }
         const bool ign = (lb == ignore);
         for (int j = 0; j < C; ++j) {
-            const float p = expf(xs[(int64_t)j * m_size] - mx) / s;
+            const float p = expf(load_one(xs + (int64_t)j * m_size) - mx) / s;
             const float dj = jacc[(int64_t)j * P + pix] * gout[j];
-            grad[base + (int64_t)j * m_size] = ign ? 0.f : p * (((lb == j) ? -dj : dj) - dot);
+            store_one(grad + (base + (int64_t)j * m_size), ign ? 0.f : p * (((lb == j) ? -dj : dj) - dot));
         }
     }
 }
@@ -686,16 +688,17 @@ extern "C" int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, i
     return rc == PLH_OK ? pl.bytes : (int64_t)rc;
 }
 
-extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, float *losses, float *jacc,
+extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *jacc,
                                   void *workspace, int64_t workspace_bytes,
                                   int64_t n_size, int64_t dimsize, int64_t m_size,
                                   int64_t ignore_index, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     LovaszPlan pl;
     int rc = make_plan(n_size, dimsize, m_size, pl);
     if (rc != PLH_OK) return rc;
     if (pl.E == 0) return PLH_OK;
     if (!logits || !labels || !losses || !jacc) return PLH_ERR_NULL_POINTER;
-    if (misaligned(logits, 4) || misaligned(losses, 4) || misaligned(jacc, 4) || misaligned(labels, 8))
+    if (misaligned(logits, dtype_size(dtype)) || misaligned(losses, 4) || misaligned(jacc, 4) || misaligned(labels, 8))
         return PLH_ERR_MISALIGNED;
     if (!workspace || misaligned(workspace, 256) || workspace_bytes < pl.bytes) return PLH_ERR_WORKSPACE;
 
@@ -712,26 +715,31 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
     float *tile_loss = reinterpret_cast<float *>(ws + pl.off_tile_loss);
     const int C = (int)dimsize;
 
-    // 1. keys
-    const Shape shape = pick_shape(dimsize, m_size, logits, keys_b, labels, nullptr, nullptr);
-    if (shape == Shape::Regs2 || shape == Shape::Regs1) {
-        const int V = (shape == Shape::Regs2) ? 2 : 1;      // m_size even => P even => rows of [C][P] stay 8-byte aligned
-        const unsigned grid = (V == 2) ? regs_grid<2>(pl.P) : regs_grid<1>(pl.P);
-        switch ((C + 3) / 4) {
-#define PLH_CASE(K)                                                                                                  \
-    case K:                                                                                                          \
-        if (V == 2) hipLaunchKernelGGL((lov_keys_regs<4 * K, 2>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels, \
-                                       keys_b, pl.P, m_size, C, ignore_index);                                       \
-        else hipLaunchKernelGGL((lov_keys_regs<4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, logits, labels,      \
-                                keys_b, pl.P, m_size, C, ignore_index);                                              \
+    // 1. keys (into keys_b = jacc: rows of [C][P] u32; a row start stays 8-/16-byte aligned when P % V == 0)
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T *x = static_cast<const T *>(logits);
+        constexpr int VT = ElemTraits<T>::kVec;
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, keys_b, nullptr);
+        if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
+            const bool vec = (shape == Shape::RegsVec);
+            const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
+            switch ((C + 3) / 4) {
+#define PLH_CASE(K)                                                                                                 \
+    case K:                                                                                                         \
+        if (vec) hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,  \
+                                    keys_b, pl.P, m_size, C, ignore_index);                                         \
+        else hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,       \
+                                keys_b, pl.P, m_size, C, ignore_index);                                             \
         break;
-            PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+                PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
+            }
+        } else {
+            hipLaunchKernelGGL(lov_keys_lane<T>, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, x, labels, keys_b, pl.P,
+                               m_size, C, ignore_index);
         }
-    } else {
-        hipLaunchKernelGGL(lov_keys_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, logits, labels, keys_b,
-                           pl.P, m_size, C, ignore_index);
-    }
+    });
 
     // 2. three stable radix passes: (keys_b, -) -> (keys_a, vals_a) -> (keys_b, vals_b) -> (keys_a, vals_a).
     //    keys_b is the jacc output buffer, free until the last pass scatters into it
@@ -785,38 +793,45 @@ extern "C" int plh_lovasz_forward(const float *logits, const int64_t *labels, fl
     return check_launch();
 }
 
-extern "C" int plh_lovasz_backward(const float *grad_output, const float *logits, const int64_t *labels,
-                                   const float *jacc, float *grad_logits,
+extern "C" int plh_lovasz_backward(const float *grad_output, const void *logits, int32_t dtype, const int64_t *labels,
+                                   const float *jacc, void *grad_logits,
                                    int64_t n_size, int64_t dimsize, int64_t m_size,
                                    int64_t ignore_index, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     LovaszPlan pl;
     const int rc = make_plan(n_size, dimsize, m_size, pl);
     if (rc != PLH_OK) return rc;
     if (pl.E == 0) return PLH_OK;
     if (!grad_output || !logits || !labels || !jacc || !grad_logits) return PLH_ERR_NULL_POINTER;
-    if (misaligned(grad_output, 4) || misaligned(logits, 4) || misaligned(jacc, 4) || misaligned(grad_logits, 4) ||
-        misaligned(labels, 8))
+    if (misaligned(grad_output, 4) || misaligned(logits, dtype_size(dtype)) || misaligned(jacc, 4) ||
+        misaligned(grad_logits, dtype_size(dtype)) || misaligned(labels, 8))
         return PLH_ERR_MISALIGNED;
     hipStream_t st = (hipStream_t)stream;
     const int C = (int)dimsize;
-    const Shape shape = pick_shape(dimsize, m_size, logits, grad_logits, labels, jacc, nullptr);
-    if (shape == Shape::Regs2 || shape == Shape::Regs1) {
-        const int V = (shape == Shape::Regs2) ? 2 : 1;
-        const unsigned grid = (V == 2) ? regs_grid<2>(pl.P) : regs_grid<1>(pl.P);
-        switch ((C + 3) / 4) {
-#define PLH_CASE(K)                                                                                                   \
-    case K:                                                                                                           \
-        if (V == 2) hipLaunchKernelGGL((lov_bwd_regs<4 * K, 2>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output,    \
-                                       logits, labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);             \
-        else hipLaunchKernelGGL((lov_bwd_regs<4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output, logits,   \
-                                labels, jacc, grad_logits, pl.P, m_size, C, ignore_index);                            \
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T *x = static_cast<const T *>(logits);
+        T *g = static_cast<T *>(grad_logits);
+        constexpr int VT = ElemTraits<T>::kVec;
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, g, labels, jacc, nullptr);
+        if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
+            const bool vec = (shape == Shape::RegsVec);
+            const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
+            switch ((C + 3) / 4) {
+#define PLH_CASE(K)                                                                                                  \
+    case K:                                                                                                          \
+        if (vec) hipLaunchKernelGGL((lov_bwd_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output,  \
+                                    x, labels, jacc, g, pl.P, m_size, C, ignore_index);                              \
+        else hipLaunchKernelGGL((lov_bwd_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output, x,    \
+                                labels, jacc, g, pl.P, m_size, C, ignore_index);                                     \
         break;
-            PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+                PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
+            }
+        } else {
+            hipLaunchKernelGGL(lov_bwd_lane<T>, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, grad_output, x, labels,
+                               jacc, g, pl.P, m_size, C, ignore_index);
         }
-    } else {
-        hipLaunchKernelGGL(lov_bwd_lane, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, grad_output, logits, labels,
-                           jacc, grad_logits, pl.P, m_size, C, ignore_index);
-    }
+    });
     return check_launch();
 }

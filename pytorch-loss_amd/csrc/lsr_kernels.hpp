@@ -1,0 +1,368 @@
+// Label-smoothed softmax cross entropy, forward and backward, for gfx950: kernels and launchers.
+//
+// Math (per pixel, target y, smoothing s, C channels):
+//   w_y = 1 - s, w_j = s / C otherwise            (csrc/lsr_kernel.cu:83-84)
+//   loss = -sum_j w_j * log_softmax(x)_j          (csrc/lsr_kernel.cu:174-182)
+//   grad_j = (sumw * softmax(x)_j - w_j) * upstream, sumw = (C-1) s/C + (1-s)
+//                                                 (csrc/lsr_kernel.cu:123-143)
+//   ignored pixel: loss 0, every grad 0.
+// Unlike the reference (ATen log_softmax/softmax into a full-size temporary, a
+// second kernel, then a Python-side multiply) each direction is ONE kernel that
+// reads the logits once: forward 4E + 12P bytes, backward 8E + 12P bytes.
+// The "reduced" forward additionally leaves per-block partial sums and valid-pixel
+// counts behind, which a one-block finishing kernel turns into sum or mean, so the
+// module-level reduction costs no further pass over the pixels.
+#pragma once
+#include "plh_common.hpp"
+
+namespace plh {
+
+struct LsrParams {
+    int64_t P;        // pixels = n_size * m_size
+    int64_t m_size;
+    int C;
+    int64_t ignore;
+    float w_pos, w_neg, sumw;
+};
+
+// ---------------------------------------------------------------- regs ----
+
+// loss = -sum_j w_j logp_j with logp_j = t_j - lse, t_j = x_j - max:
+//      = -( w_neg * (sum_j t_j - C*lse) + (w_pos - w_neg) * (t_y - lse) )
+// so one pass over the slice gathers max-shifted sum, exp-sum and the target's t.
+template <class T, int CP, int V, bool Uniform, bool Reduce>
+__global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__ x,
+                                                          const int64_t *__restrict__ lab,
+                                                          float *__restrict__ loss, Partials part,
+                                                          const LsrParams p) {
+    __shared__ float red[4];
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    if (!Reduce && !at.live) return;
+
+    float v[CP][V];
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+
+    float out[V];
+    float mine = 0.f;
+    int cnt = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        float mx = v[0][k];
+#pragma unroll
+        for (int j = 1; j < CP; ++j)
+            if (j < p.C) mx = fmaxf(mx, v[j][k]);
+        float s = 0.f, sum_t = 0.f, t_y = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < p.C) {
+                const float t = v[j][k] - mx;
+                s += fast_exp(t);
+                sum_t += t;
+                t_y = (tgt == j) ? t : t_y;
+            }
+        const float lse = fast_log(s);
+        const float all = sum_t - (float)p.C * lse;
+        // no target channel (label outside [0, C)): every weight is w_neg
+        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * (t_y - lse) : 0.f;
+        const float acc = -(p.w_neg * all + hot);
+        const bool valid = at.live && !ign;
+        out[k] = valid ? acc : 0.f;
+        mine += out[k];
+        cnt += valid ? 1 : 0;
+    }
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256((float)cnt, red);   // at most 512 per block: exact in fp32
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int CP, int V, bool Uniform>
+__global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__ x,
+                                                          const int64_t *__restrict__ lab,
+                                                          const Upstream up, T *__restrict__ grad,
+                                                          const LsrParams p) {
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    if (!at.live) return;
+
+    float v[CP][V];
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    float go[V];
+    load_upstream<V>(up, at.pix, go);
+
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float mx = v[0][k];
+#pragma unroll
+        for (int j = 1; j < CP; ++j)
+            if (j < p.C) mx = fmaxf(mx, v[j][k]);
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < p.C) {
+                v[j][k] = fast_exp(v[j][k] - mx);
+                s += v[j][k];
+            }
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        const float gk = go[k];
+        const float scale = p.sumw * gk / s;          // one division per pixel
+        const float g_pos = p.w_pos * gk, g_neg = p.w_neg * gk;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (j < p.C) {
+                const float g = v[j][k] * scale - ((tgt == j) ? g_pos : g_neg);
+                v[j][k] = ign ? 0.f : g;              // exact zero even for non-finite logits
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
+}
+
+// --------------------------------------------------------------- group ----
+// G lanes per pixel. G = 64 stages the wave's slice in LDS (each lane re-reads
+// only what it wrote, so no barrier is needed); G = 1 re-reads global memory,
+// which the preceding pass has just pulled into cache.
+
+constexpr int kStageCap = 2048;   // floats per wave -> 32 KiB of LDS per 256-thread block
+
+template <class T, int G, bool Reduce>
+__global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
+                                                     const int64_t *__restrict__ lab,
+                                                     float *__restrict__ loss, Partials part,
+                                                     const LsrParams p) {
+    constexpr int kPix = 256 / G;
+    __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
+    __shared__ float red[4];
+    const int sub = threadIdx.x % G;
+    const int grp = threadIdx.x / G;
+    float *stage = stage_mem + ((G == 64) ? grp * kStageCap : 0);
+    const bool staged = (G == 64) && (p.C <= kStageCap);
+
+    float mine = 0.f, cnt = 0.f;
+    // every lane of a group walks the same pixels, so the loop is group-uniform
+    const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
+    for (int64_t r = 0; r < rounds; ++r) {
+        const int64_t pix = (r * gridDim.x + blockIdx.x) * kPix + grp;
+        const bool live = pix < p.P;
+        const int64_t pc = live ? pix : 0;
+        const int64_t n = pc / p.m_size;
+        const T *xs = x + (pc + n * (int64_t)(p.C - 1) * p.m_size);
+        const int64_t lb = lab[pc];
+
+        float mx = -INFINITY;
+        for (int j = sub; j < p.C; j += G) {
+            const float t = load_one(xs + (int64_t)j * p.m_size);
+            if (staged) stage[j] = t;
+            mx = fmaxf(mx, t);
+        }
+        mx = group_reduce<G>(mx, OpMax());
+        float s = 0.f;
+        for (int j = sub; j < p.C; j += G) {
+            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            s += fast_exp(t - mx);
+        }
+        s = group_reduce<G>(s, OpSum());
+        const float lse = logf(s);
+        float acc = 0.f;
+        for (int j = sub; j < p.C; j += G) {
+            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            acc -= ((t - mx) - lse) * ((lb == j) ? p.w_pos : p.w_neg);
+        }
+        acc = group_reduce<G>(acc, OpSum());
+        const bool valid = live && (lb != p.ignore);
+        if (live && sub == 0) {
+            if (loss) loss[pix] = valid ? acc : 0.f;
+            mine += valid ? acc : 0.f;
+            cnt += valid ? 1.f : 0.f;
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);     // exact while a block sees < 2^24 pixels
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int G>
+__global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
+                                                     const int64_t *__restrict__ lab,
+                                                     const Upstream up, T *__restrict__ grad,
+                                                     const LsrParams p) {
+    constexpr int kPix = 256 / G;
+    __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
+    const int sub = threadIdx.x % G;
+    const int grp = threadIdx.x / G;
+    float *stage = stage_mem + ((G == 64) ? grp * kStageCap : 0);
+    const bool staged = (G == 64) && (p.C <= kStageCap);
+
+    const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
+    for (int64_t r = 0; r < rounds; ++r) {
+        const int64_t pix = (r * gridDim.x + blockIdx.x) * kPix + grp;
+        const bool live = pix < p.P;
+        const int64_t pc = live ? pix : 0;
+        const int64_t n = pc / p.m_size;
+        const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
+        const T *xs = x + base;
+        T *gs = grad + base;
+        const int64_t lb = lab[pc];
+        float go[1];
+        load_upstream<1>(up, pc, go);
+
+        float mx = -INFINITY;
+        for (int j = sub; j < p.C; j += G) {
+            const float t = load_one(xs + (int64_t)j * p.m_size);
+            if (staged) stage[j] = t;
+            mx = fmaxf(mx, t);
+        }
+        mx = group_reduce<G>(mx, OpMax());
+        float s = 0.f;
+        for (int j = sub; j < p.C; j += G) {
+            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float e = fast_exp(t - mx);
+            if (staged) stage[j] = e;
+            s += e;
+        }
+        s = group_reduce<G>(s, OpSum());
+        if (live) {
+            const float gk = (lb == p.ignore) ? 0.f : go[0];
+            const float scale = p.sumw * gk / s;
+            for (int j = sub; j < p.C; j += G) {
+                const float e = staged ? stage[j] : fast_exp(load_one(xs + (int64_t)j * p.m_size) - mx);
+                store_one(gs + (int64_t)j * p.m_size, e * scale - ((lb == j) ? p.w_pos : p.w_neg) * gk);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------ dispatch ----
+
+inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float smooth) {
+    LsrParams p;
+    p.P = n_size * m_size;
+    p.m_size = m_size;
+    p.C = (int)dimsize;
+    p.ignore = ignore;
+    p.w_pos = 1.f - smooth;                        // csrc/lsr_kernel.cu:83
+    p.w_neg = smooth / (float)dimsize;             // csrc/lsr_kernel.cu:84
+    p.sumw = p.w_neg * (float)(dimsize - 1) + p.w_pos;   // csrc/lsr_kernel.cu:125
+    return p;
+}
+
+template <class T, int V, bool Reduce>
+static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
+                                hipStream_t st) {
+    const unsigned grid = regs_grid<V>(p.P);
+    const bool uni = tiles_are_uniform(p.m_size, V);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                               \
+    case K:                                                                                                       \
+        if (uni) hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, true, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
+                                    st, x, lab, loss, part, p);                                                   \
+        else hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, false, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st,  \
+                                x, lab, loss, part, p);                                                           \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+    }
+    return grid;
+}
+
+template <class T, int V>
+static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
+                            hipStream_t st) {
+    const unsigned grid = regs_grid<V>(p.P);
+    const bool uni = tiles_are_uniform(p.m_size, V);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                              \
+    case K:                                                                                                      \
+        if (uni) hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
+                                    lab, up, grad, p);                                                           \
+        else hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, false>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, \
+                                up, grad, p);                                                                    \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+    }
+}
+
+// Launches the forward; returns the number of blocks that wrote partials.
+template <class T, bool Reduce>
+static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
+                        hipStream_t st) {
+    constexpr int V = ElemTraits<T>::kVec;
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr)) {
+        case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::Wave: {
+            const unsigned grid = group_grid(p.P, 4);
+            hipLaunchKernelGGL((lsr_fwd_group<T, 64, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            return grid;
+        }
+        case Shape::Lane: {
+            const unsigned grid = group_grid(p.P, 256);
+            hipLaunchKernelGGL((lsr_fwd_group<T, 1, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            return grid;
+        }
+    }
+    return 0;
+}
+
+template <class T>
+void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &up, T *grad_logits,
+                           const LsrParams &p, hipStream_t st) {
+    constexpr int V = ElemTraits<T>::kVec;
+    const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr)) {
+        case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::Wave:
+            hipLaunchKernelGGL((lsr_bwd_group<T, 64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, up,
+                               grad_logits, p);
+            break;
+        case Shape::Lane:
+            hipLaunchKernelGGL((lsr_bwd_group<T, 1>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, logits, labels, up,
+                               grad_logits, p);
+            break;
+    }
+}
+
+// Per-dtype entry into the kernels of this header; explicitly instantiated in lsr_f32.hip,
+// lsr_f16.hip and lsr_bf16.hip so that the three element types compile in parallel.
+template <class T>
+unsigned lsr_forward_typed(const T *logits, const int64_t *labels, float *losses, Partials part, bool reduce,
+                           const LsrParams &p, hipStream_t st) {
+    return reduce ? forward_shape<T, true>(logits, labels, losses, part, p, st)
+                  : forward_shape<T, false>(logits, labels, losses, part, p, st);
+}
+
+#define PLH_LSR_EXTERN(T)                                                                                           \
+    extern template unsigned lsr_forward_typed<T>(const T *, const int64_t *, float *, Partials, bool,              \
+                                                  const LsrParams &, hipStream_t);                                  \
+    extern template void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, \
+                                               hipStream_t);
+
+#define PLH_LSR_INSTANTIATE(T)                                                                                      \
+    template unsigned lsr_forward_typed<T>(const T *, const int64_t *, float *, Partials, bool, const LsrParams &,  \
+                                           hipStream_t);                                                            \
+    template void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, hipStream_t);
+
+}  // namespace plh

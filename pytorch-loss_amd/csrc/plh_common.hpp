@@ -39,7 +39,8 @@ __device__ __forceinline__ int64_t ceil_div_dev(int64_t a, int64_t b) { return (
 
 // Checks for the (n_size, dimsize, m_size) entry points. `out` is the tensor written.
 inline int check_slice_args(const void *logits, const void *labels, const void *out,
-                            int64_t n_size, int64_t dimsize, int64_t m_size) {
+                            int64_t n_size, int64_t dimsize, int64_t m_size, size_t logits_elem = 4,
+                            size_t out_elem = 4) {
     if (n_size < 0 || dimsize < 0 || m_size < 0) return PLH_ERR_BAD_SIZE;
     if (n_size > kMaxNumel || dimsize > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
     if (dimsize > (int64_t)1 << 30) return PLH_ERR_BAD_SIZE;
@@ -47,7 +48,7 @@ inline int check_slice_args(const void *logits, const void *labels, const void *
     if (numel > (double)kMaxNumel) return PLH_ERR_BAD_SIZE;
     if (numel == 0) return PLH_OK;
     if (!logits || !labels || !out) return PLH_ERR_NULL_POINTER;
-    if (misaligned(logits, 4) || misaligned(out, 4) || misaligned(labels, 8)) return PLH_ERR_MISALIGNED;
+    if (misaligned(logits, logits_elem) || misaligned(out, out_elem) || misaligned(labels, 8)) return PLH_ERR_MISALIGNED;
     return PLH_OK;
 }
 
@@ -58,20 +59,22 @@ inline int check_gout(const void *gout, int64_t stride) {
     return PLH_OK;
 }
 
-// Which execution shape serves a (dimsize, m_size) problem. The float pointers
-// passed in (nullptr = not used) must all be 8-byte aligned for the 2-pixel
-// vector form, and the labels 16-byte aligned.
-enum class Shape { Regs2, Regs1, Wave, Lane };
+// Which execution shape serves a (dimsize, m_size) problem. The vector form of the regs shape
+// moves V pixels per thread (2 for fp32 logits, 4 for 16-bit logits: 8 bytes per lane and channel
+// either way); it needs m_size % V == 0 and every tensor aligned to its V-element access:
+// `typed0/typed1` hold `elem`-byte elements (logits, gradient), `f32a/f32b` fp32 (losses, upstream
+// gradient), labels int64. nullptr = tensor not used.
+enum class Shape { RegsVec, RegsOne, Wave, Lane };
 
 constexpr int kMaxRegsChannels = 32;
 
-inline Shape pick_shape(int64_t dimsize, int64_t m_size, const void *f0, const void *f1,
-                        const void *labels, const void *f2, const void *f3) {
+inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, const void *typed0, const void *typed1,
+                        const void *labels, const void *f32a, const void *f32b) {
     if (dimsize <= kMaxRegsChannels) {
-        const bool vec = (m_size % 2 == 0) && !(f0 && misaligned(f0, 8)) && !(f1 && misaligned(f1, 8)) &&
-                         !(f2 && misaligned(f2, 8)) && !(f3 && misaligned(f3, 8)) &&
-                         !(labels && misaligned(labels, 16));
-        return vec ? Shape::Regs2 : Shape::Regs1;
+        const bool vec = (m_size % V == 0) && !(typed0 && misaligned(typed0, V * elem)) &&
+                         !(typed1 && misaligned(typed1, V * elem)) && !(f32a && misaligned(f32a, V * 4)) &&
+                         !(f32b && misaligned(f32b, V * 4)) && !(labels && misaligned(labels, 16));
+        return vec ? Shape::RegsVec : Shape::RegsOne;
     }
     return m_size == 1 ? Shape::Wave : Shape::Lane;
 }
@@ -83,12 +86,40 @@ inline unsigned group_grid(int64_t pixels, int pixels_per_block) {
     return (unsigned)(want < cap ? (want > 0 ? want : 1) : cap);
 }
 
-// ---- vector access -----------------------------------------------------------
+// ---- element types -----------------------------------------------------------
+// Logits and gradients may be fp32, fp16 or bf16 in memory; arithmetic is always fp32.
+struct f16 { uint16_t bits; };
+struct bf16 { uint16_t bits; };
 
-template <int V> struct Vec;
-template <> struct Vec<1> { using type = float; };
-template <> struct Vec<2> { using type = float2; };
-template <> struct Vec<4> { using type = float4; };
+template <class T> struct ElemTraits;
+template <> struct ElemTraits<float> { static constexpr int kVec = 2; static constexpr int32_t kTag = PLH_DTYPE_F32; };
+template <> struct ElemTraits<f16> { static constexpr int kVec = 4; static constexpr int32_t kTag = PLH_DTYPE_F16; };
+template <> struct ElemTraits<bf16> { static constexpr int kVec = 4; static constexpr int32_t kTag = PLH_DTYPE_BF16; };
+
+inline size_t dtype_size(int32_t dtype) { return dtype == PLH_DTYPE_F32 ? 4 : 2; }
+inline bool dtype_ok(int32_t dtype) { return dtype == PLH_DTYPE_F32 || dtype == PLH_DTYPE_F16 || dtype == PLH_DTYPE_BF16; }
+
+// Calls f(T{}) with the element type that `dtype` names.
+template <class F>
+inline int dispatch_dtype(int32_t dtype, F &&f) {
+    switch (dtype) {
+        case PLH_DTYPE_F32: f(float{}); return PLH_OK;
+        case PLH_DTYPE_F16: f(f16{}); return PLH_OK;
+        case PLH_DTYPE_BF16: f(bf16{}); return PLH_OK;
+        default: return PLH_ERR_BAD_DTYPE;
+    }
+}
+
+__device__ __forceinline__ float widen(uint16_t bits, f16) { return (float)__builtin_bit_cast(_Float16, bits); }
+__device__ __forceinline__ float widen(uint16_t bits, bf16) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
+__device__ __forceinline__ uint16_t narrow(float v, f16) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+__device__ __forceinline__ uint16_t narrow(float v, bf16) {          // round to nearest even, NaN stays NaN
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+// ---- vector access -----------------------------------------------------------
 
 // All tensors of this path are streamed exactly once, so loads and stores carry the
 // non-temporal hint: lines are not kept in L2 / Infinity Cache at the expense of others.
@@ -122,6 +153,45 @@ __device__ __forceinline__ void store_vec(float *p, const float (&v)[V]) {
     }
 }
 
+typedef unsigned short plh_h2 __attribute__((ext_vector_type(2)));
+typedef unsigned short plh_h4 __attribute__((ext_vector_type(4)));
+
+template <int V, class T>
+__device__ __forceinline__ void load_vec(const T *p, float (&out)[V]) {      // T = f16 or bf16
+    const unsigned short *q = reinterpret_cast<const unsigned short *>(p);
+    if constexpr (V == 1) {
+        out[0] = widen(__builtin_nontemporal_load(q), T{});
+    } else if constexpr (V == 2) {
+        const plh_h2 t = __builtin_nontemporal_load(reinterpret_cast<const plh_h2 *>(q));
+        out[0] = widen(t.x, T{}); out[1] = widen(t.y, T{});
+    } else {
+        const plh_h4 t = __builtin_nontemporal_load(reinterpret_cast<const plh_h4 *>(q));
+        out[0] = widen(t.x, T{}); out[1] = widen(t.y, T{}); out[2] = widen(t.z, T{}); out[3] = widen(t.w, T{});
+    }
+}
+
+template <int V, class T>
+__device__ __forceinline__ void store_vec(T *p, const float (&v)[V]) {       // T = f16 or bf16
+    unsigned short *q = reinterpret_cast<unsigned short *>(p);
+    if constexpr (V == 1) {
+        __builtin_nontemporal_store(narrow(v[0], T{}), q);
+    } else if constexpr (V == 2) {
+        const plh_h2 t = {narrow(v[0], T{}), narrow(v[1], T{})};
+        __builtin_nontemporal_store(t, reinterpret_cast<plh_h2 *>(q));
+    } else {
+        const plh_h4 t = {narrow(v[0], T{}), narrow(v[1], T{}), narrow(v[2], T{}), narrow(v[3], T{})};
+        __builtin_nontemporal_store(t, reinterpret_cast<plh_h4 *>(q));
+    }
+}
+
+// single elements, cached (the group kernels re-read what they have just touched)
+__device__ __forceinline__ float load_one(const float *p) { return *p; }
+__device__ __forceinline__ float load_one(const f16 *p) { return widen(p->bits, f16{}); }
+__device__ __forceinline__ float load_one(const bf16 *p) { return widen(p->bits, bf16{}); }
+__device__ __forceinline__ void store_one(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store_one(f16 *p, float v) { p->bits = narrow(v, f16{}); }
+__device__ __forceinline__ void store_one(bf16 *p, float v) { p->bits = narrow(v, bf16{}); }
+
 template <int V>
 __device__ __forceinline__ void load_labels(const int64_t *p, int64_t (&out)[V]) {
     if constexpr (V == 1) {
@@ -132,22 +202,6 @@ __device__ __forceinline__ void load_labels(const int64_t *p, int64_t (&out)[V])
             const plh_l2 t = __builtin_nontemporal_load(reinterpret_cast<const plh_l2 *>(p + k));
             out[k] = t.x; out[k + 1] = t.y;
         }
-    }
-}
-
-// Upstream gradient for V consecutive loss elements starting at `i`.
-// gout == nullptr: 1; stride 0: broadcast scalar; stride 1: per element.
-template <int V>
-__device__ __forceinline__ void load_gout(const float *gout, int64_t stride, int64_t i, float (&out)[V]) {
-    if (gout == nullptr) {
-#pragma unroll
-        for (int k = 0; k < V; ++k) out[k] = 1.0f;
-    } else if (stride == 0) {
-        const float g = *gout;
-#pragma unroll
-        for (int k = 0; k < V; ++k) out[k] = g;
-    } else {
-        load_vec<V>(gout + i, out);
     }
 }
 
@@ -258,10 +312,8 @@ struct PixelRef {
         }
     }
     // address of channel j for this thread's pixels
-    __device__ __forceinline__ const float *chan(const float *t, int j, int64_t m_size) const {
-        return (t + (base + (int64_t)j * m_size)) + lane_off;
-    }
-    __device__ __forceinline__ float *chan(float *t, int j, int64_t m_size) const {
+    template <class T>
+    __device__ __forceinline__ T *chan(T *t, int j, int64_t m_size) const {
         return (t + (base + (int64_t)j * m_size)) + lane_off;
     }
 };

@@ -17,35 +17,36 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpytorch_loss_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 
 _p = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _f32 = ctypes.c_float
+_i32 = ctypes.c_int32
 
 _SIGNATURES = {
     "plh_abi_version": (ctypes.c_int, []),
     "plh_error_string": (ctypes.c_char_p, [ctypes.c_int]),
-    "plh_lsr_forward": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_lsr_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_reduce_workspace_bytes": (_i64, [_i64]),
-    "plh_lsr_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_lsr_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_focal_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _f32, _f32, _p]),
-    "plh_focal_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _i64, _f32, _f32, _p]),
-    "plh_lmargin_forward_reduced": (ctypes.c_int, [_p, _p, _p, _p, _p, ctypes.c_int32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_lmargin_backward_scaled": (ctypes.c_int, [_p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_focal_forward": (ctypes.c_int, [_p, _p, _p, _i64, _f32, _f32, _p]),
-    "plh_focal_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _f32, _f32, _p]),
-    "plh_focal_forward_backward": (ctypes.c_int, [_p, _p, _p, _p, _i64, _f32, _f32, _p]),
-    "plh_lmargin_forward": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_lmargin_backward": (ctypes.c_int, [_p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
-    "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_focal_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i32, _p, _i64, _i64, _f32, _f32, _p]),
+    "plh_focal_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_lmargin_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
-    "plh_lovasz_forward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
-    "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
 
@@ -97,10 +98,27 @@ def _require_gpu(what, *tensors):
 
 
 def _f32c(t):
-    """fp32 contiguous view/copy (fp16/bf16/fp64 inputs are computed in fp32)."""
+    """fp32 contiguous view/copy."""
     if t.dtype != torch.float32:
         t = t.float()
     return t.contiguous()
+
+
+_DTYPE_TAGS = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _logits(t):
+    """-> (contiguous tensor in a dtype the kernels read natively, dtype tag). fp32, fp16 and bf16
+    are read as they are (arithmetic is fp32 in every case); anything else is cast to fp32 first."""
+    if t.dtype not in _DTYPE_TAGS:
+        t = t.float()
+    return t.contiguous(), _DTYPE_TAGS[t.dtype]
+
+
+def _loss_dtype(logits):
+    """dtype of the returned losses: the logits' own, except under autocast, where the reference's
+    custom_fwd(cast_inputs=float32) makes the whole op fp32."""
+    return torch.float32 if torch.is_autocast_enabled("cuda") else logits.dtype
 
 
 def _labels_i64(labels, logits, what):
@@ -144,34 +162,36 @@ def _back_to(t, dtype):
 
 
 # ------------------------------------------------------------------ LSR ----
+# LSR and large-margin share their marshalling: `entry` names the library function, `param` is the
+# smoothing factor or the margin weight.
 
-def lsr_forward(logits, labels, ignore_index, smooth):
-    _require_gpu("LSR loss", logits, labels)
-    n, c, m = _dims(logits, "lsr_forward")
-    x = _f32c(logits)
-    lb = _labels_i64(labels, logits, "lsr_forward")
+def _pixel_forward(entry, what, logits, labels, ignore_index, param):
+    _require_gpu(what, logits, labels)
+    n, c, m = _dims(logits, entry)
+    x, tag = _logits(logits)
+    lb = _labels_i64(labels, logits, entry)
     losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
     if x.numel() == 0:
-        return _back_to(losses.zero_(), logits.dtype)
+        return _back_to(losses.zero_(), _loss_dtype(logits))
     with torch.cuda.device_of(x):
-        _check(load().plh_lsr_forward(_ptr(x), _ptr(lb), _ptr(losses), n, c, m,
-                                      int(ignore_index), float(smooth), _stream()))
-    return _back_to(losses, logits.dtype)
+        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(losses), n, c, m, int(ignore_index), float(param),
+                                      _stream()))
+    return _back_to(losses, _loss_dtype(logits))
 
 
-def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None):
+def _pixel_backward(entry, what, logits, labels, ignore_index, param, grad_output):
     """dloss/dlogits, already multiplied by ``grad_output`` (None = unit upstream gradient)."""
-    _require_gpu("LSR loss", logits, labels)
-    n, c, m = _dims(logits, "lsr_backward")
-    x = _f32c(logits)
-    lb = _labels_i64(labels, logits, "lsr_backward")
+    _require_gpu(what, logits, labels)
+    n, c, m = _dims(logits, entry)
+    x, tag = _logits(logits)
+    lb = _labels_i64(labels, logits, entry)
     grad = torch.empty_like(x)
     if x.numel() == 0:
         return _back_to(grad, logits.dtype)
     go, stride = _upstream(grad_output, lb.shape)
     with torch.cuda.device_of(x):
-        _check(load().plh_lsr_backward(_ptr(x), _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
-                                       int(ignore_index), float(smooth), _stream()))
+        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
+                                      int(ignore_index), float(param), _stream()))
     return _back_to(grad, logits.dtype)
 
 
@@ -189,33 +209,41 @@ def _scalar_f32(t):
 
 
 def _pixel_forward_reduced(entry, what, logits, labels, ignore_index, param, mean):
-    """Shared by LSR and large-margin: -> (loss 0-dim fp32, n_valid 0-dim int64)."""
+    """-> (loss 0-dim, n_valid 0-dim int64)."""
     _require_gpu(what, logits, labels)
     n, c, m = _dims(logits, entry)
-    x = _f32c(logits)
+    x, tag = _logits(logits)
     lb = _labels_i64(labels, logits, entry)
     loss = torch.empty((), dtype=torch.float32, device=x.device)
     n_valid = torch.empty((), dtype=torch.int64, device=x.device)
     ws, ws_bytes = _reduce_workspace(n * m, x.device)
     with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), _ptr(lb), None, _ptr(loss), _ptr(n_valid), 1 if mean else 0,
+        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), None, _ptr(loss), _ptr(n_valid), 1 if mean else 0,
                                       _ptr(ws), ws_bytes, n, c, m, int(ignore_index), float(param), _stream()))
-    return _back_to(loss, logits.dtype), n_valid
+    return _back_to(loss, _loss_dtype(logits)), n_valid
 
 
 def _pixel_backward_scaled(entry, what, logits, labels, ignore_index, param, grad_scalar, divide_by):
     _require_gpu(what, logits, labels)
     n, c, m = _dims(logits, entry)
-    x = _f32c(logits)
+    x, tag = _logits(logits)
     lb = _labels_i64(labels, logits, entry)
     grad = torch.empty_like(x)
     if x.numel() == 0:
         return _back_to(grad, logits.dtype)
     go = _scalar_f32(grad_scalar)
     with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), _ptr(lb), _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), n, c, m,
+        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), n, c, m,
                                       int(ignore_index), float(param), _stream()))
     return _back_to(grad, logits.dtype)
+
+
+def lsr_forward(logits, labels, ignore_index, smooth):
+    return _pixel_forward("plh_lsr_forward", "LSR loss", logits, labels, ignore_index, smooth)
+
+
+def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None):
+    return _pixel_backward("plh_lsr_backward", "LSR loss", logits, labels, ignore_index, smooth, grad_output)
 
 
 def lsr_forward_reduced(logits, labels, ignore_index, smooth, mean):
@@ -227,69 +255,16 @@ def lsr_backward_scaled(logits, labels, ignore_index, smooth, grad_scalar, divid
                                   grad_scalar, divide_by)
 
 
-# ---------------------------------------------------------------- focal ----
-
-def _focal_pair(logits, labels, what):
-    _require_gpu("focal loss", logits, labels)
-    if tuple(labels.shape) != tuple(logits.shape):
-        raise RuntimeError("%s: labels and logits must have the same shape" % what)
-    return _f32c(logits), _f32c(labels)
-
-
-def focal_forward(logits, labels, gamma, alpha):
-    x, y = _focal_pair(logits, labels, "focalloss_forward")
-    losses = torch.empty_like(x)
-    if x.numel():
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_forward(_ptr(x), _ptr(y), _ptr(losses), x.numel(),
-                                            float(gamma), float(alpha), _stream()))
-    return _back_to(losses, logits.dtype)
-
-
-def focal_backward(logits, labels, gamma, alpha, grad_output=None):
-    x, y = _focal_pair(logits, labels, "focalloss_backward")
-    grad = torch.empty_like(x)
-    if x.numel():
-        go, stride = _upstream(grad_output, x.shape)
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_backward(_ptr(x), _ptr(y), _ptr(go), stride, _ptr(grad), x.numel(),
-                                             float(gamma), float(alpha), _stream()))
-    return _back_to(grad, logits.dtype)
-
-
-def focal_forward_backward(logits, labels, gamma, alpha):
-    x, y = _focal_pair(logits, labels, "focalloss_forward_backward")
-    losses = torch.empty_like(x)
-    grad = torch.empty_like(x)
-    if x.numel():
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_forward_backward(_ptr(x), _ptr(y), _ptr(losses), _ptr(grad), x.numel(),
-                                                     float(gamma), float(alpha), _stream()))
-    return _back_to(losses, logits.dtype), _back_to(grad, logits.dtype)
-
-
-def focal_forward_reduced(logits, labels, gamma, alpha, mean):
-    x, y = _focal_pair(logits, labels, "focalloss_forward")
-    loss = torch.empty((), dtype=torch.float32, device=x.device)
-    ws, ws_bytes = _reduce_workspace(x.numel(), x.device)
-    with torch.cuda.device_of(x):
-        _check(load().plh_focal_forward_reduced(_ptr(x), _ptr(y), None, _ptr(loss), 1 if mean else 0, _ptr(ws),
-                                                ws_bytes, x.numel(), float(gamma), float(alpha), _stream()))
-    return _back_to(loss, logits.dtype)
-
-
-def focal_backward_scaled(logits, labels, gamma, alpha, grad_scalar, scale):
-    x, y = _focal_pair(logits, labels, "focalloss_backward")
-    grad = torch.empty_like(x)
-    if x.numel():
-        go = _scalar_f32(grad_scalar)
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_backward_scaled(_ptr(x), _ptr(y), _ptr(go), float(scale), _ptr(grad), x.numel(),
-                                                    float(gamma), float(alpha), _stream()))
-    return _back_to(grad, logits.dtype)
-
-
 # -------------------------------------------------------------- lmargin ----
+
+def lmargin_forward(logits, labels, lam, ignore_index):
+    return _pixel_forward("plh_lmargin_forward", "large margin loss", logits, labels, ignore_index, lam)
+
+
+def lmargin_backward(logits, labels, lam, ignore_index, grad_output=None):
+    return _pixel_backward("plh_lmargin_backward", "large margin loss", logits, labels, ignore_index, lam,
+                           grad_output)
+
 
 def lmargin_forward_reduced(logits, labels, lam, ignore_index, mean):
     return _pixel_forward_reduced("plh_lmargin_forward_reduced", "large margin loss", logits, labels, ignore_index,
@@ -301,51 +276,87 @@ def lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_scalar, divi
                                   lam, grad_scalar, divide_by)
 
 
-def lmargin_forward(logits, labels, lam, ignore_index):
-    _require_gpu("large margin loss", logits, labels)
-    n, c, m = _dims(logits, "l_margin_forward")
-    x = _f32c(logits)
-    lb = _labels_i64(labels, logits, "l_margin_forward")
-    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
-    if x.numel() == 0:
-        return _back_to(losses.zero_(), logits.dtype)
-    with torch.cuda.device_of(x):
-        _check(load().plh_lmargin_forward(_ptr(x), _ptr(lb), _ptr(losses), n, c, m,
-                                          int(ignore_index), float(lam), _stream()))
-    return _back_to(losses, logits.dtype)
-
-
-def lmargin_backward(logits, labels, lam, ignore_index, grad_output=None):
-    _require_gpu("large margin loss", logits, labels)
-    n, c, m = _dims(logits, "l_margin_backward")
-    x = _f32c(logits)
-    lb = _labels_i64(labels, logits, "l_margin_backward")
-    grad = torch.empty_like(x)
-    if x.numel() == 0:
-        return _back_to(grad, logits.dtype)
-    go, stride = _upstream(grad_output, lb.shape)
-    with torch.cuda.device_of(x):
-        _check(load().plh_lmargin_backward(_ptr(x), _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
-                                           int(ignore_index), float(lam), _stream()))
-    return _back_to(grad, logits.dtype)
-
-
 def lmargin_forward_backward(logits, labels, lam, ignore_index):
     """-> (losses, grad under unit upstream gradient, valid_cnt int64[1])"""
     _require_gpu("large margin loss", logits, labels)
     n, c, m = _dims(logits, "l_margin_forward_backward")
-    x = _f32c(logits)
+    x, tag = _logits(logits)
     lb = _labels_i64(labels, logits, "l_margin_forward_backward")
     losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
     grad = torch.empty_like(x)
     cnt = torch.zeros(1, dtype=torch.int64, device=x.device)
     if x.numel():
         with torch.cuda.device_of(x):
-            _check(load().plh_lmargin_forward_backward(_ptr(x), _ptr(lb), _ptr(losses), _ptr(grad), _ptr(cnt),
+            _check(load().plh_lmargin_forward_backward(_ptr(x), tag, _ptr(lb), _ptr(losses), _ptr(grad), _ptr(cnt),
                                                        n, c, m, int(ignore_index), float(lam), _stream()))
     else:
         losses.zero_()
-    return _back_to(losses, logits.dtype), _back_to(grad, logits.dtype), cnt
+    return _back_to(losses, _loss_dtype(logits)), _back_to(grad, logits.dtype), cnt
+
+
+# ---------------------------------------------------------------- focal ----
+
+def _focal_pair(logits, labels, what):
+    """Logits and labels in one dtype the kernels read; mixed or exotic dtypes are computed from fp32 copies."""
+    _require_gpu("focal loss", logits, labels)
+    if tuple(labels.shape) != tuple(logits.shape):
+        raise RuntimeError("%s: labels and logits must have the same shape" % what)
+    if logits.dtype == labels.dtype and logits.dtype in _DTYPE_TAGS:
+        return logits.contiguous(), labels.contiguous(), _DTYPE_TAGS[logits.dtype]
+    return _f32c(logits), _f32c(labels), 0
+
+
+def focal_forward(logits, labels, gamma, alpha):
+    x, y, tag = _focal_pair(logits, labels, "focalloss_forward")
+    losses = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    if x.numel():
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_forward(_ptr(x), tag, _ptr(y), _ptr(losses), x.numel(),
+                                            float(gamma), float(alpha), _stream()))
+    return _back_to(losses, _loss_dtype(logits))
+
+
+def focal_backward(logits, labels, gamma, alpha, grad_output=None):
+    x, y, tag = _focal_pair(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(x)
+    if x.numel():
+        go, stride = _upstream(grad_output, x.shape)
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_backward(_ptr(x), tag, _ptr(y), _ptr(go), stride, _ptr(grad), x.numel(),
+                                             float(gamma), float(alpha), _stream()))
+    return _back_to(grad, logits.dtype)
+
+
+def focal_forward_backward(logits, labels, gamma, alpha):
+    x, y, tag = _focal_pair(logits, labels, "focalloss_forward_backward")
+    losses = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    grad = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_forward_backward(_ptr(x), tag, _ptr(y), _ptr(losses), _ptr(grad), x.numel(),
+                                                     float(gamma), float(alpha), _stream()))
+    return _back_to(losses, _loss_dtype(logits)), _back_to(grad, logits.dtype)
+
+
+def focal_forward_reduced(logits, labels, gamma, alpha, mean):
+    x, y, tag = _focal_pair(logits, labels, "focalloss_forward")
+    loss = torch.empty((), dtype=torch.float32, device=x.device)
+    ws, ws_bytes = _reduce_workspace(x.numel(), x.device)
+    with torch.cuda.device_of(x):
+        _check(load().plh_focal_forward_reduced(_ptr(x), tag, _ptr(y), None, _ptr(loss), 1 if mean else 0, _ptr(ws),
+                                                ws_bytes, x.numel(), float(gamma), float(alpha), _stream()))
+    return _back_to(loss, _loss_dtype(logits))
+
+
+def focal_backward_scaled(logits, labels, gamma, alpha, grad_scalar, scale):
+    x, y, tag = _focal_pair(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(x)
+    if x.numel():
+        go = _scalar_f32(grad_scalar)
+        with torch.cuda.device_of(x):
+            _check(load().plh_focal_backward_scaled(_ptr(x), tag, _ptr(y), _ptr(go), float(scale), _ptr(grad),
+                                                    x.numel(), float(gamma), float(alpha), _stream()))
+    return _back_to(grad, logits.dtype)
 
 
 # --------------------------------------------------------------- lovasz ----
@@ -359,31 +370,31 @@ def _lovasz_limits(logits, what):
 
 
 def lovasz_forward(logits, labels, ignore_index):
-    """-> (losses[C], jacc[C, N*M])"""
+    """-> (losses[C], jacc[C, N*M] fp32)"""
     _require_gpu("lovasz softmax function", logits, labels)
     _lovasz_limits(logits, "lovasz_softmax_forward")
     n, c, m = _dims(logits, "lovasz_softmax_forward")
-    x = _f32c(logits)
+    x, tag = _logits(logits)
     lb = _labels_i64(labels, logits, "lovasz_softmax_forward")
     losses = torch.empty((c,), dtype=torch.float32, device=x.device)
     jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
     if x.numel() == 0:
-        return _back_to(losses.zero_(), logits.dtype), jacc
+        return _back_to(losses.zero_(), _loss_dtype(logits)), jacc
     lib = load()
     ws_bytes = int(lib.plh_lovasz_workspace_bytes(n, c, m))
     if ws_bytes < 0:
         _check(ws_bytes)
     workspace = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
     with torch.cuda.device_of(x):
-        _check(lib.plh_lovasz_forward(_ptr(x), _ptr(lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
+        _check(lib.plh_lovasz_forward(_ptr(x), tag, _ptr(lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
                                       n, c, m, int(ignore_index), _stream()))
-    return _back_to(losses, logits.dtype), jacc
+    return _back_to(losses, _loss_dtype(logits)), jacc
 
 
 def lovasz_backward(grad_output, logits, labels, jacc, ignore_index):
     _require_gpu("lovasz softmax function", logits, labels, grad_output, jacc)
     n, c, m = _dims(logits, "lovasz_softmax_backward")
-    x = _f32c(logits)
+    x, tag = _logits(logits)
     lb = _labels_i64(labels, logits, "lovasz_softmax_backward")
     grad = torch.empty_like(x)
     if x.numel() == 0:
@@ -393,7 +404,7 @@ def lovasz_backward(grad_output, logits, labels, jacc, ignore_index):
         raise RuntimeError("lovasz_softmax_backward: grad_output must have C elements and jacc C*N*M fp32 elements")
     jc = jacc.contiguous()
     with torch.cuda.device_of(x):
-        _check(load().plh_lovasz_backward(_ptr(go), _ptr(x), _ptr(lb), _ptr(jc), _ptr(grad), n, c, m,
+        _check(load().plh_lovasz_backward(_ptr(go), _ptr(x), tag, _ptr(lb), _ptr(jc), _ptr(grad), n, c, m,
                                           int(ignore_index), _stream()))
     return _back_to(grad, logits.dtype)
 

@@ -18,7 +18,7 @@ class FocalSigmoidLossFuncV3(torch.autograd.Function):
     """Recomputes everything from (logits, labels) in backward: nothing but the inputs is kept."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma):
         ctx.variables = (logits, labels, alpha, gamma)
         return _native.focal_forward(logits, labels, gamma, alpha)
@@ -35,7 +35,7 @@ class FocalSigmoidLossFuncV3FB(torch.autograd.Function):
     """Forward computes loss and gradient in one pass and keeps the gradient for backward."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma):
         loss, grads = _native.focal_forward_backward(logits, labels, gamma, alpha)
         ctx.variables = grads
@@ -54,7 +54,7 @@ class _FocalReducedFunction(torch.autograd.Function):
     fixed-order finish); backward folds the scalar upstream gradient and 1/numel into its kernel."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma, mean):
         ctx.variables = (logits, labels, alpha, gamma, mean)
         return _native.focal_forward_reduced(logits, labels, gamma, alpha, mean)

@@ -17,7 +17,7 @@ class LSRCrossEntropyFunctionV3(torch.autograd.Function):
     backward -> d/dlogits, with the upstream gradient folded into the same kernel."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lb_smooth, lb_ignore):
         ctx.variables = (logits, labels, lb_ignore, lb_smooth)
         return _native.lsr_forward(logits, labels, lb_ignore, lb_smooth)
@@ -37,7 +37,7 @@ class _LSRReducedFunction(torch.autograd.Function):
     upstream gradient and the 1/n_valid of a mean into the gradient kernel."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lb_smooth, lb_ignore, mean):
         loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean)
         ctx.variables = (logits, labels, lb_ignore, lb_smooth, n_valid if mean else None)

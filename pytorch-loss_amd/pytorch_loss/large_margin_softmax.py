@@ -15,7 +15,7 @@ class LargeMarginSoftmaxFuncV3(torch.autograd.Function):
     """forward -> per-pixel losses; backward recomputes from the inputs."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
         ctx.variables = (logits, labels, lam, ignore_index)
         return _native.lmargin_forward(logits, labels, lam, ignore_index)
@@ -33,7 +33,7 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
     kernel and kept for backward."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
         losses, grads, valid_cnt = _native.lmargin_forward_backward(logits, labels, lam, ignore_index)
         ctx.variables = grads
@@ -52,7 +52,7 @@ class _LargeMarginReducedFunction(torch.autograd.Function):
     """'sum' / 'mean' produced inside the forward kernel; see label_smooth._LSRReducedFunction."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam, ignore_index, mean):
         loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean)
         ctx.variables = (logits, labels, lam, ignore_index, n_valid if mean else None)

@@ -15,7 +15,7 @@ class LovaszSoftmaxFunctionV3(torch.autograd.Function):
     """Keeps the Jaccard differences (C x pixels, fp32) between forward and backward."""
 
     @staticmethod
-    @amp.custom_fwd(cast_inputs=torch.float32, device_type="cuda")
+    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, ignore_index):
         losses, jacc = _native.lovasz_forward(logits, labels, ignore_index)
         ctx.vars = (logits, labels, jacc, ignore_index)

@@ -37,13 +37,13 @@ def test_library_exports_every_declared_symbol(native):
         assert name in native._SIGNATURES, "binding lacks " + name
         assert len(native._SIGNATURES[name][1]) == n_args, name
     assert set(native._SIGNATURES) == set(decl)
-    assert lib.plh_abi_version() == 1
+    assert lib.plh_abi_version() == 2
 
 
 def test_error_strings(native):
     lib = native.load()
     assert lib.plh_error_string(0) == b"ok"
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         assert len(lib.plh_error_string(code)) > 5
     assert b"512" in lib.plh_error_string(-4)
     assert lib.plh_error_string(-99) == b"unknown error code"
@@ -57,25 +57,37 @@ def test_arguments_are_rejected_before_any_launch(native):
     lp = ctypes.cast(lab, ctypes.c_void_p)
     odd = ctypes.c_void_p(p.value + 2)
     # zero-sized problems are fine and launch nothing
-    assert lib.plh_lsr_forward(None, None, None, 0, 19, 16, 255, 0.1, None) == 0
-    assert lib.plh_focal_forward(None, None, None, 0, 2.0, 0.25, None) == 0
-    assert lib.plh_lovasz_forward(None, None, None, None, None, 0, 0, 19, 16, 255, None) == 0
+    assert lib.plh_lsr_forward(None, 0, None, None, 0, 19, 16, 255, 0.1, None) == 0
+    assert lib.plh_focal_forward(None, 1, None, None, 0, 2.0, 0.25, None) == 0
+    assert lib.plh_lovasz_forward(None, 2, None, None, None, None, 0, 0, 19, 16, 255, None) == 0
     assert lib.plh_stream_copy(None, None, 0, None) == 0
     # NULL / negative / misaligned / stride / class-count / workspace
-    assert lib.plh_lsr_forward(None, lp, p, 1, 2, 2, 255, 0.1, None) == -1
-    assert lib.plh_lsr_forward(p, lp, p, -1, 2, 2, 255, 0.1, None) == -2
-    assert lib.plh_lsr_forward(odd, lp, p, 1, 2, 2, 255, 0.1, None) == -6
-    assert lib.plh_lsr_backward(p, lp, p, 2, p, 1, 2, 2, 255, 0.1, None) == -3
-    assert lib.plh_lmargin_backward(p, lp, p, 7, p, 1, 2, 2, 255, 0.3, None) == -3
-    assert lib.plh_focal_backward(p, p, p, 3, p, 4, 2.0, 0.25, None) == -3
-    assert lib.plh_focal_forward(p, None, p, 4, 2.0, 0.25, None) == -1
-    assert lib.plh_lovasz_forward(p, lp, p, p, p, 1 << 20, 1, 512, 2, 255, None) == -4
+    assert lib.plh_lsr_forward(None, 0, lp, p, 1, 2, 2, 255, 0.1, None) == -1
+    assert lib.plh_lsr_forward(p, 0, lp, p, -1, 2, 2, 255, 0.1, None) == -2
+    assert lib.plh_lsr_forward(odd, 0, lp, p, 1, 2, 2, 255, 0.1, None) == -6
+    assert lib.plh_lsr_backward(p, 0, lp, p, 2, p, 1, 2, 2, 255, 0.1, None) == -3
+    assert lib.plh_lmargin_backward(p, 0, lp, p, 7, p, 1, 2, 2, 255, 0.3, None) == -3
+    assert lib.plh_focal_backward(p, 0, p, p, 3, p, 4, 2.0, 0.25, None) == -3
+    assert lib.plh_focal_forward(p, 0, None, p, 4, 2.0, 0.25, None) == -1
+    assert lib.plh_lovasz_forward(p, 0, lp, p, p, p, 1 << 20, 1, 512, 2, 255, None) == -4
     assert lib.plh_lovasz_workspace_bytes(1, 512, 4) == -4
     assert lib.plh_lovasz_workspace_bytes(1 << 20, 19, 1 << 12) == -2       # numel >= 2^31
     need = lib.plh_lovasz_workspace_bytes(2, 19, 64)
     assert need > 3 * 4 * 2 * 19 * 64
-    assert lib.plh_lovasz_forward(p, lp, p, p, None, need, 2, 19, 64, 255, None) == -5
-    assert lib.plh_lsr_forward_reduced(p, lp, None, p, None, 1, None, 0, 1, 2, 2, 255, 0.1, None) == -5
+    assert lib.plh_lovasz_forward(p, 0, lp, p, p, None, need, 2, 19, 64, 255, None) == -5
+    assert lib.plh_lsr_forward_reduced(p, 0, lp, None, p, None, 1, None, 0, 1, 2, 2, 255, 0.1, None) == -5
+    # element type tags other than fp32 / fp16 / bf16, on every op and before anything else is looked at
+    for bad in (-1, 3, 7):
+        assert lib.plh_lsr_forward(p, bad, lp, p, 1, 2, 2, 255, 0.1, None) == -7
+        assert lib.plh_lsr_backward(p, bad, lp, None, 0, p, 1, 2, 2, 255, 0.1, None) == -7
+        assert lib.plh_lmargin_forward(p, bad, lp, p, 1, 2, 2, 255, 0.3, None) == -7
+        assert lib.plh_lmargin_forward_backward(p, bad, lp, p, p, p, 1, 2, 2, 255, 0.3, None) == -7
+        assert lib.plh_focal_forward(p, bad, p, p, 4, 2.0, 0.25, None) == -7
+        assert lib.plh_focal_forward_backward(p, bad, p, p, p, 4, 2.0, 0.25, None) == -7
+        assert lib.plh_lovasz_forward(p, bad, lp, p, p, p, need, 2, 19, 64, 255, None) == -7
+        assert lib.plh_lovasz_backward(p, p, bad, lp, p, p, 2, 19, 64, 255, None) == -7
+    # 16-bit logits need 2-byte alignment only; an odd address is still refused
+    assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
     assert lib.plh_reduce_workspace_bytes(-1) == -2
 
