@@ -27,6 +27,14 @@ struct LmParams {
 
 // ---------------------------------------------------------------- regs ----
 
+// The target channel is taken out of the non-target statistics by overwriting its widened logit
+// with a large negative sentinel: its exponential is an exact 0 and 0 * sentinel stays 0, so the
+// inner loops carry no per-channel selects. exp(x - m_no) is evaluated as exp2(u), u = fma(x,
+// log2e, -c), c = fl(m_no * log2e); r = m_no*log2e - c (exact, one fma) is what the rounding of c
+// left out: it scales every e_j by 2^r, cancels in q_j = e_j / s_no and is taken back out of
+// log2(s_no), sum q_j u_j and the rebuilt full sum.
+constexpr float kLmMasked = -1e30f;
+
 template <class T, int CP, int V, bool Uniform, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                      const Upstream up,
@@ -39,16 +47,16 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     if (!Reduce && !live) return;
     const int64_t pix = at.pix;
 
-    float v[CP][V];
-#pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
     load_labels<V>(lab + pix, lb);
     float go[V];
     if constexpr (WantGrad) load_upstream<V>(up, pix, go);
 
     float out[V];
+    float g[WantGrad ? CP : 1][V];
+    unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
     unsigned n_valid = 0;
     float mine = 0.f;
     int cnt = 0;
@@ -56,57 +64,74 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     for (int k = 0; k < V; ++k) {
         bool ign;
         const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        float m_no = -INFINITY, x_y = -INFINITY;
+        keep[k] = ign ? 0u : 0xFFFFFFFFu;
+        float xv[CP];
+        float sx = 0.f, x_y = -INFINITY;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
+            if (chan_ok<CP>(j, p.C)) {
+                const float xj = Pack<T, V>::get(raw[j], k);
                 const bool hot = (tgt == j);
-                m_no = hot ? m_no : fmaxf(m_no, v[j][k]);
-                x_y = hot ? v[j][k] : x_y;
+                sx += xj;
+                x_y = hot ? xj : x_y;
+                xv[j] = hot ? kLmMasked : xj;
             }
+        float m_no = xv[0];
+#pragma unroll
+        for (int j = 1; j + 1 < CP - 3; j += 2) m_no = max3(m_no, xv[j], xv[j + 1]);
+#pragma unroll
+        for (int j = CP - 3; j < CP; ++j)
+            if (j > 0 && j < p.C) m_no = max3(m_no, xv[j], xv[j]);
         const float m_all = fmaxf(m_no, x_y);
-        // one exponential per channel: with t_j = x_j - m_no and e_j = exp(t_j) over j != y,
-        //   sum_j (q_j - coeff) log q_j = (sum e_j t_j)/s_no - lse_no - coeff * (sum t_j - (C-1) lse_no)
-        float e[WantGrad ? CP : 1];
-        float s_no = 0.f, sum_et = 0.f, sum_t = 0.f;
+
+        //   sum_j (q_j - coeff) log q_j = sum q_j t_j - lse_no - coeff * (sum t_j - others * lse_no),
+        //   t_j = x_j - m_no over the non-target channels
+        const float c = m_no * kLog2e;
+        const float r = __builtin_fmaf(m_no, kLog2e, -c);
+        float s_no = 0.f, sum_eu = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const bool hot = (tgt == j);
-                const float t = v[j][k] - m_no;
-                const float ej = hot ? 0.f : fast_exp(t);
-                if constexpr (WantGrad) e[j] = ej;
-                s_no += ej;
-                sum_et += ej * (hot ? 0.f : t);
-                sum_t += hot ? 0.f : t;
+            if (chan_ok<CP>(j, p.C)) {
+                const float u = __builtin_fmaf(xv[j], kLog2e, -c);
+                const float e = __builtin_amdgcn_exp2f(u);
+                s_no += e;
+                sum_eu = __builtin_fmaf(e, u, sum_eu);
+                if constexpr (WantGrad) xv[j] = e;
             }
-        const float t_all = fast_exp(m_no - m_all);
+        const float inv_no = __builtin_amdgcn_rcpf(s_no);
+        const float sum_qt = (sum_eu * inv_no - r) * kLn2;                       // sum q_j t_j
+        // full-softmax pieces: s_all = s_no_true * exp(m_no - m_all) + exp(x_y - m_all), s_no_true = s_no * 2^-r
+        const float t_all = __builtin_amdgcn_exp2f(__builtin_fmaf(m_no - m_all, kLog2e, -r));
         const float e_y = fast_exp(x_y - m_all);
-        const float s_all = s_no * t_all + e_y;
-        const float inv_no = 1.f / s_no;
+        const float s_all = __builtin_fmaf(s_no, t_all, e_y);
         if constexpr (WantLoss) {
-            const float lse_no = fast_log(s_no);
-            const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));   // channels that are not the target
-            const float margin = sum_et * inv_no - lse_no - p.coeff * (sum_t - others * lse_no);
+            const float lse_no = (__builtin_amdgcn_logf(s_no) - r) * kLn2;
+            const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));        // channels that are not the target
+            const float sum_t = (sx - ((tgt < 0) ? 0.f : x_y)) - others * m_no;
+            const float margin = sum_qt - lse_no - p.coeff * (sum_t - others * lse_no);
             const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
             mine += out[k];
             cnt += (ign || !live) ? 0 : 1;
         }
         if constexpr (WantGrad) {
-            const float inv_all = 1.f / s_all;
-            // sum_k q_k x_k = (sum e t)/s_no + m_no
-            const float sum_qx = sum_et * inv_no + m_no;
-            const float gk = ign ? 0.f : go[k];
-            const float p_scale = t_all * inv_all;
-            const float g_hot = (e_y * inv_all - 1.f) * gk;
+            // g_j = gk * (p_j + h * ((x_j + 1 - sum_qx) * q_j - coeff))
+            //     = e_j * (x_j * B + A) - K  with  B = h gk / s_no,  A = gk * t_all / s_all + B * (1 - sum_qx),
+            //       K = h gk coeff; the target channel takes g_y = gk * (p_y - 1) instead.
+            const float inv_all = __builtin_amdgcn_rcpf(s_all);
+            const float sum_qx = sum_qt + m_no;
+            const float gk = go[k];
+            float B = p.half_lam * gk * inv_no;
+            float A = __builtin_fmaf(B, 1.f - sum_qx, gk * t_all * inv_all);
+            float nK = -p.half_lam * gk * p.coeff;
+            float g_hot = (e_y * inv_all - 1.f) * gk;
+            asm("" : "+v"(A), "+v"(B), "+v"(nK), "+v"(g_hot));                  // formed per pixel, not per channel
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (j < p.C) {
-                    const float q = e[j] * inv_no;
-                    const float g_cold = e[j] * p_scale + p.half_lam * ((v[j][k] + 1.f - sum_qx) * q - p.coeff);
-                    const float g = (tgt == j) ? g_hot : g_cold * gk;
-                    v[j][k] = ign ? 0.f : g;      // exact zero even for non-finite logits
+                if (chan_ok<CP>(j, p.C)) {
+                    const float w = __builtin_fmaf(Pack<T, V>::get(raw[j], k), B, A);
+                    const float gj = __builtin_fmaf(xv[j], w, nK);
+                    g[j][k] = (tgt == j) ? g_hot : gj;
                 }
         }
         if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
@@ -114,9 +139,12 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     if (live) {
         if (WantLoss && loss) store_vec<V>(loss + pix, out);
         if constexpr (WantGrad) {
+            // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
+            const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
+                if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(g[j]) & mask;
+            at.store_slice(grad, p.C, p.m_size, raw);
         }
     }
     if constexpr (WantCount) {
@@ -237,14 +265,19 @@ template <class T, int V, bool WantLoss, bool WantGrad, bool WantCount, bool Red
 static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                             unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
-    const bool uni = tiles_are_uniform(p.m_size, V);
+    const bool uni = tiles_are_uniform(p.m_size, V, sizeof(T));
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
-        if (uni) hipLaunchKernelGGL((lm_regs<T, 4 * K, V, true, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
-                                    dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                  \
-        else hipLaunchKernelGGL((lm_regs<T, 4 * K, V, false, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),    \
-                                dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                      \
+        if constexpr (V * sizeof(T) == 8) {                                                                          \
+            if (uni) {                                                                                               \
+                hipLaunchKernelGGL((lm_regs<T, 4 * K, V, true, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),  \
+                                   dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                   \
+                break;                                                                                               \
+            }                                                                                                        \
+        }                                                                                                            \
+        hipLaunchKernelGGL((lm_regs<T, 4 * K, V, false, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),         \
+                           dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                           \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

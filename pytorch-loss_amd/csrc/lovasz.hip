@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict_
     float v[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < C) load_vec<V>(xs + (int64_t)j * m_size, v[j]);
+        if (chan_ok<CP>(j, C)) load_vec<V>(xs + (int64_t)j * m_size, v[j]);
     int64_t lb[V];
     load_labels<V>(lab + pix, lb);
 #pragma unroll
@@ -71,22 +71,22 @@ __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict_
         float mx = v[0][k];
 #pragma unroll
         for (int j = 1; j < CP; ++j)
-            if (j < C) mx = fmaxf(mx, v[j][k]);
+            if (chan_ok<CP>(j, C)) mx = fmaxf(mx, v[j][k]);
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < C) {
+            if (chan_ok<CP>(j, C)) {
                 v[j][k] = expf(v[j][k] - mx);
                 s += v[j][k];
             }
         const bool ign = (lb[k] == ignore);
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < C) v[j][k] = __builtin_bit_cast(float, make_key(v[j][k] / s, lb[k] == j, ign));
+            if (chan_ok<CP>(j, C)) v[j][k] = __builtin_bit_cast(float, make_key(v[j][k] / s, lb[k] == j, ign));
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < C) store_vec<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
+        if (chan_ok<CP>(j, C)) store_vec<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
 }
 
 // Any channel count: a lane per pixel, three sweeps over the slice (the later ones hit cache).
@@ -575,7 +575,7 @@ __global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restri
     float v[CP][V], d[CP][V];
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < C) {
+        if (chan_ok<CP>(j, C)) {
             load_vec<V>(x + base + (int64_t)j * m_size, v[j]);
             load_vec<V>(jacc + (int64_t)j * P + pix, d[j]);
         }
@@ -586,18 +586,18 @@ __global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restri
         float mx = v[0][k];
 #pragma unroll
         for (int j = 1; j < CP; ++j)
-            if (j < C) mx = fmaxf(mx, v[j][k]);
+            if (chan_ok<CP>(j, C)) mx = fmaxf(mx, v[j][k]);
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < C) {
+            if (chan_ok<CP>(j, C)) {
                 v[j][k] = expf(v[j][k] - mx);
                 s += v[j][k];
             }
         float dot = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < C) {
+            if (chan_ok<CP>(j, C)) {
                 v[j][k] = v[j][k] / s;
                 const float dj = d[j][k] * gout[j];
                 d[j][k] = (lb[k] == j) ? -dj : dj;
@@ -606,11 +606,11 @@ __global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restri
         const bool ign = (lb[k] == ignore);
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < C) v[j][k] = ign ? 0.f : v[j][k] * (d[j][k] - dot);
+            if (chan_ok<CP>(j, C)) v[j][k] = ign ? 0.f : v[j][k] * (d[j][k] - dot);
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < C) store_vec<V>(grad + base + (int64_t)j * m_size, v[j]);
+        if (chan_ok<CP>(j, C)) store_vec<V>(grad + base + (int64_t)j * m_size, v[j]);
 }
 
 template <class T>

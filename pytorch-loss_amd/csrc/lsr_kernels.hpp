@@ -27,9 +27,12 @@ struct LsrParams {
 
 // ---------------------------------------------------------------- regs ----
 
-// loss = -sum_j w_j logp_j with logp_j = t_j - lse, t_j = x_j - max:
-//      = -( w_neg * (sum_j t_j - C*lse) + (w_pos - w_neg) * (t_y - lse) )
-// so one pass over the slice gathers max-shifted sum, exp-sum and the target's t.
+// loss = -sum_j w_j logp_j with logp_j = (x_j - mx) - lse:
+//      = -( w_neg * (sum_j x_j - C*mx - C*lse) + (w_pos - w_neg) * (x_y - mx - lse) )
+// so one pass over the slice gathers the plain sum, the exp-sum and the target's logit.
+// exp(x - mx) is evaluated as exp2(fma(x, log2e, -c)) with c = fl(mx * log2e); what the rounding
+// of c left out, r = mx*log2e - c (exact, one fma), scales every term by 2^r and is taken back
+// out of log2(sum).
 template <class T, int CP, int V, bool Uniform, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
@@ -39,37 +42,35 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
     if (!Reduce && !at.live) return;
 
-    float v[CP][V];
-#pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
     load_labels<V>(lab + at.pix, lb);
 
     float out[V];
     float mine = 0.f;
     int cnt = 0;
+    const float fc = (float)p.C;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
         const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        float mx = v[0][k];
-#pragma unroll
-        for (int j = 1; j < CP; ++j)
-            if (j < p.C) mx = fmaxf(mx, v[j][k]);
-        float s = 0.f, sum_t = 0.f, t_y = 0.f;
+        float xv[CP];
+        const float mx = widen_and_max<T, V, CP>(raw, k, p.C, xv);
+        const float c = mx * kLog2e;
+        const float r = __builtin_fmaf(mx, kLog2e, -c);
+        float s = 0.f, sx = 0.f, x_y = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const float t = v[j][k] - mx;
-                s += fast_exp(t);
-                sum_t += t;
-                t_y = (tgt == j) ? t : t_y;
+            if (chan_ok<CP>(j, p.C)) {
+                s += __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
+                sx += xv[j];
+                x_y = (tgt == j) ? xv[j] : x_y;
             }
-        const float lse = fast_log(s);
-        const float all = sum_t - (float)p.C * lse;
+        const float lse = (__builtin_amdgcn_logf(s) - r) * kLn2;
+        const float all = (sx - fc * mx) - fc * lse;
         // no target channel (label outside [0, C)): every weight is w_neg
-        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * (t_y - lse) : 0.f;
+        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - mx) - lse) : 0.f;
         const float acc = -(p.w_neg * all + hot);
         const bool valid = at.live && !ign;
         out[k] = valid ? acc : 0.f;
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     if (at.live && loss) store_vec<V>(loss + at.pix, out);
     if constexpr (Reduce) {
         const float bs = block_sum_256(mine, red);
-        const float bc = block_sum_256((float)cnt, red);   // at most 512 per block: exact in fp32
+        const float bc = block_sum_256((float)cnt, red);   // at most 1024 per block: exact in fp32
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = bs;
             part.cnt[blockIdx.x] = (int)bc;
@@ -95,43 +96,44 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
     const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
     if (!at.live) return;
 
-    float v[CP][V];
-#pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (j < p.C) load_vec<V>(at.chan(x, j, p.m_size), v[j]);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
     load_labels<V>(lab + at.pix, lb);
     float go[V];
     load_upstream<V>(up, at.pix, go);
 
+    float g[CP][V];
+    unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
 #pragma unroll
     for (int k = 0; k < V; ++k) {
-        float mx = v[0][k];
-#pragma unroll
-        for (int j = 1; j < CP; ++j)
-            if (j < p.C) mx = fmaxf(mx, v[j][k]);
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        keep[k] = ign ? 0u : 0xFFFFFFFFu;
+        float xv[CP];
+        const float mx = widen_and_max<T, V, CP>(raw, k, p.C, xv);
+        const float c = mx * kLog2e;
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                v[j][k] = fast_exp(v[j][k] - mx);
-                s += v[j][k];
+            if (chan_ok<CP>(j, p.C)) {
+                xv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
+                s += xv[j];
             }
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
         const float gk = go[k];
-        const float scale = p.sumw * gk / s;          // one division per pixel
-        const float g_pos = p.w_pos * gk, g_neg = p.w_neg * gk;
+        const float scale = p.sumw * gk * __builtin_amdgcn_rcpf(s);     // one reciprocal per pixel
+        float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+        asm("" : "+v"(n_pos), "+v"(n_neg));                             // formed per pixel, not per channel
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (j < p.C) {
-                const float g = v[j][k] * scale - ((tgt == j) ? g_pos : g_neg);
-                v[j][k] = ign ? 0.f : g;              // exact zero even for non-finite logits
-            }
+            if (chan_ok<CP>(j, p.C)) g[j][k] = __builtin_fmaf(xv[j], scale, (tgt == j) ? n_pos : n_neg);
     }
+    // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
+    const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (j < p.C) store_vec<V>(at.chan(grad, j, p.m_size), v[j]);
+        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(g[j]) & mask;
+    at.store_slice(grad, p.C, p.m_size, raw);
 }
 
 // --------------------------------------------------------------- group ----
@@ -271,14 +273,19 @@ template <class T, int V, bool Reduce>
 static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                 hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
-    const bool uni = tiles_are_uniform(p.m_size, V);
+    const bool uni = tiles_are_uniform(p.m_size, V, sizeof(T));
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                               \
     case K:                                                                                                       \
-        if (uni) hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, true, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
-                                    st, x, lab, loss, part, p);                                                   \
-        else hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, false, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st,  \
-                                x, lab, loss, part, p);                                                           \
+        if constexpr (V * sizeof(T) == 8) {                                                                       \
+            if (uni) {                                                                                            \
+                hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, true, Reduce>), dim3(grid), dim3(kRegsBlock), 0,    \
+                                   st, x, lab, loss, part, p);                                                    \
+                break;                                                                                            \
+            }                                                                                                     \
+        }                                                                                                         \
+        hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, false, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
+                           lab, loss, part, p);                                                                   \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -290,14 +297,19 @@ template <class T, int V>
 static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
                             hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
-    const bool uni = tiles_are_uniform(p.m_size, V);
+    const bool uni = tiles_are_uniform(p.m_size, V, sizeof(T));
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                              \
     case K:                                                                                                      \
-        if (uni) hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                                    lab, up, grad, p);                                                           \
-        else hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, false>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, \
-                                up, grad, p);                                                                    \
+        if constexpr (V * sizeof(T) == 8) {                                                                      \
+            if (uni) {                                                                                           \
+                hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
+                                   lab, up, grad, p);                                                            \
+                break;                                                                                           \
+            }                                                                                                    \
+        }                                                                                                        \
+        hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, false>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up,  \
+                           grad, p);                                                                             \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

@@ -205,6 +205,124 @@ __device__ __forceinline__ void load_labels(const int64_t *p, int64_t (&out)[V])
     }
 }
 
+// ---- packed register form of a channel slice -------------------------------------
+// The regs kernels keep what they loaded in the registers it arrived in (two dwords per channel
+// for V = ElemTraits<T>::kVec pixels, one for V = 1) and widen to fp32 at the point of use, so a
+// 16-bit slice costs half the registers of an fp32 one and the wavefront count per SIMD stays
+// the same for every element type.
+typedef unsigned plh_u2 __attribute__((ext_vector_type(2)));
+typedef float plh_bf_src __attribute__((ext_vector_type(2)));
+typedef __bf16 plh_bf2 __attribute__((ext_vector_type(2)));
+typedef _Float16 plh_hf2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ unsigned f32_bits(float v) { return __builtin_bit_cast(unsigned, v); }
+__device__ __forceinline__ float bits_f32(unsigned v) { return __builtin_bit_cast(float, v); }
+
+template <class T, int V> struct Pack;
+
+template <> struct Pack<float, 2> {
+    typedef plh_u2 Raw;
+    static __device__ __forceinline__ Raw load(const float *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const plh_u2 *>(p));
+    }
+    static __device__ __forceinline__ void store(float *p, Raw r) {
+        __builtin_nontemporal_store(r, reinterpret_cast<plh_u2 *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int k) { return bits_f32(k == 0 ? r.x : r.y); }
+    static __device__ __forceinline__ Raw put(const float (&g)[2]) { return Raw{f32_bits(g[0]), f32_bits(g[1])}; }
+    // AND-mask that clears pixel k of a packed gradient when keep[k] is 0 (keep[k] is 0 or ~0)
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[2]) { return Raw{keep[0], keep[1]}; }
+};
+template <> struct Pack<float, 1> {
+    typedef unsigned Raw;
+    static __device__ __forceinline__ Raw load(const float *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const unsigned *>(p));
+    }
+    static __device__ __forceinline__ void store(float *p, Raw r) {
+        __builtin_nontemporal_store(r, reinterpret_cast<unsigned *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int) { return bits_f32(r); }
+    static __device__ __forceinline__ Raw put(const float (&g)[1]) { return f32_bits(g[0]); }
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[1]) { return keep[0]; }
+};
+
+// fp32 -> 16-bit pairs, round to nearest even. bf16 uses the hardware v_cvt_pk_bf16_f32 of gfx950.
+__device__ __forceinline__ unsigned narrow2(float a, float b, bf16) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(plh_bf_src{a, b}, plh_bf2));
+}
+__device__ __forceinline__ unsigned narrow2(float a, float b, f16) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(plh_bf_src{a, b}, plh_hf2));
+}
+__device__ __forceinline__ float widen_lo(unsigned d, bf16) { return bits_f32(d << 16); }
+__device__ __forceinline__ float widen_hi(unsigned d, bf16) { return bits_f32(d & 0xFFFF0000u); }
+__device__ __forceinline__ float widen_lo(unsigned d, f16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)d); }
+__device__ __forceinline__ float widen_hi(unsigned d, f16) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(d >> 16));
+}
+
+template <class T> struct Pack<T, 4> {          // T = f16 or bf16
+    typedef plh_u2 Raw;
+    static __device__ __forceinline__ Raw load(const T *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const plh_u2 *>(p));
+    }
+    static __device__ __forceinline__ void store(T *p, Raw r) {
+        __builtin_nontemporal_store(r, reinterpret_cast<plh_u2 *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int k) {
+        const unsigned d = k < 2 ? r.x : r.y;
+        return (k & 1) ? widen_hi(d, T{}) : widen_lo(d, T{});
+    }
+    static __device__ __forceinline__ Raw put(const float (&g)[4]) {
+        return Raw{narrow2(g[0], g[1], T{}), narrow2(g[2], g[3], T{})};
+    }
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[4]) {
+        return Raw{(keep[0] & 0xFFFFu) | (keep[1] & 0xFFFF0000u), (keep[2] & 0xFFFFu) | (keep[3] & 0xFFFF0000u)};
+    }
+};
+template <class T> struct Pack<T, 1> {          // T = f16 or bf16
+    typedef unsigned Raw;
+    static __device__ __forceinline__ Raw load(const T *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const unsigned short *>(p));
+    }
+    static __device__ __forceinline__ void store(T *p, Raw r) {
+        __builtin_nontemporal_store((unsigned short)r, reinterpret_cast<unsigned short *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int) { return widen_lo(r, T{}); }
+    static __device__ __forceinline__ Raw put(const float (&g)[1]) { return narrow2(g[0], 0.f, T{}) & 0xFFFFu; }
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[1]) { return keep[0]; }
+};
+
+// A regs kernel is instantiated for CP = channels rounded up to a multiple of 4, and launched only
+// for CP-3 <= C <= CP: the first CP-3 channel slots always exist, the last three are checked.
+template <int CP>
+__device__ __forceinline__ bool chan_ok(int j, int C) { return j < CP - 3 || j < C; }
+
+// max(a, b, c) in one instruction. Like fmaxf it returns the largest non-NaN operand; a NaN logit
+// still reaches the result through the exponential sum.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Widens pixel k of a packed slice into xv[] and returns the maximum over its channels.
+template <class T, int V, int CP>
+__device__ __forceinline__ float widen_and_max(const typename Pack<T, V>::Raw (&raw)[CP], int k, int C, float (&xv)[CP]) {
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, C)) xv[j] = Pack<T, V>::get(raw[j], k);
+    float mx = xv[0];
+#pragma unroll
+    for (int j = 1; j + 1 < CP - 3; j += 2) mx = max3(mx, xv[j], xv[j + 1]);
+#pragma unroll
+    for (int j = CP - 3; j < CP; ++j)
+        if (j > 0 && j < C) mx = max3(mx, xv[j], xv[j]);
+    return mx;
+}
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kLn2 = 0.69314718055994530942f;
+
 // Upstream gradient of the fused entry points: value = gout[...] * scale / divide_by[0].
 struct Upstream {
     const float *gout;          // nullptr = 1
@@ -277,6 +395,12 @@ __device__ __forceinline__ int64_t tile_of_block() {
     return b;   // ragged tail of the grid keeps its natural order
 }
 
+// Raw buffer descriptor over [p, p + 4 GiB): no stride, no swizzle, 32-bit data format.
+constexpr int kBufferNT = 2;      // non-temporal hint of buffer loads / stores
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const void *p) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, -1, 0x00020000);
+}
+
 template <int V>
 inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(pixels, V), kRegsBlock); }
 
@@ -316,9 +440,51 @@ struct PixelRef {
     __device__ __forceinline__ T *chan(T *t, int j, int64_t m_size) const {
         return (t + (base + (int64_t)j * m_size)) + lane_off;
     }
+
+    // The channel slice of this thread's pixels, as loaded. The Uniform form addresses through a
+    // buffer descriptor that starts at the tile (scalar registers), a per-lane byte offset that is
+    // the same for every channel and a scalar channel offset: no vector ALU work per load or store.
+    template <class T, int CP>
+    __device__ __forceinline__ void load_slice(const T *t, int C, int64_t m_size,
+                                               typename Pack<T, V>::Raw (&raw)[CP]) const {
+        if constexpr (Uniform) {
+            static_assert(V * sizeof(T) == 8, "uniform tiles move 8 bytes per lane and channel");
+            const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(t + base);
+            const unsigned row = (unsigned)m_size * (unsigned)sizeof(T);
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, C))
+                    raw[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off * (unsigned)sizeof(T), j * row, kBufferNT);
+        } else {
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, C)) raw[j] = Pack<T, V>::load(chan(t, j, m_size));
+        }
+    }
+    template <class T, int CP>
+    __device__ __forceinline__ void store_slice(T *t, int C, int64_t m_size,
+                                                const typename Pack<T, V>::Raw (&raw)[CP]) const {
+        if constexpr (Uniform) {
+            const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(t + base);
+            const unsigned row = (unsigned)m_size * (unsigned)sizeof(T);
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, C))
+                    __builtin_amdgcn_raw_buffer_store_b64(raw[j], rsrc, lane_off * (unsigned)sizeof(T), j * row, kBufferNT);
+        } else {
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, C)) Pack<T, V>::store(chan(t, j, m_size), raw[j]);
+        }
+    }
 };
 
-inline bool tiles_are_uniform(int64_t m_size, int V) { return m_size % ((int64_t)kRegsBlock * V) == 0; }
+// Uniform tiles: m_size is a multiple of the tile, and the byte offset of the last channel slot
+// inside one image (what the scalar channel offset of the buffer form has to hold) fits 31 bits.
+inline bool tiles_are_uniform(int64_t m_size, int V, size_t elem) {
+    return m_size % ((int64_t)kRegsBlock * V) == 0 && V * elem == 8 &&
+           m_size * (int64_t)elem * kMaxRegsChannels < ((int64_t)1 << 31);
+}
 
 __device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.69314718055994530942f; }
 
@@ -331,7 +497,9 @@ __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp
 // (ignored pixel, or a label outside [0, C), which the reference leaves undefined).
 __device__ __forceinline__ int narrow_label(int64_t lb, int64_t ignore, int C, bool &ignored) {
     ignored = (lb == ignore);
-    return (!ignored && lb >= 0 && lb < (int64_t)C) ? (int)lb : -1;
+    int tgt = (!ignored && lb >= 0 && lb < (int64_t)C) ? (int)lb : -1;
+    asm("" : "+v"(tgt));      // opaque from here on: keeps the per-channel compares 32 bits wide
+    return tgt;
 }
 
 // log(1 + e) for e in [0, 1]: alternating series below 1/32 (relative error < 2e-7), hardware
