@@ -79,12 +79,35 @@ def _check(rc):
         raise RuntimeError("pytorch_loss HIP library: %s (code %d)" % (load().plh_error_string(rc).decode(), rc))
 
 
-def _stream():
-    return _p(torch.cuda.current_stream().cuda_stream)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream(device=None):
+    """The current HIP stream of `device` (default: the current device) as a pointer argument."""
+    if _raw_stream is not None:
+        return _p(_raw_stream(torch.cuda.current_device() if device is None or device.index is None
+                              else device.index))
+    if device is None:
+        return _p(torch.cuda.current_stream().cuda_stream)
+    return _p(torch.cuda.current_stream(device).cuda_stream)
 
 
 def _ptr(t):
     return _p(t.data_ptr()) if t is not None else _p(0)
+
+
+def _call(x, entry, *args):
+    """Run library function `entry` with `x`'s device current (the library launches on whatever
+    device is current) and on that device's current stream, appended as the last argument."""
+    fn = getattr(load(), entry)
+    dev = x.device
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        rc = fn(*args, _stream(dev))
+    else:
+        with torch.cuda.device(dev):
+            rc = fn(*args, _stream(dev))
+    if rc != 0:
+        _check(rc)
 
 
 def _require_gpu(what, *tensors):
@@ -115,10 +138,10 @@ def _logits(t):
     return t.contiguous(), _DTYPE_TAGS[t.dtype]
 
 
-def _loss_dtype(logits):
-    """dtype of the returned losses: the logits' own, except under autocast, where the reference's
-    custom_fwd(cast_inputs=float32) makes the whole op fp32."""
-    return torch.float32 if torch.is_autocast_enabled("cuda") else logits.dtype
+def _loss_dtype(dtype):
+    """dtype of the returned losses for logits of `dtype`: the same, except under autocast, where
+    the reference's custom_fwd(cast_inputs=float32) makes the whole op fp32."""
+    return torch.float32 if torch.is_autocast_enabled("cuda") else dtype
 
 
 def _labels_i64(labels, logits, what):
@@ -165,34 +188,39 @@ def _back_to(t, dtype):
 # LSR and large-margin share their marshalling: `entry` names the library function, `param` is the
 # smoothing factor or the margin weight.
 
-def _pixel_forward(entry, what, logits, labels, ignore_index, param):
+class SegArgs:
+    """Checked and marshalled (logits, labels) of a channel-dim loss: computed once in forward and
+    handed to backward, which works on the same tensors."""
+    __slots__ = ("x", "tag", "lb", "n", "c", "m", "dtype")
+
+
+def seg_args(logits, labels, what, entry):
     _require_gpu(what, logits, labels)
-    n, c, m = _dims(logits, entry)
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, entry)
-    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
-    if x.numel() == 0:
-        return _back_to(losses.zero_(), _loss_dtype(logits))
-    with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(losses), n, c, m, int(ignore_index), float(param),
-                                      _stream()))
-    return _back_to(losses, _loss_dtype(logits))
+    a = SegArgs()
+    a.n, a.c, a.m = _dims(logits, entry)
+    a.x, a.tag = _logits(logits)
+    a.lb = _labels_i64(labels, logits, entry)
+    a.dtype = logits.dtype
+    return a
 
 
-def _pixel_backward(entry, what, logits, labels, ignore_index, param, grad_output):
+def _pixel_forward(entry, a, ignore_index, param):
+    losses = torch.empty(a.lb.shape, dtype=torch.float32, device=a.x.device)
+    if a.x.numel() == 0:
+        return _back_to(losses.zero_(), _loss_dtype(a.dtype))
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), a.n, a.c, a.m, int(ignore_index), float(param))
+    return _back_to(losses, _loss_dtype(a.dtype))
+
+
+def _pixel_backward(entry, a, ignore_index, param, grad_output):
     """dloss/dlogits, already multiplied by ``grad_output`` (None = unit upstream gradient)."""
-    _require_gpu(what, logits, labels)
-    n, c, m = _dims(logits, entry)
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, entry)
-    grad = torch.empty_like(x)
-    if x.numel() == 0:
-        return _back_to(grad, logits.dtype)
-    go, stride = _upstream(grad_output, lb.shape)
-    with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(go), stride, _ptr(grad), n, c, m,
-                                      int(ignore_index), float(param), _stream()))
-    return _back_to(grad, logits.dtype)
+    grad = torch.empty_like(a.x)
+    if a.x.numel() == 0:
+        return _back_to(grad, a.dtype)
+    go, stride = _upstream(grad_output, a.lb.shape)
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(go), stride, _ptr(grad), a.n, a.c, a.m,
+          int(ignore_index), float(param))
+    return _back_to(grad, a.dtype)
 
 
 def _reduce_workspace(units, device):
@@ -204,214 +232,205 @@ def _reduce_workspace(units, device):
 
 def _scalar_f32(t):
     """A 0-dim upstream gradient as one fp32 value in device memory."""
+    if t.dtype == torch.float32 and t.numel() == 1:
+        return t
     t = t.reshape(-1)[:1]
-    return t if (t.dtype == torch.float32 and t.is_contiguous()) else t.float().contiguous()
+    return t if t.dtype == torch.float32 else t.float()
 
 
-def _pixel_forward_reduced(entry, what, logits, labels, ignore_index, param, mean):
+def _pixel_forward_reduced(entry, a, ignore_index, param, mean):
     """-> (loss 0-dim, n_valid 0-dim int64)."""
-    _require_gpu(what, logits, labels)
-    n, c, m = _dims(logits, entry)
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, entry)
-    loss = torch.empty((), dtype=torch.float32, device=x.device)
-    n_valid = torch.empty((), dtype=torch.int64, device=x.device)
-    ws, ws_bytes = _reduce_workspace(n * m, x.device)
-    with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), None, _ptr(loss), _ptr(n_valid), 1 if mean else 0,
-                                      _ptr(ws), ws_bytes, n, c, m, int(ignore_index), float(param), _stream()))
-    return _back_to(loss, _loss_dtype(logits)), n_valid
+    loss = torch.empty((), dtype=torch.float32, device=a.x.device)
+    n_valid = torch.empty((), dtype=torch.int64, device=a.x.device)
+    ws, ws_bytes = _reduce_workspace(a.n * a.m, a.x.device)
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), None, _ptr(loss), _ptr(n_valid), 1 if mean else 0,
+          _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(param))
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid
 
 
-def _pixel_backward_scaled(entry, what, logits, labels, ignore_index, param, grad_scalar, divide_by):
-    _require_gpu(what, logits, labels)
-    n, c, m = _dims(logits, entry)
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, entry)
-    grad = torch.empty_like(x)
-    if x.numel() == 0:
-        return _back_to(grad, logits.dtype)
+def _pixel_backward_scaled(entry, a, ignore_index, param, grad_scalar, divide_by):
+    grad = torch.empty_like(a.x)
+    if a.x.numel() == 0:
+        return _back_to(grad, a.dtype)
     go = _scalar_f32(grad_scalar)
-    with torch.cuda.device_of(x):
-        _check(getattr(load(), entry)(_ptr(x), tag, _ptr(lb), _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), n, c, m,
-                                      int(ignore_index), float(param), _stream()))
-    return _back_to(grad, logits.dtype)
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), a.n, a.c, a.m,
+          int(ignore_index), float(param))
+    return _back_to(grad, a.dtype)
 
 
-def lsr_forward(logits, labels, ignore_index, smooth):
-    return _pixel_forward("plh_lsr_forward", "LSR loss", logits, labels, ignore_index, smooth)
+def lsr_args(logits, labels):
+    return seg_args(logits, labels, "LSR loss", "lsr")
 
 
-def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None):
-    return _pixel_backward("plh_lsr_backward", "LSR loss", logits, labels, ignore_index, smooth, grad_output)
+def lsr_forward(logits, labels, ignore_index, smooth, args=None):
+    return _pixel_forward("plh_lsr_forward", args or lsr_args(logits, labels), ignore_index, smooth)
 
 
-def lsr_forward_reduced(logits, labels, ignore_index, smooth, mean):
-    return _pixel_forward_reduced("plh_lsr_forward_reduced", "LSR loss", logits, labels, ignore_index, smooth, mean)
+def lsr_backward(logits, labels, ignore_index, smooth, grad_output=None, args=None):
+    return _pixel_backward("plh_lsr_backward", args or lsr_args(logits, labels), ignore_index, smooth, grad_output)
 
 
-def lsr_backward_scaled(logits, labels, ignore_index, smooth, grad_scalar, divide_by=None):
-    return _pixel_backward_scaled("plh_lsr_backward_scaled", "LSR loss", logits, labels, ignore_index, smooth,
+def lsr_forward_reduced(logits, labels, ignore_index, smooth, mean, args=None):
+    return _pixel_forward_reduced("plh_lsr_forward_reduced", args or lsr_args(logits, labels), ignore_index, smooth,
+                                  mean)
+
+
+def lsr_backward_scaled(logits, labels, ignore_index, smooth, grad_scalar, divide_by=None, args=None):
+    return _pixel_backward_scaled("plh_lsr_backward_scaled", args or lsr_args(logits, labels), ignore_index, smooth,
                                   grad_scalar, divide_by)
 
 
 # -------------------------------------------------------------- lmargin ----
 
-def lmargin_forward(logits, labels, lam, ignore_index):
-    return _pixel_forward("plh_lmargin_forward", "large margin loss", logits, labels, ignore_index, lam)
+def lmargin_args(logits, labels):
+    return seg_args(logits, labels, "large margin loss", "l_margin")
 
 
-def lmargin_backward(logits, labels, lam, ignore_index, grad_output=None):
-    return _pixel_backward("plh_lmargin_backward", "large margin loss", logits, labels, ignore_index, lam,
+def lmargin_forward(logits, labels, lam, ignore_index, args=None):
+    return _pixel_forward("plh_lmargin_forward", args or lmargin_args(logits, labels), ignore_index, lam)
+
+
+def lmargin_backward(logits, labels, lam, ignore_index, grad_output=None, args=None):
+    return _pixel_backward("plh_lmargin_backward", args or lmargin_args(logits, labels), ignore_index, lam,
                            grad_output)
 
 
-def lmargin_forward_reduced(logits, labels, lam, ignore_index, mean):
-    return _pixel_forward_reduced("plh_lmargin_forward_reduced", "large margin loss", logits, labels, ignore_index,
+def lmargin_forward_reduced(logits, labels, lam, ignore_index, mean, args=None):
+    return _pixel_forward_reduced("plh_lmargin_forward_reduced", args or lmargin_args(logits, labels), ignore_index,
                                   lam, mean)
 
 
-def lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_scalar, divide_by=None):
-    return _pixel_backward_scaled("plh_lmargin_backward_scaled", "large margin loss", logits, labels, ignore_index,
+def lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_scalar, divide_by=None, args=None):
+    return _pixel_backward_scaled("plh_lmargin_backward_scaled", args or lmargin_args(logits, labels), ignore_index,
                                   lam, grad_scalar, divide_by)
 
 
 def lmargin_forward_backward(logits, labels, lam, ignore_index):
     """-> (losses, grad under unit upstream gradient, valid_cnt int64[1])"""
-    _require_gpu("large margin loss", logits, labels)
-    n, c, m = _dims(logits, "l_margin_forward_backward")
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, "l_margin_forward_backward")
-    losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
-    grad = torch.empty_like(x)
-    cnt = torch.zeros(1, dtype=torch.int64, device=x.device)
-    if x.numel():
-        with torch.cuda.device_of(x):
-            _check(load().plh_lmargin_forward_backward(_ptr(x), tag, _ptr(lb), _ptr(losses), _ptr(grad), _ptr(cnt),
-                                                       n, c, m, int(ignore_index), float(lam), _stream()))
+    a = lmargin_args(logits, labels)
+    losses = torch.empty(a.lb.shape, dtype=torch.float32, device=a.x.device)
+    grad = torch.empty_like(a.x)
+    cnt = torch.zeros(1, dtype=torch.int64, device=a.x.device)
+    if a.x.numel():
+        _call(a.x, "plh_lmargin_forward_backward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), _ptr(grad), _ptr(cnt),
+              a.n, a.c, a.m, int(ignore_index), float(lam))
     else:
         losses.zero_()
-    return _back_to(losses, _loss_dtype(logits)), _back_to(grad, logits.dtype), cnt
+    return _back_to(losses, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), cnt
 
 
 # ---------------------------------------------------------------- focal ----
 
-def _focal_pair(logits, labels, what):
-    """Logits and labels in one dtype the kernels read; mixed or exotic dtypes are computed from fp32 copies."""
+class FocalArgs:
+    """Logits and labels in one dtype the kernels read; mixed or exotic dtypes become fp32 copies."""
+    __slots__ = ("x", "y", "tag", "dtype")
+
+
+def focal_args(logits, labels, what="focalloss"):
     _require_gpu("focal loss", logits, labels)
-    if tuple(labels.shape) != tuple(logits.shape):
+    if labels.shape != logits.shape:
         raise RuntimeError("%s: labels and logits must have the same shape" % what)
+    a = FocalArgs()
+    a.dtype = logits.dtype
     if logits.dtype == labels.dtype and logits.dtype in _DTYPE_TAGS:
-        return logits.contiguous(), labels.contiguous(), _DTYPE_TAGS[logits.dtype]
-    return _f32c(logits), _f32c(labels), 0
+        a.x, a.y, a.tag = logits.contiguous(), labels.contiguous(), _DTYPE_TAGS[logits.dtype]
+    else:
+        a.x, a.y, a.tag = _f32c(logits), _f32c(labels), 0
+    return a
 
 
-def focal_forward(logits, labels, gamma, alpha):
-    x, y, tag = _focal_pair(logits, labels, "focalloss_forward")
-    losses = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-    if x.numel():
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_forward(_ptr(x), tag, _ptr(y), _ptr(losses), x.numel(),
-                                            float(gamma), float(alpha), _stream()))
-    return _back_to(losses, _loss_dtype(logits))
+def focal_forward(logits, labels, gamma, alpha, args=None):
+    a = args or focal_args(logits, labels, "focalloss_forward")
+    losses = torch.empty(a.x.shape, dtype=torch.float32, device=a.x.device)
+    if a.x.numel():
+        _call(a.x, "plh_focal_forward", _ptr(a.x), a.tag, _ptr(a.y), _ptr(losses), a.x.numel(), float(gamma),
+              float(alpha))
+    return _back_to(losses, _loss_dtype(a.dtype))
 
 
-def focal_backward(logits, labels, gamma, alpha, grad_output=None):
-    x, y, tag = _focal_pair(logits, labels, "focalloss_backward")
-    grad = torch.empty_like(x)
-    if x.numel():
-        go, stride = _upstream(grad_output, x.shape)
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_backward(_ptr(x), tag, _ptr(y), _ptr(go), stride, _ptr(grad), x.numel(),
-                                             float(gamma), float(alpha), _stream()))
-    return _back_to(grad, logits.dtype)
+def focal_backward(logits, labels, gamma, alpha, grad_output=None, args=None):
+    a = args or focal_args(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(a.x)
+    if a.x.numel():
+        go, stride = _upstream(grad_output, a.x.shape)
+        _call(a.x, "plh_focal_backward", _ptr(a.x), a.tag, _ptr(a.y), _ptr(go), stride, _ptr(grad), a.x.numel(),
+              float(gamma), float(alpha))
+    return _back_to(grad, a.dtype)
 
 
 def focal_forward_backward(logits, labels, gamma, alpha):
-    x, y, tag = _focal_pair(logits, labels, "focalloss_forward_backward")
-    losses = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-    grad = torch.empty_like(x)
-    if x.numel():
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_forward_backward(_ptr(x), tag, _ptr(y), _ptr(losses), _ptr(grad), x.numel(),
-                                                     float(gamma), float(alpha), _stream()))
-    return _back_to(losses, _loss_dtype(logits)), _back_to(grad, logits.dtype)
+    a = focal_args(logits, labels, "focalloss_forward_backward")
+    losses = torch.empty(a.x.shape, dtype=torch.float32, device=a.x.device)
+    grad = torch.empty_like(a.x)
+    if a.x.numel():
+        _call(a.x, "plh_focal_forward_backward", _ptr(a.x), a.tag, _ptr(a.y), _ptr(losses), _ptr(grad), a.x.numel(),
+              float(gamma), float(alpha))
+    return _back_to(losses, _loss_dtype(a.dtype)), _back_to(grad, a.dtype)
 
 
-def focal_forward_reduced(logits, labels, gamma, alpha, mean):
-    x, y, tag = _focal_pair(logits, labels, "focalloss_forward")
-    loss = torch.empty((), dtype=torch.float32, device=x.device)
-    ws, ws_bytes = _reduce_workspace(x.numel(), x.device)
-    with torch.cuda.device_of(x):
-        _check(load().plh_focal_forward_reduced(_ptr(x), tag, _ptr(y), None, _ptr(loss), 1 if mean else 0, _ptr(ws),
-                                                ws_bytes, x.numel(), float(gamma), float(alpha), _stream()))
-    return _back_to(loss, _loss_dtype(logits))
+def focal_forward_reduced(logits, labels, gamma, alpha, mean, args=None):
+    a = args or focal_args(logits, labels, "focalloss_forward")
+    loss = torch.empty((), dtype=torch.float32, device=a.x.device)
+    ws, ws_bytes = _reduce_workspace(a.x.numel(), a.x.device)
+    _call(a.x, "plh_focal_forward_reduced", _ptr(a.x), a.tag, _ptr(a.y), None, _ptr(loss), 1 if mean else 0, _ptr(ws),
+          ws_bytes, a.x.numel(), float(gamma), float(alpha))
+    return _back_to(loss, _loss_dtype(a.dtype))
 
 
-def focal_backward_scaled(logits, labels, gamma, alpha, grad_scalar, scale):
-    x, y, tag = _focal_pair(logits, labels, "focalloss_backward")
-    grad = torch.empty_like(x)
-    if x.numel():
+def focal_backward_scaled(logits, labels, gamma, alpha, grad_scalar, scale, args=None):
+    a = args or focal_args(logits, labels, "focalloss_backward")
+    grad = torch.empty_like(a.x)
+    if a.x.numel():
         go = _scalar_f32(grad_scalar)
-        with torch.cuda.device_of(x):
-            _check(load().plh_focal_backward_scaled(_ptr(x), tag, _ptr(y), _ptr(go), float(scale), _ptr(grad),
-                                                    x.numel(), float(gamma), float(alpha), _stream()))
-    return _back_to(grad, logits.dtype)
+        _call(a.x, "plh_focal_backward_scaled", _ptr(a.x), a.tag, _ptr(a.y), _ptr(go), float(scale), _ptr(grad),
+              a.x.numel(), float(gamma), float(alpha))
+    return _back_to(grad, a.dtype)
 
 
 # --------------------------------------------------------------- lovasz ----
 
-def _lovasz_limits(logits, what):
+def lovasz_args(logits, labels):
     # same limits and wording as csrc/lovasz_softmax.cu:664-665
     if logits.numel() >= (1 << 31):
-        raise RuntimeError("%s: input tensor too large, int32 type will overflow" % what)
+        raise RuntimeError("lovasz_softmax: input tensor too large, int32 type will overflow")
     if logits.dim() >= 2 and logits.shape[1] >= 512:
-        raise RuntimeError("%s: num of classes should be less than BLOCKSIZE" % what)
+        raise RuntimeError("lovasz_softmax: num of classes should be less than BLOCKSIZE")
+    return seg_args(logits, labels, "lovasz softmax function", "lovasz_softmax")
 
 
-def lovasz_forward(logits, labels, ignore_index):
+def lovasz_forward(logits, labels, ignore_index, args=None):
     """-> (losses[C], jacc[C, N*M] fp32)"""
-    _require_gpu("lovasz softmax function", logits, labels)
-    _lovasz_limits(logits, "lovasz_softmax_forward")
-    n, c, m = _dims(logits, "lovasz_softmax_forward")
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, "lovasz_softmax_forward")
-    losses = torch.empty((c,), dtype=torch.float32, device=x.device)
-    jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
-    if x.numel() == 0:
-        return _back_to(losses.zero_(), _loss_dtype(logits)), jacc
-    lib = load()
-    ws_bytes = int(lib.plh_lovasz_workspace_bytes(n, c, m))
+    a = args or lovasz_args(logits, labels)
+    losses = torch.empty((a.c,), dtype=torch.float32, device=a.x.device)
+    jacc = torch.empty((a.c, a.n * a.m), dtype=torch.float32, device=a.x.device)
+    if a.x.numel() == 0:
+        return _back_to(losses.zero_(), _loss_dtype(a.dtype)), jacc
+    ws_bytes = int(load().plh_lovasz_workspace_bytes(a.n, a.c, a.m))
     if ws_bytes < 0:
         _check(ws_bytes)
-    workspace = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device_of(x):
-        _check(lib.plh_lovasz_forward(_ptr(x), tag, _ptr(lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
-                                      n, c, m, int(ignore_index), _stream()))
-    return _back_to(losses, _loss_dtype(logits)), jacc
+    workspace = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=a.x.device)
+    _call(a.x, "plh_lovasz_forward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
+          a.n, a.c, a.m, int(ignore_index))
+    return _back_to(losses, _loss_dtype(a.dtype)), jacc
 
 
-def lovasz_backward(grad_output, logits, labels, jacc, ignore_index):
-    _require_gpu("lovasz softmax function", logits, labels, grad_output, jacc)
-    n, c, m = _dims(logits, "lovasz_softmax_backward")
-    x, tag = _logits(logits)
-    lb = _labels_i64(labels, logits, "lovasz_softmax_backward")
-    grad = torch.empty_like(x)
-    if x.numel() == 0:
-        return _back_to(grad, logits.dtype)
-    go = _f32c(grad_output.expand((c,)) if grad_output.numel() == 1 else grad_output)
-    if go.numel() != c or jacc.numel() != c * n * m or jacc.dtype != torch.float32:
+def lovasz_backward(grad_output, logits, labels, jacc, ignore_index, args=None):
+    a = args or lovasz_args(logits, labels)
+    _require_gpu("lovasz softmax function", a.x, grad_output, jacc)
+    grad = torch.empty_like(a.x)
+    if a.x.numel() == 0:
+        return _back_to(grad, a.dtype)
+    go = _f32c(grad_output.expand((a.c,)) if grad_output.numel() == 1 else grad_output)
+    if go.numel() != a.c or jacc.numel() != a.c * a.n * a.m or jacc.dtype != torch.float32:
         raise RuntimeError("lovasz_softmax_backward: grad_output must have C elements and jacc C*N*M fp32 elements")
     jc = jacc.contiguous()
-    with torch.cuda.device_of(x):
-        _check(load().plh_lovasz_backward(_ptr(go), _ptr(x), tag, _ptr(lb), _ptr(jc), _ptr(grad), n, c, m,
-                                          int(ignore_index), _stream()))
-    return _back_to(grad, logits.dtype)
+    _call(a.x, "plh_lovasz_backward", _ptr(go), _ptr(a.x), a.tag, _ptr(a.lb), _ptr(jc), _ptr(grad), a.n, a.c, a.m,
+          int(ignore_index))
+    return _back_to(grad, a.dtype)
 
 
 def stream_copy(src, dst):
     _require_gpu("stream copy", src, dst)
     assert src.dtype == torch.float32 and dst.dtype == torch.float32 and src.numel() == dst.numel()
     assert src.is_contiguous() and dst.is_contiguous()
-    with torch.cuda.device_of(src):
-        _check(load().plh_stream_copy(_ptr(src), _ptr(dst), src.numel(), _stream()))
+    _call(src, "plh_stream_copy", _ptr(src), _ptr(dst), src.numel())

@@ -8,7 +8,6 @@ gradient) and the module ``FocalLossV3(alpha, gamma, reduction)``.  Labels are f
 tensors with the logits' shape; soft labels are allowed.
 """
 import torch
-import torch.amp as amp
 import torch.nn as nn
 
 from . import _native
@@ -18,16 +17,15 @@ class FocalSigmoidLossFuncV3(torch.autograd.Function):
     """Recomputes everything from (logits, labels) in backward: nothing but the inputs is kept."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma):
         ctx.variables = (logits, labels, alpha, gamma)
-        return _native.focal_forward(logits, labels, gamma, alpha)
+        ctx.args = args = _native.focal_args(logits, labels)
+        return _native.focal_forward(logits, labels, gamma, alpha, args=args)
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, alpha, gamma = ctx.variables
-        grads = _native.focal_backward(logits, labels, gamma, alpha, grad_output)
+        grads = _native.focal_backward(logits, labels, gamma, alpha, grad_output, args=ctx.args)
         return grads, None, None, None
 
 
@@ -35,14 +33,12 @@ class FocalSigmoidLossFuncV3FB(torch.autograd.Function):
     """Forward computes loss and gradient in one pass and keeps the gradient for backward."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma):
         loss, grads = _native.focal_forward_backward(logits, labels, gamma, alpha)
         ctx.variables = grads
         return loss
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         grads = ctx.variables
         grads.mul_(grad_output)
@@ -54,17 +50,16 @@ class _FocalReducedFunction(torch.autograd.Function):
     fixed-order finish); backward folds the scalar upstream gradient and 1/numel into its kernel."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, alpha, gamma, mean):
         ctx.variables = (logits, labels, alpha, gamma, mean)
-        return _native.focal_forward_reduced(logits, labels, gamma, alpha, mean)
+        ctx.args = args = _native.focal_args(logits, labels)
+        return _native.focal_forward_reduced(logits, labels, gamma, alpha, mean, args=args)
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, alpha, gamma, mean = ctx.variables
         scale = 1.0 / logits.numel() if mean else 1.0
-        grads = _native.focal_backward_scaled(logits, labels, gamma, alpha, grad_output, scale)
+        grads = _native.focal_backward_scaled(logits, labels, gamma, alpha, grad_output, scale, args=ctx.args)
         return grads, None, None, None, None
 
 

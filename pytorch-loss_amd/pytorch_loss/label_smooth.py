@@ -6,7 +6,6 @@ per-pixel losses, ``LabelSmoothSoftmaxCEV3(lb_smooth, reduction, ignore_index)``
 them.  Target weight is ``1 - lb_smooth``, every other class gets ``lb_smooth / C``.
 """
 import torch
-import torch.amp as amp
 import torch.nn as nn
 
 from . import _native
@@ -17,16 +16,15 @@ class LSRCrossEntropyFunctionV3(torch.autograd.Function):
     backward -> d/dlogits, with the upstream gradient folded into the same kernel."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lb_smooth, lb_ignore):
         ctx.variables = (logits, labels, lb_ignore, lb_smooth)
-        return _native.lsr_forward(logits, labels, lb_ignore, lb_smooth)
+        ctx.args = args = _native.lsr_args(logits, labels)
+        return _native.lsr_forward(logits, labels, lb_ignore, lb_smooth, args=args)
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, lb_ignore, lb_smooth = ctx.variables
-        grad = _native.lsr_backward(logits, labels, lb_ignore, lb_smooth, grad_output)
+        grad = _native.lsr_backward(logits, labels, lb_ignore, lb_smooth, grad_output, args=ctx.args)
         return grad, None, None, None
 
 
@@ -37,17 +35,16 @@ class _LSRReducedFunction(torch.autograd.Function):
     upstream gradient and the 1/n_valid of a mean into the gradient kernel."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lb_smooth, lb_ignore, mean):
-        loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean)
+        ctx.args = args = _native.lsr_args(logits, labels)
+        loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean, args=args)
         ctx.variables = (logits, labels, lb_ignore, lb_smooth, n_valid if mean else None)
         return loss
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, lb_ignore, lb_smooth, n_valid = ctx.variables
-        grad = _native.lsr_backward_scaled(logits, labels, lb_ignore, lb_smooth, grad_output, n_valid)
+        grad = _native.lsr_backward_scaled(logits, labels, lb_ignore, lb_smooth, grad_output, n_valid, args=ctx.args)
         return grad, None, None, None, None
 
 

@@ -5,7 +5,6 @@ and the repository root copy large_margin_softmax.py:146-229, which adds the fus
 ``LargeMarginSoftmaxFuncV3FB`` and the module's ``fb`` switch).
 """
 import torch
-import torch.amp as amp
 import torch.nn as nn
 
 from . import _native
@@ -15,16 +14,15 @@ class LargeMarginSoftmaxFuncV3(torch.autograd.Function):
     """forward -> per-pixel losses; backward recomputes from the inputs."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
         ctx.variables = (logits, labels, lam, ignore_index)
-        return _native.lmargin_forward(logits, labels, lam, ignore_index)
+        ctx.args = args = _native.lmargin_args(logits, labels)
+        return _native.lmargin_forward(logits, labels, lam, ignore_index, args=args)
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, lam, ignore_index = ctx.variables
-        grads = _native.lmargin_backward(logits, labels, lam, ignore_index, grad_output)
+        grads = _native.lmargin_backward(logits, labels, lam, ignore_index, grad_output, args=ctx.args)
         return grads, None, None, None
 
 
@@ -33,7 +31,6 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
     kernel and kept for backward."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam=0.3, ignore_index=255):
         losses, grads, valid_cnt = _native.lmargin_forward_backward(logits, labels, lam, ignore_index)
         ctx.variables = grads
@@ -41,7 +38,6 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
         return losses, valid_cnt
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output, grad_cnt):
         grads = ctx.variables
         grads.mul_(grad_output.unsqueeze(1))
@@ -52,17 +48,16 @@ class _LargeMarginReducedFunction(torch.autograd.Function):
     """'sum' / 'mean' produced inside the forward kernel; see label_smooth._LSRReducedFunction."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, lam, ignore_index, mean):
-        loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean)
+        ctx.args = args = _native.lmargin_args(logits, labels)
+        loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean, args=args)
         ctx.variables = (logits, labels, lam, ignore_index, n_valid if mean else None)
         return loss
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, lam, ignore_index, n_valid = ctx.variables
-        grads = _native.lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_output, n_valid)
+        grads = _native.lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_output, n_valid, args=ctx.args)
         return grads, None, None, None, None
 
 

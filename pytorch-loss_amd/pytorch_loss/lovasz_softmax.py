@@ -5,7 +5,6 @@ Same surface as the reference's V3 pair (pytorch_loss/lovasz_softmax.py:75-116):
 class (every class, present in the batch or not), the module reduces over classes.
 """
 import torch
-import torch.amp as amp
 import torch.nn as nn
 
 from . import _native
@@ -15,17 +14,16 @@ class LovaszSoftmaxFunctionV3(torch.autograd.Function):
     """Keeps the Jaccard differences (C x pixels, fp32) between forward and backward."""
 
     @staticmethod
-    @amp.custom_fwd(device_type="cuda")
     def forward(ctx, logits, labels, ignore_index):
-        losses, jacc = _native.lovasz_forward(logits, labels, ignore_index)
+        ctx.args = args = _native.lovasz_args(logits, labels)
+        losses, jacc = _native.lovasz_forward(logits, labels, ignore_index, args=args)
         ctx.vars = (logits, labels, jacc, ignore_index)
         return losses
 
     @staticmethod
-    @amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         logits, labels, jacc, ignore_index = ctx.vars
-        grad = _native.lovasz_backward(grad_output, logits, labels, jacc, ignore_index)
+        grad = _native.lovasz_backward(grad_output, logits, labels, jacc, ignore_index, args=ctx.args)
         return grad, None, None
 
 
