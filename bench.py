@@ -42,6 +42,8 @@ WORKLOADS = {
                   "Bernoulli(0.02) labels, alpha=0.25 gamma=2, mean"),
     "lovasz": dict(shape=(4, 19, 512, 1024), desc="LovaszSoftmaxV3 fwd+bwd, fp32 logits (4,19,512,1024), "
                    "Zipf(1.1) int64 labels 5% ignore=255, mean"),
+    "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
+                 "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }
 
 
@@ -68,6 +70,9 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     E = numel(shape)
     P = E // shape[1]
     b = ELEM_BYTES[dtype]
+    if name == "ohem":     # relabelling (logits + labels read, labels written), then the LSR-shaped loss
+        relabel = b * E + 8 * P + 8 * P
+        return relabel + b * E + 8 * P + 4 * P, b * E + 8 * P + 4 * P + b * E
     if name in ("lsr", "lmargin"):
         fwd = b * E + 8 * P + 4 * P
         bwd = b * E + 8 * P + 4 * P + b * E
@@ -99,7 +104,7 @@ def _make_inputs_f32(name, shape, device, seed):
         logits = torch.randn(shape, device=device, generator=g) * 1.5 - 2.0
         labels = (torch.rand(shape, device=device, generator=g) < 0.02).float()
         return logits, labels
-    logits = torch.randn(shape, device=device, generator=g) * 2.0
+    logits = torch.randn(shape, device=device, generator=g) * (4.0 if name == "ohem" else 2.0)
     lshape = shape[:1] + shape[2:]
     if name == "lovasz":
         p = (torch.arange(19, device=device, dtype=torch.float64) + 1.0) ** -1.1
@@ -121,6 +126,8 @@ def make_criterion(name):
         return pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255)
     if name == "focal":
         return pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean")
+    if name == "ohem":
+        return pl.OhemCELoss(score_thresh=0.7, n_min=None, ignore_index=255)
     return pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255)
 
 
@@ -198,6 +205,21 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
     st = _native._stream
     P = _native._ptr
     out = {}
+    if name == "ohem":
+        # the relabelling entry point alone: logits and labels in, new labels out
+        new_labels = torch.empty_like(labels)
+        scores = torch.empty(labels.numel(), dtype=torch.float32, device=x.device)
+        ws_bytes = int(lib.plh_ohem_workspace_bytes(labels.numel()))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        nbytes = x.element_size() * x.numel() + 16 * labels.numel()
+        f = lambda: lib.plh_ohem_score_label(P(x), tag, P(labels), P(new_labels), P(scores), P(ws), ws_bytes, n, c, m,
+                                             255, 0.7, labels.numel() // 16, st())
+        assert f() == 0
+        ms = time_kernel(f)
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        return {"relabel": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(ms, 4),
+                            "algorithmic_bytes": nbytes}}
     if name in ("lsr", "lmargin"):
         losses = torch.empty(labels.shape, dtype=torch.float32, device=x.device)
         grad = torch.empty_like(x)
@@ -250,14 +272,15 @@ def cpu_baseline(name, shape):
     from oracle import synth, torch_ref
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
-    cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5"}[name]
+    cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2"}[name]
     w = synth.workload(cfg, batch=1)
     logits = torch.from_numpy(w["logits"]).requires_grad_()
     labels = torch.from_numpy(w["labels"])
     fn = {"lsr": lambda: torch_ref.lsr(logits, labels, 0.1, "mean", 255),
           "lmargin": lambda: torch_ref.lmargin(logits, labels, 0.3, "mean", 255),
           "focal": lambda: torch_ref.focal(logits, labels, 0.25, 2, "mean"),
-          "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255)}[name]
+          "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255),
+          "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255)}[name]
     times = []
     for i in range(4):
         logits.grad = None
@@ -361,8 +384,10 @@ def main():
         "config": {"workload": describe(name, args.dtype), "storage_dtype": args.dtype,
                    "algorithmic_bytes_per_step": main_res["bytes"],
                    "frac_of_hbm_peak": round(main_res["gbps"] / HBM_PEAK_GBPS, 4), "loss": main_res["loss"]},
-        "roofline": dict(main_res["roofline"]["backward"], kernel="backward entry point of the workload"),
-        "roofline_forward": main_res["roofline"]["forward"],
+        "roofline": dict(main_res["roofline"].get("backward") or main_res["roofline"]["relabel"],
+                         kernel="backward entry point of the workload" if "backward" in main_res["roofline"]
+                         else "plh_ohem_score_label"),
+        "roofline_forward": main_res["roofline"].get("forward"),
         "step_ms": main_res["step_ms"],
         "copy_kernel_GBps": ceiling,
         "other_workloads": others,

@@ -42,7 +42,7 @@ extern "C" {
 #define PLH_ERR_BAD_SIZE (-2)       /* negative size, or numel beyond the supported range */
 #define PLH_ERR_BAD_STRIDE (-3)     /* grad_output_stride not 0 or 1 */
 #define PLH_ERR_TOO_MANY_CLASSES (-4) /* Lovasz: dimsize >= 512 (csrc/lovasz_softmax.cu:665) */
-#define PLH_ERR_WORKSPACE (-5)      /* workspace smaller than plh_lovasz_workspace_bytes() */
+#define PLH_ERR_WORKSPACE (-5)      /* workspace missing, misaligned or smaller than plh_*_workspace_bytes() */
 #define PLH_ERR_MISALIGNED (-6)     /* a pointer is not aligned to its element size */
 #define PLH_ERR_BAD_DTYPE (-7)      /* dtype is not one of PLH_DTYPE_* */
 
@@ -190,6 +190,36 @@ int plh_lovasz_backward(const float *grad_output, const void *logits, int32_t dt
                         const float *jacc, void *grad_logits,
                         int64_t n_size, int64_t dimsize, int64_t m_size,
                         int64_t ignore_index, void *stream);
+
+/* ---- online hard example mining by score ---------------------------------------------
+ * Replaces ohem_cpp.score_ohem_label (csrc/ohem_label_kernel.cu:171-276), the relabelling step
+ * that pytorch_loss/ohem_loss.py:22-27 and :40-45 run before their loss: with the pixels ordered
+ * by score = softmax(logits)[label] ascending (ignored pixels score 1, ties in pixel order),
+ * every pixel at position >= n_min whose score exceeds score_thresh gets ignore_index as its
+ * label; n_min >= n_size*m_size leaves the labels as they are (:189).
+ *
+ * plh_ohem_scores        scores (n_size*m_size fp32) only               (:112-151)
+ * plh_ohem_select_labels the relabelling for given scores in [0, 1]     (:155-168, :247-262);
+ *                        out_labels may be the labels buffer itself
+ * plh_ohem_score_label   both; `scores` is scratch of n_size*m_size floats
+ * workspace: at least plh_ohem_workspace_bytes(n_size*m_size) bytes, 256-byte aligned, owned by
+ * the caller, contents undefined afterwards. Limit: n_size*m_size <= 2^31 - 1024.
+ */
+int64_t plh_ohem_workspace_bytes(int64_t n_pixels);
+
+int plh_ohem_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores,
+                    int64_t n_size, int64_t dimsize, int64_t m_size,
+                    int64_t ignore_index, void *stream);
+
+int plh_ohem_select_labels(const float *scores, const int64_t *labels, int64_t *out_labels,
+                           void *workspace, int64_t workspace_bytes, int64_t n_pixels,
+                           int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
+
+int plh_ohem_score_label(const void *logits, int32_t dtype, const int64_t *labels,
+                         int64_t *out_labels, float *scores,
+                         void *workspace, int64_t workspace_bytes,
+                         int64_t n_size, int64_t dimsize, int64_t m_size,
+                         int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
 
 /* ---- measurement aid ----------------------------------------------------------------
  * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,

@@ -169,6 +169,38 @@ def lovasz_backward(grad_out, logits, labels, jacc, ignore_index=-100):
     return out
 
 
+def ohem_scores(logits, labels, ignore_index=255):
+    """Softmax probability at the label, 1 for ignored pixels (csrc/ohem_label_kernel.cu:112-151)."""
+    logits, labels = _prep(logits, labels)
+    sfx, _ = _suffix(logits)
+    n, c, m = _dims(logits)
+    out = np.ones(labels.shape, dtype=logits.dtype)
+    if logits.size:
+        _call("oracle_ohem_scores" + sfx, _ptr(logits), _ptr(labels), _ptr(out), i64(n), i64(c), i64(m),
+              i64(ignore_index))
+    return out
+
+
+def ohem_select(scores, labels, ignore_index, score_thresh, n_min):
+    """Labels with every pixel beyond the n_min lowest scores whose score exceeds the threshold set to
+    ignore_index (csrc/ohem_label_kernel.cu:155-168, 247-262)."""
+    scores = np.ascontiguousarray(scores)
+    labels = np.ascontiguousarray(labels, dtype=np.int64)
+    assert scores.shape == labels.shape
+    sfx, _ = _suffix(scores)
+    out = np.empty_like(labels)
+    rc = _call("oracle_ohem_select" + sfx, _ptr(scores), _ptr(labels), _ptr(out), i64(labels.size),
+               i64(ignore_index), f64(score_thresh), i64(n_min))
+    if rc != 0:
+        raise MemoryError("oracle_ohem_select ran out of memory")
+    return out
+
+
+def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
+    """ohem_cpp.score_ohem_label (csrc/ohem_label_kernel.cu:171-263)."""
+    return ohem_select(ohem_scores(logits, labels, ignore_index), labels, ignore_index, score_thresh, n_min)
+
+
 # ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
 # large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
 

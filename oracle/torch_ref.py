@@ -156,3 +156,28 @@ def lovasz(logits, labels, reduction="mean", ignore_index=-100):
     if reduction == "mean":
         return losses.mean()
     return losses
+
+
+def ohem_labels(logits, labels, ignore_index, score_thresh, n_min):
+    """The relabelling of ohem_cpp.score_ohem_label as torch ops (csrc/ohem_label_kernel.cu:171-263):
+    score = softmax probability at the label (1 at ignored pixels), stable ascending sort, every
+    pixel at position >= n_min with score > score_thresh becomes ignore_index."""
+    flat = labels.reshape(-1)
+    if n_min >= flat.numel():
+        return labels
+    ign = labels == ignore_index
+    probs = torch.softmax(logits.detach().float(), dim=1)
+    score = probs.gather(1, labels.masked_fill(ign, 0).unsqueeze(1)).squeeze(1)
+    score = score.masked_fill(ign, 1.0).reshape(-1)
+    order = torch.sort(score, stable=True).indices[max(n_min, 0):]
+    drop = order[score[order] > score_thresh]
+    out = flat.clone()
+    out[drop] = ignore_index
+    return out.reshape(labels.shape)
+
+
+def ohem_ce(logits, labels, score_thresh, n_min=None, ignore_index=255):
+    """OhemCELoss.forward (pytorch_loss/ohem_loss.py:22-27)."""
+    n_min = labels.numel() // 16 if n_min is None else n_min
+    new_labels = ohem_labels(logits, labels, ignore_index, score_thresh, n_min)
+    return F.cross_entropy(logits, new_labels, ignore_index=ignore_index, reduction="mean")

@@ -1,0 +1,403 @@
+// Online hard example mining by score for gfx950: softmax probability at the label, then the
+// relabelling rule "beyond the n_min lowest scores, a pixel whose score exceeds the threshold
+// becomes ignore_index" (csrc/ohem_label_kernel.cu:112-168, 171-263).
+//
+// The reference sorts all P scores with their indices (thrust::sort_by_key, :247) only to learn,
+// per pixel, whether its sorted position is below n_min. That is an order-statistic question, so
+// nothing is sorted here:
+//   1. scores      one pass over the logits (channel slice in registers), P fp32 scores out;
+//   2. select      a 3-digit (10 bits each) radix select over the score bit patterns finds v, the
+//                  n_min-th smallest score, and how many pixels with exactly that score still
+//                  fall below position n_min (`keep_ties`);
+//   3. ties        pixels equal to v are ranked in pixel order (what a stable key sort gives):
+//                  per-tile counts, one scan over the tiles, in-tile ranks from ballots;
+//   4. relabel     drop = score > thresh && (score > v || (score == v && tie_rank >= keep_ties)).
+// When v <= thresh every pixel above the threshold lies beyond position n_min, so steps 3 is
+// skipped on the device (the kernels return at once). Scores are positive floats, whose bit
+// patterns order like the values; patterns are clamped to that of 1.0f, so a NaN score ranks as
+// 1 and, failing `score > thresh`, is never relabelled.
+#include "plh_common.hpp"
+
+namespace plh {
+
+constexpr int kOhemBins = 1024;                 // 10 bits per digit, 3 digits cover [0, 0x3F800000]
+constexpr int kOhemTile = 1024;                 // pixels per block in the tie-ranking passes (256 threads x 4)
+constexpr uint32_t kOneBits = 0x3F800000u;
+
+struct OhemTables {
+    uint32_t *hist;        // [3][kOhemBins]
+    uint32_t *tile_ties;   // [tiles], exclusive-scanned in place
+};
+
+__device__ __forceinline__ uint32_t score_key(float s) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, s);
+    return b > kOneBits ? kOneBits : b;
+}
+__device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)((key >> (20 - 10 * pass)) & 1023u); }
+
+// ------------------------------------------------------------------ scores ----
+
+template <class T, int CP, int V, bool Uniform>
+__global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                              float *__restrict__ scores, int64_t P, int64_t m_size,
+                                                              int C, int64_t ignore) {
+    const PixelRef<V, Uniform> at(P, m_size, C);
+    if (!at.live) return;
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, C, m_size, raw);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    float out[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], ignore, C, ign);
+        float xv[CP];
+        const float mx = widen_and_max<T, V, CP>(raw, k, C, xv);
+        const float c = mx * kLog2e;
+        float s = 0.f, e_y = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, C)) {
+                const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
+                s += e;
+                e_y = (tgt == j) ? e : e_y;
+            }
+        // ignored pixels score 1 (ohem_label_kernel.cu:131-134); so does a label outside [0, C),
+        // which the reference leaves undefined
+        out[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s), 1.f);
+    }
+    store_vec<V>(scores + at.pix, out);
+}
+
+// Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).
+template <class T>
+__global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                        float *__restrict__ scores, int64_t P, int64_t m_size, int C,
+                                                        int64_t ignore) {
+    for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
+        const int64_t lb = lab[pix];
+        if (lb == ignore || lb < 0 || lb >= C) {
+            scores[pix] = 1.f;
+            continue;
+        }
+        const int64_t n = pix / m_size;
+        const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
+        float mx = -INFINITY;
+        for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
+        float s = 0.f;
+        for (int j = 0; j < C; ++j) s += fast_exp(load_one(xs + (int64_t)j * m_size) - mx);
+        scores[pix] = fminf(fast_exp(load_one(xs + lb * m_size) - mx) / s, 1.f);
+    }
+}
+
+// ------------------------------------------------------------------ select ----
+
+__global__ void ohem_zero(uint32_t *p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// What the histograms of the first `passes` digits say about the n_min-th smallest key: its leading
+// digits (as a key prefix) and `rank`, its 1-based position among the keys that share them. After
+// all three passes `prefix` is the key itself and `rank` the number of pixels equal to it that lie
+// below sorted position n_min. Every thread of the 256-thread block gets the result.
+struct Resolved {
+    uint32_t prefix;
+    uint32_t rank;
+};
+
+__device__ Resolved ohem_resolve(const uint32_t *hist, int passes, uint32_t n_min, uint32_t *lds /* >= 260 words */) {
+    Resolved r{0u, n_min};
+    const int t = threadIdx.x;
+    for (int pass = 0; pass < passes; ++pass) {
+        const uint32_t *h = hist + pass * kOhemBins;
+        // 4 consecutive bins per thread, then a scan over the 256 thread sums
+        uint32_t b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b[i] = h[t * 4 + i];
+        const uint32_t mine = b[0] + b[1] + b[2] + b[3];
+        lds[t] = mine;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            const uint32_t add = (t >= off) ? lds[t - off] : 0u;
+            __syncthreads();
+            lds[t] += add;
+            __syncthreads();
+        }
+        const uint32_t incl = lds[t], excl = incl - mine;
+        // exactly one thread owns the bin where the running count first reaches `rank`
+        if (excl < r.rank && r.rank <= incl) {
+            uint32_t run = excl;
+            int d = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (run < r.rank && r.rank <= run + b[i]) {
+                    d = t * 4 + i;
+                    lds[257] = r.rank - run;
+                }
+                run += b[i];
+            }
+            lds[256] = (uint32_t)d;
+        }
+        __syncthreads();
+        r.prefix |= lds[256] << (20 - 10 * pass);
+        r.rank = lds[257];
+        __syncthreads();
+    }
+    return r;
+}
+
+// Histogram of digit `pass` over the keys that share the already resolved leading digits.
+__global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ scores, OhemTables tb, int P, int pass,
+                                                 uint32_t n_min) {
+    __shared__ uint32_t bins[kOhemBins];
+    __shared__ uint32_t scan[260];
+    const Resolved r = ohem_resolve(tb.hist, pass, n_min, scan);
+    for (int i = threadIdx.x; i < kOhemBins; i += 256) bins[i] = 0;
+    __syncthreads();
+    const uint32_t high_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (30 - 10 * pass));
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < P; i += (int64_t)gridDim.x * 256) {
+        const uint32_t key = score_key(__builtin_nontemporal_load(scores + i));
+        if ((key & high_mask) == r.prefix) atomicAdd(&bins[key_digit(key, pass)], 1u);
+    }
+    __syncthreads();
+    uint32_t *out = tb.hist + pass * kOhemBins;
+    for (int i = threadIdx.x; i < kOhemBins; i += 256)
+        if (bins[i]) atomicAdd(out + i, bins[i]);
+}
+
+// Flags of this thread's 4 pixels: is the score equal to the n_min-th smallest?
+__device__ __forceinline__ void load_tile_keys(const float *scores, int P, int base, float (&s)[4], uint32_t (&key)[4]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int i = base + k;
+        s[k] = i < P ? scores[i] : 2.f;          // beyond the end: matches no key
+        key[k] = i < P ? score_key(s[k]) : 0xFFFFFFFFu;
+    }
+}
+
+__global__ __launch_bounds__(256) void ohem_count_ties(const float *__restrict__ scores, OhemTables tb, int P,
+                                                       uint32_t n_min, float thresh) {
+    __shared__ uint32_t scan[260];
+    __shared__ float red[4];
+    const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
+    if (!(__builtin_bit_cast(float, r.prefix) > thresh)) return;      // ranks are not needed
+    float s[4];
+    uint32_t key[4];
+    load_tile_keys(scores, P, blockIdx.x * kOhemTile + threadIdx.x * 4, s, key);
+    int n = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) n += key[k] == r.prefix ? 1 : 0;
+    const float total = block_sum_256((float)n, red);                 // <= 1024: exact
+    if (threadIdx.x == 0) tb.tile_ties[blockIdx.x] = (uint32_t)total;
+}
+
+// Exclusive scan of the per-tile tie counts, one block.
+__global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles, uint32_t n_min, float thresh) {
+    __shared__ uint32_t scan[260];
+    const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
+    if (!(__builtin_bit_cast(float, r.prefix) > thresh)) return;
+    __shared__ uint32_t carry;
+    if (threadIdx.x == 0) carry = 0;
+    __syncthreads();
+    for (int base = 0; base < tiles; base += 256) {
+        const int i = base + threadIdx.x;
+        const uint32_t v = i < tiles ? tb.tile_ties[i] : 0u;
+        scan[threadIdx.x] = v;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            const uint32_t add = (threadIdx.x >= off) ? scan[threadIdx.x - off] : 0u;
+            __syncthreads();
+            scan[threadIdx.x] += add;
+            __syncthreads();
+        }
+        if (i < tiles) tb.tile_ties[i] = carry + scan[threadIdx.x] - v;
+        __syncthreads();
+        if (threadIdx.x == 255) carry += scan[255];
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ scores, const int64_t *__restrict__ lab,
+                                                    int64_t *__restrict__ out, OhemTables tb, int P, uint32_t n_min,
+                                                    float thresh, int64_t ignore) {
+    __shared__ uint32_t scan[260];
+    __shared__ uint32_t wave_ties[4];
+    const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
+    float s[4];
+    uint32_t key[4];
+    load_tile_keys(scores, P, base, s, key);
+    bool drop[4];
+    if (n_min == 0) {                            // every position is beyond n_min
+#pragma unroll
+        for (int k = 0; k < 4; ++k) drop[k] = s[k] > thresh;
+    } else {
+        const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
+        if (!(__builtin_bit_cast(float, r.prefix) > thresh)) {
+            // the n_min-th smallest score is within the threshold: all above it lie beyond n_min
+#pragma unroll
+            for (int k = 0; k < 4; ++k) drop[k] = s[k] > thresh;
+        } else {
+            // rank of this thread's ties in pixel order: tiles before, waves before, lanes before
+            int mine = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) mine += key[k] == r.prefix ? 1 : 0;
+            int lane_incl = mine;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(lane_incl, off, 64);
+                if ((threadIdx.x & 63) >= off) lane_incl += up;
+            }
+            if ((threadIdx.x & 63) == 63) wave_ties[threadIdx.x >> 6] = (uint32_t)lane_incl;
+            __syncthreads();
+            uint32_t before = tb.tile_ties[blockIdx.x] + (uint32_t)(lane_incl - mine);
+            for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) before += wave_ties[w];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const bool tie = key[k] == r.prefix;
+                // every score here exceeds the threshold or is at most v; v itself exceeds it
+                drop[k] = key[k] != 0xFFFFFFFFu && (key[k] > r.prefix || (tie && before >= r.rank)) && s[k] > thresh;
+                before += tie ? 1u : 0u;
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (base + k < P) out[base + k] = drop[k] ? ignore : lab[base + k];
+}
+
+__global__ void ohem_copy_labels(const int64_t *__restrict__ in, int64_t *__restrict__ out, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        out[i] = in[i];
+}
+
+// ------------------------------------------------------------ host side ----
+
+constexpr int64_t kOhemMaxPixels = ((int64_t)1 << 31) - kOhemTile;
+
+static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+static int64_t ohem_tiles(int64_t P) { return ceil_div(P > 0 ? P : 1, kOhemTile); }
+
+static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, int64_t n_size,
+                         int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st) {
+    const int64_t P = n_size * m_size;
+    const int C = (int)dimsize;
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        const T *x = static_cast<const T *>(logits);
+        constexpr int VT = ElemTraits<T>::kVec;
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, nullptr);
+        if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
+            const bool vec = (shape == Shape::RegsVec);
+            const bool uni = vec && tiles_are_uniform(m_size, VT, sizeof(T));
+            const unsigned grid = vec ? regs_grid<VT>(P) : regs_grid<1>(P);
+            switch ((C + 3) / 4) {
+#define PLH_CASE(K)                                                                                                   \
+    case K:                                                                                                           \
+        if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
+                                    labels, scores, P, m_size, C, ignore_index);                                      \
+        else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, false>), dim3(grid), dim3(kRegsBlock), 0,    \
+                                         st, x, labels, scores, P, m_size, C, ignore_index);                          \
+        else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, false>), dim3(grid), dim3(kRegsBlock), 0, st, x,       \
+                                labels, scores, P, m_size, C, ignore_index);                                          \
+        break;
+                PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+            }
+        } else {
+            hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, P,
+                               m_size, C, ignore_index);
+        }
+    });
+    return check_launch();
+}
+
+static int64_t select_workspace(int64_t P) { return align256(3 * kOhemBins * 4) + align256(ohem_tiles(P) * 4); }
+
+// The tables are needed unless the labels pass through unchanged (n_min >= P).
+static int check_workspace(const void *workspace, int64_t workspace_bytes, int64_t P, int64_t n_min) {
+    if (n_min >= P) return PLH_OK;
+    if (!workspace || misaligned(workspace, 256) || workspace_bytes < select_workspace(P)) return PLH_ERR_WORKSPACE;
+    return PLH_OK;
+}
+
+static int launch_select(const float *scores, const int64_t *labels, int64_t *out_labels, void *workspace,
+                         int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st) {
+    if (n_min >= P) {                            // csrc/ohem_label_kernel.cu:189: labels are returned as they are
+        if (out_labels != labels)
+            hipLaunchKernelGGL(ohem_copy_labels, dim3((unsigned)(ceil_div(P, 256) < 4096 ? ceil_div(P, 256) : 4096)),
+                               dim3(256), 0, st, labels, out_labels, P);
+        return check_launch();
+    }
+    const int64_t tiles = ohem_tiles(P);
+    OhemTables tb;
+    tb.hist = static_cast<uint32_t *>(workspace);
+    tb.tile_ties = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + align256(3 * kOhemBins * 4));
+    const uint32_t k = n_min > 0 ? (uint32_t)n_min : 0u;
+    const int Pi = (int)P;
+    if (k > 0) {
+        hipLaunchKernelGGL(ohem_zero, dim3(3 * kOhemBins / 256), dim3(256), 0, st, tb.hist, 3 * kOhemBins);
+        const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 8) < 2048 ? ceil_div(P, 256 * 8) : 2048);
+        for (int pass = 0; pass < 3; ++pass)
+            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k);
+        hipLaunchKernelGGL(ohem_count_ties, dim3((unsigned)tiles), dim3(256), 0, st, scores, tb, Pi, k, score_thresh);
+        hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, k, score_thresh);
+    }
+    hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, k,
+                       score_thresh, ignore_index);
+    return check_launch();
+}
+
+}  // namespace plh
+
+using namespace plh;
+
+extern "C" int64_t plh_ohem_workspace_bytes(int64_t n_pixels) {
+    if (n_pixels < 0 || n_pixels > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
+    return select_workspace(n_pixels);
+}
+
+extern "C" int plh_ohem_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores,
+                               int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    const int rc = check_slice_args(logits, labels, scores, n_size, dimsize, m_size, dtype_size(dtype), 4);
+    if (rc != PLH_OK) return rc;
+    if (n_size * dimsize * m_size == 0) return PLH_OK;
+    return launch_scores(logits, dtype, labels, scores, n_size, dimsize, m_size, ignore_index, (hipStream_t)stream);
+}
+
+extern "C" int plh_ohem_select_labels(const float *scores, const int64_t *labels, int64_t *out_labels,
+                                      void *workspace, int64_t workspace_bytes, int64_t n_pixels,
+                                      int64_t ignore_index, float score_thresh, int64_t n_min, void *stream) {
+    if (n_pixels < 0 || n_pixels > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
+    if (n_pixels == 0) return PLH_OK;
+    if (!scores || !labels || !out_labels) return PLH_ERR_NULL_POINTER;
+    if (misaligned(scores, 4) || misaligned(labels, 8) || misaligned(out_labels, 8)) return PLH_ERR_MISALIGNED;
+    const int rc = check_workspace(workspace, workspace_bytes, n_pixels, n_min);
+    if (rc != PLH_OK) return rc;
+    return launch_select(scores, labels, out_labels, workspace, n_pixels, ignore_index, score_thresh, n_min,
+                         (hipStream_t)stream);
+}
+
+extern "C" int plh_ohem_score_label(const void *logits, int32_t dtype, const int64_t *labels, int64_t *out_labels,
+                                    float *scores, void *workspace, int64_t workspace_bytes,
+                                    int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                    float score_thresh, int64_t n_min, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    int rc = check_slice_args(logits, labels, out_labels, n_size, dimsize, m_size, dtype_size(dtype), 8);
+    if (rc != PLH_OK) return rc;
+    if (n_size * m_size > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
+    if (n_size * dimsize * m_size == 0) return PLH_OK;
+    const int64_t P = n_size * m_size;
+    rc = check_workspace(workspace, workspace_bytes, P, n_min);
+    if (rc != PLH_OK) return rc;
+    if (n_min < P) {
+        if (!scores) return PLH_ERR_NULL_POINTER;
+        if (misaligned(scores, 4)) return PLH_ERR_MISALIGNED;
+        rc = launch_scores(logits, dtype, labels, scores, n_size, dimsize, m_size, ignore_index, (hipStream_t)stream);
+        if (rc != PLH_OK) return rc;
+    }
+    return launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min,
+                         (hipStream_t)stream);
+}

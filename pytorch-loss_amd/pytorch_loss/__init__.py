@@ -2,17 +2,20 @@
 
     from pytorch_loss import LabelSmoothSoftmaxCEV3, FocalLossV3, LargeMarginSoftmaxV3, LovaszSoftmaxV3
 
-Only this path is provided; the kernels live in libpytorch_loss_hip.so (built by
+Plus the relabelling step in front of that path in segmentation training, ``OhemCELoss`` /
+``OhemLargeMarginLoss``. Only this path is provided; the kernels live in libpytorch_loss_hip.so (built by
 ``python pytorch-loss_amd/build.py``) and there is no CPU fallback.
 """
 from .label_smooth import LabelSmoothSoftmaxCEV3, LSRCrossEntropyFunctionV3
 from .focal_loss import FocalLossV3, FocalSigmoidLossFuncV3, FocalSigmoidLossFuncV3FB
 from .large_margin_softmax import LargeMarginSoftmaxV3, LargeMarginSoftmaxFuncV3, LargeMarginSoftmaxFuncV3FB
 from .lovasz_softmax import LovaszSoftmaxV3, LovaszSoftmaxFunctionV3
+from .ohem_loss import OhemCELoss, OhemLargeMarginLoss, score_ohem_label
 
 __all__ = [
     "LabelSmoothSoftmaxCEV3", "LSRCrossEntropyFunctionV3",
     "FocalLossV3", "FocalSigmoidLossFuncV3", "FocalSigmoidLossFuncV3FB",
     "LargeMarginSoftmaxV3", "LargeMarginSoftmaxFuncV3", "LargeMarginSoftmaxFuncV3FB",
     "LovaszSoftmaxV3", "LovaszSoftmaxFunctionV3",
+    "OhemCELoss", "OhemLargeMarginLoss", "score_ohem_label",
 ]

@@ -47,6 +47,10 @@ _SIGNATURES = {
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "plh_ohem_workspace_bytes": (_i64, [_i64]),
+    "plh_ohem_scores": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _p]),
+    "plh_ohem_select_labels": (ctypes.c_int, [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _i64, _p]),
+    "plh_ohem_score_label": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
 
@@ -427,6 +431,57 @@ def lovasz_backward(grad_output, logits, labels, jacc, ignore_index, args=None):
     _call(a.x, "plh_lovasz_backward", _ptr(go), _ptr(a.x), a.tag, _ptr(a.lb), _ptr(jc), _ptr(grad), a.n, a.c, a.m,
           int(ignore_index))
     return _back_to(grad, a.dtype)
+
+
+# ----------------------------------------------------------------- ohem ----
+
+def ohem_args(logits, labels):
+    if labels.numel() > (1 << 31) - 1024:
+        raise RuntimeError("score_ohem_label: too many pixels, int32 type will overflow")
+    return seg_args(logits, labels, "ohem method", "score_ohem_label")
+
+
+def _ohem_workspace(n_pixels, device):
+    nbytes = int(load().plh_ohem_workspace_bytes(int(n_pixels)))
+    if nbytes < 0:
+        _check(nbytes)
+    return torch.empty((nbytes,), dtype=torch.uint8, device=device), nbytes
+
+
+def ohem_scores(logits, labels, ignore_index):
+    """softmax(logits)[label] per pixel as fp32, 1 at ignored pixels."""
+    a = ohem_args(logits, labels)
+    scores = torch.empty(a.lb.shape, dtype=torch.float32, device=a.x.device)
+    if a.x.numel():
+        _call(a.x, "plh_ohem_scores", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(scores), a.n, a.c, a.m, int(ignore_index))
+    return scores
+
+
+def ohem_select_labels(scores, labels, ignore_index, score_thresh, n_min):
+    _require_gpu("ohem method", scores, labels)
+    if scores.shape != labels.shape or scores.dtype != torch.float32 or labels.dtype != torch.int64:
+        raise RuntimeError("ohem_select_labels: scores (fp32) and labels (int64) must have the same shape")
+    sc, lb = scores.contiguous(), labels.contiguous()
+    out = torch.empty_like(lb)
+    if lb.numel():
+        ws, ws_bytes = _ohem_workspace(lb.numel(), lb.device)
+        _call(lb, "plh_ohem_select_labels", _ptr(sc), _ptr(lb), _ptr(out), _ptr(ws), ws_bytes, lb.numel(),
+              int(ignore_index), float(score_thresh), int(n_min))
+    return out
+
+
+def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
+    """-> new int64 labels of labels' shape; the inputs are left untouched."""
+    a = ohem_args(logits, labels)
+    out = torch.empty_like(a.lb)
+    if a.lb.numel() == 0:
+        return out
+    n_pixels = a.n * a.m
+    scores = torch.empty((n_pixels if n_min < n_pixels else 1,), dtype=torch.float32, device=a.x.device)
+    ws, ws_bytes = _ohem_workspace(n_pixels, a.x.device)
+    _call(a.x, "plh_ohem_score_label", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(out), _ptr(scores), _ptr(ws), ws_bytes,
+          a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
+    return out
 
 
 def stream_copy(src, dst):

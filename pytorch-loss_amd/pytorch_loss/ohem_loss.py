@@ -1,0 +1,49 @@
+"""Online hard example mining losses on the HIP kernels.
+
+Same surface as the reference's pytorch_loss/ohem_loss.py:13-45: both modules first relabel the
+easy pixels as ignored (``score_ohem_label``: beyond the ``n_min`` lowest-scoring pixels, every
+pixel whose softmax probability at its label exceeds ``score_thresh`` gets ``ignore_index``),
+then take the mean loss over what is left.  ``OhemCELoss`` uses plain cross entropy, which is
+the label-smoothed kernel with a smoothing factor of 0 (the reference calls
+``nn.CrossEntropyLoss(ignore_index, reduction='mean')``, ohem_loss.py:20); ``OhemLargeMarginLoss``
+uses ``LargeMarginSoftmaxV3``.
+"""
+import torch.nn as nn
+
+from . import _native
+from .label_smooth import LabelSmoothSoftmaxCEV3
+from .large_margin_softmax import LargeMarginSoftmaxV3
+
+
+def score_ohem_label(logits, labels, ignore_index, score_thresh, n_min):
+    """Stand-in for ``ohem_cpp.score_ohem_label`` (csrc/ohem_label_kernel.cu:266-276): new labels,
+    detached from any graph; logits may be fp32, fp16 or bf16 (scores are formed in fp32)."""
+    return _native.ohem_score_label(logits.detach(), labels, ignore_index, score_thresh, n_min)
+
+
+class _OhemLoss(nn.Module):
+
+    def __init__(self, score_thresh, n_min=None, ignore_index=255):
+        super().__init__()
+        self.score_thresh = score_thresh
+        self.ignore_lb = ignore_index
+        self.n_min = n_min
+
+    def forward(self, logits, labels):
+        n_min = labels.numel() // 16 if self.n_min is None else self.n_min
+        labels = score_ohem_label(logits, labels, self.ignore_lb, self.score_thresh, n_min)
+        return self.criteria(logits, labels)
+
+
+class OhemCELoss(_OhemLoss):
+
+    def __init__(self, score_thresh, n_min=None, ignore_index=255):
+        super().__init__(score_thresh, n_min, ignore_index)
+        self.criteria = LabelSmoothSoftmaxCEV3(lb_smooth=0.0, reduction="mean", ignore_index=ignore_index)
+
+
+class OhemLargeMarginLoss(_OhemLoss):
+
+    def __init__(self, score_thresh, n_min=None, ignore_index=255):
+        super().__init__(score_thresh, n_min, ignore_index)
+        self.criteria = LargeMarginSoftmaxV3(ignore_index=ignore_index, reduction="mean")

@@ -86,6 +86,24 @@ def test_arguments_are_rejected_before_any_launch(native):
         assert lib.plh_focal_forward_backward(p, bad, p, p, p, 4, 2.0, 0.25, None) == -7
         assert lib.plh_lovasz_forward(p, bad, lp, p, p, p, need, 2, 19, 64, 255, None) == -7
         assert lib.plh_lovasz_backward(p, p, bad, lp, p, p, 2, 19, 64, 255, None) == -7
+    # online hard example mining
+    assert lib.plh_ohem_workspace_bytes(-1) == -2 and lib.plh_ohem_workspace_bytes(1 << 31) == -2
+    ohem_need = lib.plh_ohem_workspace_bytes(4096)
+    assert ohem_need >= 3 * 1024 * 4 + 4 * 4 and ohem_need % 256 == 0
+    big = (ctypes.c_char * (ohem_need + 512))()
+    wsp = ctypes.c_void_p((ctypes.addressof(big) + 255) & ~255)              # 256-byte aligned, as required
+    assert lib.plh_ohem_scores(None, 0, None, None, 0, 19, 16, 255, None) == 0
+    assert lib.plh_ohem_scores(p, 5, lp, p, 1, 2, 2, 255, None) == -7
+    assert lib.plh_ohem_scores(p, 0, lp, None, 1, 2, 2, 255, None) == -1
+    assert lib.plh_ohem_select_labels(None, None, None, None, 0, 0, 255, 0.7, 0, None) == 0
+    assert lib.plh_ohem_select_labels(p, lp, None, wsp, ohem_need, 4, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_select_labels(p, lp, lp, None, 0, 4, 255, 0.7, 1, None) == -5
+    assert lib.plh_ohem_select_labels(p, lp, lp, wsp, ohem_need, -4, 255, 0.7, 1, None) == -2
+    assert lib.plh_ohem_score_label(p, 9, lp, lp, p, wsp, ohem_need, 1, 2, 2, 255, 0.7, 1, None) == -7
+    assert lib.plh_ohem_score_label(p, 0, lp, lp, None, wsp, ohem_need, 1, 2, 2, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_score_label(p, 0, lp, lp, p, None, 0, 1, 2, 2, 255, 0.7, 1, None) == -5
+    assert lib.plh_ohem_score_label(p, 0, lp, lp, p, ctypes.c_void_p(wsp.value + 8), ohem_need, 1, 2, 2, 255, 0.7, 1,
+                                    None) == -5                                  # misaligned workspace
     # 16-bit logits need 2-byte alignment only; an odd address is still refused
     assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384

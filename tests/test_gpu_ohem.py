@@ -1,0 +1,165 @@
+"""GPU parity of the online-hard-example-mining step (through the C ABI) against the CPU oracle.
+
+The relabelling is integer work on given scores, so `plh_ohem_select_labels` is held bit-exact to
+the oracle on identical fp32 scores, with tie-heavy score sets, every boundary of n_min and tile
+sizes around the kernels' 1024-pixel tiles.  The scores are floating point: 1e-6 absolute against
+the fp32 oracle.  The fused call is then (a) bit-exact to the oracle's selection applied to the
+GPU's own scores and (b) equal to the all-oracle result except at pixels whose score lies within
+2e-6 of a decision boundary (the threshold or the n_min-th smallest score), where no two fp32
+softmax evaluations need agree.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+from .test_gpu_parity import close_grad, dev, seg_inputs
+from .test_oracle_ohem import _scores
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def native():
+    from pytorch_loss import _native
+    _native.load()
+    return _native
+
+
+SCORE_CASES = [
+    ((2, 19, 64, 64), 255, 0.05),        # uniform tiles, 8 bytes per lane
+    ((2, 19, 7, 9), 255, 0.1),           # one pixel per thread
+    ((3, 2, 5, 8), -100, 0.2),
+    ((37, 10), -100, 0.1),
+    ((33, 100), -100, 0.1),              # more than 32 channels: lane per pixel
+    ((2, 33, 6, 7), 255, 0.2),
+    ((2, 19, 16, 16), 255, 1.0),         # everything ignored
+]
+
+
+@pytest.mark.parametrize("shape,ignore,frac", SCORE_CASES)
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16], ids=["fp32", "fp16", "bf16"])
+def test_scores_match_oracle(native, shape, ignore, frac, dt):
+    x, y = seg_inputs(81, shape, ignore, frac)
+    xt = dev(x).to(dt)
+    got = native.ohem_scores(xt, dev(y), ignore).cpu().numpy()
+    want = oracle.ohem_scores(xt.float().cpu().numpy(), y, ignore)
+    assert got.dtype == np.float32 and got.shape == y.shape
+    assert np.abs(got - want).max() <= 1e-6
+    assert (got[y == ignore] == 1.0).all() and got.max() <= 1.0 and got.min() >= 0.0
+
+
+@pytest.mark.parametrize("kind", ["smooth", "coarse", "saturated"])
+@pytest.mark.parametrize("n", [1, 5, 1023, 1024, 1025, 4099, 70_001])
+def test_select_is_bit_exact_on_given_scores(native, kind, n):
+    s = _scores(82, n, kind)
+    y = synth.randint(82, 2, (n,), 0, 19).astype(np.int64)
+    y[synth.bernoulli(82, 3, (n,), 0.1)] = 255
+    st, yt = dev(s), dev(y)
+    for n_min in sorted({0, 1, 2, n // 16, n // 2, n - 1, n, n + 3, -1}):
+        for thresh in (0.0, 0.5, 0.7, 0.875, 1.0):
+            got = native.ohem_select_labels(st, yt, 255, thresh, n_min).cpu().numpy()
+            want = oracle.ohem_select(s, y, 255, thresh, max(n_min, 0))
+            assert np.array_equal(got, want), (kind, n, n_min, thresh, int((got != want).sum()))
+    assert np.array_equal(yt.cpu().numpy(), y)          # the input labels are not touched
+
+
+def test_select_all_equal_scores(native):
+    n = 5000
+    y = synth.randint(83, 2, (n,), 0, 19).astype(np.int64)
+    for value in (1.0, 0.25):
+        s = np.full((n,), value, dtype=np.float32)
+        for n_min in (1, 1024, 1025, 4999):
+            got = native.ohem_select_labels(dev(s), dev(y), 255, 0.1, n_min).cpu().numpy()
+            assert np.array_equal(got, oracle.ohem_select(s, y, 255, 0.1, n_min))
+            assert (got[:n_min] == y[:n_min]).all() and (got[n_min:] == 255).all()
+
+
+def _near_boundary(scores, thresh, n_min, tol=2e-6):
+    flat = np.sort(scores.ravel())
+    near = np.abs(scores - np.float32(thresh)) <= tol
+    if 0 < n_min < flat.size:
+        near |= np.abs(scores - flat[n_min - 1]) <= tol
+    return near
+
+
+@pytest.mark.parametrize("shape,ignore,frac", SCORE_CASES)
+@pytest.mark.parametrize("thresh,div", [(0.7, 16), (0.05, 16), (0.3, 2), (0.0, 4)])
+def test_score_label_matches_oracle(native, shape, ignore, frac, thresh, div):
+    x, y = seg_inputs(84, shape, ignore, frac)
+    xt, yt = dev(x), dev(y)
+    n_min = y.size // div
+    got = native.ohem_score_label(xt, yt, ignore, thresh, n_min).cpu().numpy()
+    own = native.ohem_scores(xt, yt, ignore).cpu().numpy()
+    assert np.array_equal(got, oracle.ohem_select(own, y, ignore, thresh, n_min))
+    s = oracle.ohem_scores(x, y, ignore)
+    want = oracle.ohem_select(s, y, ignore, thresh, n_min)
+    differ = got != want
+    assert not (differ & ~_near_boundary(s, thresh, n_min)).any(), int(differ.sum())
+    assert differ.mean() < 1e-3
+
+
+def test_score_label_full_resolution(native):
+    shape = (2, 19, 1024, 1024)
+    x, y = seg_inputs(85, shape, 255, 0.05)
+    x *= 2.0                                            # a sharper softmax: scores on both sides of 0.7
+    xt, yt = dev(x), dev(y)
+    n_min = y.size // 16
+    got = native.ohem_score_label(xt, yt, 255, 0.7, n_min).cpu().numpy()
+    own = native.ohem_scores(xt, yt, 255).cpu().numpy()
+    assert np.array_equal(got, oracle.ohem_select(own, y, 255, 0.7, n_min))
+    kept = got != 255
+    assert np.array_equal(got[kept], y[kept]) and (own[~kept & (y != 255)] > 0.7).all()
+    assert kept.sum() >= n_min and kept[(own <= 0.7) & (y != 255)].all()
+    # a threshold that nothing reaches below n_min: the tie-ranked branch at full size
+    got2 = native.ohem_score_label(xt, yt, 255, 1e-7, y.size // 2).cpu().numpy()
+    assert np.array_equal(got2, oracle.ohem_select(own, y, 255, 1e-7, y.size // 2))
+
+
+@pytest.mark.parametrize("which", ["ce", "lmargin"])
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_ohem_modules(native, which, dt):
+    import pytorch_loss as pl
+    shape = (2, 19, 32, 32)
+    x, y = seg_inputs(86, shape, 255, 0.05)
+    xt = dev(x).to(dt).requires_grad_()
+    xr = xt.detach().float().cpu().numpy()
+    yt = dev(y)
+    n_min = y.size // 16
+    crit = (pl.OhemCELoss if which == "ce" else pl.OhemLargeMarginLoss)(score_thresh=0.3, n_min=n_min, ignore_index=255)
+    with torch.autocast("cuda", dtype=dt, enabled=dt != torch.float32):
+        loss = crit(xt, yt)
+    new_labels = pl.score_ohem_label(xt, yt, 255, 0.3, n_min).cpu().numpy()
+    assert (new_labels != y).any() and np.array_equal(yt.cpu().numpy(), y)
+    if which == "ce":
+        per = oracle.lsr_forward(xr.astype(np.float64), new_labels, 255, 0.0)
+        grad_of = lambda g: oracle.lsr_backward(xr, new_labels, 255, 0.0, g)
+        # plain cross entropy is what the reference's criterion computes (ohem_loss.py:20)
+        ce = torch.nn.functional.cross_entropy(torch.from_numpy(xr).double(), torch.from_numpy(new_labels),
+                                               ignore_index=255, reduction="mean").item()
+        assert abs(loss.item() - ce) <= 1e-5 * abs(ce)
+    else:
+        per = oracle.lmargin_forward(xr.astype(np.float64), new_labels, 0.3, 255)
+        grad_of = lambda g: oracle.lmargin_backward(xr, new_labels, 0.3, 255, g)
+    n_valid = int((new_labels != 255).sum())
+    want = per.sum() / n_valid
+    assert abs(loss.item() - want) <= 1e-5 * abs(want)
+    loss.backward()
+    want_g = grad_of(np.float32(1.0 / n_valid))
+    if dt == torch.float32:
+        close_grad(xt.grad.cpu().numpy(), want_g, which)
+    else:
+        err = np.abs(xt.grad.float().cpu().numpy() - want_g) - (2.0 ** -7 * np.abs(want_g) + 1e-7)
+        assert (err <= 0).all()
+    # default n_min = numel // 16 (ohem_loss.py:23)
+    crit2 = (pl.OhemCELoss if which == "ce" else pl.OhemLargeMarginLoss)(score_thresh=0.3)
+    assert crit2.n_min is None and torch.isfinite(crit2(xt.detach(), yt)).item()
+
+
+def test_ohem_refuses_cpu_tensors():
+    import pytorch_loss as pl
+    x = torch.randn(2, 5, 4, 4)
+    y = torch.randint(0, 5, (2, 4, 4))
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        pl.OhemCELoss(0.7)(x, y)
