@@ -24,10 +24,6 @@ constexpr int kOhemBins = 1024;                 // 10 bits per digit, 3 digits c
 constexpr int kOhemTile = 1024;                 // pixels per block in the tie-ranking passes (256 threads x 4)
 constexpr uint32_t kOneBits = 0x3F800000u;
 
-struct OhemTables {
-    uint32_t *hist;        // [3][kOhemBins]
-    uint32_t *tile_ties;   // [tiles], exclusive-scanned in place
-};
 
 __device__ __forceinline__ uint32_t score_key(float s) {
     const uint32_t b = __builtin_bit_cast(uint32_t, s);
@@ -93,73 +89,84 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
 
 // ------------------------------------------------------------------ select ----
 
+// Tables of the selection, all in the caller's workspace. `state` (16 words, zeroed with the
+// histograms): [2*pass] = key prefix after `pass`+1 digits, [2*pass+1] = 1-based rank of the
+// n_min-th smallest key among the keys sharing that prefix.
+struct OhemTables {
+    uint32_t *hist;        // [3][kOhemBins]
+    uint32_t *state;       // [16]
+    uint32_t *tile_ties;   // [tiles], exclusive-scanned in place
+};
+constexpr int kOhemZeroWords = 3 * kOhemBins + 16;
+
 __global__ void ohem_zero(uint32_t *p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0;
 }
 
-// What the histograms of the first `passes` digits say about the n_min-th smallest key: its leading
-// digits (as a key prefix) and `rank`, its 1-based position among the keys that share them. After
-// all three passes `prefix` is the key itself and `rank` the number of pixels equal to it that lie
-// below sorted position n_min. Every thread of the 256-thread block gets the result.
-struct Resolved {
-    uint32_t prefix;
-    uint32_t rank;
-};
-
-__device__ Resolved ohem_resolve(const uint32_t *hist, int passes, uint32_t n_min, uint32_t *lds /* >= 260 words */) {
-    Resolved r{0u, n_min};
+// One digit of the selection, by one 256-thread block: in histogram `h` (kOhemBins counts) find the
+// bin where the running count first reaches `rank` (1-based) and the rank left inside that bin.
+// Every thread gets the result. `lds` holds at least 260 words.
+__device__ void ohem_pick_digit(const uint32_t *h, uint32_t rank, uint32_t *lds, uint32_t &digit, uint32_t &rank_in_bin) {
     const int t = threadIdx.x;
-    for (int pass = 0; pass < passes; ++pass) {
-        const uint32_t *h = hist + pass * kOhemBins;
-        // 4 consecutive bins per thread, then a scan over the 256 thread sums
-        uint32_t b[4];
+    uint32_t b[4];                               // 4 consecutive bins per thread, then a scan over the 256 sums
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b[i] = h[t * 4 + i];
-        const uint32_t mine = b[0] + b[1] + b[2] + b[3];
-        lds[t] = mine;
+    for (int i = 0; i < 4; ++i) b[i] = h[t * 4 + i];
+    const uint32_t mine = b[0] + b[1] + b[2] + b[3];
+    lds[t] = mine;
+    if (t == 0) { lds[256] = 0; lds[257] = 1; }
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        const uint32_t add = (t >= off) ? lds[t - off] : 0u;
         __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {
-            const uint32_t add = (t >= off) ? lds[t - off] : 0u;
-            __syncthreads();
-            lds[t] += add;
-            __syncthreads();
-        }
-        const uint32_t incl = lds[t], excl = incl - mine;
-        // exactly one thread owns the bin where the running count first reaches `rank`
-        if (excl < r.rank && r.rank <= incl) {
-            uint32_t run = excl;
-            int d = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (run < r.rank && r.rank <= run + b[i]) {
-                    d = t * 4 + i;
-                    lds[257] = r.rank - run;
-                }
-                run += b[i];
-            }
-            lds[256] = (uint32_t)d;
-        }
-        __syncthreads();
-        r.prefix |= lds[256] << (20 - 10 * pass);
-        r.rank = lds[257];
+        lds[t] += add;
         __syncthreads();
     }
-    return r;
+    const uint32_t incl = lds[t], excl = incl - mine;
+    if (excl < rank && rank <= incl) {           // exactly one thread owns the bin
+        uint32_t run = excl;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (run < rank && rank <= run + b[i]) {
+                lds[256] = (uint32_t)(t * 4 + i);
+                lds[257] = rank - run;
+            }
+            run += b[i];
+        }
+    }
+    __syncthreads();
+    digit = lds[256];
+    rank_in_bin = lds[257];
+    __syncthreads();
+}
+
+__device__ __forceinline__ void hist_add(uint32_t *bins, float s, uint32_t high_mask, uint32_t prefix, int pass) {
+    const uint32_t key = score_key(s);
+    if ((key & high_mask) == prefix) atomicAdd(&bins[key_digit(key, pass)], 1u);
 }
 
 // Histogram of digit `pass` over the keys that share the already resolved leading digits.
 __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ scores, OhemTables tb, int P, int pass,
-                                                 uint32_t n_min) {
+                                                 uint32_t n_min, int vec) {
     __shared__ uint32_t bins[kOhemBins];
-    __shared__ uint32_t scan[260];
-    const Resolved r = ohem_resolve(tb.hist, pass, n_min, scan);
+    const uint32_t prefix = pass == 0 ? 0u : tb.state[2 * (pass - 1)];
     for (int i = threadIdx.x; i < kOhemBins; i += 256) bins[i] = 0;
     __syncthreads();
     const uint32_t high_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (30 - 10 * pass));
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < P; i += (int64_t)gridDim.x * 256) {
-        const uint32_t key = score_key(__builtin_nontemporal_load(scores + i));
-        if ((key & high_mask) == r.prefix) atomicAdd(&bins[key_digit(key, pass)], 1u);
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
+    if (vec) {
+        const int64_t quads = P / 4;
+        const plh_f4 *s4 = reinterpret_cast<const plh_f4 *>(scores);
+        for (int64_t i = gid; i < quads; i += stride) {
+            const plh_f4 v = __builtin_nontemporal_load(s4 + i);
+            hist_add(bins, v.x, high_mask, prefix, pass);
+            hist_add(bins, v.y, high_mask, prefix, pass);
+            hist_add(bins, v.z, high_mask, prefix, pass);
+            hist_add(bins, v.w, high_mask, prefix, pass);
+        }
+        if (gid < P - quads * 4) hist_add(bins, scores[quads * 4 + gid], high_mask, prefix, pass);
+    } else {
+        for (int64_t i = gid; i < P; i += stride) hist_add(bins, scores[i], high_mask, prefix, pass);
     }
     __syncthreads();
     uint32_t *out = tb.hist + pass * kOhemBins;
@@ -167,38 +174,62 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
         if (bins[i]) atomicAdd(out + i, bins[i]);
 }
 
-// Flags of this thread's 4 pixels: is the score equal to the n_min-th smallest?
-__device__ __forceinline__ void load_tile_keys(const float *scores, int P, int base, float (&s)[4], uint32_t (&key)[4]) {
+// One block: resolves digit `pass` from its finished histogram and publishes prefix and rank for
+// the kernels that follow. (A kernel of its own rather than the last block of ohem_hist: that would
+// need a device-wide release fence in every block, which costs far more than a launch on a GPU
+// whose XCDs have separate L2s.)
+__global__ __launch_bounds__(256) void ohem_pick(OhemTables tb, int pass, uint32_t n_min) {
+    __shared__ uint32_t scan[260];
+    const uint32_t prefix = pass == 0 ? 0u : tb.state[2 * (pass - 1)];
+    const uint32_t rank = pass == 0 ? n_min : tb.state[2 * (pass - 1) + 1];
+    uint32_t digit, rank_in_bin;
+    ohem_pick_digit(tb.hist + pass * kOhemBins, rank, scan, digit, rank_in_bin);
+    if (threadIdx.x == 0) {
+        tb.state[2 * pass] = prefix | (digit << (20 - 10 * pass));
+        tb.state[2 * pass + 1] = rank_in_bin;
+    }
+}
+
+// This thread's 4 consecutive scores and their keys; pixels beyond the end match no key.
+__device__ __forceinline__ void load_tile_keys(const float *scores, int P, int base, bool vec, float (&s)[4],
+                                               uint32_t (&key)[4]) {
+    if (vec && base + 3 < P) {
+        const plh_f4 v = __builtin_nontemporal_load(reinterpret_cast<const plh_f4 *>(scores + base));
+        s[0] = v.x; s[1] = v.y; s[2] = v.z; s[3] = v.w;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) key[k] = score_key(s[k]);
+        return;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int i = base + k;
-        s[k] = i < P ? scores[i] : 2.f;          // beyond the end: matches no key
+        s[k] = i < P ? scores[i] : 2.f;
         key[k] = i < P ? score_key(s[k]) : 0xFFFFFFFFu;
     }
 }
 
+// state[4], state[5]: v = the n_min-th smallest key, and how many pixels equal to it lie below
+// sorted position n_min. Ranks among the ties are needed only when v exceeds the threshold.
 __global__ __launch_bounds__(256) void ohem_count_ties(const float *__restrict__ scores, OhemTables tb, int P,
-                                                       uint32_t n_min, float thresh) {
-    __shared__ uint32_t scan[260];
+                                                       float thresh, int vec) {
     __shared__ float red[4];
-    const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
-    if (!(__builtin_bit_cast(float, r.prefix) > thresh)) return;      // ranks are not needed
+    const uint32_t v = tb.state[4];
+    if (!(__builtin_bit_cast(float, v) > thresh)) return;
     float s[4];
     uint32_t key[4];
-    load_tile_keys(scores, P, blockIdx.x * kOhemTile + threadIdx.x * 4, s, key);
+    load_tile_keys(scores, P, blockIdx.x * kOhemTile + threadIdx.x * 4, vec != 0, s, key);
     int n = 0;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) n += key[k] == r.prefix ? 1 : 0;
+    for (int k = 0; k < 4; ++k) n += key[k] == v ? 1 : 0;
     const float total = block_sum_256((float)n, red);                 // <= 1024: exact
     if (threadIdx.x == 0) tb.tile_ties[blockIdx.x] = (uint32_t)total;
 }
 
 // Exclusive scan of the per-tile tie counts, one block.
-__global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles, uint32_t n_min, float thresh) {
-    __shared__ uint32_t scan[260];
-    const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
-    if (!(__builtin_bit_cast(float, r.prefix) > thresh)) return;
+__global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles, float thresh) {
+    __shared__ uint32_t scan[256];
     __shared__ uint32_t carry;
+    if (!(__builtin_bit_cast(float, tb.state[4]) > thresh)) return;
     if (threadIdx.x == 0) carry = 0;
     __syncthreads();
     for (int base = 0; base < tiles; base += 256) {
@@ -221,46 +252,51 @@ __global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles,
 
 __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ scores, const int64_t *__restrict__ lab,
                                                     int64_t *__restrict__ out, OhemTables tb, int P, uint32_t n_min,
-                                                    float thresh, int64_t ignore) {
-    __shared__ uint32_t scan[260];
+                                                    float thresh, int64_t ignore, int vec) {
     __shared__ uint32_t wave_ties[4];
     const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
     float s[4];
     uint32_t key[4];
-    load_tile_keys(scores, P, base, s, key);
+    load_tile_keys(scores, P, base, vec != 0, s, key);
     bool drop[4];
-    if (n_min == 0) {                            // every position is beyond n_min
+    const uint32_t v = n_min == 0 ? 0u : tb.state[4];
+    if (n_min == 0 || !(__builtin_bit_cast(float, v) > thresh)) {
+        // every position is beyond n_min, or the n_min-th smallest score is within the threshold:
+        // all scores above the threshold lie beyond position n_min
 #pragma unroll
         for (int k = 0; k < 4; ++k) drop[k] = s[k] > thresh;
     } else {
-        const Resolved r = ohem_resolve(tb.hist, 3, n_min, scan);
-        if (!(__builtin_bit_cast(float, r.prefix) > thresh)) {
-            // the n_min-th smallest score is within the threshold: all above it lie beyond n_min
+        // rank of this thread's ties in pixel order: tiles before, waves before, lanes before
+        const uint32_t keep_ties = tb.state[5];
+        int mine = 0;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) drop[k] = s[k] > thresh;
-        } else {
-            // rank of this thread's ties in pixel order: tiles before, waves before, lanes before
-            int mine = 0;
+        for (int k = 0; k < 4; ++k) mine += key[k] == v ? 1 : 0;
+        int lane_incl = mine;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) mine += key[k] == r.prefix ? 1 : 0;
-            int lane_incl = mine;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int up = __shfl_up(lane_incl, off, 64);
-                if ((threadIdx.x & 63) >= off) lane_incl += up;
-            }
-            if ((threadIdx.x & 63) == 63) wave_ties[threadIdx.x >> 6] = (uint32_t)lane_incl;
-            __syncthreads();
-            uint32_t before = tb.tile_ties[blockIdx.x] + (uint32_t)(lane_incl - mine);
-            for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) before += wave_ties[w];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const bool tie = key[k] == r.prefix;
-                // every score here exceeds the threshold or is at most v; v itself exceeds it
-                drop[k] = key[k] != 0xFFFFFFFFu && (key[k] > r.prefix || (tie && before >= r.rank)) && s[k] > thresh;
-                before += tie ? 1u : 0u;
-            }
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(lane_incl, off, 64);
+            if ((threadIdx.x & 63) >= off) lane_incl += up;
         }
+        if ((threadIdx.x & 63) == 63) wave_ties[threadIdx.x >> 6] = (uint32_t)lane_incl;
+        __syncthreads();
+        uint32_t before = tb.tile_ties[blockIdx.x] + (uint32_t)(lane_incl - mine);
+        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) before += wave_ties[w];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const bool tie = key[k] == v;
+            drop[k] = key[k] != 0xFFFFFFFFu && (key[k] > v || (tie && before >= keep_ties)) && s[k] > thresh;
+            before += tie ? 1u : 0u;
+        }
+    }
+    if (vec && base + 3 < P) {
+        const plh_l2 *in2 = reinterpret_cast<const plh_l2 *>(lab + base);
+        plh_l2 *out2 = reinterpret_cast<plh_l2 *>(out + base);
+        plh_l2 a = __builtin_nontemporal_load(in2), b = __builtin_nontemporal_load(in2 + 1);
+        a.x = drop[0] ? ignore : a.x; a.y = drop[1] ? ignore : a.y;
+        b.x = drop[2] ? ignore : b.x; b.y = drop[3] ? ignore : b.y;
+        __builtin_nontemporal_store(a, out2);
+        __builtin_nontemporal_store(b, out2 + 1);
+        return;
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -313,7 +349,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
     return check_launch();
 }
 
-static int64_t select_workspace(int64_t P) { return align256(3 * kOhemBins * 4) + align256(ohem_tiles(P) * 4); }
+static int64_t select_workspace(int64_t P) { return align256(kOhemZeroWords * 4) + align256(ohem_tiles(P) * 4); }
 
 // The tables are needed unless the labels pass through unchanged (n_min >= P).
 static int check_workspace(const void *workspace, int64_t workspace_bytes, int64_t P, int64_t n_min) {
@@ -333,19 +369,24 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
     const int64_t tiles = ohem_tiles(P);
     OhemTables tb;
     tb.hist = static_cast<uint32_t *>(workspace);
-    tb.tile_ties = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + align256(3 * kOhemBins * 4));
+    tb.state = tb.hist + 3 * kOhemBins;
+    tb.tile_ties = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + align256(kOhemZeroWords * 4));
     const uint32_t k = n_min > 0 ? (uint32_t)n_min : 0u;
     const int Pi = (int)P;
+    // 16-byte accesses when every tensor allows them (tile bases are multiples of 4 pixels)
+    const int vec = !misaligned(scores, 16) && !misaligned(labels, 16) && !misaligned(out_labels, 16);
     if (k > 0) {
-        hipLaunchKernelGGL(ohem_zero, dim3(3 * kOhemBins / 256), dim3(256), 0, st, tb.hist, 3 * kOhemBins);
-        const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 8) < 2048 ? ceil_div(P, 256 * 8) : 2048);
-        for (int pass = 0; pass < 3; ++pass)
-            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k);
-        hipLaunchKernelGGL(ohem_count_ties, dim3((unsigned)tiles), dim3(256), 0, st, scores, tb, Pi, k, score_thresh);
-        hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, k, score_thresh);
+        hipLaunchKernelGGL(ohem_zero, dim3((kOhemZeroWords + 255) / 256), dim3(256), 0, st, tb.hist, kOhemZeroWords);
+        const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 2048 ? ceil_div(P, 256 * 16) : 2048);
+        for (int pass = 0; pass < 3; ++pass) {
+            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, vec);
+            hipLaunchKernelGGL(ohem_pick, dim3(1), dim3(256), 0, st, tb, pass, k);
+        }
+        hipLaunchKernelGGL(ohem_count_ties, dim3((unsigned)tiles), dim3(256), 0, st, scores, tb, Pi, score_thresh, vec);
+        hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, score_thresh);
     }
     hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, k,
-                       score_thresh, ignore_index);
+                       score_thresh, ignore_index, vec);
     return check_launch();
 }
 
