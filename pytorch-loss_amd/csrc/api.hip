@@ -1,5 +1,7 @@
 // Library-level entry points: ABI version, error text, and the plain copy kernel
 // used to calibrate byte counters and to measure achievable copy bandwidth.
+#include <stdlib.h>
+
 #include "plh_common.hpp"
 
 namespace plh {
@@ -16,6 +18,23 @@ __global__ __launch_bounds__(256) void stream_copy_scalar(const float *__restric
     if (i < numel) dst[i] = src[i];
 }
 
+// Run length of the XCD-aware tile permutation (tile_of_block). Measured on MI355X over six
+// segmentation shapes, both element sizes and five kernels (LSR and large-margin forward and
+// backward, OHEM scores): runs of 8..32 tiles are within 1 % of the best almost everywhere, runs of
+// 64..288 lose 3..20 % on several shapes. The one systematic exception: fp32 logits whose channel
+// plane is a multiple of 4 MiB (1024x1024, 2048x1024) run 3 % faster with runs of 1024 tiles, which
+// costs 16-bit logits of the same shapes up to 13 %, hence the element-size condition.
+// PLH_XCD_RUN=<tiles> in the environment overrides the choice (read once; a tuning aid).
+unsigned xcd_run_for(size_t elem_bytes, int64_t m_size) {
+    static const long forced = [] {
+        const char *e = getenv("PLH_XCD_RUN");
+        return e ? strtol(e, nullptr, 10) : 0L;
+    }();
+    if (forced > 0) return (unsigned)forced;
+    if (elem_bytes == 4 && m_size > 0 && (m_size * 4) % ((int64_t)4 << 20) == 0) return 1024u;
+    return 32u;
+}
+
 }  // namespace plh
 
 using namespace plh;
@@ -29,7 +48,7 @@ extern "C" const char *plh_error_string(int code) {
         case PLH_ERR_BAD_SIZE: return "negative or unsupported size";
         case PLH_ERR_BAD_STRIDE: return "grad_output_stride must be 0 (broadcast scalar) or 1 (per element)";
         case PLH_ERR_TOO_MANY_CLASSES: return "num of classes should be less than 512";
-        case PLH_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than plh_lovasz_workspace_bytes()";
+        case PLH_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than the op's plh_*_workspace_bytes()";
         case PLH_ERR_MISALIGNED: return "a pointer is not aligned to its element size";
         case PLH_ERR_BAD_DTYPE: return "dtype must be PLH_DTYPE_F32, PLH_DTYPE_F16 or PLH_DTYPE_BF16";
         default: break;

@@ -38,6 +38,7 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     p.ignore = ignore;
     p.half_lam = lam / 2.f;                          // csrc/large_margin_kernel.cu:188
     p.coeff = 1.f / (float)(dimsize - 1);            // csrc/large_margin_kernel.cu:404
+    p.xcd_run = xcd_run_for(es, m_size);
     unsigned blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);

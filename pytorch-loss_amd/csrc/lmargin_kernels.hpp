@@ -23,6 +23,7 @@ struct LmParams {
     int C;
     int64_t ignore;
     float half_lam, coeff;
+    unsigned xcd_run;   // tile permutation run length (xcd_run_for)
 };
 
 // ---------------------------------------------------------------- regs ----
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
     __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
     const bool live = at.live;
     if (!Reduce && !live) return;
     const int64_t pix = at.pix;

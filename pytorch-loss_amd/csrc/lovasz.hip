@@ -55,8 +55,8 @@ __device__ __forceinline__ float key_error(uint32_t key) {
 template <class T, int CP, int V>
 __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
-                                                           int64_t ignore) {
-    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+                                                           int64_t ignore, unsigned xcd_run) {
+    const int64_t pix = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
     const int64_t n = pix / m_size;
     const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
@@ -567,8 +567,8 @@ template <class T, int CP, int V>
 __global__ __launch_bounds__(kRegsBlock) void lov_bwd_regs(const float *__restrict__ gout, const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab, const float *__restrict__ jacc,
                                                           T *__restrict__ grad, int64_t P, int64_t m_size, int C,
-                                                          int64_t ignore) {
-    const int64_t pix = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+                                                          int64_t ignore, unsigned xcd_run) {
+    const int64_t pix = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
     if (pix >= P) return;
     const int64_t n = pix / m_size;
     const int64_t base = pix + n * (int64_t)(C - 1) * m_size;
@@ -724,13 +724,14 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                 \
     case K:                                                                                                         \
         if (vec) hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,  \
-                                    keys_b, pl.P, m_size, C, ignore_index);                                         \
+                                    keys_b, pl.P, m_size, C, ignore_index, run);                                    \
         else hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,       \
-                                keys_b, pl.P, m_size, C, ignore_index);                                             \
+                                keys_b, pl.P, m_size, C, ignore_index, run);                                        \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -817,13 +818,14 @@ extern "C" int plh_lovasz_backward(const float *grad_output, const void *logits,
         if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
         if (vec) hipLaunchKernelGGL((lov_bwd_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output,  \
-                                    x, labels, jacc, g, pl.P, m_size, C, ignore_index);                              \
+                                    x, labels, jacc, g, pl.P, m_size, C, ignore_index, run);                         \
         else hipLaunchKernelGGL((lov_bwd_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, grad_output, x,    \
-                                labels, jacc, g, pl.P, m_size, C, ignore_index);                                     \
+                                labels, jacc, g, pl.P, m_size, C, ignore_index, run);                                \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

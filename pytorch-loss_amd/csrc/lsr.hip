@@ -16,7 +16,7 @@ static int backward(const void *logits, int32_t dtype, const int64_t *labels, co
                                     dtype_size(dtype));
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
-    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         lsr_backward_typed<T>(static_cast<const T *>(logits), labels, up, static_cast<T *>(grad_logits), p,
@@ -36,7 +36,7 @@ extern "C" int plh_lsr_forward(const void *logits, int32_t dtype, const int64_t 
     const int rc = check_slice_args(logits, labels, losses, n_size, dimsize, m_size, dtype_size(dtype), 4);
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
-    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         lsr_forward_typed<T>(static_cast<const T *>(logits), labels, losses, Partials{nullptr, nullptr}, false, p,
@@ -60,7 +60,7 @@ extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const 
     hipStream_t st = (hipStream_t)stream;
     unsigned blocks = 0;
     if (n_size * dimsize * m_size != 0) {
-        const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth);
+        const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
         dispatch_dtype(dtype, [&](auto tag) {
             using T = decltype(tag);
             blocks = lsr_forward_typed<T>(static_cast<const T *>(logits), labels, losses, part, true, p, st);

@@ -23,6 +23,7 @@ struct LsrParams {
     int C;
     int64_t ignore;
     float w_pos, w_neg, sumw;
+    unsigned xcd_run;   // tile permutation run length (xcd_run_for)
 };
 
 // ---------------------------------------------------------------- regs ----
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
                                                           float *__restrict__ loss, Partials part,
                                                           const LsrParams p) {
     __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
 
     typename Pack<T, V>::Raw raw[CP];
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
                                                           const int64_t *__restrict__ lab,
                                                           const Upstream up, T *__restrict__ grad,
                                                           const LsrParams p) {
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C);
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
 
     typename Pack<T, V>::Raw raw[CP];
@@ -257,7 +258,8 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 
 // ------------------------------------------------------------ dispatch ----
 
-inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float smooth) {
+inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float smooth,
+                             size_t elem_bytes) {
     LsrParams p;
     p.P = n_size * m_size;
     p.m_size = m_size;
@@ -266,6 +268,7 @@ inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, in
     p.w_pos = 1.f - smooth;                        // csrc/lsr_kernel.cu:83
     p.w_neg = smooth / (float)dimsize;             // csrc/lsr_kernel.cu:84
     p.sumw = p.w_neg * (float)(dimsize - 1) + p.w_pos;   // csrc/lsr_kernel.cu:125
+    p.xcd_run = xcd_run_for(elem_bytes, m_size);
     return p;
 }
 

@@ -36,8 +36,8 @@ __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)(
 template <class T, int CP, int V, bool Uniform>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                               float *__restrict__ scores, int64_t P, int64_t m_size,
-                                                              int C, int64_t ignore) {
-    const PixelRef<V, Uniform> at(P, m_size, C);
+                                                              int C, int64_t ignore, unsigned xcd_run) {
+    const PixelRef<V, Uniform> at(P, m_size, C, xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, C, m_size, raw);
@@ -328,15 +328,16 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
             const bool vec = (shape == Shape::RegsVec);
             const bool uni = vec && tiles_are_uniform(m_size, VT, sizeof(T));
             const unsigned grid = vec ? regs_grid<VT>(P) : regs_grid<1>(P);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
         if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                                    labels, scores, P, m_size, C, ignore_index);                                      \
+                                    labels, scores, P, m_size, C, ignore_index, run);                                 \
         else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, false>), dim3(grid), dim3(kRegsBlock), 0,    \
-                                         st, x, labels, scores, P, m_size, C, ignore_index);                          \
+                                         st, x, labels, scores, P, m_size, C, ignore_index, run);                     \
         else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, false>), dim3(grid), dim3(kRegsBlock), 0, st, x,       \
-                                labels, scores, P, m_size, C, ignore_index);                                          \
+                                labels, scores, P, m_size, C, ignore_index, run);                                     \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

@@ -378,22 +378,24 @@ void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int
 
 // ---- the "regs" launch shape ---------------------------------------------------
 // 256 threads per block, V pixels per thread; block b of the grid owns the pixel tile
-// tile_of(b). Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; the
-// tile order is permuted so that each XCD walks runs of kXcdRun consecutive tiles: every
-// XCD (own L2, own slice of the fabric) then streams a few contiguous address ranges per
-// tensor instead of every eighth kilobyte of all of them. Measured on the LSR backward at
-// (8,19,1024,1024): 5.4 -> 6.1 TB/s.
+// tile_of_block(run). Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; the
+// tile order is permuted so that each XCD walks runs of `run` consecutive tiles: every XCD
+// (own L2, own slice of the fabric) then streams contiguous address ranges per tensor instead
+// of every eighth tile of all of them. The run length is chosen on the host (xcd_run_for).
 constexpr int kRegsBlock = 256;
 constexpr int kXcds = 8;
-constexpr int kXcdRun = 256;
 
-__device__ __forceinline__ int64_t tile_of_block() {
+// Run length (in tiles) of the permutation; see xcd_run_for() for how the host picks it.
+__device__ __forceinline__ int64_t tile_of_block(unsigned run) {
     const unsigned b = blockIdx.x;
-    const unsigned span = kXcds * kXcdRun;
+    const unsigned span = kXcds * run;
     const unsigned sup = b / span, in = b % span;
-    if ((sup + 1) * span <= gridDim.x) return (int64_t)sup * span + (in % kXcds) * kXcdRun + in / kXcds;
+    if ((sup + 1) * span <= gridDim.x) return (int64_t)sup * span + (in % kXcds) * run + in / kXcds;
     return b;   // ragged tail of the grid keeps its natural order
 }
+
+// Defined in api.hip.
+unsigned xcd_run_for(size_t elem_bytes, int64_t m_size);
 
 // Raw buffer descriptor over [p, p + 4 GiB): no stride, no swizzle, 32-bit data format.
 constexpr int kBufferNT = 2;      // non-temporal hint of buffer loads / stores
@@ -418,16 +420,16 @@ struct PixelRef {
     unsigned lane_off;  // 32-bit per-thread part (Uniform), else 0
     bool live;
 
-    __device__ __forceinline__ PixelRef(int64_t P, int64_t m_size, int C) {
+    __device__ __forceinline__ PixelRef(int64_t P, int64_t m_size, int C, unsigned xcd_run) {
         if constexpr (Uniform) {
-            const int64_t start = tile_of_block() * (kRegsBlock * V);
+            const int64_t start = tile_of_block(xcd_run) * (kRegsBlock * V);
             const int64_t n = start / m_size;
             lane_off = threadIdx.x * V;
             base = start + n * (int64_t)(C - 1) * m_size;
             pix = start + lane_off;
             live = true;
         } else {
-            const int64_t want = (tile_of_block() * kRegsBlock + threadIdx.x) * V;
+            const int64_t want = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
             live = want < P;
             pix = live ? want : 0;
             const int64_t n = pix / m_size;
