@@ -52,12 +52,39 @@ __device__ __forceinline__ float key_error(uint32_t key) {
 
 // ------------------------------------------------------ 1. build keys ----
 
+// Besides the keys, both kernels leave per block and class the largest key among the block's
+// positives of that class, plus 1 (0 = none), in block_table[block][C]; lov_class_max folds the
+// table into pos_max[c], the error of the class's lowest-ranked positive. Everything sorted after
+// that one has a Jaccard difference of exactly 0 (see keep_key), so the sort never sees it.
+__device__ __forceinline__ void publish_block_max(const uint32_t *block_max, uint32_t *block_table, int C) {
+    uint32_t *row = block_table + (int64_t)blockIdx.x * C;
+    for (int j = threadIdx.x; j < C; j += blockDim.x) row[j] = block_max[j];
+}
+
+__global__ __launch_bounds__(256) void lov_class_max(const uint32_t *__restrict__ block_table, int blocks, int C,
+                                                     uint32_t *__restrict__ pos_max) {
+    __shared__ uint32_t wave_max[4];
+    const int c = blockIdx.x;
+    uint32_t m = 0;
+    for (int b = threadIdx.x; b < blocks; b += 256) m = max(m, block_table[(int64_t)b * C + c]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, 64));
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) pos_max[c] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+}
+
 template <class T, int CP, int V>
 __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
-                                                           uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
+                                                           uint32_t *__restrict__ keys, uint32_t *__restrict__ block_table,
+                                                           int64_t P, int64_t m_size, int C,
                                                            int64_t ignore, unsigned xcd_run) {
-    const int64_t pix = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
-    if (pix >= P) return;
+    __shared__ uint32_t block_max[kMaxRegsChannels];
+    if (threadIdx.x < kMaxRegsChannels) block_max[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t want = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
+    const bool live = want < P;
+    const int64_t pix = live ? want : 0;
     const int64_t n = pix / m_size;
     const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
     float v[CP][V];
@@ -80,20 +107,36 @@ __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict_
                 s += v[j][k];
             }
         const bool ign = (lb[k] == ignore);
+        uint32_t key_y = 0;                     // the positive's key, if the pixel has one
+        bool has_y = false;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, C)) v[j][k] = __builtin_bit_cast(float, make_key(v[j][k] / s, lb[k] == j, ign));
+            if (chan_ok<CP>(j, C)) {
+                const bool hot = (lb[k] == j);
+                const uint32_t key = make_key(v[j][k] / s, hot, ign);
+                key_y = hot ? key : key_y;
+                has_y = has_y || hot;
+                v[j][k] = __builtin_bit_cast(float, key);
+            }
+        if (live && !ign && has_y) atomicMax(&block_max[(int)lb[k]], (key_y & 0x7FFFFFFFu) + 1u);
     }
+    if (live) {
 #pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (chan_ok<CP>(j, C)) store_vec<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, C)) store_vec<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
+    }
+    __syncthreads();
+    publish_block_max(block_max, block_table, C);
 }
 
 // Any channel count: a lane per pixel, three sweeps over the slice (the later ones hit cache).
 template <class T>
 __global__ __launch_bounds__(256) void lov_keys_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
-                                                     uint32_t *__restrict__ keys, int64_t P, int64_t m_size, int C,
-                                                     int64_t ignore) {
+                                                     uint32_t *__restrict__ keys, uint32_t *__restrict__ block_table,
+                                                     int64_t P, int64_t m_size, int C, int64_t ignore) {
+    __shared__ uint32_t block_max[512];              // C < 512
+    for (int j = threadIdx.x; j < C; j += 256) block_max[j] = 0;
+    __syncthreads();
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t n = pix / m_size;
         const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
@@ -102,9 +145,14 @@ __global__ __launch_bounds__(256) void lov_keys_lane(const T *__restrict__ x, co
         for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
         for (int j = 0; j < C; ++j) s += expf(load_one(xs + (int64_t)j * m_size) - mx);
-        for (int j = 0; j < C; ++j)
-            keys[(int64_t)j * P + pix] = make_key(expf(load_one(xs + (int64_t)j * m_size) - mx) / s, lb == j, lb == ignore);
+        for (int j = 0; j < C; ++j) {
+            const uint32_t key = make_key(expf(load_one(xs + (int64_t)j * m_size) - mx) / s, lb == j, lb == ignore);
+            keys[(int64_t)j * P + pix] = key;
+            if (lb == j && lb != ignore) atomicMax(&block_max[j], (key & 0x7FFFFFFFu) + 1u);
+        }
     }
+    __syncthreads();
+    publish_block_max(block_max, block_table, C);
 }
 
 // --------------------------------------------------- 2. radix sort pass ----
@@ -118,11 +166,30 @@ struct SortArgs {
     uint32_t *digit_total;       // [C][kRadix]: keys per digit
     uint32_t *tile_hot;          // last pass only: the same two tables for the positives
     uint32_t *hot_total;
-    int P;                       // keys per class row
+    const uint32_t *pos_max;     // first pass only: per class, largest positive key + 1 (see keep_key)
+    const uint32_t *kept_in;     // later passes: keys per class that the first pass let through
+    uint32_t *kept_out;          // first pass: where that count goes
+    int P;                       // row stride; keys per class row in the first pass
     int tiles;                   // ceil(P / kSortTile)
     int shift;                   // 0, 8, 16, 24
     uint32_t digit_mask;         // 0xFF, or 0x7F for the top digit (bit 31 is the positive flag)
 };
+
+// A key takes part in the sort iff its error is not below that of the class's lowest-ranked positive
+// (error bits of the key <= limit). What is left out would be sorted after every positive, where
+// the intersection is empty: J = 1 - 0/(k+1) = 1 on both sides of the difference, so its Jaccard
+// difference is exactly 0 and it adds exactly 0 to the loss; lov_unbin writes those zeros. Ignored
+// pixels (error bits 0x7FFFFFFF) are always left out. A class without positives keeps every valid
+// key. Keys equal to the limit stay in, so ties with the last positive keep their pixel order.
+__device__ __forceinline__ uint32_t keep_limit(const uint32_t *pos_max, int c) {
+    if (!pos_max) return 0x7FFFFFFFu;            // later passes: everything that is there takes part
+    const uint32_t m = pos_max[c];
+    return m ? m - 1u : kOne;
+}
+__device__ __forceinline__ bool keep_key(uint32_t key, uint32_t limit) { return (key & 0x7FFFFFFFu) <= limit; }
+
+// Keys of class c that enter this pass.
+__device__ __forceinline__ int row_items(const SortArgs &a, int c) { return a.kept_in ? (int)a.kept_in[c] : a.P; }
 
 // Inclusive scan over the 64 lanes of a wave.
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
@@ -211,7 +278,15 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         if constexpr (Hot) (&counts_hot[0][0])[i] = 0;
     }
     const int begin = tile * kSortTile;
-    const int count = min(kSortTile, a.P - begin);
+    const int count = min(kSortTile, row_items(a, c) - begin);
+    if (count <= 0) {                           // block-uniform: the row ends before this tile
+        if (threadIdx.x < kRadix) {
+            a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile] = 0;
+            if constexpr (Hot) a.tile_hot[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile] = 0;
+        }
+        return;
+    }
+    const uint32_t limit = keep_limit(a.pos_max, c);
     const uint32_t *kin = a.keys_in + (int64_t)c * a.P + begin;
     uint32_t key[kSortItems];
 #pragma unroll
@@ -223,10 +298,28 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
-        const bool valid = li < count;
+        const bool valid = li < count && keep_key(key[r], limit);
         const uint32_t digit = (key[r] >> a.shift) & a.digit_mask;
         const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
         if (vmask == 0) continue;               // wave-uniform
+        if constexpr (Hot) {
+            // top digit: a wave holds a handful of distinct values, so one lane adds each group's size
+            // (per-lane atomics on two or three addresses would serialise)
+            const uint64_t hmask = __builtin_amdgcn_ballot_w64(valid && (key[r] >> 31));
+            uint64_t remaining = vmask;
+            while (remaining) {                 // wave-uniform
+                const int leader = __builtin_ffsll((long long)remaining) - 1;
+                const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)digit, leader);
+                const uint64_t same = __builtin_amdgcn_ballot_w64(valid && digit == dl);
+                if (lane == 0) {
+                    atomicAdd(&counts[wave][dl], (uint32_t)__builtin_popcountll(same));
+                    const uint64_t hs = same & hmask;
+                    if (hs) atomicAdd(&counts_hot[wave][dl], (uint32_t)__builtin_popcountll(hs));
+                }
+                remaining &= ~same;
+            }
+            continue;
+        }
         const uint32_t first = __builtin_amdgcn_readfirstlane(digit);   // first active lane = lowest valid one here
         const uint64_t same = __builtin_amdgcn_ballot_w64(valid && digit == first);
         if (same == vmask) {                    // wave-uniform branch
@@ -298,15 +391,18 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 
     const int c = blockIdx.y, tile = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, row_items(a, c) - begin);
+    if (count <= 0) return;                     // block-uniform: the row ends before this tile
     for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
     __syncthreads();
 
-    const int begin = tile * kSortTile;
-    const int count = min(kSortTile, a.P - begin);
+    const uint32_t limit = keep_limit(a.pos_max, c);
     const int64_t row = (int64_t)c * a.P;
     const uint32_t *kin = a.keys_in + row + begin;
     const uint32_t *vin = a.vals_in ? a.vals_in + row + begin : nullptr;
 
+    // keys beyond the row's end read as ignored, which keep_key never lets through
     uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
@@ -319,10 +415,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         uint32_t unused;
-        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, li < count, false, counts[wave], nullptr, rank[r], unused);
+        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, li < count && keep_key(key[r], limit), false, counts[wave],
+                         nullptr, rank[r], unused);
     }
     __syncthreads();
 
+    uint32_t n_local;                           // keys of this tile that take part
     {
         uint32_t mine = 0, dtot = 0;
         const int d = threadIdx.x;
@@ -337,20 +435,22 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
             mine = run;
             dtot = a.digit_total[(int64_t)c * kRadix + d];
         }
-        uint32_t total;
-        const uint32_t local_start = block_excl_scan(mine, scan_tmp, total);
-        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, total);
+        uint32_t row_total;
+        const uint32_t local_start = block_excl_scan(mine, scan_tmp, n_local);
+        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, row_total);
         if (d < kRadix) {
             digit_start[d] = local_start;
             out_base[d] = global_start + a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
         }
+        // the digit totals of the row add up to the keys this pass lets through
+        if (a.kept_out && tile == 0 && threadIdx.x == 0) a.kept_out[c] = row_total;
     }
     __syncthreads();
 
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
-        if (li < count) {
+        if (li < count && keep_key(key[r], limit)) {
             const uint32_t d = (key[r] >> a.shift) & a.digit_mask;
             const uint32_t pos = digit_start[d] + counts[wave][d] + rank[r];
             s_keys[pos] = key[r];
@@ -361,7 +461,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 
     uint32_t *kout = a.keys_out + row;
     uint32_t *vout = a.vals_out + row;
-    for (int i = threadIdx.x; i < count; i += kSortThreads) {
+    for (int i = threadIdx.x; i < (int)n_local; i += kSortThreads) {
         const uint32_t k = s_keys[i];
         const uint32_t d = (k >> a.shift) & a.digit_mask;
         const uint32_t dst = out_base[d] + ((uint32_t)i - digit_start[d]);
@@ -406,6 +506,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 
     const int c = blockIdx.y, tile = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int begin = tile * kSortTile;
+    const int count = min(kSortTile, row_items(a, c) - begin);
+    if (count <= 0) {                           // block-uniform: the row ends before this tile
+        if (threadIdx.x == 0) tile_loss[(int64_t)c * a.tiles + tile] = 0.f;
+        return;
+    }
     for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
         (&counts[0][0])[i] = 0;
         (&counts_hot[0][0])[i] = 0;
@@ -414,8 +520,6 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
     __syncthreads();
 
-    const int begin = tile * kSortTile;
-    const int count = min(kSortTile, a.P - begin);
     const int64_t row = (int64_t)c * a.P;
     const uint32_t *kin = a.keys_in + row + begin;
     const uint32_t *vin = a.vals_in + row + begin;
@@ -533,15 +637,23 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     }
 }
 
-// One block per (region, class): the region's staged values are permuted to pixel order inside LDS.
+// One block per (region, class): the region's staged values (as many as its cursor counted) are
+// permuted to pixel order inside LDS; pixels whose keys stayed out of the sort get their exact 0.
 __global__ __launch_bounds__(256) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
-                                                 int P) {
+                                                 const uint32_t *__restrict__ cursors, int regions, int P) {
     __shared__ float sorted[kRegion];
     const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
     const int n = min(kRegion, P - (int)(blockIdx.x << kRegionBits));
-    for (int i = threadIdx.x; i < n; i += 256) sorted[idx_stage[first + i]] = jacc[first + i];
+    const int staged = min(n, (int)cursors[(int64_t)blockIdx.y * regions + blockIdx.x]);
+    for (int i = threadIdx.x; i < n; i += 256) sorted[i] = 0.f;
+    __syncthreads();
+    for (int i = threadIdx.x; i < staged; i += 256) sorted[idx_stage[first + i] & (kRegion - 1)] = jacc[first + i];
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += 256) jacc[first + i] = sorted[i];
+}
+
+__global__ __launch_bounds__(256) void lov_zero_f32(float *p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
 }
 
 __global__ __launch_bounds__(256) void lov_zero_u32(uint32_t *p, int n) {
@@ -649,7 +761,7 @@ struct LovaszPlan {
     int tiles;
     int regions;            // pixel regions per class row (0 = direct scatter)
     int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss,
-        off_cursors, bytes;
+        off_cursors, off_class, off_block_max, bytes;
 };
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -674,6 +786,8 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     const int64_t regions = ceil_div(pl.P, kRegion);
     pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
+    pl.off_class = off;       off += round_up(4 * dimsize * 2, 256);      // pos_max[C], kept[C]
+    pl.off_block_max = off;   off += round_up(4 * dimsize * ceil_div(pl.P, 256), 256);   // [key blocks][C]
     pl.bytes = off;
     return PLH_OK;
 }
@@ -713,7 +827,12 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     uint32_t *digit_total = reinterpret_cast<uint32_t *>(ws + pl.off_digit_total);
     uint32_t *hot_total = reinterpret_cast<uint32_t *>(ws + pl.off_hot_total);
     float *tile_loss = reinterpret_cast<float *>(ws + pl.off_tile_loss);
+    uint32_t *pos_max = reinterpret_cast<uint32_t *>(ws + pl.off_class);
+    uint32_t *kept = pos_max + dimsize;
     const int C = (int)dimsize;
+
+    uint32_t *block_table = reinterpret_cast<uint32_t *>(ws + pl.off_block_max);
+    unsigned key_blocks = 0;
 
     // 1. keys (into keys_b = jacc: rows of [C][P] u32; a row start stays 8-/16-byte aligned when P % V == 0)
     dispatch_dtype(dtype, [&](auto tag) {
@@ -725,25 +844,30 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
             const bool vec = (shape == Shape::RegsVec);
             const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
             const unsigned run = xcd_run_for(sizeof(T), m_size);
+            key_blocks = grid;
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                 \
     case K:                                                                                                         \
         if (vec) hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,  \
-                                    keys_b, pl.P, m_size, C, ignore_index, run);                                    \
+                                    keys_b, block_table, pl.P, m_size, C, ignore_index, run);                       \
         else hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,       \
-                                keys_b, pl.P, m_size, C, ignore_index, run);                                        \
+                                keys_b, block_table, pl.P, m_size, C, ignore_index, run);                           \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
         } else {
-            hipLaunchKernelGGL(lov_keys_lane<T>, dim3(group_grid(pl.P, 256)), dim3(256), 0, st, x, labels, keys_b, pl.P,
-                               m_size, C, ignore_index);
+            key_blocks = group_grid(pl.P, 256);
+            hipLaunchKernelGGL(lov_keys_lane<T>, dim3(key_blocks), dim3(256), 0, st, x, labels, keys_b, block_table,
+                               pl.P, m_size, C, ignore_index);
         }
     });
+    hipLaunchKernelGGL(lov_class_max, dim3((unsigned)C), dim3(256), 0, st, block_table, (int)key_blocks, C, pos_max);
 
     // 2. three stable radix passes: (keys_b, -) -> (keys_a, vals_a) -> (keys_b, vals_b) -> (keys_a, vals_a).
-    //    keys_b is the jacc output buffer, free until the last pass scatters into it
+    //    keys_b is the jacc output buffer, free until the last pass scatters into it. The first pass
+    //    drops the keys whose Jaccard difference is known to be 0 (keep_key) and counts what is left
+    //    per class; the later passes work on those counts and their surplus blocks return at once.
     const dim3 tile_grid((unsigned)pl.tiles, (unsigned)C);
     SortArgs a;
     a.tile_hist = hist;
@@ -760,6 +884,9 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         a.vals_out = even ? vals_a : vals_b;
         a.shift = 8 * pass;
         a.digit_mask = 0xFFu;
+        a.pos_max = (pass == 0) ? pos_max : nullptr;
+        a.kept_in = (pass == 0) ? nullptr : kept;
+        a.kept_out = (pass == 0) ? kept : nullptr;
         hipLaunchKernelGGL(lov_tile_hist<false>, tile_grid, dim3(kSortThreads), 0, st, a);
         hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 1), dim3(256), 0, st, hist, digit_total, hot,
                            hot_total, pl.tiles);
@@ -774,6 +901,9 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     a.vals_out = nullptr;
     a.shift = 24;
     a.digit_mask = 0x7Fu;
+    a.pos_max = nullptr;
+    a.kept_in = kept;
+    a.kept_out = nullptr;
     hipLaunchKernelGGL(lov_tile_hist<true>, tile_grid, dim3(kSortThreads), 0, st, a);
     hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
                        pl.tiles);
@@ -785,8 +915,11 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
                            pl.regions);
         hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(256), 0, st, jacc, vals_b,
-                           (int)pl.P);
+                           cursors, pl.regions, (int)pl.P);
     } else {
+        // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
+        // (jacc stopped being a key buffer when the third pass read it)
+        hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, jacc, pl.E);
         hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, nullptr,
                            0);
     }
