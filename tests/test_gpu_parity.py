@@ -345,6 +345,50 @@ def test_lovasz_jacc_is_exact_for_the_computed_order(pl):
     np.testing.assert_allclose(l32, l64, rtol=1e-4)
 
 
+@pytest.mark.parametrize("case", ["confident", "one_positive", "absent_and_present", "ties_at_the_limit"])
+def test_lovasz_keys_left_out_of_the_sort_get_exact_zeros(pl, case):
+    """The kernels sort only the keys that can have a non-zero Jaccard difference (those not ranked
+    after the class's last positive).  What they leave out must come back as exact zeros, and what
+    they keep must match the oracle, which sorts everything."""
+    from pytorch_loss import _native
+    shape = (2, 6, 96, 96)
+    x, y = seg_inputs(53, shape, 255, 0.1)
+    if case == "confident":                      # a trained model: the label's logit dominates
+        onehot = (np.arange(shape[1])[None, :, None, None] == np.where(y == 255, 0, y)[:, None]).astype(np.float32)
+        x = (x * 0.5 + 6.0 * onehot).astype(np.float32)
+    elif case == "one_positive":                 # class 5 has a single, well classified pixel
+        y[y == 5] = 4
+        y[0, 3, 7] = 5
+        x[0, 5, 3, 7] = 9.0
+    elif case == "absent_and_present":           # classes 4 and 5 never occur
+        y[(y == 4) | (y == 5)] = 1
+    elif case == "ties_at_the_limit":            # identical pixels: every error is tied with the last positive's
+        x[:] = x[0:1, :, 0:1, 0:1]
+    losses, jacc = _native.lovasz_forward(dev(x), dev(y), 255)
+    jacc = jacc.cpu().numpy()
+    l64, j64 = oracle.lovasz_forward(x.astype(np.float64), y, 255)
+    _, j32 = oracle.lovasz_forward(x, y, 255)
+    np.testing.assert_allclose(losses.cpu().numpy(), l64, rtol=1e-5, atol=1e-7)
+    # wherever the oracle's difference is an exact zero the kernel's must be too, and vice versa
+    # (up to near-tie reorderings, which never cross the zero / non-zero boundary by more than a pixel)
+    assert ((jacc == 0) != (j32 == 0)).mean() < 1e-3
+    if case != "ties_at_the_limit":              # with all-equal errors the order is pixel order in both
+        same = (jacc.view(np.uint32) == j32.view(np.uint32)).mean()
+        assert same > 0.99, same
+    else:
+        assert np.array_equal(jacc.view(np.uint32), j32.view(np.uint32))
+    np.testing.assert_allclose(jacc.sum(axis=1), 1.0, rtol=1e-4)
+    if case == "confident":
+        assert (jacc == 0).mean() > 0.15          # a good part of the keys was not sorted at all
+    # gradient through the public surface
+    xt = dev(x).requires_grad_()
+    out = pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255)(xt, dev(y))
+    out.backward()
+    want_g = oracle.lovasz_backward(np.full(shape[1], 1.0 / shape[1]), x.astype(np.float64), y, j64, 255)
+    err = np.abs(xt.grad.cpu().numpy() - want_g)
+    assert np.median(err) <= 1e-7 and err.max() <= max(GRAD_ATOL, 2e-3 * np.abs(j64).max() / shape[1]), err.max()
+
+
 @pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
 def test_lovasz_module_reductions(pl, reduction):
     w = synth.workload("cfg5", scale=1 / 16, batch=2)
