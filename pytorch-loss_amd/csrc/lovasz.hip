@@ -9,20 +9,24 @@
 //   d_ic = (c == y_i ? -1 : +1) * jacc[c,i] * grad_out[c];  g_ic = p_ic * (d_ic - sum_k p_ik d_ik)
 //
 // Pipeline (all launches on the caller's stream, nothing allocated here):
-//   1. build_keys     one pass over the logits: softmax in registers, one 32-bit key per
+//   1. keys           one pass over the logits: softmax in registers, one 32-bit key per
 //                     (class, pixel):  bit 31 = positive flag, bits 0..30 = 0x3F800000 - bits(e)
 //                     (ascending key order = descending error; e lies in [0,1] so its bit
-//                     pattern is monotone), ignored pixel = 0x7FFFFFFF (sorts last).
-//   2. 4 x (tile_hist, offsets_scan, scatter): stable LSD radix sort, 8 bits per pass, batched
-//                     over classes with blockIdx.y. Ranking inside a tile is done per wavefront
-//                     with ballot-built match masks, tiles are re-ordered in LDS so that the
-//                     global writes are runs of consecutive addresses. The positive flag rides
-//                     along in bit 31 and is masked out of the top digit; the payload (pixel
-//                     index) is generated from the position in the first pass.
-//   3. count_pos + scan_tiles: positives per tile, exclusive scan over tiles, n_pos per class.
-//   4. jaccard        cumulative positives -> J, dJ, per-tile partial of the loss, dJ scattered
-//                     to pixel order.
-//   5. reduce_loss    fixed-order sum of the per-tile partials (no floating-point atomics, so
+//                     pattern is monotone), ignored pixel = 0x7FFFFFFF (sorts last). Also the
+//                     largest positive key per class (per-block table + lov_class_max): keys
+//                     beyond it have dJ = 0 exactly and are left out of the sort (keep_key).
+//   2. 3 x (tile_hist, row_scan, scatter): stable LSD radix passes, 8 bits each, batched over
+//                     classes with blockIdx.y. Ranking inside a tile is done per wavefront with
+//                     ballot-built match masks, tiles are re-ordered in LDS so that the global
+//                     writes are runs of consecutive addresses. The positive flag rides along in
+//                     bit 31; the payload (pixel index) is generated from the position in the
+//                     first pass, which also drops the keys that take no part and counts the rest.
+//   3. tile_hist<hot>, row_scan, final: the last (top-digit) pass is not written out: a key's
+//                     destination is its rank k, the positives counted the same way give cs_k,
+//                     so J, dJ and the tile's share of the loss follow at once; dJ goes to
+//                     pixel order through region-binned staging (final) and an in-LDS permute
+//                     per region (unbin), which also writes the zeros of the keys left out.
+//   4. reduce_loss    fixed-order sum of the per-tile partials (no floating-point atomics, so
 //                     results are deterministic).
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
 #include "plh_common.hpp"
