@@ -42,6 +42,8 @@ WORKLOADS = {
                   "Bernoulli(0.02) labels, alpha=0.25 gamma=2, mean"),
     "lovasz": dict(shape=(4, 19, 512, 1024), desc="LovaszSoftmaxV3 fwd+bwd, fp32 logits (4,19,512,1024), "
                    "Zipf(1.1) int64 labels 5% ignore=255, mean"),
+    "onehot": dict(shape=(8, 19, 1024, 1024), desc="OnehotEncoder forward, int64 labels (8,1024,1024) 5% ignore=255 -> "
+                   "fp32 (8,19,1024,1024), lb_smooth=0.1"),
     "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
                  "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }
@@ -298,8 +300,39 @@ def cpu_baseline(name, shape):
                       "images of the workload, fwd+bwd, median of 3, time scaled x%d" % (scale, scale)}
 
 
+def run_onehot(steps, warmup, device):
+    """The target encoder is a forward-only write stream: labels (8,1024,1024) -> fp32 (8,19,1024,1024)."""
+    import torch
+    import pytorch_loss as pl
+    from pytorch_loss import _native
+    shape = WORKLOADS["onehot"]["shape"]
+    _, labels = make_inputs("lsr", shape, device)
+    enc = pl.OnehotEncoder(shape[1], lb_smooth=0.1, ignore_idx=255, check=False)
+    for _ in range(warmup):
+        enc(labels)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = enc(labels)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    nbytes = 4 * numel(shape) + 8 * labels.numel()
+    lib = _native.load()
+    n, c, m = shape[0], shape[1], labels.numel() // shape[0]
+    k_ms = time_kernel(lambda: lib.plh_onehot(_native._ptr(labels), _native._ptr(out), None, n, c, m, 255, 0.1,
+                                               _native._stream()))
+    gbps = nbytes / (k_ms * 1e-3) / 1e9
+    roof = {"encode": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(k_ms, 4),
+                       "algorithmic_bytes": nbytes}}
+    return dict(ms_per_step=ms, gbps=nbytes / (ms * 1e-3) / 1e9, loss=float(out[0, 0, 0, 0].item()), roofline=roof,
+                bytes=nbytes, step_ms={"warm": {"median": round(ms, 4), "iters": steps, "input_sets": 1}})
+
+
 def run_workload(name, steps, warmup, device, dtype="f32"):
     import torch
+    if name == "onehot":
+        return run_onehot(max(steps, 20), warmup, device)
     shape = WORKLOADS[name]["shape"]
     logits, labels = make_inputs(name, shape, device, dtype=dtype)
     crit = make_criterion(name)
@@ -384,9 +417,9 @@ def main():
         "config": {"workload": describe(name, args.dtype), "storage_dtype": args.dtype,
                    "algorithmic_bytes_per_step": main_res["bytes"],
                    "frac_of_hbm_peak": round(main_res["gbps"] / HBM_PEAK_GBPS, 4), "loss": main_res["loss"]},
-        "roofline": dict(main_res["roofline"].get("backward") or main_res["roofline"]["relabel"],
+        "roofline": dict(main_res["roofline"].get("backward") or list(main_res["roofline"].values())[0],
                          kernel="backward entry point of the workload" if "backward" in main_res["roofline"]
-                         else "plh_ohem_score_label"),
+                         else "the workload's single entry point"),
         "roofline_forward": main_res["roofline"].get("forward"),
         "step_ms": main_res["step_ms"],
         "copy_kernel_GBps": ceiling,

@@ -221,6 +221,19 @@ int plh_ohem_score_label(const void *logits, int32_t dtype, const int64_t *label
                          int64_t n_size, int64_t dimsize, int64_t m_size,
                          int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
 
+/* ---- one-hot / label-smoothed targets -------------------------------------------------
+ * Replaces one_hot_cpp.label_one_hot (csrc/one_hot_kernel.cu:265-350).
+ * labels (n_size, m_size) int64 -> one_hot (n_size, dimsize, m_size) fp32: 0 in every channel of an
+ * ignored pixel, else 1 - smooth at the label and smooth / dimsize elsewhere (:305-306).
+ * range_flags: NULL, or two int32 in device memory that the call clears and then sets:
+ *   [0] = 1 if some non-ignored label is >= dimsize, [1] = 1 if some is negative
+ * (the reference finds max and min and synchronises to refuse such input, :301-304; here the
+ * caller decides when to look). Labels outside [0, dimsize) match no channel and address nothing.
+ */
+int plh_onehot(const int64_t *labels, float *one_hot, int32_t *range_flags,
+               int64_t n_size, int64_t dimsize, int64_t m_size,
+               int64_t ignore_index, float smooth, void *stream);
+
 /* ---- measurement aid ----------------------------------------------------------------
  * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,
  * 4*numel written), used to calibrate hardware byte counters and to measure the

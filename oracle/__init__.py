@@ -201,6 +201,19 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
     return ohem_select(ohem_scores(logits, labels, ignore_index), labels, ignore_index, score_thresh, n_min)
 
 
+def onehot(labels, n_classes, smooth=0.0, ignore_index=-1, dtype=np.float32):
+    """(N, *) int labels -> (N, n_classes, *) targets: 1 - smooth at the label, smooth / n_classes
+    elsewhere, all zeros at ignored pixels (csrc/one_hot_kernel.cu:231-261, 305-306)."""
+    labels = np.ascontiguousarray(labels, dtype=np.int64)
+    n = int(labels.shape[0]) if labels.ndim else 1
+    m = int(labels.size // max(1, n))
+    out = np.zeros((n, n_classes) + tuple(labels.shape[1:]), dtype=dtype)
+    if labels.size:
+        _call("oracle_onehot" + ("_f32" if dtype == np.float32 else "_f64"), _ptr(labels), _ptr(out), i64(n),
+              i64(n_classes), i64(m), i64(ignore_index), f64(smooth))
+    return out
+
+
 # ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
 # large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
 

@@ -3,7 +3,7 @@
     from pytorch_loss import LabelSmoothSoftmaxCEV3, FocalLossV3, LargeMarginSoftmaxV3, LovaszSoftmaxV3
 
 Plus the relabelling step in front of that path in segmentation training, ``OhemCELoss`` /
-``OhemLargeMarginLoss``. Only this path is provided; the kernels live in libpytorch_loss_hip.so (built by
+``OhemLargeMarginLoss``, and the target encoder ``OnehotEncoder``. Only this path is provided; the kernels live in libpytorch_loss_hip.so (built by
 ``python pytorch-loss_amd/build.py``) and there is no CPU fallback.
 """
 from .label_smooth import LabelSmoothSoftmaxCEV3, LSRCrossEntropyFunctionV3
@@ -11,6 +11,7 @@ from .focal_loss import FocalLossV3, FocalSigmoidLossFuncV3, FocalSigmoidLossFun
 from .large_margin_softmax import LargeMarginSoftmaxV3, LargeMarginSoftmaxFuncV3, LargeMarginSoftmaxFuncV3FB
 from .lovasz_softmax import LovaszSoftmaxV3, LovaszSoftmaxFunctionV3
 from .ohem_loss import OhemCELoss, OhemLargeMarginLoss, score_ohem_label
+from .one_hot import convert_to_one_hot, convert_to_one_hot_cu, OnehotEncoder
 
 __all__ = [
     "LabelSmoothSoftmaxCEV3", "LSRCrossEntropyFunctionV3",
@@ -18,4 +19,5 @@ __all__ = [
     "LargeMarginSoftmaxV3", "LargeMarginSoftmaxFuncV3", "LargeMarginSoftmaxFuncV3FB",
     "LovaszSoftmaxV3", "LovaszSoftmaxFunctionV3",
     "OhemCELoss", "OhemLargeMarginLoss", "score_ohem_label",
+    "convert_to_one_hot", "convert_to_one_hot_cu", "OnehotEncoder",
 ]

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "plh_ohem_scores": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "plh_ohem_select_labels": (ctypes.c_int, [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _i64, _p]),
     "plh_ohem_score_label": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _p]),
+    "plh_onehot": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
 
@@ -481,6 +482,31 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
     ws, ws_bytes = _ohem_workspace(n_pixels, a.x.device)
     _call(a.x, "plh_ohem_score_label", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(out), _ptr(scores), _ptr(ws), ws_bytes,
           a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
+    return out
+
+
+# -------------------------------------------------------------- one-hot ----
+
+def onehot(labels, n_classes, smooth, ignore_index, check=True):
+    """(N, *) int64 labels -> (N, n_classes, *) fp32 targets. check=True reads the two range flags
+    back (one small device-to-host copy, as the reference's max/min test does) and raises."""
+    _require_gpu("onehot method", labels)
+    if labels.dtype != torch.int64:
+        raise RuntimeError("label_one_hot: date type should be kLong")      # csrc/one_hot_kernel.cu:271
+    lb = labels.contiguous()
+    n_size = int(lb.shape[0]) if lb.dim() else 1
+    m_size = lb.numel() // max(1, n_size)
+    shape = (n_size, int(n_classes)) + tuple(lb.shape[1:])
+    out = torch.empty(shape, dtype=torch.float32, device=lb.device)
+    flags = torch.empty((2,), dtype=torch.int32, device=lb.device) if check else None
+    _call(lb, "plh_onehot", _ptr(lb), _ptr(out), _ptr(flags), n_size, int(n_classes), m_size, int(ignore_index),
+          float(smooth))
+    if check:
+        too_big, negative = flags.tolist()
+        if too_big:
+            raise RuntimeError("label should be less than min_len")           # csrc/one_hot_kernel.cu:301
+        if negative:
+            raise RuntimeError("label should be more than 0")                 # csrc/one_hot_kernel.cu:302
     return out
 
 

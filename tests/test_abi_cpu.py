@@ -104,6 +104,13 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_ohem_score_label(p, 0, lp, lp, p, None, 0, 1, 2, 2, 255, 0.7, 1, None) == -5
     assert lib.plh_ohem_score_label(p, 0, lp, lp, p, ctypes.c_void_p(wsp.value + 8), ohem_need, 1, 2, 2, 255, 0.7, 1,
                                     None) == -5                                  # misaligned workspace
+    # one-hot encoder
+    assert lib.plh_onehot(None, None, None, 0, 19, 16, 255, 0.1, None) == 0
+    assert lib.plh_onehot(lp, None, None, 1, 2, 2, 255, 0.1, None) == -1
+    assert lib.plh_onehot(None, p, None, 1, 2, 2, 255, 0.1, None) == -1
+    assert lib.plh_onehot(lp, p, None, 1, -2, 2, 255, 0.1, None) == -2
+    assert lib.plh_onehot(lp, odd, None, 1, 2, 2, 255, 0.1, None) == -6
+    assert lib.plh_onehot(lp, p, odd, 1, 2, 2, 255, 0.1, None) == -6
     # 16-bit logits need 2-byte alignment only; an odd address is still refused
     assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
