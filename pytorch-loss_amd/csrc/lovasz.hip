@@ -75,7 +75,29 @@ __global__ __launch_bounds__(256) void lov_class_max(const uint32_t *__restrict_
     for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, 64));
     if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
     __syncthreads();
-    if (threadIdx.x == 0) pos_max[c] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+    if (threadIdx.x == 0) {
+        pos_max[c] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+        pos_max[2 * C + c] = 0xFFFFFFFFu;       // all_min[c], for lov_absent_min
+    }
+}
+
+// A class without positives has J = 1 from the first sorted key on: only its largest error (smallest
+// key) has a non-zero Jaccard difference. For such classes (blocks of the others return at once)
+// this finds the smallest key of the row, which then serves as the class's limit.
+constexpr int kAbsentBlocks = 64;
+__global__ __launch_bounds__(256) void lov_absent_min(const uint32_t *__restrict__ keys, const uint32_t *pos_max,
+                                                      uint32_t *all_min, int P) {
+    __shared__ uint32_t wave_min[4];
+    const int c = blockIdx.y;
+    if (pos_max[c] != 0) return;                // block-uniform
+    const uint32_t *row = keys + (int64_t)c * P;
+    uint32_t m = 0xFFFFFFFFu;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < P; i += kAbsentBlocks * 256) m = min(m, row[i] & 0x7FFFFFFFu);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = min(m, (uint32_t)__shfl_xor((int)m, off, 64));
+    if ((threadIdx.x & 63) == 0) wave_min[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMin(all_min + c, min(min(wave_min[0], wave_min[1]), min(wave_min[2], wave_min[3])));
 }
 
 template <class T, int CP, int V>
@@ -171,6 +193,7 @@ struct SortArgs {
     uint32_t *tile_hot;          // last pass only: the same two tables for the positives
     uint32_t *hot_total;
     const uint32_t *pos_max;     // first pass only: per class, largest positive key + 1 (see keep_key)
+    const uint32_t *all_min;     // first pass only: per class without positives, its smallest key
     const uint32_t *kept_in;     // later passes: keys per class that the first pass let through
     uint32_t *kept_out;          // first pass: where that count goes
     int P;                       // row stride; keys per class row in the first pass
@@ -183,12 +206,16 @@ struct SortArgs {
 // (error bits of the key <= limit). What is left out would be sorted after every positive, where
 // the intersection is empty: J = 1 - 0/(k+1) = 1 on both sides of the difference, so its Jaccard
 // difference is exactly 0 and it adds exactly 0 to the loss; lov_unbin writes those zeros. Ignored
-// pixels (error bits 0x7FFFFFFF) are always left out. A class without positives keeps every valid
-// key. Keys equal to the limit stay in, so ties with the last positive keep their pixel order.
-__device__ __forceinline__ uint32_t keep_limit(const uint32_t *pos_max, int c) {
-    if (!pos_max) return 0x7FFFFFFFu;            // later passes: everything that is there takes part
-    const uint32_t m = pos_max[c];
-    return m ? m - 1u : kOne;
+// pixels (error bits 0x7FFFFFFF) are always left out. A class without positives has J = 1 from the
+// first key on, so only its largest error counts: its limit is the smallest key of the row. Keys
+// equal to the limit stay in, so ties with the last positive (or at the largest error) keep their
+// pixel order.
+__device__ __forceinline__ uint32_t keep_limit(const SortArgs &a, int c) {
+    if (!a.pos_max) return 0x7FFFFFFFu;          // later passes: everything that is there takes part
+    const uint32_t m = a.pos_max[c];
+    if (m) return m - 1u;
+    const uint32_t lowest = a.all_min[c];
+    return lowest <= kOne ? lowest : kOne;       // no valid key at all: nothing passes anyway
 }
 __device__ __forceinline__ bool keep_key(uint32_t key, uint32_t limit) { return (key & 0x7FFFFFFFu) <= limit; }
 
@@ -290,7 +317,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         }
         return;
     }
-    const uint32_t limit = keep_limit(a.pos_max, c);
+    const uint32_t limit = keep_limit(a, c);
     const uint32_t *kin = a.keys_in + (int64_t)c * a.P + begin;
     uint32_t key[kSortItems];
 #pragma unroll
@@ -401,7 +428,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
     __syncthreads();
 
-    const uint32_t limit = keep_limit(a.pos_max, c);
+    const uint32_t limit = keep_limit(a, c);
     const int64_t row = (int64_t)c * a.P;
     const uint32_t *kin = a.keys_in + row + begin;
     const uint32_t *vin = a.vals_in ? a.vals_in + row + begin : nullptr;
@@ -418,9 +445,13 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+        const bool valid = li < count && keep_key(key[r], limit);
+        if (__builtin_amdgcn_ballot_w64(valid) == 0) {      // wave-uniform: nothing of this round takes part
+            rank[r] = 0;
+            continue;
+        }
         uint32_t unused;
-        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, li < count && keep_key(key[r], limit), false, counts[wave],
-                         nullptr, rank[r], unused);
+        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, valid, false, counts[wave], nullptr, rank[r], unused);
     }
     __syncthreads();
 
@@ -790,7 +821,7 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     const int64_t regions = ceil_div(pl.P, kRegion);
     pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
-    pl.off_class = off;       off += round_up(4 * dimsize * 2, 256);      // pos_max[C], kept[C]
+    pl.off_class = off;       off += round_up(4 * dimsize * 3, 256);      // pos_max[C], kept[C], all_min[C]
     pl.off_block_max = off;   off += round_up(4 * dimsize * ceil_div(pl.P, 256), 256);   // [key blocks][C]
     pl.bytes = off;
     return PLH_OK;
@@ -833,6 +864,7 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     float *tile_loss = reinterpret_cast<float *>(ws + pl.off_tile_loss);
     uint32_t *pos_max = reinterpret_cast<uint32_t *>(ws + pl.off_class);
     uint32_t *kept = pos_max + dimsize;
+    uint32_t *all_min = pos_max + 2 * dimsize;
     const int C = (int)dimsize;
 
     uint32_t *block_table = reinterpret_cast<uint32_t *>(ws + pl.off_block_max);
@@ -867,6 +899,8 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         }
     });
     hipLaunchKernelGGL(lov_class_max, dim3((unsigned)C), dim3(256), 0, st, block_table, (int)key_blocks, C, pos_max);
+    hipLaunchKernelGGL(lov_absent_min, dim3(kAbsentBlocks, (unsigned)C), dim3(256), 0, st, keys_b, pos_max, all_min,
+                       (int)pl.P);
 
     // 2. three stable radix passes: (keys_b, -) -> (keys_a, vals_a) -> (keys_b, vals_b) -> (keys_a, vals_a).
     //    keys_b is the jacc output buffer, free until the last pass scatters into it. The first pass
@@ -889,6 +923,7 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         a.shift = 8 * pass;
         a.digit_mask = 0xFFu;
         a.pos_max = (pass == 0) ? pos_max : nullptr;
+        a.all_min = (pass == 0) ? all_min : nullptr;
         a.kept_in = (pass == 0) ? nullptr : kept;
         a.kept_out = (pass == 0) ? kept : nullptr;
         hipLaunchKernelGGL(lov_tile_hist<false>, tile_grid, dim3(kSortThreads), 0, st, a);
@@ -906,6 +941,7 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     a.shift = 24;
     a.digit_mask = 0x7Fu;
     a.pos_max = nullptr;
+    a.all_min = nullptr;
     a.kept_in = kept;
     a.kept_out = nullptr;
     hipLaunchKernelGGL(lov_tile_hist<true>, tile_grid, dim3(kSortThreads), 0, st, a);
