@@ -42,6 +42,8 @@ WORKLOADS = {
                   "Bernoulli(0.02) labels, alpha=0.25 gamma=2, mean"),
     "lovasz": dict(shape=(4, 19, 512, 1024), desc="LovaszSoftmaxV3 fwd+bwd, fp32 logits (4,19,512,1024), "
                    "Zipf(1.1) int64 labels 5% ignore=255, mean"),
+    "taylor": dict(shape=(8, 19, 1024, 1024), desc="TaylorCrossEntropyLossV3 fwd+bwd, fp32 logits (8,19,1024,1024), "
+                   "int64 labels 5% ignore=255, n=4, mean"),
     "onehot": dict(shape=(8, 19, 1024, 1024), desc="OnehotEncoder forward, int64 labels (8,1024,1024) 5% ignore=255 -> "
                    "fp32 (8,19,1024,1024), lb_smooth=0.1"),
     "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
@@ -75,7 +77,7 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     if name == "ohem":     # relabelling (logits + labels read, labels written), then the LSR-shaped loss
         relabel = b * E + 8 * P + 8 * P
         return relabel + b * E + 8 * P + 4 * P, b * E + 8 * P + 4 * P + b * E
-    if name in ("lsr", "lmargin"):
+    if name in ("lsr", "lmargin", "taylor"):
         fwd = b * E + 8 * P + 4 * P
         bwd = b * E + 8 * P + 4 * P + b * E
     elif name == "focal":   # the labels are floating point and share the logits' type
@@ -130,6 +132,8 @@ def make_criterion(name):
         return pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean")
     if name == "ohem":
         return pl.OhemCELoss(score_thresh=0.7, n_min=None, ignore_index=255)
+    if name == "taylor":
+        return pl.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="mean")
     return pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255)
 
 
@@ -222,11 +226,16 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         return {"relabel": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(ms, 4),
                             "algorithmic_bytes": nbytes}}
-    if name in ("lsr", "lmargin"):
+    if name in ("lsr", "lmargin", "taylor"):
         losses = torch.empty(labels.shape, dtype=torch.float32, device=x.device)
         grad = torch.empty_like(x)
         gout = torch.full(labels.shape, 1.0 / labels.numel(), dtype=torch.float32, device=x.device)
-        if name == "lsr":
+        if name == "taylor":
+            f = lambda: lib.plh_taylor_ce_forward(P(x), tag, P(labels), P(losses), None, None, 0, None, 0, n, c, m, 4,
+                                                  255, st())
+            b = lambda: lib.plh_taylor_ce_backward(P(x), tag, P(labels), P(gout), 1, 1.0, None, P(grad), n, c, m, 4,
+                                                   255, st())
+        elif name == "lsr":
             f = lambda: lib.plh_lsr_forward(P(x), tag, P(labels), P(losses), n, c, m, 255, 0.1, st())
             b = lambda: lib.plh_lsr_backward(P(x), tag, P(labels), P(gout), 1, P(grad), n, c, m, 255, 0.1, st())
         else:
@@ -274,7 +283,7 @@ def cpu_baseline(name, shape):
     from oracle import synth, torch_ref
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
-    cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2"}[name]
+    cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2", "taylor": "cfg2"}[name]
     w = synth.workload(cfg, batch=1)
     logits = torch.from_numpy(w["logits"]).requires_grad_()
     labels = torch.from_numpy(w["labels"])
@@ -282,7 +291,8 @@ def cpu_baseline(name, shape):
           "lmargin": lambda: torch_ref.lmargin(logits, labels, 0.3, "mean", 255),
           "focal": lambda: torch_ref.focal(logits, labels, 0.25, 2, "mean"),
           "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255),
-          "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255)}[name]
+          "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255),
+          "taylor": lambda: torch_ref.taylor_ce(logits, labels, 4, "mean", 255)}[name]
     times = []
     for i in range(4):
         logits.grad = None

@@ -234,6 +234,44 @@ int plh_onehot(const int64_t *labels, float *one_hot, int32_t *range_flags,
                int64_t n_size, int64_t dimsize, int64_t m_size,
                int64_t ignore_index, float smooth, void *stream);
 
+/* ---- Taylor softmax ------------------------------------------------------------------
+ * Replaces taylor_softmax_cpp.taylor_softmax_forward / taylor_softmax_backward
+ * (csrc/taylor_softmax.cu:270-417). The tensor is (n_size, dimsize, m_size) around the dimension
+ * the softmax runs over; feat, out, grad_output and grad_feat share `dtype`.
+ *   f(x) = sum_{i=0..order} x^i / i!   (order even, 2..64),   S = sum_j f(x_j)
+ *   out = f(x_j) / S, or log f(x_j) - log S with use_log               (:50-86)
+ *   grad_feat from grad_output as in :140-192.
+ */
+int plh_taylor_softmax_forward(const void *feat, int32_t dtype, void *out,
+                               int64_t n_size, int64_t dimsize, int64_t m_size,
+                               int64_t order, int32_t use_log, void *stream);
+
+int plh_taylor_softmax_backward(const void *grad_output, const void *feat, int32_t dtype,
+                                void *grad_feat,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t order, int32_t use_log, void *stream);
+
+/* Cross entropy on the logarithmic Taylor softmax in one kernel per direction: what
+ * TaylorCrossEntropyLossV3 composes from the Function above and F.nll_loss
+ * (pytorch_loss/taylor_softmax.py:175-198). loss_i = log S - log f(x_y), 0 at ignored pixels.
+ * forward: losses (n_size*m_size fp32) and/or, with loss_out != NULL, the 'sum' (mean = 0) or the
+ *   mean over the non-ignored pixels (mean = 1) in *loss_out and their count in *n_valid_out
+ *   (may be NULL); the reduced form needs a workspace of plh_reduce_workspace_bytes(n_size*m_size).
+ * backward: grad_logits = dloss/dlogits * grad_output[i * stride] * scale / *divide_by
+ *   (grad_output NULL = 1, stride 0 = one scalar; divide_by NULL = 1).
+ */
+int plh_taylor_ce_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                          float *loss_out, int64_t *n_valid_out, int32_t mean,
+                          void *workspace, int64_t workspace_bytes,
+                          int64_t n_size, int64_t dimsize, int64_t m_size,
+                          int64_t order, int64_t ignore_index, void *stream);
+
+int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *labels,
+                           const float *grad_output, int64_t grad_output_stride, float scale,
+                           const int64_t *divide_by, void *grad_logits,
+                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                           int64_t order, int64_t ignore_index, void *stream);
+
 /* ---- measurement aid ----------------------------------------------------------------
  * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,
  * 4*numel written), used to calibrate hardware byte counters and to measure the

@@ -214,6 +214,57 @@ def onehot(labels, n_classes, smooth=0.0, ignore_index=-1, dtype=np.float32):
     return out
 
 
+def _around(a, dim):
+    dim = dim % a.ndim
+    n = int(np.prod(a.shape[:dim], dtype=np.int64))
+    m = int(np.prod(a.shape[dim + 1:], dtype=np.int64))
+    return n, int(a.shape[dim]), m
+
+
+def taylor_forward(feat, dim=1, order=2, use_log=False):
+    """Taylor softmax of even `order` along `dim` (csrc/taylor_softmax.cu:50-86)."""
+    feat = np.ascontiguousarray(feat)
+    sfx, _ = _suffix(feat)
+    n, d, m = _around(feat, dim)
+    out = np.empty_like(feat)
+    if feat.size:
+        _call("oracle_taylor_forward" + sfx, _ptr(feat), _ptr(out), i64(n), i64(d), i64(m), i64(order),
+              ctypes.c_int(1 if use_log else 0))
+    return out
+
+
+def taylor_backward(grad, feat, dim=1, order=2, use_log=False):
+    feat = np.ascontiguousarray(feat)
+    grad = np.ascontiguousarray(grad, dtype=feat.dtype)
+    sfx, _ = _suffix(feat)
+    n, d, m = _around(feat, dim)
+    out = np.empty_like(feat)
+    if feat.size:
+        _call("oracle_taylor_backward" + sfx, _ptr(grad), _ptr(feat), _ptr(out), i64(n), i64(d), i64(m), i64(order),
+              ctypes.c_int(1 if use_log else 0))
+    return out
+
+
+def taylor_ce(logits, labels, order=2, ignore_index=-1):
+    """Per-pixel -log_taylor_softmax(logits)[label], 0 at ignored pixels: what F.nll_loss(reduction=
+    'none') makes of the log form (pytorch_loss/taylor_softmax.py:175-198)."""
+    logits, labels = _prep(logits, labels)
+    logp = taylor_forward(logits, 1, order, True)
+    safe = np.where(labels == ignore_index, 0, labels)
+    picked = np.take_along_axis(logp, np.expand_dims(safe, 1), 1).squeeze(1)
+    return np.where(labels == ignore_index, 0, -picked).astype(logits.dtype)
+
+
+def taylor_ce_backward(logits, labels, order, ignore_index, grad_out):
+    """Gradient of taylor_ce under the per-pixel upstream gradient `grad_out`."""
+    logits, labels = _prep(logits, labels)
+    g = np.zeros_like(logits)
+    go = np.broadcast_to(np.asarray(grad_out, dtype=logits.dtype), labels.shape)
+    safe = np.where(labels == ignore_index, 0, labels)
+    np.put_along_axis(g, np.expand_dims(safe, 1), np.expand_dims(np.where(labels == ignore_index, 0, -go), 1), 1)
+    return taylor_backward(g, logits, 1, order, True)
+
+
 # ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
 # large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
 

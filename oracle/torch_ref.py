@@ -181,3 +181,18 @@ def ohem_ce(logits, labels, score_thresh, n_min=None, ignore_index=255):
     n_min = labels.numel() // 16 if n_min is None else n_min
     new_labels = ohem_labels(logits, labels, ignore_index, score_thresh, n_min)
     return F.cross_entropy(logits, new_labels, ignore_index=ignore_index, reduction="mean")
+
+
+def taylor_log_softmax(x, dim=1, n=4):
+    """LogTaylorSoftmaxV1 (pytorch_loss/taylor_softmax.py:35-44): exp replaced by its order-n series."""
+    fn = torch.ones_like(x)
+    denor = 1.0
+    for i in range(1, n + 1):
+        denor *= i
+        fn = fn + x.pow(i) / denor
+    return (fn / fn.sum(dim=dim, keepdim=True)).log()
+
+
+def taylor_ce(logits, labels, n=4, reduction="mean", ignore_index=-1):
+    """TaylorCrossEntropyLossV1.forward (pytorch_loss/taylor_softmax.py:160-173)."""
+    return F.nll_loss(taylor_log_softmax(logits, 1, n), labels, reduction=reduction, ignore_index=ignore_index)

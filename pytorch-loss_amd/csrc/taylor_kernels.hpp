@@ -1,0 +1,390 @@
+// Taylor softmax (de Brebisson & Vincent; "Exploring Alternatives to Softmax Function") along one
+// dimension, forward and backward, plus the cross entropy built on its logarithm, for gfx950.
+//
+// With f(x) = sum_{i=0..n} x^i / i!  (n even, so f > 0) and S = sum_j f(x_j) over the dimension:
+//   y_j      = f(x_j) / S                    or, with use_log,  log f(x_j) - log S
+//   backward = f'(x_k) * (g_k - sum_j g_j y_j) / S                          (plain)
+//            = f'(x_k) * (g_k / f(x_k) - (sum_j g_j) / S)                   (log)
+// where f' is the series of order n-1 (csrc/taylor_softmax.cu:24-33 series, :50-86 forward,
+// :140-192 backward). The tensor is seen as (n_size, dimsize, m_size) around the chosen dimension.
+// Cross entropy on the log form (what TaylorCrossEntropyLossV3 composes from the Function and
+// F.nll_loss, pytorch_loss/taylor_softmax.py:175-198) in one kernel per direction:
+//   loss_i = log S - log f(x_y),   grad_k = gout_i * (f'(x_k) / S - [k == y] f'(x_k) / f(x_k)).
+#pragma once
+#include "plh_common.hpp"
+
+namespace plh {
+
+struct TaylorParams {
+    int64_t P;          // n_size * m_size
+    int64_t m_size;
+    int C;              // dimsize
+    int order;          // n
+    int use_log;
+    int64_t ignore;     // cross entropy only
+    unsigned xcd_run;
+};
+
+// 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and
+// its terms vanish, which the zero past the end of the table reproduces).
+struct InvFactorials {
+    float v[36];
+    constexpr InvFactorials() : v{} {
+        double f = 1.0;
+        for (int i = 0; i < 36; ++i) {
+            if (i > 1) f *= (double)i;
+            v[i] = (i <= 33) ? (float)(1.0 / f) : 0.f;
+        }
+    }
+};
+__device__ constexpr InvFactorials kInvFact{};
+
+// f of order n (>= 2) and, as a by-product, of order n-1 (its derivative). The orders in common use
+// (2 and 4; `order` is uniform, so the branch is scalar) are evaluated in nested form, everything
+// else term by term upwards like the reference's recurrence (csrc/taylor_softmax.cu:24-33).
+__device__ __forceinline__ void taylor_pair(float x, int order, float &f, float &df) {
+    if (order == 2) {
+        df = 1.f + x;
+        f = __builtin_fmaf(x * x, 0.5f, df);
+        return;
+    }
+    if (order == 4) {
+        const float x2 = x * x;
+        df = __builtin_fmaf(x, __builtin_fmaf(x, __builtin_fmaf(x, 1.f / 6.f, 0.5f), 1.f), 1.f);
+        f = __builtin_fmaf(x2 * x2, 1.f / 24.f, df);
+        return;
+    }
+    float res = 1.f + x, prev = 1.f, mid = x;
+    for (int i = 2; i <= order; ++i) {
+        prev = res;
+        mid *= x;
+        res = __builtin_fmaf(mid, kInvFact.v[i < 35 ? i : 35], res);
+    }
+    f = res;
+    df = prev;
+}
+
+// ---------------------------------------------------------------- regs ----
+
+template <class T, int CP, int V, bool Uniform>
+__global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restrict__ x, T *__restrict__ out,
+                                                             const TaylorParams p) {
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    if (!at.live) return;
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
+    float y[CP][V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                y[j][k] = f;
+                s += f;
+            }
+        const float inv = 1.f / s, ls = logf(s);
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) y[j][k] = p.use_log ? logf(y[j][k]) - ls : y[j][k] * inv;
+    }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(y[j]);
+    at.store_slice(out, p.C, p.m_size, raw);
+}
+
+template <class T, int CP, int V, bool Uniform>
+__global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restrict__ g, const T *__restrict__ x,
+                                                             T *__restrict__ gx, const TaylorParams p) {
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    if (!at.live) return;
+    typename Pack<T, V>::Raw raw[CP], graw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
+    at.load_slice(g, p.C, p.m_size, graw);
+    // the series is cheap: it is evaluated again in the second sweep rather than kept in registers
+    float r[CP][V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f, dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                const float gj = Pack<T, V>::get(graw[j], k);
+                s += f;
+                dot += p.use_log ? gj : f * gj;
+            }
+        const float inv = 1.f / s;
+        const float mid = p.use_log ? dot * inv : dot * inv * inv;       // csrc/taylor_softmax.cu:163-173
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                const float gj = Pack<T, V>::get(graw[j], k);
+                r[j][k] = p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(r[j]);
+    at.store_slice(gx, p.C, p.m_size, raw);
+}
+
+// Cross entropy on the log form: loss per pixel (fp32), and its gradient with the upstream folded in.
+template <class T, int CP, int V, bool Uniform, bool Reduce>
+__global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                float *__restrict__ loss, Partials part,
+                                                                const TaylorParams p) {
+    __shared__ float red[4];
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    if (!Reduce && !at.live) return;
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    float out[V];
+    float mine = 0.f;
+    int cnt = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        float s = 0.f, f_y = 1.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                s += f;
+                f_y = (tgt == j) ? f : f_y;
+            }
+        const bool valid = at.live && !ign && tgt >= 0;
+        out[k] = valid ? logf(s) - logf(f_y) : 0.f;
+        mine += out[k];
+        cnt += (at.live && !ign) ? 1 : 0;
+    }
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256((float)cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int CP, int V, bool Uniform>
+__global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                const Upstream up, T *__restrict__ gx,
+                                                                const TaylorParams p) {
+    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    if (!at.live) return;
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    float go[V];
+    load_upstream<V>(up, at.pix, go);
+    float r[CP][V];
+    unsigned keep[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        keep[k] = (ign || tgt < 0) ? 0u : 0xFFFFFFFFu;
+        float s = 0.f, f_y = 1.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                s += f;
+                f_y = (tgt == j) ? f : f_y;
+            }
+        const float scale = go[k] * __builtin_amdgcn_rcpf(s);
+        float hot = go[k] / f_y;                                   // per pixel
+        asm("" : "+v"(hot));
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, p.C)) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                r[j][k] = df * ((tgt == j) ? scale - hot : scale);
+            }
+    }
+    const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(r[j]) & mask;
+    at.store_slice(gx, p.C, p.m_size, raw);
+}
+
+// --------------------------------------------------------------- group ----
+// Any dimsize: G lanes share one slice and stride over it (G = 64: a wavefront per row when the
+// dimension is the contiguous one; G = 1: a lane per slice). The series is re-evaluated in each
+// sweep; re-reads hit cache.
+
+enum TaylorKind { kTaylorFwd = 0, kTaylorBwd = 1, kTaylorCeFwd = 2, kTaylorCeBwd = 3 };
+
+template <class T, int G, int Kind, bool Reduce>
+__global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, const T *__restrict__ g,
+                                                    const int64_t *__restrict__ lab, const Upstream up,
+                                                    T *__restrict__ out, float *__restrict__ loss, Partials part,
+                                                    const TaylorParams p) {
+    constexpr int kPix = 256 / G;
+    __shared__ float red[4];
+    const int sub = threadIdx.x % G, grp = threadIdx.x / G;
+    float mine = 0.f, cnt = 0.f;
+    const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
+    for (int64_t rd = 0; rd < rounds; ++rd) {
+        const int64_t pix = (rd * gridDim.x + blockIdx.x) * kPix + grp;
+        const bool live = pix < p.P;
+        const int64_t pc = live ? pix : 0;
+        const int64_t n = pc / p.m_size;
+        const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
+        const T *xs = x + base;
+        float s = 0.f, dot = 0.f;
+        for (int j = sub; j < p.C; j += G) {
+            float f, df;
+            taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
+            s += f;
+            if constexpr (Kind == kTaylorBwd) {
+                const float gj = load_one(g + base + (int64_t)j * p.m_size);
+                dot += p.use_log ? gj : f * gj;
+            }
+        }
+        s = group_reduce<G>(s, OpSum());
+        if constexpr (Kind == kTaylorBwd) dot = group_reduce<G>(dot, OpSum());
+        const float inv = 1.f / s;
+        if constexpr (Kind == kTaylorFwd) {
+            const float ls = logf(s);
+            if (live)
+                for (int j = sub; j < p.C; j += G) {
+                    float f, df;
+                    taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
+                    store_one(out + base + (int64_t)j * p.m_size, p.use_log ? logf(f) - ls : f * inv);
+                }
+        } else if constexpr (Kind == kTaylorBwd) {
+            const float mid = p.use_log ? dot * inv : dot * inv * inv;
+            if (live)
+                for (int j = sub; j < p.C; j += G) {
+                    float f, df;
+                    taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
+                    const float gj = load_one(g + base + (int64_t)j * p.m_size);
+                    store_one(out + base + (int64_t)j * p.m_size,
+                              p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid);
+                }
+        } else {
+            const int64_t lb = lab[pc];
+            const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
+            if constexpr (Kind == kTaylorCeFwd) {
+                float f_y = 1.f, df;
+                if (has_y) taylor_pair(load_one(xs + lb * p.m_size), p.order, f_y, df);
+                const float v = (live && has_y) ? logf(s) - logf(f_y) : 0.f;
+                if (live && sub == 0) {
+                    if (loss) loss[pix] = v;
+                    mine += v;
+                    cnt += (lb != p.ignore) ? 1.f : 0.f;
+                }
+            } else {
+                float go[1];
+                load_upstream<1>(up, pc, go);
+                const float gk = has_y ? go[0] : 0.f;
+                if (live)
+                    for (int j = sub; j < p.C; j += G) {
+                        float f, df;
+                        taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
+                        store_one(out + base + (int64_t)j * p.m_size,
+                                  has_y ? df * inv * gk - ((lb == j) ? df / f * gk : 0.f) : 0.f);
+                    }
+            }
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+// ------------------------------------------------------------ dispatch ----
+
+template <class T, int Kind, bool Reduce>
+unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstream &up, T *out, float *loss, Partials part,
+                       const TaylorParams &p, hipStream_t st) {
+    constexpr int VT = ElemTraits<T>::kVec;
+    const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
+    const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec);
+    const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
+    if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
+        const bool vec = (shape == Shape::RegsVec) && g_ok;
+        const bool uni = vec && tiles_are_uniform(p.m_size, VT, sizeof(T));
+        const unsigned grid = vec ? regs_grid<VT>(p.P) : regs_grid<1>(p.P);
+#define PLH_GO(CPV, VV, UU)                                                                                          \
+    do {                                                                                                             \
+        if constexpr (Kind == kTaylorFwd)                                                                            \
+            hipLaunchKernelGGL((taylor_fwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, out, p);   \
+        else if constexpr (Kind == kTaylorBwd)                                                                       \
+            hipLaunchKernelGGL((taylor_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, g, x, out, p); \
+        else if constexpr (Kind == kTaylorCeFwd)                                                                     \
+            hipLaunchKernelGGL((taylor_ce_fwd_regs<T, CPV, VV, UU, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
+                               lab, loss, part, p);                                                                  \
+        else                                                                                                         \
+            hipLaunchKernelGGL((taylor_ce_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab,    \
+                               up, out, p);                                                                          \
+    } while (0)
+        switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                       \
+    case K:                               \
+        if (uni) PLH_GO(4 * K, VT, true); \
+        else if (vec) PLH_GO(4 * K, VT, false); \
+        else PLH_GO(4 * K, 1, false);     \
+        break;
+            PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+#undef PLH_GO
+        }
+        return grid;
+    }
+    if (p.m_size == 1) {
+        const unsigned grid = group_grid(p.P, 4);
+        hipLaunchKernelGGL((taylor_group<T, 64, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss,
+                           part, p);
+        return grid;
+    }
+    const unsigned grid = group_grid(p.P, 256);
+    hipLaunchKernelGGL((taylor_group<T, 1, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss, part, p);
+    return grid;
+}
+
+// Per-dtype entry, instantiated in taylor_f32.hip / taylor_f16.hip / taylor_bf16.hip.
+template <class T>
+unsigned taylor_run_typed(int kind, bool reduce, const T *x, const T *g, const int64_t *lab, const Upstream &up, T *out,
+                          float *loss, Partials part, const TaylorParams &p, hipStream_t st) {
+    switch (kind) {
+        case kTaylorFwd: return taylor_launch<T, kTaylorFwd, false>(x, g, lab, up, out, loss, part, p, st);
+        case kTaylorBwd: return taylor_launch<T, kTaylorBwd, false>(x, g, lab, up, out, loss, part, p, st);
+        case kTaylorCeFwd:
+            return reduce ? taylor_launch<T, kTaylorCeFwd, true>(x, g, lab, up, out, loss, part, p, st)
+                          : taylor_launch<T, kTaylorCeFwd, false>(x, g, lab, up, out, loss, part, p, st);
+        default: return taylor_launch<T, kTaylorCeBwd, false>(x, g, lab, up, out, loss, part, p, st);
+    }
+}
+
+#define PLH_TAYLOR_SIGNATURE(T)                                                                                       \
+    unsigned taylor_run_typed<T>(int, bool, const T *, const T *, const int64_t *, const Upstream &, T *, float *,    \
+                                 Partials, const TaylorParams &, hipStream_t);
+#define PLH_TAYLOR_EXTERN(T) extern template PLH_TAYLOR_SIGNATURE(T)
+#define PLH_TAYLOR_INSTANTIATE(T) template PLH_TAYLOR_SIGNATURE(T)
+
+}  // namespace plh

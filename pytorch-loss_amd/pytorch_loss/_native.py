@@ -51,6 +51,10 @@ _SIGNATURES = {
     "plh_ohem_scores": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "plh_ohem_select_labels": (ctypes.c_int, [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _i64, _p]),
     "plh_ohem_score_label": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _p]),
+    "plh_taylor_softmax_forward": (ctypes.c_int, [_p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_taylor_ce_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _f32, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_onehot": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
@@ -483,6 +487,92 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
     _call(a.x, "plh_ohem_score_label", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(out), _ptr(scores), _ptr(ws), ws_bytes,
           a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
     return out
+
+
+# --------------------------------------------------------------- taylor ----
+
+def _check_order(n):
+    if n <= 0 or n % 2 != 0:
+        raise AssertionError("taylor softmax: n must be a positive even number")   # taylor_softmax.py:36
+
+
+def _around_dim(t, dim):
+    if t.dim() == 0:
+        raise RuntimeError("taylor softmax: input needs at least one dimension")
+    dim = dim % t.dim()
+    n_size = 1
+    for d in t.shape[:dim]:
+        n_size *= int(d)
+    m_size = 1
+    for d in t.shape[dim + 1:]:
+        m_size *= int(d)
+    return n_size, int(t.shape[dim]), m_size
+
+
+def taylor_softmax_forward(feat, dim, n, use_log):
+    _require_gpu("taylor softmax function", feat)
+    _check_order(n)
+    x, tag = _logits(feat)
+    n_size, dimsize, m_size = _around_dim(x, dim)
+    out = torch.empty_like(x)
+    if x.numel():
+        _call(x, "plh_taylor_softmax_forward", _ptr(x), tag, _ptr(out), n_size, dimsize, m_size, int(n),
+              1 if use_log else 0)
+    return _back_to(out, feat.dtype) if out.dtype != feat.dtype else out
+
+
+def taylor_softmax_backward(grad_output, feat, dim, n, use_log):
+    _require_gpu("taylor softmax function", feat, grad_output)
+    _check_order(n)
+    x, tag = _logits(feat)
+    g = grad_output if grad_output.dtype == x.dtype else grad_output.to(x.dtype)
+    g = g.expand(x.shape).contiguous()
+    n_size, dimsize, m_size = _around_dim(x, dim)
+    out = torch.empty_like(x)
+    if x.numel():
+        _call(x, "plh_taylor_softmax_backward", _ptr(g), _ptr(x), tag, _ptr(out), n_size, dimsize, m_size, int(n),
+              1 if use_log else 0)
+    return out if out.dtype == feat.dtype else out.to(feat.dtype)
+
+
+def taylor_args(logits, labels):
+    return seg_args(logits, labels, "taylor cross entropy", "taylor_ce")
+
+
+def taylor_ce_forward(logits, labels, n, ignore_index, reduction, args=None):
+    """-> (loss, n_valid or None). reduction 'mean' / 'sum' give a 0-dim loss, anything else per pixel."""
+    _check_order(n)
+    a = args or taylor_args(logits, labels)
+    reduced = reduction in ("mean", "sum") and a.x.numel() > 0
+    dev = a.x.device
+    if reduced:
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        n_valid = torch.empty((), dtype=torch.int64, device=dev)
+        ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
+        _call(a.x, "plh_taylor_ce_forward", _ptr(a.x), a.tag, _ptr(a.lb), None, _ptr(loss), _ptr(n_valid),
+              1 if reduction == "mean" else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(n), int(ignore_index))
+        return _back_to(loss, _loss_dtype(a.dtype)), n_valid
+    losses = torch.empty(a.lb.shape, dtype=torch.float32, device=dev)
+    if a.x.numel():
+        _call(a.x, "plh_taylor_ce_forward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), None, None, 0, None, 0,
+              a.n, a.c, a.m, int(n), int(ignore_index))
+    else:
+        losses.zero_()
+    return _back_to(losses, _loss_dtype(a.dtype)), None
+
+
+def taylor_ce_backward(logits, labels, n, ignore_index, grad_output, divide_by=None, args=None):
+    a = args or taylor_args(logits, labels)
+    grad = torch.empty_like(a.x)
+    if a.x.numel() == 0:
+        return _back_to(grad, a.dtype)
+    if grad_output.numel() == 1:
+        go, stride = _scalar_f32(grad_output), 0
+    else:
+        go, stride = _upstream(grad_output, a.lb.shape)
+    _call(a.x, "plh_taylor_ce_backward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(go), stride, 1.0, _ptr(divide_by),
+          _ptr(grad), a.n, a.c, a.m, int(n), int(ignore_index))
+    return _back_to(grad, a.dtype)
 
 
 # -------------------------------------------------------------- one-hot ----

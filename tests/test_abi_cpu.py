@@ -111,6 +111,20 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_onehot(lp, p, None, 1, -2, 2, 255, 0.1, None) == -2
     assert lib.plh_onehot(lp, odd, None, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_onehot(lp, p, odd, 1, 2, 2, 255, 0.1, None) == -6
+    # Taylor softmax and its cross entropy
+    assert lib.plh_taylor_softmax_forward(None, 0, None, 0, 19, 16, 4, 0, None) == 0
+    assert lib.plh_taylor_softmax_forward(p, 0, p, 1, 2, 2, 3, 0, None) == -2          # odd order
+    assert lib.plh_taylor_softmax_forward(p, 0, p, 1, 2, 2, 0, 0, None) == -2
+    assert lib.plh_taylor_softmax_forward(p, 4, p, 1, 2, 2, 2, 0, None) == -7
+    assert lib.plh_taylor_softmax_forward(p, 0, None, 1, 2, 2, 2, 0, None) == -1
+    assert lib.plh_taylor_softmax_forward(odd, 0, p, 1, 2, 2, 2, 0, None) == -6
+    assert lib.plh_taylor_softmax_backward(None, p, 0, p, 1, 2, 2, 2, 1, None) == -1
+    assert lib.plh_taylor_softmax_backward(odd, p, 0, p, 1, 2, 2, 2, 1, None) == -6
+    assert lib.plh_taylor_ce_forward(p, 0, lp, None, None, None, 0, None, 0, 1, 2, 2, 2, 255, None) == -1
+    assert lib.plh_taylor_ce_forward(p, 0, lp, None, p, None, 1, None, 0, 1, 2, 2, 2, 255, None) == -5
+    assert lib.plh_taylor_ce_forward(p, 0, lp, p, None, None, 0, None, 0, 1, 2, 2, 5, 255, None) == -2
+    assert lib.plh_taylor_ce_backward(p, 0, lp, p, 2, 1.0, None, p, 1, 2, 2, 2, 255, None) == -3
+    assert lib.plh_taylor_ce_backward(p, 0, None, None, 0, 1.0, None, p, 1, 2, 2, 2, 255, None) == -1
     # 16-bit logits need 2-byte alignment only; an odd address is still refused
     assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
