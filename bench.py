@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -46,6 +46,8 @@ WORKLOADS = {
                    "int64 labels 5% ignore=255, n=4, mean"),
     "onehot": dict(shape=(8, 19, 1024, 1024), desc="OnehotEncoder forward, int64 labels (8,1024,1024) 5% ignore=255 -> "
                    "fp32 (8,19,1024,1024), lb_smooth=0.1"),
+    "dice": dict(shape=(64, 1, 1024, 1024), desc="SoftDiceLossV3 fwd+bwd, fp32 logits/labels (64,1,1024,1024) as one row, "
+                 "Bernoulli(0.3) labels, p=1 smooth=1"),
     "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
                  "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }
@@ -83,6 +85,9 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     elif name == "focal":   # the labels are floating point and share the logits' type
         fwd = 2 * b * E + 4 * E
         bwd = 2 * b * E + 4 * E + b * E
+    elif name == "dice":    # float labels in the logits' type; one loss and two sums per row
+        fwd = 2 * b * E
+        bwd = 2 * b * E + b * E
     else:  # lovasz: compulsory I/O only (logits, labels, saved Jaccard differences, gradient)
         fwd = b * E + 8 * P + 4 * E
         bwd = b * E + 4 * E + 8 * P + b * E
@@ -95,7 +100,7 @@ def make_inputs(name, shape, device, seed=15, dtype="f32"):
         import torch
         td = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
         logits = logits.to(td)
-        if name == "focal":
+        if name in ("focal", "dice"):
             labels = labels.to(td)
     return logits, labels
 
@@ -108,6 +113,9 @@ def _make_inputs_f32(name, shape, device, seed):
         logits = torch.randn(shape, device=device, generator=g) * 1.5 - 2.0
         labels = (torch.rand(shape, device=device, generator=g) < 0.02).float()
         return logits, labels
+    if name == "dice":
+        logits = torch.randn(shape, device=device, generator=g) * 2.0
+        return logits, (torch.rand(shape, device=device, generator=g) < 0.3).float()
     logits = torch.randn(shape, device=device, generator=g) * (4.0 if name == "ohem" else 2.0)
     lshape = shape[:1] + shape[2:]
     if name == "lovasz":
@@ -134,6 +142,8 @@ def make_criterion(name):
         return pl.OhemCELoss(score_thresh=0.7, n_min=None, ignore_index=255)
     if name == "taylor":
         return pl.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="mean")
+    if name == "dice":
+        return pl.SoftDiceLossV3(p=1, smooth=1.0)
     return pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255)
 
 
@@ -247,6 +257,16 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         gout = torch.full(shape, 1.0 / x.numel(), dtype=torch.float32, device=x.device)
         f = lambda: lib.plh_focal_forward(P(x), tag, P(labels), P(losses), x.numel(), 2.0, 0.25, st())
         b = lambda: lib.plh_focal_backward(P(x), tag, P(labels), P(gout), 1, P(grad), x.numel(), 2.0, 0.25, st())
+    elif name == "dice":
+        losses = torch.empty(1, dtype=torch.float32, device=x.device)
+        stats = torch.empty(2, dtype=torch.float32, device=x.device)
+        grad = torch.empty_like(x)
+        gout = torch.ones(1, dtype=torch.float32, device=x.device)
+        ws_bytes = int(lib.plh_soft_dice_workspace_bytes(1, x.numel()))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        f = lambda: lib.plh_soft_dice_forward(P(x), tag, P(labels), P(losses), P(stats), P(ws), ws_bytes, 1, x.numel(),
+                                              1.0, 1.0, st())
+        b = lambda: lib.plh_soft_dice_backward(P(gout), P(x), tag, P(labels), P(stats), P(grad), 1, x.numel(), 1.0, st())
     else:
         losses = torch.empty(c, dtype=torch.float32, device=x.device)
         jacc = torch.empty((c, n * m), dtype=torch.float32, device=x.device)
@@ -283,6 +303,11 @@ def cpu_baseline(name, shape):
     from oracle import synth, torch_ref
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
+    if name == "dice":
+        g = torch.Generator().manual_seed(15)
+        logits = (torch.randn((1,) + tuple(shape[1:]), generator=g) * 2.0).requires_grad_()
+        labels = (torch.rand(logits.shape, generator=g) < 0.3).float()
+        return _time_cpu(name, shape, cores, lambda: torch_ref.soft_dice(logits, labels, 1, 1.0), logits)
     cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2", "taylor": "cfg2"}[name]
     w = synth.workload(cfg, batch=1)
     logits = torch.from_numpy(w["logits"]).requires_grad_()
@@ -293,6 +318,10 @@ def cpu_baseline(name, shape):
           "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255),
           "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255),
           "taylor": lambda: torch_ref.taylor_ce(logits, labels, 4, "mean", 255)}[name]
+    return _time_cpu(name, shape, cores, fn, logits)
+
+
+def _time_cpu(name, shape, cores, fn, logits):
     times = []
     for i in range(4):
         logits.grad = None
@@ -351,7 +380,7 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
     gbps = (fwd + bwd) / (ms * 1e-3) / 1e9
     roof = kernel_rooflines(name, logits, labels, dtype)
     dist = {"warm": step_distribution(crit, [(logits, labels)])}
-    set_bytes = ELEM_BYTES[dtype] * numel(shape) * (2 if name == "focal" else 1)
+    set_bytes = ELEM_BYTES[dtype] * numel(shape) * (2 if name in ("focal", "dice") else 1)
     if set_bytes < (256 << 20):
         # working set fits the Infinity Cache: also rotate enough input sets to defeat it
         n_sets = max(4, -(-(768 << 20) // set_bytes))

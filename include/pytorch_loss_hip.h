@@ -272,6 +272,28 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
                            int64_t n_size, int64_t dimsize, int64_t m_size,
                            int64_t order, int64_t ignore_index, void *stream);
 
+/* ---- soft dice loss ---------------------------------------------------------------------
+ * Replaces soft_dice_cpp.soft_dice_forward / soft_dice_backward (csrc/soft_dice_kernel_v2.cu:258-436).
+ * logits and labels are (batchsize, sample_size) tensors of one floating type (`dtype`); with
+ * q = sigmoid(logits): numer = 2 sum(q y) + smooth, denor = sum(q^p + y^p) + smooth per row,
+ * losses[n] = 1 - numer / denor (fp32).
+ * forward also leaves (numer, denor) per row in stats (batchsize x 2 fp32), which the backward
+ * reads instead of reducing the rows again; workspace: plh_soft_dice_workspace_bytes() bytes,
+ * 256-byte aligned. backward: grad_logits[n, l] = grad_output[n] * dloss_n/dlogits[n, l].
+ * Limit: batchsize <= 65535.
+ */
+int64_t plh_soft_dice_workspace_bytes(int64_t batchsize, int64_t sample_size);
+
+int plh_soft_dice_forward(const void *logits, int32_t dtype, const void *labels,
+                          float *losses, float *stats,
+                          void *workspace, int64_t workspace_bytes,
+                          int64_t batchsize, int64_t sample_size,
+                          float p, float smooth, void *stream);
+
+int plh_soft_dice_backward(const float *grad_output, const void *logits, int32_t dtype,
+                           const void *labels, const float *stats, void *grad_logits,
+                           int64_t batchsize, int64_t sample_size, float p, void *stream);
+
 /* ---- measurement aid ----------------------------------------------------------------
  * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,
  * 4*numel written), used to calibrate hardware byte counters and to measure the

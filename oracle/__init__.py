@@ -265,6 +265,33 @@ def taylor_ce_backward(logits, labels, order, ignore_index, grad_out):
     return taylor_backward(g, logits, 1, order, True)
 
 
+def soft_dice_forward(logits, labels, p=1.0, smooth=1.0):
+    """(N, L) -> (losses (N,), stats (N, 2) = numer, denor) (pytorch_loss/soft_dice_loss.py:72-93)."""
+    logits = np.ascontiguousarray(logits)
+    labels = np.ascontiguousarray(labels, dtype=logits.dtype)
+    assert logits.ndim == 2 and logits.shape == labels.shape
+    sfx, _ = _suffix(logits)
+    n, length = logits.shape
+    losses = np.zeros((n,), dtype=logits.dtype)
+    stats = np.zeros((n, 2), dtype=logits.dtype)
+    _call("oracle_soft_dice_forward" + sfx, _ptr(logits), _ptr(labels), _ptr(losses), _ptr(stats), i64(n), i64(length),
+          f64(p), f64(smooth))
+    return losses, stats
+
+
+def soft_dice_backward(grad_out, logits, labels, stats, p=1.0):
+    logits = np.ascontiguousarray(logits)
+    labels = np.ascontiguousarray(labels, dtype=logits.dtype)
+    sfx, _ = _suffix(logits)
+    n, length = logits.shape
+    grad_out = np.ascontiguousarray(np.broadcast_to(grad_out, (n,)), dtype=logits.dtype)
+    stats = np.ascontiguousarray(stats, dtype=logits.dtype)
+    out = np.zeros_like(logits)
+    _call("oracle_soft_dice_backward" + sfx, _ptr(grad_out), _ptr(logits), _ptr(labels), _ptr(stats), _ptr(out),
+          i64(n), i64(length), f64(p))
+    return out
+
+
 # ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
 # large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
 

@@ -196,3 +196,12 @@ def taylor_log_softmax(x, dim=1, n=4):
 def taylor_ce(logits, labels, n=4, reduction="mean", ignore_index=-1):
     """TaylorCrossEntropyLossV1.forward (pytorch_loss/taylor_softmax.py:160-173)."""
     return F.nll_loss(taylor_log_softmax(logits, 1, n), labels, reduction=reduction, ignore_index=ignore_index)
+
+
+def soft_dice(logits, labels, p=1, smooth=1.0):
+    """Soft dice over everything as one row (pytorch_loss/soft_dice_loss.py:10-33):
+    1 - (2 sum(sigmoid(x) y) + smooth) / (sum(sigmoid(x)^p + y^p) + smooth)."""
+    probs = torch.sigmoid(logits)
+    numer = 2 * (probs * labels).sum() + smooth
+    denor = (probs.pow(p) + labels.pow(p)).sum() + smooth
+    return 1.0 - numer / denor

@@ -55,6 +55,9 @@ _SIGNATURES = {
     "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_taylor_ce_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _f32, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_soft_dice_workspace_bytes": (_i64, [_i64, _i64]),
+    "plh_soft_dice_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _f32, _p]),
+    "plh_soft_dice_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _f32, _p]),
     "plh_onehot": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
@@ -572,6 +575,37 @@ def taylor_ce_backward(logits, labels, n, ignore_index, grad_output, divide_by=N
         go, stride = _upstream(grad_output, a.lb.shape)
     _call(a.x, "plh_taylor_ce_backward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(go), stride, 1.0, _ptr(divide_by),
           _ptr(grad), a.n, a.c, a.m, int(n), int(ignore_index))
+    return _back_to(grad, a.dtype)
+
+
+# ------------------------------------------------------------ soft dice ----
+
+def soft_dice_forward(logits, labels, p, smooth):
+    """(N, L) logits and float labels -> (losses (N,), stats (N, 2) = numer, denor per row, marshalled inputs)."""
+    if logits.shape != labels.shape or logits.dim() != 2:
+        raise AssertionError("soft dice: logits and labels must both be (N, L)")     # soft_dice_loss.py:152
+    a = focal_args(logits, labels, "soft_dice_forward")
+    n, length = int(a.x.shape[0]), int(a.x.shape[1])
+    losses = torch.empty((n,), dtype=torch.float32, device=a.x.device)
+    stats = torch.empty((n, 2), dtype=torch.float32, device=a.x.device)
+    if n:
+        nbytes = int(load().plh_soft_dice_workspace_bytes(n, length))
+        if nbytes < 0:
+            _check(nbytes)
+        ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=a.x.device)
+        _call(a.x, "plh_soft_dice_forward", _ptr(a.x), a.tag, _ptr(a.y), _ptr(losses), _ptr(stats), _ptr(ws), nbytes,
+              n, length, float(p), float(smooth))
+    return _back_to(losses, _loss_dtype(a.dtype)), stats, a
+
+
+def soft_dice_backward(grad_output, stats, p, args):
+    a = args
+    n, length = int(a.x.shape[0]), int(a.x.shape[1])
+    grad = torch.empty_like(a.x)
+    if a.x.numel():
+        go = _f32c(grad_output.expand((n,)) if grad_output.numel() == 1 else grad_output.reshape(n))
+        _call(a.x, "plh_soft_dice_backward", _ptr(go), _ptr(a.x), a.tag, _ptr(a.y), _ptr(stats), _ptr(grad), n, length,
+              float(p))
     return _back_to(grad, a.dtype)
 
 

@@ -125,6 +125,18 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_taylor_ce_forward(p, 0, lp, p, None, None, 0, None, 0, 1, 2, 2, 5, 255, None) == -2
     assert lib.plh_taylor_ce_backward(p, 0, lp, p, 2, 1.0, None, p, 1, 2, 2, 2, 255, None) == -3
     assert lib.plh_taylor_ce_backward(p, 0, None, None, 0, 1.0, None, p, 1, 2, 2, 2, 255, None) == -1
+    # soft dice
+    assert lib.plh_soft_dice_workspace_bytes(-1, 4) == -2 and lib.plh_soft_dice_workspace_bytes(70000, 4) == -2
+    dice_need = lib.plh_soft_dice_workspace_bytes(2, 5000)
+    assert dice_need >= 2 * 5 * 8 and dice_need % 256 == 0
+    assert lib.plh_soft_dice_forward(None, 0, None, None, None, None, 0, 0, 16, 1.0, 1.0, None) == 0
+    assert lib.plh_soft_dice_forward(p, 3, p, p, p, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -7
+    assert lib.plh_soft_dice_forward(p, 0, None, p, p, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -1
+    assert lib.plh_soft_dice_forward(p, 0, p, p, None, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -1
+    assert lib.plh_soft_dice_forward(p, 0, p, p, p, None, 0, 2, 8, 1.0, 1.0, None) == -5
+    assert lib.plh_soft_dice_forward(odd, 0, p, p, p, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -6
+    assert lib.plh_soft_dice_backward(None, p, 0, p, p, p, 2, 8, 1.0, None) == -1
+    assert lib.plh_soft_dice_backward(p, p, 0, p, None, p, 2, 8, 1.0, None) == -1
     # 16-bit logits need 2-byte alignment only; an odd address is still refused
     assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
