@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -48,6 +48,8 @@ WORKLOADS = {
                    "fp32 (8,19,1024,1024), lb_smooth=0.1"),
     "dice": dict(shape=(64, 1, 1024, 1024), desc="SoftDiceLossV3 fwd+bwd, fp32 logits/labels (64,1,1024,1024) as one row, "
                  "Bernoulli(0.3) labels, p=1 smooth=1"),
+    "layernorm": dict(shape=(16, 256, 128, 128), desc="LayerNormV3Func fwd+bwd, fp32 (16,256,128,128) normalised over C, "
+                      "eps=1e-6, per-element upstream gradient"),
     "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
                  "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }
@@ -85,6 +87,9 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     elif name == "focal":   # the labels are floating point and share the logits' type
         fwd = 2 * b * E + 4 * E
         bwd = 2 * b * E + 4 * E + b * E
+    elif name == "layernorm":   # x in, y out; x and the upstream gradient in, the result out
+        fwd = 2 * b * E
+        bwd = 3 * b * E
     elif name == "dice":    # float labels in the logits' type; one loss and two sums per row
         fwd = 2 * b * E
         bwd = 2 * b * E + b * E
@@ -303,6 +308,11 @@ def cpu_baseline(name, shape):
     from oracle import synth, torch_ref
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
+    if name == "layernorm":
+        g = torch.Generator().manual_seed(15)
+        logits = (torch.randn((1, shape[1], shape[2] * shape[3]), generator=g) * 2.0 + 0.5).requires_grad_()
+        go = torch.randn(logits.shape, generator=g)
+        return _time_cpu(name, shape, cores, lambda: (torch_ref.layer_norm(logits, 1e-6) * go).sum(), logits)
     if name == "dice":
         g = torch.Generator().manual_seed(15)
         logits = (torch.randn((1,) + tuple(shape[1:]), generator=g) * 2.0).requires_grad_()
@@ -368,10 +378,58 @@ def run_onehot(steps, warmup, device):
                 bytes=nbytes, step_ms={"warm": {"median": round(ms, 4), "iters": steps, "input_sets": 1}})
 
 
+def run_layernorm(steps, warmup, device, dtype):
+    """Not a loss: a step is Function forward + backward with a per-element upstream gradient."""
+    import torch
+    import pytorch_loss as pl
+    from pytorch_loss import _native
+    shape = WORKLOADS["layernorm"]["shape"]
+    td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    g = torch.Generator(device=device)
+    g.manual_seed(15)
+    n, c = shape[0], shape[1]
+    m = numel(shape) // (n * c)
+    x = (torch.randn((n, c, m), device=device, generator=g) * 2.0 + 0.5).to(td).requires_grad_()
+    go = torch.randn((n, c, m), device=device, generator=g).to(td)
+
+    def step():
+        x.grad = None
+        y = pl.LayerNormV3Func.apply(x, 1e-6)
+        y.backward(go)
+        return y
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        y = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    fwd, bwd = algorithmic_bytes("layernorm", shape, dtype)
+    lib = _native.load()
+    P, st, tag = _native._ptr, _native._stream, DTYPE_TAG[dtype]
+    xd, out = x.detach(), torch.empty_like(x)
+    f = lambda: lib.plh_layer_norm_forward(P(xd), tag, P(out), n, c, m, 1e-6, st())
+    b = lambda: lib.plh_layer_norm_backward(P(go), P(xd), tag, P(out), n, c, m, 1e-6, st())
+    assert f() == 0 and b() == 0
+    roof = {}
+    for key, fn, nbytes in (("forward", f, fwd), ("backward", b, bwd)):
+        k_ms = time_kernel(fn)
+        gbps = nbytes / (k_ms * 1e-3) / 1e9
+        roof[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(k_ms, 4),
+                     "algorithmic_bytes": nbytes}
+    return dict(ms_per_step=ms, gbps=(fwd + bwd) / (ms * 1e-3) / 1e9, loss=float(y[0, 0, 0].item()), roofline=roof,
+                bytes=fwd + bwd, step_ms={"warm": {"median": round(ms, 4), "iters": steps, "input_sets": 1}})
+
+
 def run_workload(name, steps, warmup, device, dtype="f32"):
     import torch
     if name == "onehot":
         return run_onehot(max(steps, 20), warmup, device)
+    if name == "layernorm":
+        return run_layernorm(max(steps, 20), warmup, device, dtype)
     shape = WORKLOADS[name]["shape"]
     logits, labels = make_inputs(name, shape, device, dtype=dtype)
     crit = make_criterion(name)

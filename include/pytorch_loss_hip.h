@@ -294,6 +294,22 @@ int plh_soft_dice_backward(const float *grad_output, const void *logits, int32_t
                            const void *labels, const float *stats, void *grad_logits,
                            int64_t batchsize, int64_t sample_size, float p, void *stream);
 
+/* ---- layer norm over the channel dimension --------------------------------------------
+ * Replaces layer_norm_cpp.layer_norm_forward / layer_norm_backward (csrc/layer_norm.cu:377-393;
+ * kernels :53-257). x, out, grad_output, grad_x: (n_size, dimsize, m_size) contiguous in `dtype`.
+ * forward: out = (x - mean) * rsqrt(var + eps), mean and population variance over dimsize for
+ * each (n, m). backward returns what the reference's kernel returns (:212-216),
+ *   -rsqrt(v) * (1/C + (x - mean) * (x - 1/C) * mean * v) * grad_output,  v = var + eps.
+ * Arithmetic is fp32 for every dtype. Limit: n_size * m_size <= 64 * (2^31 - 1).
+ */
+int plh_layer_norm_forward(const void *x, int32_t dtype, void *out,
+                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                           float eps, void *stream);
+
+int plh_layer_norm_backward(const void *grad_output, const void *x, int32_t dtype, void *grad_x,
+                            int64_t n_size, int64_t dimsize, int64_t m_size,
+                            float eps, void *stream);
+
 /* ---- measurement aid ----------------------------------------------------------------
  * Plain fp32 device-to-device copy kernel of known traffic (4*numel bytes read,
  * 4*numel written), used to calibrate hardware byte counters and to measure the

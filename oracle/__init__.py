@@ -292,6 +292,29 @@ def soft_dice_backward(grad_out, logits, labels, stats, p=1.0):
     return out
 
 
+def layer_norm_forward(x, eps=1e-6):
+    """(N, C, M) normalised over C (csrc/layer_norm.cu:102-129)."""
+    x = np.ascontiguousarray(x)
+    assert x.ndim == 3
+    sfx, _ = _suffix(x)
+    out = np.zeros_like(x)
+    _call("oracle_layer_norm_forward" + sfx, _ptr(x), _ptr(out), i64(x.shape[0]), i64(x.shape[1]), i64(x.shape[2]),
+          f64(eps))
+    return out
+
+
+def layer_norm_backward(grad, x, eps=1e-6):
+    """What the reference's backward kernel returns (csrc/layer_norm.cu:200-216); see oracle_body.inc."""
+    x = np.ascontiguousarray(x)
+    grad = np.ascontiguousarray(grad, dtype=x.dtype)
+    assert x.ndim == 3 and grad.shape == x.shape
+    sfx, _ = _suffix(x)
+    out = np.zeros_like(x)
+    _call("oracle_layer_norm_backward" + sfx, _ptr(grad), _ptr(x), _ptr(out), i64(x.shape[0]), i64(x.shape[1]),
+          i64(x.shape[2]), f64(eps))
+    return out
+
+
 # ---- module-level reductions (label_smooth.py:162-171, focal_loss.py(root):195-200,
 # large_margin_softmax.py(root):221-229, lovasz_softmax.py:110-116) ----------------
 

@@ -2,9 +2,11 @@
  * TEST INFRASTRUCTURE ONLY -- never linked into, imported by or called from the
  * shipped library. CPU restatement (plain C, optional OpenMP) of the algorithms
  * behind pytorch-loss's LabelSmoothSoftmaxCE / FocalLoss / LargeMarginSoftmax /
- * LovaszSoftmax, used by the tests as the parity checker and by the benchmark's
+ * LovaszSoftmax and the ops next to them (OHEM relabelling, one-hot, Taylor softmax,
+ * soft dice, channel layer norm), used by the tests as the parity checker and by the benchmark's
  * cpu_baseline leg. Every function in oracle_body.inc cites the reference lines
- * it follows. Built by oracle/build.py into oracle/liboracle.so.
+ * it follows. One function is PARITY UNPINNED: oracle_layer_norm_backward (see its
+ * comment). Built by oracle/build.py into oracle/liboracle.so.
  *
  * Each function exists as <name>_f32 (the arithmetic type of the shipped path)
  * and <name>_f64 (a higher-precision check on the fp32 restatement itself).
@@ -20,6 +22,7 @@
 #define LOG1P log1pf
 #define POW powf
 #define FABS fabsf
+#define SQRT sqrtf
 #include "oracle_body.inc"
 #undef REAL
 #undef FN
@@ -28,6 +31,7 @@
 #undef LOG1P
 #undef POW
 #undef FABS
+#undef SQRT
 
 #define REAL double
 #define FN(name) name##_f64
@@ -36,6 +40,7 @@
 #define LOG1P log1p
 #define POW pow
 #define FABS fabs
+#define SQRT sqrt
 #include "oracle_body.inc"
 
 int oracle_abi_version(void) { return 1; }

@@ -205,3 +205,10 @@ def soft_dice(logits, labels, p=1, smooth=1.0):
     numer = 2 * (probs * labels).sum() + smooth
     denor = (probs.pow(p) + labels.pow(p)).sum() + smooth
     return 1.0 - numer / denor
+
+
+def layer_norm(x, eps=1e-6):
+    """(N, C, M) normalised over C with autograd's own backward (pytorch_loss/layer_norm.py:32-38)."""
+    mean = x.mean(dim=1, keepdim=True)
+    std = (x.var(dim=1, keepdim=True, unbiased=False) + eps).rsqrt()
+    return (x - mean) * std

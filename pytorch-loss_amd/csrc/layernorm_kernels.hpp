@@ -1,0 +1,239 @@
+// Layer norm over the channel dimension of (N, C, M) tensors on gfx950 (csrc/layer_norm.cu:53-257).
+//   forward   out = (x - mean) * rsqrt(var + eps),  mean / var (population) over C per (n, m)   (:102-129)
+//   backward  res = -rsqrt(v) * (1/C + (x - mean) * (x - 1/C) * mean * v) * grad,  v = var + eps  (:200-216)
+// The backward is the reference's expression, kept as it is (it is not the derivative of the forward).
+//
+// The op has to see a slice twice (statistics, then the normalised values), and a slice of C
+// channels times a wavefront's pixels is far more than caches keep per wave, so the slice stays in
+// REGISTERS between the two uses: lanes run along pixels (8 bytes per lane and channel), and for
+// C > 32 the four (C > 64: eight) waves of a block split the channels of one pixel group between
+// them and exchange per-wave (mean, centred square sum) pairs through LDS, merged by the
+// pairwise-variance rule. A wave holds at most 64 packed channels, which covers C <= 512; C <= 1024
+// runs one pixel per lane; anything larger, and m_size == 1 (rows contiguous), takes a two-sweep
+// kernel whose second sweep is served by cache.
+#pragma once
+#include "plh_common.hpp"
+
+namespace plh {
+
+struct LnParams {
+    int64_t P;          // n_size * m_size
+    int64_t m_size;
+    int C;
+    int per_wave;       // channels per wave when the waves of a block share a pixel group
+    float eps;
+};
+
+constexpr int kLnBlock = 256;
+
+// KW = channel slots per wave (>= the channels it holds), V = pixels per lane, WS = waves sharing a
+// pixel group (1: each of a block's four waves has its own group and all channels; 4 or 8: the block
+// is WS waves with 1/WS of the channels each).
+template <class T, int KW, int V, int WS, bool Bwd>
+__global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *__restrict__ x, const T *__restrict__ g,
+                                                    T *__restrict__ out, const LnParams p) {
+    using PK = Pack<T, V>;
+    __shared__ float ex[WS][2][V][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t group = WS > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+    const int64_t pix = (group * 64 + lane) * V;
+    const bool live = pix < p.P;
+    const int64_t pc = live ? pix : 0;                 // dead lanes read pixel 0 and store nothing
+    const int64_t n = pc / p.m_size;
+    const int c0 = WS > 1 ? wave * p.per_wave : 0;
+    int cnt = WS > 1 ? p.C - c0 : p.C;
+    cnt = cnt < 1 ? 1 : (WS > 1 && cnt > p.per_wave ? p.per_wave : cnt);   // a split always leaves every wave >= 1 channel
+    cnt = __builtin_amdgcn_readfirstlane(cnt);
+    const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size + (int64_t)c0 * p.m_size;
+
+    // Slots past the wave's last channel re-read that channel (same address, served by cache) and are
+    // weighted out of the sums: straight-line code, no per-slot control flow.
+    typename PK::Raw raw[KW];
+#pragma unroll
+    for (int j = 0; j < KW; ++j) raw[j] = PK::load(x + base + (int64_t)(j < cnt ? j : cnt - 1) * p.m_size);
+
+    const float inv_c = 1.f / (float)p.C;
+    float mean[V], v[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < KW; ++j) s += j < cnt ? PK::get(raw[j], k) : 0.f;
+        const float mw = s / (float)cnt;
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < KW; ++j) {
+            const float d = j < cnt ? PK::get(raw[j], k) - mw : 0.f;
+            q = __builtin_fmaf(d, d, q);
+        }
+        if constexpr (WS > 1) {
+            ex[wave][0][k][lane] = mw;
+            ex[wave][1][k][lane] = q;
+        } else {
+            mean[k] = mw;
+            v[k] = q * inv_c + p.eps;
+        }
+    }
+    if constexpr (WS > 1) {
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float mw[WS], cw[WS], tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < WS; ++w) {
+                int c = p.C - w * p.per_wave;
+                c = c < 0 ? 0 : (c > p.per_wave ? p.per_wave : c);
+                cw[w] = (float)c;
+                mw[w] = ex[w][0][k][lane];
+                tot = __builtin_fmaf(cw[w], mw[w], tot);
+            }
+            const float m = tot * inv_c;
+            float m2 = 0.f;
+#pragma unroll
+            for (int w = 0; w < WS; ++w) {
+                const float d = mw[w] - m;
+                m2 += ex[w][1][k][lane] + cw[w] * d * d;
+            }
+            mean[k] = m;
+            v[k] = m2 * inv_c + p.eps;
+        }
+    }
+    float rstd[V], mv[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        rstd[k] = 1.f / sqrtf(v[k]);
+        mv[k] = mean[k] * v[k];
+    }
+
+    if constexpr (!Bwd) {
+#pragma unroll
+        for (int j = 0; j < KW; ++j) {
+            float r[V];
+#pragma unroll
+            for (int k = 0; k < V; ++k) r[k] = (PK::get(raw[j], k) - mean[k]) * rstd[k];
+            if (live && j < cnt) PK::store(out + base + (int64_t)j * p.m_size, PK::put(r));
+        }
+    } else {
+        constexpr int kChunk = KW < 8 ? KW : 8;        // gradient slices in flight per trip
+#pragma unroll
+        for (int j0 = 0; j0 < KW; j0 += kChunk) {
+            typename PK::Raw graw[kChunk];
+#pragma unroll
+            for (int jj = 0; jj < kChunk; ++jj)
+                graw[jj] = PK::load(g + base + (int64_t)(j0 + jj < cnt ? j0 + jj : cnt - 1) * p.m_size);
+#pragma unroll
+            for (int jj = 0; jj < kChunk; ++jj) {
+                float r[V];
+#pragma unroll
+                for (int k = 0; k < V; ++k) {
+                    const float val = PK::get(raw[j0 + jj], k);
+                    const float inner = __builtin_fmaf((val - mean[k]) * (val - inv_c), mv[k], inv_c);
+                    r[k] = -rstd[k] * inner * PK::get(graw[jj], k);
+                }
+                if (live && j0 + jj < cnt) PK::store(out + base + (int64_t)(j0 + jj) * p.m_size, PK::put(r));
+            }
+        }
+    }
+}
+
+// Any C: G lanes share one slice and stride over it (G = 64: a wavefront per contiguous row;
+// G = 1: a lane per slice). Statistics from sums shifted by the slice's first element, which keeps
+// the one-pass variance well conditioned; the second sweep re-reads the slice through cache.
+template <class T, int G, bool Bwd>
+__global__ __launch_bounds__(256) void ln_group(const T *__restrict__ x, const T *__restrict__ g, T *__restrict__ out,
+                                                const LnParams p) {
+    constexpr int kPix = 256 / G;
+    const int sub = threadIdx.x % G, grp = threadIdx.x / G;
+    const float inv_c = 1.f / (float)p.C;
+    const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
+    for (int64_t rd = 0; rd < rounds; ++rd) {
+        const int64_t pix = (rd * gridDim.x + blockIdx.x) * kPix + grp;
+        const bool live = pix < p.P;
+        const int64_t pc = live ? pix : 0;
+        const int64_t n = pc / p.m_size;
+        const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
+        const float shift = load_one(x + base);
+        float s1 = 0.f, s2 = 0.f;
+        for (int j = sub; j < p.C; j += G) {
+            const float d = load_one(x + base + (int64_t)j * p.m_size) - shift;
+            s1 += d;
+            s2 = __builtin_fmaf(d, d, s2);
+        }
+        s1 = group_reduce<G>(s1, OpSum());
+        s2 = group_reduce<G>(s2, OpSum());
+        const float dm = s1 * inv_c;
+        const float mean = shift + dm;
+        const float var = fmaxf(s2 * inv_c - dm * dm, 0.f);
+        const float v = var + p.eps;
+        const float rstd = 1.f / sqrtf(v), mv = mean * v;
+        if (!live) continue;
+        for (int j = sub; j < p.C; j += G) {
+            const int64_t at = base + (int64_t)j * p.m_size;
+            const float val = load_one(x + at);
+            if constexpr (Bwd) {
+                const float inner = __builtin_fmaf((val - mean) * (val - inv_c), mv, inv_c);
+                store_one(out + at, -rstd * inner * load_one(g + at));
+            } else {
+                store_one(out + at, (val - mean) * rstd);
+            }
+        }
+    }
+}
+
+template <class T, bool Bwd>
+void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, int64_t m_size, float eps,
+               hipStream_t st) {
+    constexpr int VT = ElemTraits<T>::kVec;
+    LnParams p;
+    p.P = n_size * m_size;
+    p.m_size = m_size;
+    p.C = (int)dimsize;
+    p.eps = eps;
+    // Channels per wave: all of them up to 32, a quarter up to 64, an eighth beyond (smaller register
+    // chunks in more waves measured better: they overlap one wave's loads with another's stores).
+    // With 4 waves and C > 32, or 8 waves and C > 64, every wave holds at least one channel.
+    const int ws = dimsize > 64 ? 8 : (dimsize > 32 ? 4 : 1);
+    p.per_wave = (int)ceil_div(dimsize, ws);
+    if (m_size == 1 || dimsize > 1024) {
+        if (m_size == 1) {
+            hipLaunchKernelGGL((ln_group<T, 64, Bwd>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, x, g, out, p);
+        } else {
+            hipLaunchKernelGGL((ln_group<T, 1, Bwd>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, x, g, out, p);
+        }
+        return;
+    }
+    const bool vec = dimsize <= 512 && m_size % VT == 0 && !misaligned(x, VT * sizeof(T)) &&
+                     !misaligned(out, VT * sizeof(T)) && !(Bwd && misaligned(g, VT * sizeof(T)));
+    const int64_t groups = ceil_div(p.P, 64 * (vec ? VT : 1));
+    const unsigned grid = (unsigned)(ws > 1 ? groups : ceil_div(groups, 4));
+    const int slots = p.per_wave;
+#define PLH_LN(KW, VV, WS) \
+    hipLaunchKernelGGL((ln_regs<T, KW, VV, WS, Bwd>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
+#define PLH_LN_V(KW, WS) do { if (vec) PLH_LN(KW, VT, WS); else PLH_LN(KW, 1, WS); } while (0)
+    if (ws == 1) {
+        if (slots <= 8) PLH_LN_V(8, 1);
+        else if (slots <= 16) PLH_LN_V(16, 1);
+        else PLH_LN_V(32, 1);
+    } else if (ws == 4) {
+        PLH_LN_V(16, 4);
+    } else if (slots <= 16) PLH_LN_V(16, 8);
+    else if (slots <= 32) PLH_LN_V(32, 8);
+    else if (slots <= 64) PLH_LN_V(64, 8);
+    else PLH_LN(128, 1, 8);                            // 512 < C <= 1024: one pixel per lane
+#undef PLH_LN_V
+#undef PLH_LN
+}
+
+// Per-dtype entry, instantiated in layernorm_f32.hip / layernorm_f16.hip / layernorm_bf16.hip.
+template <class T>
+void ln_run_typed(bool bwd, const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, int64_t m_size, float eps,
+                  hipStream_t st) {
+    if (bwd) ln_launch<T, true>(x, g, out, n_size, dimsize, m_size, eps, st);
+    else ln_launch<T, false>(x, g, out, n_size, dimsize, m_size, eps, st);
+}
+
+#define PLH_LN_SIGNATURE(T) void ln_run_typed<T>(bool, const T *, const T *, T *, int64_t, int64_t, int64_t, float, hipStream_t);
+#define PLH_LN_EXTERN(T) extern template PLH_LN_SIGNATURE(T)
+#define PLH_LN_INSTANTIATE(T) template PLH_LN_SIGNATURE(T)
+
+}  // namespace plh

@@ -13,6 +13,7 @@ from .lovasz_softmax import LovaszSoftmaxV3, LovaszSoftmaxFunctionV3
 from .ohem_loss import OhemCELoss, OhemLargeMarginLoss, score_ohem_label
 from .one_hot import convert_to_one_hot, convert_to_one_hot_cu, OnehotEncoder
 from .soft_dice_loss import SoftDiceLossV3, SoftDiceLossV3Func
+from .layer_norm import LayerNormV3, LayerNormV3Func
 from .taylor_softmax import (TaylorSoftmaxV3, LogTaylorSoftmaxV3, TaylorCrossEntropyLossV3, TaylorSoftmaxFunc,
                              TaylorCrossEntropyFunctionV3, taylor_softmax_v3)
 
@@ -24,6 +25,7 @@ __all__ = [
     "OhemCELoss", "OhemLargeMarginLoss", "score_ohem_label",
     "convert_to_one_hot", "convert_to_one_hot_cu", "OnehotEncoder",
     "SoftDiceLossV3", "SoftDiceLossV3Func",
+    "LayerNormV3", "LayerNormV3Func",
     "TaylorSoftmaxV3", "LogTaylorSoftmaxV3", "TaylorCrossEntropyLossV3", "TaylorSoftmaxFunc",
     "TaylorCrossEntropyFunctionV3", "taylor_softmax_v3",
 ]

@@ -58,6 +58,8 @@ _SIGNATURES = {
     "plh_soft_dice_workspace_bytes": (_i64, [_i64, _i64]),
     "plh_soft_dice_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _f32, _p]),
     "plh_soft_dice_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _f32, _p]),
+    "plh_layer_norm_forward": (ctypes.c_int, [_p, _i32, _p, _i64, _i64, _i64, _f32, _p]),
+    "plh_layer_norm_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p]),
     "plh_onehot": (ctypes.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_stream_copy": (ctypes.c_int, [_p, _p, _i64, _p]),
 }
@@ -639,3 +641,28 @@ def stream_copy(src, dst):
     assert src.dtype == torch.float32 and dst.dtype == torch.float32 and src.numel() == dst.numel()
     assert src.is_contiguous() and dst.is_contiguous()
     _call(src, "plh_stream_copy", _ptr(src), _ptr(dst), src.numel())
+
+
+# ----------------------------------------------------------- layer norm ----
+
+def layer_norm_forward(x, eps):
+    """(N, C, M) normalised over C. -> (out, the contiguous input the backward reads, dtype tag)."""
+    _require_gpu("layernorm loss", x)                                  # csrc/layer_norm.cu:380
+    if x.dim() != 3:
+        raise RuntimeError("layer norm: expected a (N, C, M) tensor, got %s" % (tuple(x.shape),))
+    xc, tag = _logits(x)
+    out = torch.empty_like(xc)
+    if xc.numel():
+        n, c, m = xc.shape
+        _call(xc, "plh_layer_norm_forward", _ptr(xc), tag, _ptr(out), n, c, m, float(eps))
+    return out.to(_loss_dtype(x.dtype)), xc, tag
+
+
+def layer_norm_backward(grad_output, xc, tag, eps, dtype):
+    g = grad_output if grad_output.dtype == xc.dtype else grad_output.to(xc.dtype)
+    g = g.expand(xc.shape).contiguous()
+    out = torch.empty_like(xc)
+    if xc.numel():
+        n, c, m = xc.shape
+        _call(xc, "plh_layer_norm_backward", _ptr(g), _ptr(xc), tag, _ptr(out), n, c, m, float(eps))
+    return out if out.dtype == dtype else out.to(dtype)

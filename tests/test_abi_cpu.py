@@ -137,6 +137,15 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_soft_dice_forward(odd, 0, p, p, p, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -6
     assert lib.plh_soft_dice_backward(None, p, 0, p, p, p, 2, 8, 1.0, None) == -1
     assert lib.plh_soft_dice_backward(p, p, 0, p, None, p, 2, 8, 1.0, None) == -1
+    # layer norm
+    assert lib.plh_layer_norm_forward(None, 0, None, 0, 4, 4, 1e-6, None) == 0
+    assert lib.plh_layer_norm_forward(p, 5, p, 1, 4, 4, 1e-6, None) == -7
+    assert lib.plh_layer_norm_forward(p, 0, None, 1, 4, 4, 1e-6, None) == -1
+    assert lib.plh_layer_norm_forward(p, 0, p, -1, 4, 4, 1e-6, None) == -2
+    assert lib.plh_layer_norm_forward(odd, 0, p, 1, 4, 4, 1e-6, None) == -6
+    assert lib.plh_layer_norm_backward(None, p, 0, p, 1, 4, 4, 1e-6, None) == -1
+    assert lib.plh_layer_norm_backward(p, p, 0, None, 1, 4, 4, 1e-6, None) == -1
+    assert lib.plh_layer_norm_backward(odd, p, 0, p, 1, 4, 4, 1e-6, None) == -6
     # 16-bit logits need 2-byte alignment only; an odd address is still refused
     assert lib.plh_lsr_forward(ctypes.c_void_p(p.value + 1), 1, lp, p, 1, 2, 2, 255, 0.1, None) == -6
     assert lib.plh_reduce_workspace_bytes(100) == 8 * 16384
