@@ -157,7 +157,20 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
     if (vec) {
         const int64_t quads = P / 4;
         const plh_f4 *s4 = reinterpret_cast<const plh_f4 *>(scores);
-        for (int64_t i = gid; i < quads; i += stride) {
+        int64_t i = gid;
+        for (; i + 3 * stride < quads; i += 4 * stride) {        // four loads in flight per lane
+            plh_f4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(s4 + i + u * stride);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                hist_add(bins, v[u].x, high_mask, prefix, pass);
+                hist_add(bins, v[u].y, high_mask, prefix, pass);
+                hist_add(bins, v[u].z, high_mask, prefix, pass);
+                hist_add(bins, v[u].w, high_mask, prefix, pass);
+            }
+        }
+        for (; i < quads; i += stride) {
             const plh_f4 v = __builtin_nontemporal_load(s4 + i);
             hist_add(bins, v.x, high_mask, prefix, pass);
             hist_add(bins, v.y, high_mask, prefix, pass);
@@ -378,7 +391,9 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
     const int vec = !misaligned(scores, 16) && !misaligned(labels, 16) && !misaligned(out_labels, 16);
     if (k > 0) {
         hipLaunchKernelGGL(ohem_zero, dim3((kOhemZeroWords + 255) / 256), dim3(256), 0, st, tb.hist, kOhemZeroWords);
-        const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 2048 ? ceil_div(P, 256 * 16) : 2048);
+        // every block ends with one global atomic per non-empty bin, all blocks on the same few hundred
+        // addresses: 512 blocks (two per compute unit) measured 30 us faster than 2048 on 8 M scores
+        const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
         for (int pass = 0; pass < 3; ++pass) {
             hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, vec);
             hipLaunchKernelGGL(ohem_pick, dim3(1), dim3(256), 0, st, tb, pass, k);
