@@ -30,6 +30,14 @@ HBM_PEAK_GBPS = 8000.0
 # Only valid for the exact workload shape they were taken on; anything else reports null.
 MEASURED_TRAFFIC = {
     ("lsr", (8, 19, 1024, 1024)): {"forward": 704.8e6 + 33.6e6, "backward": 735.0e6 + 637.5e6},
+    # profiles/all_workloads_hbm_traffic.txt (KiB per dispatch x 1024; kernels launched with both kinds of
+    # upstream gradient are scaled from the dispatch-weighted average to the per-element launch timed here)
+    ("lmargin", (8, 19, 1024, 1024)): {"forward": (688217 + 32768) * 1024, "backward": (721019 + 622597) * 1024},
+    ("taylor", (8, 19, 1024, 1024)): {"forward": (688318 + 32768) * 1024, "backward": (721267 + 622674) * 1024},
+    ("focal", (16, 80, 128, 128)): {"forward": (163862 + 81920) * 1024, "backward": (245815 + 81920) * 1024},
+    ("dice", (64, 1, 1024, 1024)): {"forward": (524531 + 32) * 1024, "backward": (524369 + 262151) * 1024},
+    ("layernorm", (16, 256, 128, 128)): {"forward": (262298 + 262197) * 1024, "backward": (524469 + 262173) * 1024},
+    ("lovasz", (4, 19, 512, 1024)): {"backward": (327860 + 155681) * 1024},
 }
 
 WORKLOADS = {
@@ -417,8 +425,9 @@ def run_layernorm(steps, warmup, device, dtype):
     for key, fn, nbytes in (("forward", f, fwd), ("backward", b, bwd)):
         k_ms = time_kernel(fn)
         gbps = nbytes / (k_ms * 1e-3) / 1e9
+        traffic = MEASURED_TRAFFIC.get(("layernorm", shape), {}).get(key) if dtype == "f32" else None
         roof[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(k_ms, 4),
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic, "ms": round(k_ms, 4),
                      "algorithmic_bytes": nbytes}
     return dict(ms_per_step=ms, gbps=(fwd + bwd) / (ms * 1e-3) / 1e9, loss=float(y[0, 0, 0].item()), roofline=roof,
                 bytes=fwd + bwd, step_ms={"warm": {"median": round(ms, 4), "iters": steps, "input_sets": 1}})
