@@ -222,6 +222,17 @@ __device__ __forceinline__ bool keep_key(uint32_t key, uint32_t limit) { return 
 // Keys of class c that enter this pass.
 __device__ __forceinline__ int row_items(const SortArgs &a, int c) { return a.kept_in ? (int)a.kept_in[c] : a.P; }
 
+// Tile of this block. Workgroups go to the 8 XCDs round-robin, each with an L2 of its own; taking
+// the tiles of a class row in 8 contiguous chunks, one per XCD, puts neighbouring tiles behind the
+// same L2, where what they share merges: the table words of consecutive tiles (4-byte stores into
+// one sector) and the sectors in which one tile's run of a digit ends and the next tile's begins.
+// Only the tiles that hold keys are permuted (the rest of a pruned row exits at once, and would
+// leave the XCDs of the last chunks idle).
+__device__ __forceinline__ int sort_tile(int items) {
+    const int x = blockIdx.x, q = ((items + kSortTile - 1) / kSortTile) >> 3;
+    return x < 8 * q ? (x & 7) * q + (x >> 3) : x;
+}
+
 // Inclusive scan over the 64 lanes of a wave.
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
     const int lane = __lane_id();
@@ -302,7 +313,7 @@ template <bool Hot>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];
     __shared__ uint32_t counts_hot[Hot ? kSortWaves : 1][kRadix];
-    const int c = blockIdx.y, tile = blockIdx.x;
+    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
         (&counts[0][0])[i] = 0;
@@ -420,7 +431,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
     __shared__ uint32_t scan_tmp[kSortWaves];
 
-    const int c = blockIdx.y, tile = blockIdx.x;
+    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
@@ -539,7 +550,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     __shared__ uint32_t scan_tmp[kSortWaves];
     __shared__ float wave_loss[kSortWaves];
 
-    const int c = blockIdx.y, tile = blockIdx.x;
+    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
