@@ -58,7 +58,7 @@ WORKLOADS = {
                  "Bernoulli(0.3) labels, p=1 smooth=1"),
     "layernorm": dict(shape=(16, 256, 128, 128), desc="LayerNormV3Func fwd+bwd, fp32 (16,256,128,128) normalised over C, "
                       "eps=1e-6, per-element upstream gradient"),
-    "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss (relabel + CE fwd+bwd), fp32 logits (8,19,1024,1024) "
+    "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss fwd+bwd (relabelling and cross entropy in one forward pass), fp32 logits (8,19,1024,1024) "
                  "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }
 
@@ -86,9 +86,8 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     E = numel(shape)
     P = E // shape[1]
     b = ELEM_BYTES[dtype]
-    if name == "ohem":     # relabelling (logits + labels read, labels written), then the LSR-shaped loss
-        relabel = b * E + 8 * P + 8 * P
-        return relabel + b * E + 8 * P + 4 * P, b * E + 8 * P + 4 * P + b * E
+    if name == "ohem":     # forward: logits and labels in, new labels (and one loss) out; backward: logits, new labels, gradient
+        return b * E + 8 * P + 8 * P, b * E + 8 * P + b * E
     if name in ("lsr", "lmargin", "taylor"):
         fwd = b * E + 8 * P + 4 * P
         bwd = b * E + 8 * P + 4 * P + b * E
@@ -235,20 +234,26 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
     P = _native._ptr
     out = {}
     if name == "ohem":
-        # the relabelling entry point alone: logits and labels in, new labels out
+        # forward = relabelling + mean cross entropy in one entry point; backward = cross-entropy gradient on the new labels
         new_labels = torch.empty_like(labels)
-        scores = torch.empty(labels.numel(), dtype=torch.float32, device=x.device)
-        ws_bytes = int(lib.plh_ohem_workspace_bytes(labels.numel()))
+        scratch = torch.empty((2, labels.numel()), dtype=torch.float32, device=x.device)
+        loss = torch.empty((), dtype=torch.float32, device=x.device)
+        n_valid = torch.empty((), dtype=torch.int64, device=x.device)
+        grad = torch.empty_like(x)
+        ws_bytes = int(lib.plh_ohem_ce_workspace_bytes(labels.numel()))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-        nbytes = x.element_size() * x.numel() + 16 * labels.numel()
-        f = lambda: lib.plh_ohem_score_label(P(x), tag, P(labels), P(new_labels), P(scores), P(ws), ws_bytes, n, c, m,
-                                             255, 0.7, labels.numel() // 16, st())
-        assert f() == 0
-        ms = time_kernel(f)
-        gbps = nbytes / (ms * 1e-3) / 1e9
-        return {"relabel": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(ms, 4),
-                            "algorithmic_bytes": nbytes}}
+        f = lambda: lib.plh_ohem_ce_forward(P(x), tag, P(labels), P(new_labels), P(scratch[0]), P(scratch[1]), P(loss),
+                                            P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.7, labels.numel() // 16, st())
+        b = lambda: lib.plh_lsr_backward_scaled(P(x), tag, P(new_labels), P(loss), 1.0, P(n_valid), P(grad), n, c, m, 255,
+                                                0.0, st())
+        assert f() == 0 and b() == 0
+        for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
+            ms = time_kernel(fn)
+            gbps = nbytes / (ms * 1e-3) / 1e9
+            out[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "ms": round(ms, 4),
+                        "algorithmic_bytes": nbytes}
+        return out
     if name in ("lsr", "lmargin", "taylor"):
         losses = torch.empty(labels.shape, dtype=torch.float32, device=x.device)
         grad = torch.empty_like(x)

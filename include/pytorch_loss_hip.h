@@ -221,6 +221,25 @@ int plh_ohem_score_label(const void *logits, int32_t dtype, const int64_t *label
                          int64_t n_size, int64_t dimsize, int64_t m_size,
                          int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
 
+/* OhemCELoss.forward in one call (pytorch_loss/ohem_loss.py:22-30: score_ohem_label, then
+ * nn.CrossEntropyLoss(ignore_index, reduction='mean') on the new labels). The score pass already
+ * holds each pixel's log-sum-exp and target logit, so it also writes the pixel's cross entropy
+ * (pixel_ce, scratch of n_size*m_size floats like `scores`), and the relabelling pass adds up the
+ * kept pixels': the forward reads the logits once instead of twice. out_labels: the new labels
+ * (what the backward needs; plh_lsr_backward_scaled with smooth = 0 and divide_by = n_valid_out is
+ * the matching gradient). loss_out: fp32 mean over the pixels whose new label is not ignore_index
+ * (NaN if there are none), n_valid_out (may be NULL): their number. n_min >= n_size*m_size keeps
+ * every label. workspace: plh_ohem_ce_workspace_bytes(n_size*m_size) bytes, 256-byte aligned.
+ */
+int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels);
+
+int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int64_t *labels,
+                        int64_t *out_labels, float *scores, float *pixel_ce,
+                        float *loss_out, int64_t *n_valid_out,
+                        void *workspace, int64_t workspace_bytes,
+                        int64_t n_size, int64_t dimsize, int64_t m_size,
+                        int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
+
 /* ---- one-hot / label-smoothed targets -------------------------------------------------
  * Replaces one_hot_cpp.label_one_hot (csrc/one_hot_kernel.cu:265-350).
  * labels (n_size, m_size) int64 -> one_hot (n_size, dimsize, m_size) fp32: 0 in every channel of an

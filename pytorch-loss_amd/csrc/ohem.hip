@@ -35,15 +35,16 @@ __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)(
 
 template <class T, int CP, int V, bool Uniform>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
-                                                              float *__restrict__ scores, int64_t P, int64_t m_size,
-                                                              int C, int64_t ignore, unsigned xcd_run) {
+                                                              float *__restrict__ scores, float *__restrict__ ce,
+                                                              int64_t P, int64_t m_size, int C, int64_t ignore,
+                                                              unsigned xcd_run) {
     const PixelRef<V, Uniform> at(P, m_size, C, xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, C, m_size, raw);
     int64_t lb[V];
     load_labels<V>(lab + at.pix, lb);
-    float out[V];
+    float out[V], loss[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
@@ -51,30 +52,35 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
         float xv[CP];
         const float mx = widen_and_max<T, V, CP>(raw, k, C, xv);
         const float c = mx * kLog2e;
-        float s = 0.f, e_y = 0.f;
+        float s = 0.f, e_y = 0.f, x_y = mx;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, C)) {
                 const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
                 s += e;
                 e_y = (tgt == j) ? e : e_y;
+                x_y = (tgt == j) ? xv[j] : x_y;
             }
         // ignored pixels score 1 (ohem_label_kernel.cu:131-134); so does a label outside [0, C),
         // which the reference leaves undefined
         out[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s), 1.f);
+        // the pixel's cross entropy from the same sums, exact also where the score underflows
+        loss[k] = (tgt < 0) ? 0.f : __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, mx - x_y);
     }
     store_vec<V>(scores + at.pix, out);
+    if (ce) store_vec<V>(ce + at.pix, loss);
 }
 
 // Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).
 template <class T>
 __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
-                                                        float *__restrict__ scores, int64_t P, int64_t m_size, int C,
-                                                        int64_t ignore) {
+                                                        float *__restrict__ scores, float *__restrict__ ce, int64_t P,
+                                                        int64_t m_size, int C, int64_t ignore) {
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t lb = lab[pix];
         if (lb == ignore || lb < 0 || lb >= C) {
             scores[pix] = 1.f;
+            if (ce) ce[pix] = 0.f;
             continue;
         }
         const int64_t n = pix / m_size;
@@ -83,7 +89,9 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
         for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
         for (int j = 0; j < C; ++j) s += fast_exp(load_one(xs + (int64_t)j * m_size) - mx);
-        scores[pix] = fminf(fast_exp(load_one(xs + lb * m_size) - mx) / s, 1.f);
+        const float x_y = load_one(xs + lb * m_size);
+        scores[pix] = fminf(fast_exp(x_y - mx) / s, 1.f);
+        if (ce) ce[pix] = logf(s) + (mx - x_y);
     }
 }
 
@@ -263,10 +271,15 @@ __global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles,
     }
 }
 
+// With `part`, the block also leaves the sum of `ce` over the pixels that keep a label other than
+// `ignore`, and their number: the mean cross entropy of the relabelled batch needs no further pass
+// over the logits.
 __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ scores, const int64_t *__restrict__ lab,
                                                     int64_t *__restrict__ out, OhemTables tb, int P, uint32_t n_min,
-                                                    float thresh, int64_t ignore, int vec) {
+                                                    float thresh, int64_t ignore, int vec,
+                                                    const float *__restrict__ ce, Partials part) {
     __shared__ uint32_t wave_ties[4];
+    __shared__ float red[4];
     const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
     float s[4];
     uint32_t key[4];
@@ -301,6 +314,7 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
             before += tie ? 1u : 0u;
         }
     }
+    bool kept[4] = {false, false, false, false};
     if (vec && base + 3 < P) {
         const plh_l2 *in2 = reinterpret_cast<const plh_l2 *>(lab + base);
         plh_l2 *out2 = reinterpret_cast<plh_l2 *>(out + base);
@@ -309,11 +323,30 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
         b.x = drop[2] ? ignore : b.x; b.y = drop[3] ? ignore : b.y;
         __builtin_nontemporal_store(a, out2);
         __builtin_nontemporal_store(b, out2 + 1);
-        return;
+        kept[0] = a.x != ignore; kept[1] = a.y != ignore; kept[2] = b.x != ignore; kept[3] = b.y != ignore;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (base + k < P) {
+                const int64_t nl = drop[k] ? ignore : lab[base + k];
+                out[base + k] = nl;
+                kept[k] = nl != ignore;
+            }
     }
+    if (part.sum == nullptr) return;            // uniform over the grid
+    float mine = 0.f, cnt = 0.f;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-        if (base + k < P) out[base + k] = drop[k] ? ignore : lab[base + k];
+        if (kept[k]) {
+            mine += ce[base + k];
+            cnt += 1.f;
+        }
+    const float bs = block_sum_256(mine, red);
+    const float bc = block_sum_256(cnt, red);
+    if (threadIdx.x == 0) {
+        part.sum[blockIdx.x] = bs;
+        part.cnt[blockIdx.x] = (int)bc;
+    }
 }
 
 __global__ void ohem_copy_labels(const int64_t *__restrict__ in, int64_t *__restrict__ out, int64_t n) {
@@ -328,15 +361,15 @@ constexpr int64_t kOhemMaxPixels = ((int64_t)1 << 31) - kOhemTile;
 static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 static int64_t ohem_tiles(int64_t P) { return ceil_div(P > 0 ? P : 1, kOhemTile); }
 
-static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, int64_t n_size,
-                         int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st) {
+static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, float *ce,
+                         int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st) {
     const int64_t P = n_size * m_size;
     const int C = (int)dimsize;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, nullptr);
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce);
         if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const bool uni = vec && tiles_are_uniform(m_size, VT, sizeof(T));
@@ -346,17 +379,17 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
         if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                                    labels, scores, P, m_size, C, ignore_index, run);                                 \
+                                    labels, scores, ce, P, m_size, C, ignore_index, run);                             \
         else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, false>), dim3(grid), dim3(kRegsBlock), 0,    \
-                                         st, x, labels, scores, P, m_size, C, ignore_index, run);                     \
+                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run);                 \
         else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, false>), dim3(grid), dim3(kRegsBlock), 0, st, x,       \
-                                labels, scores, P, m_size, C, ignore_index, run);                                     \
+                                labels, scores, ce, P, m_size, C, ignore_index, run);                                 \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
         } else {
-            hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, P,
+            hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,
                                m_size, C, ignore_index);
         }
     });
@@ -373,7 +406,12 @@ static int check_workspace(const void *workspace, int64_t workspace_bytes, int64
 }
 
 static int launch_select(const float *scores, const int64_t *labels, int64_t *out_labels, void *workspace,
-                         int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st) {
+                         int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st,
+                         const float *ce = nullptr, Partials part = Partials{nullptr, nullptr}) {
+    if (n_min >= P && part.sum) {                // nothing is relabelled, the loss is still wanted
+        n_min = 0;
+        score_thresh = INFINITY;
+    }
     if (n_min >= P) {                            // csrc/ohem_label_kernel.cu:189: labels are returned as they are
         if (out_labels != labels)
             hipLaunchKernelGGL(ohem_copy_labels, dim3((unsigned)(ceil_div(P, 256) < 4096 ? ceil_div(P, 256) : 4096)),
@@ -402,7 +440,7 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, score_thresh);
     }
     hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, k,
-                       score_thresh, ignore_index, vec);
+                       score_thresh, ignore_index, vec, ce, part);
     return check_launch();
 }
 
@@ -421,7 +459,8 @@ extern "C" int plh_ohem_scores(const void *logits, int32_t dtype, const int64_t 
     const int rc = check_slice_args(logits, labels, scores, n_size, dimsize, m_size, dtype_size(dtype), 4);
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
-    return launch_scores(logits, dtype, labels, scores, n_size, dimsize, m_size, ignore_index, (hipStream_t)stream);
+    return launch_scores(logits, dtype, labels, scores, nullptr, n_size, dimsize, m_size, ignore_index,
+                         (hipStream_t)stream);
 }
 
 extern "C" int plh_ohem_select_labels(const float *scores, const int64_t *labels, int64_t *out_labels,
@@ -452,9 +491,48 @@ extern "C" int plh_ohem_score_label(const void *logits, int32_t dtype, const int
     if (n_min < P) {
         if (!scores) return PLH_ERR_NULL_POINTER;
         if (misaligned(scores, 4)) return PLH_ERR_MISALIGNED;
-        rc = launch_scores(logits, dtype, labels, scores, n_size, dimsize, m_size, ignore_index, (hipStream_t)stream);
+        rc = launch_scores(logits, dtype, labels, scores, nullptr, n_size, dimsize, m_size, ignore_index,
+                           (hipStream_t)stream);
         if (rc != PLH_OK) return rc;
     }
     return launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min,
                          (hipStream_t)stream);
+}
+
+extern "C" int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels) {
+    if (n_pixels < 0 || n_pixels > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
+    return select_workspace(n_pixels) + align256(8 * ohem_tiles(n_pixels));
+}
+
+extern "C" int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int64_t *labels, int64_t *out_labels,
+                                   float *scores, float *pixel_ce, float *loss_out, int64_t *n_valid_out,
+                                   void *workspace, int64_t workspace_bytes,
+                                   int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                   float score_thresh, int64_t n_min, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    int rc = check_slice_args(logits, labels, out_labels, n_size, dimsize, m_size, dtype_size(dtype), 8);
+    if (rc != PLH_OK) return rc;
+    if (n_size * m_size > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
+    if (!loss_out) return PLH_ERR_NULL_POINTER;
+    if (misaligned(loss_out, 4) || misaligned(n_valid_out, 8)) return PLH_ERR_MISALIGNED;
+    const int64_t P = n_size * m_size;
+    hipStream_t st = (hipStream_t)stream;
+    if (n_size * dimsize * m_size == 0) {        // the mean over no pixels, as the other reduced entry points give it
+        finish_partials(Partials{nullptr, nullptr}, 0, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
+        return check_launch();
+    }
+    if (!scores || !pixel_ce) return PLH_ERR_NULL_POINTER;
+    if (misaligned(scores, 4) || misaligned(pixel_ce, 4)) return PLH_ERR_MISALIGNED;
+    if (!workspace || misaligned(workspace, 256) || workspace_bytes < plh_ohem_ce_workspace_bytes(P))
+        return PLH_ERR_WORKSPACE;
+    const int64_t tiles = ohem_tiles(P);
+    Partials part;
+    part.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P));
+    part.cnt = reinterpret_cast<int *>(part.sum + tiles);
+    rc = launch_scores(logits, dtype, labels, scores, pixel_ce, n_size, dimsize, m_size, ignore_index, st);
+    if (rc != PLH_OK) return rc;
+    rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_ce, part);
+    if (rc != PLH_OK) return rc;
+    finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
+    return check_launch();
 }

@@ -51,6 +51,9 @@ _SIGNATURES = {
     "plh_ohem_scores": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "plh_ohem_select_labels": (ctypes.c_int, [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _i64, _p]),
     "plh_ohem_score_label": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64, _p]),
+    "plh_ohem_ce_workspace_bytes": (_i64, [_i64]),
+    "plh_ohem_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64,
+                                           _p]),
     "plh_taylor_softmax_forward": (ctypes.c_int, [_p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
@@ -492,6 +495,26 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
     _call(a.x, "plh_ohem_score_label", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(out), _ptr(scores), _ptr(ws), ws_bytes,
           a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
     return out
+
+
+def ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min):
+    """Relabelling and mean cross entropy of what is left, with one pass over the logits.
+    -> (loss 0-dim, n_valid 0-dim int64, args whose labels are the NEW labels, for the backward)."""
+    a = ohem_args(logits, labels)
+    dev = a.x.device
+    n_pixels = a.n * a.m
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    n_valid = torch.empty((), dtype=torch.int64, device=dev)
+    new_labels = torch.empty_like(a.lb)
+    scratch = torch.empty((2, max(n_pixels, 1)), dtype=torch.float32, device=dev)
+    nbytes = int(load().plh_ohem_ce_workspace_bytes(n_pixels))
+    if nbytes < 0:
+        _check(nbytes)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
+    _call(a.x, "plh_ohem_ce_forward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(new_labels), _ptr(scratch[0]), _ptr(scratch[1]),
+          _ptr(loss), _ptr(n_valid), _ptr(ws), nbytes, a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
+    a.lb = new_labels
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, a
 
 
 # --------------------------------------------------------------- taylor ----

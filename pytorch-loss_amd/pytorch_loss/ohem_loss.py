@@ -3,15 +3,16 @@
 Same surface as the reference's pytorch_loss/ohem_loss.py:13-45: both modules first relabel the
 easy pixels as ignored (``score_ohem_label``: beyond the ``n_min`` lowest-scoring pixels, every
 pixel whose softmax probability at its label exceeds ``score_thresh`` gets ``ignore_index``),
-then take the mean loss over what is left.  ``OhemCELoss`` uses plain cross entropy, which is
-the label-smoothed kernel with a smoothing factor of 0 (the reference calls
-``nn.CrossEntropyLoss(ignore_index, reduction='mean')``, ohem_loss.py:20); ``OhemLargeMarginLoss``
-uses ``LargeMarginSoftmaxV3``.
+then take the mean loss over what is left.  ``OhemCELoss`` uses plain cross entropy (the reference calls
+``nn.CrossEntropyLoss(ignore_index, reduction='mean')``, ohem_loss.py:20): the relabelling pass over
+the logits already has every pixel's cross entropy at hand, so the forward is that one pass, and
+the backward is the label-smoothed kernel with a smoothing factor of 0 on the new labels;
+``OhemLargeMarginLoss`` uses ``LargeMarginSoftmaxV3``.
 """
+import torch
 import torch.nn as nn
 
 from . import _native
-from .label_smooth import LabelSmoothSoftmaxCEV3
 from .large_margin_softmax import LargeMarginSoftmaxV3
 
 
@@ -35,11 +36,28 @@ class _OhemLoss(nn.Module):
         return self.criteria(logits, labels)
 
 
+class _OhemCEFunction(torch.autograd.Function):
+    """Mean cross entropy over the pixels that keep their label; no gradient flows through the
+    relabelling (the reference runs it under no_grad, ohem_loss.py:25)."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, ignore_index, score_thresh, n_min):
+        loss, n_valid, args = _native.ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min)
+        ctx.vars = args, n_valid, ignore_index
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        args, n_valid, ignore_index = ctx.vars
+        grad = _native.lsr_backward_scaled(None, None, ignore_index, 0.0, grad_output, n_valid, args=args)
+        return grad, None, None, None, None
+
+
 class OhemCELoss(_OhemLoss):
 
-    def __init__(self, score_thresh, n_min=None, ignore_index=255):
-        super().__init__(score_thresh, n_min, ignore_index)
-        self.criteria = LabelSmoothSoftmaxCEV3(lb_smooth=0.0, reduction="mean", ignore_index=ignore_index)
+    def forward(self, logits, labels):
+        n_min = labels.numel() // 16 if self.n_min is None else self.n_min
+        return _OhemCEFunction.apply(logits, labels, self.ignore_lb, self.score_thresh, n_min)
 
 
 class OhemLargeMarginLoss(_OhemLoss):

@@ -137,6 +137,16 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_soft_dice_forward(odd, 0, p, p, p, wsp, dice_need, 2, 8, 1.0, 1.0, None) == -6
     assert lib.plh_soft_dice_backward(None, p, 0, p, p, p, 2, 8, 1.0, None) == -1
     assert lib.plh_soft_dice_backward(p, p, 0, p, None, p, 2, 8, 1.0, None) == -1
+    # fused OHEM cross entropy
+    ce_need = lib.plh_ohem_ce_workspace_bytes(5000)
+    assert ce_need >= lib.plh_ohem_workspace_bytes(5000) + 8 * 5 and ce_need % 256 == 0
+    assert lib.plh_ohem_ce_workspace_bytes(-1) == -2
+    assert lib.plh_ohem_ce_forward(p, 4, p, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -7
+    assert lib.plh_ohem_ce_forward(p, 0, None, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, None, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_ce_forward(p, 0, p, p, p, None, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, None, 0, 1, 4, 16, 255, 0.7, 1, None) == -5
+    assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, wsp, 16, 1, 4, 16, 255, 0.7, 1, None) == -5
     # layer norm
     assert lib.plh_layer_norm_forward(None, 0, None, 0, 4, 4, 1e-6, None) == 0
     assert lib.plh_layer_norm_forward(p, 5, p, 1, 4, 4, 1e-6, None) == -7

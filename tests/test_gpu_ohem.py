@@ -163,3 +163,34 @@ def test_ohem_refuses_cpu_tensors():
     y = torch.randint(0, 5, (2, 4, 4))
     with pytest.raises(RuntimeError, match="only supports gpu mode"):
         pl.OhemCELoss(0.7)(x, y)
+
+
+@pytest.mark.parametrize("case", ["n_min_covers_everything", "all_ignored", "huge_logit_gaps", "ragged"])
+def test_ohem_ce_fused_forward_edge_cases(native, case):
+    import pytorch_loss as pl
+    """The one-pass forward (scores and cross entropy from the same sums) against the oracle's
+    relabelling followed by torch's cross entropy."""
+    shape = (2, 7, 9, 11) if case == "ragged" else (2, 19, 16, 24)
+    x, y = seg_inputs(91, shape, 255, 0.05)
+    n_min, thresh = y.size // 16, 0.3
+    if case == "n_min_covers_everything":
+        n_min = y.size + 5
+    if case == "all_ignored":
+        y[...] = 255
+    if case == "huge_logit_gaps":
+        x = x * 60.0            # softmax at the label underflows to 0 for many pixels; their loss is ~1e2
+    xt = dev(x).requires_grad_()
+    loss = pl.OhemCELoss(score_thresh=thresh, n_min=n_min, ignore_index=255)(xt, dev(y))
+    new_labels = oracle.ohem_score_label(x, y, 255, thresh, n_min)
+    if case == "n_min_covers_everything":
+        assert np.array_equal(new_labels, y)
+    n_valid = int((new_labels != 255).sum())
+    if n_valid == 0:
+        assert torch.isnan(loss).item()        # the mean over no pixels, as nn.CrossEntropyLoss gives it
+        return
+    ce = torch.nn.functional.cross_entropy(torch.from_numpy(x).double(), torch.from_numpy(new_labels),
+                                           ignore_index=255, reduction="mean").item()
+    assert np.isfinite(loss.item()) and abs(loss.item() - ce) <= 1e-5 * abs(ce), (loss.item(), ce)
+    loss.backward()
+    want_g = oracle.lsr_backward(x, new_labels, 255, 0.0, np.float32(1.0 / n_valid))
+    close_grad(xt.grad.cpu().numpy(), want_g, case)
