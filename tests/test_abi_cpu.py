@@ -195,6 +195,43 @@ def test_constructor_defaults_match_the_reference():
         assert issubclass(getattr(pl, name), torch.autograd.Function)
 
 
+def test_neighbouring_ops_mirror_the_reference_surface():
+    # pytorch_loss/ohem_loss.py:15,32; one_hot.py:57-67; taylor_softmax.py:107,129,179; soft_dice_loss.py:117-123;
+    # layer_norm.py:114-121
+    import pytorch_loss as pl
+    o = pl.OhemCELoss(0.7)
+    assert (o.score_thresh, o.n_min, o.ignore_lb) == (0.7, None, 255)
+    o = pl.OhemLargeMarginLoss(0.6, n_min=10, ignore_index=-1)
+    assert (o.score_thresh, o.n_min, o.ignore_lb) == (0.6, 10, -1) and isinstance(o.criteria, pl.LargeMarginSoftmaxV3)
+    e = pl.OnehotEncoder(19)
+    assert (e.n_classes, e.lb_smooth, e.ignore_idx) == (19, 0., -1)
+    for cls in (pl.TaylorSoftmaxV3, pl.LogTaylorSoftmaxV3):
+        t = cls()
+        assert (t.dim, t.n) == (1, 2)
+    t = pl.TaylorCrossEntropyLossV3()
+    assert (t.n, t.ignore_index, t.reduction) == (2, -1, "mean")
+    d = pl.SoftDiceLossV3()
+    assert (d.p, d.smooth) == (1, 1.)
+    n = pl.LayerNormV3(8)
+    assert (n.n_chan, n.affine, n.eps) == (8, True, 1e-6)
+    assert n.weight.shape == (1, 8, 1) and n.bias.shape == (1, 8, 1)
+    assert torch.equal(n.weight.data, torch.ones(1, 8, 1)) and torch.equal(n.bias.data, torch.zeros(1, 8, 1))
+    assert pl.LayerNormV3(8, affine=False).weight is None
+    for name in ("TaylorSoftmaxFunc", "TaylorCrossEntropyFunctionV3", "SoftDiceLossV3Func", "LayerNormV3Func"):
+        assert issubclass(getattr(pl, name), torch.autograd.Function)
+    x = torch.randn(2, 5, 4, 4)
+    y = torch.randint(0, 5, (2, 4, 4))
+    for call in (lambda: pl.OhemCELoss(0.7)(x, y), lambda: pl.OhemLargeMarginLoss(0.7)(x, y),
+                 lambda: pl.OnehotEncoder(5)(y), lambda: pl.TaylorSoftmaxV3()(x), lambda: pl.LogTaylorSoftmaxV3()(x),
+                 lambda: pl.TaylorCrossEntropyLossV3()(x, y), lambda: pl.SoftDiceLossV3()(x, torch.rand_like(x)),
+                 lambda: pl.LayerNormV3(5)(x), lambda: pl.score_ohem_label(x, y, 255, 0.7, 2)):
+        with pytest.raises(RuntimeError, match="only supports gpu mode"):
+            call()
+    # odd Taylor orders are refused before anything is launched (csrc/taylor_softmax.cu:295)
+    with pytest.raises((RuntimeError, AssertionError)):
+        pl.TaylorSoftmaxV3(n=3)(x)
+
+
 def test_upstream_gradient_marshalling(native):
     like = (2, 3, 4)
     t, stride = native._upstream(None, like)
