@@ -11,7 +11,24 @@ __global__ __launch_bounds__(1024) void finish_kernel(const float *__restrict__ 
     __shared__ long long s_cnt[1024];
     double acc = 0.0;
     long long cnt = 0;
-    for (unsigned i = threadIdx.x; i < blocks; i += 1024) {
+    // eight partials per trip, loaded before the first is added: the trip count is small and each
+    // trip would otherwise wait out a full memory round trip (the order of the additions stays fixed)
+    unsigned i = threadIdx.x;
+    for (; i + 7 * 1024 < blocks; i += 8 * 1024) {
+        float v[8];
+        int n[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            v[u] = sums[i + u * 1024];
+            n[u] = cnts ? cnts[i + u * 1024] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            acc += (double)v[u];
+            cnt += n[u];
+        }
+    }
+    for (; i < blocks; i += 1024) {
         acc += (double)sums[i];
         if (cnts) cnt += cnts[i];
     }
