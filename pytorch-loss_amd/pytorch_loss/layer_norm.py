@@ -20,32 +20,29 @@ class LayerNormV3Func(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, eps):
-        out, xc, tag = _native.layer_norm_forward(x, eps)
-        ctx.vars = xc, tag, eps, x.dtype
-        return out
+        y, xc, tag = _native.layer_norm_forward(x, eps)
+        ctx.saved = (xc, tag, eps, x.dtype)
+        return y
 
     @staticmethod
     def backward(ctx, grad_output):
-        xc, tag, eps, dtype = ctx.vars
-        return _native.layer_norm_backward(grad_output, xc, tag, eps, dtype), None
+        return _native.layer_norm_backward(grad_output, *ctx.saved), None
 
 
 class LayerNormV3(nn.Module):
 
     def __init__(self, n_chan, affine=True, eps=1e-6):
         super().__init__()
-        self.n_chan, self.affine = n_chan, affine
-        self.weight, self.bias = None, None
+        self.n_chan = n_chan
+        self.affine = affine
         self.eps = eps
-        if affine:
-            self.weight = nn.Parameter(torch.ones(1, n_chan, 1))
-            self.bias = nn.Parameter(torch.zeros(1, n_chan, 1))
+        per_channel = (1, n_chan, 1)
+        self.weight = nn.Parameter(torch.ones(per_channel)) if affine else None
+        self.bias = nn.Parameter(torch.zeros(per_channel)) if affine else None
 
     def forward(self, x):
-        N, C, H, W = x.size()
-        x = x.view(N, C, -1)
-        dt = x.dtype
-        x = LayerNormV3Func.apply(x, self.eps).to(dt)
+        n, c, h, w = x.shape                     # NCHW only, like the reference
+        y = LayerNormV3Func.apply(x.view(n, c, h * w), self.eps).to(x.dtype)
         if self.affine:
-            x = self.weight * x + self.bias
-        return x.view(N, C, H, W)
+            y = self.weight * y + self.bias
+        return y.view(n, c, h, w)

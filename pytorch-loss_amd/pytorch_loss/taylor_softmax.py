@@ -17,46 +17,47 @@ import torch.nn as nn
 from . import _native
 
 
+def _even_order(n, strictly_positive=True):
+    """The reference asserts on the order where it is given (taylor_softmax.py:89, 110, 132, 182)."""
+    ok = n % 2 == 0 and (n > 0 or not strictly_positive)
+    assert ok, "the order of the Taylor polynomial must be even and positive"
+    return n
+
+
 class TaylorSoftmaxFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, feat, dim=1, n=2, use_log=False):
-        ctx.vars = feat, dim, n, use_log
-        return _native.taylor_softmax_forward(feat, dim, n, use_log)
+        ctx.call = (feat, dim, n, use_log)
+        return _native.taylor_softmax_forward(*ctx.call)
 
     @staticmethod
     def backward(ctx, grad_output):
-        feat, dim, n, use_log = ctx.vars
-        return _native.taylor_softmax_backward(grad_output, feat, dim, n, use_log), None, None, None
+        return (_native.taylor_softmax_backward(grad_output, *ctx.call),) + (None,) * 3
 
 
 def taylor_softmax_v3(inten, dim=1, n=4, use_log=False):
-    assert n % 2 == 0 and n > 0
-    return TaylorSoftmaxFunc.apply(inten, dim, n, use_log)
+    return TaylorSoftmaxFunc.apply(inten, dim, _even_order(n), use_log)
 
 
-class TaylorSoftmaxV3(nn.Module):
-
-    def __init__(self, dim=1, n=2):
-        super().__init__()
-        assert n % 2 == 0 and n > 0
-        self.dim = dim
-        self.n = n
-
-    def forward(self, x):
-        return taylor_softmax_v3(x, self.dim, self.n, use_log=False)
-
-
-class LogTaylorSoftmaxV3(nn.Module):
+class _TaylorAlongDim(nn.Module):
+    use_log = False
 
     def __init__(self, dim=1, n=2):
         super().__init__()
-        assert n % 2 == 0
-        self.dim = dim
-        self.n = n
+        self.dim, self.n = dim, _even_order(n, strictly_positive=not self.use_log)
 
     def forward(self, x):
-        return taylor_softmax_v3(x, self.dim, self.n, use_log=True)
+        return taylor_softmax_v3(x, self.dim, self.n, self.use_log)
+
+
+class TaylorSoftmaxV3(_TaylorAlongDim):
+    """Usage as ``nn.Softmax(dim)``."""
+
+
+class LogTaylorSoftmaxV3(_TaylorAlongDim):
+    """Usage as ``nn.LogSoftmax(dim)``."""
+    use_log = True
 
 
 class TaylorCrossEntropyFunctionV3(torch.autograd.Function):
@@ -82,10 +83,7 @@ class TaylorCrossEntropyLossV3(nn.Module):
 
     def __init__(self, n=2, ignore_index=-1, reduction='mean'):
         super().__init__()
-        assert n % 2 == 0
-        self.n = n
-        self.reduction = reduction
-        self.ignore_index = ignore_index
+        self.n, self.ignore_index, self.reduction = _even_order(n, strictly_positive=False), ignore_index, reduction
 
     def forward(self, logits, labels):
         return TaylorCrossEntropyFunctionV3.apply(logits, labels, self.n, self.ignore_index, self.reduction)
