@@ -153,3 +153,75 @@ def test_lovasz_rows_longer_than_the_staging_regions(pl):
     # many keys that are not left out, so the zero pattern is only comparable in fp32)
     _, j32 = oracle.lovasz_forward(x, y, 255)
     assert (jacc.view(np.uint32) == j32.view(np.uint32)).mean() > 0.99
+
+
+def test_neighbouring_ops_full_size(pl):
+    """Taylor cross entropy, the OHEM cross entropy, the target encoder and soft dice at the benchmark
+    shapes, against fp64 torch library routines evaluated on the same GPU tensors, and the first
+    image against the oracle."""
+    import torch.nn.functional as F
+    x, y = _seg_full("cfg2")
+    xt = torch.from_numpy(x).cuda()
+    yt = torch.from_numpy(y).cuda()
+    n_valid = int((y != 255).sum())
+
+    # target encoder: exact values everywhere
+    enc = pl.OnehotEncoder(19, lb_smooth=0.1, ignore_idx=255)(yt)
+    assert enc.shape == xt.shape
+    valid = (yt != 255)
+    assert torch.equal(enc.argmax(dim=1)[valid], yt[valid])
+    assert (enc.sum(dim=1)[~valid] == 0).all()
+    hot, cold = np.float32(1.0 - 0.1), np.float32(0.1 / 19)
+    assert int((enc == float(hot)).sum()) == n_valid and int((enc == float(cold)).sum()) == 18 * n_valid
+    assert np.array_equal(enc[:1].cpu().numpy(), oracle.onehot(y[:1], 19, 0.1, 255))
+    del enc
+
+    # Taylor cross entropy: -log of the order-4 series ratio, with torch ops in fp64 on one image at a time
+    leaf = xt.clone().requires_grad_()
+    loss = pl.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="sum")(leaf, yt)
+    want = 0.0
+    for i in range(xt.shape[0]):
+        xd = xt[i:i + 1].double()
+        f = 1 + xd + xd ** 2 / 2 + xd ** 3 / 6 + xd ** 4 / 24
+        want += F.nll_loss((f / f.sum(dim=1, keepdim=True)).log(), yt[i:i + 1], ignore_index=255, reduction="sum").item()
+    assert abs(loss.item() - want) <= 1e-5 * abs(want)
+    loss.backward()
+    g = leaf.grad
+    assert (g.permute(0, 2, 3, 1)[~valid] == 0).all()
+    want_g = oracle.taylor_ce_backward(x[:1], y[:1], 4, 255, np.float32(1.0))
+    assert np.abs(g[:1].cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max()
+    del leaf, g, loss
+
+    # OHEM cross entropy: the fused forward against torch's cross entropy on the relabelled batch
+    n_min = y.size // 16
+    leaf = xt.clone().requires_grad_()
+    loss = pl.OhemCELoss(score_thresh=0.7, n_min=n_min, ignore_index=255)(leaf, yt)
+    new_labels = pl.score_ohem_label(xt, yt, 255, 0.7, n_min)
+    kept = int((new_labels != 255).sum())
+    assert n_min <= kept < n_valid
+    want = sum(F.cross_entropy(xt[i:i + 1].double(), new_labels[i:i + 1], ignore_index=255, reduction="sum").item()
+               for i in range(xt.shape[0])) / kept
+    assert abs(loss.item() - want) <= 1e-5 * abs(want)
+    loss.backward()
+    gone = (new_labels == 255)
+    assert (leaf.grad.permute(0, 2, 3, 1)[gone] == 0).all()
+    rows = leaf.grad.permute(0, 2, 3, 1)[~gone].double().sum(dim=1)
+    assert rows.abs().max().item() <= 1e-6 / kept * 19
+    del leaf, rows
+
+    # soft dice at (64, 1, 1024, 1024) as one row
+    g = torch.Generator(device="cuda").manual_seed(3)
+    dx = (torch.randn((64, 1, 1024, 1024), device="cuda", generator=g) * 2.0).requires_grad_()
+    dy = (torch.rand(dx.shape, device="cuda", generator=g) < 0.3).float()
+    for p in (1, 2):
+        dx.grad = None
+        loss = pl.SoftDiceLossV3(p=p, smooth=1.0)(dx, dy)
+        loss.backward()
+        q = torch.sigmoid(dx.detach().double())
+        numer = 2 * (q * dy).sum() + 1.0
+        denor = (q.pow(p) + dy.double().pow(p)).sum() + 1.0
+        want = (1 - numer / denor).item()
+        assert abs(loss.item() - want) <= 1e-5 * abs(want)
+        want_g = p * q.pow(p) * (1 - q) * numer / denor ** 2 - 2 * dy * q * (1 - q) / denor
+        assert (dx.grad.double() - want_g).abs().max().item() <= 1e-5 * want_g.abs().max().item()
+        del q, want_g
