@@ -295,7 +295,16 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         f = lambda: lib.plh_lovasz_forward(P(x), tag, P(labels), P(losses), P(jacc), P(ws), ws_bytes, n, c, m, 255, st())
         b = lambda: lib.plh_lovasz_backward(P(gout), P(x), tag, P(labels), P(jacc), P(grad), n, c, m, 255, st())
     assert f() == 0 and b() == 0
-    for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
+    legs = [("forward", f, fwd_bytes), ("backward", b, bwd_bytes)]
+    if name == "taylor":
+        # the softmax Function itself (TaylorSoftmaxV3 / LogTaylorSoftmaxV3): x in, y out; grad and x in, grad out
+        y_out = torch.empty_like(x)
+        eb = x.element_size() * x.numel()
+        sf = lambda: lib.plh_taylor_softmax_forward(P(x), tag, P(y_out), n, c, m, 4, 1, st())
+        sb = lambda: lib.plh_taylor_softmax_backward(P(y_out), P(x), tag, P(grad), n, c, m, 4, 1, st())
+        assert sf() == 0 and sb() == 0
+        legs += [("log_softmax_forward", sf, 2 * eb), ("log_softmax_backward", sb, 3 * eb)]
+    for key, fn, nbytes in legs:
         ms = time_kernel(fn)
         gbps = nbytes / (ms * 1e-3) / 1e9
         traffic = MEASURED_TRAFFIC.get((name, shape), {}).get(key) if dtype == "f32" else None
@@ -532,6 +541,8 @@ def main():
                          kernel="backward entry point of the workload" if "backward" in main_res["roofline"]
                          else "the workload's single entry point"),
         "roofline_forward": main_res["roofline"].get("forward"),
+        "roofline_kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
+                             for k, v in main_res["roofline"].items()},
         "step_ms": main_res["step_ms"],
         "copy_kernel_GBps": ceiling,
         "other_workloads": others,

@@ -292,6 +292,13 @@ template <class T> struct Pack<T, 1> {          // T = f16 or bf16
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[1]) { return keep[0]; }
 };
 
+// Makes a packed slice element opaque to the optimiser: what is computed from it afterwards is not
+// merged with what was computed from it before (used between two sweeps over a register-resident
+// slice, where keeping every first-sweep intermediate alive would cost far more registers than
+// the second evaluation costs instructions).
+__device__ __forceinline__ void forget_origin(unsigned &r) { asm volatile("" : "+v"(r)); }
+__device__ __forceinline__ void forget_origin(plh_u2 &r) { asm volatile("" : "+v"(r.x), "+v"(r.y)); }
+
 // A regs kernel is instantiated for CP = channels rounded up to a multiple of 4, and launched only
 // for CP-3 <= C <= CP: the first CP-3 channel slots always exist, the last three are checked.
 template <int CP>

@@ -104,8 +104,9 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
     typename Pack<T, V>::Raw raw[CP], graw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     at.load_slice(g, p.C, p.m_size, graw);
-    // the series is cheap: it is evaluated again in the second sweep rather than kept in registers
-    float r[CP][V];
+    // the series is cheap: it is evaluated again in the second sweep rather than kept in registers,
+    // and the second sweep goes channel by channel so that only one packed result is live at a time
+    float inv[V], mid[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         float s = 0.f, dot = 0.f;
@@ -118,20 +119,28 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
                 s += f;
                 dot += p.use_log ? gj : f * gj;
             }
-        const float inv = 1.f / s;
-        const float mid = p.use_log ? dot * inv : dot * inv * inv;       // csrc/taylor_softmax.cu:163-173
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) {
-                float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
-                const float gj = Pack<T, V>::get(graw[j], k);
-                r[j][k] = p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
-            }
+        inv[k] = 1.f / s;
+        mid[k] = p.use_log ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(r[j]);
+        if (chan_ok<CP>(j, p.C)) {
+            forget_origin(raw[j]);
+            forget_origin(graw[j]);
+        }
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, p.C)) {
+            float r[V];
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                const float gj = Pack<T, V>::get(graw[j], k);
+                r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
+            }
+            raw[j] = Pack<T, V>::put(r);
+        }
     at.store_slice(gx, p.C, p.m_size, raw);
 }
 
@@ -191,13 +200,16 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
     load_labels<V>(lab + at.pix, lb);
     float go[V];
     load_upstream<V>(up, at.pix, go);
-    float r[CP][V];
+    // first per pixel (sum of the series, the target's term), then channel by channel so that only one
+    // packed result is live at a time
     unsigned keep[V];
+    int tgt[V];
+    float scale[V], hot[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        keep[k] = (ign || tgt < 0) ? 0u : 0xFFFFFFFFu;
+        tgt[k] = narrow_label(lb[k], p.ignore, p.C, ign);
+        keep[k] = (ign || tgt[k] < 0) ? 0u : 0xFFFFFFFFu;
         float s = 0.f, f_y = 1.f;
 #pragma unroll
         for (int j = 0; j < CP; ++j)
@@ -205,23 +217,28 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
                 float f, df;
                 taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 s += f;
-                f_y = (tgt == j) ? f : f_y;
+                f_y = (tgt[k] == j) ? f : f_y;
             }
-        const float scale = go[k] * __builtin_amdgcn_rcpf(s);
-        float hot = go[k] / f_y;                                   // per pixel
-        asm("" : "+v"(hot));
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) {
-                float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
-                r[j][k] = df * ((tgt == j) ? scale - hot : scale);
-            }
+        scale[k] = go[k] * __builtin_amdgcn_rcpf(s);
+        hot[k] = scale[k] - go[k] / f_y;                           // per pixel: what the target channel takes
+        asm("" : "+v"(hot[k]));
     }
     const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(r[j]) & mask;
+        if (chan_ok<CP>(j, p.C)) forget_origin(raw[j]);
+#pragma unroll
+    for (int j = 0; j < CP; ++j)
+        if (chan_ok<CP>(j, p.C)) {
+            float r[V];
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                r[k] = df * ((tgt[k] == j) ? hot[k] : scale[k]);
+            }
+            raw[j] = Pack<T, V>::put(r) & mask;
+        }
     at.store_slice(gx, p.C, p.m_size, raw);
 }
 
