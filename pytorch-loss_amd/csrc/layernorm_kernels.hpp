@@ -60,6 +60,10 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
 #pragma unroll
         for (int j = 0; j < KW; ++j) s += j < cnt ? PK::get(raw[j], k) : 0.f;
         const float mw = s / (float)cnt;
+        // every sweep widens the packed slice again: kept apart for the optimiser, which would
+        // otherwise hold all widened values of the first sweep in registers for the later ones
+#pragma unroll
+        for (int j = 0; j < KW; ++j) forget_origin(raw[j]);
         float q = 0.f;
 #pragma unroll
         for (int j = 0; j < KW; ++j) {
@@ -104,6 +108,8 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
         rstd[k] = 1.f / sqrtf(v[k]);
         mv[k] = mean[k] * v[k];
     }
+#pragma unroll
+    for (int j = 0; j < KW; ++j) forget_origin(raw[j]);
 
     if constexpr (!Bwd) {
 #pragma unroll

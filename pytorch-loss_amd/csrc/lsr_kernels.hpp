@@ -104,36 +104,46 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
     float go[V];
     load_upstream<V>(up, at.pix, go);
 
-    float g[CP][V];
+    // The gradient of a pixel replaces its logits in the slice as soon as they are no longer needed
+    // (one pixel at a time for fp32, two for 16-bit elements, which share a dword): no second array.
+    using PK = Pack<T, V>;
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        keep[k] = ign ? 0u : 0xFFFFFFFFu;
-        float xv[CP];
-        const float mx = widen_and_max<T, V, CP>(raw, k, p.C, xv);
-        const float c = mx * kLog2e;
-        float s = 0.f;
+    for (int k0 = 0; k0 < V; k0 += PK::kStep) {
+        float g[CP][PK::kStep];
+#pragma unroll
+        for (int kk = 0; kk < PK::kStep; ++kk) {
+            const int k = k0 + kk;
+            bool ign;
+            const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+            keep[k] = ign ? 0u : 0xFFFFFFFFu;
+            float xv[CP];
+            const float mx = widen_and_max<T, V, CP>(raw, k, p.C, xv);
+            const float c = mx * kLog2e;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, p.C)) {
+                    xv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
+                    s += xv[j];
+                }
+            const float gk = go[k];
+            const float scale = p.sumw * gk * __builtin_amdgcn_rcpf(s);     // one reciprocal per pixel
+            float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+            asm("" : "+v"(n_pos), "+v"(n_neg));                             // formed per pixel, not per channel
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, p.C)) g[j][kk] = __builtin_fmaf(xv[j], scale, (tgt == j) ? n_pos : n_neg);
+        }
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) {
-                xv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
-                s += xv[j];
-            }
-        const float gk = go[k];
-        const float scale = p.sumw * gk * __builtin_amdgcn_rcpf(s);     // one reciprocal per pixel
-        float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
-        asm("" : "+v"(n_pos), "+v"(n_neg));                             // formed per pixel, not per channel
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) g[j][k] = __builtin_fmaf(xv[j], scale, (tgt == j) ? n_pos : n_neg);
+            if (chan_ok<CP>(j, p.C)) PK::set(raw[j], k0 / PK::kStep, g[j]);
     }
     // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
-    const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
+    const typename PK::Raw mask = PK::mask(keep);
 #pragma unroll
     for (int j = 0; j < CP; ++j)
-        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(g[j]) & mask;
+        if (chan_ok<CP>(j, p.C)) raw[j] = raw[j] & mask;
     at.store_slice(grad, p.C, p.m_size, raw);
 }
 

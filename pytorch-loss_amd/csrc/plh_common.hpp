@@ -230,6 +230,13 @@ template <> struct Pack<float, 2> {
     }
     static __device__ __forceinline__ float get(Raw r, int k) { return bits_f32(k == 0 ? r.x : r.y); }
     static __device__ __forceinline__ Raw put(const float (&g)[2]) { return Raw{f32_bits(g[0]), f32_bits(g[1])}; }
+    // In-place update: pixels [k, k + kStep) of a slice element are replaced by results. A kernel that
+    // is done with the inputs of those pixels writes its outputs over them and needs no second array.
+    static constexpr int kStep = 1;
+    static __device__ __forceinline__ void set(Raw &r, int k, const float (&g)[1]) {
+        if (k == 0) r.x = f32_bits(g[0]);
+        else r.y = f32_bits(g[0]);
+    }
     // AND-mask that clears pixel k of a packed gradient when keep[k] is 0 (keep[k] is 0 or ~0)
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[2]) { return Raw{keep[0], keep[1]}; }
 };
@@ -243,6 +250,8 @@ template <> struct Pack<float, 1> {
     }
     static __device__ __forceinline__ float get(Raw r, int) { return bits_f32(r); }
     static __device__ __forceinline__ Raw put(const float (&g)[1]) { return f32_bits(g[0]); }
+    static constexpr int kStep = 1;
+    static __device__ __forceinline__ void set(Raw &r, int, const float (&g)[1]) { r = f32_bits(g[0]); }
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[1]) { return keep[0]; }
 };
 
@@ -275,6 +284,11 @@ template <class T> struct Pack<T, 4> {          // T = f16 or bf16
     static __device__ __forceinline__ Raw put(const float (&g)[4]) {
         return Raw{narrow2(g[0], g[1], T{}), narrow2(g[2], g[3], T{})};
     }
+    static constexpr int kStep = 2;              // a dword holds two pixels
+    static __device__ __forceinline__ void set(Raw &r, int k, const float (&g)[2]) {
+        if (k == 0) r.x = narrow2(g[0], g[1], T{});
+        else r.y = narrow2(g[0], g[1], T{});
+    }
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[4]) {
         return Raw{(keep[0] & 0xFFFFu) | (keep[1] & 0xFFFF0000u), (keep[2] & 0xFFFFu) | (keep[3] & 0xFFFF0000u)};
     }
@@ -289,6 +303,8 @@ template <class T> struct Pack<T, 1> {          // T = f16 or bf16
     }
     static __device__ __forceinline__ float get(Raw r, int) { return widen_lo(r, T{}); }
     static __device__ __forceinline__ Raw put(const float (&g)[1]) { return narrow2(g[0], 0.f, T{}) & 0xFFFFu; }
+    static constexpr int kStep = 1;
+    static __device__ __forceinline__ void set(Raw &r, int, const float (&g)[1]) { r = narrow2(g[0], 0.f, T{}) & 0xFFFFu; }
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[1]) { return keep[0]; }
 };
 
