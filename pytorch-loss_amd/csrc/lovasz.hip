@@ -263,6 +263,32 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *lds, u
     return before + incl - v;
 }
 
+// Two independent exclusive scans behind one pair of barriers. lds must hold 2 * kSortWaves words.
+__device__ __forceinline__ void block_excl_scan2(uint32_t a, uint32_t b, uint32_t *lds, uint32_t &excl_a,
+                                                 uint32_t &total_a, uint32_t &excl_b, uint32_t &total_b) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t incl_a = wave_incl_scan(a), incl_b = wave_incl_scan(b);
+    if (lane == 63) {
+        lds[wave] = incl_a;
+        lds[kSortWaves + wave] = incl_b;
+    }
+    __syncthreads();
+    uint32_t before_a = 0, all_a = 0, before_b = 0, all_b = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) {
+        const uint32_t ta = lds[w], tb = lds[kSortWaves + w];
+        before_a += (w < wave) ? ta : 0u;
+        before_b += (w < wave) ? tb : 0u;
+        all_a += ta;
+        all_b += tb;
+    }
+    total_a = all_a;
+    total_b = all_b;
+    excl_a = before_a + incl_a - a;
+    excl_b = before_b + incl_b - b;
+    __syncthreads();
+}
+
 // Match mask: the valid lanes of the wave whose digit equals this lane's. One ballot per digit bit;
 // each lane ORs up, in two 32-bit halves, the lanes that differ from it in that bit
 // (vote XOR own bit splatted), so a bit costs one field extract, one compare and two 3-input bit ops.
@@ -429,22 +455,22 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];   // per-wave digit counts, then exclusive over waves
     __shared__ uint32_t digit_start[kRadix];          // first local position of each digit
     __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
-    __shared__ uint32_t scan_tmp[kSortWaves];
+    __shared__ uint32_t scan_tmp[2 * kSortWaves];
 
     const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
     if (count <= 0) return;                     // block-uniform: the row ends before this tile
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
-    __syncthreads();
 
     const uint32_t limit = keep_limit(a, c);
     const int64_t row = (int64_t)c * a.P;
     const uint32_t *kin = a.keys_in + row + begin;
     const uint32_t *vin = a.vals_in ? a.vals_in + row + begin : nullptr;
 
-    // keys beyond the row's end read as ignored, which keep_key never lets through
+    // Every global read of the block is issued up front, so that the table entries (needed only after
+    // the ranking) and the keys travel together. Keys beyond the row's end read as ignored, which
+    // keep_key never lets through.
     uint32_t key[kSortItems], val[kSortItems], rank[kSortItems];
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
@@ -453,6 +479,13 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
         key[r] = valid ? kin[li] : kIgnoredKey;
         val[r] = vin ? (valid ? vin[li] : 0u) : (uint32_t)(begin + li);
     }
+    uint32_t dtot = 0, tile_before = 0;         // thread d < kRadix: digit d's total in the row, and in the tiles before this one
+    if (threadIdx.x < kRadix) {
+        dtot = a.digit_total[(int64_t)c * kRadix + threadIdx.x];
+        tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile];
+    }
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    __syncthreads();
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
@@ -468,7 +501,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 
     uint32_t n_local;                           // keys of this tile that take part
     {
-        uint32_t mine = 0, dtot = 0;
+        uint32_t mine = 0;
         const int d = threadIdx.x;
         if (d < kRadix) {
             uint32_t run = 0;
@@ -479,14 +512,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
                 run += t;
             }
             mine = run;
-            dtot = a.digit_total[(int64_t)c * kRadix + d];
         }
-        uint32_t row_total;
-        const uint32_t local_start = block_excl_scan(mine, scan_tmp, n_local);
-        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, row_total);
+        uint32_t row_total, local_start, global_start;
+        block_excl_scan2(mine, dtot, scan_tmp, local_start, n_local, global_start, row_total);
         if (d < kRadix) {
             digit_start[d] = local_start;
-            out_base[d] = global_start + a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
+            out_base[d] = global_start + tile_before;
         }
         // the digit totals of the row add up to the keys this pass lets through
         if (a.kept_out && tile == 0 && threadIdx.x == 0) a.kept_out[c] = row_total;
@@ -547,7 +578,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     __shared__ uint32_t counts_hot[kSortWaves][kRadix];
     __shared__ uint32_t out_base[kRadix];     // global position of the tile's first key with digit d
     __shared__ uint32_t hot_base[kRadix];     // positives sorted before that position
-    __shared__ uint32_t scan_tmp[kSortWaves];
+    __shared__ uint32_t scan_tmp[2 * kSortWaves];
     __shared__ float wave_loss[kSortWaves];
 
     const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
@@ -558,18 +589,11 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         if (threadIdx.x == 0) tile_loss[(int64_t)c * a.tiles + tile] = 0.f;
         return;
     }
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
-        (&counts[0][0])[i] = 0;
-        (&counts_hot[0][0])[i] = 0;
-    }
-    if constexpr (Binned)
-        for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
-    __syncthreads();
-
     const int64_t row = (int64_t)c * a.P;
     const uint32_t *kin = a.keys_in + row + begin;
     const uint32_t *vin = a.vals_in + row + begin;
 
+    // every global read of the block is issued up front (the table entries are needed only after the ranking)
     uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], hrank[kSortItems];
     uint32_t slot[Binned ? kSortItems : 1];
 #pragma unroll
@@ -579,6 +603,21 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         key[r] = valid ? kin[li] : kIgnoredKey;
         val[r] = valid ? vin[li] : 0u;
     }
+    uint32_t dtot = 0, htot = 0, tile_before = 0, hot_before = 0;
+    if (threadIdx.x < kRadix) {
+        const int64_t at = (int64_t)c * kRadix + threadIdx.x;
+        dtot = a.digit_total[at];
+        htot = a.hot_total[at];
+        tile_before = a.tile_hist[at * a.tiles + tile];
+        hot_before = a.tile_hot[at * a.tiles + tile];
+    }
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
+        (&counts[0][0])[i] = 0;
+        (&counts_hot[0][0])[i] = 0;
+    }
+    if constexpr (Binned)
+        for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
+    __syncthreads();
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
@@ -609,7 +648,6 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 
     uint32_t n_pos_u;
     {
-        uint32_t dtot = 0, htot = 0;
         const int d = threadIdx.x;
         if (d < kRadix) {
             uint32_t run = 0, run_hot = 0;
@@ -621,15 +659,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                 run += t;
                 run_hot += th;
             }
-            dtot = a.digit_total[(int64_t)c * kRadix + d];
-            htot = a.hot_total[(int64_t)c * kRadix + d];
         }
-        uint32_t total;
-        const uint32_t global_start = block_excl_scan(dtot, scan_tmp, total);
-        const uint32_t hot_start = block_excl_scan(htot, scan_tmp, n_pos_u);
+        uint32_t total, global_start, hot_start;
+        block_excl_scan2(dtot, htot, scan_tmp, global_start, total, hot_start, n_pos_u);
         if (d < kRadix) {
-            out_base[d] = global_start + a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile];
-            hot_base[d] = hot_start + a.tile_hot[((int64_t)c * kRadix + d) * a.tiles + tile];
+            out_base[d] = global_start + tile_before;
+            hot_base[d] = hot_start + hot_before;
         }
     }
     __syncthreads();
