@@ -37,8 +37,8 @@ constexpr uint32_t kOne = 0x3F800000u;          // bits of 1.0f
 constexpr uint32_t kIgnoredKey = 0x7FFFFFFFu;
 constexpr uint32_t kHotBit = 0x80000000u;
 
-constexpr int kSortThreads = 256;
-constexpr int kSortItems = 16;
+constexpr int kSortThreads = 512;
+constexpr int kSortItems = 8;
 constexpr int kSortTile = kSortThreads * kSortItems;   // 4096 keys per block
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kRadix = 256;
