@@ -720,17 +720,35 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 
 // One block per (region, class): the region's staged values (as many as its cursor counted) are
 // permuted to pixel order inside LDS; pixels whose keys stayed out of the sort get their exact 0.
-__global__ __launch_bounds__(256) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
-                                                 const uint32_t *__restrict__ cursors, int regions, int P) {
-    __shared__ float sorted[kRegion];
+constexpr int kUnbinThreads = 1024;
+
+__global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
+                                                           const uint32_t *__restrict__ cursors, int regions, int P) {
+    typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) float sorted[kRegion];
     const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
     const int n = min(kRegion, P - (int)(blockIdx.x << kRegionBits));
     const int staged = min(n, (int)cursors[(int64_t)blockIdx.y * regions + blockIdx.x]);
-    for (int i = threadIdx.x; i < n; i += 256) sorted[i] = 0.f;
+    // 16-byte accesses where the region starts on a 16-byte boundary (rows of a multiple of 4 pixels)
+    const bool vec = (first & 3) == 0;
+    const int staged_v = vec ? (staged & ~3) : 0, n_v = vec ? (n & ~3) : 0;
+    plh_f4 *sorted4 = reinterpret_cast<plh_f4 *>(sorted);
+    for (int i = threadIdx.x; i < kRegion / 4; i += kUnbinThreads) sorted4[i] = plh_f4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
-    for (int i = threadIdx.x; i < staged; i += 256) sorted[idx_stage[first + i] & (kRegion - 1)] = jacc[first + i];
+    for (int i = threadIdx.x * 4; i < staged_v; i += kUnbinThreads * 4) {
+        const plh_u4 at = __builtin_nontemporal_load(reinterpret_cast<const plh_u4 *>(idx_stage + first + i));
+        const plh_f4 v = __builtin_nontemporal_load(reinterpret_cast<const plh_f4 *>(jacc + first + i));
+        sorted[at.x & (kRegion - 1)] = v.x;
+        sorted[at.y & (kRegion - 1)] = v.y;
+        sorted[at.z & (kRegion - 1)] = v.z;
+        sorted[at.w & (kRegion - 1)] = v.w;
+    }
+    for (int i = staged_v + threadIdx.x; i < staged; i += kUnbinThreads)
+        sorted[idx_stage[first + i] & (kRegion - 1)] = jacc[first + i];
     __syncthreads();
-    for (int i = threadIdx.x; i < n; i += 256) jacc[first + i] = sorted[i];
+    for (int i = threadIdx.x * 4; i < n_v; i += kUnbinThreads * 4)
+        __builtin_nontemporal_store(sorted4[i / 4], reinterpret_cast<plh_f4 *>(jacc + first + i));
+    for (int i = n_v + threadIdx.x; i < n; i += kUnbinThreads) jacc[first + i] = sorted[i];
 }
 
 __global__ __launch_bounds__(256) void lov_zero_f32(float *p, int64_t n) {
@@ -1000,7 +1018,7 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         // vals_b is free by now: it receives the pixel offsets that go with the staged values
         hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
                            pl.regions);
-        hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(256), 0, st, jacc, vals_b,
+        hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(kUnbinThreads), 0, st, jacc, vals_b,
                            cursors, pl.regions, (int)pl.P);
     } else {
         // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
