@@ -309,8 +309,8 @@ __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
 // through the wave's private counters, this round through the match mask). With Hot, the same for
 // the positives only (hrank = positives with this digit before this key).
 template <bool Hot>
-__device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, uint32_t *counts,
-                                          uint32_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
+__device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, uint16_t *counts,
+                                          uint16_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
     const int lane = __lane_id();
     const uint64_t peers = wave_peers(digit, valid);
     const uint64_t below = (1ull << lane) - 1ull;
@@ -320,10 +320,10 @@ __device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, 
     if constexpr (Hot) hot_peers = peers & __builtin_amdgcn_ballot_w64(hot && valid);
     if (valid && lane == leader) {
         seen = counts[digit];
-        counts[digit] = seen + __builtin_popcountll(peers);
+        counts[digit] = (uint16_t)(seen + __builtin_popcountll(peers));
         if constexpr (Hot) {
             seen_hot = counts_hot[digit];
-            counts_hot[digit] = seen_hot + __builtin_popcountll(hot_peers);
+            counts_hot[digit] = (uint16_t)(seen_hot + __builtin_popcountll(hot_peers));
         }
     }
     rank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen) + __builtin_popcountll(peers & below);
@@ -452,7 +452,10 @@ __global__ __launch_bounds__(256) void lov_row_scan(uint32_t *table0, uint32_t *
 __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t s_keys[kSortTile];
     __shared__ uint32_t s_vals[kSortTile];
-    __shared__ uint32_t counts[kSortWaves][kRadix];   // per-wave digit counts, then exclusive over waves
+    // per-wave digit counts, then exclusive over waves: never more than the tile's 4096 keys, so 16 bits
+    // do (only a wave's leader lane updates an entry, with plain loads and stores); the smaller tables
+    // let one more block fit a CU's LDS
+    __shared__ __align__(4) uint16_t counts[kSortWaves][kRadix];
     __shared__ uint32_t digit_start[kRadix];          // first local position of each digit
     __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
     __shared__ uint32_t scan_tmp[2 * kSortWaves];
@@ -484,7 +487,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
         dtot = a.digit_total[(int64_t)c * kRadix + threadIdx.x];
         tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile];
     }
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 #pragma unroll
             for (int w = 0; w < kSortWaves; ++w) {
                 const uint32_t t = counts[w][d];
-                counts[w][d] = run;
+                counts[w][d] = (uint16_t)run;
                 run += t;
             }
             mine = run;
@@ -570,12 +573,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                                                           uint32_t *__restrict__ idx_stage,
                                                           uint32_t *__restrict__ cursors, int regions) {
     __shared__ uint32_t region_cnt[Binned ? kMaxRegions : 1];    // keys of this tile per region
-    __shared__ uint32_t region_start[Binned ? kMaxRegions : 1];  // first position of the region in the re-ordered tile
+    __shared__ uint16_t region_start[Binned ? kMaxRegions : 1];  // first position of the region in the re-ordered tile (< 4096)
     __shared__ uint32_t region_base[Binned ? kMaxRegions : 1];   // this tile's run inside the region's staging range
     __shared__ float s_dj[Binned ? kSortTile : 1];               // tile re-ordered by region, so that the stores
     __shared__ uint32_t s_val[Binned ? kSortTile : 1];           // of neighbouring threads fall into the same run
-    __shared__ uint32_t counts[kSortWaves][kRadix];
-    __shared__ uint32_t counts_hot[kSortWaves][kRadix];
+    __shared__ __align__(4) uint16_t counts[kSortWaves][kRadix];       // 16 bits: see lov_scatter
+    __shared__ __align__(4) uint16_t counts_hot[kSortWaves][kRadix];
     __shared__ uint32_t out_base[kRadix];     // global position of the tile's first key with digit d
     __shared__ uint32_t hot_base[kRadix];     // positives sorted before that position
     __shared__ uint32_t scan_tmp[2 * kSortWaves];
@@ -611,9 +614,9 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         tile_before = a.tile_hist[at * a.tiles + tile];
         hot_before = a.tile_hot[at * a.tiles + tile];
     }
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
-        (&counts[0][0])[i] = 0;
-        (&counts_hot[0][0])[i] = 0;
+    for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) {
+        reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
+        reinterpret_cast<uint32_t *>(&counts_hot[0][0])[i] = 0;
     }
     if constexpr (Binned)
         for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
@@ -640,7 +643,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         uint32_t run = block_excl_scan(mine, scan_tmp, total);
         for (int i = r0; i < min(regions, r0 + per); ++i) {
             const uint32_t n = region_cnt[i];
-            region_start[i] = run;
+            region_start[i] = (uint16_t)run;
             run += n;
             region_base[i] = n ? atomicAdd(&cursors[(int64_t)c * regions + i], n) : 0u;
         }
@@ -654,8 +657,8 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 #pragma unroll
             for (int w = 0; w < kSortWaves; ++w) {
                 const uint32_t t = counts[w][d], th = counts_hot[w][d];
-                counts[w][d] = run;
-                counts_hot[w][d] = run_hot;
+                counts[w][d] = (uint16_t)run;
+                counts_hot[w][d] = (uint16_t)run_hot;
                 run += t;
                 run_hot += th;
             }
