@@ -749,8 +749,9 @@ __global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ j
     for (int i = staged_v + threadIdx.x; i < staged; i += kUnbinThreads)
         sorted[idx_stage[first + i] & (kRegion - 1)] = jacc[first + i];
     __syncthreads();
+    // plain stores: the backward reads these values next, and what the caches keep of them helps it
     for (int i = threadIdx.x * 4; i < n_v; i += kUnbinThreads * 4)
-        __builtin_nontemporal_store(sorted4[i / 4], reinterpret_cast<plh_f4 *>(jacc + first + i));
+        *reinterpret_cast<plh_f4 *>(jacc + first + i) = sorted4[i / 4];
     for (int i = n_v + threadIdx.x; i < n; i += kUnbinThreads) jacc[first + i] = sorted[i];
 }
 
