@@ -149,13 +149,8 @@ __global__ __launch_bounds__(kRegsBlock) void lov_keys_regs(const T *__restrict_
     if (live) {
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, C)) {
-                // plain stores: the radix passes read the keys next, partly out of the last-level cache
-                float *dst = reinterpret_cast<float *>(keys) + (int64_t)j * P + pix;
-                if constexpr (V == 1) *dst = v[j][0];
-                else if constexpr (V == 2) *reinterpret_cast<plh_f2 *>(dst) = plh_f2{v[j][0], v[j][1]};
-                else *reinterpret_cast<plh_f4 *>(dst) = plh_f4{v[j][0], v[j][1], v[j][2], v[j][3]};
-            }
+            // cache-allocating stores: the radix passes read the keys next, partly out of the last-level cache
+            if (chan_ok<CP>(j, C)) store_vec_cached<V>(reinterpret_cast<float *>(keys) + (int64_t)j * P + pix, v[j]);
     }
     __syncthreads();
     publish_block_max(block_max, block_table, C);

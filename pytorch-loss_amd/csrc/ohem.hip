@@ -67,8 +67,9 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
         // the pixel's cross entropy from the same sums, exact also where the score underflows
         loss[k] = (tgt < 0) ? 0.f : __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, mx - x_y);
     }
-    store_vec<V>(scores + at.pix, out);
-    if (ce) store_vec<V>(ce + at.pix, loss);
+    // the selection kernels read both back several times: leave them to the caches
+    store_vec_cached<V>(scores + at.pix, out);
+    if (ce) store_vec_cached<V>(ce + at.pix, loss);
 }
 
 // Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
         for (; i + 3 * stride < quads; i += 4 * stride) {        // four loads in flight per lane
             plh_f4 v[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(s4 + i + u * stride);
+            for (int u = 0; u < 4; ++u) v[u] = s4[i + u * stride];     // scores are read again: ordinary loads
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 hist_add(bins, v[u].x, high_mask, prefix, pass);
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
             }
         }
         for (; i < quads; i += stride) {
-            const plh_f4 v = __builtin_nontemporal_load(s4 + i);
+            const plh_f4 v = s4[i];
             hist_add(bins, v.x, high_mask, prefix, pass);
             hist_add(bins, v.y, high_mask, prefix, pass);
             hist_add(bins, v.z, high_mask, prefix, pass);
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(256) void ohem_pick(OhemTables tb, int pass, uint32
 __device__ __forceinline__ void load_tile_keys(const float *scores, int P, int base, bool vec, float (&s)[4],
                                                uint32_t (&key)[4]) {
     if (vec && base + 3 < P) {
-        const plh_f4 v = __builtin_nontemporal_load(reinterpret_cast<const plh_f4 *>(scores + base));
+        const plh_f4 v = *reinterpret_cast<const plh_f4 *>(scores + base);
         s[0] = v.x; s[1] = v.y; s[2] = v.z; s[3] = v.w;
 #pragma unroll
         for (int k = 0; k < 4; ++k) key[k] = score_key(s[k]);

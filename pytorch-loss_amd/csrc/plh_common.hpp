@@ -153,6 +153,19 @@ __device__ __forceinline__ void store_vec(float *p, const float (&v)[V]) {
     }
 }
 
+// Same, with ordinary (cache-allocating) stores: for intermediates that the next kernel reads back
+// and that are small enough for the last-level cache to keep.
+template <int V>
+__device__ __forceinline__ void store_vec_cached(float *p, const float (&v)[V]) {
+    if constexpr (V == 1) {
+        *p = v[0];
+    } else if constexpr (V == 2) {
+        *reinterpret_cast<plh_f2 *>(p) = plh_f2{v[0], v[1]};
+    } else {
+        *reinterpret_cast<plh_f4 *>(p) = plh_f4{v[0], v[1], v[2], v[3]};
+    }
+}
+
 typedef unsigned short plh_h2 __attribute__((ext_vector_type(2)));
 typedef unsigned short plh_h4 __attribute__((ext_vector_type(4)));
 
