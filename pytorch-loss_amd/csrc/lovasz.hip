@@ -42,6 +42,7 @@ constexpr int kSortItems = 8;
 constexpr int kSortTile = kSortThreads * kSortItems;   // 4096 keys per block
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kRadix = 256;
+constexpr int kRankGroup = 2;     // rounds whose match masks are formed together (see lov_scatter)
 
 __device__ __forceinline__ uint32_t make_key(float prob, bool hot, bool ignored) {
     const float err = hot ? fabsf(1.f - prob) : fabsf(prob);
@@ -292,13 +293,15 @@ __device__ __forceinline__ void block_excl_scan2(uint32_t a, uint32_t b, uint32_
 
 // Match mask: the valid lanes of the wave whose digit equals this lane's. One ballot per digit bit;
 // each lane ORs up, in two 32-bit halves, the lanes that differ from it in that bit
-// (vote XOR own bit splatted), so a bit costs one field extract, one compare and two 3-input bit ops.
+// (vote XOR own bit splatted), so a bit costs one field extract, one compare, two XORs and its share
+// of two 3-input ORs.
 __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
     uint32_t diff_lo = 0, diff_hi = 0;
 #pragma unroll
     for (int b = 0; b < 8; ++b) {
-        const uint32_t splat = (uint32_t)((int32_t)(digit << (31 - b)) >> 31);   // bit b splatted: 0 or ~0
-        const uint64_t vote = __builtin_amdgcn_ballot_w64((digit & (1u << b)) != 0u);
+        uint32_t splat = (uint32_t)((int32_t)(digit << (31 - b)) >> 31);   // bit b splatted: 0 or ~0
+        asm("" : "+v"(splat));      // the vote is taken from the splat itself: one field extract serves both
+        const uint64_t vote = __builtin_amdgcn_ballot_w64(splat != 0u);
         diff_lo |= (uint32_t)vote ^ splat;
         diff_hi |= (uint32_t)(vote >> 32) ^ splat;
     }
@@ -310,10 +313,9 @@ __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
 // through the wave's private counters, this round through the match mask). With Hot, the same for
 // the positives only (hrank = positives with this digit before this key).
 template <bool Hot>
-__device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, uint16_t *counts,
-                                          uint16_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
+__device__ __forceinline__ void wave_rank_of(uint64_t peers, uint32_t digit, bool valid, bool hot, uint16_t *counts,
+                                             uint16_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
     const int lane = __lane_id();
-    const uint64_t peers = wave_peers(digit, valid);
     const uint64_t below = (1ull << lane) - 1ull;
     const int leader = peers ? (__builtin_ffsll((long long)peers) - 1) : lane;
     uint32_t seen = 0, seen_hot = 0;
@@ -331,6 +333,12 @@ __device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, 
     if constexpr (Hot)
         hrank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen_hot) +
                 __builtin_popcountll(hot_peers & below);
+}
+
+template <bool Hot>
+__device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, uint16_t *counts,
+                                          uint16_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
+    wave_rank_of<Hot>(wave_peers(digit, valid), digit, valid, hot, counts, counts_hot, rank, hrank);
 }
 
 // Per-tile digit counts (and, for the last pass, the same for the positives). Counting needs no
@@ -490,16 +498,36 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     }
     for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
     __syncthreads();
+    // kRankGroup rounds at a time: their match masks do not depend on each other, so the compiler can fill
+    // the wait between a vote and its use in one round with the other round's instructions; only the
+    // counter updates have to follow the rounds' order.
+    static_assert(kSortItems % kRankGroup == 0, "rounds are ranked in groups");
 #pragma unroll
-    for (int r = 0; r < kSortItems; ++r) {
-        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
-        const bool valid = li < count && keep_key(key[r], limit);
-        if (__builtin_amdgcn_ballot_w64(valid) == 0) {      // wave-uniform: nothing of this round takes part
-            rank[r] = 0;
+    for (int r = 0; r < kSortItems; r += kRankGroup) {
+        bool valid[kRankGroup];
+        uint32_t digit[kRankGroup];
+        uint64_t peers[kRankGroup];
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) {
+            const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
+            valid[h] = li < count && keep_key(key[r + h], limit);
+            digit[h] = (key[r + h] >> a.shift) & a.digit_mask;
+        }
+        bool any = false;
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) any = any || valid[h];
+        if (__builtin_amdgcn_ballot_w64(any) == 0) {        // wave-uniform: nothing of these rounds takes part
+#pragma unroll
+            for (int h = 0; h < kRankGroup; ++h) rank[r + h] = 0;
             continue;
         }
-        uint32_t unused;
-        wave_rank<false>((key[r] >> a.shift) & a.digit_mask, valid, false, counts[wave], nullptr, rank[r], unused);
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) peers[h] = wave_peers(digit[h], valid[h]);
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) {
+            uint32_t unused;
+            wave_rank_of<false>(peers[h], digit[h], valid[h], false, counts[wave], nullptr, rank[r + h], unused);
+        }
     }
     __syncthreads();
 
@@ -623,13 +651,22 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         for (int i = threadIdx.x; i < regions; i += kSortThreads) region_cnt[i] = 0;
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < kSortItems; ++r) {
-        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
-        wave_rank<true>((key[r] >> a.shift) & a.digit_mask, li < count, key[r] >> 31, counts[wave], counts_hot[wave],
-                        rank[r], hrank[r]);
-        if constexpr (Binned) {
-            // order inside a region's staging range is irrelevant: lov_unbin puts every value at its pixel
-            if (li < count) slot[r] = atomicAdd(&region_cnt[val[r] >> kRegionBits], 1u);
+    for (int r = 0; r < kSortItems; r += kRankGroup) {      // in groups, as in lov_scatter
+        uint64_t peers[kRankGroup];
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) {
+            const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
+            peers[h] = wave_peers((key[r + h] >> a.shift) & a.digit_mask, li < count);
+        }
+#pragma unroll
+        for (int h = 0; h < kRankGroup; ++h) {
+            const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
+            wave_rank_of<true>(peers[h], (key[r + h] >> a.shift) & a.digit_mask, li < count, key[r + h] >> 31, counts[wave],
+                               counts_hot[wave], rank[r + h], hrank[r + h]);
+            if constexpr (Binned) {
+                // order inside a region's staging range is irrelevant: lov_unbin puts every value at its pixel
+                if (li < count) slot[r + h] = atomicAdd(&region_cnt[val[r + h] >> kRegionBits], 1u);
+            }
         }
     }
     __syncthreads();
