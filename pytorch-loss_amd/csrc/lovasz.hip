@@ -312,27 +312,38 @@ __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
 // Stable rank of this lane's key among the equal digits the wave has seen so far (earlier rounds
 // through the wave's private counters, this round through the match mask). With Hot, the same for
 // the positives only (hrank = positives with this digit before this key).
+// Peers of this lane that sit in lower lanes: the masked bit count does the AND with "lanes below me"
+// and the population count in two instructions.
+__device__ __forceinline__ uint32_t peers_below(uint64_t peers) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+}
+
 template <bool Hot>
 __device__ __forceinline__ void wave_rank_of(uint64_t peers, uint32_t digit, bool valid, bool hot, uint16_t *counts,
                                              uint16_t *counts_hot, uint32_t &rank, uint32_t &hrank) {
-    const int lane = __lane_id();
-    const uint64_t below = (1ull << lane) - 1ull;
-    const int leader = peers ? (__builtin_ffsll((long long)peers) - 1) : lane;
-    uint32_t seen = 0, seen_hot = 0;
+    // Every lane of a group reads the group's counter (one LDS address: a broadcast), then the group's
+    // first lane moves it on. LDS executes a wave's instructions in issue order, so the reads see the
+    // value from before this round, and the next round's reads see the update.
+    const uint32_t before = peers_below(peers);
     uint64_t hot_peers = 0;
-    if constexpr (Hot) hot_peers = peers & __builtin_amdgcn_ballot_w64(hot && valid);
-    if (valid && lane == leader) {
-        seen = counts[digit];
-        counts[digit] = (uint16_t)(seen + __builtin_popcountll(peers));
-        if constexpr (Hot) {
-            seen_hot = counts_hot[digit];
-            counts_hot[digit] = (uint16_t)(seen_hot + __builtin_popcountll(hot_peers));
-        }
+    uint32_t hot_before = 0;
+    if constexpr (Hot) {
+        hot_peers = peers & __builtin_amdgcn_ballot_w64(hot && valid);
+        hot_before = peers_below(hot_peers);
     }
-    rank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen) + __builtin_popcountll(peers & below);
-    if constexpr (Hot)
-        hrank = (uint32_t)__builtin_amdgcn_ds_bpermute(leader << 2, (int)seen_hot) +
-                __builtin_popcountll(hot_peers & below);
+    uint32_t seen = 0, seen_hot = 0;
+    if (valid) {
+        seen = counts[digit];
+        if constexpr (Hot) seen_hot = counts_hot[digit];
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (valid && before == 0u) {
+        counts[digit] = (uint16_t)(seen + __builtin_popcountll(peers));
+        if constexpr (Hot) counts_hot[digit] = (uint16_t)(seen_hot + __builtin_popcountll(hot_peers));
+    }
+    __builtin_amdgcn_wave_barrier();
+    rank = seen + before;
+    if constexpr (Hot) hrank = seen_hot + hot_before;
 }
 
 template <bool Hot>
@@ -466,7 +477,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     // let one more block fit a CU's LDS
     __shared__ __align__(4) uint16_t counts[kSortWaves][kRadix];
     __shared__ uint32_t digit_start[kRadix];          // first local position of each digit
-    __shared__ uint32_t out_base[kRadix];             // first global position of each digit of this tile
+    __shared__ uint32_t out_base[kRadix];             // global minus local position of each digit's run in this tile
     __shared__ uint32_t scan_tmp[2 * kSortWaves];
 
     const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
@@ -549,7 +560,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
         block_excl_scan2(mine, dtot, scan_tmp, local_start, n_local, global_start, row_total);
         if (d < kRadix) {
             digit_start[d] = local_start;
-            out_base[d] = global_start + tile_before;
+            out_base[d] = global_start + tile_before - local_start;   // global position minus local one (mod 2^32)
         }
         // the digit totals of the row add up to the keys this pass lets through
         if (a.kept_out && tile == 0 && threadIdx.x == 0) a.kept_out[c] = row_total;
@@ -573,7 +584,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     for (int i = threadIdx.x; i < (int)n_local; i += kSortThreads) {
         const uint32_t k = s_keys[i];
         const uint32_t d = (k >> a.shift) & a.digit_mask;
-        const uint32_t dst = out_base[d] + ((uint32_t)i - digit_start[d]);
+        const uint32_t dst = out_base[d] + (uint32_t)i;
         kout[dst] = k;
         vout[dst] = s_vals[i];
     }
