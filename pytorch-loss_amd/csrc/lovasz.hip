@@ -67,9 +67,12 @@ __device__ __forceinline__ void publish_block_max(const uint32_t *block_max, uin
 }
 
 __global__ __launch_bounds__(256) void lov_class_max(const uint32_t *__restrict__ block_table, int blocks, int C,
-                                                     uint32_t *__restrict__ pos_max) {
+                                                     uint32_t *__restrict__ pos_max, uint32_t *__restrict__ cursors,
+                                                     int regions) {
     __shared__ uint32_t wave_max[4];
     const int c = blockIdx.x;
+    // the class's staging cursors start at zero (they are first used by the last pass)
+    for (int i = threadIdx.x; i < regions; i += 256) cursors[(int64_t)c * regions + i] = 0;
     uint32_t m = 0;
     for (int b = threadIdx.x; b < blocks; b += 256) m = max(m, block_table[(int64_t)b * C + c]);
 #pragma unroll
@@ -775,7 +778,9 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 constexpr int kUnbinThreads = 1024;
 
 __global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
-                                                           const uint32_t *__restrict__ cursors, int regions, int P) {
+                                                           const uint32_t *__restrict__ cursors, int regions, int P,
+                                                           const float *__restrict__ tile_loss, float *__restrict__ losses,
+                                                           int tiles) {
     typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
     __shared__ __align__(16) float sorted[kRegion];
     const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
@@ -802,15 +807,25 @@ __global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ j
     for (int i = threadIdx.x * 4; i < n_v; i += kUnbinThreads * 4)
         *reinterpret_cast<plh_f4 *>(jacc + first + i) = sorted4[i / 4];
     for (int i = n_v + threadIdx.x; i < n; i += kUnbinThreads) jacc[first + i] = sorted[i];
+
+    // the first block of a class also adds up the class's per-tile shares of the loss, in a fixed order
+    if (blockIdx.x != 0) return;
+    __syncthreads();                                // `sorted` is free again
+    const int c = blockIdx.y;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < tiles; i += kUnbinThreads) sum += tile_loss[(int64_t)c * tiles + i];
+    sum = group_reduce<64>(sum, OpSum());
+    if ((threadIdx.x & 63) == 0) sorted[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int w = 0; w < kUnbinThreads / 64; ++w) total += sorted[w];
+        losses[c] = total;
+    }
 }
 
 __global__ __launch_bounds__(256) void lov_zero_f32(float *p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0.f;
-}
-
-__global__ __launch_bounds__(256) void lov_zero_u32(uint32_t *p, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0;
 }
 
 __global__ __launch_bounds__(256) void lov_reduce_loss(const float *__restrict__ tile_loss, float *__restrict__ losses,
@@ -1015,7 +1030,8 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
                                pl.P, m_size, C, ignore_index);
         }
     });
-    hipLaunchKernelGGL(lov_class_max, dim3((unsigned)C), dim3(256), 0, st, block_table, (int)key_blocks, C, pos_max);
+    hipLaunchKernelGGL(lov_class_max, dim3((unsigned)C), dim3(256), 0, st, block_table, (int)key_blocks, C, pos_max,
+                       reinterpret_cast<uint32_t *>(ws + pl.off_cursors), pl.regions);
     hipLaunchKernelGGL(lov_absent_min, dim3(kAbsentBlocks, (unsigned)C), dim3(256), 0, st, keys_b, pos_max, all_min,
                        (int)pl.P);
 
@@ -1065,22 +1081,20 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
                        pl.tiles);
     if (pl.regions > 0) {
-        uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);
-        const int n_cur = C * pl.regions;
-        hipLaunchKernelGGL(lov_zero_u32, dim3((unsigned)ceil_div(n_cur, 256)), dim3(256), 0, st, cursors, n_cur);
+        uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);      // zeroed by lov_class_max
         // vals_b is free by now: it receives the pixel offsets that go with the staged values
         hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
                            pl.regions);
         hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(kUnbinThreads), 0, st, jacc, vals_b,
-                           cursors, pl.regions, (int)pl.P);
+                           cursors, pl.regions, (int)pl.P, tile_loss, losses, pl.tiles);
     } else {
         // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
         // (jacc stopped being a key buffer when the third pass read it)
         hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, jacc, pl.E);
         hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, nullptr,
                            0);
+        hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     }
-    hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     return check_launch();
 }
 
