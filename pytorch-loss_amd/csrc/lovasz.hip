@@ -26,8 +26,11 @@
 //                     so J, dJ and the tile's share of the loss follow at once; dJ goes to
 //                     pixel order through region-binned staging (final) and an in-LDS permute
 //                     per region (unbin), which also writes the zeros of the keys left out.
-//   4. reduce_loss    fixed-order sum of the per-tile partials (no floating-point atomics, so
-//                     results are deterministic).
+//   4. loss per class fixed-order sum of the per-tile partials (no floating-point atomics, so
+//                     results are deterministic): by the first unbin block of the class, or by
+//                     reduce_loss when the rows are too long for the staging regions.
+// A 4096-key tile is handled by 512 threads with 8 keys each; neighbouring tiles of a class row run
+// on the same XCD (sort_tile) so that the sectors they share merge in one L2.
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
 #include "plh_common.hpp"
 
