@@ -22,6 +22,7 @@ namespace plh {
 
 constexpr int kOhemBins = 1024;                 // 10 bits per digit, 3 digits cover [0, 0x3F800000]
 constexpr int kOhemTile = 1024;                 // pixels per block in the tie-ranking passes (256 threads x 4)
+constexpr int kOhemZeroWords = 3 * kOhemBins + 16;   // histograms and state of the selection: zero before use
 constexpr uint32_t kOneBits = 0x3F800000u;
 
 
@@ -37,7 +38,10 @@ template <class T, int CP, int V, bool Uniform>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                               float *__restrict__ scores, float *__restrict__ ce,
                                                               int64_t P, int64_t m_size, int C, int64_t ignore,
-                                                              unsigned xcd_run) {
+                                                              unsigned xcd_run, uint32_t *__restrict__ tables) {
+    // the selection's tables start at zero; the kernels that fill them are launched after this one
+    if (tables && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kOhemZeroWords; i += kRegsBlock) tables[i] = 0;
     const PixelRef<V, Uniform> at(P, m_size, C, xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
@@ -76,7 +80,10 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
 template <class T>
 __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         float *__restrict__ scores, float *__restrict__ ce, int64_t P,
-                                                        int64_t m_size, int C, int64_t ignore) {
+                                                        int64_t m_size, int C, int64_t ignore,
+                                                        uint32_t *__restrict__ tables) {
+    if (tables && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kOhemZeroWords; i += 256) tables[i] = 0;
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t lb = lab[pix];
         if (lb == ignore || lb < 0 || lb >= C) {
@@ -106,7 +113,6 @@ struct OhemTables {
     uint32_t *state;       // [16]
     uint32_t *tile_ties;   // [tiles], exclusive-scanned in place
 };
-constexpr int kOhemZeroWords = 3 * kOhemBins + 16;
 
 __global__ void ohem_zero(uint32_t *p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -363,7 +369,8 @@ static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 static int64_t ohem_tiles(int64_t P) { return ceil_div(P > 0 ? P : 1, kOhemTile); }
 
 static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, float *ce,
-                         int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st) {
+                         int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st,
+                         uint32_t *tables = nullptr) {
     const int64_t P = n_size * m_size;
     const int C = (int)dimsize;
     dispatch_dtype(dtype, [&](auto tag) {
@@ -380,18 +387,18 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
         if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                                    labels, scores, ce, P, m_size, C, ignore_index, run);                             \
+                                    labels, scores, ce, P, m_size, C, ignore_index, run, tables);                     \
         else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, false>), dim3(grid), dim3(kRegsBlock), 0,    \
-                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run);                 \
+                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);         \
         else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, false>), dim3(grid), dim3(kRegsBlock), 0, st, x,       \
-                                labels, scores, ce, P, m_size, C, ignore_index, run);                                 \
+                                labels, scores, ce, P, m_size, C, ignore_index, run, tables);                         \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
         } else {
             hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,
-                               m_size, C, ignore_index);
+                               m_size, C, ignore_index, tables);
         }
     });
     return check_launch();
@@ -408,7 +415,8 @@ static int check_workspace(const void *workspace, int64_t workspace_bytes, int64
 
 static int launch_select(const float *scores, const int64_t *labels, int64_t *out_labels, void *workspace,
                          int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st,
-                         const float *ce = nullptr, Partials part = Partials{nullptr, nullptr}) {
+                         const float *ce = nullptr, Partials part = Partials{nullptr, nullptr},
+                         bool tables_zeroed = false) {
     if (n_min >= P && part.sum) {                // nothing is relabelled, the loss is still wanted
         n_min = 0;
         score_thresh = INFINITY;
@@ -429,7 +437,8 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
     // 16-byte accesses when every tensor allows them (tile bases are multiples of 4 pixels)
     const int vec = !misaligned(scores, 16) && !misaligned(labels, 16) && !misaligned(out_labels, 16);
     if (k > 0) {
-        hipLaunchKernelGGL(ohem_zero, dim3((kOhemZeroWords + 255) / 256), dim3(256), 0, st, tb.hist, kOhemZeroWords);
+        if (!tables_zeroed)     // the score kernel of the one-call entry points has done it
+            hipLaunchKernelGGL(ohem_zero, dim3((kOhemZeroWords + 255) / 256), dim3(256), 0, st, tb.hist, kOhemZeroWords);
         // every block ends with one global atomic per non-empty bin, all blocks on the same few hundred
         // addresses: 512 blocks (two per compute unit) measured 30 us faster than 2048 on 8 M scores
         const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
@@ -493,11 +502,11 @@ extern "C" int plh_ohem_score_label(const void *logits, int32_t dtype, const int
         if (!scores) return PLH_ERR_NULL_POINTER;
         if (misaligned(scores, 4)) return PLH_ERR_MISALIGNED;
         rc = launch_scores(logits, dtype, labels, scores, nullptr, n_size, dimsize, m_size, ignore_index,
-                           (hipStream_t)stream);
+                           (hipStream_t)stream, static_cast<uint32_t *>(workspace));
         if (rc != PLH_OK) return rc;
     }
     return launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min,
-                         (hipStream_t)stream);
+                         (hipStream_t)stream, nullptr, Partials{nullptr, nullptr}, n_min < P);
 }
 
 extern "C" int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels) {
@@ -530,9 +539,11 @@ extern "C" int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int6
     Partials part;
     part.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P));
     part.cnt = reinterpret_cast<int *>(part.sum + tiles);
-    rc = launch_scores(logits, dtype, labels, scores, pixel_ce, n_size, dimsize, m_size, ignore_index, st);
+    rc = launch_scores(logits, dtype, labels, scores, pixel_ce, n_size, dimsize, m_size, ignore_index, st,
+                       static_cast<uint32_t *>(workspace));
     if (rc != PLH_OK) return rc;
-    rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_ce, part);
+    rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_ce, part,
+                       true);
     if (rc != PLH_OK) return rc;
     finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
     return check_launch();
