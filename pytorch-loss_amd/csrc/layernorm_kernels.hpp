@@ -8,7 +8,7 @@
 // REGISTERS between the two uses: lanes run along pixels (8 bytes per lane and channel), and for
 // C > 32 the four (C > 64: eight) waves of a block split the channels of one pixel group between
 // them and exchange per-wave (mean, centred square sum) pairs through LDS, merged by the
-// pairwise-variance rule. A wave holds at most 64 packed channels, which covers C <= 512; C <= 1024
+// pairwise-variance rule. A wave holds at most 96 packed channels, which covers C <= 768; C <= 1024
 // runs one pixel per lane; anything larger, and m_size == 1 (rows contiguous), takes a two-sweep
 // kernel whose second sweep is served by cache.
 #pragma once
@@ -160,7 +160,8 @@ __global__ __launch_bounds__(256) void ln_group(const T *__restrict__ x, const T
         const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
         const float shift = load_one(x + base);
         float s1 = 0.f, s2 = 0.f;
-        for (int j = sub; j < p.C; j += G) {
+#pragma unroll 8
+        for (int j = sub; j < p.C; j += G) {          // unrolled: eight loads in flight per lane
             const float d = load_one(x + base + (int64_t)j * p.m_size) - shift;
             s1 += d;
             s2 = __builtin_fmaf(d, d, s2);
@@ -173,6 +174,7 @@ __global__ __launch_bounds__(256) void ln_group(const T *__restrict__ x, const T
         const float v = var + p.eps;
         const float rstd = 1.f / sqrtf(v), mv = mean * v;
         if (!live) continue;
+#pragma unroll 8
         for (int j = sub; j < p.C; j += G) {
             const int64_t at = base + (int64_t)j * p.m_size;
             const float val = load_one(x + at);
@@ -208,7 +210,7 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
         }
         return;
     }
-    const bool vec = dimsize <= 512 && m_size % VT == 0 && !misaligned(x, VT * sizeof(T)) &&
+    const bool vec = dimsize <= 768 && m_size % VT == 0 && !misaligned(x, VT * sizeof(T)) &&
                      !misaligned(out, VT * sizeof(T)) && !(Bwd && misaligned(g, VT * sizeof(T)));
     const int64_t groups = ceil_div(p.P, 64 * (vec ? VT : 1));
     const unsigned grid = (unsigned)(ws > 1 ? groups : ceil_div(groups, 4));
@@ -216,16 +218,25 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
 #define PLH_LN(KW, VV, WS) \
     hipLaunchKernelGGL((ln_regs<T, KW, VV, WS, Bwd>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
 #define PLH_LN_V(KW, WS) do { if (vec) PLH_LN(KW, VT, WS); else PLH_LN(KW, 1, WS); } while (0)
+    // Slot counts in steps of about 1.5x: a wave whose channels fall short of its slots re-reads its last
+    // channel for the rest, and at 12 channels in 16 slots that cost a third of the bandwidth.
     if (ws == 1) {
         if (slots <= 8) PLH_LN_V(8, 1);
+        else if (slots <= 12) PLH_LN_V(12, 1);
         else if (slots <= 16) PLH_LN_V(16, 1);
+        else if (slots <= 24) PLH_LN_V(24, 1);
         else PLH_LN_V(32, 1);
     } else if (ws == 4) {
-        PLH_LN_V(16, 4);
-    } else if (slots <= 16) PLH_LN_V(16, 8);
+        if (slots <= 12) PLH_LN_V(12, 4);
+        else PLH_LN_V(16, 4);
+    } else if (slots <= 12) PLH_LN_V(12, 8);
+    else if (slots <= 16) PLH_LN_V(16, 8);
+    else if (slots <= 24) PLH_LN_V(24, 8);
     else if (slots <= 32) PLH_LN_V(32, 8);
+    else if (slots <= 48) PLH_LN_V(48, 8);
     else if (slots <= 64) PLH_LN_V(64, 8);
-    else PLH_LN(128, 1, 8);                            // 512 < C <= 1024: one pixel per lane
+    else if (slots <= 96) PLH_LN_V(96, 8);             // C <= 768
+    else PLH_LN(128, 1, 8);                            // 768 < C <= 1024: one pixel per lane
 #undef PLH_LN_V
 #undef PLH_LN
 }
