@@ -447,7 +447,7 @@ inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(p
 //   Uniform  - m_size is a multiple of the tile (kRegsBlock*V pixels), so a tile never straddles two
 //              images and the grid has no ragged end: the image index and the channel base are
 //              block-uniform (one scalar division per block, scalar base + 32-bit lane offset
-//              addressing) and no bounds check is needed. Every BASELINE shape takes this form.
+//              addressing) and no bounds check is needed. Power-of-two image sizes take this form.
 //   general  - any m_size: per-thread 64-bit index arithmetic and a bounds check.
 template <int V, bool Uniform>
 struct PixelRef {
