@@ -8,7 +8,8 @@
 //   1. scores      one pass over the logits (channel slice in registers), P fp32 scores out;
 //   2. select      a 3-digit (10 bits each) radix select over the score bit patterns finds v, the
 //                  n_min-th smallest score, and how many pixels with exactly that score still
-//                  fall below position n_min (`keep_ties`);
+//                  fall below position n_min (`keep_ties`); the histogram kernel of a digit first
+//                  resolves the digit before it (every block for itself, from the finished table);
 //   3. ties        pixels equal to v are ranked in pixel order (what a stable key sort gives):
 //                  per-tile counts, one scan over the tiles, in-tile ranks from ballots;
 //   4. relabel     drop = score > thresh && (score > v || (score == v && tie_rank >= keep_ties)).
@@ -155,17 +156,37 @@ __device__ void ohem_pick_digit(const uint32_t *h, uint32_t rank, uint32_t *lds,
     __syncthreads();
 }
 
+// Digit `pass` of the selection from its finished histogram: returns the key prefix including that
+// digit. Every block of a kernel may call it (same inputs, same answer); the one with `publish`
+// stores prefix and remaining rank for the kernels launched later.
+__device__ uint32_t ohem_resolve_digit(const OhemTables &tb, int pass, uint32_t n_min, uint32_t *lds, bool publish) {
+    const uint32_t before = pass == 0 ? 0u : tb.state[2 * (pass - 1)];
+    const uint32_t rank = pass == 0 ? n_min : tb.state[2 * (pass - 1) + 1];
+    uint32_t digit, rank_in_bin;
+    ohem_pick_digit(tb.hist + pass * kOhemBins, rank, lds, digit, rank_in_bin);
+    const uint32_t prefix = before | (digit << (20 - 10 * pass));
+    if (publish && threadIdx.x == 0) {
+        tb.state[2 * pass] = prefix;
+        tb.state[2 * pass + 1] = rank_in_bin;
+    }
+    return prefix;
+}
+
 __device__ __forceinline__ void hist_add(uint32_t *bins, float s, uint32_t high_mask, uint32_t prefix, int pass) {
     const uint32_t key = score_key(s);
     if ((key & high_mask) == prefix) atomicAdd(&bins[key_digit(key, pass)], 1u);
 }
 
-// Histogram of digit `pass` over the keys that share the already resolved leading digits.
+// Histogram of digit `pass` over the keys that share the leading digits, the last of which the
+// block resolves first. (A device-wide "last block resolves it" would need a release fence in every
+// block, which costs more than this redundant scan of 1024 counts on a GPU whose XCDs have separate
+// L2s; so does a launch of its own.)
 __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ scores, OhemTables tb, int P, int pass,
                                                  uint32_t n_min, int vec) {
     __shared__ uint32_t bins[kOhemBins];
-    const uint32_t prefix = pass == 0 ? 0u : tb.state[2 * (pass - 1)];
+    __shared__ uint32_t scan[260];
     for (int i = threadIdx.x; i < kOhemBins; i += 256) bins[i] = 0;
+    const uint32_t prefix = pass == 0 ? 0u : ohem_resolve_digit(tb, pass - 1, n_min, scan, blockIdx.x == 0);
     __syncthreads();
     const uint32_t high_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (30 - 10 * pass));
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
@@ -202,20 +223,10 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
         if (bins[i]) atomicAdd(out + i, bins[i]);
 }
 
-// One block: resolves digit `pass` from its finished histogram and publishes prefix and rank for
-// the kernels that follow. (A kernel of its own rather than the last block of ohem_hist: that would
-// need a device-wide release fence in every block, which costs far more than a launch on a GPU
-// whose XCDs have separate L2s.)
+// One block: the last digit, for the kernels that follow.
 __global__ __launch_bounds__(256) void ohem_pick(OhemTables tb, int pass, uint32_t n_min) {
     __shared__ uint32_t scan[260];
-    const uint32_t prefix = pass == 0 ? 0u : tb.state[2 * (pass - 1)];
-    const uint32_t rank = pass == 0 ? n_min : tb.state[2 * (pass - 1) + 1];
-    uint32_t digit, rank_in_bin;
-    ohem_pick_digit(tb.hist + pass * kOhemBins, rank, scan, digit, rank_in_bin);
-    if (threadIdx.x == 0) {
-        tb.state[2 * pass] = prefix | (digit << (20 - 10 * pass));
-        tb.state[2 * pass + 1] = rank_in_bin;
-    }
+    ohem_resolve_digit(tb, pass, n_min, scan, true);
 }
 
 // This thread's 4 consecutive scores and their keys; pixels beyond the end match no key.
@@ -442,10 +453,9 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         // every block ends with one global atomic per non-empty bin, all blocks on the same few hundred
         // addresses: 512 blocks (two per compute unit) measured 30 us faster than 2048 on 8 M scores
         const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
-        for (int pass = 0; pass < 3; ++pass) {
+        for (int pass = 0; pass < 3; ++pass)
             hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, vec);
-            hipLaunchKernelGGL(ohem_pick, dim3(1), dim3(256), 0, st, tb, pass, k);
-        }
+        hipLaunchKernelGGL(ohem_pick, dim3(1), dim3(256), 0, st, tb, 2, k);
         hipLaunchKernelGGL(ohem_count_ties, dim3((unsigned)tiles), dim3(256), 0, st, scores, tb, Pi, score_thresh, vec);
         hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, score_thresh);
     }
