@@ -246,8 +246,15 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
                                             P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.7, labels.numel() // 16, st())
         b = lambda: lib.plh_lsr_backward_scaled(P(x), tag, P(new_labels), P(loss), 1.0, P(n_valid), P(grad), n, c, m, 255,
                                                 0.0, st())
-        assert f() == 0 and b() == 0
-        for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes)):
+        # OhemLargeMarginLoss: the same pipeline behind the large-margin forward kernel, and that loss's gradient
+        fl = lambda: lib.plh_ohem_lmargin_forward(P(x), tag, P(labels), P(new_labels), P(scratch[0]), P(scratch[1]),
+                                                  P(loss), P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.3, 0.7,
+                                                  labels.numel() // 16, st())
+        bl = lambda: lib.plh_lmargin_backward_scaled(P(x), tag, P(new_labels), P(loss), 1.0, P(n_valid), P(grad), n, c, m,
+                                                     255, 0.3, st())
+        assert f() == 0 and b() == 0 and fl() == 0 and bl() == 0
+        for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes),
+                                ("large_margin_forward", fl, fwd_bytes), ("large_margin_backward", bl, bwd_bytes)):
             ms = time_kernel(fn)
             gbps = nbytes / (ms * 1e-3) / 1e9
             out[key] = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

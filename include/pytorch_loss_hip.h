@@ -240,6 +240,21 @@ int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int64_t *labels
                         int64_t n_size, int64_t dimsize, int64_t m_size,
                         int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
 
+/* OhemLargeMarginLoss.forward in one call (pytorch_loss/ohem_loss.py:33-45: score_ohem_label, then
+ * LargeMarginSoftmaxV3(ignore_index, reduction='mean') on the new labels). The large-margin forward
+ * kernel holds the full softmax of every pixel, so it also writes the pixel's score; the relabelling
+ * pass then adds up the kept pixels' losses (pixel_loss, scratch of n_size*m_size floats like
+ * `scores`): one pass over the logits instead of two. plh_lmargin_backward_scaled on out_labels with
+ * divide_by = n_valid_out is the matching gradient. Sizes, outputs and workspace as for
+ * plh_ohem_ce_forward (plh_ohem_ce_workspace_bytes).
+ */
+int plh_ohem_lmargin_forward(const void *logits, int32_t dtype, const int64_t *labels,
+                             int64_t *out_labels, float *scores, float *pixel_loss,
+                             float *loss_out, int64_t *n_valid_out,
+                             void *workspace, int64_t workspace_bytes,
+                             int64_t n_size, int64_t dimsize, int64_t m_size,
+                             int64_t ignore_index, float lam, float score_thresh, int64_t n_min, void *stream);
+
 /* ---- one-hot / label-smoothed targets -------------------------------------------------
  * Replaces one_hot_cpp.label_one_hot (csrc/one_hot_kernel.cu:265-350).
  * labels (n_size, m_size) int64 -> one_hot (n_size, dimsize, m_size) fp32: 0 in every channel of an

@@ -12,7 +12,7 @@ PLH_LM_EXTERN(bf16)
 // Launches one direction (or the fused pair). blocks_out: blocks that wrote partials (Reduce only).
 static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,
                   int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
-                  int64_t m_size, int64_t ignore, float lam, void *stream) {
+                  int64_t m_size, int64_t ignore, float lam, void *stream, float *scores = nullptr) {
     const bool WantLoss = variant != kLmBackward, WantGrad = variant == kLmBackward || variant == kLmForwardBackwardCount;
     const bool WantCount = variant == kLmForwardBackwardCount, Reduce = variant == kLmForwardReduced;
     if (blocks_out) *blocks_out = 0;
@@ -39,6 +39,7 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     p.half_lam = lam / 2.f;                          // csrc/large_margin_kernel.cu:188
     p.coeff = 1.f / (float)(dimsize - 1);            // csrc/large_margin_kernel.cu:404
     p.xcd_run = xcd_run_for(es, m_size);
+    p.scores = scores;
     unsigned blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
@@ -49,11 +50,21 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     return check_launch();
 }
 
+static const Partials kNoPartials{nullptr, nullptr};
+
+// Declared in plh_common.hpp for the OHEM entry point: the per-pixel forward that also leaves each
+// pixel's score.
+int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
+                                int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
+                                hipStream_t stream) {
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    return launch(kLmForward, logits, dtype, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr, n_size, dimsize,
+                  m_size, ignore_index, lam, stream, scores);
+}
+
 }  // namespace plh
 
 using namespace plh;
-
-static const Partials kNoPartials{nullptr, nullptr};
 
 extern "C" int plh_lmargin_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
                                    int64_t n_size, int64_t dimsize, int64_t m_size,

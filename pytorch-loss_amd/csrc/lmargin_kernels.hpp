@@ -24,6 +24,8 @@ struct LmParams {
     int64_t ignore;
     float half_lam, coeff;
     unsigned xcd_run;   // tile permutation run length (xcd_run_for)
+    float *scores;      // forward kernels: if set, also the softmax probability at the label per pixel
+                        // (1 for a pixel without a target), what the OHEM relabelling ranks
 };
 
 // ---------------------------------------------------------------- regs ----
@@ -55,7 +57,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     float go[V];
     if constexpr (WantGrad) load_upstream<V>(up, pix, go);
 
-    float out[V];
+    float out[V], score[V];
     float g[WantGrad ? CP : 1][V];
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
     unsigned n_valid = 0;
@@ -112,6 +114,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             const float margin = sum_qt - lse_no - p.coeff * (sum_t - others * lse_no);
             const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
+            score[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
             mine += out[k];
             cnt += (ign || !live) ? 0 : 1;
         }
@@ -139,6 +142,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     }
     if (live) {
         if (WantLoss && loss) store_vec<V>(loss + pix, out);
+        if (WantLoss && p.scores) store_vec_cached<V>(p.scores + pix, score);
         if constexpr (WantGrad) {
             // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
             const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
@@ -237,6 +241,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
             acc += -(x_y - m_all) + logf(s_all);
             if (live && sub == 0) {
                 if (loss) loss[pix] = ign ? 0.f : acc;
+                if (p.scores) p.scores[pix] = (ign || lb < 0 || lb >= p.C) ? 1.f : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0.f : 1.f;
             }
@@ -291,8 +296,10 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
                              unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    const float *second_f32 = go_vec ? go_vec : p.scores;      // the score output belongs to forwards without upstream
     unsigned blocks = 0;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr, go_vec)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
+                       second_f32)) {
         case Shape::RegsVec:
             blocks = launch_regs<T, V, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;

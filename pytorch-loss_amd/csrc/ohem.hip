@@ -524,11 +524,14 @@ extern "C" int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels) {
     return select_workspace(n_pixels) + align256(8 * ohem_tiles(n_pixels));
 }
 
-extern "C" int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int64_t *labels, int64_t *out_labels,
-                                   float *scores, float *pixel_ce, float *loss_out, int64_t *n_valid_out,
-                                   void *workspace, int64_t workspace_bytes,
-                                   int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
-                                   float score_thresh, int64_t n_min, void *stream) {
+// The one-call forwards: scores and per-pixel loss in one pass over the logits (cross entropy: the
+// score kernel itself; large margin: that loss's forward kernel, which then also leaves the scores),
+// relabelling that adds up the kept pixels' losses, fixed-order finish.
+static int ohem_loss_forward(bool large_margin, float lam, const void *logits, int32_t dtype, const int64_t *labels,
+                             int64_t *out_labels, float *scores, float *pixel_loss, float *loss_out,
+                             int64_t *n_valid_out, void *workspace, int64_t workspace_bytes, int64_t n_size,
+                             int64_t dimsize, int64_t m_size, int64_t ignore_index, float score_thresh, int64_t n_min,
+                             void *stream) {
     if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     int rc = check_slice_args(logits, labels, out_labels, n_size, dimsize, m_size, dtype_size(dtype), 8);
     if (rc != PLH_OK) return rc;
@@ -541,20 +544,42 @@ extern "C" int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int6
         finish_partials(Partials{nullptr, nullptr}, 0, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
         return check_launch();
     }
-    if (!scores || !pixel_ce) return PLH_ERR_NULL_POINTER;
-    if (misaligned(scores, 4) || misaligned(pixel_ce, 4)) return PLH_ERR_MISALIGNED;
+    if (!scores || !pixel_loss) return PLH_ERR_NULL_POINTER;
+    if (misaligned(scores, 4) || misaligned(pixel_loss, 4)) return PLH_ERR_MISALIGNED;
     if (!workspace || misaligned(workspace, 256) || workspace_bytes < plh_ohem_ce_workspace_bytes(P))
         return PLH_ERR_WORKSPACE;
     const int64_t tiles = ohem_tiles(P);
     Partials part;
     part.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P));
     part.cnt = reinterpret_cast<int *>(part.sum + tiles);
-    rc = launch_scores(logits, dtype, labels, scores, pixel_ce, n_size, dimsize, m_size, ignore_index, st,
-                       static_cast<uint32_t *>(workspace));
+    if (large_margin)
+        rc = lmargin_forward_with_scores(logits, dtype, labels, pixel_loss, scores, n_size, dimsize, m_size, ignore_index,
+                                         lam, st);
+    else
+        rc = launch_scores(logits, dtype, labels, scores, pixel_loss, n_size, dimsize, m_size, ignore_index, st,
+                           static_cast<uint32_t *>(workspace));
     if (rc != PLH_OK) return rc;
-    rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_ce, part,
-                       true);
+    rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_loss, part,
+                       /*tables_zeroed=*/!large_margin);
     if (rc != PLH_OK) return rc;
     finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
     return check_launch();
+}
+
+extern "C" int plh_ohem_ce_forward(const void *logits, int32_t dtype, const int64_t *labels, int64_t *out_labels,
+                                   float *scores, float *pixel_ce, float *loss_out, int64_t *n_valid_out,
+                                   void *workspace, int64_t workspace_bytes,
+                                   int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                   float score_thresh, int64_t n_min, void *stream) {
+    return ohem_loss_forward(false, 0.f, logits, dtype, labels, out_labels, scores, pixel_ce, loss_out, n_valid_out,
+                             workspace, workspace_bytes, n_size, dimsize, m_size, ignore_index, score_thresh, n_min, stream);
+}
+
+extern "C" int plh_ohem_lmargin_forward(const void *logits, int32_t dtype, const int64_t *labels, int64_t *out_labels,
+                                        float *scores, float *pixel_loss, float *loss_out, int64_t *n_valid_out,
+                                        void *workspace, int64_t workspace_bytes,
+                                        int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                        float lam, float score_thresh, int64_t n_min, void *stream) {
+    return ohem_loss_forward(true, lam, logits, dtype, labels, out_labels, scores, pixel_loss, loss_out, n_valid_out,
+                             workspace, workspace_bytes, n_size, dimsize, m_size, ignore_index, score_thresh, n_min, stream);
 }

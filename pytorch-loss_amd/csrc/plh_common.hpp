@@ -412,6 +412,12 @@ inline int carve_partials(void *workspace, int64_t workspace_bytes, int64_t unit
 void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int64_t *count_out, FinishMode mode,
                      int64_t fixed_count, hipStream_t stream);
 
+// Defined in lmargin.hip: plh_lmargin_forward that also writes each pixel's softmax probability at
+// its label (1 where there is no target) into `scores`.
+int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
+                                int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
+                                hipStream_t stream);
+
 // ---- the "regs" launch shape ---------------------------------------------------
 // 256 threads per block, V pixels per thread; block b of the grid owns the pixel tile
 // tile_of_block(run). Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; the

@@ -54,6 +54,8 @@ _SIGNATURES = {
     "plh_ohem_ce_workspace_bytes": (_i64, [_i64]),
     "plh_ohem_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32, _i64,
                                            _p]),
+    "plh_ohem_lmargin_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32,
+                                                _f32, _i64, _p]),
     "plh_taylor_softmax_forward": (ctypes.c_int, [_p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
@@ -497,8 +499,9 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
     return out
 
 
-def ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min):
-    """Relabelling and mean cross entropy of what is left, with one pass over the logits.
+def ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min, lam=None):
+    """Relabelling and mean loss of what is left, with one pass over the logits: cross entropy, or
+    the large-margin loss when `lam` is given.
     -> (loss 0-dim, n_valid 0-dim int64, args whose labels are the NEW labels, for the backward)."""
     a = ohem_args(logits, labels)
     dev = a.x.device
@@ -511,8 +514,12 @@ def ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min):
     if nbytes < 0:
         _check(nbytes)
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
-    _call(a.x, "plh_ohem_ce_forward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(new_labels), _ptr(scratch[0]), _ptr(scratch[1]),
-          _ptr(loss), _ptr(n_valid), _ptr(ws), nbytes, a.n, a.c, a.m, int(ignore_index), float(score_thresh), int(n_min))
+    head = (_ptr(a.x), a.tag, _ptr(a.lb), _ptr(new_labels), _ptr(scratch[0]), _ptr(scratch[1]), _ptr(loss), _ptr(n_valid),
+            _ptr(ws), nbytes, a.n, a.c, a.m, int(ignore_index))
+    if lam is None:
+        _call(a.x, "plh_ohem_ce_forward", *head, float(score_thresh), int(n_min))
+    else:
+        _call(a.x, "plh_ohem_lmargin_forward", *head, float(lam), float(score_thresh), int(n_min))
     a.lb = new_labels
     return _back_to(loss, _loss_dtype(a.dtype)), n_valid, a
 

@@ -7,7 +7,8 @@ then take the mean loss over what is left.  ``OhemCELoss`` uses plain cross entr
 ``nn.CrossEntropyLoss(ignore_index, reduction='mean')``, ohem_loss.py:20): the relabelling pass over
 the logits already has every pixel's cross entropy at hand, so the forward is that one pass, and
 the backward is the label-smoothed kernel with a smoothing factor of 0 on the new labels;
-``OhemLargeMarginLoss`` uses ``LargeMarginSoftmaxV3``.
+``OhemLargeMarginLoss`` uses ``LargeMarginSoftmaxV3`` (ohem_loss.py:33-45), whose forward kernel
+holds every pixel's softmax and so leaves the scores as well: again one pass over the logits.
 """
 import torch
 import torch.nn as nn
@@ -22,7 +23,29 @@ def score_ohem_label(logits, labels, ignore_index, score_thresh, n_min):
     return _native.ohem_score_label(logits.detach(), labels, ignore_index, score_thresh, n_min)
 
 
+class _OhemLossFunction(torch.autograd.Function):
+    """Mean loss over the pixels that keep their label: cross entropy, or the large-margin loss when
+    `lam` is not None. No gradient flows through the relabelling (the reference runs it under
+    no_grad, ohem_loss.py:25)."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, ignore_index, score_thresh, n_min, lam):
+        loss, n_valid, args = _native.ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min, lam)
+        ctx.vars = args, n_valid, ignore_index, lam
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        args, n_valid, ignore_index, lam = ctx.vars
+        if lam is None:
+            grad = _native.lsr_backward_scaled(None, None, ignore_index, 0.0, grad_output, n_valid, args=args)
+        else:
+            grad = _native.lmargin_backward_scaled(None, None, lam, ignore_index, grad_output, n_valid, args=args)
+        return grad, None, None, None, None, None
+
+
 class _OhemLoss(nn.Module):
+    lam = None       # None: cross entropy
 
     def __init__(self, score_thresh, n_min=None, ignore_index=255):
         super().__init__()
@@ -32,36 +55,23 @@ class _OhemLoss(nn.Module):
 
     def forward(self, logits, labels):
         n_min = labels.numel() // 16 if self.n_min is None else self.n_min
-        labels = score_ohem_label(logits, labels, self.ignore_lb, self.score_thresh, n_min)
-        return self.criteria(logits, labels)
-
-
-class _OhemCEFunction(torch.autograd.Function):
-    """Mean cross entropy over the pixels that keep their label; no gradient flows through the
-    relabelling (the reference runs it under no_grad, ohem_loss.py:25)."""
-
-    @staticmethod
-    def forward(ctx, logits, labels, ignore_index, score_thresh, n_min):
-        loss, n_valid, args = _native.ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min)
-        ctx.vars = args, n_valid, ignore_index
-        return loss
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        args, n_valid, ignore_index = ctx.vars
-        grad = _native.lsr_backward_scaled(None, None, ignore_index, 0.0, grad_output, n_valid, args=args)
-        return grad, None, None, None, None
+        return _OhemLossFunction.apply(logits, labels, self.ignore_lb, self.score_thresh, n_min, self.lam)
 
 
 class OhemCELoss(_OhemLoss):
 
-    def forward(self, logits, labels):
-        n_min = labels.numel() // 16 if self.n_min is None else self.n_min
-        return _OhemCEFunction.apply(logits, labels, self.ignore_lb, self.score_thresh, n_min)
+    def __init__(self, score_thresh, n_min=None, ignore_index=255):
+        super().__init__(score_thresh, n_min, ignore_index)
+        self.criteria = nn.CrossEntropyLoss(ignore_index=ignore_index, reduction="mean")    # ohem_loss.py:20; not called
 
 
 class OhemLargeMarginLoss(_OhemLoss):
 
     def __init__(self, score_thresh, n_min=None, ignore_index=255):
         super().__init__(score_thresh, n_min, ignore_index)
+        # kept for its parameters, as the reference keeps it (ohem_loss.py:40); `lam` is read per call
         self.criteria = LargeMarginSoftmaxV3(ignore_index=ignore_index, reduction="mean")
+
+    @property
+    def lam(self):
+        return self.criteria.lam

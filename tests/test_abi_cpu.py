@@ -147,6 +147,11 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_ohem_ce_forward(p, 0, p, p, p, None, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -1
     assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, None, 0, 1, 4, 16, 255, 0.7, 1, None) == -5
     assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, wsp, 16, 1, 4, 16, 255, 0.7, 1, None) == -5
+    # fused OHEM large margin: the same checks behind one more scalar
+    assert lib.plh_ohem_lmargin_forward(p, 4, p, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -7
+    assert lib.plh_ohem_lmargin_forward(p, 0, None, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
+    assert lib.plh_ohem_lmargin_forward(p, 0, p, p, None, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
+    assert lib.plh_ohem_lmargin_forward(p, 0, p, p, p, p, p, p, wsp, 16, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -5
     # layer norm
     assert lib.plh_layer_norm_forward(None, 0, None, 0, 4, 4, 1e-6, None) == 0
     assert lib.plh_layer_norm_forward(p, 5, p, 1, 4, 4, 1e-6, None) == -7

@@ -165,12 +165,15 @@ def test_ohem_refuses_cpu_tensors():
         pl.OhemCELoss(0.7)(x, y)
 
 
-@pytest.mark.parametrize("case", ["n_min_covers_everything", "all_ignored", "huge_logit_gaps", "ragged"])
-def test_ohem_ce_fused_forward_edge_cases(native, case):
+@pytest.mark.parametrize("which", ["ce", "lm"])
+@pytest.mark.parametrize("case", ["n_min_covers_everything", "all_ignored", "huge_logit_gaps", "ragged", "deep",
+                                  "rows"])
+def test_ohem_ce_fused_forward_edge_cases(native, case, which):
+    """The one-pass forwards (scores and per-pixel loss from the same sums) against the oracle's
+    relabelling followed by torch's cross entropy or the oracle's large-margin loss."""
     import pytorch_loss as pl
-    """The one-pass forward (scores and cross entropy from the same sums) against the oracle's
-    relabelling followed by torch's cross entropy."""
-    shape = (2, 7, 9, 11) if case == "ragged" else (2, 19, 16, 24)
+    # deep: more channels than the register-resident form holds; rows: (N, C) inputs
+    shape = {"ragged": (2, 7, 9, 11), "deep": (2, 40, 6, 10), "rows": (300, 23)}.get(case, (2, 19, 16, 24))
     x, y = seg_inputs(91, shape, 255, 0.05)
     n_min, thresh = y.size // 16, 0.3
     if case == "n_min_covers_everything":
@@ -180,7 +183,8 @@ def test_ohem_ce_fused_forward_edge_cases(native, case):
     if case == "huge_logit_gaps":
         x = x * 60.0            # softmax at the label underflows to 0 for many pixels; their loss is ~1e2
     xt = dev(x).requires_grad_()
-    loss = pl.OhemCELoss(score_thresh=thresh, n_min=n_min, ignore_index=255)(xt, dev(y))
+    crit = (pl.OhemCELoss if which == "ce" else pl.OhemLargeMarginLoss)(score_thresh=thresh, n_min=n_min, ignore_index=255)
+    loss = crit(xt, dev(y))
     new_labels = oracle.ohem_score_label(x, y, 255, thresh, n_min)
     if case == "n_min_covers_everything":
         assert np.array_equal(new_labels, y)
@@ -188,9 +192,18 @@ def test_ohem_ce_fused_forward_edge_cases(native, case):
     if n_valid == 0:
         assert torch.isnan(loss).item()        # the mean over no pixels, as nn.CrossEntropyLoss gives it
         return
-    ce = torch.nn.functional.cross_entropy(torch.from_numpy(x).double(), torch.from_numpy(new_labels),
-                                           ignore_index=255, reduction="mean").item()
-    assert np.isfinite(loss.item()) and abs(loss.item() - ce) <= 1e-5 * abs(ce), (loss.item(), ce)
+    if which == "ce":
+        want = torch.nn.functional.cross_entropy(torch.from_numpy(x).double(), torch.from_numpy(new_labels),
+                                                 ignore_index=255, reduction="mean").item()
+        want_g = oracle.lsr_backward(x, new_labels, 255, 0.0, np.float32(1.0 / n_valid))
+    else:
+        want = oracle.lmargin_forward(x.astype(np.float64), new_labels, 0.3, 255).sum() / n_valid
+        want_g = oracle.lmargin_backward(x, new_labels, 0.3, 255, np.float32(1.0 / n_valid))
+    assert np.isfinite(loss.item()) and abs(loss.item() - want) <= 1e-5 * abs(want), (loss.item(), want)
     loss.backward()
-    want_g = oracle.lsr_backward(x, new_labels, 255, 0.0, np.float32(1.0 / n_valid))
     close_grad(xt.grad.cpu().numpy(), want_g, case)
+    # the same loss as the two-step composition the reference runs (ohem_loss.py:41-45)
+    if which == "lm":
+        two_step = pl.LargeMarginSoftmaxV3(ignore_index=255, reduction="mean")(
+            xt.detach(), pl.score_ohem_label(xt, dev(y), 255, thresh, n_min))
+        assert abs(two_step.item() - loss.item()) <= 1e-6 * abs(loss.item())
