@@ -32,6 +32,8 @@
 // A 4096-key tile is handled by 512 threads with 8 keys each; neighbouring tiles of a class row run
 // on the same XCD (sort_tile) so that the sectors they share merge in one L2.
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
+#include <stdlib.h>
+
 #include "plh_common.hpp"
 
 namespace plh {
@@ -358,9 +360,9 @@ __device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, 
     wave_rank_of<Hot>(wave_peers(digit, valid), digit, valid, hot, counts, counts_hot, rank, hrank);
 }
 
-// Per-tile digit counts (and, for the last pass, the same for the positives). Counting needs no
-// ranks, so it uses LDS atomics on per-wave counters instead of match masks; a round whose keys all
-// share one digit (the rule for the top digit, where errors cluster) is added by a single lane.
+// Per-tile digit counts (and, for the last pass, the same for the positives). The lower digits are
+// close to uniform: LDS atomics on per-wave counters, and a round whose keys all share one digit is
+// added by a single lane. The top digit goes through match masks (see below).
 template <bool Hot>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];
@@ -397,20 +399,15 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
         if (vmask == 0) continue;               // wave-uniform
         if constexpr (Hot) {
-            // top digit: a wave holds a handful of distinct values, so one lane adds each group's size
-            // (per-lane atomics on two or three addresses would serialise)
-            const uint64_t hmask = __builtin_amdgcn_ballot_w64(valid && (key[r] >> 31));
-            uint64_t remaining = vmask;
-            while (remaining) {                 // wave-uniform
-                const int leader = __builtin_ffsll((long long)remaining) - 1;
-                const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)digit, leader);
-                const uint64_t same = __builtin_amdgcn_ballot_w64(valid && digit == dl);
-                if (lane == 0) {
-                    atomicAdd(&counts[wave][dl], (uint32_t)__builtin_popcountll(same));
-                    const uint64_t hs = same & hmask;
-                    if (hs) atomicAdd(&counts_hot[wave][dl], (uint32_t)__builtin_popcountll(hs));
-                }
-                remaining &= ~same;
+            // top digit: errors cluster, so per-lane atomics would serialise on two or three addresses
+            // with soft predictions, while confident ones spread over dozens of binades. The match mask
+            // costs the same either way: the lowest lane of every group of equal digits adds the group.
+            const bool hot = valid && (key[r] >> 31);
+            const uint64_t peers = wave_peers(digit, valid);
+            const uint64_t hot_peers = peers & __builtin_amdgcn_ballot_w64(hot);
+            if (valid && peers_below(peers) == 0u) {
+                atomicAdd(&counts[wave][digit], (uint32_t)__builtin_popcountll(peers));
+                if (hot_peers) atomicAdd(&counts_hot[wave][digit], (uint32_t)__builtin_popcountll(hot_peers));
             }
             continue;
         }
@@ -420,15 +417,6 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
             if (lane == 0) atomicAdd(&counts[wave][first], (uint32_t)__builtin_popcountll(vmask));
         } else if (valid) {
             atomicAdd(&counts[wave][digit], 1u);
-        }
-        if constexpr (Hot) {
-            const bool hot = valid && (key[r] >> 31);
-            if (same == vmask) {
-                const uint64_t hmask = __builtin_amdgcn_ballot_w64(hot);
-                if (lane == 0 && hmask) atomicAdd(&counts_hot[wave][first], (uint32_t)__builtin_popcountll(hmask));
-            } else if (hot) {
-                atomicAdd(&counts_hot[wave][digit], 1u);
-            }
         }
     }
     __syncthreads();
@@ -609,15 +597,16 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 // values and can be staged in place: the kernel appends (value -> jacc, pixel offset -> idx_stage)
 // at a cursor inside the region's own range [b*kRegion, ...), in runs per (tile, region); a second
 // kernel (lov_unbin) then permutes each region inside LDS and writes it back coalesced.
-constexpr int kRegionBits = 13;
-constexpr int kRegion = 1 << kRegionBits;     // 8192 pixels = 32 KiB of fp32
+// The region size grows with the row so that a 4096-key tile still sends runs of ~16 values to a
+// region: 2^13 pixels (32 KiB of fp32 in lov_unbin's LDS) up to 2^15 (128 KiB).
+constexpr int kMinRegionBits = 13, kMaxRegionBits = 15;
 constexpr int kMaxRegions = 1024;             // per class row; larger rows take the direct scatter
 
 template <bool Binned>
 __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, float *__restrict__ jacc,
                                                           float *__restrict__ tile_loss,
                                                           uint32_t *__restrict__ idx_stage,
-                                                          uint32_t *__restrict__ cursors, int regions) {
+                                                          uint32_t *__restrict__ cursors, int regions, int region_bits) {
     __shared__ uint32_t region_cnt[Binned ? kMaxRegions : 1];    // keys of this tile per region
     __shared__ uint16_t region_start[Binned ? kMaxRegions : 1];  // first position of the region in the re-ordered tile (< 4096)
     __shared__ uint32_t region_base[Binned ? kMaxRegions : 1];   // this tile's run inside the region's staging range
@@ -682,7 +671,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                                counts_hot[wave], rank[r + h], hrank[r + h]);
             if constexpr (Binned) {
                 // order inside a region's staging range is irrelevant: lov_unbin puts every value at its pixel
-                if (li < count) slot[r + h] = atomicAdd(&region_cnt[val[r + h] >> kRegionBits], 1u);
+                if (li < count) slot[r + h] = atomicAdd(&region_cnt[val[r + h] >> region_bits], 1u);
             }
         }
     }
@@ -748,7 +737,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                 part += key_error(k) * dj;
             }
             if constexpr (Binned) {
-                const uint32_t lp = region_start[val[r] >> kRegionBits] + slot[r];
+                const uint32_t lp = region_start[val[r] >> region_bits] + slot[r];
                 s_dj[lp] = dj;
                 s_val[lp] = val[r];
             } else {
@@ -768,10 +757,10 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     if constexpr (Binned) {
         for (int i = threadIdx.x; i < count; i += kSortThreads) {
             const uint32_t v = s_val[i];
-            const uint32_t region = v >> kRegionBits;
-            const int64_t at = row + ((int64_t)region << kRegionBits) + region_base[region] + ((uint32_t)i - region_start[region]);
+            const uint32_t region = v >> region_bits;
+            const int64_t at = row + ((int64_t)region << region_bits) + region_base[region] + ((uint32_t)i - region_start[region]);
             jacc[at] = s_dj[i];
-            idx_stage[at] = v & (kRegion - 1);
+            idx_stage[at] = v & ((1u << region_bits) - 1u);
         }
     }
 }
@@ -780,11 +769,13 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 // permuted to pixel order inside LDS; pixels whose keys stayed out of the sort get their exact 0.
 constexpr int kUnbinThreads = 1024;
 
+template <int kRegionBits>
 __global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
                                                            const uint32_t *__restrict__ cursors, int regions, int P,
                                                            const float *__restrict__ tile_loss, float *__restrict__ losses,
                                                            int tiles) {
     typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
+    constexpr int kRegion = 1 << kRegionBits;
     __shared__ __align__(16) float sorted[kRegion];
     const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
     const int n = min(kRegion, P - (int)(blockIdx.x << kRegionBits));
@@ -930,6 +921,7 @@ struct LovaszPlan {
     int64_t P, E;
     int tiles;
     int regions;            // pixel regions per class row (0 = direct scatter)
+    int region_bits;        // log2 of the pixels per region
     int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss,
         off_cursors, off_class, off_block_max, bytes;
 };
@@ -953,7 +945,12 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.off_digit_total = off; off += round_up(4 * dimsize * kRadix, 256);
     pl.off_hot_total = off;   off += round_up(4 * dimsize * kRadix, 256);
     pl.off_tile_loss = off;   off += round_up(4 * dimsize * pl.tiles, 256);
-    const int64_t regions = ceil_div(pl.P, kRegion);
+    // the smallest region size that keeps a row within 256 regions (runs of >= 16 values per tile and region)
+    static const int forced = getenv("PLH_LOV_REGION_BITS") ? atoi(getenv("PLH_LOV_REGION_BITS")) : 0;
+    pl.region_bits = kMinRegionBits;
+    while (pl.region_bits < kMaxRegionBits && ceil_div(pl.P, (int64_t)1 << pl.region_bits) > 256) ++pl.region_bits;
+    if (forced) pl.region_bits = forced;
+    const int64_t regions = ceil_div(pl.P, (int64_t)1 << pl.region_bits);
     pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
     pl.off_class = off;       off += round_up(4 * dimsize * 3, 256);      // pos_max[C], kept[C], all_min[C]
@@ -1087,15 +1084,23 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);      // zeroed by lov_class_max
         // vals_b is free by now: it receives the pixel offsets that go with the staged values
         hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
-                           pl.regions);
-        hipLaunchKernelGGL(lov_unbin, dim3((unsigned)pl.regions, (unsigned)C), dim3(kUnbinThreads), 0, st, jacc, vals_b,
-                           cursors, pl.regions, (int)pl.P, tile_loss, losses, pl.tiles);
+                           pl.regions, pl.region_bits);
+        const dim3 unbin_grid((unsigned)pl.regions, (unsigned)C);
+        switch (pl.region_bits) {
+#define PLH_UNBIN(B)                                                                                                  \
+    case B:                                                                                                           \
+        hipLaunchKernelGGL(lov_unbin<B>, unbin_grid, dim3(kUnbinThreads), 0, st, jacc, vals_b, cursors, pl.regions,   \
+                           (int)pl.P, tile_loss, losses, pl.tiles);                                                   \
+        break;
+            PLH_UNBIN(13) PLH_UNBIN(14) PLH_UNBIN(15)
+#undef PLH_UNBIN
+        }
     } else {
         // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
         // (jacc stopped being a key buffer when the third pass read it)
         hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, jacc, pl.E);
         hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, nullptr,
-                           0);
+                           0, 0);
         hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     }
     return check_launch();

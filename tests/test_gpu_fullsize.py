@@ -134,11 +134,11 @@ def test_lovasz_full_size(pl):
     assert (lp - losses.detach()).abs().max().item() <= 2e-6
 
 
-def test_lovasz_rows_longer_than_the_staging_regions(pl):
-    """More than 1024 regions of 8192 pixels per class row: the Jaccard differences are scattered
-    straight to pixel order, and the pixels left out of the sort are cleared beforehand."""
+@pytest.mark.parametrize("n_pix", [2 ** 21 + 4096 + 3, 8192 * 1024 + 4096 + 3], ids=["regions_of_16k", "regions_of_32k"])
+def test_lovasz_long_rows_use_larger_staging_regions(pl, n_pix):
+    """Class rows of more than 256 regions of 8192 pixels: the staging regions double in size (up to
+    32768 pixels) so that a tile still sends runs of values to each of them."""
     from pytorch_loss import _native
-    n_pix = 8192 * 1024 + 4096 + 3
     x = synth.normal(91, 1, (n_pix, 2), 0.0, 2.0)
     y = synth.randint(91, 2, (n_pix,), 0, 2).astype(np.int64)
     y[synth.bernoulli(91, 3, (n_pix,), 0.05)] = 255
@@ -153,6 +153,35 @@ def test_lovasz_rows_longer_than_the_staging_regions(pl):
     # many keys that are not left out, so the zero pattern is only comparable in fp32)
     _, j32 = oracle.lovasz_forward(x, y, 255)
     assert (jacc.view(np.uint32) == j32.view(np.uint32)).mean() > 0.99
+
+
+def test_lovasz_rows_longer_than_the_staging_regions(pl):
+    """More than 1024 regions of 32768 pixels per class row: the Jaccard differences are scattered
+    straight to pixel order, and the pixels left out of the sort are cleared beforehand. The CPU
+    oracle needs a minute at this length; the check is the torch restatement of the V1 flow
+    (stable sort, cumulative sums) in fp64 on the same device, plus the size-independent properties."""
+    from oracle import torch_ref
+    n_pix = 32768 * 1024 + 4096 + 3
+    g = torch.Generator(device="cuda").manual_seed(91)
+    x = 2 * torch.randn(n_pix, 2, device="cuda", generator=g)
+    y = torch.randint(0, 2, (n_pix,), device="cuda", generator=g)
+    y[torch.rand(n_pix, device="cuda", generator=g) < 0.05] = 255
+    xt = x.clone().requires_grad_()
+    losses = pl.LovaszSoftmaxV3(reduction="none", ignore_index=255)(xt, y)
+    losses.sum().backward()
+    xr = x.double().requires_grad_()
+    want, _ = torch_ref.lovasz_per_class(xr, y, 255)
+    want.sum().backward()
+    np.testing.assert_allclose(losses.detach().cpu().numpy(), want.detach().cpu().numpy(), rtol=1e-5)
+    # J is within one fp32 ulp of 1 over most of a row this long, and so are its differences
+    # (csrc/lovasz_softmax.cu:124-147 forms them in fp32 as well): that ulp bounds the gradient error
+    err = (xt.grad.double() - xr.grad).abs()
+    assert err.max().item() <= 2.0 ** -23 and err.median().item() <= 2.0 ** -26, (err.median().item(), err.max().item())
+    assert (xt.grad[y == 255] == 0).all()
+    from pytorch_loss import _native
+    _, jacc = _native.lovasz_forward(x, y, 255)
+    assert (jacc[:, y == 255] == 0).all()
+    np.testing.assert_allclose(jacc.double().sum(dim=1).cpu().numpy(), 1.0, rtol=1e-4)
 
 
 def test_neighbouring_ops_full_size(pl):

@@ -345,6 +345,22 @@ def test_lovasz_jacc_is_exact_for_the_computed_order(pl):
     np.testing.assert_allclose(l32, l64, rtol=1e-4)
 
 
+def test_lovasz_errors_spread_over_many_binades(pl):
+    """Logits of a saturated model: errors from 1e-30 to 1, some exactly 0 (softmax rounds to 1), so
+    nothing can be left out of the sort and the top digit takes dozens of values per wavefront."""
+    from pytorch_loss import _native
+    x, y = seg_inputs(57, (2, 19, 128, 128), 255, 0.05)
+    x = (x * 8.0).astype(np.float32)
+    losses, jacc = _native.lovasz_forward(dev(x), dev(y), 255)
+    jacc = jacc.cpu().numpy()
+    l64, _ = oracle.lovasz_forward(x.astype(np.float64), y, 255)
+    np.testing.assert_allclose(losses.cpu().numpy(), l64, rtol=1e-5)
+    _, j32 = oracle.lovasz_forward(x, y, 255)
+    assert (jacc.view(np.uint32) == j32.view(np.uint32)).mean() > 0.99
+    np.testing.assert_allclose(jacc.sum(axis=1), 1.0, rtol=1e-4)
+    assert (jacc[:, y.reshape(-1) == 255] == 0).all()
+
+
 @pytest.mark.parametrize("case", ["confident", "one_positive", "absent_and_present", "ties_at_the_limit"])
 def test_lovasz_keys_left_out_of_the_sort_get_exact_zeros(pl, case):
     """The kernels sort only the keys that can have a non-zero Jaccard difference (those not ranked
