@@ -32,8 +32,6 @@
 // A 4096-key tile is handled by 512 threads with 8 keys each; neighbouring tiles of a class row run
 // on the same XCD (sort_tile) so that the sectors they share merge in one L2.
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
-#include <stdlib.h>
-
 #include "plh_common.hpp"
 
 namespace plh {
@@ -946,10 +944,8 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.off_hot_total = off;   off += round_up(4 * dimsize * kRadix, 256);
     pl.off_tile_loss = off;   off += round_up(4 * dimsize * pl.tiles, 256);
     // the smallest region size that keeps a row within 256 regions (runs of >= 16 values per tile and region)
-    static const int forced = getenv("PLH_LOV_REGION_BITS") ? atoi(getenv("PLH_LOV_REGION_BITS")) : 0;
     pl.region_bits = kMinRegionBits;
     while (pl.region_bits < kMaxRegionBits && ceil_div(pl.P, (int64_t)1 << pl.region_bits) > 256) ++pl.region_bits;
-    if (forced) pl.region_bits = forced;
     const int64_t regions = ceil_div(pl.P, (int64_t)1 << pl.region_bits);
     pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
