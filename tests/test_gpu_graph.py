@@ -36,6 +36,7 @@ CASES = {
     "lovasz": (lambda pl: pl.LovaszSoftmaxV3(reduction="mean", ignore_index=255), _seg),
     "taylor": (lambda pl: pl.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="mean"), _seg),
     "ohem": (lambda pl: pl.OhemCELoss(score_thresh=0.7, n_min=500, ignore_index=255), _seg),
+    "ohem_lmargin": (lambda pl: pl.OhemLargeMarginLoss(score_thresh=0.7, n_min=500, ignore_index=255), _seg),
     "focal": (lambda pl: pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean"), _binary),
     "dice": (lambda pl: pl.SoftDiceLossV3(p=1, smooth=1.0), _binary),
 }
