@@ -147,6 +147,167 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
     at.store_slice(grad, p.C, p.m_size, raw);
 }
 
+// --------------------------------------------------------------- split ----
+// 33..256 channels in NCHW: the 8 wavefronts of a block hold KW channels each (SplitSlice). Every
+// wavefront reduces its part of a pixel's slice, the parts meet in LDS:
+//   forward   (m_w, s_w, d_w, y_w) = max, sum_j exp(x_j - m_w), sum_j (x_j - m_w), target logit if it is here;
+//             with M = max_w m_w:  S = sum_w s_w exp(m_w - M),  sum_j (x_j - M) = sum_w d_w + n_w (m_w - M),
+//             and wavefront 0 forms the loss as the regs kernel does;
+//   backward  (c_w, s_w) in the base-2 domain, c_w = fl(m_w log2e), s_w = sum_j 2^(x_j log2e - c_w); every
+//             wavefront then evaluates 2^(x_j log2e - max_w c_w) / sum_w s_w 2^(c_w - max c) for its channels.
+
+template <class T, int KW, int V, bool Reduce>
+__global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                            float *__restrict__ loss, Partials part,
+                                                            const LsrParams p) {
+    __shared__ float parts[4][kSplitWaves][kWave * V];
+    __shared__ float red[2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    if (at.here > 0) {                                  // wave-uniform
+        typename Pack<T, V>::Raw raw[KW];
+        at.load(x, p.C, p.m_size, raw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            float xv[KW];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                xv[i] = (i < at.here) ? Pack<T, V>::get(raw[i], k) : -INFINITY;
+                mx = fmaxf(mx, xv[i]);
+            }
+            const float c = mx * kLog2e;
+            const float r = __builtin_fmaf(mx, kLog2e, -c);
+            float s = 0.f, d = 0.f, x_y = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                s += __builtin_amdgcn_exp2f(__builtin_fmaf(xv[i], kLog2e, -c));
+                d += (i < at.here) ? xv[i] - mx : 0.f;
+                x_y = (rel == i) ? xv[i] : x_y;
+            }
+            const int q = lane * V + k;
+            parts[0][wave][q] = mx;
+            parts[1][wave][q] = s * __builtin_amdgcn_exp2f(-r);      // 2^r is what the rounding of c left in every term
+            parts[2][wave][q] = d;
+            parts[3][wave][q] = x_y;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const int used = (p.C + KW - 1) / KW;               // wavefronts that hold channels
+    float out[V];
+    float mine = 0.f;
+    int cnt = 0;
+    const float fc = (float)p.C;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        const int q = lane * V + k;
+        float M = parts[0][0][q];
+        for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
+        float S = 0.f, D = 0.f, x_y = 0.f;
+        for (int w = 0; w < used; ++w) {
+            const float shift = parts[0][w][q] - M;
+            S = __builtin_fmaf(parts[1][w][q], fast_exp(shift), S);
+            D += __builtin_fmaf((float)split_count(w, KW, p.C), shift, parts[2][w][q]);
+            x_y += parts[3][w][q];
+        }
+        const float lse = fast_log(S);
+        const float all = D - fc * lse;
+        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - M) - lse) : 0.f;
+        const float acc = -(p.w_neg * all + hot);
+        const bool valid = at.live && !ign;
+        out[k] = valid ? acc : 0.f;
+        mine += out[k];
+        cnt += valid ? 1 : 0;
+    }
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if constexpr (Reduce) {
+        const float bs = group_reduce<64>(mine, OpSum());
+        const float bc = group_reduce<64>((float)cnt, OpSum());      // at most 256 per block: exact in fp32
+        if (lane == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int KW, int V>
+__global__ __launch_bounds__(kSplitBlock) void lsr_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                            const Upstream up, T *__restrict__ grad,
+                                                            const LsrParams p) {
+    __shared__ float parts[2][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    using PK = Pack<T, V>;
+    typename PK::Raw raw[KW];
+    int64_t lb[V];
+    float go[V];
+    if (at.here > 0) {                                  // wave-uniform
+        at.load(x, p.C, p.m_size, raw);
+        load_labels<V>(lab + at.pix, lb);
+        load_upstream<V>(up, at.pix, go);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float xv[KW];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                xv[i] = (i < at.here) ? PK::get(raw[i], k) : -INFINITY;
+                mx = fmaxf(mx, xv[i]);
+            }
+            const float c = mx * kLog2e;
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) s += __builtin_amdgcn_exp2f(__builtin_fmaf(xv[i], kLog2e, -c));
+            parts[0][wave][lane * V + k] = c;
+            parts[1][wave][lane * V + k] = s;
+        }
+    }
+    __syncthreads();
+    if (at.here == 0 || !at.live) return;
+    const int used = (p.C + KW - 1) / KW;
+    unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
+#pragma unroll
+    for (int k0 = 0; k0 < V; k0 += PK::kStep) {
+        float g[KW][PK::kStep];
+#pragma unroll
+        for (int kk = 0; kk < PK::kStep; ++kk) {
+            const int k = k0 + kk;
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            keep[k] = ign ? 0u : 0xFFFFFFFFu;
+            const int q = lane * V + k;
+            float cmax = parts[0][0][q];
+            for (int w = 1; w < used; ++w) cmax = fmaxf(cmax, parts[0][w][q]);
+            float S = 0.f;
+            for (int w = 0; w < used; ++w)
+                S = __builtin_fmaf(parts[1][w][q], __builtin_amdgcn_exp2f(parts[0][w][q] - cmax), S);
+            const float gk = go[k];
+            const float scale = p.sumw * gk * __builtin_amdgcn_rcpf(S);
+            float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+            asm("" : "+v"(n_pos), "+v"(n_neg));                             // formed per pixel, not per channel
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(PK::get(raw[i], k), kLog2e, -cmax));
+                g[i][kk] = __builtin_fmaf(e, scale, (rel == i) ? n_pos : n_neg);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < KW; ++i) PK::set(raw[i], k0 / PK::kStep, g[i]);
+    }
+    // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
+    const typename PK::Raw mask = PK::mask(keep);
+#pragma unroll
+    for (int i = 0; i < KW; ++i) raw[i] = raw[i] & mask;
+    at.store(grad, p.m_size, raw);
+}
+
 // --------------------------------------------------------------- group ----
 // G lanes per pixel. G = 64 stages the wave's slice in LDS (each lane re-reads
 // only what it wrote, so no barrier is needed); G = 1 re-reads global memory,
@@ -329,14 +490,45 @@ static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, 
     }
 }
 
+template <class T, int V, bool Reduce>
+static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
+                                 hipStream_t st) {
+    const unsigned grid = split_grid<V>(p.P);
+    switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
+                           part, p);                                                                              \
+        break;
+        PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+#undef PLH_CASE
+    }
+    return grid;
+}
+
+template <class T, int V>
+static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
+                             hipStream_t st) {
+    const unsigned grid = split_grid<V>(p.P);
+    switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_bwd_split<T, KW, V>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
+        break;
+        PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+#undef PLH_CASE
+    }
+}
+
 // Launches the forward; returns the number of blocks that wrote partials.
 template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
                         hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
             const unsigned grid = group_grid(p.P, 4);
             hipLaunchKernelGGL((lsr_fwd_group<T, 64, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
@@ -356,9 +548,10 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
             hipLaunchKernelGGL((lsr_bwd_group<T, 64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, up,
                                grad_logits, p);

@@ -64,18 +64,21 @@ inline int check_gout(const void *gout, int64_t stride) {
 // either way); it needs m_size % V == 0 and every tensor aligned to its V-element access:
 // `typed0/typed1` hold `elem`-byte elements (logits, gradient), `f32a/f32b` fp32 (losses, upstream
 // gradient), labels int64. nullptr = tensor not used.
-enum class Shape { RegsVec, RegsOne, Wave, Lane };
+// Split: the regs shape with the channels of a pixel shared out over the 8 wavefronts of a block
+// (see "the split launch shape" below); only for kernels that have that form (`with_split`).
+enum class Shape { RegsVec, RegsOne, Split, Wave, Lane };
 
 constexpr int kMaxRegsChannels = 32;
+constexpr int kSplitWaves = 8;
+constexpr int kMaxSplitChannels = kMaxRegsChannels * kSplitWaves;
 
 inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, const void *typed0, const void *typed1,
-                        const void *labels, const void *f32a, const void *f32b) {
-    if (dimsize <= kMaxRegsChannels) {
-        const bool vec = (m_size % V == 0) && !(typed0 && misaligned(typed0, V * elem)) &&
-                         !(typed1 && misaligned(typed1, V * elem)) && !(f32a && misaligned(f32a, V * 4)) &&
-                         !(f32b && misaligned(f32b, V * 4)) && !(labels && misaligned(labels, 16));
-        return vec ? Shape::RegsVec : Shape::RegsOne;
-    }
+                        const void *labels, const void *f32a, const void *f32b, bool with_split = false) {
+    const bool vec = (m_size % V == 0) && !(typed0 && misaligned(typed0, V * elem)) &&
+                     !(typed1 && misaligned(typed1, V * elem)) && !(f32a && misaligned(f32a, V * 4)) &&
+                     !(f32b && misaligned(f32b, V * 4)) && !(labels && misaligned(labels, 16));
+    if (dimsize <= kMaxRegsChannels) return vec ? Shape::RegsVec : Shape::RegsOne;
+    if (with_split && vec && dimsize <= kMaxSplitChannels && m_size >= 64) return Shape::Split;
     return m_size == 1 ? Shape::Wave : Shape::Lane;
 }
 
@@ -393,7 +396,8 @@ enum FinishMode { kFinishSum = 0, kFinishMeanOverCount = 1, kFinishMeanOverFixed
 constexpr int64_t kMinPartialSlots = 16384;   // the looping kernels cap their grid at this many blocks
 
 inline int64_t partial_slots(int64_t units) {
-    const int64_t blocks = ceil_div(units > 0 ? units : 1, 256);
+    // the smallest tile any reducing kernel gives a block: 128 pixels (split shape, fp32)
+    const int64_t blocks = ceil_div(units > 0 ? units : 1, 128);
     return blocks > kMinPartialSlots ? blocks : kMinPartialSlots;
 }
 
@@ -528,6 +532,65 @@ struct PixelRef {
 inline bool tiles_are_uniform(int64_t m_size, int V, size_t elem) {
     return m_size % ((int64_t)kRegsBlock * V) == 0 && V * elem == 8 &&
            m_size * (int64_t)elem * kMaxRegsChannels < ((int64_t)1 << 31);
+}
+
+// ---- the "split" launch shape ---------------------------------------------------
+// Channel dimensions of 33..256 in NCHW: the slice of a pixel no longer fits one thread's registers,
+// so the 8 wavefronts of a 512-thread block share it. Lanes still run along the pixels (V per lane,
+// 8 bytes per lane and channel), wavefront w keeps channels [w*KW, (w+1)*KW) in registers, and the
+// per-wavefront softmax statistics of a pixel meet in LDS. Logits are read once, and every
+// per-channel access of a wavefront is one contiguous run of 512 bytes, as in the regs shape.
+constexpr int kSplitBlock = kWave * kSplitWaves;
+
+template <int V>
+inline unsigned split_grid(int64_t pixels) { return (unsigned)ceil_div(pixels, (int64_t)kWave * V); }
+
+// Slots per wavefront for C channels: C/8 rounded up to a multiple of 4 (the kernels are instantiated
+// for 8, 12, ..., 32 slots).
+inline int split_slots(int64_t dimsize) {
+    const int per = (int)ceil_div(dimsize, kSplitWaves);
+    const int kw = (per + 3) / 4 * 4;
+    return kw < 8 ? 8 : kw;
+}
+
+template <class T, int V, int KW>
+struct SplitSlice {
+    int64_t pix;      // first of this lane's V pixels (0 for a lane beyond the end: it still loads, never stores)
+    int64_t base;     // element offset of (image, channel 0, pix)
+    int first;        // first channel of this wavefront
+    int here;         // channels of this wavefront that exist (0..KW), wave-uniform
+    bool live;
+
+    __device__ __forceinline__ SplitSlice(int64_t P, int64_t m_size, int C, unsigned xcd_run) {
+        const int64_t want = (tile_of_block(xcd_run) * kWave + (threadIdx.x & 63)) * V;
+        live = want < P;
+        pix = live ? want : 0;
+        const int64_t n = pix / m_size;
+        base = pix + n * (int64_t)(C - 1) * m_size;
+        first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * KW;
+        const int left = C - first;
+        here = left < 0 ? 0 : (left > KW ? KW : left);
+    }
+    // Slot i holds channel min(first + i, C - 1): a slot beyond the last channel repeats it, so that no
+    // load sits behind a branch; what is computed from such a slot is masked by the caller (i < here).
+    __device__ __forceinline__ void load(const T *t, int C, int64_t m_size, typename Pack<T, V>::Raw (&raw)[KW]) const {
+#pragma unroll
+        for (int i = 0; i < KW; ++i) {
+            const int j = (first + i < C) ? first + i : C - 1;
+            raw[i] = Pack<T, V>::load(t + (base + (int64_t)j * m_size));
+        }
+    }
+    __device__ __forceinline__ void store(T *t, int64_t m_size, const typename Pack<T, V>::Raw (&raw)[KW]) const {
+#pragma unroll
+        for (int i = 0; i < KW; ++i)
+            if (i < here) Pack<T, V>::store(t + (base + (int64_t)(first + i) * m_size), raw[i]);
+    }
+};
+
+// Channels that wavefront w of a split block holds.
+__device__ __forceinline__ int split_count(int w, int KW, int C) {
+    const int left = C - w * KW;
+    return left < 0 ? 0 : (left > KW ? KW : left);
 }
 
 __device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.69314718055994530942f; }

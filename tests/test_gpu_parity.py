@@ -73,6 +73,12 @@ SEG_CASES = [
     ((2, 33, 6, 7), 255, 0.2),                      # deep channel dim in NCHW: one lane per pixel
     ((2, 227, 5, 5), 255, 0.1),
     ((1, 64, 2, 3, 4), 0, 0.3),                     # 5-D input, ignore_index inside the class range
+    ((2, 33, 9, 8), -100, 0.2),                     # 33..256 channels, 64 pixels or more per image: the channels of
+    ((2, 40, 16, 16), 255, 0.1),                    #   a pixel are shared out over the 8 wavefronts of a block;
+    ((3, 100, 10, 10), 255, 0.1),                   #   slots per wavefront 8 .. 32, last wavefronts partly or
+    ((1, 150, 12, 16), 255, 0.05),                  #   wholly empty, pixel counts that leave lanes idle
+    ((2, 256, 8, 8), 255, 0.1),
+    ((2, 257, 8, 8), 255, 0.1),                     # one channel more: a lane per pixel again
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
