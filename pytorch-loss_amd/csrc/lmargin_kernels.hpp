@@ -166,6 +166,201 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     }
 }
 
+// --------------------------------------------------------------- split ----
+// 33..256 channels in NCHW (SplitSlice): every wavefront reduces its channels other than the target,
+//   m_w = max x_j,  s_w = sum e^(x_j - m_w),  a_w = sum e^(x_j - m_w) (x_j - m_w),  d_w = sum (x_j - m_w),
+//   n_w = their number, y_w = the target logit if it is held here,
+// and with M = max_w m_w, h_w = m_w - M the parts combine to
+//   S_no = sum_w s_w e^h_w,  sum_j e^(x_j - M)(x_j - M) = sum_w e^h_w (a_w + h_w s_w),  sum_j (x_j - M) = sum_w d_w + n_w h_w.
+// From there on the formulas are those of lm_regs. Forward: wavefront 0 finishes the pixel; backward:
+// every wavefront finishes it and writes the gradient of its own channels.
+
+template <int V>
+struct LmSplitStats {
+    float m_no, s_no, sum_qt, sum_t, x_y;
+};
+
+template <class T, int KW, int V, bool WantSumT>
+__device__ __forceinline__ void lm_split_parts(const SplitSlice<T, V, KW> &at, const typename Pack<T, V>::Raw (&raw)[KW],
+                                               int k, int rel, float (*parts)[kSplitWaves][kWave * V], int q, int wave) {
+    float xv[KW];
+    float mx = -INFINITY, x_y = -INFINITY;
+    int others = 0;
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        const float xi = Pack<T, V>::get(raw[i], k);
+        const bool hot = (rel == i);
+        x_y = hot ? xi : x_y;
+        xv[i] = (i < at.here && !hot) ? xi : -INFINITY;
+        mx = fmaxf(mx, xv[i]);
+        others += (i < at.here && !hot) ? 1 : 0;
+    }
+    // a wavefront that holds nothing but the target has no maximum: its parts must stay neutral
+    const float ref = (others > 0) ? mx : 0.f;
+    float s = 0.f, a = 0.f, d = 0.f;
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        const float t = xv[i] - ref;                    // -inf for a slot that takes no part
+        const float e = fast_exp(t);
+        s += e;
+        a += (xv[i] > -INFINITY) ? e * t : 0.f;
+        if constexpr (WantSumT) d += (xv[i] > -INFINITY) ? t : 0.f;
+    }
+    parts[0][wave][q] = (others > 0) ? mx : -INFINITY;
+    parts[1][wave][q] = s;
+    parts[2][wave][q] = a;
+    parts[3][wave][q] = x_y;
+    if constexpr (WantSumT) {
+        parts[4][wave][q] = d;
+        parts[5][wave][q] = (float)others;
+    }
+}
+
+template <int V, bool WantSumT>
+__device__ __forceinline__ LmSplitStats<V> lm_split_combine(float (*parts)[kSplitWaves][kWave * V], int q, int used) {
+    LmSplitStats<V> r;
+    float M = parts[0][0][q];
+    for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
+    float S = 0.f, A = 0.f, D = 0.f, x_y = -INFINITY;
+    for (int w = 0; w < used; ++w) {
+        const float m_w = parts[0][w][q];
+        x_y = fmaxf(x_y, parts[3][w][q]);
+        if (m_w == -INFINITY) continue;                 // nothing but the target there
+        const float h = m_w - M;
+        const float eh = fast_exp(h);
+        const float s_w = parts[1][w][q];
+        S = __builtin_fmaf(s_w, eh, S);
+        A = __builtin_fmaf(eh, __builtin_fmaf(h, s_w, parts[2][w][q]), A);
+        if constexpr (WantSumT) D += __builtin_fmaf(parts[5][w][q], h, parts[4][w][q]);
+    }
+    r.m_no = M;
+    r.s_no = S;
+    r.sum_qt = A * __builtin_amdgcn_rcpf(S);
+    r.sum_t = D;
+    r.x_y = x_y;
+    return r;
+}
+
+template <class T, int KW, int V, bool Reduce>
+__global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                           float *__restrict__ loss, Partials part, const LmParams p) {
+    __shared__ float parts[6][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    if (at.here > 0) {                                  // wave-uniform
+        typename Pack<T, V>::Raw raw[KW];
+        at.load(x, p.C, p.m_size, raw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            lm_split_parts<T, KW, V, true>(at, raw, k, rel, parts, lane * V + k, wave);
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const int used = (p.C + KW - 1) / KW;
+    float out[V], score[V];
+    float mine = 0.f;
+    int cnt = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        const LmSplitStats<V> st = lm_split_combine<V, true>(parts, lane * V + k, used);
+        const float m_all = fmaxf(st.m_no, st.x_y);
+        const float t_all = fast_exp(st.m_no - m_all);
+        const float e_y = fast_exp(st.x_y - m_all);
+        const float s_all = __builtin_fmaf(st.s_no, t_all, e_y);
+        const float lse_no = fast_log(st.s_no);
+        const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));
+        const float margin = st.sum_qt - lse_no - p.coeff * (st.sum_t - others * lse_no);
+        const float acc = p.half_lam * margin - (st.x_y - m_all) + fast_log(s_all);
+        const bool valid = at.live && !ign;
+        out[k] = valid ? acc : 0.f;
+        score[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
+        mine += out[k];
+        cnt += valid ? 1 : 0;
+    }
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if (at.live && p.scores) store_vec_cached<V>(p.scores + at.pix, score);
+    if constexpr (Reduce) {
+        const float bs = group_reduce<64>(mine, OpSum());
+        const float bc = group_reduce<64>((float)cnt, OpSum());
+        if (lane == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int KW, int V>
+__global__ __launch_bounds__(kSplitBlock) void lm_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                           const Upstream up, T *__restrict__ grad, const LmParams p) {
+    __shared__ float parts[4][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    using PK = Pack<T, V>;
+    typename PK::Raw raw[KW];
+    int64_t lb[V];
+    float go[V];
+    if (at.here > 0) {                                  // wave-uniform
+        at.load(x, p.C, p.m_size, raw);
+        load_labels<V>(lab + at.pix, lb);
+        load_upstream<V>(up, at.pix, go);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            lm_split_parts<T, KW, V, false>(at, raw, k, rel, parts, lane * V + k, wave);
+        }
+    }
+    __syncthreads();
+    if (at.here == 0 || !at.live) return;
+    const int used = (p.C + KW - 1) / KW;
+    unsigned keep[V];
+#pragma unroll
+    for (int k0 = 0; k0 < V; k0 += PK::kStep) {
+        float g[KW][PK::kStep];
+#pragma unroll
+        for (int kk = 0; kk < PK::kStep; ++kk) {
+            const int k = k0 + kk;
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            keep[k] = ign ? 0u : 0xFFFFFFFFu;
+            const LmSplitStats<V> st = lm_split_combine<V, false>(parts, lane * V + k, used);
+            const float m_all = fmaxf(st.m_no, st.x_y);
+            const float t_all = fast_exp(st.m_no - m_all);
+            const float e_y = fast_exp(st.x_y - m_all);
+            const float s_all = __builtin_fmaf(st.s_no, t_all, e_y);
+            const float inv_all = __builtin_amdgcn_rcpf(s_all);
+            const float sum_qx = st.sum_qt + st.m_no;
+            const float gk = go[k];
+            // g_j = e_j (x_j B + A) - K, e_j = e^(x_j - m_no); the target takes g_y = gk (p_y - 1): see lm_regs
+            float B = p.half_lam * gk * __builtin_amdgcn_rcpf(st.s_no);
+            float A = __builtin_fmaf(B, 1.f - sum_qx, gk * t_all * inv_all);
+            float nK = -p.half_lam * gk * p.coeff;
+            float g_hot = (e_y * inv_all - 1.f) * gk;
+            asm("" : "+v"(A), "+v"(B), "+v"(nK), "+v"(g_hot));                  // formed per pixel, not per channel
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                const float xi = PK::get(raw[i], k);
+                const float e = fast_exp(xi - st.m_no);
+                const float gj = __builtin_fmaf(e, __builtin_fmaf(xi, B, A), nK);
+                g[i][kk] = (rel == i) ? g_hot : gj;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < KW; ++i) PK::set(raw[i], k0 / PK::kStep, g[i]);
+    }
+    const typename PK::Raw mask = PK::mask(keep);
+#pragma unroll
+    for (int i = 0; i < KW; ++i) raw[i] = raw[i] & mask;
+    at.store(grad, p.m_size, raw);
+}
+
 // --------------------------------------------------------------- group ----
 
 constexpr int kLmStageCap = 2048;
@@ -298,8 +493,27 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     const float *second_f32 = go_vec ? go_vec : p.scores;      // the score output belongs to forwards without upstream
     unsigned blocks = 0;
+    // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
+    constexpr bool kHasSplit = !(WantLoss && WantGrad);
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
-                       second_f32)) {
+                       second_f32, kHasSplit)) {
+        case Shape::Split:
+            if constexpr (kHasSplit) {
+                blocks = split_grid<V>(p.P);
+                switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (WantLoss)                                                                                       \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, V, Reduce>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
+                               part, p);                                                                              \
+        else                                                                                                          \
+            hipLaunchKernelGGL((lm_bwd_split<T, KW, V>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
+        break;
+                    PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+#undef PLH_CASE
+                }
+            }
+            break;
         case Shape::RegsVec:
             blocks = launch_regs<T, V, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
