@@ -77,6 +77,67 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
     if (ce) store_vec_cached<V>(ce + at.pix, loss);
 }
 
+// 33..256 channels in NCHW (SplitSlice): per wavefront the maximum, the exponential sum and the target's
+// logit of its channels; wavefront 0 combines them into the pixel's score and cross entropy.
+template <class T, int KW, int V>
+__global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                float *__restrict__ scores, float *__restrict__ ce,
+                                                                int64_t P, int64_t m_size, int C, int64_t ignore,
+                                                                unsigned xcd_run, uint32_t *__restrict__ tables) {
+    __shared__ float parts[3][kSplitWaves][kWave * V];
+    if (tables && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kOhemZeroWords; i += kSplitBlock) tables[i] = 0;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(P, m_size, C, xcd_run);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    if (at.here > 0) {                                  // wave-uniform
+        typename Pack<T, V>::Raw raw[KW];
+        at.load(x, C, m_size, raw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int rel = narrow_label(lb[k], ignore, C, ign) - at.first;
+            float xv[KW];
+            float mx = -INFINITY, x_y = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                xv[i] = (i < at.here) ? Pack<T, V>::get(raw[i], k) : -INFINITY;
+                mx = fmaxf(mx, xv[i]);
+                x_y = (rel == i) ? xv[i] : x_y;
+            }
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) s += fast_exp(xv[i] - mx);
+            const int q = lane * V + k;
+            parts[0][wave][q] = mx;
+            parts[1][wave][q] = s;
+            parts[2][wave][q] = x_y;
+        }
+    }
+    __syncthreads();
+    if (wave != 0 || !at.live) return;
+    const int used = (C + KW - 1) / KW;
+    float out[V], loss[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], ignore, C, ign);
+        const int q = lane * V + k;
+        float M = parts[0][0][q];
+        for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
+        float S = 0.f, x_y = -INFINITY;
+        for (int w = 0; w < used; ++w) {
+            S = __builtin_fmaf(parts[1][w][q], fast_exp(parts[0][w][q] - M), S);
+            x_y = fmaxf(x_y, parts[2][w][q]);
+        }
+        out[k] = (tgt < 0) ? 1.f : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
+        loss[k] = (tgt < 0) ? 0.f : fast_log(S) + (M - x_y);
+    }
+    store_vec_cached<V>(scores + at.pix, out);
+    if (ce) store_vec_cached<V>(ce + at.pix, loss);
+}
+
 // Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).
 template <class T>
 __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
@@ -388,8 +449,20 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce);
-        if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true);
+        if (shape == Shape::Split) {
+            const unsigned grid = split_grid<VT>(P);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
+            switch (split_slots(dimsize)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        hipLaunchKernelGGL((ohem_scores_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, ce, \
+                           P, m_size, C, ignore_index, run, tables);                                                  \
+        break;
+                PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+#undef PLH_CASE
+            }
+        } else if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const bool uni = vec && tiles_are_uniform(m_size, VT, sizeof(T));
             const unsigned grid = vec ? regs_grid<VT>(P) : regs_grid<1>(P);

@@ -242,6 +242,135 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
     at.store_slice(gx, p.C, p.m_size, raw);
 }
 
+// --------------------------------------------------------------- split ----
+// Cross entropy for 33..256 channels in NCHW (SplitSlice). The series needs no maximum, so the parts of
+// a pixel are just each wavefront's sum of the series and the target's term if it is held there.
+
+template <class T, int KW, int V, bool Reduce>
+__global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                  float *__restrict__ loss, Partials part,
+                                                                  const TaylorParams p) {
+    __shared__ float parts[2][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    int64_t lb[V];
+    load_labels<V>(lab + at.pix, lb);
+    if (at.here > 0) {                                  // wave-uniform
+        typename Pack<T, V>::Raw raw[KW];
+        at.load(x, p.C, p.m_size, raw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int rel = narrow_label(lb[k], p.ignore, p.C, ign) - at.first;
+            float s = 0.f, f_y = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                s += (i < at.here) ? f : 0.f;
+                f_y = (rel == i) ? f : f_y;
+            }
+            parts[0][wave][lane * V + k] = s;
+            parts[1][wave][lane * V + k] = f_y;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const int used = (p.C + KW - 1) / KW;
+    float out[V];
+    float mine = 0.f;
+    int cnt = 0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        bool ign;
+        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+        float s = 0.f, f_y = 0.f;
+        for (int w = 0; w < used; ++w) {
+            s += parts[0][w][lane * V + k];
+            f_y += parts[1][w][lane * V + k];
+        }
+        const bool valid = at.live && !ign && tgt >= 0;
+        out[k] = valid ? logf(s) - logf(f_y) : 0.f;
+        mine += out[k];
+        cnt += (at.live && !ign) ? 1 : 0;
+    }
+    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if constexpr (Reduce) {
+        const float bs = group_reduce<64>(mine, OpSum());
+        const float bc = group_reduce<64>((float)cnt, OpSum());
+        if (lane == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int KW, int V>
+__global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                  const Upstream up, T *__restrict__ gx,
+                                                                  const TaylorParams p) {
+    __shared__ float parts[2][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    typename Pack<T, V>::Raw raw[KW];
+    int64_t lb[V];
+    float go[V];
+    int rel[V];
+    unsigned keep[V];
+    if (at.here > 0) {                                  // wave-uniform
+        at.load(x, p.C, p.m_size, raw);
+        load_labels<V>(lab + at.pix, lb);
+        load_upstream<V>(up, at.pix, go);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            bool ign;
+            const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
+            rel[k] = tgt - at.first;
+            keep[k] = (ign || tgt < 0) ? 0u : 0xFFFFFFFFu;
+            float s = 0.f, f_y = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                float f, df;
+                taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                s += (i < at.here) ? f : 0.f;
+                f_y = (rel[k] == i) ? f : f_y;
+            }
+            parts[0][wave][lane * V + k] = s;
+            parts[1][wave][lane * V + k] = f_y;
+        }
+    }
+    __syncthreads();
+    if (at.here == 0 || !at.live) return;
+    const int used = (p.C + KW - 1) / KW;
+    float scale[V], hot[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f, f_y = 0.f;
+        for (int w = 0; w < used; ++w) {
+            s += parts[0][w][lane * V + k];
+            f_y += parts[1][w][lane * V + k];
+        }
+        scale[k] = go[k] * __builtin_amdgcn_rcpf(s);
+        hot[k] = scale[k] - go[k] / f_y;                           // per pixel: what the target channel takes
+        asm("" : "+v"(hot[k]));
+    }
+    const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
+#pragma unroll
+    for (int i = 0; i < KW; ++i) forget_origin(raw[i]);
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        float r[V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float f, df;
+            taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+            r[k] = df * ((rel[k] == i) ? hot[k] : scale[k]);
+        }
+        raw[i] = Pack<T, V>::put(r) & mask;
+    }
+    at.store(gx, p.m_size, raw);
+}
+
 // --------------------------------------------------------------- group ----
 // Any dimsize: G lanes share one slice and stride over it (G = 64: a wavefront per row when the
 // dimension is the contiguous one; G = 1: a lane per slice). The series is re-evaluated in each
@@ -340,8 +469,28 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                        const TaylorParams &p, hipStream_t st) {
     constexpr int VT = ElemTraits<T>::kVec;
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
+    constexpr bool kHasSplit = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);
     const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
-                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec);
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit);
+    if constexpr (kHasSplit) {
+        if (shape == Shape::Split) {
+            const unsigned grid = split_grid<VT>(p.P);
+            switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (Kind == kTaylorCeFwd)                                                                           \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+                               loss, part, p);                                                                        \
+        else                                                                                                          \
+            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
+                               p);                                                                                    \
+        break;
+                PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+#undef PLH_CASE
+            }
+            return grid;
+        }
+    }
     const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
     if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
         const bool vec = (shape == Shape::RegsVec) && g_ok;

@@ -34,6 +34,9 @@ SCORE_CASES = [
     ((37, 10), -100, 0.1),
     ((33, 100), -100, 0.1),              # more than 32 channels: lane per pixel
     ((2, 33, 6, 7), 255, 0.2),
+    ((2, 40, 16, 16), 255, 0.1),         # 33..256 channels: shared out over the wavefronts of a block
+    ((1, 150, 12, 16), 255, 0.05),
+    ((2, 256, 8, 8), 255, 0.1),
     ((2, 19, 16, 16), 255, 1.0),         # everything ignored
 ]
 
@@ -167,13 +170,14 @@ def test_ohem_refuses_cpu_tensors():
 
 @pytest.mark.parametrize("which", ["ce", "lm"])
 @pytest.mark.parametrize("case", ["n_min_covers_everything", "all_ignored", "huge_logit_gaps", "ragged", "deep",
-                                  "rows"])
+                                  "split", "rows"])
 def test_ohem_ce_fused_forward_edge_cases(native, case, which):
     """The one-pass forwards (scores and per-pixel loss from the same sums) against the oracle's
     relabelling followed by torch's cross entropy or the oracle's large-margin loss."""
     import pytorch_loss as pl
     # deep: more channels than the register-resident form holds; rows: (N, C) inputs
-    shape = {"ragged": (2, 7, 9, 11), "deep": (2, 40, 6, 10), "rows": (300, 23)}.get(case, (2, 19, 16, 24))
+    shape = {"ragged": (2, 7, 9, 11), "deep": (2, 40, 6, 10), "split": (2, 150, 8, 16), "rows": (300, 23)}.get(
+        case, (2, 19, 16, 24))
     x, y = seg_inputs(91, shape, 255, 0.05)
     n_min, thresh = y.size // 16, 0.3
     if case == "n_min_covers_everything":
