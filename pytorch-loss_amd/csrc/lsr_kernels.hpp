@@ -161,7 +161,6 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
                                                             float *__restrict__ loss, Partials part,
                                                             const LsrParams p) {
     __shared__ float parts[4][kSplitWaves][kWave * V];
-    __shared__ float red[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
     int64_t lb[V];
@@ -427,6 +426,151 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
     }
 }
 
+// ----------------------------------------------------------------- row ----
+// (N, C) inputs with rows longer than the staging buffer (a vocabulary): one block per row at a time,
+// 16-byte loads, four of them in flight per lane, and a running (maximum, exponential sum) per lane
+// that is rescaled when the maximum moves, so the forward reads the row once; the backward reads it a
+// second time (from cache for all but the longest rows) to write the gradient.
+
+struct RowStats { float m, s, sx; };
+
+template <int L>
+__device__ __forceinline__ void row_absorb(const float (&v)[L], RowStats &st) {
+    float cm = v[0];
+#pragma unroll
+    for (int i = 1; i < L; ++i) cm = fmaxf(cm, v[i]);
+    if (cm > st.m) {
+        st.s *= fast_exp(st.m - cm);               // 0 * exp(-inf) on the first chunk
+        st.m = cm;
+    }
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+        st.s += fast_exp(v[i] - st.m);
+        st.sx += v[i];
+    }
+}
+
+// How a row splits into 16-byte chunks: `head` leading elements up to the first 16-byte boundary,
+// `chunks` chunks, then the rest. Rows of any length qualify as long as the tensor itself starts on a
+// 16-byte boundary (`aligned`); otherwise the whole row is the head.
+template <class T>
+struct RowSplit {
+    int head, chunks, tail_from;
+    __device__ __forceinline__ RowSplit(const T *xs, int C, bool aligned) {
+        constexpr int L = RowChunk<T>::kLen;
+        const int mis = (int)((reinterpret_cast<uintptr_t>(xs) / sizeof(T)) % L);
+        const int lead = (L - mis) % L;
+        head = aligned ? (lead < C ? lead : C) : C;
+        chunks = (C - head) / L;
+        tail_from = head + chunks * L;
+    }
+};
+
+template <class T>
+__device__ __forceinline__ RowStats row_sweep(const T *xs, int C, bool aligned) {
+    constexpr int L = RowChunk<T>::kLen;
+    const RowSplit<T> sp(xs, C, aligned);
+    RowStats st{-INFINITY, 0.f, 0.f};
+    const T *body = xs + sp.head;
+    int i = threadIdx.x;
+    for (; i + 3 * 256 < sp.chunks; i += 4 * 256) {
+        float v[4][L];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * 256) * L, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) row_absorb<L>(v[u], st);
+    }
+    for (; i < sp.chunks; i += 256) {
+        float v[L];
+        RowChunk<T>::load(body + (int64_t)i * L, v);
+        row_absorb<L>(v, st);
+    }
+    // head and tail, element by element (the whole row when it cannot be moved in chunks)
+    for (int j = threadIdx.x; j < sp.head; j += 256) {
+        const float v[1] = {load_one(xs + j)};
+        row_absorb<1>(v, st);
+    }
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += 256) {
+        const float v[1] = {load_one(xs + j)};
+        row_absorb<1>(v, st);
+    }
+    return st;
+}
+
+// Block-wide (M, S [, sum x]) from the per-lane running values. lds4: 4 floats.
+__device__ __forceinline__ RowStats row_combine(RowStats st, float *lds4, bool want_sx) {
+    RowStats r;
+    r.m = block_max_256(st.m, lds4);
+    const float mine = (st.m == -INFINITY) ? 0.f : st.s * fast_exp(st.m - r.m);
+    r.s = block_sum_256(mine, lds4);
+    r.sx = want_sx ? block_sum_256(st.sx, lds4) : 0.f;
+    return r;
+}
+
+template <class T, bool Reduce>
+__global__ __launch_bounds__(256) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                   float *__restrict__ loss, Partials part, const LsrParams p, int vec) {
+    __shared__ float red[4];
+    float mine = 0.f;
+    int cnt = 0;
+    const float fc = (float)p.C;
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
+        const T *xs = x + row * p.C;
+        const RowStats st = row_combine(row_sweep<T>(xs, p.C, vec != 0), red, true);
+        if (threadIdx.x == 0) {
+            const int64_t lb = lab[row];
+            const bool ign = (lb == p.ignore);
+            const bool has_y = !ign && lb >= 0 && lb < p.C;
+            const float x_y = has_y ? load_one(xs + lb) : 0.f;
+            const float lse = fast_log(st.s);
+            const float all = (st.sx - fc * st.m) - fc * lse;
+            const float hot = has_y ? (p.w_pos - p.w_neg) * ((x_y - st.m) - lse) : 0.f;
+            const float acc = ign ? 0.f : -(p.w_neg * all + hot);
+            if (loss) loss[row] = acc;
+            mine += acc;
+            cnt += ign ? 0 : 1;
+        }
+    }
+    if constexpr (Reduce) {
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = mine;
+            part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void lsr_bwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                   const Upstream up, T *__restrict__ grad, const LsrParams p, int vec) {
+    __shared__ float red[4];
+    constexpr int L = RowChunk<T>::kLen;
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
+        const T *xs = x + row * p.C;
+        T *gs = grad + row * p.C;
+        const RowStats st = row_combine(row_sweep<T>(xs, p.C, vec != 0), red, false);
+        const int64_t lb = lab[row];
+        float go[1];
+        load_upstream<1>(up, row, go);
+        const float gk = (lb == p.ignore) ? 0.f : go[0];
+        const float scale = p.sumw * gk / st.s;
+        const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        const RowSplit<T> sp(xs, p.C, vec != 0);         // the gradient row sits at the same offset from its own boundary
+        for (int i = threadIdx.x; i < sp.chunks; i += 256) {
+            float v[L];
+            RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
+#pragma unroll
+            for (int e = 0; e < L; ++e)
+                v[e] = __builtin_fmaf(fast_exp(v[e] - st.m), scale, (sp.head + i * L + e == tgt) ? n_pos : n_neg);
+            RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
+        }
+        for (int j = threadIdx.x; j < sp.head; j += 256)
+            store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
+        for (int j = sp.tail_from + threadIdx.x; j < p.C; j += 256)
+            store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
+    }
+}
+
 // ------------------------------------------------------------ dispatch ----
 
 inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float smooth,
@@ -520,6 +664,13 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     }
 }
 
+// Rows are moved in 16-byte chunks when the tensors start on 16-byte boundaries (a row of the gradient
+// then sits at the same offset from a boundary as the row of logits it belongs to).
+template <class T>
+static int row_chunks_ok(const T *x, const T *grad, int C) {
+    return (!misaligned(x, 16) && !(grad && misaligned(grad, 16))) ? 1 : 0;
+}
+
 // Launches the forward; returns the number of blocks that wrote partials.
 template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
@@ -530,6 +681,12 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
+            if (p.C > kStageCap) {
+                const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p,
+                                   row_chunks_ok<T>(logits, nullptr, p.C));
+                return grid;
+            }
             const unsigned grid = group_grid(p.P, 4);
             hipLaunchKernelGGL((lsr_fwd_group<T, 64, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
             return grid;
@@ -553,6 +710,12 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
+            if (p.C > kStageCap) {
+                const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+                hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(256), 0, st, logits, labels, up, grad_logits, p,
+                                   row_chunks_ok<T>(logits, grad_logits, p.C));
+                break;
+            }
             hipLaunchKernelGGL((lsr_bwd_group<T, 64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, up,
                                grad_logits, p);
             break;

@@ -669,4 +669,45 @@ __device__ __forceinline__ float block_sum_256(float v, float *lds4) {
     return r;
 }
 
+__device__ __forceinline__ float block_max_256(float v, float *lds4) {
+    v = group_reduce<64>(v, OpMax());
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+    __syncthreads();
+    const float r = fmaxf(fmaxf(lds4[0], lds4[1]), fmaxf(lds4[2], lds4[3]));
+    __syncthreads();
+    return r;
+}
+
+// ---- 16-byte chunks of a contiguous row (4 fp32 or 8 16-bit elements) -------------------
+typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
+template <class T> struct RowChunk;
+template <> struct RowChunk<float> {
+    static constexpr int kLen = 4;
+    static __device__ __forceinline__ void load(const float *p, float (&v)[4]) {
+        const plh_f4 t = *reinterpret_cast<const plh_f4 *>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float *p, const float (&v)[4]) {
+        __builtin_nontemporal_store(plh_f4{v[0], v[1], v[2], v[3]}, reinterpret_cast<plh_f4 *>(p));
+    }
+};
+template <class T> struct RowChunk {             // T = f16 or bf16
+    static constexpr int kLen = 8;
+    static __device__ __forceinline__ void load(const T *p, float (&v)[8]) {
+        const plh_u4 t = *reinterpret_cast<const plh_u4 *>(p);
+        const unsigned d[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = widen_lo(d[i], T{});
+            v[2 * i + 1] = widen_hi(d[i], T{});
+        }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&v)[8]) {
+        const plh_u4 t = {narrow2(v[0], v[1], T{}), narrow2(v[2], v[3], T{}), narrow2(v[4], v[5], T{}),
+                          narrow2(v[6], v[7], T{})};
+        __builtin_nontemporal_store(t, reinterpret_cast<plh_u4 *>(p));
+    }
+};
+
 }  // namespace plh

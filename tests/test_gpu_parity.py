@@ -70,6 +70,9 @@ SEG_CASES = [
     ((33, 100), -100, 0.1),                         # (N, C): one wavefront per row
     ((5, 1000), 255, 0.3),
     ((3, 4100), 255, 0.0),                          # row longer than the LDS staging buffer
+    ((5, 4104), 255, 0.2),                          # ... a multiple of 8 elements: 16-byte chunks for 16-bit rows too
+    ((2, 4099), -100, 0.0),                         # ... an odd length: element by element
+    ((3, 50000), 255, 0.3),                         # a vocabulary
     ((2, 33, 6, 7), 255, 0.2),                      # deep channel dim in NCHW: one lane per pixel
     ((2, 227, 5, 5), 255, 0.1),
     ((1, 64, 2, 3, 4), 0, 0.3),                     # 5-D input, ignore_index inside the class range
