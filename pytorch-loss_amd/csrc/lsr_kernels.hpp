@@ -432,7 +432,22 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 // that is rescaled when the maximum moves, so the forward reads the row once; the backward reads it a
 // second time (from cache for all but the longest rows) to write the gradient.
 
+constexpr int kRowBlock = 1024;      // few, large blocks: the rows in flight stay within the last-level cache
+                                     // for the backward's second sweep
 struct RowStats { float m, s, sx; };
+
+// Block-wide reductions for kRowBlock threads; every thread gets the result. lds: kRowBlock / 64 floats.
+template <class Op>
+__device__ __forceinline__ float row_block_reduce(float v, float *lds, Op op) {
+    v = group_reduce<64>(v, op);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = lds[0];
+#pragma unroll
+    for (int w = 1; w < kRowBlock / 64; ++w) r = op(r, lds[w]);
+    __syncthreads();
+    return r;
+}
 
 template <int L>
 __device__ __forceinline__ void row_absorb(const float (&v)[L], RowStats &st) {
@@ -473,44 +488,44 @@ __device__ __forceinline__ RowStats row_sweep(const T *xs, int C, bool aligned) 
     RowStats st{-INFINITY, 0.f, 0.f};
     const T *body = xs + sp.head;
     int i = threadIdx.x;
-    for (; i + 3 * 256 < sp.chunks; i += 4 * 256) {
+    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
         float v[4][L];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * 256) * L, v[u]);
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
 #pragma unroll
         for (int u = 0; u < 4; ++u) row_absorb<L>(v[u], st);
     }
-    for (; i < sp.chunks; i += 256) {
+    for (; i < sp.chunks; i += kRowBlock) {
         float v[L];
         RowChunk<T>::load(body + (int64_t)i * L, v);
         row_absorb<L>(v, st);
     }
     // head and tail, element by element (the whole row when it cannot be moved in chunks)
-    for (int j = threadIdx.x; j < sp.head; j += 256) {
+    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) {
         const float v[1] = {load_one(xs + j)};
         row_absorb<1>(v, st);
     }
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += 256) {
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) {
         const float v[1] = {load_one(xs + j)};
         row_absorb<1>(v, st);
     }
     return st;
 }
 
-// Block-wide (M, S [, sum x]) from the per-lane running values. lds4: 4 floats.
-__device__ __forceinline__ RowStats row_combine(RowStats st, float *lds4, bool want_sx) {
+// Block-wide (M, S [, sum x]) from the per-lane running values.
+__device__ __forceinline__ RowStats row_combine(RowStats st, float *lds, bool want_sx) {
     RowStats r;
-    r.m = block_max_256(st.m, lds4);
+    r.m = row_block_reduce(st.m, lds, OpMax());
     const float mine = (st.m == -INFINITY) ? 0.f : st.s * fast_exp(st.m - r.m);
-    r.s = block_sum_256(mine, lds4);
-    r.sx = want_sx ? block_sum_256(st.sx, lds4) : 0.f;
+    r.s = row_block_reduce(mine, lds, OpSum());
+    r.sx = want_sx ? row_block_reduce(st.sx, lds, OpSum()) : 0.f;
     return r;
 }
 
 template <class T, bool Reduce>
-__global__ __launch_bounds__(256) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+__global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                    float *__restrict__ loss, Partials part, const LsrParams p, int vec) {
-    __shared__ float red[4];
+    __shared__ float red[kRowBlock / 64];
     float mine = 0.f;
     int cnt = 0;
     const float fc = (float)p.C;
@@ -540,9 +555,9 @@ __global__ __launch_bounds__(256) void lsr_fwd_row(const T *__restrict__ x, cons
 }
 
 template <class T>
-__global__ __launch_bounds__(256) void lsr_bwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+__global__ __launch_bounds__(kRowBlock) void lsr_bwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                    const Upstream up, T *__restrict__ grad, const LsrParams p, int vec) {
-    __shared__ float red[4];
+    __shared__ float red[kRowBlock / 64];
     constexpr int L = RowChunk<T>::kLen;
     for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
         const T *xs = x + row * p.C;
@@ -556,7 +571,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_row(const T *__restrict__ x, cons
         const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
         const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
         const RowSplit<T> sp(xs, p.C, vec != 0);         // the gradient row sits at the same offset from its own boundary
-        for (int i = threadIdx.x; i < sp.chunks; i += 256) {
+        for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
             float v[L];
             RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
 #pragma unroll
@@ -564,9 +579,9 @@ __global__ __launch_bounds__(256) void lsr_bwd_row(const T *__restrict__ x, cons
                 v[e] = __builtin_fmaf(fast_exp(v[e] - st.m), scale, (sp.head + i * L + e == tgt) ? n_pos : n_neg);
             RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
         }
-        for (int j = threadIdx.x; j < sp.head; j += 256)
+        for (int j = threadIdx.x; j < sp.head; j += kRowBlock)
             store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
-        for (int j = sp.tail_from + threadIdx.x; j < p.C; j += 256)
+        for (int j = sp.tail_from + threadIdx.x; j < p.C; j += kRowBlock)
             store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
     }
 }
@@ -683,7 +698,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::Wave: {
             if (p.C > kStageCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p,
+                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
@@ -712,7 +727,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::Wave:
             if (p.C > kStageCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(256), 0, st, logits, labels, up, grad_logits, p,
+                hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, up, grad_logits, p,
                                    row_chunks_ok<T>(logits, grad_logits, p.C));
                 break;
             }
