@@ -1,15 +1,19 @@
 // Shared device/host helpers for the gfx950 loss kernels.
 //
-// Two execution shapes are used for every channel-dim reduction:
-//   "regs"  : lanes run along consecutive pixels, each thread owns V pixels and
-//             keeps the whole channel slice in VGPRs. Each per-channel load of a
-//             wavefront is one contiguous 64*V*4-byte run, logits are read from
-//             HBM exactly once and no cross-lane traffic is needed.
-//   "group" : G lanes share one pixel and stride over its channels (G = 64: a
-//             wavefront per row, for (N, C) inputs where the channel dim is the
-//             contiguous one; G = 1: a lane per pixel for deep channel dims in
-//             NCHW). Reductions inside a group use DPP/swizzle, the slice is
-//             staged in LDS when it has to be read more than once.
+// Execution shapes of the channel-dim reductions:
+//   "regs"  : up to 32 channels. Lanes run along consecutive pixels, each thread owns V
+//             pixels and keeps the whole channel slice in VGPRs. Each per-channel load of
+//             a wavefront is one contiguous 64*V*4-byte run, logits are read from HBM
+//             exactly once and no cross-lane traffic is needed.
+//   "split" : 33..256 channels in NCHW. The regs shape with the slice of a pixel shared out
+//             over the 8 wavefronts of a block; per-wavefront statistics meet in LDS.
+//   "row"   : (N, C) rows longer than an LDS staging buffer (label smoothing only): a block
+//             per row, 16-byte chunks, running maximum and sum.
+//   "group" : everything else. G lanes share one pixel and stride over its channels (G = 64:
+//             a wavefront per row, for (N, C) inputs where the channel dim is the contiguous
+//             one; G = 1: a lane per pixel for deep channel dims in NCHW). Reductions inside
+//             a group use DPP/swizzle, the slice is staged in LDS when it has to be read
+//             more than once.
 #pragma once
 
 #include <hip/hip_runtime.h>
