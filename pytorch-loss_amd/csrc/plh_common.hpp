@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/pytorch_loss_hip.h"
 
 namespace plh {
@@ -463,12 +465,24 @@ inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(p
 //              block-uniform (one scalar division per block, scalar base + 32-bit lane offset
 //              addressing) and no bounds check is needed. Power-of-two image sizes take this form.
 //   general  - any m_size: per-thread 64-bit index arithmetic and a bounds check.
+//   rows     - the general form with one pixel per thread when m_size == 1, i.e. (N, C) inputs (flattened
+//              channels-last segmentation logits, classification): a lane's channels are contiguous and
+//              neighbouring lanes sit C elements apart, so direct loads would touch 64 cache lines per
+//              instruction. Instead a wavefront copies its 64 rows (one contiguous run of 64*C elements)
+//              through LDS with consecutive lanes on consecutive addresses, and every lane then picks its
+//              row out of LDS; stores go the same way back. The LDS index is skewed by one word per 32
+//              (e + e/32), which keeps the row reads of 64 lanes off a common bank for every C.
+constexpr int kRowsTileWords = 64 * kMaxRegsChannels + 64 * kMaxRegsChannels / 32 + 8;
+__device__ __forceinline__ int rows_skew(int e) { return e + (e >> 5); }
+
 template <int V, bool Uniform>
 struct PixelRef {
     int64_t pix;        // first pixel of this thread (index into labels / losses)
     int64_t base;       // block-uniform part of the channel-0 offset (Uniform) or the whole of it
     unsigned lane_off;  // 32-bit per-thread part (Uniform), else 0
     bool live;
+    int64_t wave_first; // rows form: the first row of this wavefront, and how many of its 64 rows exist
+    int rows_here;
 
     __device__ __forceinline__ PixelRef(int64_t P, int64_t m_size, int C, unsigned xcd_run) {
         if constexpr (Uniform) {
@@ -479,13 +493,63 @@ struct PixelRef {
             pix = start + lane_off;
             live = true;
         } else {
-            const int64_t want = (tile_of_block(xcd_run) * kRegsBlock + threadIdx.x) * V;
+            const int64_t tile = tile_of_block(xcd_run);
+            const int64_t want = (tile * kRegsBlock + threadIdx.x) * V;
             live = want < P;
             pix = live ? want : 0;
             const int64_t n = pix / m_size;
             base = pix + n * (int64_t)(C - 1) * m_size;
             lane_off = 0;
+            if constexpr (V == 1) {
+                wave_first = tile * kRegsBlock + (threadIdx.x & ~63u);
+                const int64_t left = P - wave_first;
+                rows_here = left < 0 ? 0 : (left > 64 ? 64 : (int)left);
+            }
         }
+    }
+    // (N, C) input with more than one channel: the rows form
+    static __device__ __forceinline__ bool rows_form(int C, int64_t m_size) { return V == 1 && !Uniform && m_size == 1 && C > 1; }
+
+    template <class T>
+    static __device__ __forceinline__ typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type *rows_tile() {
+        typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
+        __shared__ Word tile[kRegsBlock / 64][kRowsTileWords];
+        return tile[threadIdx.x >> 6];
+    }
+    template <class T, int CP>
+    __device__ __forceinline__ void rows_load(const T *t, int C, unsigned (&raw)[CP]) const {
+        typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
+        Word *tile = rows_tile<T>();
+        const int lane = threadIdx.x & 63;
+        const Word *src = reinterpret_cast<const Word *>(t) + wave_first * C;
+        const int n = rows_here * C;
+        // the lanes that are still here are the first rows_here of the wavefront (kernels may have let the others go)
+        if (lane < rows_here)
+            for (int e = lane; e < n; e += rows_here) tile[rows_skew(e)] = src[e];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, C)) raw[j] = tile[rows_skew(lane * C + j)];
+        __builtin_amdgcn_wave_barrier();        // the tile is free again only when every lane has its row
+    }
+    template <class T, int CP>
+    __device__ __forceinline__ void rows_store(T *t, int C, const unsigned (&raw)[CP]) const {
+        typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
+        Word *tile = rows_tile<T>();
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+            if (chan_ok<CP>(j, C)) tile[rows_skew(lane * C + j)] = (Word)raw[j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        Word *dst = reinterpret_cast<Word *>(t) + wave_first * C;
+        const int n = rows_here * C;
+        if (lane < rows_here)
+            for (int e = lane; e < n; e += rows_here) dst[e] = tile[rows_skew(e)];
+        __builtin_amdgcn_wave_barrier();
     }
     // address of channel j for this thread's pixels
     template <class T>
@@ -508,6 +572,12 @@ struct PixelRef {
                 if (chan_ok<CP>(j, C))
                     raw[j] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off * (unsigned)sizeof(T), j * row, kBufferNT);
         } else {
+            if constexpr (V == 1) {
+                if (rows_form(C, m_size)) {         // kernel-uniform
+                    rows_load<T, CP>(t, C, raw);
+                    return;
+                }
+            }
 #pragma unroll
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, C)) raw[j] = Pack<T, V>::load(chan(t, j, m_size));
@@ -524,6 +594,12 @@ struct PixelRef {
                 if (chan_ok<CP>(j, C))
                     __builtin_amdgcn_raw_buffer_store_b64(raw[j], rsrc, lane_off * (unsigned)sizeof(T), j * row, kBufferNT);
         } else {
+            if constexpr (V == 1) {
+                if (rows_form(C, m_size)) {         // kernel-uniform
+                    rows_store<T, CP>(t, C, raw);
+                    return;
+                }
+            }
 #pragma unroll
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, C)) Pack<T, V>::store(chan(t, j, m_size), raw[j]);

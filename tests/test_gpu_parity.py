@@ -66,7 +66,10 @@ SEG_CASES = [
     ((3, 2, 5, 8), -100, 0.2),
     ((4, 32, 4, 4), 255, 0.0),
     ((2, 3, 1, 1), 255, 0.0),
-    ((37, 10), -100, 0.1),                          # (N, C) classification input, C <= 32
+    ((37, 10), -100, 0.1),                          # (N, C) classification input, C <= 32: a wavefront moves
+    ((300, 19), 255, 0.1),                          #   its 64 rows through LDS; full and partly filled wavefronts,
+    ((1000, 32), -100, 0.1),                        #   even and odd row lengths
+    ((129, 2), 255, 0.2),
     ((33, 100), -100, 0.1),                         # (N, C): one wavefront per row
     ((5, 1000), 255, 0.3),
     ((3, 4100), 255, 0.0),                          # row longer than the LDS staging buffer
