@@ -475,6 +475,39 @@ inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(p
 constexpr int kRowsTileWords = 64 * kMaxRegsChannels + 64 * kMaxRegsChannels / 32 + 8;
 __device__ __forceinline__ int rows_skew(int e) { return e + (e >> 5); }
 
+typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes of consecutive elements starting at element e (a multiple of 4 or 8, so the skew is the same
+// for all of them) into / out of a skewed tile.
+template <class Word>
+__device__ __forceinline__ void rows_scatter16(Word *tile, int e, plh_u4 v) {
+    Word *at = tile + rows_skew(e);
+    const unsigned d[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (sizeof(Word) == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) at[i] = d[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            at[2 * i] = (Word)(d[i] & 0xFFFFu);
+            at[2 * i + 1] = (Word)(d[i] >> 16);
+        }
+    }
+}
+template <class Word>
+__device__ __forceinline__ plh_u4 rows_gather16(const Word *tile, int e) {
+    const Word *at = tile + rows_skew(e);
+    unsigned d[4];
+    if constexpr (sizeof(Word) == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) d[i] = at[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) d[i] = (unsigned)at[2 * i] | ((unsigned)at[2 * i + 1] << 16);
+    }
+    return plh_u4{d[0], d[1], d[2], d[3]};
+}
+
 template <int V, bool Uniform>
 struct PixelRef {
     int64_t pix;        // first pixel of this thread (index into labels / losses)
@@ -523,9 +556,22 @@ struct PixelRef {
         const int lane = threadIdx.x & 63;
         const Word *src = reinterpret_cast<const Word *>(t) + wave_first * C;
         const int n = rows_here * C;
-        // the lanes that are still here are the first rows_here of the wavefront (kernels may have let the others go)
-        if (lane < rows_here)
+        if (rows_here == 64 && (reinterpret_cast<uintptr_t>(t) & 15) == 0) {
+            // a full wavefront: 64*C elements from a 16-byte boundary on, moved 16 bytes per lane and step
+            constexpr int kPer = 16 / (int)sizeof(Word);
+            const plh_u4 *src4 = reinterpret_cast<const plh_u4 *>(src);
+            const int groups = n / kPer;
+            for (int g = lane; g < groups; g += 128) {
+                const bool two = g + 64 < groups;
+                const plh_u4 a = src4[g];
+                const plh_u4 b = two ? src4[g + 64] : a;
+                rows_scatter16<Word>(tile, g * kPer, a);
+                if (two) rows_scatter16<Word>(tile, (g + 64) * kPer, b);
+            }
+        } else if (lane < rows_here) {
+            // the lanes that are still here are the first rows_here of the wavefront (kernels may have let the others go)
             for (int e = lane; e < n; e += rows_here) tile[rows_skew(e)] = src[e];
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -547,8 +593,15 @@ struct PixelRef {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         Word *dst = reinterpret_cast<Word *>(t) + wave_first * C;
         const int n = rows_here * C;
-        if (lane < rows_here)
+        if (rows_here == 64 && (reinterpret_cast<uintptr_t>(t) & 15) == 0) {
+            constexpr int kPer = 16 / (int)sizeof(Word);
+            plh_u4 *dst4 = reinterpret_cast<plh_u4 *>(dst);
+            const int groups = n / kPer;
+            for (int g = lane; g < groups; g += 64)
+                __builtin_nontemporal_store(rows_gather16<Word>(tile, g * kPer), dst4 + g);
+        } else if (lane < rows_here) {
             for (int e = lane; e < n; e += rows_here) dst[e] = tile[rows_skew(e)];
+        }
         __builtin_amdgcn_wave_barrier();
     }
     // address of channel j for this thread's pixels
@@ -760,7 +813,6 @@ __device__ __forceinline__ float block_max_256(float v, float *lds4) {
 }
 
 // ---- 16-byte chunks of a contiguous row (4 fp32 or 8 16-bit elements) -------------------
-typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
 template <class T> struct RowChunk;
 template <> struct RowChunk<float> {
     static constexpr int kLen = 4;
