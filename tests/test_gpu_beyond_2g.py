@@ -136,6 +136,62 @@ def test_per_pixel_losses(pl, op, case):
         assert np.all(np.abs(got_g - want_g) <= 2 ** -8 * np.abs(want_g) + 1e-6)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_rows_of_few_channels(pl, dtype):
+    """(N, C) logits (flattened channels-last segmentation): wavefronts move their 64 rows through LDS."""
+    n, c = 113100001, 19
+    assert n * c > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(29)
+    x = torch.empty(n, c, device="cuda", dtype=dtype)
+    step = 1 << 24
+    for i in range(0, n, step):
+        x[i:i + step] = (2 * torch.randn(min(step, n - i), c, device="cuda", generator=g)).to(dtype)
+    y = torch.randint(0, c, (n,), device="cuda", generator=g)
+    y[torch.rand(n, device="cuda", generator=g) < 0.05] = IGN
+    x.requires_grad_()
+    per = pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="none", ignore_index=IGN)(x, y)
+    gout = (torch.rand(n, device="cuda") + 0.5).to(dtype)
+    per.backward(gout)
+    ign = y == IGN
+    assert (per[ign] == 0).all() and (per[~ign] > 0).all() and (x.grad[ign] == 0).all()
+    rows = np.concatenate([np.arange(0, 600), np.arange(n - 600, n), np.random.default_rng(4).integers(0, n, 2048)]
+                          + [np.arange(b // c - 300, b // c + 300) for b in range(2 ** 31, n * c, 2 ** 31)])
+    it = torch.from_numpy(rows).cuda()
+    xs, ys, gs = x.detach()[it].float().cpu().numpy(), y[it].cpu().numpy(), gout[it].float().cpu().numpy()
+    want, want_g = oracle.lsr_forward(xs, ys, IGN, 0.1), oracle.lsr_backward(xs, ys, IGN, 0.1, gs)
+    got, got_g = per.detach()[it].float().cpu().numpy(), x.grad[it].float().cpu().numpy()
+    if dtype == torch.float32:
+        assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6)
+        assert np.abs(got_g - want_g).max() <= 1e-5
+    else:
+        assert np.all(np.abs(got - want) <= 2 ** -8 * np.abs(want) + 1e-6)
+        assert np.all(np.abs(got_g - want_g) <= 2 ** -8 * np.abs(want_g) + 1e-6)
+
+
+def test_long_rows(pl):
+    """Vocabulary-sized rows, more than 2^31 elements in all: a block per row."""
+    n, c = 43000, 50257
+    assert n * c > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.empty(n, c, device="cuda")
+    for i in range(0, n, 4096):
+        x[i:i + 4096] = 2 * torch.randn(min(4096, n - i), c, device="cuda", generator=g)
+    y = torch.randint(0, c, (n,), device="cuda", generator=g)
+    y[torch.rand(n, device="cuda", generator=g) < 0.05] = IGN
+    x.requires_grad_()
+    per = pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="none", ignore_index=IGN)(x, y)
+    gout = torch.rand(n, device="cuda") + 0.5
+    per.backward(gout)
+    rows = np.concatenate([np.arange(0, 8), np.arange(n - 8, n), np.arange(2 ** 31 // c - 4, 2 ** 31 // c + 4)])
+    it = torch.from_numpy(rows).cuda()
+    xs, ys, gs = x.detach()[it].cpu().numpy(), y[it].cpu().numpy(), gout[it].cpu().numpy()
+    want, want_g = oracle.lsr_forward(xs, ys, IGN, 0.1), oracle.lsr_backward(xs, ys, IGN, 0.1, gs)
+    assert np.all(np.abs(per.detach()[it].cpu().numpy() - want) <= 1e-5 * np.abs(want) + 1e-6)
+    assert np.abs(x.grad[it].cpu().numpy() - want_g).max() <= 1e-5
+    # every row's gradient sums to gout * (sumw - sum of the weights) = 0 for valid rows
+    assert x.grad.sum(dim=1).abs().max().item() < 1e-4
+
+
 def test_focal(pl):
     numel = 2 ** 31 + 12345
     g = torch.Generator(device="cuda").manual_seed(5)
