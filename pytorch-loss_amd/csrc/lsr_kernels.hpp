@@ -426,6 +426,127 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
     }
 }
 
+// ------------------------------------------------- wavefront per row, in registers ----
+// (N, C) inputs with 33..2048 channels: a wavefront holds a whole row in registers (NI steps of 64 lanes,
+// 16 bytes per lane and step where the rows allow it, else one element), so the row is read once and
+// every load of the row is in flight before the first one is used. Four rows per block at a time.
+
+template <class T, int NI, bool Wide>
+struct WaveRow {
+    static constexpr int L = Wide ? RowChunk<T>::kLen : 1;
+    float v[NI][L];
+    // elements beyond the row read as -inf (and are never stored)
+    __device__ __forceinline__ void load(const T *xs, int C, int lane) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e0 = (lane + 64 * i) * L;
+            const bool ok = e0 < C;                   // rows moved in chunks hold a whole number of them
+            const T *at = xs + (ok ? e0 : 0);
+            if constexpr (Wide) RowChunk<T>::load(at, v[i]);
+            else v[i][0] = load_one(at);
+#pragma unroll
+            for (int l = 0; l < L; ++l) v[i][l] = ok ? v[i][l] : -INFINITY;
+        }
+    }
+    __device__ __forceinline__ float max() const {
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int l = 0; l < L; ++l) m = fmaxf(m, v[i][l]);
+        return group_reduce<64>(m, OpMax());
+    }
+};
+
+template <class T, int NI, bool Wide, bool Reduce>
+__global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                    float *__restrict__ loss, Partials part, const LsrParams p) {
+    __shared__ float red[4];
+    constexpr int L = WaveRow<T, NI, Wide>::L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mine = 0.f, cnt = 0.f;
+    const float fc = (float)p.C;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+        const T *xs = x + row * p.C;
+        WaveRow<T, NI, Wide> r;
+        r.load(xs, p.C, lane);
+        const float mx = r.max();
+        float s = 0.f, d = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                const float t = r.v[i][l] - mx;       // -inf beyond the row
+                s += fast_exp(t);
+                d += (t > -INFINITY) ? t : 0.f;
+            }
+        s = group_reduce<64>(s, OpSum());
+        d = group_reduce<64>(d, OpSum());             // sum_j (x_j - mx)
+        if (lane == 0) {
+            const int64_t lb = lab[row];
+            const bool ign = (lb == p.ignore);
+            const bool has_y = !ign && lb >= 0 && lb < p.C;
+            const float x_y = has_y ? load_one(xs + lb) : 0.f;
+            const float lse = fast_log(s);
+            const float all = d - fc * lse;
+            const float hot = has_y ? (p.w_pos - p.w_neg) * ((x_y - mx) - lse) : 0.f;
+            const float acc = ign ? 0.f : -(p.w_neg * all + hot);
+            if (loss) loss[row] = acc;
+            mine += acc;
+            cnt += ign ? 0.f : 1.f;
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+template <class T, int NI, bool Wide>
+__global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                    const Upstream up, T *__restrict__ grad, const LsrParams p) {
+    constexpr int L = WaveRow<T, NI, Wide>::L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+        const T *xs = x + row * p.C;
+        T *gs = grad + row * p.C;
+        WaveRow<T, NI, Wide> r;
+        r.load(xs, p.C, lane);
+        const int64_t lb = lab[row];
+        float go[1];
+        load_upstream<1>(up, row, go);
+        const float mx = r.max();
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                r.v[i][l] = fast_exp(r.v[i][l] - mx);
+                s += r.v[i][l];
+            }
+        s = group_reduce<64>(s, OpSum());
+        const float gk = (lb == p.ignore) ? 0.f : go[0];
+        const float scale = p.sumw * gk / s;
+        const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e0 = (lane + 64 * i) * L;
+            if (e0 < p.C) {
+                float g[L];
+#pragma unroll
+                for (int l = 0; l < L; ++l) g[l] = __builtin_fmaf(r.v[i][l], scale, (e0 + l == tgt) ? n_pos : n_neg);
+                if constexpr (Wide) RowChunk<T>::store(gs + e0, g);
+                else store_one(gs + e0, g[0]);
+            }
+        }
+    }
+}
+
 // ----------------------------------------------------------------- row ----
 // (N, C) inputs with rows longer than the staging buffer (a vocabulary): one block per row at a time,
 // 16-byte loads, four of them in flight per lane, and a running (maximum, exponential sum) per lane
@@ -679,6 +800,28 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     }
 }
 
+// Steps a wavefront needs for a row of C elements (2, 8 or 32: the instantiated sizes), and whether its
+// rows can be moved in 16-byte chunks (every row then starts on a 16-byte boundary).
+template <class T>
+static bool wrow_wide(const T *x, const T *grad, int C) {
+    return C % RowChunk<T>::kLen == 0 && !misaligned(x, 16) && !(grad && misaligned(grad, 16));
+}
+template <class T>
+static int wrow_steps(int C, bool wide) {
+    const int per = 64 * (wide ? RowChunk<T>::kLen : 1);
+    const int need = (C + per - 1) / per;
+    return need <= 2 ? 2 : (need <= 8 ? 8 : 32);
+}
+#define PLH_WROW_DISPATCH(LAUNCH)                                        \
+    do {                                                                 \
+        const bool wide = wrow_wide<T>(logits, wrow_grad, p.C);         \
+        switch (wrow_steps<T>(p.C, wide)) {                              \
+            case 2: if (wide) LAUNCH(2, true); else LAUNCH(2, false); break; \
+            case 8: if (wide) LAUNCH(8, true); else LAUNCH(8, false); break; \
+            default: LAUNCH(32, false); break;                           \
+        }                                                                \
+    } while (0)
+
 // Rows are moved in 16-byte chunks when the tensors start on 16-byte boundaries (a row of the gradient
 // then sits at the same offset from a boundary as the row of logits it belongs to).
 template <class T>
@@ -703,7 +846,10 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
                 return grid;
             }
             const unsigned grid = group_grid(p.P, 4);
-            hipLaunchKernelGGL((lsr_fwd_group<T, 64, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            const T *wrow_grad = nullptr;
+#define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p)
+            PLH_WROW_DISPATCH(PLH_GO);
+#undef PLH_GO
             return grid;
         }
         case Shape::Lane: {
@@ -731,8 +877,13 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                                    row_chunks_ok<T>(logits, grad_logits, p.C));
                 break;
             }
-            hipLaunchKernelGGL((lsr_bwd_group<T, 64>), dim3(group_grid(p.P, 4)), dim3(256), 0, st, logits, labels, up,
-                               grad_logits, p);
+            {
+                const unsigned grid = group_grid(p.P, 4);
+                const T *wrow_grad = grad_logits;
+#define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W>), dim3(grid), dim3(256), 0, st, logits, labels, up, grad_logits, p)
+                PLH_WROW_DISPATCH(PLH_GO);
+#undef PLH_GO
+            }
             break;
         case Shape::Lane:
             hipLaunchKernelGGL((lsr_bwd_group<T, 1>), dim3(group_grid(p.P, 256)), dim3(256), 0, st, logits, labels, up,
