@@ -395,6 +395,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         if constexpr (WantGrad) load_upstream<1>(up, pc, go);
 
         float m_no = -INFINITY, x_y = -INFINITY;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -404,6 +405,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         x_y = group_reduce<G>(x_y, OpMax());
         const float m_all = fmaxf(m_no, x_y);
         float s_no = 0.f, sum_ex = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const float e = (lb == j) ? 0.f : fast_exp(t - m_no);
@@ -419,6 +421,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         const float sum_qx = sum_ex * inv_no;
         const float lse_no = logf(s_no);
         float acc = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float xv = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const bool hot = (lb == j);

@@ -176,9 +176,12 @@ __global__ __launch_bounds__(256) void lov_keys_lane(const T *__restrict__ x, co
         const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
         const int64_t lb = lab[pix];
         float mx = -INFINITY;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) s += expf(load_one(xs + (int64_t)j * m_size) - mx);
+#pragma unroll 8
         for (int j = 0; j < C; ++j) {
             const uint32_t key = make_key(expf(load_one(xs + (int64_t)j * m_size) - mx) / s, lb == j, lb == ignore);
             keys[(int64_t)j * P + pix] = key;
@@ -895,16 +898,20 @@ __global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ go
         const T *xs = x + base;
         const int64_t lb = lab[pix];
         float mx = -INFINITY;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) s += expf(load_one(xs + (int64_t)j * m_size) - mx);
         float dot = 0.f;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) {
             const float p = expf(load_one(xs + (int64_t)j * m_size) - mx) / s;
             const float dj = jacc[(int64_t)j * P + pix] * gout[j];
             dot += p * ((lb == j) ? -dj : dj);
         }
         const bool ign = (lb == ignore);
+#pragma unroll 8
         for (int j = 0; j < C; ++j) {
             const float p = expf(load_one(xs + (int64_t)j * m_size) - mx) / s;
             const float dj = jacc[(int64_t)j * P + pix] * gout[j];

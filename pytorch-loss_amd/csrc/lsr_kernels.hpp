@@ -339,6 +339,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         const int64_t lb = lab[pc];
 
         float mx = -INFINITY;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -346,6 +347,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             s += fast_exp(t - mx);
@@ -353,6 +355,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         s = group_reduce<G>(s, OpSum());
         const float lse = logf(s);
         float acc = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             acc -= ((t - mx) - lse) * ((lb == j) ? p.w_pos : p.w_neg);
@@ -401,6 +404,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         load_upstream<1>(up, pc, go);
 
         float mx = -INFINITY;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -408,6 +412,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const float e = fast_exp(t - mx);
@@ -418,6 +423,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         if (live) {
             const float gk = (lb == p.ignore) ? 0.f : go[0];
             const float scale = p.sumw * gk / s;
+#pragma unroll (G == 1 ? 4 : 1)
             for (int j = sub; j < p.C; j += G) {
                 const float e = staged ? stage[j] : fast_exp(load_one(xs + (int64_t)j * p.m_size) - mx);
                 store_one(gs + (int64_t)j * p.m_size, e * scale - ((lb == j) ? p.w_pos : p.w_neg) * gk);

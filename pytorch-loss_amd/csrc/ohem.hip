@@ -156,8 +156,10 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
         const int64_t n = pix / m_size;
         const T *xs = x + (pix + n * (int64_t)(C - 1) * m_size);
         float mx = -INFINITY;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) mx = fmaxf(mx, load_one(xs + (int64_t)j * m_size));
         float s = 0.f;
+#pragma unroll 8
         for (int j = 0; j < C; ++j) s += fast_exp(load_one(xs + (int64_t)j * m_size) - mx);
         const float x_y = load_one(xs + lb * m_size);
         scores[pix] = fminf(fast_exp(x_y - mx) / s, 1.f);

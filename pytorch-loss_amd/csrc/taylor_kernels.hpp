@@ -396,6 +396,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
         const T *xs = x + base;
         float s = 0.f, dot = 0.f;
+#pragma unroll (G == 1 ? 4 : 1)
         for (int j = sub; j < p.C; j += G) {
             float f, df;
             taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -411,6 +412,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         if constexpr (Kind == kTaylorFwd) {
             const float ls = logf(s);
             if (live)
+#pragma unroll (G == 1 ? 4 : 1)
                 for (int j = sub; j < p.C; j += G) {
                     float f, df;
                     taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -419,6 +421,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         } else if constexpr (Kind == kTaylorBwd) {
             const float mid = p.use_log ? dot * inv : dot * inv * inv;
             if (live)
+#pragma unroll (G == 1 ? 4 : 1)
                 for (int j = sub; j < p.C; j += G) {
                     float f, df;
                     taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -443,6 +446,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
                 load_upstream<1>(up, pc, go);
                 const float gk = has_y ? go[0] : 0.f;
                 if (live)
+#pragma unroll (G == 1 ? 4 : 1)
                     for (int j = sub; j < p.C; j += G) {
                         float f, df;
                         taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
