@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         if constexpr (WantGrad) load_upstream<1>(up, pc, go);
 
         float m_no = -INFINITY, x_y = -INFINITY;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         x_y = group_reduce<G>(x_y, OpMax());
         const float m_all = fmaxf(m_no, x_y);
         float s_no = 0.f, sum_ex = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const float e = (lb == j) ? 0.f : fast_exp(t - m_no);
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         const float sum_qx = sum_ex * inv_no;
         const float lse_no = logf(s_no);
         float acc = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float xv = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const bool hot = (lb == j);
@@ -450,6 +450,117 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
     }
     if constexpr (WantCount) {
         if ((threadIdx.x & 63) == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+// ------------------------------------------------- wavefront per row, in registers ----
+// (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
+// sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group<64>.
+
+template <class T, int NI, bool Wide, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+__global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                               const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
+                                               unsigned long long *__restrict__ valid_cnt, Partials part,
+                                               const LmParams p) {
+    __shared__ float red[4];
+    constexpr int L = WaveRow<T, NI, Wide>::L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mine = 0.f, cnt = 0.f;
+    unsigned long long n_valid = 0;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+        const T *xs = x + row * p.C;
+        WaveRow<T, NI, Wide> r;
+        r.load(xs, p.C, lane);
+        const int64_t lb = lab[row];
+        const bool ign = (lb == p.ignore);
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        float go[1] = {1.f};
+        if constexpr (WantGrad) load_upstream<1>(up, row, go);
+
+        float m_no = -INFINITY, x_y = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                const float t = r.v[i][l];              // -inf beyond the row
+                const bool hot = ((lane + 64 * i) * L + l == tgt);
+                x_y = hot ? t : x_y;
+                m_no = hot ? m_no : fmaxf(m_no, t);
+            }
+        m_no = group_reduce<64>(m_no, OpMax());
+        x_y = group_reduce<64>(x_y, OpMax());
+        const float m_all = fmaxf(m_no, x_y);
+        float s_no = 0.f, sum_ex = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool ok = (lane + 64 * i) * L < p.C;
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                const float t = r.v[i][l];
+                const bool hot = ((lane + 64 * i) * L + l == tgt);
+                const float e = hot ? 0.f : fast_exp(t - m_no);
+                s_no += e;
+                sum_ex += ok ? e * t : 0.f;
+            }
+        }
+        s_no = group_reduce<64>(s_no, OpSum());
+        sum_ex = group_reduce<64>(sum_ex, OpSum());
+        const float t_all = fast_exp(m_no - m_all);
+        const float e_y = fast_exp(x_y - m_all);
+        const float s_all = s_no * t_all + e_y;
+        const float inv_no = 1.f / s_no, inv_all = 1.f / s_all;
+        const float sum_qx = sum_ex * inv_no;
+        const float lse_no = logf(s_no);
+        const float g_hot = (e_y * inv_all - 1.f) * go[0];
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e0 = (lane + 64 * i) * L;
+            const bool ok = e0 < p.C;
+            float g[L];
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                const float xv = r.v[i][l];
+                const bool hot = (e0 + l == tgt);
+                const float e = fast_exp(xv - m_no);
+                const float q = e * inv_no;
+                if constexpr (WantLoss)
+                    acc += (hot || !ok) ? 0.f : p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
+                if constexpr (WantGrad) {
+                    const float g_cold = (e * t_all * inv_all + p.half_lam * ((xv + 1.f - sum_qx) * q - p.coeff)) * go[0];
+                    g[l] = ign ? 0.f : (hot ? g_hot : g_cold);
+                }
+            }
+            if constexpr (WantGrad) {
+                if (ok) {
+                    T *gs = grad + row * p.C + e0;
+                    if constexpr (Wide) RowChunk<T>::store(gs, g);
+                    else store_one(gs, g[0]);
+                }
+            }
+        }
+        if constexpr (WantLoss) {
+            acc = group_reduce<64>(acc, OpSum());
+            acc += -(x_y - m_all) + logf(s_all);
+            if (lane == 0) {
+                if (loss) loss[row] = ign ? 0.f : acc;
+                if (p.scores) p.scores[row] = (ign || tgt < 0) ? 1.f : fminf(e_y * inv_all, 1.f);
+                mine += ign ? 0.f : acc;
+                cnt += ign ? 0.f : 1.f;
+            }
+        }
+        if constexpr (WantCount) n_valid += (lane == 0 && !ign) ? 1 : 0;
+    }
+    if constexpr (WantCount) {
+        if (lane == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
     if constexpr (Reduce) {
         const float bs = block_sum_256(mine, red);
@@ -525,6 +636,15 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             break;
         case Shape::Wave:
             blocks = group_grid(p.P, 4);
+            if (p.C <= kLmStageCap) {
+                const T *wrow_grad = WantGrad ? grad : nullptr;
+#define PLH_GO(NI, W)                                                                                              \
+    hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st, \
+                       x, lab, up, loss, grad, cnt, part, p)
+                PLH_WROW_DISPATCH(x, wrow_grad, p.C, PLH_GO);
+#undef PLH_GO
+                break;
+            }
             hipLaunchKernelGGL((lm_group<T, 64, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
                                x, lab, up, loss, grad, cnt, part, p);
             break;

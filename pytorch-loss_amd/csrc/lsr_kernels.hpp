@@ -339,7 +339,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         const int64_t lb = lab[pc];
 
         float mx = -INFINITY;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             s += fast_exp(t - mx);
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         s = group_reduce<G>(s, OpSum());
         const float lse = logf(s);
         float acc = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             acc -= ((t - mx) - lse) * ((lb == j) ? p.w_pos : p.w_neg);
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         load_upstream<1>(up, pc, go);
 
         float mx = -INFINITY;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
             if (staged) stage[j] = t;
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
             const float e = fast_exp(t - mx);
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
         if (live) {
             const float gk = (lb == p.ignore) ? 0.f : go[0];
             const float scale = p.sumw * gk / s;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
             for (int j = sub; j < p.C; j += G) {
                 const float e = staged ? stage[j] : fast_exp(load_one(xs + (int64_t)j * p.m_size) - mx);
                 store_one(gs + (int64_t)j * p.m_size, e * scale - ((lb == j) ? p.w_pos : p.w_neg) * gk);
@@ -436,33 +436,6 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 // (N, C) inputs with 33..2048 channels: a wavefront holds a whole row in registers (NI steps of 64 lanes,
 // 16 bytes per lane and step where the rows allow it, else one element), so the row is read once and
 // every load of the row is in flight before the first one is used. Four rows per block at a time.
-
-template <class T, int NI, bool Wide>
-struct WaveRow {
-    static constexpr int L = Wide ? RowChunk<T>::kLen : 1;
-    float v[NI][L];
-    // elements beyond the row read as -inf (and are never stored)
-    __device__ __forceinline__ void load(const T *xs, int C, int lane) {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int e0 = (lane + 64 * i) * L;
-            const bool ok = e0 < C;                   // rows moved in chunks hold a whole number of them
-            const T *at = xs + (ok ? e0 : 0);
-            if constexpr (Wide) RowChunk<T>::load(at, v[i]);
-            else v[i][0] = load_one(at);
-#pragma unroll
-            for (int l = 0; l < L; ++l) v[i][l] = ok ? v[i][l] : -INFINITY;
-        }
-    }
-    __device__ __forceinline__ float max() const {
-        float m = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-#pragma unroll
-            for (int l = 0; l < L; ++l) m = fmaxf(m, v[i][l]);
-        return group_reduce<64>(m, OpMax());
-    }
-};
 
 template <class T, int NI, bool Wide, bool Reduce>
 __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
@@ -806,28 +779,6 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     }
 }
 
-// Steps a wavefront needs for a row of C elements (2, 8 or 32: the instantiated sizes), and whether its
-// rows can be moved in 16-byte chunks (every row then starts on a 16-byte boundary).
-template <class T>
-static bool wrow_wide(const T *x, const T *grad, int C) {
-    return C % RowChunk<T>::kLen == 0 && !misaligned(x, 16) && !(grad && misaligned(grad, 16));
-}
-template <class T>
-static int wrow_steps(int C, bool wide) {
-    const int per = 64 * (wide ? RowChunk<T>::kLen : 1);
-    const int need = (C + per - 1) / per;
-    return need <= 2 ? 2 : (need <= 8 ? 8 : 32);
-}
-#define PLH_WROW_DISPATCH(LAUNCH)                                        \
-    do {                                                                 \
-        const bool wide = wrow_wide<T>(logits, wrow_grad, p.C);         \
-        switch (wrow_steps<T>(p.C, wide)) {                              \
-            case 2: if (wide) LAUNCH(2, true); else LAUNCH(2, false); break; \
-            case 8: if (wide) LAUNCH(8, true); else LAUNCH(8, false); break; \
-            default: LAUNCH(32, false); break;                           \
-        }                                                                \
-    } while (0)
-
 // Rows are moved in 16-byte chunks when the tensors start on 16-byte boundaries (a row of the gradient
 // then sits at the same offset from a boundary as the row of logits it belongs to).
 template <class T>
@@ -854,7 +805,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
             const unsigned grid = group_grid(p.P, 4);
             const T *wrow_grad = nullptr;
 #define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p)
-            PLH_WROW_DISPATCH(PLH_GO);
+            PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
         }
@@ -887,7 +838,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                 const unsigned grid = group_grid(p.P, 4);
                 const T *wrow_grad = grad_logits;
 #define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W>), dim3(grid), dim3(256), 0, st, logits, labels, up, grad_logits, p)
-                PLH_WROW_DISPATCH(PLH_GO);
+                PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
 #undef PLH_GO
             }
             break;

@@ -88,6 +88,10 @@ inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, con
     return m_size == 1 ? Shape::Wave : Shape::Lane;
 }
 
+// Channel-loop unrolling of the group kernels: with one lane per pixel (G = 1) the loads of a loop are
+// a channel plane apart, and unrolling keeps four of them in flight per lane.
+template <int G> constexpr int kGroupUnroll = (G == 1) ? 4 : 1;
+
 // Grid for the group kernels: they loop, so the grid is capped.
 inline unsigned group_grid(int64_t pixels, int pixels_per_block) {
     const int64_t want = ceil_div(pixels, pixels_per_block);
@@ -841,5 +845,71 @@ template <class T> struct RowChunk {             // T = f16 or bf16
         __builtin_nontemporal_store(t, reinterpret_cast<plh_u4 *>(p));
     }
 };
+
+// ---- a wavefront holds one row of an (N, C) input in registers ----------------------------
+// NI steps of 64 lanes, 16 bytes per lane and step where the rows allow it, else one element: the row is
+// read once and every load of it is in flight before the first one is used.
+template <class T, int NI, bool Wide>
+struct WaveRow {
+    static constexpr int L = Wide ? RowChunk<T>::kLen : 1;
+    float v[NI][L];
+    // elements beyond the row read as -inf (and are never stored)
+    __device__ __forceinline__ void load(const T *xs, int C, int lane) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e0 = (lane + 64 * i) * L;
+            const bool ok = e0 < C;                   // rows moved in chunks hold a whole number of them
+            const T *at = xs + (ok ? e0 : 0);
+            if constexpr (Wide) RowChunk<T>::load(at, v[i]);
+            else v[i][0] = load_one(at);
+#pragma unroll
+            for (int l = 0; l < L; ++l) v[i][l] = ok ? v[i][l] : -INFINITY;
+        }
+    }
+    __device__ __forceinline__ float max() const {
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int l = 0; l < L; ++l) m = fmaxf(m, v[i][l]);
+        return group_reduce<64>(m, OpMax());
+    }
+};
+
+// Steps a wavefront needs for a row of C elements (the instantiated sizes: 2, 4 or 8 steps of 16-byte
+// chunks -- 8 only for fp32, whose chunks hold 4 elements -- and 2 .. 32 steps of single elements), and
+// whether its rows can be moved in 16-byte chunks (every row then starts on a 16-byte boundary).
+constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
+
+template <class T>
+static bool wrow_wide(const T *x, const T *grad, int C) {
+    return C % RowChunk<T>::kLen == 0 && !misaligned(x, 16) && !(grad && misaligned(grad, 16));
+}
+template <class T>
+static int wrow_steps(int C, bool wide) {
+    const int per = 64 * (wide ? RowChunk<T>::kLen : 1);
+    const int need = (C + per - 1) / per;
+    int steps = 2;
+    while (steps < need) steps *= 2;
+    return steps;
+}
+#define PLH_WROW_DISPATCH_WIDE(WIDE, C, LAUNCH)                              \
+    do {                                                                     \
+        const bool wrow_is_wide = (WIDE);                                    \
+        switch (wrow_steps<T>(C, wrow_is_wide)) {                            \
+            case 2: if (wrow_is_wide) LAUNCH(2, true); else LAUNCH(2, false); break; \
+            case 4: if (wrow_is_wide) LAUNCH(4, true); else LAUNCH(4, false); break; \
+            case 8:                                                          \
+                if constexpr (RowChunk<T>::kLen == 4) {                      \
+                    if (wrow_is_wide) { LAUNCH(8, true); break; }            \
+                }                                                            \
+                LAUNCH(8, false);                                            \
+                break;                                                       \
+            case 16: LAUNCH(16, false); break;                               \
+            default: LAUNCH(32, false); break;                               \
+        }                                                                    \
+    } while (0)
+#define PLH_WROW_DISPATCH(X, GRAD, C, LAUNCH) PLH_WROW_DISPATCH_WIDE(wrow_wide<T>(X, GRAD, C), C, LAUNCH)
+
 
 }  // namespace plh

@@ -396,7 +396,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
         const T *xs = x + base;
         float s = 0.f, dot = 0.f;
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             float f, df;
             taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         if constexpr (Kind == kTaylorFwd) {
             const float ls = logf(s);
             if (live)
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
                 for (int j = sub; j < p.C; j += G) {
                     float f, df;
                     taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
         } else if constexpr (Kind == kTaylorBwd) {
             const float mid = p.use_log ? dot * inv : dot * inv * inv;
             if (live)
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
                 for (int j = sub; j < p.C; j += G) {
                     float f, df;
                     taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
@@ -446,13 +446,111 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
                 load_upstream<1>(up, pc, go);
                 const float gk = has_y ? go[0] : 0.f;
                 if (live)
-#pragma unroll (G == 1 ? 4 : 1)
+#pragma unroll kGroupUnroll<G>
                     for (int j = sub; j < p.C; j += G) {
                         float f, df;
                         taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
                         store_one(out + base + (int64_t)j * p.m_size,
                                   has_y ? df * inv * gk - ((lb == j) ? df / f * gk : 0.f) : 0.f);
                     }
+            }
+        }
+    }
+    if constexpr (Reduce) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256(cnt, red);
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
+}
+
+// ------------------------------------------------- wavefront per row, in registers ----
+// (N, C) inputs along dim 1 with 33..2048 channels: the row (and, for the softmax backward, the row of
+// upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
+// taylor_group<64>.
+
+template <class T, int NI, bool Wide, int Kind, bool Reduce>
+__global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
+                                                   const int64_t *__restrict__ lab, const Upstream up,
+                                                   T *__restrict__ out, float *__restrict__ loss, Partials part,
+                                                   const TaylorParams p) {
+    __shared__ float red[4];
+    constexpr int L = WaveRow<T, NI, Wide>::L;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mine = 0.f, cnt = 0.f;
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+        const T *xs = x + row * p.C;
+        WaveRow<T, NI, Wide> r;
+        r.load(xs, p.C, lane);
+        WaveRow<T, (Kind == kTaylorBwd) ? NI : 1, Wide> rg;
+        if constexpr (Kind == kTaylorBwd) rg.load(g + row * p.C, p.C, lane);
+        float s = 0.f, dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool ok = (lane + 64 * i) * L < p.C;          // elements beyond the row hold -inf
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+                float f, df;
+                taylor_pair(r.v[i][l], p.order, f, df);
+                s += ok ? f : 0.f;
+                if constexpr (Kind == kTaylorBwd) {
+                    const float gj = rg.v[i][l];
+                    dot += ok ? (p.use_log ? gj : f * gj) : 0.f;
+                }
+            }
+        }
+        s = group_reduce<64>(s, OpSum());
+        if constexpr (Kind == kTaylorBwd) dot = group_reduce<64>(dot, OpSum());
+        const float inv = 1.f / s;
+        if constexpr (Kind == kTaylorCeFwd) {
+            if (lane == 0) {
+                const int64_t lb = lab[row];
+                const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
+                float f_y = 1.f, df;
+                if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df);
+                const float v = has_y ? logf(s) - logf(f_y) : 0.f;
+                if (loss) loss[row] = v;
+                mine += v;
+                cnt += (lb != p.ignore) ? 1.f : 0.f;
+            }
+        } else {
+            const float ls = logf(s);
+            const float mid = p.use_log ? dot * inv : dot * inv * inv;
+            int tgt = -1;
+            float gk = 0.f;
+            if constexpr (Kind == kTaylorCeBwd) {
+                const int64_t lb = lab[row];
+                float go[1];
+                load_upstream<1>(up, row, go);
+                if (lb != p.ignore && lb >= 0 && lb < p.C) {
+                    tgt = (int)lb;
+                    gk = go[0];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int e0 = (lane + 64 * i) * L;
+                float o[L];
+#pragma unroll
+                for (int l = 0; l < L; ++l) {
+                    float f, df;
+                    taylor_pair(r.v[i][l], p.order, f, df);
+                    if constexpr (Kind == kTaylorFwd) {
+                        o[l] = p.use_log ? logf(f) - ls : f * inv;
+                    } else if constexpr (Kind == kTaylorBwd) {
+                        const float gj = rg.v[i][l];
+                        o[l] = p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
+                    } else {
+                        o[l] = (tgt >= 0) ? df * inv * gk - ((e0 + l == tgt) ? df / f * gk : 0.f) : 0.f;
+                    }
+                }
+                if (e0 < p.C) {
+                    T *at = out + row * p.C + e0;
+                    if constexpr (Wide) RowChunk<T>::store(at, o);
+                    else store_one(at, o[0]);
+                }
             }
         }
     }
@@ -528,6 +626,16 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     }
     if (p.m_size == 1) {
         const unsigned grid = group_grid(p.P, 4);
+        if (p.C <= kWaveRowCap) {
+            const bool wide = wrow_wide<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C) &&
+                              !(Kind == kTaylorBwd && misaligned(g, 16));
+#define PLH_GO(NI, W)                                                                                             \
+    hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss, \
+                       part, p)
+            PLH_WROW_DISPATCH_WIDE(wide, p.C, PLH_GO);
+#undef PLH_GO
+            return grid;
+        }
         hipLaunchKernelGGL((taylor_group<T, 64, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss,
                            part, p);
         return grid;

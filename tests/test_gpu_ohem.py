@@ -32,7 +32,14 @@ SCORE_CASES = [
     ((2, 19, 7, 9), 255, 0.1),           # one pixel per thread
     ((3, 2, 5, 8), -100, 0.2),
     ((37, 10), -100, 0.1),
-    ((33, 100), -100, 0.1),              # more than 32 channels: lane per pixel
+    ((33, 100), -100, 0.1),              # (N, C) rows of 33..2048 channels: a wavefront per row, in registers
+    ((9, 77), -100, 0.1),                #   (odd lengths element by element, others in 16-byte chunks)
+    ((6, 1000), 255, 0.2),
+    ((7, 201), 255, 0.1),
+    ((4, 1001), -100, 0.1),
+    ((5, 1544), 255, 0.1),
+    ((3, 2047), 255, 0.1),
+    ((2, 2056), 255, 0.0),               # longer rows: lane per pixel
     ((2, 33, 6, 7), 255, 0.2),
     ((2, 40, 16, 16), 255, 0.1),         # 33..256 channels: shared out over the wavefronts of a block
     ((1, 150, 12, 16), 255, 0.05),

@@ -72,6 +72,13 @@ SEG_CASES = [
     ((129, 2), 255, 0.2),
     ((33, 100), -100, 0.1),                         # (N, C): one wavefront per row
     ((5, 1000), 255, 0.3),
+    ((9, 77), -100, 0.1),                           # ... rows of 33..2048 channels sit in a wavefront's registers:
+    ((6, 501), 255, 0.2),                           #   2 .. 32 steps, element by element for odd lengths,
+    ((7, 201), 255, 0.1),
+    ((4, 1001), -100, 0.1),
+    ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
+    ((2, 2048), 255, 0.0),
+    ((2, 2049), -100, 0.0),                         # one channel more: staged or swept rows
     ((3, 4100), 255, 0.0),                          # row longer than the LDS staging buffer
     ((5, 4104), 255, 0.2),                          # ... a multiple of 8 elements: 16-byte chunks for 16-bit rows too
     ((2, 4099), -100, 0.0),                         # ... an odd length: element by element

@@ -17,12 +17,19 @@ CASES = [
     ((2, 19, 7, 9), 1),                          # one pixel per thread
     ((3, 2, 5, 8), 1),
     ((37, 10), 1),                               # (N, C), C <= 32
-    ((33, 100), 1),                              # wavefront per row
+    ((33, 100), 1),                              # wavefront per row, the row in registers
+    ((9, 77), 1),                                #   odd length: element by element
     ((2, 33, 6, 7), 1),                          # lane per slice
     ((24, 6, 5), 0),                             # dim 0: 24 channels 30 apart
     ((2, 3, 4, 40), 3),                          # last dim of a 4-D tensor: rows of 40
     ((2, 3, 16, 5), -2),
     ((64, 8, 8, 8), 0),                          # dim 0 with 64 channels: lane per slice
+    ((6, 1000), 1),                              # longer register rows: 8 and 32 steps per wavefront
+    ((3, 2047), -1),
+    ((7, 201), 1),
+    ((4, 1001), 1),
+    ((5, 1544), 1),
+    ((2, 2056), 1),                              # beyond the register rows: strided sweeps
 ]
 
 
@@ -61,7 +68,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:6])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-6:-1])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
