@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|lsr_c150|lsr_vocab]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|lsr_c150|lsr_vocab|lmargin_rows]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -64,6 +64,9 @@ WORKLOADS = {
                      "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lsr_vocab": dict(base="lsr", shape=(8192, 32000), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8192,32000), "
                       "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
+    # classifier-sized rows: a wavefront holds a row in its registers
+    "lmargin_rows": dict(base="lmargin", shape=(65536, 1000), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (65536,1000), "
+                         "int64 labels 5% ignore=255, lam=0.3, mean"),
     "ohem": dict(shape=(8, 19, 1024, 1024), desc="OhemCELoss fwd+bwd (relabelling and cross entropy in one forward pass), fp32 logits (8,19,1024,1024) "
                  "= 4*N(0,1), int64 labels 5% ignore=255, score_thresh=0.7, n_min=P/16"),
 }

@@ -465,19 +465,22 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 // (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
 // sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group<64>.
 
-template <class T, int NI, bool Wide, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, int NI, bool Wide, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G>
 __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
                                                const LmParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide>::L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    const WaveRowAt<G> at;
+    const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
     unsigned long long n_valid = 0;
-    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+    for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
+        const bool live = r0 + at.grp < p.P;
+        const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide> r;
+        WaveRow<T, NI, Wide, G> r;
         r.load(xs, p.C, lane);
         const int64_t lb = lab[row];
         const bool ign = (lb == p.ignore);
@@ -491,28 +494,28 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 const float t = r.v[i][l];              // -inf beyond the row
-                const bool hot = ((lane + 64 * i) * L + l == tgt);
+                const bool hot = ((lane + G * i) * L + l == tgt);
                 x_y = hot ? t : x_y;
                 m_no = hot ? m_no : fmaxf(m_no, t);
             }
-        m_no = group_reduce<64>(m_no, OpMax());
-        x_y = group_reduce<64>(x_y, OpMax());
+        m_no = group_reduce<G>(m_no, OpMax());
+        x_y = group_reduce<G>(x_y, OpMax());
         const float m_all = fmaxf(m_no, x_y);
         float s_no = 0.f, sum_ex = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const bool ok = (lane + 64 * i) * L < p.C;
+            const bool ok = (lane + G * i) * L < p.C;
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 const float t = r.v[i][l];
-                const bool hot = ((lane + 64 * i) * L + l == tgt);
+                const bool hot = ((lane + G * i) * L + l == tgt);
                 const float e = hot ? 0.f : fast_exp(t - m_no);
                 s_no += e;
                 sum_ex += ok ? e * t : 0.f;
             }
         }
-        s_no = group_reduce<64>(s_no, OpSum());
-        sum_ex = group_reduce<64>(sum_ex, OpSum());
+        s_no = group_reduce<G>(s_no, OpSum());
+        sum_ex = group_reduce<G>(sum_ex, OpSum());
         const float t_all = fast_exp(m_no - m_all);
         const float e_y = fast_exp(x_y - m_all);
         const float s_all = s_no * t_all + e_y;
@@ -523,7 +526,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int e0 = (lane + 64 * i) * L;
+            const int e0 = (lane + G * i) * L;
             const bool ok = e0 < p.C;
             float g[L];
 #pragma unroll
@@ -540,7 +543,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                 }
             }
             if constexpr (WantGrad) {
-                if (ok) {
+                if (ok && live) {
                     T *gs = grad + row * p.C + e0;
                     if constexpr (Wide) RowChunk<T>::store(gs, g);
                     else store_one(gs, g[0]);
@@ -548,16 +551,16 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             }
         }
         if constexpr (WantLoss) {
-            acc = group_reduce<64>(acc, OpSum());
+            acc = group_reduce<G>(acc, OpSum());
             acc += -(x_y - m_all) + logf(s_all);
-            if (lane == 0) {
+            if (lane == 0 && live) {
                 if (loss) loss[row] = ign ? 0.f : acc;
                 if (p.scores) p.scores[row] = (ign || tgt < 0) ? 1.f : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0.f : 1.f;
             }
         }
-        if constexpr (WantCount) n_valid += (lane == 0 && !ign) ? 1 : 0;
+        if constexpr (WantCount) n_valid += (lane == 0 && live && !ign) ? 1 : 0;
     }
     if constexpr (WantCount) {
         if (lane == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
@@ -635,16 +638,19 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::Wave:
-            blocks = group_grid(p.P, 4);
-            if (p.C <= kLmStageCap) {
+            if (p.C <= kWaveRowCap) {
                 const T *wrow_grad = WantGrad ? grad : nullptr;
-#define PLH_GO(NI, W)                                                                                              \
-    hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st, \
-                       x, lab, up, loss, grad, cnt, part, p)
+#define PLH_GO(NI, W, G)                                                                                           \
+    do {                                                                                                           \
+        blocks = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                     \
+        hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G>), dim3(blocks), dim3(256), 0, \
+                           st, x, lab, up, loss, grad, cnt, part, p);                                              \
+    } while (0)
                 PLH_WROW_DISPATCH(x, wrow_grad, p.C, PLH_GO);
 #undef PLH_GO
                 break;
             }
+            blocks = group_grid(p.P, 4);
             hipLaunchKernelGGL((lm_group<T, 64, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
                                x, lab, up, loss, grad, cnt, part, p);
             break;

@@ -437,18 +437,20 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 // 16 bytes per lane and step where the rows allow it, else one element), so the row is read once and
 // every load of the row is in flight before the first one is used. Four rows per block at a time.
 
-template <class T, int NI, bool Wide, bool Reduce>
+template <class T, int NI, bool Wide, bool Reduce, int G>
 __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     float *__restrict__ loss, Partials part, const LsrParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide>::L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    const WaveRowAt<G> at;
     float mine = 0.f, cnt = 0.f;
     const float fc = (float)p.C;
-    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+    for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
+        const bool live = r0 + at.grp < p.P;
+        const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide> r;
-        r.load(xs, p.C, lane);
+        WaveRow<T, NI, Wide, G> r;
+        r.load(xs, p.C, at.sub);
         const float mx = r.max();
         float s = 0.f, d = 0.f;
 #pragma unroll
@@ -459,9 +461,9 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
                 s += fast_exp(t);
                 d += (t > -INFINITY) ? t : 0.f;
             }
-        s = group_reduce<64>(s, OpSum());
-        d = group_reduce<64>(d, OpSum());             // sum_j (x_j - mx)
-        if (lane == 0) {
+        s = group_reduce<G>(s, OpSum());
+        d = group_reduce<G>(d, OpSum());              // sum_j (x_j - mx)
+        if (at.sub == 0 && live) {
             const int64_t lb = lab[row];
             const bool ign = (lb == p.ignore);
             const bool has_y = !ign && lb >= 0 && lb < p.C;
@@ -485,16 +487,18 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
     }
 }
 
-template <class T, int NI, bool Wide>
+template <class T, int NI, bool Wide, int G>
 __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, T *__restrict__ grad, const LsrParams p) {
-    constexpr int L = WaveRow<T, NI, Wide>::L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    const WaveRowAt<G> at;
+    for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
+        const bool live = r0 + at.grp < p.P;
+        const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
         T *gs = grad + row * p.C;
-        WaveRow<T, NI, Wide> r;
-        r.load(xs, p.C, lane);
+        WaveRow<T, NI, Wide, G> r;
+        r.load(xs, p.C, at.sub);
         const int64_t lb = lab[row];
         float go[1];
         load_upstream<1>(up, row, go);
@@ -507,15 +511,15 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
                 r.v[i][l] = fast_exp(r.v[i][l] - mx);
                 s += r.v[i][l];
             }
-        s = group_reduce<64>(s, OpSum());
+        s = group_reduce<G>(s, OpSum());
         const float gk = (lb == p.ignore) ? 0.f : go[0];
         const float scale = p.sumw * gk / s;
         const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
         const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int e0 = (lane + 64 * i) * L;
-            if (e0 < p.C) {
+            const int e0 = (at.sub + G * i) * L;
+            if (e0 < p.C && live) {
                 float g[L];
 #pragma unroll
                 for (int l = 0; l < L; ++l) g[l] = __builtin_fmaf(r.v[i][l], scale, (e0 + l == tgt) ? n_pos : n_neg);
@@ -802,9 +806,14 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
-            const unsigned grid = group_grid(p.P, 4);
+            unsigned grid = 0;
             const T *wrow_grad = nullptr;
-#define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p)
+#define PLH_GO(NI, W, G)                                                                                            \
+    do {                                                                                                            \
+        grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                        \
+        hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce, G>), dim3(grid), dim3(256), 0, st, logits, labels, losses, \
+                           part, p);                                                                                \
+    } while (0)
             PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
@@ -835,9 +844,10 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                 break;
             }
             {
-                const unsigned grid = group_grid(p.P, 4);
                 const T *wrow_grad = grad_logits;
-#define PLH_GO(NI, W) hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W>), dim3(grid), dim3(256), 0, st, logits, labels, up, grad_logits, p)
+#define PLH_GO(NI, W, G)                                                                                          \
+    hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
+                       st, logits, labels, up, grad_logits, p)
                 PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
 #undef PLH_GO
             }

@@ -169,37 +169,42 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
 
 // (N, C) inputs with 33..2048 channels: a wavefront per row, the row in its registers (one read of HBM,
 // every access a contiguous run), where the lane-per-pixel kernel would have each lane walk its own row.
-template <class T, int NI, bool Wide>
+template <class T, int NI, bool Wide, int G>
 __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         float *__restrict__ scores, float *__restrict__ ce, int64_t P,
                                                         int C, int64_t ignore, uint32_t *__restrict__ tables) {
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += 256) tables[i] = 0;
-    constexpr int L = WaveRow<T, NI, Wide>::L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    const WaveRowAt<G> at;
+    for (int64_t r0 = at.start; r0 < P; r0 += at.stride) {   // wave-uniform
+        const bool live = r0 + at.grp < P;
+        const int64_t row = live ? r0 + at.grp : P - 1;
         const int64_t lb = lab[row];
-        if (lb == ignore || lb < 0 || lb >= C) {
-            if (lane == 0) {
-                scores[row] = 1.f;
-                if (ce) ce[row] = 0.f;
+        const bool no_target = (lb == ignore || lb < 0 || lb >= C);
+        if constexpr (G == 64) {                              // the wavefront has one row: skip its loads
+            if (no_target) {
+                if (at.sub == 0) {
+                    scores[row] = 1.f;
+                    if (ce) ce[row] = 0.f;
+                }
+                continue;
             }
-            continue;
         }
         const T *xs = x + row * C;
-        WaveRow<T, NI, Wide> r;
-        r.load(xs, C, lane);
+        WaveRow<T, NI, Wide, G> r;
+        r.load(xs, C, at.sub);
         const float mx = r.max();
         float s = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int l = 0; l < L; ++l) s += fast_exp(r.v[i][l] - mx);      // -inf beyond the row
-        s = group_reduce<64>(s, OpSum());
-        if (lane == 0) {
-            const float x_y = load_one(xs + lb);
-            scores[row] = fminf(fast_exp(x_y - mx) / s, 1.f);
-            if (ce) ce[row] = logf(s) + (mx - x_y);
+        s = group_reduce<G>(s, OpSum());
+        if (at.sub == 0 && live) {
+            const float x_y = load_one(xs + (no_target ? 0 : lb));
+            scores[row] = no_target ? 1.f : fminf(fast_exp(x_y - mx) / s, 1.f);
+            if (ce) ce[row] = no_target ? 0.f : logf(s) + (mx - x_y);
         }
     }
 }
@@ -520,10 +525,9 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #undef PLH_CASE
             }
         } else if (shape == Shape::Wave && C <= kWaveRowCap) {
-            const unsigned grid = group_grid(P, 4);
-#define PLH_GO(NI, W)                                                                                               \
-    hipLaunchKernelGGL((ohem_scores_wrow<T, NI, W>), dim3(grid), dim3(256), 0, st, x, labels, scores, ce, P, C,     \
-                       ignore_index, tables)
+#define PLH_GO(NI, W, G)                                                                                            \
+    hipLaunchKernelGGL((ohem_scores_wrow<T, NI, W, G>), dim3(group_grid(P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
+                       st, x, labels, scores, ce, P, C, ignore_index, tables)
             PLH_WROW_DISPATCH(x, (const T *)nullptr, C, PLH_GO);
 #undef PLH_GO
         } else {

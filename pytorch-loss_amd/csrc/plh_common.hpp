@@ -778,7 +778,7 @@ __device__ __forceinline__ float bpermute_xor32(float v) {
 struct OpSum { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
-// Reduce over groups of G consecutive lanes (G = 1, 16 or 64).
+// Reduce over groups of G consecutive lanes (G = 1, 16, 32 or 64).
 template <int G, class Op>
 __device__ __forceinline__ float group_reduce(float v, Op op) {
     if constexpr (G >= 16) {
@@ -787,10 +787,8 @@ __device__ __forceinline__ float group_reduce(float v, Op op) {
         v = op(v, dpp_move<0x141>(v));   // row_half_mirror
         v = op(v, dpp_move<0x140>(v));   // row_mirror
     }
-    if constexpr (G >= 64) {
-        v = op(v, swizzle_xor16(v));
-        v = op(v, bpermute_xor32(v));
-    }
+    if constexpr (G >= 32) v = op(v, swizzle_xor16(v));
+    if constexpr (G >= 64) v = op(v, bpermute_xor32(v));
     return v;
 }
 
@@ -846,18 +844,20 @@ template <class T> struct RowChunk {             // T = f16 or bf16
     }
 };
 
-// ---- a wavefront holds one row of an (N, C) input in registers ----------------------------
-// NI steps of 64 lanes, 16 bytes per lane and step where the rows allow it, else one element: the row is
-// read once and every load of it is in flight before the first one is used.
-template <class T, int NI, bool Wide>
+// ---- a wavefront holds rows of an (N, C) input in registers --------------------------------
+// G lanes share a row (G = 64: one row per wavefront; G = 16: four short rows per wavefront, so that a
+// wavefront still has a few KB in flight), NI steps of G lanes, 16 bytes per lane and step where the rows
+// allow it, else one element: a row is read once and every load of it is in flight before the first one
+// is used.
+template <class T, int NI, bool Wide, int G = 64>
 struct WaveRow {
     static constexpr int L = Wide ? RowChunk<T>::kLen : 1;
     float v[NI][L];
-    // elements beyond the row read as -inf (and are never stored)
-    __device__ __forceinline__ void load(const T *xs, int C, int lane) {
+    // `sub` = lane within the row's group; elements beyond the row read as -inf (and are never stored)
+    __device__ __forceinline__ void load(const T *xs, int C, int sub) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int e0 = (lane + 64 * i) * L;
+            const int e0 = (sub + G * i) * L;
             const bool ok = e0 < C;                   // rows moved in chunks hold a whole number of them
             const T *at = xs + (ok ? e0 : 0);
             if constexpr (Wide) RowChunk<T>::load(at, v[i]);
@@ -872,44 +872,78 @@ struct WaveRow {
         for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int l = 0; l < L; ++l) m = fmaxf(m, v[i][l]);
-        return group_reduce<64>(m, OpMax());
+        return group_reduce<G>(m, OpMax());
     }
 };
 
-// Steps a wavefront needs for a row of C elements (the instantiated sizes: 2, 4 or 8 steps of 16-byte
-// chunks -- 8 only for fp32, whose chunks hold 4 elements -- and 2 .. 32 steps of single elements), and
-// whether its rows can be moved in 16-byte chunks (every row then starts on a 16-byte boundary).
+// The rows a wavefront works on in one round of a kernel's loop: 64 / G of them, consecutive; a group
+// past the last row repeats the last row and stores nothing.
+template <int G>
+struct WaveRowAt {
+    static constexpr int kRowsPerWave = 64 / G;
+    static constexpr int kRowsPerBlock = 4 * kRowsPerWave;          // 256-thread blocks
+    int sub, grp;               // lane within its row's group, group within the wavefront
+    int64_t start, stride;      // wave-uniform: first row of the wavefront's first round, rows per round of the grid
+    __device__ __forceinline__ WaveRowAt() {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        sub = lane % G;
+        grp = lane / G;
+        start = ((int64_t)blockIdx.x * 4 + wave) * kRowsPerWave;
+        stride = (int64_t)gridDim.x * kRowsPerBlock;
+    }
+};
+
+// Lanes per row and steps for a row of C elements. Rows of up to 256 elements get 16 lanes (at most 16
+// elements per lane); longer ones a whole wavefront. Instantiated sizes -- 16 lanes: 2 or 4 steps of
+// 16-byte chunks (4 only for fp32, whose chunks hold 4 elements), 4, 8 or 16 steps of single elements;
+// 64 lanes: 2, 4 or 8 steps of chunks (8 only for fp32), 8, 16 or 32 steps of single elements. Rows can be
+// moved in 16-byte chunks when every row starts on a 16-byte boundary.
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
+constexpr int kWaveRowShort = 256;
 
 template <class T>
 static bool wrow_wide(const T *x, const T *grad, int C) {
     return C % RowChunk<T>::kLen == 0 && !misaligned(x, 16) && !(grad && misaligned(grad, 16));
 }
 template <class T>
-static int wrow_steps(int C, bool wide) {
-    const int per = 64 * (wide ? RowChunk<T>::kLen : 1);
+static int wrow_steps(int C, bool wide, int lanes) {
+    const int per = lanes * (wide ? RowChunk<T>::kLen : 1);
     const int need = (C + per - 1) / per;
-    int steps = 2;
+    int steps = wide ? 2 : (lanes == 16 ? 4 : 8);      // the smallest instantiated size of each kind
     while (steps < need) steps *= 2;
     return steps;
 }
-#define PLH_WROW_DISPATCH_WIDE(WIDE, C, LAUNCH)                              \
-    do {                                                                     \
-        const bool wrow_is_wide = (WIDE);                                    \
-        switch (wrow_steps<T>(C, wrow_is_wide)) {                            \
-            case 2: if (wrow_is_wide) LAUNCH(2, true); else LAUNCH(2, false); break; \
-            case 4: if (wrow_is_wide) LAUNCH(4, true); else LAUNCH(4, false); break; \
-            case 8:                                                          \
-                if constexpr (RowChunk<T>::kLen == 4) {                      \
-                    if (wrow_is_wide) { LAUNCH(8, true); break; }            \
-                }                                                            \
-                LAUNCH(8, false);                                            \
-                break;                                                       \
-            case 16: LAUNCH(16, false); break;                               \
-            default: LAUNCH(32, false); break;                               \
-        }                                                                    \
+// LAUNCH(NI, Wide, G) launches the kernel instance; its grid is group_grid(rows, WaveRowAt<G>::kRowsPerBlock).
+#define PLH_WROW_DISPATCH_WIDE(WIDE, C, LAUNCH)                                          \
+    do {                                                                                 \
+        const bool wrow_is_wide = (WIDE);                                                \
+        if ((C) <= kWaveRowShort) {                                                      \
+            switch (wrow_steps<T>(C, wrow_is_wide, 16)) {                                \
+                case 2: LAUNCH(2, true, 16); break;              /* chunks only */      \
+                case 4:                                                                  \
+                    if constexpr (RowChunk<T>::kLen == 4) {                              \
+                        if (wrow_is_wide) { LAUNCH(4, true, 16); break; }                \
+                    }                                                                    \
+                    LAUNCH(4, false, 16);   /* 16-bit chunks never need 4 steps here */  \
+                    break;                                                               \
+                case 8: LAUNCH(8, false, 16); break;                                     \
+                default: LAUNCH(16, false, 16); break;                                   \
+            }                                                                            \
+        } else {                                                                         \
+            switch (wrow_steps<T>(C, wrow_is_wide, 64)) {                                \
+                case 2: LAUNCH(2, true, 64); break;              /* chunks only */      \
+                case 4: LAUNCH(4, true, 64); break;              /* chunks only */      \
+                case 8:                                                                  \
+                    if constexpr (RowChunk<T>::kLen == 4) {                              \
+                        if (wrow_is_wide) { LAUNCH(8, true, 64); break; }                \
+                    }                                                                    \
+                    LAUNCH(8, false, 64);   /* 16-bit chunks never need 8 steps */       \
+                    break;                                                               \
+                case 16: LAUNCH(16, false, 64); break;                                   \
+                default: LAUNCH(32, false, 64); break;                                   \
+            }                                                                            \
+        }                                                                                \
     } while (0)
 #define PLH_WROW_DISPATCH(X, GRAD, C, LAUNCH) PLH_WROW_DISPATCH_WIDE(wrow_wide<T>(X, GRAD, C), C, LAUNCH)
-
 
 }  // namespace plh

@@ -471,25 +471,28 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
 // upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
 // taylor_group<64>.
 
-template <class T, int NI, bool Wide, int Kind, bool Reduce>
+template <class T, int NI, bool Wide, int Kind, bool Reduce, int G>
 __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
                                                    const int64_t *__restrict__ lab, const Upstream up,
                                                    T *__restrict__ out, float *__restrict__ loss, Partials part,
                                                    const TaylorParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide>::L;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    const WaveRowAt<G> at;
+    const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
-    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.P; row += (int64_t)gridDim.x * 4) {   // wave-uniform
+    for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
+        const bool live = r0 + at.grp < p.P;
+        const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide> r;
+        WaveRow<T, NI, Wide, G> r;
         r.load(xs, p.C, lane);
-        WaveRow<T, (Kind == kTaylorBwd) ? NI : 1, Wide> rg;
+        WaveRow<T, (Kind == kTaylorBwd) ? NI : 1, Wide, G> rg;
         if constexpr (Kind == kTaylorBwd) rg.load(g + row * p.C, p.C, lane);
         float s = 0.f, dot = 0.f;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const bool ok = (lane + 64 * i) * L < p.C;          // elements beyond the row hold -inf
+            const bool ok = (lane + G * i) * L < p.C;           // elements beyond the row hold -inf
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 float f, df;
@@ -501,11 +504,11 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 }
             }
         }
-        s = group_reduce<64>(s, OpSum());
-        if constexpr (Kind == kTaylorBwd) dot = group_reduce<64>(dot, OpSum());
+        s = group_reduce<G>(s, OpSum());
+        if constexpr (Kind == kTaylorBwd) dot = group_reduce<G>(dot, OpSum());
         const float inv = 1.f / s;
         if constexpr (Kind == kTaylorCeFwd) {
-            if (lane == 0) {
+            if (lane == 0 && live) {
                 const int64_t lb = lab[row];
                 const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
                 float f_y = 1.f, df;
@@ -531,7 +534,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
             }
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
-                const int e0 = (lane + 64 * i) * L;
+                const int e0 = (lane + G * i) * L;
                 float o[L];
 #pragma unroll
                 for (int l = 0; l < L; ++l) {
@@ -546,10 +549,10 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                         o[l] = (tgt >= 0) ? df * inv * gk - ((e0 + l == tgt) ? df / f * gk : 0.f) : 0.f;
                     }
                 }
-                if (e0 < p.C) {
-                    T *at = out + row * p.C + e0;
-                    if constexpr (Wide) RowChunk<T>::store(at, o);
-                    else store_one(at, o[0]);
+                if (e0 < p.C && live) {
+                    T *dst = out + row * p.C + e0;
+                    if constexpr (Wide) RowChunk<T>::store(dst, o);
+                    else store_one(dst, o[0]);
                 }
             }
         }
@@ -625,17 +628,21 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         return grid;
     }
     if (p.m_size == 1) {
-        const unsigned grid = group_grid(p.P, 4);
         if (p.C <= kWaveRowCap) {
+            unsigned grid = 0;
             const bool wide = wrow_wide<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C) &&
                               !(Kind == kTaylorBwd && misaligned(g, 16));
-#define PLH_GO(NI, W)                                                                                             \
-    hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss, \
-                       part, p)
+#define PLH_GO(NI, W, G)                                                                                          \
+    do {                                                                                                          \
+        grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                      \
+        hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
+                           loss, part, p);                                                                        \
+    } while (0)
             PLH_WROW_DISPATCH_WIDE(wide, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
         }
+        const unsigned grid = group_grid(p.P, 4);
         hipLaunchKernelGGL((taylor_group<T, 64, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss,
                            part, p);
         return grid;

@@ -36,6 +36,9 @@ SCORE_CASES = [
     ((9, 77), -100, 0.1),                #   (odd lengths element by element, others in 16-byte chunks)
     ((6, 1000), 255, 0.2),
     ((7, 201), 255, 0.1),
+    ((70, 33), -100, 0.1),
+    ((21, 136), 255, 0.1),
+    ((5, 260), 255, 0.2),
     ((4, 1001), -100, 0.1),
     ((5, 1544), 255, 0.1),
     ((3, 2047), 255, 0.1),

@@ -75,6 +75,10 @@ SEG_CASES = [
     ((9, 77), -100, 0.1),                           # ... rows of 33..2048 channels sit in a wavefront's registers:
     ((6, 501), 255, 0.2),                           #   2 .. 32 steps, element by element for odd lengths,
     ((7, 201), 255, 0.1),
+    ((70, 33), -100, 0.1),                          #   rows of up to 256 channels: four rows per wavefront,
+    ((21, 136), 255, 0.1),                          #   the last wavefront partly filled
+    ((3, 256), 255, 0.0),
+    ((5, 260), 255, 0.2),
     ((4, 1001), -100, 0.1),
     ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
     ((2, 2048), 255, 0.0),

@@ -27,6 +27,9 @@ CASES = [
     ((6, 1000), 1),                              # longer register rows: 8 and 32 steps per wavefront
     ((3, 2047), -1),
     ((7, 201), 1),
+    ((70, 33), 1),
+    ((21, 136), 1),
+    ((5, 260), 1),
     ((4, 1001), 1),
     ((5, 1544), 1),
     ((2, 2056), 1),                              # beyond the register rows: strided sweeps
@@ -68,7 +71,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-6:-1])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-9:-1])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
