@@ -575,6 +575,145 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
     }
 }
 
+// ------------------------------------------------------- a block per row ----
+// (N, C) inputs with rows of more than 2048 channels: a 1024-thread block per row at a time. One sweep
+// with running statistics over the channels other than the target -- maximum, sum e, sum e*x (rescaled
+// when the maximum moves) and sum x -- gives the loss in closed form:
+//   sum_{j != y} (q_j - c) log q_j = (sum q_j x_j - m - lse) - c * (sum x_j - n * (m + lse)),  log q_j = x_j - m - lse;
+// the backward sweeps the row a second time (from cache for all but the longest rows) to write the gradient.
+
+struct LmRowStats { float m, s, ex, sx; };
+
+template <int L>
+__device__ __forceinline__ void lm_row_absorb(const float (&v)[L], int idx0, int tgt, LmRowStats &st) {
+    float cm = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < L; ++i) cm = (idx0 + i == tgt) ? cm : fmaxf(cm, v[i]);
+    if (cm > st.m) {
+        const float f = fast_exp(st.m - cm);           // 0 on the first chunk
+        st.s *= f;
+        st.ex *= f;
+        st.m = cm;
+    }
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+        const bool hot = (idx0 + i == tgt);
+        const float e = hot ? 0.f : fast_exp(v[i] - st.m);
+        st.s += e;
+        st.ex += hot ? 0.f : e * v[i];
+        st.sx += hot ? 0.f : v[i];
+    }
+}
+
+template <class T>
+__device__ __forceinline__ LmRowStats lm_row_sweep(const T *xs, int C, int tgt, bool aligned, float *lds) {
+    constexpr int L = RowChunk<T>::kLen;
+    const RowSplit<T> sp(xs, C, aligned);
+    LmRowStats st{-INFINITY, 0.f, 0.f, 0.f};
+    const T *body = xs + sp.head;
+    int i = threadIdx.x;
+    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
+        float v[4][L];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) lm_row_absorb<L>(v[u], sp.head + (i + u * kRowBlock) * L, tgt, st);
+    }
+    for (; i < sp.chunks; i += kRowBlock) {
+        float v[L];
+        RowChunk<T>::load(body + (int64_t)i * L, v);
+        lm_row_absorb<L>(v, sp.head + i * L, tgt, st);
+    }
+    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) {
+        const float v[1] = {load_one(xs + j)};
+        lm_row_absorb<1>(v, j, tgt, st);
+    }
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) {
+        const float v[1] = {load_one(xs + j)};
+        lm_row_absorb<1>(v, j, tgt, st);
+    }
+    LmRowStats r;
+    r.m = row_block_reduce(st.m, lds, OpMax());
+    const float f = (st.m == -INFINITY) ? 0.f : fast_exp(st.m - r.m);
+    r.s = row_block_reduce(st.s * f, lds, OpSum());
+    r.ex = row_block_reduce(st.ex * f, lds, OpSum());
+    r.sx = row_block_reduce(st.sx, lds, OpSum());
+    return r;
+}
+
+template <class T, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+__global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                    const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
+                                                    unsigned long long *__restrict__ valid_cnt, Partials part,
+                                                    const LmParams p, int vec) {
+    __shared__ float red[kRowBlock / 64];
+    constexpr int L = RowChunk<T>::kLen;
+    float mine = 0.f;
+    int cnt = 0;
+    unsigned long long n_valid = 0;
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {       // block-uniform
+        const T *xs = x + row * p.C;
+        const int64_t lb = lab[row];
+        const bool ign = (lb == p.ignore);
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        const LmRowStats st = lm_row_sweep<T>(xs, p.C, tgt, vec != 0, red);
+        const float x_y = (tgt >= 0) ? load_one(xs + tgt) : -INFINITY;
+        const float m_all = fmaxf(st.m, x_y);
+        const float t_all = fast_exp(st.m - m_all);
+        const float e_y = fast_exp(x_y - m_all);
+        const float s_all = st.s * t_all + e_y;
+        const float inv_no = 1.f / st.s, inv_all = 1.f / s_all;
+        const float sum_qx = st.ex * inv_no;
+        const float lse_no = logf(st.s);
+        if constexpr (WantLoss) {
+            if (threadIdx.x == 0) {
+                const float n_no = (float)(p.C - (tgt >= 0 ? 1 : 0));
+                const float off = st.m + lse_no;
+                const float margin = p.half_lam * ((sum_qx - off) - p.coeff * (st.sx - n_no * off));
+                const float acc = margin - (x_y - m_all) + logf(s_all);
+                if (loss) loss[row] = ign ? 0.f : acc;
+                if (p.scores) p.scores[row] = (ign || tgt < 0) ? 1.f : fminf(e_y * inv_all, 1.f);
+                mine += ign ? 0.f : acc;
+                cnt += ign ? 0 : 1;
+            }
+        }
+        if constexpr (WantCount) n_valid += (threadIdx.x == 0 && !ign) ? 1 : 0;
+        if constexpr (WantGrad) {
+            float go[1];
+            load_upstream<1>(up, row, go);
+            const float gk = ign ? 0.f : go[0];
+            const float g_hot = (e_y * inv_all - 1.f) * gk;
+            const float k_all = t_all * inv_all;
+            T *gs = grad + row * p.C;
+            auto one = [&](float xv, int j) {
+                const float e = fast_exp(xv - st.m);
+                const float q = e * inv_no;
+                const float g_cold = (e * k_all + p.half_lam * ((xv + 1.f - sum_qx) * q - p.coeff)) * gk;
+                return ign ? 0.f : ((j == tgt) ? g_hot : g_cold);
+            };
+            const RowSplit<T> sp(xs, p.C, vec != 0);     // the gradient row sits at the same offset from its own boundary
+            for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
+                float v[L];
+                RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
+#pragma unroll
+                for (int e = 0; e < L; ++e) v[e] = one(v[e], sp.head + i * L + e);
+                RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
+            }
+            for (int j = threadIdx.x; j < sp.head; j += kRowBlock) store_one(gs + j, one(load_one(xs + j), j));
+            for (int j = sp.tail_from + threadIdx.x; j < p.C; j += kRowBlock) store_one(gs + j, one(load_one(xs + j), j));
+        }
+    }
+    if constexpr (WantCount) {
+        if (threadIdx.x == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
+    }
+    if constexpr (Reduce) {
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = mine;
+            part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
 static __global__ void lm_zero_count(unsigned long long *cnt) { *cnt = 0; }
 
 // ------------------------------------------------------------ dispatch ----
@@ -650,9 +789,9 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
 #undef PLH_GO
                 break;
             }
-            blocks = group_grid(p.P, 4);
-            hipLaunchKernelGGL((lm_group<T, 64, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
-                               x, lab, up, loss, grad, cnt, part, p);
+            blocks = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(kRowBlock), 0, st,
+                               x, lab, up, loss, grad, cnt, part, p, row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C));
             break;
         case Shape::Lane:
             blocks = group_grid(p.P, 256);

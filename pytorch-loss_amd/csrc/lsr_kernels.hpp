@@ -536,96 +536,6 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
 // that is rescaled when the maximum moves, so the forward reads the row once; the backward reads it a
 // second time (from cache for all but the longest rows) to write the gradient.
 
-constexpr int kRowBlock = 1024;      // few, large blocks: the rows in flight stay within the last-level cache
-                                     // for the backward's second sweep
-struct RowStats { float m, s, sx; };
-
-// Block-wide reductions for kRowBlock threads; every thread gets the result. lds: kRowBlock / 64 floats.
-template <class Op>
-__device__ __forceinline__ float row_block_reduce(float v, float *lds, Op op) {
-    v = group_reduce<64>(v, op);
-    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float r = lds[0];
-#pragma unroll
-    for (int w = 1; w < kRowBlock / 64; ++w) r = op(r, lds[w]);
-    __syncthreads();
-    return r;
-}
-
-template <int L>
-__device__ __forceinline__ void row_absorb(const float (&v)[L], RowStats &st) {
-    float cm = v[0];
-#pragma unroll
-    for (int i = 1; i < L; ++i) cm = fmaxf(cm, v[i]);
-    if (cm > st.m) {
-        st.s *= fast_exp(st.m - cm);               // 0 * exp(-inf) on the first chunk
-        st.m = cm;
-    }
-#pragma unroll
-    for (int i = 0; i < L; ++i) {
-        st.s += fast_exp(v[i] - st.m);
-        st.sx += v[i];
-    }
-}
-
-// How a row splits into 16-byte chunks: `head` leading elements up to the first 16-byte boundary,
-// `chunks` chunks, then the rest. Rows of any length qualify as long as the tensor itself starts on a
-// 16-byte boundary (`aligned`); otherwise the whole row is the head.
-template <class T>
-struct RowSplit {
-    int head, chunks, tail_from;
-    __device__ __forceinline__ RowSplit(const T *xs, int C, bool aligned) {
-        constexpr int L = RowChunk<T>::kLen;
-        const int mis = (int)((reinterpret_cast<uintptr_t>(xs) / sizeof(T)) % L);
-        const int lead = (L - mis) % L;
-        head = aligned ? (lead < C ? lead : C) : C;
-        chunks = (C - head) / L;
-        tail_from = head + chunks * L;
-    }
-};
-
-template <class T>
-__device__ __forceinline__ RowStats row_sweep(const T *xs, int C, bool aligned) {
-    constexpr int L = RowChunk<T>::kLen;
-    const RowSplit<T> sp(xs, C, aligned);
-    RowStats st{-INFINITY, 0.f, 0.f};
-    const T *body = xs + sp.head;
-    int i = threadIdx.x;
-    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
-        float v[4][L];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) row_absorb<L>(v[u], st);
-    }
-    for (; i < sp.chunks; i += kRowBlock) {
-        float v[L];
-        RowChunk<T>::load(body + (int64_t)i * L, v);
-        row_absorb<L>(v, st);
-    }
-    // head and tail, element by element (the whole row when it cannot be moved in chunks)
-    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) {
-        const float v[1] = {load_one(xs + j)};
-        row_absorb<1>(v, st);
-    }
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) {
-        const float v[1] = {load_one(xs + j)};
-        row_absorb<1>(v, st);
-    }
-    return st;
-}
-
-// Block-wide (M, S [, sum x]) from the per-lane running values.
-__device__ __forceinline__ RowStats row_combine(RowStats st, float *lds, bool want_sx) {
-    RowStats r;
-    r.m = row_block_reduce(st.m, lds, OpMax());
-    const float mine = (st.m == -INFINITY) ? 0.f : st.s * fast_exp(st.m - r.m);
-    r.s = row_block_reduce(mine, lds, OpSum());
-    r.sx = want_sx ? row_block_reduce(st.sx, lds, OpSum()) : 0.f;
-    return r;
-}
-
 template <class T, bool Reduce>
 __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                    float *__restrict__ loss, Partials part, const LsrParams p, int vec) {
@@ -781,13 +691,6 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
         PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
 #undef PLH_CASE
     }
-}
-
-// Rows are moved in 16-byte chunks when the tensors start on 16-byte boundaries (a row of the gradient
-// then sits at the same offset from a boundary as the row of logits it belongs to).
-template <class T>
-static int row_chunks_ok(const T *x, const T *grad, int C) {
-    return (!misaligned(x, 16) && !(grad && misaligned(grad, 16))) ? 1 : 0;
 }
 
 // Launches the forward; returns the number of blocks that wrote partials.

@@ -209,6 +209,35 @@ __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x,
     }
 }
 
+// (N, C) inputs with longer rows (a vocabulary): a 1024-thread block per row at a time, the row read once
+// with running (maximum, exponential sum) statistics per lane.
+template <class T>
+__global__ __launch_bounds__(kRowBlock) void ohem_scores_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                             float *__restrict__ scores, float *__restrict__ ce,
+                                                             int64_t P, int C, int64_t ignore,
+                                                             uint32_t *__restrict__ tables, int vec) {
+    __shared__ float red[kRowBlock / 64];
+    if (tables && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kOhemZeroWords; i += kRowBlock) tables[i] = 0;
+    for (int64_t row = blockIdx.x; row < P; row += gridDim.x) {       // block-uniform
+        const int64_t lb = lab[row];
+        if (lb == ignore || lb < 0 || lb >= C) {
+            if (threadIdx.x == 0) {
+                scores[row] = 1.f;
+                if (ce) ce[row] = 0.f;
+            }
+            continue;
+        }
+        const T *xs = x + row * C;
+        const RowStats st = row_combine(row_sweep<T>(xs, C, vec != 0), red, false);
+        if (threadIdx.x == 0) {
+            const float x_y = load_one(xs + lb);
+            scores[row] = fminf(fast_exp(x_y - st.m) / st.s, 1.f);
+            if (ce) ce[row] = logf(st.s) + (st.m - x_y);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ select ----
 
 // Tables of the selection, all in the caller's workspace. `state` (16 words, zeroed with the
@@ -530,6 +559,10 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
                        st, x, labels, scores, ce, P, C, ignore_index, tables)
             PLH_WROW_DISPATCH(x, (const T *)nullptr, C, PLH_GO);
 #undef PLH_GO
+        } else if (shape == Shape::Wave) {
+            const unsigned grid = (unsigned)(P < 1 ? 1 : (P < kMinPartialSlots ? P : kMinPartialSlots));
+            hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(kRowBlock), 0, st, x, labels, scores, ce, P, C,
+                               ignore_index, tables, row_chunks_ok<T>(x, nullptr, C));
         } else {
             hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,
                                m_size, C, ignore_index, tables);

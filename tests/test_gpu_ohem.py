@@ -42,7 +42,10 @@ SCORE_CASES = [
     ((4, 1001), -100, 0.1),
     ((5, 1544), 255, 0.1),
     ((3, 2047), 255, 0.1),
-    ((2, 2056), 255, 0.0),               # longer rows: lane per pixel
+    ((2, 2056), 255, 0.0),               # longer rows: a block per row, 16-byte chunks
+    ((3, 4100), 255, 0.3),
+    ((2, 4099), -100, 0.0),              #   odd length: element by element
+    ((2, 50000), 255, 0.0),
     ((2, 33, 6, 7), 255, 0.2),
     ((2, 40, 16, 16), 255, 0.1),         # 33..256 channels: shared out over the wavefronts of a block
     ((1, 150, 12, 16), 255, 0.05),
