@@ -1029,6 +1029,49 @@ __device__ __forceinline__ RowStats row_sweep(const T *xs, int C, bool aligned) 
     return st;
 }
 
+// Calls fn(value, index) for this thread's share of a row: chunks of 16 bytes, four loads in flight,
+// then the head and tail element by element.
+template <class T, class Fn>
+__device__ __forceinline__ void row_visit(const T *xs, int C, bool aligned, Fn fn) {
+    constexpr int L = RowChunk<T>::kLen;
+    const RowSplit<T> sp(xs, C, aligned);
+    const T *body = xs + sp.head;
+    int i = threadIdx.x;
+    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
+        float v[4][L];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < L; ++e) fn(v[u][e], sp.head + (i + u * kRowBlock) * L + e);
+    }
+    for (; i < sp.chunks; i += kRowBlock) {
+        float v[L];
+        RowChunk<T>::load(body + (int64_t)i * L, v);
+#pragma unroll
+        for (int e = 0; e < L; ++e) fn(v[e], sp.head + i * L + e);
+    }
+    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) fn(load_one(xs + j), j);
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) fn(load_one(xs + j), j);
+}
+
+// Writes fn(value, index) over a row of `out` that sits at the same offset from a 16-byte boundary as `xs`.
+template <class T, class Fn>
+__device__ __forceinline__ void row_map(const T *xs, T *out, int C, bool aligned, Fn fn) {
+    constexpr int L = RowChunk<T>::kLen;
+    const RowSplit<T> sp(xs, C, aligned);
+    for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
+        float v[L];
+        RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
+#pragma unroll
+        for (int e = 0; e < L; ++e) v[e] = fn(v[e], sp.head + i * L + e);
+        RowChunk<T>::store(out + sp.head + (int64_t)i * L, v);
+    }
+    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) store_one(out + j, fn(load_one(xs + j), j));
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) store_one(out + j, fn(load_one(xs + j), j));
+}
+
 // Block-wide (M, S [, sum x]) from the per-lane running values.
 __device__ __forceinline__ RowStats row_combine(RowStats st, float *lds, bool want_sx) {
     RowStats r;

@@ -567,6 +567,61 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
     }
 }
 
+// ------------------------------------------------------- a block per row ----
+// Taylor cross entropy on (N, C) inputs with rows of more than 2048 channels: a 1024-thread block per row
+// at a time, 16-byte chunks, four loads in flight; the backward sweeps the row a second time (from cache
+// for all but the longest rows) to write the gradient.
+
+template <class T, int Kind, bool Reduce>
+__global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                           const Upstream up, T *__restrict__ out,
+                                                           float *__restrict__ loss, Partials part,
+                                                           const TaylorParams p, int vec) {
+    static_assert(Kind == kTaylorCeFwd || Kind == kTaylorCeBwd, "cross entropy only");
+    __shared__ float red[kRowBlock / 64];
+    float mine = 0.f;
+    int cnt = 0;
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {       // block-uniform
+        const T *xs = x + row * p.C;
+        const int64_t lb = lab[row];
+        const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
+        float s = 0.f;
+        row_visit<T>(xs, p.C, vec != 0, [&](float v, int) {
+            float f, df;
+            taylor_pair(v, p.order, f, df);
+            s += f;
+        });
+        s = row_block_reduce(s, red, OpSum());
+        if constexpr (Kind == kTaylorCeFwd) {
+            if (threadIdx.x == 0) {
+                float f_y = 1.f, df;
+                if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df);
+                const float v = has_y ? logf(s) - logf(f_y) : 0.f;
+                if (loss) loss[row] = v;
+                mine += v;
+                cnt += (lb != p.ignore) ? 1 : 0;
+            }
+        } else {
+            float go[1];
+            load_upstream<1>(up, row, go);
+            const float gk = has_y ? go[0] : 0.f;
+            const float inv = 1.f / s;
+            const int tgt = has_y ? (int)lb : -1;
+            row_map<T>(xs, out + row * p.C, p.C, vec != 0, [&](float v, int j) {
+                float f, df;
+                taylor_pair(v, p.order, f, df);
+                return has_y ? df * inv * gk - ((j == tgt) ? df / f * gk : 0.f) : 0.f;
+            });
+        }
+    }
+    if constexpr (Reduce) {
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = mine;
+            part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
 // ------------------------------------------------------------ dispatch ----
 
 template <class T, int Kind, bool Reduce>
@@ -640,6 +695,12 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     } while (0)
             PLH_WROW_DISPATCH_WIDE(wide, p.C, PLH_GO);
 #undef PLH_GO
+            return grid;
+        }
+        if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
+            const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(kRowBlock), 0, st, x, lab, up, out, loss,
+                               part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
             return grid;
         }
         const unsigned grid = group_grid(p.P, 4);
