@@ -362,8 +362,8 @@ __global__ __launch_bounds__(kSplitBlock) void lm_bwd_split(const T *__restrict_
 }
 
 // --------------------------------------------------------------- group ----
-
-constexpr int kLmStageCap = 2048;
+// G lanes per pixel, striding over its channels; three sweeps, the later ones re-reading what the first
+// pulled into cache. Launched with G = 1: a lane per pixel, for channel counts no other shape takes.
 
 template <class T, int G, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const int64_t *__restrict__ lab,
@@ -372,13 +372,10 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
                                                 unsigned long long *__restrict__ valid_cnt, Partials part,
                                                 const LmParams p) {
     constexpr int kPix = 256 / G;
-    __shared__ float stage_mem[(G == 64) ? 4 * kLmStageCap : 1];
     __shared__ float red[4];
     float mine = 0.f, cnt = 0.f;
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
-    float *stage = stage_mem + ((G == 64) ? grp * kLmStageCap : 0);
-    const bool staged = (G == 64) && (p.C <= kLmStageCap);
 
     unsigned long long n_valid = 0;
     const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
@@ -398,7 +395,6 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
-            if (staged) stage[j] = t;
             if (lb == j) x_y = t; else m_no = fmaxf(m_no, t);
         }
         m_no = group_reduce<G>(m_no, OpMax());
@@ -407,7 +403,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         float s_no = 0.f, sum_ex = 0.f;
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
-            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float t = load_one(xs + (int64_t)j * p.m_size);
             const float e = (lb == j) ? 0.f : fast_exp(t - m_no);
             s_no += e;
             sum_ex += e * t;
@@ -423,7 +419,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
         float acc = 0.f;
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
-            const float xv = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float xv = load_one(xs + (int64_t)j * p.m_size);
             const bool hot = (lb == j);
             const float e = fast_exp(xv - m_no);
             const float q = e * inv_no;
@@ -463,7 +459,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 
 // ------------------------------------------------- wavefront per row, in registers ----
 // (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
-// sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group<64>.
+// sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group.
 
 template <class T, int NI, bool Wide, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G>
 __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,

@@ -308,11 +308,8 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_bwd_split(const T *__restrict
 }
 
 // --------------------------------------------------------------- group ----
-// G lanes per pixel. G = 64 stages the wave's slice in LDS (each lane re-reads
-// only what it wrote, so no barrier is needed); G = 1 re-reads global memory,
-// which the preceding pass has just pulled into cache.
-
-constexpr int kStageCap = 2048;   // floats per wave -> 32 KiB of LDS per 256-thread block
+// G lanes per pixel, striding over its channels and re-reading global memory in each sweep (the
+// preceding sweep has just pulled the slice into cache). Launched with G = 1: a lane per pixel.
 
 template <class T, int G, bool Reduce>
 __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
@@ -320,12 +317,9 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
                                                      float *__restrict__ loss, Partials part,
                                                      const LsrParams p) {
     constexpr int kPix = 256 / G;
-    __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
     __shared__ float red[4];
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
-    float *stage = stage_mem + ((G == 64) ? grp * kStageCap : 0);
-    const bool staged = (G == 64) && (p.C <= kStageCap);
 
     float mine = 0.f, cnt = 0.f;
     // every lane of a group walks the same pixels, so the loop is group-uniform
@@ -342,14 +336,13 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
-            if (staged) stage[j] = t;
             mx = fmaxf(mx, t);
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
-            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float t = load_one(xs + (int64_t)j * p.m_size);
             s += fast_exp(t - mx);
         }
         s = group_reduce<G>(s, OpSum());
@@ -357,7 +350,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         float acc = 0.f;
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
-            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float t = load_one(xs + (int64_t)j * p.m_size);
             acc -= ((t - mx) - lse) * ((lb == j) ? p.w_pos : p.w_neg);
         }
         acc = group_reduce<G>(acc, OpSum());
@@ -384,11 +377,8 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
                                                      const Upstream up, T *__restrict__ grad,
                                                      const LsrParams p) {
     constexpr int kPix = 256 / G;
-    __shared__ float stage_mem[(G == 64) ? 4 * kStageCap : 1];
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
-    float *stage = stage_mem + ((G == 64) ? grp * kStageCap : 0);
-    const bool staged = (G == 64) && (p.C <= kStageCap);
 
     const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
     for (int64_t r = 0; r < rounds; ++r) {
@@ -407,16 +397,14 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
             const float t = load_one(xs + (int64_t)j * p.m_size);
-            if (staged) stage[j] = t;
             mx = fmaxf(mx, t);
         }
         mx = group_reduce<G>(mx, OpMax());
         float s = 0.f;
 #pragma unroll kGroupUnroll<G>
         for (int j = sub; j < p.C; j += G) {
-            const float t = staged ? stage[j] : load_one(xs + (int64_t)j * p.m_size);
+            const float t = load_one(xs + (int64_t)j * p.m_size);
             const float e = fast_exp(t - mx);
-            if (staged) stage[j] = e;
             s += e;
         }
         s = group_reduce<G>(s, OpSum());
@@ -425,7 +413,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
             const float scale = p.sumw * gk / s;
 #pragma unroll kGroupUnroll<G>
             for (int j = sub; j < p.C; j += G) {
-                const float e = staged ? stage[j] : fast_exp(load_one(xs + (int64_t)j * p.m_size) - mx);
+                const float e = fast_exp(load_one(xs + (int64_t)j * p.m_size) - mx);
                 store_one(gs + (int64_t)j * p.m_size, e * scale - ((lb == j) ? p.w_pos : p.w_neg) * gk);
             }
         }
@@ -703,7 +691,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
-            if (p.C > kStageCap) {
+            if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
                 hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
@@ -740,7 +728,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
-            if (p.C > kStageCap) {
+            if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
                 hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, up, grad_logits, p,
                                    row_chunks_ok<T>(logits, grad_logits, p.C));
