@@ -183,13 +183,14 @@ def test_ohem_refuses_cpu_tensors():
 
 @pytest.mark.parametrize("which", ["ce", "lm"])
 @pytest.mark.parametrize("case", ["n_min_covers_everything", "all_ignored", "huge_logit_gaps", "ragged", "deep",
-                                  "split", "rows"])
+                                  "split", "rows", "register_rows", "short_register_rows", "block_rows"])
 def test_ohem_ce_fused_forward_edge_cases(native, case, which):
     """The one-pass forwards (scores and per-pixel loss from the same sums) against the oracle's
     relabelling followed by torch's cross entropy or the oracle's large-margin loss."""
     import pytorch_loss as pl
     # deep: more channels than the register-resident form holds; rows: (N, C) inputs
-    shape = {"ragged": (2, 7, 9, 11), "deep": (2, 40, 6, 10), "split": (2, 150, 8, 16), "rows": (300, 23)}.get(
+    shape = {"ragged": (2, 7, 9, 11), "deep": (2, 40, 6, 10), "split": (2, 150, 8, 16), "rows": (300, 23),
+             "register_rows": (90, 1000), "short_register_rows": (203, 150), "block_rows": (40, 2500)}.get(
         case, (2, 19, 16, 24))
     x, y = seg_inputs(91, shape, 255, 0.05)
     n_min, thresh = y.size // 16, 0.3
