@@ -761,7 +761,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
         else                                                                                                          \
             hipLaunchKernelGGL((lm_bwd_split<T, KW, V>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
         break;
-                    PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+                    PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
                 }
             }

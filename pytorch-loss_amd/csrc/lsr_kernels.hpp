@@ -661,7 +661,7 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
         hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
                            part, p);                                                                              \
         break;
-        PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+        PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
     }
     return grid;
@@ -676,7 +676,7 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     case KW:                                                                                                      \
         hipLaunchKernelGGL((lsr_bwd_split<T, KW, V>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
         break;
-        PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+        PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
     }
 }

@@ -532,7 +532,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         hipLaunchKernelGGL((ohem_scores_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, ce, \
                            P, m_size, C, ignore_index, run, tables);                                                  \
         break;
-                PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+                PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
             }
         } else if (shape == Shape::RegsVec || shape == Shape::RegsOne) {

@@ -645,7 +645,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
             hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
                                p);                                                                                    \
         break;
-                PLH_CASE(8) PLH_CASE(12) PLH_CASE(16) PLH_CASE(20) PLH_CASE(24) PLH_CASE(28) PLH_CASE(32)
+                PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
             }
             return grid;

@@ -50,6 +50,10 @@ SCORE_CASES = [
     ((2, 40, 16, 16), 255, 0.1),         # 33..256 channels: shared out over the wavefronts of a block
     ((1, 150, 12, 16), 255, 0.05),
     ((2, 256, 8, 8), 255, 0.1),
+    ((2, 52, 8, 8), 255, 0.1),
+    ((2, 65, 8, 8), 255, 0.1),
+    ((1, 133, 8, 8), 255, 0.1),
+    ((1, 171, 8, 8), 255, 0.1),
     ((2, 19, 16, 16), 255, 1.0),         # everything ignored
 ]
 

@@ -95,6 +95,13 @@ SEG_CASES = [
     ((3, 100, 10, 10), 255, 0.1),                   #   slots per wavefront 8 .. 32, last wavefronts partly or
     ((1, 150, 12, 16), 255, 0.05),                  #   wholly empty, pixel counts that leave lanes idle
     ((2, 256, 8, 8), 255, 0.1),
+    ((2, 52, 8, 8), 255, 0.1),                      #   more channel counts of real label sets: the last
+    ((2, 65, 8, 8), 255, 0.1),                      #   wavefront that holds channels holds 1 .. all of its slots
+    ((1, 73, 8, 16), -100, 0.1),
+    ((1, 112, 8, 8), 255, 0.1),
+    ((1, 133, 8, 8), 255, 0.1),
+    ((1, 171, 8, 8), 255, 0.1),
+    ((1, 200, 8, 8), 255, 0.1),
     ((2, 257, 8, 8), 255, 0.1),                     # one channel more: a lane per pixel again
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
