@@ -608,23 +608,23 @@ __device__ __forceinline__ LmRowStats lm_row_sweep(const T *xs, int C, int tgt, 
     LmRowStats st{-INFINITY, 0.f, 0.f, 0.f};
     const T *body = xs + sp.head;
     int i = threadIdx.x;
-    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
+    for (; i + 3 * row_threads() < sp.chunks; i += 4 * row_threads()) {
         float v[4][L];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * row_threads()) * L, v[u]);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) lm_row_absorb<L>(v[u], sp.head + (i + u * kRowBlock) * L, tgt, st);
+        for (int u = 0; u < 4; ++u) lm_row_absorb<L>(v[u], sp.head + (i + u * row_threads()) * L, tgt, st);
     }
-    for (; i < sp.chunks; i += kRowBlock) {
+    for (; i < sp.chunks; i += row_threads()) {
         float v[L];
         RowChunk<T>::load(body + (int64_t)i * L, v);
         lm_row_absorb<L>(v, sp.head + i * L, tgt, st);
     }
-    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) {
+    for (int j = threadIdx.x; j < sp.head; j += row_threads()) {
         const float v[1] = {load_one(xs + j)};
         lm_row_absorb<1>(v, j, tgt, st);
     }
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) {
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += row_threads()) {
         const float v[1] = {load_one(xs + j)};
         lm_row_absorb<1>(v, j, tgt, st);
     }
@@ -688,15 +688,15 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                 return ign ? 0.f : ((j == tgt) ? g_hot : g_cold);
             };
             const RowSplit<T> sp(xs, p.C, vec != 0);     // the gradient row sits at the same offset from its own boundary
-            for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
+            for (int i = threadIdx.x; i < sp.chunks; i += row_threads()) {
                 float v[L];
                 RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
 #pragma unroll
                 for (int e = 0; e < L; ++e) v[e] = one(v[e], sp.head + i * L + e);
                 RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
             }
-            for (int j = threadIdx.x; j < sp.head; j += kRowBlock) store_one(gs + j, one(load_one(xs + j), j));
-            for (int j = sp.tail_from + threadIdx.x; j < p.C; j += kRowBlock) store_one(gs + j, one(load_one(xs + j), j));
+            for (int j = threadIdx.x; j < sp.head; j += row_threads()) store_one(gs + j, one(load_one(xs + j), j));
+            for (int j = sp.tail_from + threadIdx.x; j < p.C; j += row_threads()) store_one(gs + j, one(load_one(xs + j), j));
         }
     }
     if constexpr (WantCount) {
@@ -786,7 +786,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
                 break;
             }
             blocks = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(kRowBlock), 0, st,
+            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(row_threads_for(p.C)), 0, st,
                                x, lab, up, loss, grad, cnt, part, p, row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C));
             break;
         case Shape::Lane:

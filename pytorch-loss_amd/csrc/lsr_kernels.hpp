@@ -573,7 +573,7 @@ __global__ __launch_bounds__(kRowBlock) void lsr_bwd_row(const T *__restrict__ x
         const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
         const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
         const RowSplit<T> sp(xs, p.C, vec != 0);         // the gradient row sits at the same offset from its own boundary
-        for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
+        for (int i = threadIdx.x; i < sp.chunks; i += row_threads()) {
             float v[L];
             RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
 #pragma unroll
@@ -581,9 +581,9 @@ __global__ __launch_bounds__(kRowBlock) void lsr_bwd_row(const T *__restrict__ x
                 v[e] = __builtin_fmaf(fast_exp(v[e] - st.m), scale, (sp.head + i * L + e == tgt) ? n_pos : n_neg);
             RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
         }
-        for (int j = threadIdx.x; j < sp.head; j += kRowBlock)
+        for (int j = threadIdx.x; j < sp.head; j += row_threads())
             store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
-        for (int j = sp.tail_from + threadIdx.x; j < p.C; j += kRowBlock)
+        for (int j = sp.tail_from + threadIdx.x; j < p.C; j += row_threads())
             store_one(gs + j, __builtin_fmaf(fast_exp(load_one(xs + j) - st.m), scale, (j == tgt) ? n_pos : n_neg));
     }
 }
@@ -693,7 +693,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::Wave: {
             if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, losses, part, p,
+                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
@@ -730,7 +730,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::Wave:
             if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(kRowBlock), 0, st, logits, labels, up, grad_logits, p,
+                hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, logits, labels, up, grad_logits, p,
                                    row_chunks_ok<T>(logits, grad_logits, p.C));
                 break;
             }

@@ -218,7 +218,7 @@ __global__ __launch_bounds__(kRowBlock) void ohem_scores_row(const T *__restrict
                                                              uint32_t *__restrict__ tables, int vec) {
     __shared__ float red[kRowBlock / 64];
     if (tables && blockIdx.x == 0)
-        for (int i = threadIdx.x; i < kOhemZeroWords; i += kRowBlock) tables[i] = 0;
+        for (int i = threadIdx.x; i < kOhemZeroWords; i += row_threads()) tables[i] = 0;
     for (int64_t row = blockIdx.x; row < P; row += gridDim.x) {       // block-uniform
         const int64_t lb = lab[row];
         if (lb == ignore || lb < 0 || lb >= C) {
@@ -561,7 +561,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #undef PLH_GO
         } else if (shape == Shape::Wave) {
             const unsigned grid = (unsigned)(P < 1 ? 1 : (P < kMinPartialSlots ? P : kMinPartialSlots));
-            hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(kRowBlock), 0, st, x, labels, scores, ce, P, C,
+            hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(row_threads_for(C)), 0, st, x, labels, scores, ce, P, C,
                                ignore_index, tables, row_chunks_ok<T>(x, nullptr, C));
         } else {
             hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,

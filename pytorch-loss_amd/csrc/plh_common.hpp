@@ -951,21 +951,25 @@ static int wrow_steps(int C, bool wide, int lanes) {
 #define PLH_WROW_DISPATCH(X, GRAD, C, LAUNCH) PLH_WROW_DISPATCH_WIDE(wrow_wide<T>(X, GRAD, C), C, LAUNCH)
 
 // ---- a block per row: rows longer than a wavefront's registers (a vocabulary) ------------------
-// One 1024-thread block per row at a time, 16-byte loads, four of them in flight per lane, and running
+// One block of 1024 (or, for shorter rows, 256) threads per row at a time, 16-byte loads, four of them in flight per lane, and running
 // per-lane statistics that are rescaled when the maximum moves, so a sweep reads the row once.
-constexpr int kRowBlock = 1024;      // few, large blocks: the rows in flight stay within the last-level cache
-                                     // for the backward's second sweep
+constexpr int kRowBlock = 1024;      // long rows: few, large blocks, so that the rows in flight stay within the
+                                     // last-level cache for the backward's second sweep
+constexpr int kRowBlockShort = 256;  // rows of up to kRowShortMax elements: more rows in flight, four chunks
+constexpr int kRowShortMax = 8192;   // per lane instead of one, a quarter of the wavefronts in every barrier
+inline int row_threads_for(int C) { return C <= kRowShortMax ? kRowBlockShort : kRowBlock; }
+__device__ __forceinline__ int row_threads() { return (int)blockDim.x; }      // either of the two
+
 struct RowStats { float m, s, sx; };
 
-// Block-wide reductions for kRowBlock threads; every thread gets the result. lds: kRowBlock / 64 floats.
+// Block-wide reductions over the block's threads; every thread gets the result. lds: kRowBlock / 64 floats.
 template <class Op>
 __device__ __forceinline__ float row_block_reduce(float v, float *lds, Op op) {
     v = group_reduce<64>(v, op);
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
     __syncthreads();
     float r = lds[0];
-#pragma unroll
-    for (int w = 1; w < kRowBlock / 64; ++w) r = op(r, lds[w]);
+    for (int w = 1; w < row_threads() / 64; ++w) r = op(r, lds[w]);
     __syncthreads();
     return r;
 }
@@ -1009,24 +1013,24 @@ __device__ __forceinline__ RowStats row_sweep(const T *xs, int C, bool aligned) 
     RowStats st{-INFINITY, 0.f, 0.f};
     const T *body = xs + sp.head;
     int i = threadIdx.x;
-    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
+    for (; i + 3 * row_threads() < sp.chunks; i += 4 * row_threads()) {
         float v[4][L];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * row_threads()) * L, v[u]);
 #pragma unroll
         for (int u = 0; u < 4; ++u) row_absorb<L>(v[u], st);
     }
-    for (; i < sp.chunks; i += kRowBlock) {
+    for (; i < sp.chunks; i += row_threads()) {
         float v[L];
         RowChunk<T>::load(body + (int64_t)i * L, v);
         row_absorb<L>(v, st);
     }
     // head and tail, element by element (the whole row when it cannot be moved in chunks)
-    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) {
+    for (int j = threadIdx.x; j < sp.head; j += row_threads()) {
         const float v[1] = {load_one(xs + j)};
         row_absorb<1>(v, st);
     }
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) {
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += row_threads()) {
         const float v[1] = {load_one(xs + j)};
         row_absorb<1>(v, st);
     }
@@ -1041,23 +1045,23 @@ __device__ __forceinline__ void row_visit(const T *xs, int C, bool aligned, Fn f
     const RowSplit<T> sp(xs, C, aligned);
     const T *body = xs + sp.head;
     int i = threadIdx.x;
-    for (; i + 3 * kRowBlock < sp.chunks; i += 4 * kRowBlock) {
+    for (; i + 3 * row_threads() < sp.chunks; i += 4 * row_threads()) {
         float v[4][L];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * kRowBlock) * L, v[u]);
+        for (int u = 0; u < 4; ++u) RowChunk<T>::load(body + (int64_t)(i + u * row_threads()) * L, v[u]);
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
-            for (int e = 0; e < L; ++e) fn(v[u][e], sp.head + (i + u * kRowBlock) * L + e);
+            for (int e = 0; e < L; ++e) fn(v[u][e], sp.head + (i + u * row_threads()) * L + e);
     }
-    for (; i < sp.chunks; i += kRowBlock) {
+    for (; i < sp.chunks; i += row_threads()) {
         float v[L];
         RowChunk<T>::load(body + (int64_t)i * L, v);
 #pragma unroll
         for (int e = 0; e < L; ++e) fn(v[e], sp.head + i * L + e);
     }
-    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) fn(load_one(xs + j), j);
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) fn(load_one(xs + j), j);
+    for (int j = threadIdx.x; j < sp.head; j += row_threads()) fn(load_one(xs + j), j);
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += row_threads()) fn(load_one(xs + j), j);
 }
 
 // Writes fn(value, index) over a row of `out` that sits at the same offset from a 16-byte boundary as `xs`.
@@ -1065,15 +1069,15 @@ template <class T, class Fn>
 __device__ __forceinline__ void row_map(const T *xs, T *out, int C, bool aligned, Fn fn) {
     constexpr int L = RowChunk<T>::kLen;
     const RowSplit<T> sp(xs, C, aligned);
-    for (int i = threadIdx.x; i < sp.chunks; i += kRowBlock) {
+    for (int i = threadIdx.x; i < sp.chunks; i += row_threads()) {
         float v[L];
         RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
 #pragma unroll
         for (int e = 0; e < L; ++e) v[e] = fn(v[e], sp.head + i * L + e);
         RowChunk<T>::store(out + sp.head + (int64_t)i * L, v);
     }
-    for (int j = threadIdx.x; j < sp.head; j += kRowBlock) store_one(out + j, fn(load_one(xs + j), j));
-    for (int j = sp.tail_from + threadIdx.x; j < C; j += kRowBlock) store_one(out + j, fn(load_one(xs + j), j));
+    for (int j = threadIdx.x; j < sp.head; j += row_threads()) store_one(out + j, fn(load_one(xs + j), j));
+    for (int j = sp.tail_from + threadIdx.x; j < C; j += row_threads()) store_one(out + j, fn(load_one(xs + j), j));
 }
 
 // Block-wide (M, S [, sum x]) from the per-lane running values.

@@ -699,7 +699,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         }
         if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
             const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(kRowBlock), 0, st, x, lab, up, out, loss,
+            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, x, lab, up, out, loss,
                                part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
             return grid;
         }
