@@ -192,6 +192,42 @@ def test_long_rows(pl):
     assert x.grad.sum(dim=1).abs().max().item() < 1e-4
 
 
+@pytest.mark.parametrize("op", ["lsr", "lmargin"])
+@pytest.mark.parametrize("shape", [(2_200_000, 1000), (14_500_000, 150)], ids=["wavefront_per_row", "16_lanes_per_row"])
+def test_register_rows(pl, op, shape):
+    """(N, C) rows that sit in a wavefront's registers, more than 2^31 elements in all."""
+    n, c = shape
+    assert n * c > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(33)
+    x = torch.empty(n, c, device="cuda")
+    step = 1 << 20
+    for i in range(0, n, step):
+        x[i:i + step] = 2 * torch.randn(min(step, n - i), c, device="cuda", generator=g)
+    y = torch.randint(0, c, (n,), device="cuda", generator=g)
+    y[torch.rand(n, device="cuda", generator=g) < 0.05] = IGN
+    x.requires_grad_()
+    if op == "lsr":
+        per = pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="none", ignore_index=IGN)(x, y)
+    else:
+        per = pl.LargeMarginSoftmaxV3(lam=0.3, reduction="none", ignore_index=IGN)(x, y)
+    gout = torch.rand(n, device="cuda") + 0.5
+    per.backward(gout)
+    mid = 2 ** 31 // c
+    rows = np.concatenate([np.arange(0, 70), np.arange(n - 70, n), np.arange(mid - 70, mid + 70),
+                           np.random.default_rng(5).integers(0, n, 1024)])
+    it = torch.from_numpy(rows).cuda()
+    xs, ys, gs = x.detach()[it].cpu().numpy(), y[it].cpu().numpy(), gout[it].cpu().numpy()
+    if op == "lsr":
+        want, want_g = oracle.lsr_forward(xs, ys, IGN, 0.1), oracle.lsr_backward(xs, ys, IGN, 0.1, gs)
+    else:
+        want, want_g = oracle.lmargin_forward(xs, ys, 0.3, IGN), oracle.lmargin_backward(xs, ys, 0.3, IGN, gs)
+    assert np.all(np.abs(per.detach()[it].cpu().numpy() - want) <= 1e-5 * np.abs(want) + 1e-6)
+    assert np.abs(x.grad[it].cpu().numpy() - want_g).max() <= 1e-5
+    # the gradient of a valid row sums to 0 for both losses, and ignored rows are exact zeros
+    assert x.grad.sum(dim=1).abs().max().item() < 1e-4
+    assert (x.grad[y == IGN] == 0).all().item() and (per.detach()[y == IGN] == 0).all().item()
+
+
 def test_focal(pl):
     numel = 2 ** 31 + 12345
     g = torch.Generator(device="cuda").manual_seed(5)
