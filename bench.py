@@ -529,6 +529,12 @@ def main():
                                  "GB/s": round(r["gbps"], 1), "frac_of_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
                                  "kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
                                              for k, v in r["roofline"].items()}}
+                if other == "focal":
+                    others[other]["note"] = ("GB/s divides the Function-level algorithmic bytes (28E: unreduced losses "
+                                             "written, an upstream gradient read) by the module-level step, which moves "
+                                             "20E (reduced forward, scalar upstream) and partly runs from the 256 MB "
+                                             "last-level cache: the ratio to the HBM peak can exceed 1; the per-kernel "
+                                             "figures are the Function-level ones")
             except Exception as e:  # a secondary workload must not take the headline down
                 others[other] = {"error": "%s: %s" % (type(e).__name__, e)}
             torch.cuda.empty_cache()
