@@ -372,9 +372,8 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
 }
 
 // --------------------------------------------------------------- group ----
-// Any dimsize: G lanes share one slice and stride over it (G = 64: a wavefront per row when the
-// dimension is the contiguous one; G = 1: a lane per slice). The series is re-evaluated in each
-// sweep; re-reads hit cache.
+// Any dimsize: G lanes share one slice and stride over it (launched with G = 1: a lane per slice, for what
+// no other shape takes). The series is re-evaluated in each sweep; re-reads hit cache.
 
 enum TaylorKind { kTaylorFwd = 0, kTaylorBwd = 1, kTaylorCeFwd = 2, kTaylorCeBwd = 3 };
 
@@ -572,6 +571,65 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
 // at a time, 16-byte chunks, four loads in flight; the backward sweeps the row a second time (from cache
 // for all but the longest rows) to write the gradient.
 
+// Taylor softmax / log-softmax and their backward on such rows. The backward's first sweep walks the row
+// of logits and the row of upstream gradients together, element by element unless both can move in chunks.
+template <class T, int Kind>
+__global__ __launch_bounds__(kRowBlock) void taylor_sm_row(const T *__restrict__ x, const T *__restrict__ g,
+                                                           T *__restrict__ out, const TaylorParams p, int vec) {
+    static_assert(Kind == kTaylorFwd || Kind == kTaylorBwd, "softmax forms only");
+    __shared__ float red[kRowBlock / 64];
+    constexpr int L = RowChunk<T>::kLen;
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {       // block-uniform
+        const T *xs = x + row * p.C;
+        float s = 0.f, dot = 0.f;
+        if constexpr (Kind == kTaylorFwd) {
+            row_visit<T>(xs, p.C, vec != 0, [&](float v, int) {
+                float f, df;
+                taylor_pair(v, p.order, f, df);
+                s += f;
+            });
+        } else {
+            const T *gr = g + row * p.C;
+            const RowSplit<T> sp(xs, p.C, vec != 0);       // the row of g sits at the same offset from its boundary
+            auto term = [&](float v, float gj) {
+                float f, df;
+                taylor_pair(v, p.order, f, df);
+                s += f;
+                dot += p.use_log ? gj : f * gj;
+            };
+            for (int i = threadIdx.x; i < sp.chunks; i += row_threads()) {
+                float v[L], gv[L];
+                RowChunk<T>::load(xs + sp.head + (int64_t)i * L, v);
+                RowChunk<T>::load(gr + sp.head + (int64_t)i * L, gv);
+#pragma unroll
+                for (int e = 0; e < L; ++e) term(v[e], gv[e]);
+            }
+            for (int j = threadIdx.x; j < sp.head; j += row_threads()) term(load_one(xs + j), load_one(gr + j));
+            for (int j = sp.tail_from + threadIdx.x; j < p.C; j += row_threads()) term(load_one(xs + j), load_one(gr + j));
+            dot = row_block_reduce(dot, red, OpSum());
+        }
+        s = row_block_reduce(s, red, OpSum());
+        const float inv = 1.f / s;
+        if constexpr (Kind == kTaylorFwd) {
+            const float ls = logf(s);
+            row_map<T>(xs, out + row * p.C, p.C, vec != 0, [&](float v, int) {
+                float f, df;
+                taylor_pair(v, p.order, f, df);
+                return p.use_log ? logf(f) - ls : f * inv;
+            });
+        } else {
+            const float mid = p.use_log ? dot * inv : dot * inv * inv;
+            const T *gr = g + row * p.C;
+            row_map<T>(xs, out + row * p.C, p.C, vec != 0, [&](float v, int j) {
+                float f, df;
+                taylor_pair(v, p.order, f, df);
+                const float gj = load_one(gr + j);
+                return p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
+            });
+        }
+    }
+}
+
 template <class T, int Kind, bool Reduce>
 __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            const Upstream up, T *__restrict__ out,
@@ -697,15 +755,14 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
 #undef PLH_GO
             return grid;
         }
+        const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
         if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
-            const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
             hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, x, lab, up, out, loss,
                                part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
-            return grid;
+        } else {
+            const int vec = row_chunks_ok<T>(x, out, p.C) && !(Kind == kTaylorBwd && misaligned(g, 16));
+            hipLaunchKernelGGL((taylor_sm_row<T, Kind>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, x, g, out, p, vec);
         }
-        const unsigned grid = group_grid(p.P, 4);
-        hipLaunchKernelGGL((taylor_group<T, 64, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss,
-                           part, p);
         return grid;
     }
     const unsigned grid = group_grid(p.P, 256);

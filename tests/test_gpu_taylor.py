@@ -32,7 +32,9 @@ CASES = [
     ((5, 260), 1),
     ((4, 1001), 1),
     ((5, 1544), 1),
-    ((2, 2056), 1),                              # beyond the register rows: strided sweeps
+    ((2, 2056), 1),                              # beyond the register rows: a block per row
+    ((3, 4099), 1),                              #   odd length: element by element
+    ((2, 30000), -1),                            #   1024-thread blocks
 ]
 
 
@@ -71,7 +73,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-9:-1])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-11:])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
