@@ -468,7 +468,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
 // ------------------------------------------------- wavefront per row, in registers ----
 // (N, C) inputs along dim 1 with 33..2048 channels: the row (and, for the softmax backward, the row of
 // upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
-// taylor_group<64>.
+// the group kernel.
 
 template <class T, int NI, bool Wide, int Kind, bool Reduce, int G>
 __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
