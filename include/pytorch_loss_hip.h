@@ -12,7 +12,8 @@
  *     same way, csrc/lsr_kernel.cu:199-202); integer labels are int64 (n_size, m_size);
  *   - `stream` is a hipStream_t (NULL = the default stream); launches are
  *     asynchronous and the library never synchronises, allocates or frees
- *     device memory, and keeps no state between calls (re-entrant);
+ *     device memory, and keeps no state between calls (re-entrant; the one exception,
+ *     plh_lsr_forward_reduced_static, says so);
  *   - the caller sets the current device to the one that owns the pointers;
  *   - return value: PLH_OK (0), a negative PLH_ERR_* for rejected arguments
  *     (nothing was launched), or a positive hipError_t from the launch;
@@ -100,6 +101,21 @@ int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *la
                             void *grad_logits,
                             int64_t n_size, int64_t dimsize, int64_t m_size,
                             int64_t ignore_index, float smooth, void *stream);
+
+/* plh_lsr_forward_reduced for callers that cannot allocate device memory or bring a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference. Same arguments and results as plh_lsr_forward_reduced, without the
+ * workspace: the per-block partials live in a 1 MiB device array that is part of the library's
+ * code object (each GPU that the library runs on holds its own copy until the process ends); its
+ * address is looked up on the first call on each device. The call allocates and frees nothing.
+ * Limit: n_size * m_size <= 2^24 pixels, else PLH_ERR_BAD_SIZE. All calls on one GPU share the one
+ * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream
+ * are ordered and need no clearing in between.
+ */
+int plh_lsr_forward_reduced_static(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                                   float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                   int64_t n_size, int64_t dimsize, int64_t m_size,
+                                   int64_t ignore_index, float smooth, void *stream);
 
 /* ---- sigmoid focal loss -------------------------------------------------------
  * Replaces focal_cpp.focalloss_forward / focalloss_backward /

@@ -1,8 +1,39 @@
 // Label-smoothed softmax cross entropy for gfx950: the C entry points. The kernels live in
 // lsr_kernels.hpp and are compiled once per element type (lsr_f32.hip, lsr_f16.hip, lsr_bf16.hip).
+#include <mutex>
+
 #include "lsr_kernels.hpp"
 
 namespace plh {
+
+// Partials buffer of plh_lsr_forward_reduced_static: device memory that belongs to the loaded code
+// object (every GPU the library runs on holds its own copy at its own address until the process ends).
+// Host code never uses this name as an address; scratch_for_current_device() asks the runtime for it.
+constexpr int64_t kStaticMaxPixels = (int64_t)1 << 24;
+constexpr int64_t kStaticScratchBytes = 8 * (kStaticMaxPixels / 128);   // = 8 * partial_slots(kStaticMaxPixels) = 1 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+
+// The device address of `scratch` on the current device, looked up once per device.
+static int scratch_for_current_device(void **out) {
+    static std::mutex mu;
+    static void *ptrs[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return PLH_ERR_BAD_SIZE;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return PLH_ERR_WORKSPACE;
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return PLH_OK;
+}
 
 PLH_LSR_EXTERN(float)
 PLH_LSR_EXTERN(f16)
@@ -68,6 +99,24 @@ extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const 
     }
     finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
     return check_launch();
+}
+
+extern "C" int plh_lsr_forward_reduced_static(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                                              float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                              int64_t n_size, int64_t dimsize, int64_t m_size,
+                                              int64_t ignore_index, float smooth, void *stream) {
+    if (n_size < 0 || m_size < 0 || n_size > kStaticMaxPixels || m_size > kStaticMaxPixels ||
+        n_size * m_size > kStaticMaxPixels)
+        return PLH_ERR_BAD_SIZE;
+    static_assert(8 * ((kStaticMaxPixels + 127) / 128) <= kStaticScratchBytes && kStaticMaxPixels / 128 >= kMinPartialSlots,
+                  "the static buffer holds the partials of the largest accepted input");
+    void *ws = nullptr;
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != PLH_OK) return rc;
+    // Every partial that the finishing kernel reads was written by this call's forward kernel, so
+    // nothing has to be cleared between calls.
+    return plh_lsr_forward_reduced(logits, dtype, labels, losses, loss_out, n_valid_out, mean, ws, kStaticScratchBytes,
+                                   n_size, dimsize, m_size, ignore_index, smooth, stream);
 }
 
 extern "C" int plh_lsr_backward(const void *logits, int32_t dtype, const int64_t *labels,

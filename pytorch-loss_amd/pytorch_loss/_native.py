@@ -33,6 +33,7 @@ _SIGNATURES = {
     "plh_lsr_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lsr_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lsr_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_forward_reduced_static": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lsr_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_focal_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _f32, _f32, _p]),
     "plh_focal_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _f32, _f32, _p]),
