@@ -325,7 +325,8 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
 /* ---- soft dice loss ---------------------------------------------------------------------
  * Replaces soft_dice_cpp.soft_dice_forward / soft_dice_backward (csrc/soft_dice_kernel_v2.cu:258-436).
  * logits and labels are (batchsize, sample_size) tensors of one floating type (`dtype`); with
- * q = sigmoid(logits): numer = 2 sum(q y) + smooth, denor = sum(q^p + y^p) + smooth per row,
+ * q = sigmoid(logits): numer = 2 sum(q y) + smooth, denor = sum(q^p + y) + smooth per row
+ * (the label is not raised to p, csrc/soft_dice_kernel_v2.cu:90; equal to y^p for binary labels),
  * losses[n] = 1 - numer / denor (fp32).
  * forward also leaves (numer, denor) per row in stats (batchsize x 2 fp32), which the backward
  * reads instead of reducing the rows again; workspace: plh_soft_dice_workspace_bytes() bytes,

@@ -199,11 +199,12 @@ def taylor_ce(logits, labels, n=4, reduction="mean", ignore_index=-1):
 
 
 def soft_dice(logits, labels, p=1, smooth=1.0):
-    """Soft dice over everything as one row (pytorch_loss/soft_dice_loss.py:10-33):
-    1 - (2 sum(sigmoid(x) y) + smooth) / (sum(sigmoid(x)^p + y^p) + smooth)."""
+    """Soft dice over everything as one row (pytorch_loss/soft_dice_loss.py:10-33 with the denominator of the
+    fused kernel, csrc/soft_dice_kernel_v2.cu:90, where the label is not raised to p):
+    1 - (2 sum(sigmoid(x) y) + smooth) / (sum(sigmoid(x)^p + y) + smooth)."""
     probs = torch.sigmoid(logits)
     numer = 2 * (probs * labels).sum() + smooth
-    denor = (probs.pow(p) + labels.pow(p)).sum() + smooth
+    denor = (probs.pow(p) + labels).sum() + smooth
     return 1.0 - numer / denor
 
 

@@ -4,16 +4,19 @@
 //   "regs"  : up to 32 channels. Lanes run along consecutive pixels, each thread owns V
 //             pixels and keeps the whole channel slice in VGPRs. Each per-channel load of
 //             a wavefront is one contiguous 64*V*4-byte run, logits are read from HBM
-//             exactly once and no cross-lane traffic is needed.
+//             exactly once and no cross-lane traffic is needed. (N, C) inputs with C <= 32
+//             take the same kernels; a wavefront moves its 64 rows through a private LDS tile.
 //   "split" : 33..256 channels in NCHW. The regs shape with the slice of a pixel shared out
 //             over the 8 wavefronts of a block; per-wavefront statistics meet in LDS.
-//   "row"   : (N, C) rows longer than an LDS staging buffer (label smoothing only): a block
-//             per row, 16-byte chunks, running maximum and sum.
-//   "group" : everything else. G lanes share one pixel and stride over its channels (G = 64:
-//             a wavefront per row, for (N, C) inputs where the channel dim is the contiguous
-//             one; G = 1: a lane per pixel for deep channel dims in NCHW). Reductions inside
-//             a group use DPP/swizzle, the slice is staged in LDS when it has to be read
-//             more than once.
+//   "wrow"  : (N, C) rows of 33..2048 elements held in the registers of the 64 (or 16) lanes
+//             that share a row; every sweep after the first runs on registers.
+//   "row"   : (N, C) rows longer than that (every loss, the OHEM scores and the Taylor ops): a
+//             block per row, 16-byte chunks, running statistics that are rescaled when the
+//             maximum moves, a second sweep from cache where a gradient is written.
+//   "group" : everything else. G = 64: a wavefront per row striding over its channels (layer norm
+//             on long rows); G = 1: a lane per pixel for more than 256 channels in NCHW, channel
+//             loop through the caches. Reductions inside a group use DPP/swizzle; nothing is
+//             staged in LDS.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -985,9 +988,12 @@ __device__ __forceinline__ void row_absorb(const float (&v)[L], RowStats &st) {
         st.s *= fast_exp(st.m - cm);               // 0 * exp(-inf) on the first chunk
         st.m = cm;
     }
+    // while everything seen so far is -inf (masked vocabulary entries) the terms are exp(-inf - 0) = 0,
+    // not exp(-inf + inf) = NaN
+    const float ref = (st.m == -INFINITY) ? 0.f : st.m;
 #pragma unroll
     for (int i = 0; i < L; ++i) {
-        st.s += fast_exp(v[i] - st.m);
+        st.s += fast_exp(v[i] - ref);
         st.sx += v[i];
     }
 }

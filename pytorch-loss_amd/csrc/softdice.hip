@@ -1,6 +1,8 @@
 // Soft dice loss for binary segmentation on gfx950 (csrc/soft_dice_kernel_v2.cu:54-407).
 // Per row n of (batchsize, sample_size) logits x and float labels y, with q = sigmoid(x):
-//   numer = 2 sum(q y) + smooth,  denor = sum(q^p + y^p) + smooth,  loss_n = 1 - numer / denor
+//   numer = 2 sum(q y) + smooth,  denor = sum(q^p + y) + smooth,  loss_n = 1 - numer / denor
+// The label enters the denominator as it is, not raised to p (:86-91); the pure-torch V1/V2 classes use y^p
+// (pytorch_loss/soft_dice_loss.py:35, :84), which is the same number for the binary labels the loss is meant for.
 //   dloss_n/dx = p q^p (1 - q) numer / denor^2 - 2 y q (1 - q) / denor        (:236-247)
 // Forward is a two-stage fixed-order reduction (per-block partial sums, then one block per row that
 // adds them in double), so results do not depend on scheduling. It leaves (numer, denor) per row in
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(kDiceBlock) void dice_partial(const T *__restrict__
                 const bool in = Vec || (i + h * step + k < L);
                 const float q = sigmoid_fast(xv[h][k]);
                 a += in ? q * yv[h][k] : 0.f;
-                d += in ? dice_pow(q, p, mode) + dice_pow(yv[h][k], p, mode) : 0.f;
+                d += in ? dice_pow(q, p, mode) + yv[h][k] : 0.f;
             }
         }
     }

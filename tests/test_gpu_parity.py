@@ -500,3 +500,36 @@ def test_runs_on_a_side_stream(pl):
         out = pl.LSRCrossEntropyFunctionV3.apply(xt, yt, 0.1, 255)
     side.synchronize()
     close_loss(out.cpu().numpy(), oracle.lsr_forward(x, y, 255, 0.1), "side stream")
+
+
+@pytest.mark.parametrize("n_cls,masked", [(5000, 4200), (40000, 33000), (3001, 1500)])
+def test_rows_with_masked_vocabulary_entries_stay_finite(pl, n_cls, masked):
+    """(N, C) rows of more than 2048 logits whose leading entries are -inf (a masked vocabulary): whole
+    16-byte chunks of -inf reach a lane before its first finite value. Cross entropy (smoothing 0), its
+    gradient and the OHEM scores stay finite and match the oracle, as for the shorter row shapes (the
+    smoothed loss itself is 0 * inf = NaN there in the reference's arithmetic too)."""
+    from pytorch_loss import _native
+    x = synth.normal(77, 1, (6, n_cls), 0.0, 2.0)
+    x[:, :masked] = -np.inf
+    x[1, masked:masked + 7] = -np.inf
+    y = synth.randint(77, 11, (6,), masked + 7, n_cls)
+    y[4] = 255
+    xt, yt = dev(x), dev(y)
+    # OhemCELoss with a threshold nothing exceeds: the mean cross entropy of the valid rows
+    xr = xt.clone().requires_grad_()
+    loss = pl.OhemCELoss(score_thresh=2.0, n_min=1, ignore_index=255)(xr, yt)
+    x64 = x.astype(np.float64)
+    keep = y != 255
+    mx = x64.max(axis=1)
+    lse = np.log(np.exp(x64 - mx[:, None]).sum(axis=1)) + mx
+    want = (lse - x64[np.arange(6), np.where(keep, y, 0)])[keep].mean()
+    close_loss(loss.item(), want, "masked rows, OhemCELoss")
+    loss.backward()
+    assert torch.isfinite(xr.grad).all()
+    close_grad(xr.grad.cpu().numpy(), oracle.lsr_backward(x, y, 255, 0.0, np.float32(1.0 / keep.sum())), "masked rows, OhemCELoss")
+    grad = _native.lsr_backward(xt, yt, 255, 0.0).cpu().numpy()
+    assert np.isfinite(grad).all() and np.all(grad[:, :masked] == 0)
+    close_grad(grad, oracle.lsr_backward(x, y, 255, 0.0), "masked rows")
+    scores = _native.ohem_scores(xt, yt, 255).cpu().numpy()
+    assert np.isfinite(scores).all()
+    np.testing.assert_allclose(scores, oracle.ohem_scores(x, y, 255), rtol=2e-5, atol=1e-7)

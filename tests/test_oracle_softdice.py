@@ -21,8 +21,26 @@ def _inputs(seed, n, length, soft=False):
 def _defining(xt, yt, p, smooth):
     q = torch.sigmoid(xt)
     numer = 2 * (q * yt).sum(dim=1) + smooth
-    denor = (q.pow(p) + yt.pow(p)).sum(dim=1) + smooth
+    denor = (q.pow(p) + yt).sum(dim=1) + smooth      # the label as it is (csrc/soft_dice_kernel_v2.cu:90)
     return 1.0 - numer / denor
+
+
+def test_binary_labels_agree_with_the_power_form():
+    """For labels in {0, 1} the fused kernel's q^p + y and the pure-torch classes' q^p + y^p
+    (pytorch_loss/soft_dice_loss.py:35) are the same number; for soft labels with p != 1 they are not,
+    and the oracle follows the kernel."""
+    x, y = _inputs(74, 2, 300)
+    q = 1 / (1 + np.exp(-x))
+    for p in (1, 2, 2.5):
+        want = 1 - (2 * (q * y).sum(1) + 1.0) / ((q ** p + y ** p).sum(1) + 1.0)
+        np.testing.assert_allclose(oracle.soft_dice_forward(x, y, p, 1.0)[0], want, rtol=1e-12)
+    xs, ys = _inputs(74, 2, 300, soft=True)
+    qs = 1 / (1 + np.exp(-xs))
+    kernel_form = 1 - (2 * (qs * ys).sum(1) + 1.0) / ((qs ** 2 + ys).sum(1) + 1.0)
+    power_form = 1 - (2 * (qs * ys).sum(1) + 1.0) / ((qs ** 2 + ys ** 2).sum(1) + 1.0)
+    got = oracle.soft_dice_forward(xs, ys, 2, 1.0)[0]
+    np.testing.assert_allclose(got, kernel_form, rtol=1e-12)
+    assert np.abs(got - power_form).min() > 1e-3
 
 
 @pytest.mark.parametrize("n,length", [(1, 1000), (4, 37), (3, 4096)])
