@@ -44,7 +44,8 @@ constexpr int kSortThreads = 512;
 constexpr int kSortItems = 8;
 constexpr int kSortTile = kSortThreads * kSortItems;   // 4096 keys per block
 constexpr int kSortWaves = kSortThreads / kWave;
-constexpr int kRadix = 256;
+constexpr int kRadixBits = 8;                    // widest digit of a pass
+constexpr int kRadix = 1 << kRadixBits;          // bins per (class, tile) table row set
 constexpr int kRankGroup = 2;     // rounds whose match masks are formed together (see lov_scatter)
 
 __device__ __forceinline__ uint32_t make_key(float prob, bool hot, bool ignored) {
@@ -69,6 +70,8 @@ __device__ __forceinline__ void publish_block_max(const uint32_t *block_max, uin
     for (int j = threadIdx.x; j < C; j += blockDim.x) row[j] = block_max[j];
 }
 
+// It also leaves, per class, the number of key bits the sort has to look at: keys that take part are
+// not above the limit, so the bits above the limit's highest set bit are zero in every one of them.
 __global__ __launch_bounds__(256) void lov_class_max(const uint32_t *__restrict__ block_table, int blocks, int C,
                                                      uint32_t *__restrict__ pos_max, uint32_t *__restrict__ cursors,
                                                      int regions) {
@@ -83,8 +86,11 @@ __global__ __launch_bounds__(256) void lov_class_max(const uint32_t *__restrict_
     if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-        pos_max[c] = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+        const uint32_t top = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+        pos_max[c] = top;
         pos_max[2 * C + c] = 0xFFFFFFFFu;       // all_min[c], for lov_absent_min
+        // key_bits[c]: a class without positives keeps a single key value, wherever it lies
+        pos_max[3 * C + c] = (top > 1u) ? (uint32_t)(32 - __builtin_clz(top - 1u)) : (top ? 1u : 30u);
     }
 }
 
@@ -199,7 +205,9 @@ struct SortArgs {
     const uint32_t *vals_in;     // nullptr in the first pass: payload = position
     uint32_t *keys_out;
     uint32_t *vals_out;
-    uint32_t *tile_hist;         // [C][kRadix][tiles]: keys per (digit, tile); row-scanned in place
+    const uint32_t *keys_alt;    // last pass only: where the rows of classes with two scatter passes are
+    const uint32_t *vals_alt;    //   (keys_alt, vals_alt); the others are in (keys_in, vals_in)
+    uint32_t *tile_hist;         // [C][kRadix][tiles_pad]: keys per (digit, tile); row-scanned in place
     uint32_t *digit_total;       // [C][kRadix]: keys per digit
     uint32_t *tile_hot;          // last pass only: the same two tables for the positives
     uint32_t *hot_total;
@@ -207,11 +215,33 @@ struct SortArgs {
     const uint32_t *all_min;     // first pass only: per class without positives, its smallest key
     const uint32_t *kept_in;     // later passes: keys per class that the first pass let through
     uint32_t *kept_out;          // first pass: where that count goes
+    const uint32_t *key_bits;    // per class: key bits that the sort has to look at (see DigitPlan)
     int P;                       // row stride; keys per class row in the first pass
     int tiles;                   // ceil(P / kSortTile)
-    int shift;                   // 0, 8, 16, 24
-    uint32_t digit_mask;         // 0xFF, or 0x7F for the top digit (bit 31 is the positive flag)
+    int tiles_pad;               // tiles rounded up to a multiple of kSortWaves: row length of the tile tables
+    int pass;                    // 0, 1, 2: scatter pass; the last (fused) pass of a class is passes - 1
 };
+
+// The digits of a class. Keys that take part in a class's sort are below 2^bits (bits from the
+// class's limit, lov_class_max), so the sort runs over `bits` bits only: in 2, 3 or 4 stable passes
+// of at most kRadixBits bits each, the first passes - 1 of them scatter passes and the last one
+// fused with the Jaccard step. The bits are shared out evenly: 27 bits (best positive's error
+// around 1e-4) are 7 + 7 + 7 + 6, whose runs per tile and digit are twice as long as those of
+// 8-bit digits; 24 bits or fewer (best error above 0.008) take three passes, 16 or fewer two.
+// Measured on the benchmark's rows with 9-bit digits (27 bits in three passes): a scatter pass
+// 104 us against 70 us, the three-pass forward no faster than the four-pass one.
+struct DigitPlan {
+    int passes, shift;
+    uint32_t mask;
+};
+__device__ __forceinline__ DigitPlan digit_plan(uint32_t bits, int pass) {
+    const int np = bits <= 2u * kRadixBits ? 2 : (bits <= 3u * kRadixBits ? 3 : 4);
+    const int base = (int)bits / np, rem = (int)bits % np;       // the first `rem` passes take one bit more
+    const int p = pass < 0 ? np - 1 : pass;
+    const int width = base + (p < rem ? 1 : 0);
+    return DigitPlan{np, p * base + min(p, rem), (1u << width) - 1u};
+}
+constexpr int kLastPass = -1;
 
 // A key takes part in the sort iff its error is not below that of the class's lowest-ranked positive
 // (error bits of the key <= limit). What is left out would be sorted after every positive, where
@@ -307,7 +337,7 @@ __device__ __forceinline__ void block_excl_scan2(uint32_t a, uint32_t b, uint32_
 __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
     uint32_t diff_lo = 0, diff_hi = 0;
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < kRadixBits; ++b) {
         uint32_t splat = (uint32_t)((int32_t)(digit << (31 - b)) >> 31);   // bit b splatted: 0 or ~0
         asm("" : "+v"(splat));      // the vote is taken from the splat itself: one field extract serves both
         const uint64_t vote = __builtin_amdgcn_ballot_w64(splat != 0u);
@@ -361,30 +391,48 @@ __device__ __forceinline__ void wave_rank(uint32_t digit, bool valid, bool hot, 
     wave_rank_of<Hot>(wave_peers(digit, valid), digit, valid, hot, counts, counts_hot, rank, hrank);
 }
 
-// Per-tile digit counts (and, for the last pass, the same for the positives). The lower digits are
-// close to uniform: LDS atomics on per-wave counters, and a round whose keys all share one digit is
-// added by a single lane. The top digit goes through match masks (see below).
-template <bool Hot>
+// Where the rows of class c are when its last pass starts: after an odd number of scatter passes in
+// (keys_in, vals_in), after two in (keys_alt, vals_alt); the other value buffer is free for staging.
+struct LastPassRows {
+    const uint32_t *keys, *vals;
+    uint32_t *stage;
+};
+__device__ __forceinline__ LastPassRows last_pass_rows(const SortArgs &a, int passes) {
+    const bool alt = (passes - 1) == 2;
+    return LastPassRows{alt ? a.keys_alt : a.keys_in, alt ? a.vals_alt : a.vals_in,
+                        const_cast<uint32_t *>(alt ? a.vals_in : a.vals_alt)};
+}
+
+// Per-tile digit counts (and, for the last pass, the same for the positives): a block per tile,
+// per-wave tables, all loads up front. The lower digits are spread evenly: LDS atomics per lane, and
+// a round whose keys all share one digit (a row of equal keys) is added by a single lane. The top
+// digit clusters (a handful of values per round with soft predictions, dozens of binades with
+// confident ones), so per-lane atomics would queue on a few addresses: the lowest lane of every
+// group of equal digits, found through the match mask, adds the group.
+template <bool Top>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
     __shared__ uint32_t counts[kSortWaves][kRadix];
-    __shared__ uint32_t counts_hot[Hot ? kSortWaves : 1][kRadix];
+    __shared__ uint32_t counts_hot[Top ? kSortWaves : 1][kRadix];
     const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
-        (&counts[0][0])[i] = 0;
-        if constexpr (Hot) (&counts_hot[0][0])[i] = 0;
-    }
+    const DigitPlan dp = digit_plan(a.key_bits[c], Top ? kLastPass : a.pass);
+    if (!Top && a.pass >= dp.passes - 1) return;        // block-uniform: this class has fewer scatter passes
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
-    if (count <= 0) {                           // block-uniform: the row ends before this tile
-        if (threadIdx.x < kRadix) {
-            a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile] = 0;
-            if constexpr (Hot) a.tile_hot[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile] = 0;
+    if (count <= 0) {                           // block-uniform: the row ends before this tile; lov_row_scan
+        if (threadIdx.x <= dp.mask) {           // reads the live tiles in whole groups of kSortWaves
+            a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile] = 0;
+            if constexpr (Top) a.tile_hot[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile] = 0;
         }
         return;
     }
+    for (int i = threadIdx.x; i < kSortWaves * kRadix; i += kSortThreads) {
+        (&counts[0][0])[i] = 0;
+        if constexpr (Top) (&counts_hot[0][0])[i] = 0;
+    }
     const uint32_t limit = keep_limit(a, c);
-    const uint32_t *kin = a.keys_in + (int64_t)c * a.P + begin;
+    const uint32_t *rows = Top ? last_pass_rows(a, dp.passes).keys : a.keys_in;
+    const uint32_t *kin = rows + (int64_t)c * a.P + begin;
     uint32_t key[kSortItems];
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {      // all loads in flight before the first one is used
@@ -396,53 +444,59 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         const bool valid = li < count && keep_key(key[r], limit);
-        const uint32_t digit = (key[r] >> a.shift) & a.digit_mask;
+        const uint32_t digit = (key[r] >> dp.shift) & dp.mask;
         const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
         if (vmask == 0) continue;               // wave-uniform
-        if constexpr (Hot) {
-            // top digit: errors cluster, so per-lane atomics would serialise on two or three addresses
-            // with soft predictions, while confident ones spread over dozens of binades. The match mask
-            // costs the same either way: the lowest lane of every group of equal digits adds the group.
-            const bool hot = valid && (key[r] >> 31);
+        if constexpr (Top) {
             const uint64_t peers = wave_peers(digit, valid);
-            const uint64_t hot_peers = peers & __builtin_amdgcn_ballot_w64(hot);
+            const uint64_t hot_peers = peers & __builtin_amdgcn_ballot_w64(valid && (key[r] >> 31));
             if (valid && peers_below(peers) == 0u) {
                 atomicAdd(&counts[wave][digit], (uint32_t)__builtin_popcountll(peers));
                 if (hot_peers) atomicAdd(&counts_hot[wave][digit], (uint32_t)__builtin_popcountll(hot_peers));
             }
             continue;
         }
-        const uint32_t first = __builtin_amdgcn_readfirstlane(digit);   // first active lane = lowest valid one here
-        const uint64_t same = __builtin_amdgcn_ballot_w64(valid && digit == first);
-        if (same == vmask) {                    // wave-uniform branch
-            if (lane == 0) atomicAdd(&counts[wave][first], (uint32_t)__builtin_popcountll(vmask));
+        const uint32_t value = (uint32_t)__builtin_amdgcn_readlane((int)digit, __builtin_ctzll(vmask));
+        if (__builtin_amdgcn_ballot_w64(valid && digit == value) == vmask) {        // wave-uniform
+            if (lane == 0) atomicAdd(&counts[wave][value], (uint32_t)__builtin_popcountll(vmask));
         } else if (valid) {
             atomicAdd(&counts[wave][digit], 1u);
         }
     }
     __syncthreads();
-    if (threadIdx.x < kRadix) {
+    if (threadIdx.x <= dp.mask) {
         const int d = threadIdx.x;
         uint32_t n = 0, nh = 0;
 #pragma unroll
         for (int w = 0; w < kSortWaves; ++w) {
             n += counts[w][d];
-            if constexpr (Hot) nh += counts_hot[w][d];
+            if constexpr (Top) nh += counts_hot[w][d];
         }
-        a.tile_hist[((int64_t)c * kRadix + d) * a.tiles + tile] = n;
-        if constexpr (Hot) a.tile_hot[((int64_t)c * kRadix + d) * a.tiles + tile] = nh;
+        a.tile_hist[((int64_t)c * kRadix + d) * a.tiles_pad + tile] = n;
+        if constexpr (Top) a.tile_hot[((int64_t)c * kRadix + d) * a.tiles_pad + tile] = nh;
     }
 }
 
-// One block per (digit, class) row of a tile table: exclusive scan over the tiles in place, row
-// total to totals[c][d]. blockIdx.z selects the table (keys / positives).
+// One block per (digit, class) row of a tile table: exclusive scan over the row's live tiles in
+// place, row total to totals[c][d]. blockIdx.z selects the table (keys / positives). pass as in
+// SortArgs (kLastPass for the fused pass); kept = nullptr in the first pass (every tile is live).
 __global__ __launch_bounds__(256) void lov_row_scan(uint32_t *table0, uint32_t *totals0, uint32_t *table1,
-                                                    uint32_t *totals1, int tiles) {
+                                                    uint32_t *totals1, int tiles_pad, const uint32_t *key_bits, int pass,
+                                                    const uint32_t *kept, int P) {
     __shared__ uint32_t wave_tot[4];
     uint32_t *table = blockIdx.z ? table1 : table0;
     uint32_t *totals = blockIdx.z ? totals1 : totals0;
-    const int64_t rid = (int64_t)blockIdx.y * kRadix + blockIdx.x;
-    uint32_t *row = table + rid * tiles;
+    const int c = blockIdx.y;
+    const DigitPlan dp = digit_plan(key_bits[c], pass);
+    if (pass >= 0 && pass >= dp.passes - 1) return;
+    const int64_t rid = (int64_t)c * kRadix + blockIdx.x;
+    if (blockIdx.x > dp.mask) {                     // no key has this digit; the tile table has no row for it
+        if (threadIdx.x == 0) totals[rid] = 0;
+        return;
+    }
+    const int items = kept ? (int)kept[c] : P;
+    const int tiles = ((items + kSortTile - 1) / kSortTile + kSortWaves - 1) / kSortWaves * kSortWaves;
+    uint32_t *row = table + rid * tiles_pad;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t carry = 0;
     for (int base = 0; base < tiles; base += 256) {
@@ -477,6 +531,8 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 
     const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const DigitPlan dp = digit_plan(a.key_bits[c], a.pass);
+    if (a.pass >= dp.passes - 1) return;        // block-uniform: this class has fewer scatter passes
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
     if (count <= 0) return;                     // block-uniform: the row ends before this tile
@@ -500,7 +556,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     uint32_t dtot = 0, tile_before = 0;         // thread d < kRadix: digit d's total in the row, and in the tiles before this one
     if (threadIdx.x < kRadix) {
         dtot = a.digit_total[(int64_t)c * kRadix + threadIdx.x];
-        tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles + tile];
+        if (threadIdx.x <= dp.mask) tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile];
     }
     for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
     __syncthreads();
@@ -517,7 +573,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
         for (int h = 0; h < kRankGroup; ++h) {
             const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
             valid[h] = li < count && keep_key(key[r + h], limit);
-            digit[h] = (key[r + h] >> a.shift) & a.digit_mask;
+            digit[h] = (key[r + h] >> dp.shift) & dp.mask;
         }
         bool any = false;
 #pragma unroll
@@ -566,7 +622,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     for (int r = 0; r < kSortItems; ++r) {
         const int li = wave * (kSortItems * kWave) + r * kWave + lane;
         if (li < count && keep_key(key[r], limit)) {
-            const uint32_t d = (key[r] >> a.shift) & a.digit_mask;
+            const uint32_t d = (key[r] >> dp.shift) & dp.mask;
             const uint32_t pos = digit_start[d] + counts[wave][d] + rank[r];
             s_keys[pos] = key[r];
             s_vals[pos] = val[r];
@@ -578,7 +634,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     uint32_t *vout = a.vals_out + row;
     for (int i = threadIdx.x; i < (int)n_local; i += kSortThreads) {
         const uint32_t k = s_keys[i];
-        const uint32_t d = (k >> a.shift) & a.digit_mask;
+        const uint32_t d = (k >> dp.shift) & dp.mask;
         const uint32_t dst = out_base[d] + (uint32_t)i;
         kout[dst] = k;
         vout[dst] = s_vals[i];
@@ -606,7 +662,6 @@ constexpr int kMaxRegions = 1024;             // per class row; larger rows take
 template <bool Binned>
 __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, float *__restrict__ jacc,
                                                           float *__restrict__ tile_loss,
-                                                          uint32_t *__restrict__ idx_stage,
                                                           uint32_t *__restrict__ cursors, int regions, int region_bits) {
     __shared__ uint32_t region_cnt[Binned ? kMaxRegions : 1];    // keys of this tile per region
     __shared__ uint16_t region_start[Binned ? kMaxRegions : 1];  // first position of the region in the re-ordered tile (< 4096)
@@ -628,9 +683,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         if (threadIdx.x == 0) tile_loss[(int64_t)c * a.tiles + tile] = 0.f;
         return;
     }
+    const DigitPlan dp = digit_plan(a.key_bits[c], kLastPass);
+    const LastPassRows in = last_pass_rows(a, dp.passes);
     const int64_t row = (int64_t)c * a.P;
-    const uint32_t *kin = a.keys_in + row + begin;
-    const uint32_t *vin = a.vals_in + row + begin;
+    const uint32_t *kin = in.keys + row + begin;
+    const uint32_t *vin = in.vals + row + begin;
+    uint32_t *idx_stage = in.stage;
 
     // every global read of the block is issued up front (the table entries are needed only after the ranking)
     uint32_t key[kSortItems], val[kSortItems], rank[kSortItems], hrank[kSortItems];
@@ -647,8 +705,10 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         const int64_t at = (int64_t)c * kRadix + threadIdx.x;
         dtot = a.digit_total[at];
         htot = a.hot_total[at];
-        tile_before = a.tile_hist[at * a.tiles + tile];
-        hot_before = a.tile_hot[at * a.tiles + tile];
+        if (threadIdx.x <= dp.mask) {
+            tile_before = a.tile_hist[at * a.tiles_pad + tile];
+            hot_before = a.tile_hot[at * a.tiles_pad + tile];
+        }
     }
     for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) {
         reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
@@ -663,12 +723,12 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 #pragma unroll
         for (int h = 0; h < kRankGroup; ++h) {
             const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
-            peers[h] = wave_peers((key[r + h] >> a.shift) & a.digit_mask, li < count);
+            peers[h] = wave_peers((key[r + h] >> dp.shift) & dp.mask, li < count);
         }
 #pragma unroll
         for (int h = 0; h < kRankGroup; ++h) {
             const int li = wave * (kSortItems * kWave) + (r + h) * kWave + lane;
-            wave_rank_of<true>(peers[h], (key[r + h] >> a.shift) & a.digit_mask, li < count, key[r + h] >> 31, counts[wave],
+            wave_rank_of<true>(peers[h], (key[r + h] >> dp.shift) & dp.mask, li < count, key[r + h] >> 31, counts[wave],
                                counts_hot[wave], rank[r + h], hrank[r + h]);
             if constexpr (Binned) {
                 // order inside a region's staging range is irrelevant: lov_unbin puts every value at its pixel
@@ -725,7 +785,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         if (li < count) {
             const uint32_t k = key[r];
             const uint32_t hot = k >> 31;
-            const uint32_t d = (k >> a.shift) & a.digit_mask;
+            const uint32_t d = (k >> dp.shift) & dp.mask;
             float dj = 0.f;
             if ((k & 0x7FFFFFFFu) != kIgnoredKey) {
                 const uint32_t pos = out_base[d] + counts[wave][d] + rank[r];            // rank in the descending order
@@ -771,13 +831,14 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
 constexpr int kUnbinThreads = 1024;
 
 template <int kRegionBits>
-__global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ jacc, const uint32_t *__restrict__ idx_stage,
+__global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ jacc, const SortArgs a,
                                                            const uint32_t *__restrict__ cursors, int regions, int P,
                                                            const float *__restrict__ tile_loss, float *__restrict__ losses,
                                                            int tiles) {
     typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
     constexpr int kRegion = 1 << kRegionBits;
     __shared__ __align__(16) float sorted[kRegion];
+    const uint32_t *idx_stage = last_pass_rows(a, digit_plan(a.key_bits[blockIdx.y], kLastPass).passes).stage;
     const int64_t first = (int64_t)blockIdx.y * P + ((int64_t)blockIdx.x << kRegionBits);
     const int n = min(kRegion, P - (int)(blockIdx.x << kRegionBits));
     const int staged = min(n, (int)cursors[(int64_t)blockIdx.y * regions + blockIdx.x]);
@@ -924,11 +985,11 @@ __global__ __launch_bounds__(256) void lov_bwd_lane(const float *__restrict__ go
 
 struct LovaszPlan {
     int64_t P, E;
-    int tiles;
+    int tiles, tiles_pad;
     int regions;            // pixel regions per class row (0 = direct scatter)
     int region_bits;        // log2 of the pixels per region
-    int64_t off_keys, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total, off_tile_loss,
-        off_cursors, off_class, off_block_max, bytes;
+    int64_t off_keys_a, off_keys_c, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total,
+        off_tile_loss, off_cursors, off_class, off_block_max, bytes;
 };
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -941,12 +1002,14 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.P = n_size * m_size;
     pl.E = pl.P * dimsize;
     pl.tiles = (int)ceil_div(pl.P, kSortTile);
+    pl.tiles_pad = (int)round_up(pl.tiles, kSortWaves);
     int64_t off = 0;
-    pl.off_keys = off;        off += round_up(4 * pl.E, 256);
+    pl.off_keys_a = off;      off += round_up(4 * pl.E, 256);
+    pl.off_keys_c = off;      off += round_up(4 * pl.E, 256);
     pl.off_vals_a = off;      off += round_up(4 * pl.E, 256);
     pl.off_vals_b = off;      off += round_up(4 * pl.E, 256);
-    pl.off_hist = off;        off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
-    pl.off_hot = off;         off += round_up(4 * dimsize * kRadix * pl.tiles, 256);
+    pl.off_hist = off;        off += round_up(4 * dimsize * kRadix * pl.tiles_pad, 256);
+    pl.off_hot = off;         off += round_up(4 * dimsize * kRadix * pl.tiles_pad, 256);
     pl.off_digit_total = off; off += round_up(4 * dimsize * kRadix, 256);
     pl.off_hot_total = off;   off += round_up(4 * dimsize * kRadix, 256);
     pl.off_tile_loss = off;   off += round_up(4 * dimsize * pl.tiles, 256);
@@ -956,7 +1019,7 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     const int64_t regions = ceil_div(pl.P, (int64_t)1 << pl.region_bits);
     pl.regions = (regions <= kMaxRegions) ? (int)regions : 0;
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
-    pl.off_class = off;       off += round_up(4 * dimsize * 3, 256);      // pos_max[C], kept[C], all_min[C]
+    pl.off_class = off;       off += round_up(4 * dimsize * 4, 256);      // pos_max[C], kept[C], all_min[C], key_bits[C]
     pl.off_block_max = off;   off += round_up(4 * dimsize * ceil_div(pl.P, 256), 256);   // [key blocks][C]
     pl.bytes = off;
     return PLH_OK;
@@ -988,8 +1051,9 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
 
     hipStream_t st = (hipStream_t)stream;
     char *ws = static_cast<char *>(workspace);
-    uint32_t *keys_a = reinterpret_cast<uint32_t *>(ws + pl.off_keys);
-    uint32_t *keys_b = reinterpret_cast<uint32_t *>(jacc);          // free until the Jaccard pass writes it
+    uint32_t *keys_0 = reinterpret_cast<uint32_t *>(jacc);          // the keys as built, in pixel order; jacc is free until the last pass
+    uint32_t *keys_a = reinterpret_cast<uint32_t *>(ws + pl.off_keys_a);
+    uint32_t *keys_c = reinterpret_cast<uint32_t *>(ws + pl.off_keys_c);
     uint32_t *vals_a = reinterpret_cast<uint32_t *>(ws + pl.off_vals_a);
     uint32_t *vals_b = reinterpret_cast<uint32_t *>(ws + pl.off_vals_b);
     uint32_t *hist = reinterpret_cast<uint32_t *>(ws + pl.off_hist);
@@ -1000,17 +1064,18 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     uint32_t *pos_max = reinterpret_cast<uint32_t *>(ws + pl.off_class);
     uint32_t *kept = pos_max + dimsize;
     uint32_t *all_min = pos_max + 2 * dimsize;
+    uint32_t *key_bits = pos_max + 3 * dimsize;
     const int C = (int)dimsize;
 
     uint32_t *block_table = reinterpret_cast<uint32_t *>(ws + pl.off_block_max);
     unsigned key_blocks = 0;
 
-    // 1. keys (into keys_b = jacc: rows of [C][P] u32; a row start stays 8-/16-byte aligned when P % V == 0)
+    // 1. keys (into keys_0 = jacc: rows of [C][P] u32; a row start stays 8-/16-byte aligned when P % V == 0)
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, keys_b, nullptr);
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, keys_0, nullptr);
         if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const unsigned grid = vec ? regs_grid<VT>(pl.P) : regs_grid<1>(pl.P);
@@ -1020,79 +1085,85 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
 #define PLH_CASE(K)                                                                                                 \
     case K:                                                                                                         \
         if (vec) hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, VT>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,  \
-                                    keys_b, block_table, pl.P, m_size, C, ignore_index, run);                       \
+                                    keys_0, block_table, pl.P, m_size, C, ignore_index, run);                       \
         else hipLaunchKernelGGL((lov_keys_regs<T, 4 * K, 1>), dim3(grid), dim3(kRegsBlock), 0, st, x, labels,       \
-                                keys_b, block_table, pl.P, m_size, C, ignore_index, run);                           \
+                                keys_0, block_table, pl.P, m_size, C, ignore_index, run);                           \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
         } else {
             key_blocks = group_grid(pl.P, 256);
-            hipLaunchKernelGGL(lov_keys_lane<T>, dim3(key_blocks), dim3(256), 0, st, x, labels, keys_b, block_table,
+            hipLaunchKernelGGL(lov_keys_lane<T>, dim3(key_blocks), dim3(256), 0, st, x, labels, keys_0, block_table,
                                pl.P, m_size, C, ignore_index);
         }
     });
     hipLaunchKernelGGL(lov_class_max, dim3((unsigned)C), dim3(256), 0, st, block_table, (int)key_blocks, C, pos_max,
                        reinterpret_cast<uint32_t *>(ws + pl.off_cursors), pl.regions);
-    hipLaunchKernelGGL(lov_absent_min, dim3(kAbsentBlocks, (unsigned)C), dim3(256), 0, st, keys_b, pos_max, all_min,
+    hipLaunchKernelGGL(lov_absent_min, dim3(kAbsentBlocks, (unsigned)C), dim3(256), 0, st, keys_0, pos_max, all_min,
                        (int)pl.P);
 
-    // 2. three stable radix passes: (keys_b, -) -> (keys_a, vals_a) -> (keys_b, vals_b) -> (keys_a, vals_a).
-    //    keys_b is the jacc output buffer, free until the last pass scatters into it. The first pass
-    //    drops the keys whose Jaccard difference is known to be 0 (keep_key) and counts what is left
-    //    per class; the later passes work on those counts and their surplus blocks return at once.
+    // 2. up to three stable scatter passes: (keys_0, -) -> (keys_a, vals_a) -> (keys_c, vals_b) -> (keys_a, vals_a);
+    //    how many a class takes follows from the width of its keys (DigitPlan), the blocks of a pass
+    //    that a class does not take return at once. The first pass drops the keys whose Jaccard
+    //    difference is known to be 0 (keep_key) and counts what is left per class; the later passes
+    //    work on those counts and their surplus blocks return at once.
     const dim3 tile_grid((unsigned)pl.tiles, (unsigned)C);
+    const dim3 hist_grid((unsigned)pl.tiles_pad, (unsigned)C);      // lov_row_scan reads the live tiles in whole groups of kSortWaves
     SortArgs a;
+    a.keys_alt = nullptr;
+    a.vals_alt = nullptr;
     a.tile_hist = hist;
     a.digit_total = digit_total;
     a.tile_hot = hot;
     a.hot_total = hot_total;
+    a.key_bits = key_bits;
     a.P = (int)pl.P;
     a.tiles = pl.tiles;
+    a.tiles_pad = pl.tiles_pad;
     for (int pass = 0; pass < 3; ++pass) {
-        const bool even = (pass % 2 == 0);
-        a.keys_in = even ? keys_b : keys_a;
-        a.vals_in = (pass == 0) ? nullptr : (even ? vals_b : vals_a);
-        a.keys_out = even ? keys_a : keys_b;
-        a.vals_out = even ? vals_a : vals_b;
-        a.shift = 8 * pass;
-        a.digit_mask = 0xFFu;
+        a.keys_in = pass == 0 ? keys_0 : (pass == 1 ? keys_a : keys_c);
+        a.vals_in = pass == 0 ? nullptr : (pass == 1 ? vals_a : vals_b);
+        a.keys_out = pass == 1 ? keys_c : keys_a;
+        a.vals_out = pass == 1 ? vals_b : vals_a;
+        a.pass = pass;
         a.pos_max = (pass == 0) ? pos_max : nullptr;
         a.all_min = (pass == 0) ? all_min : nullptr;
         a.kept_in = (pass == 0) ? nullptr : kept;
         a.kept_out = (pass == 0) ? kept : nullptr;
-        hipLaunchKernelGGL(lov_tile_hist<false>, tile_grid, dim3(kSortThreads), 0, st, a);
+        hipLaunchKernelGGL(lov_tile_hist<false>, hist_grid, dim3(kSortThreads), 0, st, a);
         hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 1), dim3(256), 0, st, hist, digit_total, hot,
-                           hot_total, pl.tiles);
+                           hot_total, pl.tiles_pad, key_bits, pass, a.kept_in, (int)pl.P);
         hipLaunchKernelGGL(lov_scatter, tile_grid, dim3(kSortThreads), 0, st, a);
     }
 
-    // 3. last pass (top digit; bit 31 masked out) fused with the Jaccard step: reads the sorted-so-far
-    //    rows from (keys_a, vals_a) and scatters the Jaccard differences into jacc
+    // 3. last pass (the top digit of the class; bit 31 is never part of a digit) fused with the Jaccard
+    //    step: reads the sorted-so-far rows and scatters the Jaccard differences into jacc
     a.keys_in = keys_a;
     a.vals_in = vals_a;
+    a.keys_alt = keys_c;
+    a.vals_alt = vals_b;
     a.keys_out = nullptr;
     a.vals_out = nullptr;
-    a.shift = 24;
-    a.digit_mask = 0x7Fu;
+    a.pass = kLastPass;
     a.pos_max = nullptr;
     a.all_min = nullptr;
     a.kept_in = kept;
     a.kept_out = nullptr;
-    hipLaunchKernelGGL(lov_tile_hist<true>, tile_grid, dim3(kSortThreads), 0, st, a);
+    hipLaunchKernelGGL(lov_tile_hist<true>, hist_grid, dim3(kSortThreads), 0, st, a);
     hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
-                       pl.tiles);
+                       pl.tiles_pad, key_bits, kLastPass, kept, (int)pl.P);
     if (pl.regions > 0) {
         uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);      // zeroed by lov_class_max
-        // vals_b is free by now: it receives the pixel offsets that go with the staged values
-        hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, vals_b, cursors,
+        // the value buffer that a class's last pass does not read receives the pixel offsets that go with
+        // the staged values
+        hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, cursors,
                            pl.regions, pl.region_bits);
         const dim3 unbin_grid((unsigned)pl.regions, (unsigned)C);
         switch (pl.region_bits) {
 #define PLH_UNBIN(B)                                                                                                  \
     case B:                                                                                                           \
-        hipLaunchKernelGGL(lov_unbin<B>, unbin_grid, dim3(kUnbinThreads), 0, st, jacc, vals_b, cursors, pl.regions,   \
+        hipLaunchKernelGGL(lov_unbin<B>, unbin_grid, dim3(kUnbinThreads), 0, st, jacc, a, cursors, pl.regions,        \
                            (int)pl.P, tile_loss, losses, pl.tiles);                                                   \
         break;
             PLH_UNBIN(13) PLH_UNBIN(14) PLH_UNBIN(15)
@@ -1100,10 +1171,9 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         }
     } else {
         // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
-        // (jacc stopped being a key buffer when the third pass read it)
+        // (jacc stopped being a key buffer when the first pass read it)
         hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, jacc, pl.E);
-        hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, nullptr,
-                           0, 0);
+        hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, 0, 0);
         hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     }
     return check_launch();
