@@ -225,13 +225,14 @@ struct SortArgs {
 // The digits of a class. Keys that take part in a class's sort are below 2^bits (bits from the
 // class's limit, lov_class_max), so the sort runs over `bits` bits only: in 2, 3 or 4 stable passes
 // of at most kRadixBits bits each, the first passes - 1 of them scatter passes and the last one
-// fused with the Jaccard step. The bits are shared out evenly: 27 bits (best positive's error
-// around 1e-4) are 7 + 7 + 7 + 6, whose runs per tile and digit are twice as long as those of
-// 8-bit digits; 24 bits or fewer (best error above 0.008) take three passes, 16 or fewer two.
-// Measured on the benchmark's rows with 9-bit digits (27 bits in three passes): a scatter pass
-// 104 us against 70 us, the three-pass forward no faster than the four-pass one.
+// fused with the Jaccard step (16 bits or fewer, i.e. a best positive's error above 0.99: two
+// passes; up to 24 bits, error above 0.008: three). The bits are shared out evenly: 27 bits (best
+// error around 1e-4) are 7 + 7 + 7 + 6. Measured on the benchmark's rows, forward in us: 7+7+7+6
+// 682, 7+8+8+4 684, 5+8+7+7 688, 8+8+8+6 (all 30 bits) 701, 9+9+9 735: a pass costs by the bit
+// (a scatter pass 70 us at 7 bits, 79 at 8, 104 at 9: the runs a tile writes per digit halve with
+// every bit), so what counts is the number of bits, not how they are cut.
 struct DigitPlan {
-    int passes, shift;
+    int passes, shift, width;
     uint32_t mask;
 };
 __device__ __forceinline__ DigitPlan digit_plan(uint32_t bits, int pass) {
@@ -239,7 +240,7 @@ __device__ __forceinline__ DigitPlan digit_plan(uint32_t bits, int pass) {
     const int base = (int)bits / np, rem = (int)bits % np;       // the first `rem` passes take one bit more
     const int p = pass < 0 ? np - 1 : pass;
     const int width = base + (p < rem ? 1 : 0);
-    return DigitPlan{np, p * base + min(p, rem), (1u << width) - 1u};
+    return DigitPlan{np, p * base + min(p, rem), width, (1u << width) - 1u};
 }
 constexpr int kLastPass = -1;
 
@@ -334,6 +335,22 @@ __device__ __forceinline__ void block_excl_scan2(uint32_t a, uint32_t b, uint32_
 // each lane ORs up, in two 32-bit halves, the lanes that differ from it in that bit
 // (vote XOR own bit splatted), so a bit costs one field extract, one compare, two XORs and its share
 // of two 3-input ORs.
+// The same with a number of digit bits that is known at run time only (wave-uniform), for the last
+// pass's histogram. (In lov_final the loop costs more than the ballots it leaves out: 138 us against 132.)
+__device__ __forceinline__ uint64_t wave_peers_n(uint32_t digit, bool valid, int bits) {
+    uint32_t diff_lo = 0, diff_hi = 0;
+#pragma unroll 1
+    for (int b = 0; b < bits; ++b) {
+        uint32_t splat = 0u - ((digit >> b) & 1u);
+        asm("" : "+v"(splat));
+        const uint64_t vote = __builtin_amdgcn_ballot_w64(splat != 0u);
+        diff_lo |= (uint32_t)vote ^ splat;
+        diff_hi |= (uint32_t)(vote >> 32) ^ splat;
+    }
+    const uint64_t diff = ((uint64_t)diff_hi << 32) | diff_lo;
+    return __builtin_amdgcn_ballot_w64(valid) & ~diff;
+}
+
 __device__ __forceinline__ uint64_t wave_peers(uint32_t digit, bool valid) {
     uint32_t diff_lo = 0, diff_hi = 0;
 #pragma unroll
@@ -448,7 +465,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
         const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
         if (vmask == 0) continue;               // wave-uniform
         if constexpr (Top) {
-            const uint64_t peers = wave_peers(digit, valid);
+            const uint64_t peers = wave_peers_n(digit, valid, dp.width);
             const uint64_t hot_peers = peers & __builtin_amdgcn_ballot_w64(valid && (key[r] >> 31));
             if (valid && peers_below(peers) == 0u) {
                 atomicAdd(&counts[wave][digit], (uint32_t)__builtin_popcountll(peers));
