@@ -7,10 +7,18 @@
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
 already resident in HBM:  loss = criterion(logits, labels); loss.backward().
 The headline workload is LabelSmoothSoftmaxCEV3 on fp32 logits (8, 19, 1024, 1024).
-Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step (GB/s);
+Prints ONE JSON line.  `value` is the bytes the timed module step has to move / time per step
+(GB/s): with reduction='mean' the forward writes no per-pixel losses and the backward reads a
+scalar upstream gradient, so the step moves less than the autograd-Function contract (unreduced
+losses written, per-element upstream gradient read); `function_level` times that contract too
+(reduction='none' and a per-element upstream gradient) with its own, larger byte count.
 `roofline` prices the dominant kernel (the backward) against the 8 TB/s HBM peak with
 HIP events on the launch stream; `cpu_baseline` times the pure-torch restatement of the
 reference's CPU path on a bounded sample on the host cores.
+Inputs of the configurations that the metric names (LSR, large-margin, focal, Lovasz, and the losses
+that share their tensors) come from oracle/synth.py, a counter-based generator in numpy integer
+arithmetic: the same bits on every box and under every torch version, so the printed losses can be
+compared between runs and with the CPU oracle.
 """
 import argparse
 import json
@@ -115,6 +123,29 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     return fwd, bwd
 
 
+def module_bytes(name, shape, dtype="f32"):
+    """Bytes the module-level step has to move (what `value` divides): as algorithmic_bytes(), minus what
+    reduction='mean' leaves out: LSR, large-margin and Taylor CE write no per-pixel losses (4P) and read
+    one scalar instead of a per-pixel upstream gradient (4P): 3bE + 16P; focal likewise (4E each way): 5bE."""
+    fwd, bwd = algorithmic_bytes(name, shape, dtype)
+    E = numel(shape)
+    P = E // shape[1]
+    if name in ("lsr", "lmargin", "taylor"):
+        return fwd - 4 * P, bwd - 4 * P
+    if name == "focal":
+        return fwd - 4 * E, bwd - 4 * E
+    return fwd, bwd
+
+
+# Workloads whose tensors are one of oracle/synth.py's named configurations (seed 15): (configuration, logits factor)
+SYNTH_CONFIG = {
+    ("lsr", (8, 19, 1024, 1024)): ("cfg2", 1.0), ("lmargin", (8, 19, 1024, 1024)): ("cfg2", 1.0),
+    ("taylor", (8, 19, 1024, 1024)): ("cfg2", 1.0), ("ohem", (8, 19, 1024, 1024)): ("cfg2", 2.0),
+    ("focal", (16, 80, 128, 128)): ("cfg3", 1.0), ("lovasz", (4, 19, 512, 1024)): ("cfg5", 1.0),
+}
+_SYNTH_CACHE = {}
+
+
 def make_inputs(name, shape, device, seed=15, dtype="f32"):
     logits, labels = _make_inputs_f32(name, shape, device, seed)
     if dtype != "f32":
@@ -128,6 +159,15 @@ def make_inputs(name, shape, device, seed=15, dtype="f32"):
 
 def _make_inputs_f32(name, shape, device, seed):
     import torch
+    if seed == 15 and (name, tuple(shape)) in SYNTH_CONFIG:
+        from oracle import synth     # input generation only; nothing of the oracle runs in a timed region
+        cfg, factor = SYNTH_CONFIG[(name, tuple(shape))]
+        if cfg not in _SYNTH_CACHE:
+            w = synth.workload(cfg)
+            _SYNTH_CACHE[cfg] = (torch.from_numpy(w["logits"]), torch.from_numpy(w["labels"]))
+        logits, labels = _SYNTH_CACHE[cfg]
+        logits = logits.to(device)
+        return (logits * factor if factor != 1.0 else logits), labels.to(device)
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     if name == "focal":
@@ -187,6 +227,42 @@ def time_steps(crit, logits, labels, steps, warmup):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     return (t1 - t0) * 1e3 / steps, float(loss.item())
+
+
+def function_level_step(name, logits, labels, steps, warmup, dtype):
+    """The autograd-Function contract, timed: unreduced losses out (reduction='none'), a per-element upstream
+    gradient in. None for the ops whose module step already is that contract."""
+    import torch
+    import pytorch_loss as pl
+    if name not in ("lsr", "lmargin", "taylor", "focal"):
+        return None
+    crit = {"lsr": lambda: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="none", ignore_index=255),
+            "lmargin": lambda: pl.LargeMarginSoftmaxV3(lam=0.3, reduction="none", ignore_index=255),
+            "taylor": lambda: pl.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="none"),
+            "focal": lambda: pl.FocalLossV3(alpha=0.25, gamma=2, reduction="none")}[name]()
+    logits.requires_grad_(True)
+    with torch.no_grad():
+        like = crit(logits, labels)
+    go = torch.full(like.shape, 1.0 / like.numel(), dtype=like.dtype, device=like.device)
+    del like
+
+    def step():
+        logits.grad = None
+        crit(logits, labels).backward(go)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    nbytes = sum(algorithmic_bytes(name, tuple(logits.shape), dtype))
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    return {"what": "reduction='none' and a per-element upstream gradient: unreduced losses written, upstream gradient read",
+            "ms_per_step": round(ms, 4), "GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes_per_step": nbytes}
 
 
 def step_distribution(crit, inputs, iters=100):
@@ -366,7 +442,17 @@ def cpu_baseline(name, shape):
           "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255),
           "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255),
           "taylor": lambda: torch_ref.taylor_ce(logits, labels, 4, "mean", 255)}[name]
-    return _time_cpu(name, shape, cores, fn, logits)
+    res = _time_cpu(name, shape, cores, fn, logits)
+    # the same image through the HIP module: the two losses are printed side by side
+    try:
+        with torch.no_grad():
+            want = float(fn().item())
+        got = float(make_criterion(name)(logits.detach().to("cuda:0"), labels.to("cuda:0")).item())
+        res["parity_spot_check"] = {"what": "loss of image 0 of the workload: HIP module on cuda:0 against the CPU restatement",
+                                    "hip": got, "cpu": want, "rel_err": abs(got - want) / max(abs(want), 1e-30)}
+    except Exception as e:
+        res["parity_spot_check"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    return res
 
 
 def _time_cpu(name, shape, cores, fn, logits):
@@ -474,8 +560,9 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
     logits, labels = make_inputs(name, shape, device, dtype=dtype)
     crit = make_criterion(name)
     ms, loss = time_steps(crit, logits, labels, steps, warmup)
-    fwd, bwd = algorithmic_bytes(name, shape, dtype)
+    fwd, bwd = module_bytes(name, shape, dtype)
     gbps = (fwd + bwd) / (ms * 1e-3) / 1e9
+    func = function_level_step(name, logits, labels, steps, warmup, dtype)
     roof = kernel_rooflines(name, logits, labels, dtype)
     dist = {"warm": step_distribution(crit, [(logits, labels)])}
     set_bytes = ELEM_BYTES[dtype] * numel(shape) * (2 if name in ("focal", "dice") else 1)
@@ -487,7 +574,7 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
         del sets
     del crit
     logits.grad = None
-    return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist)
+    return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist, function_level=func)
 
 
 def main():
@@ -525,16 +612,11 @@ def main():
             try:
                 r = run_workload(other, max(5, args.steps // 2), max(2, args.warmup // 2), device, args.dtype)
                 others[other] = {"workload": describe(other, args.dtype), "ms_per_step": round(r["ms_per_step"], 4),
-                                 "step_ms": r["step_ms"],
+                                 "step_ms": r["step_ms"], "algorithmic_bytes_per_step": r["bytes"], "loss": r["loss"],
                                  "GB/s": round(r["gbps"], 1), "frac_of_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
+                                 "function_level": r.get("function_level"),
                                  "kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
                                              for k, v in r["roofline"].items()}}
-                if other == "focal":
-                    others[other]["note"] = ("GB/s divides the Function-level algorithmic bytes (28E: unreduced losses "
-                                             "written, an upstream gradient read) by the module-level step, which moves "
-                                             "20E (reduced forward, scalar upstream) and partly runs from the 256 MB "
-                                             "last-level cache: the ratio to the HBM peak can exceed 1; the per-kernel "
-                                             "figures are the Function-level ones")
             except Exception as e:  # a secondary workload must not take the headline down
                 others[other] = {"error": "%s: %s" % (type(e).__name__, e)}
             torch.cuda.empty_cache()
@@ -564,6 +646,7 @@ def main():
                          kernel="backward entry point of the workload" if "backward" in main_res["roofline"]
                          else "the workload's single entry point"),
         "roofline_forward": main_res["roofline"].get("forward"),
+        "function_level": main_res.get("function_level"),
         "roofline_kernels": {k: {"ms": v["ms"], "GB/s": v["achieved"], "frac": v["frac"]}
                              for k, v in main_res["roofline"].items()},
         "step_ms": main_res["step_ms"],

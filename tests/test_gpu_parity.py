@@ -533,3 +533,121 @@ def test_rows_with_masked_vocabulary_entries_stay_finite(pl, n_cls, masked):
     scores = _native.ohem_scores(xt, yt, 255).cpu().numpy()
     assert np.isfinite(scores).all()
     np.testing.assert_allclose(scores, oracle.ohem_scores(x, y, 255), rtol=2e-5, atol=1e-7)
+
+
+def _prototype_logits(seed, shape, n_proto):
+    """Pixels draw their logit vector from a small set of prototypes. Pixels of one prototype get bit-equal
+    errors on the GPU and in the oracle alike (exact ties, ordered by pixel index on both sides); errors of
+    different prototypes are far apart, so no rounding difference can reorder them."""
+    n, c = shape[0], shape[1]
+    protos = synth.normal(seed, 5, (n_proto, c), 0.0, 2.0)
+    which = synth.randint(seed, 6, (n,) + tuple(shape[2:]), 0, n_proto)
+    x = np.moveaxis(protos[which], -1, 1)
+    return np.ascontiguousarray(x, dtype=np.float32), which
+
+
+def _errors_well_separated(x, y, ignore):
+    """fp64: within every class, two distinct errors differ by more than ten times what fp32 rounding can
+    move them by (relative 1e-6 for an error p, absolute 1e-6 for an error 1 - p)."""
+    p = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    yy = y.reshape(-1)
+    for c in range(x.shape[1]):
+        pc = np.moveaxis(p, 1, 0)[c].reshape(-1)
+        hot = (yy == c)[yy != ignore]
+        e = np.where(yy == c, 1.0 - pc, pc)[yy != ignore]
+        order = np.argsort(e, kind="stable")
+        e, hot = e[order], hot[order]
+        d = np.diff(e)
+        tol = np.where(hot, 1e-5, 1e-5 * e)
+        if np.any((d > 1e-12 * e[1:]) & (d <= tol[:-1] + tol[1:])):
+            return False
+    return True
+
+
+@pytest.mark.parametrize("shape,n_proto", [((2, 19, 64, 64), 16), ((2, 19, 16, 16), 24), ((3, 5, 33, 17), 48)])
+def test_lovasz_gradient_without_near_ties(pl, shape, n_proto):
+    """Where no two distinct errors of a class come close, the fp32 order is the fp64 order and the gradient is
+    held to 1e-5 max-abs, the bar the other losses meet (the looser bound of test_lovasz_function_matches_oracle
+    applies only where near-ties exist)."""
+    ignore = 255
+    for seed in range(70, 100):
+        x, which = _prototype_logits(seed, shape, n_proto)
+        y = synth.seg_labels(seed, shape[:1] + shape[2:], shape[1], ignore, 0.05)
+        ok = _errors_well_separated(x, y, ignore)
+        if ok:
+            break
+    assert ok, "no seed in range gave well separated errors"
+    xt = dev(x).requires_grad_()
+    losses = pl.LovaszSoftmaxFunctionV3.apply(xt, dev(y), ignore)
+    want, want_jacc = oracle.lovasz_forward(x.astype(np.float64), y, ignore)
+    assert np.abs(losses.detach().cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max()
+    w = synth.normal(8, 3, (shape[1],), 0.5, 1.0)
+    losses.backward(dev(w))
+    want_g = oracle.lovasz_backward(w.astype(np.float64), x.astype(np.float64), y, want_jacc, ignore)
+    err = np.abs(xt.grad.cpu().numpy() - want_g).max()
+    assert err <= GRAD_ATOL, err
+    # and with the module's 'mean' over classes
+    xt.grad = None
+    pl.LovaszSoftmaxV3(reduction="mean", ignore_index=ignore)(xt, dev(y)).backward()
+    want_g = oracle.lovasz_backward(np.full(shape[1], 1.0 / shape[1]), x.astype(np.float64), y, want_jacc, ignore)
+    assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= GRAD_ATOL
+
+
+def _one_rounding(got, want, dtype):
+    """|got - want| within one rounding step of `dtype` at want's magnitude (plus a denormal-sized floor)."""
+    eps = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    return np.all(np.abs(got - want) <= eps * np.abs(want) + 1e-7)
+
+
+@pytest.mark.parametrize("amp_dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("in_dtype", ["amp", torch.float32])
+@pytest.mark.parametrize("op", ["lsr", "focal", "lmargin", "lovasz"])
+def test_autocast_gives_fp32_losses_and_input_typed_gradients(pl, op, in_dtype, amp_dtype):
+    """What custom_fwd(cast_inputs=torch.float32) / custom_bwd give in the reference
+    (pytorch_loss/label_smooth.py:131,139): under autocast the loss is fp32 whatever the logits' type, the
+    gradient comes back in the logits' type, and the values are those of the fp32 op on the widened inputs."""
+    in_dtype = amp_dtype if in_dtype == "amp" else in_dtype
+    if op == "focal":
+        shape = (2, 8, 16, 16)
+        x = synth.normal(64, 1, shape, -2.0, 1.5)
+        y = synth.bernoulli(64, 2, shape, 0.2).astype(np.float32)
+        yt = dev(y)                                            # fp32 labels next to 16-bit logits: both are widened
+    else:
+        x, y = seg_inputs(64, (2, 19, 16, 16), 255, 0.1)
+        yt = dev(y)
+    xt = dev(x).to(in_dtype).requires_grad_()
+    xw = xt.detach().float().cpu().numpy()                     # the widened inputs the oracle sees
+    crit = {"lsr": lambda: pl.LabelSmoothSoftmaxCEV3(ignore_index=255),
+            "focal": lambda: pl.FocalLossV3(),
+            "lmargin": lambda: pl.LargeMarginSoftmaxV3(ignore_index=255),
+            "lovasz": lambda: pl.LovaszSoftmaxV3(ignore_index=255)}[op]()
+    with torch.autocast("cuda", dtype=amp_dtype):
+        out = crit(xt, yt)
+        assert out.dtype == torch.float32
+        out.backward()
+    assert xt.grad.dtype == in_dtype
+    n_valid = (y != 255).sum() if op != "focal" else y.size
+    if op == "lsr":
+        want = oracle.reduce_pixels(oracle.lsr_forward(xw.astype(np.float64), y, 255, 0.1), y, "mean", 255)
+        want_g = oracle.lsr_backward(xw.astype(np.float64), y, 255, 0.1, 1.0 / n_valid)
+    elif op == "lmargin":
+        want = oracle.reduce_pixels(oracle.lmargin_forward(xw.astype(np.float64), y, 0.3, 255), y, "mean", 255)
+        want_g = oracle.lmargin_backward(xw.astype(np.float64), y, 0.3, 255, 1.0 / n_valid)
+    elif op == "focal":
+        want = oracle.focal_forward(xw.astype(np.float64), y.astype(np.float64), 0.25, 2.0).mean()
+        want_g = oracle.focal_backward(xw.astype(np.float64), y.astype(np.float64), 0.25, 2.0, 1.0 / y.size)
+    else:
+        l64, j64 = oracle.lovasz_forward(xw.astype(np.float64), y, 255)
+        want = l64.mean()
+        want_g = oracle.lovasz_backward(np.full(19, 1.0 / 19), xw.astype(np.float64), y, j64, 255)
+    assert abs(out.item() - want) <= LOSS_RTOL * abs(want), (op, out.item(), want)
+    got_g = xt.grad.float().cpu().numpy()
+    if in_dtype == torch.float32:
+        tol = GRAD_ATOL if op != "lovasz" else max(GRAD_ATOL, 2e-3 * np.abs(j64).max() / 19)
+        assert np.abs(got_g - want_g).max() <= tol
+    elif op == "lovasz":
+        # near-ties may swap neighbours' Jaccard differences (see test_lovasz_function_matches_oracle)
+        assert np.median(np.abs(got_g - want_g)) <= 1e-6
+    else:
+        assert _one_rounding(got_g, want_g, in_dtype)
