@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|lsr_c150|lsr_vocab|lmargin_rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|lsr_c150|lsr_c300|lsr_vocab|lmargin_rows]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -66,9 +66,11 @@ WORKLOADS = {
                  "Bernoulli(0.3) labels, p=1 smooth=1"),
     "layernorm": dict(shape=(16, 256, 128, 128), desc="LayerNormV3Func fwd+bwd, fp32 (16,256,128,128) normalised over C, "
                       "eps=1e-6, per-element upstream gradient"),
-    # the same loss away from the register-resident channel counts: 150 classes in NCHW (the channels of a
-    # pixel shared out over the wavefronts of a block) and vocabulary-sized rows (a block per row)
+    # the same loss away from the register-resident channel counts: 150 and 300 classes in NCHW (the channels of
+    # a pixel shared out over the wavefronts of a block) and vocabulary-sized rows (a block per row)
     "lsr_c150": dict(base="lsr", shape=(8, 150, 512, 512), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8,150,512,512), "
+                     "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
+    "lsr_c300": dict(base="lsr", shape=(8, 300, 256, 256), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8,300,256,256), "
                      "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lsr_vocab": dict(base="lsr", shape=(8192, 32000), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8192,32000), "
                       "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),

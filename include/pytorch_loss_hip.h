@@ -105,7 +105,7 @@ int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *la
 /* plh_lsr_forward_reduced for callers that cannot allocate device memory or bring a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
  * counterpart in the reference. Same arguments and results as plh_lsr_forward_reduced, without the
- * workspace: the per-block partials live in a 1 MiB device array that is part of the library's
+ * workspace: the per-block partials live in a 2 MiB device array that is part of the library's
  * code object (each GPU that the library runs on holds its own copy until the process ends); its
  * address is looked up on the first call on each device. The call allocates and frees nothing.
  * Limit: n_size * m_size <= 2^24 pixels, else PLH_ERR_BAD_SIZE. All calls on one GPU share the one

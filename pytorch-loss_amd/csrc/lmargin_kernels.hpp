@@ -752,7 +752,25 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
     // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
     constexpr bool kHasSplit = !(WantLoss && WantGrad);
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
-                       second_f32, kHasSplit)) {
+                       second_f32, kHasSplit, kHasSplit)) {
+        case Shape::SplitDeep:
+            if constexpr (kHasSplit) {
+                constexpr int VD = V / 2;
+                blocks = split_grid<VD>(p.P);
+                switch (split_slots_deep(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (WantLoss)                                                                                       \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, VD, Reduce>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
+                               part, p);                                                                              \
+        else                                                                                                          \
+            hipLaunchKernelGGL((lm_bwd_split<T, KW, VD>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
+        break;
+                    PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+                }
+            }
+            break;
         case Shape::Split:
             if constexpr (kHasSplit) {
                 blocks = split_grid<V>(p.P);

@@ -10,7 +10,7 @@ namespace plh {
 // object (every GPU the library runs on holds its own copy at its own address until the process ends).
 // Host code never uses this name as an address; scratch_for_current_device() asks the runtime for it.
 constexpr int64_t kStaticMaxPixels = (int64_t)1 << 24;
-constexpr int64_t kStaticScratchBytes = 8 * (kStaticMaxPixels / 128);   // = 8 * partial_slots(kStaticMaxPixels) = 1 MiB
+constexpr int64_t kStaticScratchBytes = 8 * (kStaticMaxPixels / 64);    // = 8 * partial_slots(kStaticMaxPixels) = 2 MiB
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
@@ -108,7 +108,7 @@ extern "C" int plh_lsr_forward_reduced_static(const void *logits, int32_t dtype,
     if (n_size < 0 || m_size < 0 || n_size > kStaticMaxPixels || m_size > kStaticMaxPixels ||
         n_size * m_size > kStaticMaxPixels)
         return PLH_ERR_BAD_SIZE;
-    static_assert(8 * ((kStaticMaxPixels + 127) / 128) <= kStaticScratchBytes && kStaticMaxPixels / 128 >= kMinPartialSlots,
+    static_assert(8 * ((kStaticMaxPixels + 63) / 64) <= kStaticScratchBytes && kStaticMaxPixels / 64 >= kMinPartialSlots,
                   "the static buffer holds the partials of the largest accepted input");
     void *ws = nullptr;
     const int rc = scratch_for_current_device(&ws);

@@ -655,6 +655,18 @@ template <class T, int V, bool Reduce>
 static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                  hipStream_t st) {
     const unsigned grid = split_grid<V>(p.P);
+    if constexpr (V < ElemTraits<T>::kVec) {        // the deep form
+        switch (split_slots_deep(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
+                           part, p);                                                                              \
+        break;
+            PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+        }
+        return grid;
+    }
     switch (split_slots(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
@@ -671,6 +683,17 @@ template <class T, int V>
 static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
                              hipStream_t st) {
     const unsigned grid = split_grid<V>(p.P);
+    if constexpr (V < ElemTraits<T>::kVec) {        // the deep form
+        switch (split_slots_deep(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_bwd_split<T, KW, V>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
+        break;
+            PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+        }
+        return;
+    }
     switch (split_slots(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
@@ -686,10 +709,11 @@ template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
                         hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
             if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
@@ -723,10 +747,11 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::SplitDeep: launch_bwd_split<T, V / 2>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
             if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);

@@ -75,19 +75,29 @@ inline int check_gout(const void *gout, int64_t stride) {
 // gradient), labels int64. nullptr = tensor not used.
 // Split: the regs shape with the channels of a pixel shared out over the 8 wavefronts of a block
 // (see "the split launch shape" below); only for kernels that have that form (`with_split`).
-enum class Shape { RegsVec, RegsOne, Split, Wave, Lane };
+// SplitDeep: the split shape with half the pixels per lane (4 bytes per lane and channel) and up to 64
+// channel slots per wavefront, for 257..512 channels; only for kernels that have it (`with_deep`).
+enum class Shape { RegsVec, RegsOne, Split, SplitDeep, Wave, Lane };
 
 constexpr int kMaxRegsChannels = 32;
 constexpr int kSplitWaves = 8;
 constexpr int kMaxSplitChannels = kMaxRegsChannels * kSplitWaves;
+constexpr int kMaxDeepSlots = 64;
+constexpr int kMaxDeepChannels = kMaxDeepSlots * kSplitWaves;
 
 inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, const void *typed0, const void *typed1,
-                        const void *labels, const void *f32a, const void *f32b, bool with_split = false) {
-    const bool vec = (m_size % V == 0) && !(typed0 && misaligned(typed0, V * elem)) &&
-                     !(typed1 && misaligned(typed1, V * elem)) && !(f32a && misaligned(f32a, V * 4)) &&
-                     !(f32b && misaligned(f32b, V * 4)) && !(labels && misaligned(labels, 16));
+                        const void *labels, const void *f32a, const void *f32b, bool with_split = false,
+                        bool with_deep = false) {
+    auto fits = [&](int v) {
+        return (m_size % v == 0) && !(typed0 && misaligned(typed0, v * elem)) &&
+               !(typed1 && misaligned(typed1, v * elem)) && !(f32a && misaligned(f32a, v * 4)) &&
+               !(f32b && misaligned(f32b, v * 4)) && !(labels && misaligned(labels, v > 1 ? 16 : 8));
+    };
+    const bool vec = fits(V) && !(labels && misaligned(labels, 16));
     if (dimsize <= kMaxRegsChannels) return vec ? Shape::RegsVec : Shape::RegsOne;
     if (with_split && vec && dimsize <= kMaxSplitChannels && m_size >= 64) return Shape::Split;
+    if (with_deep && dimsize > kMaxSplitChannels && dimsize <= kMaxDeepChannels && m_size >= 64 && fits(V / 2))
+        return Shape::SplitDeep;
     return m_size == 1 ? Shape::Wave : Shape::Lane;
 }
 
@@ -322,6 +332,22 @@ template <class T> struct Pack<T, 4> {          // T = f16 or bf16
         return Raw{(keep[0] & 0xFFFFu) | (keep[1] & 0xFFFF0000u), (keep[2] & 0xFFFFu) | (keep[3] & 0xFFFF0000u)};
     }
 };
+template <class T> struct Pack<T, 2> {          // T = f16 or bf16: one dword, two pixels
+    typedef unsigned Raw;
+    static __device__ __forceinline__ Raw load(const T *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const unsigned *>(p));
+    }
+    static __device__ __forceinline__ void store(T *p, Raw r) {
+        __builtin_nontemporal_store(r, reinterpret_cast<unsigned *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int k) { return (k & 1) ? widen_hi(r, T{}) : widen_lo(r, T{}); }
+    static __device__ __forceinline__ Raw put(const float (&g)[2]) { return narrow2(g[0], g[1], T{}); }
+    static constexpr int kStep = 2;
+    static __device__ __forceinline__ void set(Raw &r, int, const float (&g)[2]) { r = narrow2(g[0], g[1], T{}); }
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[2]) {
+        return (keep[0] & 0xFFFFu) | (keep[1] & 0xFFFF0000u);
+    }
+};
 template <class T> struct Pack<T, 1> {          // T = f16 or bf16
     typedef unsigned Raw;
     static __device__ __forceinline__ Raw load(const T *p) {
@@ -409,8 +435,8 @@ enum FinishMode { kFinishSum = 0, kFinishMeanOverCount = 1, kFinishMeanOverFixed
 constexpr int64_t kMinPartialSlots = 16384;   // the looping kernels cap their grid at this many blocks
 
 inline int64_t partial_slots(int64_t units) {
-    // the smallest tile any reducing kernel gives a block: 128 pixels (split shape, fp32)
-    const int64_t blocks = ceil_div(units > 0 ? units : 1, 128);
+    // the smallest tile any reducing kernel gives a block: 64 pixels (deep split shape, fp32)
+    const int64_t blocks = ceil_div(units > 0 ? units : 1, 64);
     return blocks > kMinPartialSlots ? blocks : kMinPartialSlots;
 }
 
@@ -695,6 +721,13 @@ inline int split_slots(int64_t dimsize) {
     const int per = (int)ceil_div(dimsize, kSplitWaves);
     const int kw = (per + 3) / 4 * 4;
     return kw < 8 ? 8 : kw;
+}
+// The deep form (257..512 channels): 40, 48, 56 or 64 slots per wavefront.
+#define PLH_SPLIT_DEEP_CASES PLH_CASE(40) PLH_CASE(48) PLH_CASE(56) PLH_CASE(64)
+inline int split_slots_deep(int64_t dimsize) {
+    const int per = (int)ceil_div(dimsize, kSplitWaves);
+    const int kw = (per + 7) / 8 * 8;
+    return kw < 40 ? 40 : kw;
 }
 
 template <class T, int V, int KW>

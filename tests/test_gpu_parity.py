@@ -102,7 +102,13 @@ SEG_CASES = [
     ((1, 133, 8, 8), 255, 0.1),
     ((1, 171, 8, 8), 255, 0.1),
     ((1, 200, 8, 8), 255, 0.1),
-    ((2, 257, 8, 8), 255, 0.1),                     # one channel more: a lane per pixel again
+    ((2, 257, 8, 8), 255, 0.1),                     # 257..512 channels: the same with up to 64 slots per wavefront
+    ((1, 300, 9, 8), 255, 0.1),                     #   and half the pixels per lane (LSR, large-margin); slot counts
+    ((2, 321, 8, 8), -100, 0.2),                    #   40, 48, 56, 64, last wavefronts partly or wholly empty,
+    ((1, 400, 8, 9), 255, 0.1),                     #   pixel counts that leave lanes idle
+    ((1, 449, 8, 8), 255, 0.1),
+    ((1, 512, 8, 8), 255, 0.1),
+    ((1, 513, 8, 8), 255, 0.1),                     # one channel more: a lane per pixel
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
