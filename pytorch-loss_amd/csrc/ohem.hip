@@ -10,8 +10,9 @@
 //                  n_min-th smallest score, and how many pixels with exactly that score still
 //                  fall below position n_min (`keep_ties`); the histogram kernel of a digit first
 //                  resolves the digit before it (every block for itself, from the finished table);
-//   3. ties        pixels equal to v are ranked in pixel order (what a stable key sort gives):
-//                  per-tile counts, one scan over the tiles, in-tile ranks from ballots;
+//   3. ties        pixels equal to v are ranked in pixel order (what a stable key sort gives): a
+//                  wavefront per run of tiles counts them (running count per tile, total per run),
+//                  the relabelling adds up the runs before its own, in-tile ranks from ballots;
 //   4. relabel     drop = score > thresh && (score > v || (score == v && tie_rank >= keep_ties)).
 // When v <= thresh every pixel above the threshold lies beyond position n_min, so steps 3 is
 // skipped on the device (the kernels return at once). Scores are positive floats, whose bit
@@ -246,8 +247,12 @@ __global__ __launch_bounds__(kRowBlock) void ohem_scores_row(const T *__restrict
 struct OhemTables {
     uint32_t *hist;        // [3][kOhemBins]
     uint32_t *state;       // [16]
-    uint32_t *tile_ties;   // [tiles], exclusive-scanned in place
+    uint32_t *tile_ties;   // [tiles]: ties in the earlier tiles of the same run; then [kTieRuns]: ties per run
 };
+
+// The tie count: kTieRuns runs of consecutive tiles, a wavefront per run.
+constexpr int kTieRuns = 1024;
+__host__ __device__ inline int tie_run_tiles(int tiles) { return (tiles + kTieRuns - 1) / kTieRuns; }
 
 __global__ void ohem_zero(uint32_t *p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -357,12 +362,6 @@ __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ score
         if (bins[i]) atomicAdd(out + i, bins[i]);
 }
 
-// One block: the last digit, for the kernels that follow.
-__global__ __launch_bounds__(256) void ohem_pick(OhemTables tb, int pass, uint32_t n_min) {
-    __shared__ uint32_t scan[260];
-    ohem_resolve_digit(tb, pass, n_min, scan, true);
-}
-
 // This thread's 4 consecutive scores and their keys; pixels beyond the end match no key.
 __device__ __forceinline__ void load_tile_keys(const float *scores, int P, int base, bool vec, float (&s)[4],
                                                uint32_t (&key)[4]) {
@@ -381,56 +380,45 @@ __device__ __forceinline__ void load_tile_keys(const float *scores, int P, int b
     }
 }
 
-// state[4], state[5]: v = the n_min-th smallest key, and how many pixels equal to it lie below
-// sorted position n_min. Ranks among the ties are needed only when v exceeds the threshold.
-__global__ __launch_bounds__(256) void ohem_count_ties(const float *__restrict__ scores, OhemTables tb, int P,
-                                                       float thresh, int vec) {
-    __shared__ float red[4];
-    const uint32_t v = tb.state[4];
-    if (!(__builtin_bit_cast(float, v) > thresh)) return;
-    float s[4];
-    uint32_t key[4];
-    load_tile_keys(scores, P, blockIdx.x * kOhemTile + threadIdx.x * 4, vec != 0, s, key);
-    int n = 0;
+// The last digit (every block for itself, block 0 publishes: state[4] = v, the n_min-th smallest key,
+// state[5] = how many pixels equal to it lie below sorted position n_min), then, only when v exceeds
+// the threshold (otherwise no rank among the ties is ever looked at), the ties in pixel order: each
+// wavefront walks one run of consecutive tiles and leaves, per tile, the ties in the run's earlier
+// tiles, and per run its total. One launch where a pick, a count and a scan kernel were three.
+__global__ __launch_bounds__(256) void ohem_ties(const float *__restrict__ scores, OhemTables tb, int P, int tiles,
+                                                 uint32_t n_min, float thresh, int vec) {
+    __shared__ uint32_t scan[260];
+    const uint32_t v = ohem_resolve_digit(tb, 2, n_min, scan, blockIdx.x == 0);
+    if (!(__builtin_bit_cast(float, v) > thresh)) return;       // block-uniform
+    const int lane = threadIdx.x & 63;
+    const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int per = tie_run_tiles(tiles);
+    uint32_t before = 0;
+    for (int t = run * per; t < min(tiles, (run + 1) * per); ++t) {      // wave-uniform
+        uint32_t n = 0;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) n += key[k] == v ? 1 : 0;
-    const float total = block_sum_256((float)n, red);                 // <= 1024: exact
-    if (threadIdx.x == 0) tb.tile_ties[blockIdx.x] = (uint32_t)total;
-}
-
-// Exclusive scan of the per-tile tie counts, one block.
-__global__ __launch_bounds__(256) void ohem_scan_tiles(OhemTables tb, int tiles, float thresh) {
-    __shared__ uint32_t scan[256];
-    __shared__ uint32_t carry;
-    if (!(__builtin_bit_cast(float, tb.state[4]) > thresh)) return;
-    if (threadIdx.x == 0) carry = 0;
-    __syncthreads();
-    for (int base = 0; base < tiles; base += 256) {
-        const int i = base + threadIdx.x;
-        const uint32_t v = i < tiles ? tb.tile_ties[i] : 0u;
-        scan[threadIdx.x] = v;
-        __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {
-            const uint32_t add = (threadIdx.x >= off) ? scan[threadIdx.x - off] : 0u;
-            __syncthreads();
-            scan[threadIdx.x] += add;
-            __syncthreads();
+        for (int q = 0; q < kOhemTile / 256; ++q) {             // a tile is 1024 pixels: 4 x (64 lanes x 4)
+            float s[4];
+            uint32_t key[4];
+            load_tile_keys(scores, P, t * kOhemTile + (q * 64 + lane) * 4, vec != 0, s, key);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) n += key[k] == v ? 1u : 0u;
         }
-        if (i < tiles) tb.tile_ties[i] = carry + scan[threadIdx.x] - v;
-        __syncthreads();
-        if (threadIdx.x == 255) carry += scan[255];
-        __syncthreads();
+        n = (uint32_t)group_reduce<64>((float)n, OpSum());      // <= 1024: exact
+        if (lane == 0) tb.tile_ties[t] = before;
+        before += n;
     }
+    if (lane == 0 && run < kTieRuns) tb.tile_ties[tiles + run] = before;
 }
 
 // With `part`, the block also leaves the sum of `ce` over the pixels that keep a label other than
 // `ignore`, and their number: the mean cross entropy of the relabelled batch needs no further pass
 // over the logits.
 __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ scores, const int64_t *__restrict__ lab,
-                                                    int64_t *__restrict__ out, OhemTables tb, int P, uint32_t n_min,
+                                                    int64_t *__restrict__ out, OhemTables tb, int P, int tiles, uint32_t n_min,
                                                     float thresh, int64_t ignore, int vec,
                                                     const float *__restrict__ ce, Partials part) {
-    __shared__ uint32_t wave_ties[4];
+    __shared__ uint32_t wave_ties[4], run_ties[4];
     __shared__ float red[4];
     const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
     float s[4];
@@ -456,8 +444,20 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
             if ((threadIdx.x & 63) >= off) lane_incl += up;
         }
         if ((threadIdx.x & 63) == 63) wave_ties[threadIdx.x >> 6] = (uint32_t)lane_incl;
-        __syncthreads();
-        uint32_t before = tb.tile_ties[blockIdx.x] + (uint32_t)(lane_incl - mine);
+        // ties in the runs of tiles before this tile's run (ohem_ties): kTieRuns totals, 4 per thread
+        const int my_run = blockIdx.x / tie_run_tiles(tiles);
+        uint32_t earlier = 0;
+#pragma unroll
+        for (int q = 0; q < kTieRuns / 256; ++q) {
+            const int r = q * 256 + threadIdx.x;
+            earlier += r < my_run ? tb.tile_ties[tiles + r] : 0u;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) earlier += (uint32_t)__shfl_xor((int)earlier, off, 64);
+        if ((threadIdx.x & 63) == 0) run_ties[threadIdx.x >> 6] = earlier;
+        __syncthreads();                                           // also what wave_ties needs
+        const uint32_t runs_before = (run_ties[0] + run_ties[1]) + (run_ties[2] + run_ties[3]);
+        uint32_t before = runs_before + tb.tile_ties[blockIdx.x] + (uint32_t)(lane_incl - mine);
         for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) before += wave_ties[w];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -571,7 +571,9 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
     return check_launch();
 }
 
-static int64_t select_workspace(int64_t P) { return align256(kOhemZeroWords * 4) + align256(ohem_tiles(P) * 4); }
+static int64_t select_workspace(int64_t P) {
+    return align256(kOhemZeroWords * 4) + align256((ohem_tiles(P) + kTieRuns) * 4);
+}
 
 // The tables are needed unless the labels pass through unchanged (n_min >= P).
 static int check_workspace(const void *workspace, int64_t workspace_bytes, int64_t P, int64_t n_min) {
@@ -611,11 +613,9 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
         for (int pass = 0; pass < 3; ++pass)
             hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, vec);
-        hipLaunchKernelGGL(ohem_pick, dim3(1), dim3(256), 0, st, tb, 2, k);
-        hipLaunchKernelGGL(ohem_count_ties, dim3((unsigned)tiles), dim3(256), 0, st, scores, tb, Pi, score_thresh, vec);
-        hipLaunchKernelGGL(ohem_scan_tiles, dim3(1), dim3(256), 0, st, tb, (int)tiles, score_thresh);
+        hipLaunchKernelGGL(ohem_ties, dim3(kTieRuns / 4), dim3(256), 0, st, scores, tb, Pi, (int)tiles, k, score_thresh, vec);
     }
-    hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, k,
+    hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, (int)tiles, k,
                        score_thresh, ignore_index, vec, ce, part);
     return check_launch();
 }
