@@ -17,10 +17,11 @@ import torch.nn as nn
 from . import _native
 
 
-def _even_order(n, strictly_positive=True):
-    """The reference asserts on the order where it is given (taylor_softmax.py:89, 110, 132, 182)."""
-    ok = n % 2 == 0 and (n > 0 or not strictly_positive)
-    assert ok, "the order of the Taylor polynomial must be even and positive"
+def _even_order(n):
+    """The reference asserts on the order where it is given (taylor_softmax.py:89, 110, 132, 182). Its log
+    module and its cross entropy let n = 0 through their constructors (`assert n % 2 == 0`) and fail on it
+    in the first forward (`assert n % 2 == 0 and n > 0`, :36); here the constructor already refuses it."""
+    assert n % 2 == 0 and n > 0, "the order of the Taylor polynomial must be even and positive"
     return n
 
 
@@ -45,7 +46,7 @@ class _TaylorAlongDim(nn.Module):
 
     def __init__(self, dim=1, n=2):
         super().__init__()
-        self.dim, self.n = dim, _even_order(n, strictly_positive=not self.use_log)
+        self.dim, self.n = dim, _even_order(n)
 
     def forward(self, x):
         return taylor_softmax_v3(x, self.dim, self.n, self.use_log)
@@ -83,7 +84,7 @@ class TaylorCrossEntropyLossV3(nn.Module):
 
     def __init__(self, n=2, ignore_index=-1, reduction='mean'):
         super().__init__()
-        self.n, self.ignore_index, self.reduction = _even_order(n, strictly_positive=False), ignore_index, reduction
+        self.n, self.ignore_index, self.reduction = _even_order(n), ignore_index, reduction
 
     def forward(self, logits, labels):
         return TaylorCrossEntropyFunctionV3.apply(logits, labels, self.n, self.ignore_index, self.reduction)

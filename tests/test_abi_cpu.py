@@ -264,3 +264,14 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_taylor_orders_are_checked_at_construction():
+    import pytorch_loss as pl
+    for bad in (0, 3, -2):
+        for make in (pl.TaylorSoftmaxV3, pl.LogTaylorSoftmaxV3):
+            with pytest.raises(AssertionError):
+                make(dim=1, n=bad)
+        with pytest.raises(AssertionError):
+            pl.TaylorCrossEntropyLossV3(n=bad)
+    assert pl.TaylorCrossEntropyLossV3(n=4).n == 4 and pl.LogTaylorSoftmaxV3(n=2).n == 2
