@@ -588,6 +588,88 @@ __global__ __launch_bounds__(kRowBlock) void lsr_bwd_row(const T *__restrict__ x
     }
 }
 
+// The same with the row kept in the block's registers between the two uses (NCH 16-byte chunks per
+// thread, as loaded; widened where they are used): rows of up to 16 chunks per thread, i.e. 65536 fp32
+// or 131072 16-bit elements with 1024 threads, are read from memory once, where the kernel above reads
+// them twice (the second time through the caches, for as long as the rows in flight fit them). The few
+// elements before the first and after the last 16-byte boundary of a row are re-read instead.
+template <class T> __device__ __forceinline__ void chunk_widen(const plh_u4 &t, float (&v)[RowChunk<T>::kLen]) {
+    if constexpr (sizeof(T) == 4) {
+        v[0] = bits_f32(t.x); v[1] = bits_f32(t.y); v[2] = bits_f32(t.z); v[3] = bits_f32(t.w);
+    } else {
+        const unsigned d[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = widen_lo(d[i], T{});
+            v[2 * i + 1] = widen_hi(d[i], T{});
+        }
+    }
+}
+
+template <class T, int NCH>
+__global__ __launch_bounds__(kRowBlock) void lsr_bwd_rowregs(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                            const Upstream up, T *__restrict__ grad, const LsrParams p) {
+    __shared__ float red[kRowBlock / 64];
+    constexpr int L = RowChunk<T>::kLen;
+    const int threads = row_threads();
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
+        const T *xs = x + row * p.C;
+        T *gs = grad + row * p.C;
+        const RowSplit<T> sp(xs, p.C, true);
+        plh_u4 raw[NCH];
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            const int i = threadIdx.x + u * threads;
+            if (i < sp.chunks) raw[u] = __builtin_nontemporal_load(reinterpret_cast<const plh_u4 *>(xs + sp.head + (int64_t)i * L));
+        }
+        // the row's ends: at most L - 1 elements each, one per thread
+        const int n_edge = sp.head + (p.C - sp.tail_from);
+        const int edge_at = (int)threadIdx.x < sp.head ? (int)threadIdx.x : sp.tail_from + ((int)threadIdx.x - sp.head);
+        const bool has_edge = (int)threadIdx.x < n_edge;
+        const float edge = has_edge ? load_one(xs + edge_at) : -INFINITY;
+        float mx = edge;
+#pragma unroll
+        for (int u = 0; u < NCH; ++u)
+            if (threadIdx.x + u * threads < sp.chunks) {
+                float v[L];
+                chunk_widen<T>(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < L; ++e) mx = fmaxf(mx, v[e]);
+            }
+        const float m = row_block_reduce(mx, red, OpMax());
+        float s = fast_exp(edge - m);                                   // 0 for a thread without an edge element
+#pragma unroll
+        for (int u = 0; u < NCH; ++u)
+            if (threadIdx.x + u * threads < sp.chunks) {
+                float v[L];
+                chunk_widen<T>(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < L; ++e) s += fast_exp(v[e] - m);
+            }
+        const float total = row_block_reduce(s, red, OpSum());
+        const int64_t lb = lab[row];
+        float go[1];
+        load_upstream<1>(up, row, go);
+        const float gk = (lb == p.ignore) ? 0.f : go[0];
+        const float scale = p.sumw * gk / total;
+        const float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            const int i = threadIdx.x + u * threads;
+            if (i < sp.chunks) {
+                float v[L];
+                chunk_widen<T>(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < L; ++e)
+                    v[e] = __builtin_fmaf(fast_exp(v[e] - m), scale, (sp.head + i * L + e == tgt) ? n_pos : n_neg);
+                RowChunk<T>::store(gs + sp.head + (int64_t)i * L, v);
+            }
+        }
+        if (has_edge) store_one(gs + edge_at, __builtin_fmaf(fast_exp(edge - m), scale, (edge_at == tgt) ? n_pos : n_neg));
+    }
+}
+
 // ------------------------------------------------------------ dispatch ----
 
 inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore, float smooth,
@@ -755,6 +837,22 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::Wave:
             if (p.C > kWaveRowCap) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+                // chunks a row can have at most, and the threads that share them: 256 while 16 chunks per thread do
+                const int chunks = p.C / RowChunk<T>::kLen + 1;
+                const int threads = chunks <= kRowBlockShort * 16 ? kRowBlockShort : kRowBlock;
+                const int per = (chunks + threads - 1) / threads;
+                if (row_chunks_ok<T>(logits, grad_logits, p.C) && per <= 16) {
+                    if (per <= 4)
+                        hipLaunchKernelGGL((lsr_bwd_rowregs<T, 4>), dim3(grid), dim3(threads), 0, st, logits, labels, up,
+                                           grad_logits, p);
+                    else if (per <= 8)
+                        hipLaunchKernelGGL((lsr_bwd_rowregs<T, 8>), dim3(grid), dim3(threads), 0, st, logits, labels, up,
+                                           grad_logits, p);
+                    else
+                        hipLaunchKernelGGL((lsr_bwd_rowregs<T, 16>), dim3(grid), dim3(threads), 0, st, logits, labels, up,
+                                           grad_logits, p);
+                    break;
+                }
                 hipLaunchKernelGGL((lsr_bwd_row<T>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, logits, labels, up, grad_logits, p,
                                    row_chunks_ok<T>(logits, grad_logits, p.C));
                 break;
