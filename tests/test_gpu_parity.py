@@ -657,3 +657,38 @@ def test_autocast_gives_fp32_losses_and_input_typed_gradients(pl, op, in_dtype, 
         assert np.median(np.abs(got_g - want_g)) <= 1e-6
     else:
         assert _one_rounding(got_g, want_g, in_dtype)
+
+
+@pytest.mark.parametrize("n_cls,scale,boost,passes", [(400, 0.002, 0.0, 2), (120, 0.3, 0.0, 3), (120, 1.0, 12.0, 4)])
+def test_lovasz_sort_passes_follow_the_key_width(pl, n_cls, scale, boost, passes):
+    """The sort looks only at the key bits below a class's limit: near-uniform predictions over many classes
+    (best positive's error above 0.996: at most 16 key bits) take two passes, soft ones three, confident ones
+    all four. Every plan against the fp32 restatement bit for bit, and the loss against the fp64 one."""
+    from pytorch_loss import _native
+    shape = (2, n_cls, 40, 50)
+    y = synth.seg_labels(53, (2, 40, 50), n_cls, 255, 0.1)
+    x = synth.normal(53, 1, shape, 0.0, scale)
+    if boost:
+        onehot = np.moveaxis(np.eye(n_cls, dtype=np.float32)[np.where(y == 255, 0, y)], -1, 1)
+        x = x + np.float32(boost) * onehot
+    # the number of passes each class with positives takes, from the key of its best classified positive
+    p = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    need = []
+    for c in range(n_cls):
+        hot = (y == c)
+        if hot.any():
+            err = np.float32(1.0) - np.moveaxis(p, 1, 0)[c][hot].astype(np.float32)
+            key = int(np.float32(1.0).view(np.uint32)) - int(np.float32(err.min()).view(np.uint32))
+            width = max(1, key.bit_length())
+            need.append(2 if width <= 16 else (3 if width <= 24 else 4))
+    assert need.count(passes) > 0.9 * len(need), {k: need.count(k) for k in set(need)}
+    losses, jacc = _native.lovasz_forward(dev(x), dev(y), 255)
+    jacc = jacc.cpu().numpy()
+    l32, j32 = oracle.lovasz_forward(x, y, 255)
+    assert (jacc.view(np.uint32) == j32.view(np.uint32)).mean() > 0.995
+    assert (jacc[:, y.reshape(-1) == 255] == 0).all()
+    l64, _ = oracle.lovasz_forward(x.astype(np.float64), y, 255)
+    # confident predictions: a positive's error 1 - p with p = 0.9993 carries p's fp32 rounding 1400 times enlarged,
+    # in the reference's fp32 kernels too; the loss, which those errors make up, inherits it
+    np.testing.assert_allclose(losses.cpu().numpy(), l64, rtol=3e-4 if boost else 1e-5)
