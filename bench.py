@@ -289,6 +289,33 @@ def step_distribution(crit, inputs, iters=100):
             "p90": round(ms[(9 * len(ms)) // 10], 4), "iters": iters, "input_sets": len(inputs)}
 
 
+def graph_step(crit, logits, labels, iters=100):
+    """The module step captured once in a HIP graph and replayed: its time on the GPU alone, without the
+    host's share (Python, the autograd engine's thread hand-over, launch latency). None if capture fails."""
+    import torch
+    try:
+        logits.requires_grad_(True)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                logits.grad = None
+                crit(logits, labels).backward()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        logits.grad = None
+        with torch.cuda.graph(graph):
+            crit(logits, labels).backward()
+        torch.cuda.synchronize()
+        ms = time_kernel(graph.replay, iters=iters, warmup=10)
+        del graph
+        logits.grad = None
+        return {"ms": round(ms, 4), "iters": iters,
+                "what": "the same fwd+bwd step captured in a HIP graph and replayed (GPU time without the host's share)"}
+    except Exception as e:
+        return {"error": "%s: %s" % (type(e).__name__, e)}
+
+
 def time_kernel(launch, iters=30, warmup=5):
     """Average duration (ms) of one launch: HIP events on the stream the kernel runs on."""
     import torch
@@ -574,6 +601,7 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
         sets = [(logits, labels)] + [make_inputs(name, shape, device, seed=100 + i, dtype=dtype) for i in range(n_sets - 1)]
         dist["cold"] = step_distribution(crit, sets)
         del sets
+    dist["graph"] = graph_step(crit, logits, labels)
     del crit
     logits.grad = None
     return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist, function_level=func)
