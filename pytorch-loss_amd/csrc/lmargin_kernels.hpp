@@ -38,24 +38,23 @@ struct LmParams {
 // log2(s_no), sum q_j u_j and the rebuilt full sum.
 constexpr float kLmMasked = -1e30f;
 
-template <class T, int CP, int V, bool Uniform, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, int CP, int V, int Form, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                      const Upstream up,
                                                      float *__restrict__ loss, T *__restrict__ grad,
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
     __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     const bool live = at.live;
     if (!Reduce && !live) return;
-    const int64_t pix = at.pix;
 
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + pix, lb);
+    at.labels(lab, p.ignore, lb);
     float go[V];
-    if constexpr (WantGrad) load_upstream<V>(up, pix, go);
+    if constexpr (WantGrad) at.upstream(up, go);
 
     float out[V], score[V];
     float g[WantGrad ? CP : 1][V];
@@ -141,8 +140,8 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
         if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
     }
     if (live) {
-        if (WantLoss && loss) store_vec<V>(loss + pix, out);
-        if (WantLoss && p.scores) store_vec_cached<V>(p.scores + pix, score);
+        if (WantLoss && loss) at.store_f32(loss, out);
+        if (WantLoss && p.scores) at.store_f32_cached(p.scores, score);
         if constexpr (WantGrad) {
             // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
             const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
@@ -728,15 +727,32 @@ static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, 
     case K:                                                                                                          \
         if constexpr (V * sizeof(T) == 8) {                                                                          \
             if (uni) {                                                                                               \
-                hipLaunchKernelGGL((lm_regs<T, 4 * K, V, true, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),  \
+                hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kUniform, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),  \
                                    dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                   \
                 break;                                                                                               \
             }                                                                                                        \
         }                                                                                                            \
-        hipLaunchKernelGGL((lm_regs<T, 4 * K, V, false, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),         \
+        hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kGeneral, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),         \
                            dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                           \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
+#undef PLH_CASE
+    }
+    return grid;
+}
+
+// fp32 NCHW whose channel planes have odd length: the per-image form, four pixels per lane.
+template <bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+static unsigned launch_image(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
+                             unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
+    const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                                  \
+    case K:                                                                                                          \
+        hipLaunchKernelGGL((lm_regs<float, 4 * K, 4, kPerImage, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
+                           dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                           \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
 #undef PLH_CASE
     }
     return grid;
@@ -792,6 +808,12 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             blocks = launch_regs<T, V, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::RegsOne:
+            if constexpr (std::is_same<T, float>::value) {
+                if (image_form_pays(p.C, p.m_size)) {
+                    blocks = launch_image<WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+                    break;
+                }
+            }
             blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::Wave:

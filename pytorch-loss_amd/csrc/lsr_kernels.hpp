@@ -34,19 +34,19 @@ struct LsrParams {
 // exp(x - mx) is evaluated as exp2(fma(x, log2e, -c)) with c = fl(mx * log2e); what the rounding
 // of c left out, r = mx*log2e - c (exact, one fma), scales every term by 2^r and is taken back
 // out of log2(sum).
-template <class T, int CP, int V, bool Uniform, bool Reduce>
+template <class T, int CP, int V, int Form, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           float *__restrict__ loss, Partials part,
                                                           const LsrParams p) {
     __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
 
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
 
     float out[V];
     float mine = 0.f;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
         mine += out[k];
         cnt += valid ? 1 : 0;
     }
-    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if (at.live && loss) at.store_f32(loss, out);
     if constexpr (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);   // at most 1024 per block: exact in fp32
@@ -89,20 +89,20 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     }
 }
 
-template <class T, int CP, int V, bool Uniform>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           const Upstream up, T *__restrict__ grad,
                                                           const LsrParams p) {
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
 
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     float go[V];
-    load_upstream<V>(up, at.pix, go);
+    at.upstream(up, go);
 
     // The gradient of a pixel replaces its logits in the slice as soon as they are no longer needed
     // (one pixel at a time for fp32, two for 16-bit elements, which share a dword): no second array.
@@ -696,12 +696,12 @@ static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Par
     case K:                                                                                                       \
         if constexpr (V * sizeof(T) == 8) {                                                                       \
             if (uni) {                                                                                            \
-                hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, true, Reduce>), dim3(grid), dim3(kRegsBlock), 0,    \
+                hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kUniform, Reduce>), dim3(grid), dim3(kRegsBlock), 0,    \
                                    st, x, lab, loss, part, p);                                                    \
                 break;                                                                                            \
             }                                                                                                     \
         }                                                                                                         \
-        hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, false, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
+        hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kGeneral, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
                            lab, loss, part, p);                                                                   \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -720,12 +720,12 @@ static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, 
     case K:                                                                                                      \
         if constexpr (V * sizeof(T) == 8) {                                                                      \
             if (uni) {                                                                                           \
-                hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
+                hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kUniform>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
                                    lab, up, grad, p);                                                            \
                 break;                                                                                           \
             }                                                                                                    \
         }                                                                                                        \
-        hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, false>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up,  \
+        hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up,  \
                            grad, p);                                                                             \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -786,6 +786,37 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     }
 }
 
+// fp32 NCHW whose channel planes have odd length: the per-image form, four pixels per lane.
+template <bool Reduce>
+static unsigned launch_fwd_image(const float *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
+                                 hipStream_t st) {
+    const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                               \
+    case K:                                                                                                       \
+        hipLaunchKernelGGL((lsr_fwd_regs<float, 4 * K, 4, kPerImage, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
+                           st, x, lab, loss, part, p);                                                            \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
+#undef PLH_CASE
+    }
+    return grid;
+}
+
+static void launch_bwd_image(const float *x, const int64_t *lab, const Upstream &up, float *grad, const LsrParams &p,
+                             hipStream_t st) {
+    const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
+    switch ((p.C + 3) / 4) {
+#define PLH_CASE(K)                                                                                              \
+    case K:                                                                                                      \
+        hipLaunchKernelGGL((lsr_bwd_regs<float, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
+                           lab, up, grad, p);                                                                    \
+        break;
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
+#undef PLH_CASE
+    }
+}
+
 // Launches the forward; returns the number of blocks that wrote partials.
 template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
@@ -793,7 +824,11 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
     constexpr int V = ElemTraits<T>::kVec;
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
-        case Shape::RegsOne: return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::RegsOne:
+            if constexpr (std::is_same<T, float>::value) {
+                if (image_form_pays(p.C, p.m_size)) return launch_fwd_image<Reduce>(logits, labels, losses, part, p, st);
+            }
+            return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
@@ -831,7 +866,15 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
-        case Shape::RegsOne: launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::RegsOne:
+            if constexpr (std::is_same<T, float>::value) {
+                if (image_form_pays(p.C, p.m_size)) {
+                    launch_bwd_image(logits, labels, up, grad_logits, p, st);
+                    break;
+                }
+            }
+            launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st);
+            break;
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::SplitDeep: launch_bwd_split<T, V / 2>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:

@@ -279,6 +279,34 @@ template <> struct Pack<float, 2> {
     // AND-mask that clears pixel k of a packed gradient when keep[k] is 0 (keep[k] is 0 or ~0)
     static __device__ __forceinline__ Raw mask(const unsigned (&keep)[2]) { return Raw{keep[0], keep[1]}; }
 };
+// Four fp32 pixels per lane, for the per-image form of the regs shape (channel planes of odd length:
+// a lane's 16 bytes start on a 4-byte boundary; the hardware takes such accesses, the types say so).
+typedef unsigned plh_u4w __attribute__((ext_vector_type(4)));
+typedef unsigned plh_u4w_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef float plh_f4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef long long plh_l2_a8 __attribute__((ext_vector_type(2), aligned(8)));
+template <> struct Pack<float, 4> {
+    typedef plh_u4w Raw;
+    static __device__ __forceinline__ Raw load(const float *p) {
+        const plh_u4w_a4 t = __builtin_nontemporal_load(reinterpret_cast<const plh_u4w_a4 *>(p));
+        return Raw{t.x, t.y, t.z, t.w};
+    }
+    static __device__ __forceinline__ void store(float *p, Raw r) {
+        __builtin_nontemporal_store(plh_u4w_a4{r.x, r.y, r.z, r.w}, reinterpret_cast<plh_u4w_a4 *>(p));
+    }
+    static __device__ __forceinline__ float get(Raw r, int k) { return bits_f32(k == 0 ? r.x : (k == 1 ? r.y : (k == 2 ? r.z : r.w))); }
+    static __device__ __forceinline__ Raw put(const float (&g)[4]) {
+        return Raw{f32_bits(g[0]), f32_bits(g[1]), f32_bits(g[2]), f32_bits(g[3])};
+    }
+    static constexpr int kStep = 1;
+    static __device__ __forceinline__ void set(Raw &r, int k, const float (&g)[1]) {
+        if (k == 0) r.x = f32_bits(g[0]);
+        else if (k == 1) r.y = f32_bits(g[0]);
+        else if (k == 2) r.z = f32_bits(g[0]);
+        else r.w = f32_bits(g[0]);
+    }
+    static __device__ __forceinline__ Raw mask(const unsigned (&keep)[4]) { return Raw{keep[0], keep[1], keep[2], keep[3]}; }
+};
 template <> struct Pack<float, 1> {
     typedef unsigned Raw;
     static __device__ __forceinline__ Raw load(const float *p) {
@@ -541,17 +569,52 @@ __device__ __forceinline__ plh_u4 rows_gather16(const Word *tile, int e) {
     return plh_u4{d[0], d[1], d[2], d[3]};
 }
 
-template <int V, bool Uniform>
+//   per image - (Form == kPerImage) tiles that never straddle two images whatever m_size is: the grid is
+//              (images) x (tiles per image), a lane takes V consecutive pixels of ONE image and the last
+//              lane of an image may hold fewer (`nv`); its accesses then go pixel by pixel, and the pixels
+//              it does not have read as ignored. Channel planes of odd length (513 x 513, 769 x 769 crops)
+//              start on 4-byte boundaries only, which would leave one pixel per lane and 256-byte runs of
+//              which every third cache line is shared with a neighbour; V = 4 with 16-byte accesses on
+//              4-byte boundaries makes that every ninth.
+constexpr int kGeneral = 0, kUniform = 1, kPerImage = 2;
+
+// Grid of the per-image form.
+template <int V>
+inline unsigned image_grid(int64_t n_size, int64_t m_size) {
+    return (unsigned)(n_size * ceil_div(m_size, (int64_t)kRegsBlock * V));
+}
+
+// Where the host picks it over one pixel per lane: planes long enough that the partly filled last
+// block of every image is a small share, and slices that four pixels per lane still keep in registers.
+constexpr int kImageFormMaxChannels = 24;
+inline bool image_form_pays(int C, int64_t m_size) { return C <= kImageFormMaxChannels && m_size >= 4096; }
+
+template <int V, int Form>
 struct PixelRef {
+    static constexpr bool Uniform = (Form == kUniform);
     int64_t pix;        // first pixel of this thread (index into labels / losses)
     int64_t base;       // block-uniform part of the channel-0 offset (Uniform) or the whole of it
     unsigned lane_off;  // 32-bit per-thread part (Uniform), else 0
     bool live;
+    int nv;             // per-image form: pixels this lane has (0..V); V in the other forms
     int64_t wave_first; // rows form: the first row of this wavefront, and how many of its 64 rows exist
     int rows_here;
 
     __device__ __forceinline__ PixelRef(int64_t P, int64_t m_size, int C, unsigned xcd_run) {
-        if constexpr (Uniform) {
+        nv = V;
+        if constexpr (Form == kPerImage) {
+            const int64_t tiles = ceil_div_dev(m_size, (int64_t)kRegsBlock * V);
+            const int64_t b = tile_of_block(xcd_run);
+            const int64_t n = b / tiles;                        // block-uniform
+            const int64_t local = ((b - n * tiles) * kRegsBlock + threadIdx.x) * V;
+            const int64_t left = m_size - local;
+            nv = left >= V ? V : (left > 0 ? (int)left : 0);
+            live = nv > 0;
+            const int64_t safe = live ? local : 0;
+            pix = n * m_size + safe;
+            base = n * (int64_t)C * m_size + safe;
+            lane_off = 0;
+        } else if constexpr (Uniform) {
             const int64_t start = tile_of_block(xcd_run) * (kRegsBlock * V);
             const int64_t n = start / m_size;
             lane_off = threadIdx.x * V;
@@ -574,7 +637,68 @@ struct PixelRef {
         }
     }
     // (N, C) input with more than one channel: the rows form
-    static __device__ __forceinline__ bool rows_form(int C, int64_t m_size) { return V == 1 && !Uniform && m_size == 1 && C > 1; }
+    static __device__ __forceinline__ bool rows_form(int C, int64_t m_size) { return V == 1 && Form == kGeneral && m_size == 1 && C > 1; }
+
+    // Labels, per-pixel fp32 outputs and the upstream gradient of this thread's pixels. In the per-image
+    // form a lane with fewer than V pixels goes pixel by pixel and reads `ignore` for those it lacks.
+    __device__ __forceinline__ void labels(const int64_t *lab, int64_t ignore, int64_t (&lb)[V]) const {
+        if constexpr (Form == kPerImage) {
+            if (nv == V) {
+#pragma unroll
+                for (int k = 0; k < V; k += 2) {
+                    const plh_l2_a8 t = __builtin_nontemporal_load(reinterpret_cast<const plh_l2_a8 *>(lab + pix + k));
+                    lb[k] = t.x; lb[k + 1] = t.y;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; ++k) lb[k] = k < nv ? lab[pix + k] : ignore;
+            }
+        } else {
+            load_labels<V>(lab + pix, lb);
+        }
+    }
+    __device__ __forceinline__ void store_f32(float *out, const float (&v)[V]) const {
+        if constexpr (Form == kPerImage) {
+            if (nv == V) {
+                __builtin_nontemporal_store(plh_f4_a4{v[0], v[1], v[2], v[3]}, reinterpret_cast<plh_f4_a4 *>(out + pix));
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; ++k)
+                    if (k < nv) out[pix + k] = v[k];
+            }
+        } else {
+            store_vec<V>(out + pix, v);
+        }
+    }
+    // the same through the cache (an output that a later kernel of the same call reads)
+    __device__ __forceinline__ void store_f32_cached(float *out, const float (&v)[V]) const {
+        if constexpr (Form == kPerImage) {
+            if (nv == V) {
+                *reinterpret_cast<plh_f4_a4 *>(out + pix) = plh_f4_a4{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; ++k)
+                    if (k < nv) out[pix + k] = v[k];
+            }
+        } else {
+            store_vec_cached<V>(out + pix, v);
+        }
+    }
+    __device__ __forceinline__ void upstream(const Upstream &up, float (&go)[V]) const {
+        if constexpr (Form == kPerImage) {
+            if (up.gout != nullptr && up.stride != 0) {
+                if (nv == V) {
+                    const plh_f4_a4 t = __builtin_nontemporal_load(reinterpret_cast<const plh_f4_a4 *>(up.gout + pix));
+                    go[0] = t.x; go[1] = t.y; go[2] = t.z; go[3] = t.w;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < V; ++k) go[k] = k < nv ? up.gout[pix + k] : 0.f;
+                }
+                return;
+            }
+        }
+        load_upstream<V>(up, pix, go);
+    }
 
     template <class T>
     static __device__ __forceinline__ typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type *rows_tile() {
@@ -664,6 +788,19 @@ struct PixelRef {
                     return;
                 }
             }
+            if constexpr (Form == kPerImage) {
+                if (nv < V) {                       // the last lane of an image (or a lane beyond it: zeros)
+#pragma unroll
+                    for (int j = 0; j < CP; ++j)
+                        if (chan_ok<CP>(j, C)) {
+                            float one[V];
+#pragma unroll
+                            for (int k = 0; k < V; ++k) one[k] = k < nv ? load_one(chan(t, j, m_size) + k) : 0.f;
+                            raw[j] = Pack<T, V>::put(one);
+                        }
+                    return;
+                }
+            }
 #pragma unroll
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, C)) raw[j] = Pack<T, V>::load(chan(t, j, m_size));
@@ -683,6 +820,18 @@ struct PixelRef {
             if constexpr (V == 1) {
                 if (rows_form(C, m_size)) {         // kernel-uniform
                     rows_store<T, CP>(t, C, raw);
+                    return;
+                }
+            }
+            if constexpr (Form == kPerImage) {
+                if (nv < V) {
+#pragma unroll
+                    for (int j = 0; j < CP; ++j)
+                        if (chan_ok<CP>(j, C)) {
+#pragma unroll
+                            for (int k = 0; k < V; ++k)
+                                if (k < nv) store_one(chan(t, j, m_size) + k, Pack<T, V>::get(raw[j], k));
+                        }
                     return;
                 }
             }

@@ -109,6 +109,11 @@ SEG_CASES = [
     ((1, 449, 8, 8), 255, 0.1),
     ((1, 512, 8, 8), 255, 0.1),
     ((1, 513, 8, 8), 255, 0.1),                     # one channel more: a lane per pixel
+    ((2, 19, 65, 65), 255, 0.05),                   # fp32 planes of odd length, 4096 pixels or more: tiles per
+    ((3, 5, 71, 61), -100, 0.1),                    #   image, 4 pixels per lane; the last lane of an image holds
+    ((2, 24, 4097, 1), 255, 0.1),                   #   1 or 3 pixels; the widest slice that takes this form,
+    ((1, 25, 65, 65), 255, 0.1),                    #   one channel more and one pixel fewer than its limits
+    ((2, 24, 63, 65), 255, 0.1),
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
