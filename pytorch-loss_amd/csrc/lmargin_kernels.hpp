@@ -56,8 +56,12 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     float go[V];
     if constexpr (WantGrad) at.upstream(up, go);
 
+    // Four pixels per lane: a pixel's gradient takes the place of its logits in the slice as soon as it
+    // is formed, and the pixels are worked through one after the other (no second array, no four
+    // pixels' intermediates alive at once).
+    constexpr bool kInPlace = (Form == kPerImage);
     float out[V], score[V];
-    float g[WantGrad ? CP : 1][V];
+    float g[(WantGrad && !kInPlace) ? CP : 1][V];
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
     unsigned n_valid = 0;
     float mine = 0.f;
@@ -114,6 +118,9 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
             score[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
+            // formed here: left to itself the compiler moves a pixel's whole reduction down to the guarded
+            // stores at the end and keeps every pixel's exponentials alive until then
+            asm volatile("" : "+v"(out[k]), "+v"(score[k]));
             mine += out[k];
             cnt += (ign || !live) ? 0 : 1;
         }
@@ -134,10 +141,18 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                 if (chan_ok<CP>(j, p.C)) {
                     const float w = __builtin_fmaf(Pack<T, V>::get(raw[j], k), B, A);
                     const float gj = __builtin_fmaf(xv[j], w, nK);
-                    g[j][k] = (tgt == j) ? g_hot : gj;
+                    float gv = (tgt == j) ? g_hot : gj;
+                    asm volatile("" : "+v"(gv));        // formed here, not down at the guarded stores
+                    if constexpr (kInPlace) {
+                        const float one[1] = {gv};
+                        Pack<T, V>::set(raw[j], k, one);
+                    } else {
+                        g[j][k] = gv;
+                    }
                 }
         }
         if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
+        if constexpr (kInPlace) __builtin_amdgcn_sched_barrier(0);
     }
     if (live) {
         if (WantLoss && loss) at.store_f32(loss, out);
@@ -147,7 +162,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(g[j]) & mask;
+                if (chan_ok<CP>(j, p.C)) {
+                    if constexpr (kInPlace) raw[j] = raw[j] & mask;
+                    else raw[j] = Pack<T, V>::put(g[j]) & mask;
+                }
             at.store_slice(grad, p.C, p.m_size, raw);
         }
     }
