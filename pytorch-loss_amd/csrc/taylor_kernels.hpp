@@ -73,26 +73,33 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
-    float y[CP][V];
+    // a pixel's results replace its inputs in the slice as soon as they are formed (one pixel at a time
+    // for fp32, two for 16-bit elements, which share a dword): no second array
+    using PK = Pack<T, V>;
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-        float s = 0.f;
+    for (int k0 = 0; k0 < V; k0 += PK::kStep) {
+        float y[CP][PK::kStep];
+#pragma unroll
+        for (int kk = 0; kk < PK::kStep; ++kk) {
+            const int k = k0 + kk;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, p.C)) {
+                    float f, df;
+                    taylor_pair(PK::get(raw[j], k), p.order, f, df);
+                    y[j][kk] = f;
+                    s += f;
+                }
+            const float inv = 1.f / s, ls = logf(s);
+#pragma unroll
+            for (int j = 0; j < CP; ++j)
+                if (chan_ok<CP>(j, p.C)) y[j][kk] = p.use_log ? logf(y[j][kk]) - ls : y[j][kk] * inv;
+        }
 #pragma unroll
         for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) {
-                float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
-                y[j][k] = f;
-                s += f;
-            }
-        const float inv = 1.f / s, ls = logf(s);
-#pragma unroll
-        for (int j = 0; j < CP; ++j)
-            if (chan_ok<CP>(j, p.C)) y[j][k] = p.use_log ? logf(y[j][k]) - ls : y[j][k] * inv;
+            if (chan_ok<CP>(j, p.C)) PK::set(raw[j], k0 / PK::kStep, y[j]);
     }
-#pragma unroll
-    for (int j = 0; j < CP; ++j)
-        if (chan_ok<CP>(j, p.C)) raw[j] = Pack<T, V>::put(y[j]);
     at.store_slice(out, p.C, p.m_size, raw);
 }
 
@@ -140,6 +147,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
                 r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
             }
             raw[j] = Pack<T, V>::put(r);
+            forget_origin(raw[j]);      // packed here, channel by channel: nothing of the sweep waits for the stores
         }
     at.store_slice(gx, p.C, p.m_size, raw);
 }
@@ -238,6 +246,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
                 r[k] = df * ((tgt[k] == j) ? hot[k] : scale[k]);
             }
             raw[j] = Pack<T, V>::put(r) & mask;
+            forget_origin(raw[j]);      // packed here, channel by channel: nothing of the sweep waits for the stores
         }
     at.store_slice(gx, p.C, p.m_size, raw);
 }
