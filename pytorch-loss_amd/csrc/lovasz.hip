@@ -270,8 +270,8 @@ __device__ __forceinline__ int row_items(const SortArgs &a, int c) { return a.ke
 // one sector) and the sectors in which one tile's run of a digit ends and the next tile's begins.
 // Only the tiles that hold keys are permuted (the rest of a pruned row exits at once, and would
 // leave the XCDs of the last chunks idle).
-__device__ __forceinline__ int sort_tile(int items) {
-    const int x = blockIdx.x, q = ((items + kSortTile - 1) / kSortTile) >> 3;
+__device__ __forceinline__ int sort_tile(int items, int tile_keys = kSortTile) {
+    const int x = blockIdx.x, q = ((items + tile_keys - 1) / tile_keys) >> 3;
     return x < 8 * q ? (x & 7) * q + (x >> 3) : x;
 }
 
@@ -428,18 +428,24 @@ __device__ __forceinline__ LastPassRows last_pass_rows(const SortArgs &a, int pa
 // group of equal digits, found through the match mask, adds the group.
 template <bool Top>
 __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) {
+    // A block counts two neighbouring tiles, the first with its wavefronts 0..3 and the second with 4..7: twice
+    // the loads in flight per block and half the blocks (a block of one tile spends most of its life waiting
+    // for its 8 loads per lane), and the two table words of a digit leave in one 8-byte store.
+    constexpr int kPair = 2, kItems = kPair * kSortItems, kWavesPerTile = kSortWaves / kPair;
     __shared__ uint32_t counts[kSortWaves][kRadix];
     __shared__ uint32_t counts_hot[Top ? kSortWaves : 1][kRadix];
-    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
+    const int c = blockIdx.y, pair = sort_tile(row_items(a, c), kPair * kSortTile);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const DigitPlan dp = digit_plan(a.key_bits[c], Top ? kLastPass : a.pass);
     if (!Top && a.pass >= dp.passes - 1) return;        // block-uniform: this class has fewer scatter passes
-    const int begin = tile * kSortTile;
-    const int count = min(kSortTile, row_items(a, c) - begin);
-    if (count <= 0) {                           // block-uniform: the row ends before this tile; lov_row_scan
-        if (threadIdx.x <= dp.mask) {           // reads the live tiles in whole groups of kSortWaves
-            a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile] = 0;
-            if constexpr (Top) a.tile_hot[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile] = 0;
+    const int begin = pair * (kPair * kSortTile);
+    const int count = min(kPair * kSortTile, row_items(a, c) - begin);
+    const int64_t cell = ((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + kPair * pair;
+    const bool in_table = kPair * pair < a.tiles_pad;   // the grid covers the padded row in pairs: it may end one pair late
+    if (count <= 0) {                           // block-uniform: the row ends before these tiles; lov_row_scan
+        if (threadIdx.x <= dp.mask && in_table) {       // reads the live tiles in whole groups of kSortWaves
+            *reinterpret_cast<uint2 *>(a.tile_hist + cell) = make_uint2(0u, 0u);
+            if constexpr (Top) *reinterpret_cast<uint2 *>(a.tile_hot + cell) = make_uint2(0u, 0u);
         }
         return;
     }
@@ -450,16 +456,16 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
     const uint32_t limit = keep_limit(a, c);
     const uint32_t *rows = Top ? last_pass_rows(a, dp.passes).keys : a.keys_in;
     const uint32_t *kin = rows + (int64_t)c * a.P + begin;
-    uint32_t key[kSortItems];
+    uint32_t key[kItems];
 #pragma unroll
-    for (int r = 0; r < kSortItems; ++r) {      // all loads in flight before the first one is used
-        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+    for (int r = 0; r < kItems; ++r) {          // all loads in flight before the first one is used
+        const int li = wave * (kItems * kWave) + r * kWave + lane;
         key[r] = (li < count) ? kin[li] : kIgnoredKey;
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < kSortItems; ++r) {
-        const int li = wave * (kSortItems * kWave) + r * kWave + lane;
+    for (int r = 0; r < kItems; ++r) {
+        const int li = wave * (kItems * kWave) + r * kWave + lane;
         const bool valid = li < count && keep_key(key[r], limit);
         const uint32_t digit = (key[r] >> dp.shift) & dp.mask;
         const uint64_t vmask = __builtin_amdgcn_ballot_w64(valid);
@@ -483,14 +489,14 @@ __global__ __launch_bounds__(kSortThreads) void lov_tile_hist(const SortArgs a) 
     __syncthreads();
     if (threadIdx.x <= dp.mask) {
         const int d = threadIdx.x;
-        uint32_t n = 0, nh = 0;
+        uint32_t n[kPair] = {0, 0}, nh[kPair] = {0, 0};
 #pragma unroll
         for (int w = 0; w < kSortWaves; ++w) {
-            n += counts[w][d];
-            if constexpr (Top) nh += counts_hot[w][d];
+            n[w / kWavesPerTile] += counts[w][d];
+            if constexpr (Top) nh[w / kWavesPerTile] += counts_hot[w][d];
         }
-        a.tile_hist[((int64_t)c * kRadix + d) * a.tiles_pad + tile] = n;
-        if constexpr (Top) a.tile_hot[((int64_t)c * kRadix + d) * a.tiles_pad + tile] = nh;
+        *reinterpret_cast<uint2 *>(a.tile_hist + cell) = make_uint2(n[0], n[1]);
+        if constexpr (Top) *reinterpret_cast<uint2 *>(a.tile_hot + cell) = make_uint2(nh[0], nh[1]);
     }
 }
 
@@ -1126,7 +1132,8 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     //    difference is known to be 0 (keep_key) and counts what is left per class; the later passes
     //    work on those counts and their surplus blocks return at once.
     const dim3 tile_grid((unsigned)pl.tiles, (unsigned)C);
-    const dim3 hist_grid((unsigned)pl.tiles_pad, (unsigned)C);      // lov_row_scan reads the live tiles in whole groups of kSortWaves
+    // a histogram block counts two tiles; lov_row_scan reads the live tiles in whole groups of kSortWaves
+    const dim3 hist_grid((unsigned)round_up(ceil_div(pl.tiles, 2), kSortWaves / 2), (unsigned)C);
     SortArgs a;
     a.keys_alt = nullptr;
     a.vals_alt = nullptr;
