@@ -37,15 +37,16 @@ HBM_PEAK_GBPS = 8000.0
 # what the same counters read for the plain copy kernel): see profiles/*_hbm_traffic.txt.
 # Only valid for the exact workload shape they were taken on; anything else reports null.
 MEASURED_TRAFFIC = {
-    ("lsr", (8, 19, 1024, 1024)): {"forward": 704.8e6 + 33.6e6, "backward": 735.0e6 + 637.5e6},
-    # profiles/all_workloads_hbm_traffic.txt (KiB per dispatch x 1024; kernels launched with both kinds of
-    # upstream gradient are scaled from the dispatch-weighted average to the per-element launch timed here)
-    ("lmargin", (8, 19, 1024, 1024)): {"forward": (688217 + 32768) * 1024, "backward": (721019 + 622597) * 1024},
-    ("taylor", (8, 19, 1024, 1024)): {"forward": (688318 + 32768) * 1024, "backward": (721267 + 622674) * 1024},
-    ("focal", (16, 80, 128, 128)): {"forward": (163862 + 81920) * 1024, "backward": (245815 + 81920) * 1024},
-    ("dice", (64, 1, 1024, 1024)): {"forward": (524531 + 32) * 1024, "backward": (524369 + 262151) * 1024},
-    ("layernorm", (16, 256, 128, 128)): {"forward": (262298 + 262197) * 1024, "backward": (524469 + 262173) * 1024},
-    ("lovasz", (4, 19, 512, 1024)): {"backward": (327860 + 155681) * 1024},
+    # profiles/lsr_8x19x1024x1024_hbm_traffic.txt and profiles/all_workloads_hbm_traffic.txt (KiB per dispatch x 1024;
+    # for kernels launched with both kinds of upstream gradient, the launches with one value per loss element,
+    # which are the ones timed here: the largest FETCH_SIZE of the run)
+    ("lsr", (8, 19, 1024, 1024)): {"forward": (688199 + 32768) * 1024, "backward": (720985 + 622623) * 1024},
+    ("lmargin", (8, 19, 1024, 1024)): {"forward": (688218 + 32768) * 1024, "backward": (721014 + 622648) * 1024},
+    ("taylor", (8, 19, 1024, 1024)): {"forward": (688322 + 32768) * 1024, "backward": (721261 + 622847) * 1024},
+    ("focal", (16, 80, 128, 128)): {"forward": (163862 + 81921) * 1024, "backward": (245799 + 81920) * 1024},
+    ("dice", (64, 1, 1024, 1024)): {"forward": (524418 + 32) * 1024, "backward": (524377 + 262148) * 1024},
+    ("layernorm", (16, 256, 128, 128)): {"forward": (262290 + 262221) * 1024, "backward": (524484 + 262176) * 1024},
+    ("lovasz", (4, 19, 512, 1024)): {"forward": 2391274 * 1024, "backward": (327869 + 155670) * 1024},
 }
 
 WORKLOADS = {
