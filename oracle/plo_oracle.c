@@ -5,8 +5,9 @@
  * LovaszSoftmax and the ops next to them (OHEM relabelling, one-hot, Taylor softmax,
  * soft dice, channel layer norm), used by the tests as the parity checker and by the benchmark's
  * cpu_baseline leg. Every function in oracle_body.inc cites the reference lines
- * it follows. One function is PARITY UNPINNED: oracle_layer_norm_backward (see its
- * comment). Built by oracle/build.py into oracle/liboracle.so.
+ * it follows and is pinned by tests/test_oracle_*.py without the reference (library
+ * routines, closed forms, brute force, known answers worked by hand). Built by
+ * oracle/build.py into oracle/liboracle.so.
  *
  * Each function exists as <name>_f32 (the arithmetic type of the shipped path)
  * and <name>_f64 (a higher-precision check on the fp32 restatement itself).
