@@ -45,6 +45,20 @@ def test_function_matches_oracle(pl, shape):
     assert err <= 1e-5 * np.abs(want_g).max(), (err, np.abs(want_g).max())
 
 
+def test_backward_known_answers(pl):
+    """The hand-worked values of csrc/layer_norm.cu:214 that pin the oracle (tests/test_oracle_layernorm.py),
+    straight through the HIP path: pixels (1,3), (0,2), (3,1) at eps = 0 and the constant pixel (2,2) at eps = 1/4."""
+    x = torch.tensor([[[1.0, 0.0], [3.0, 2.0]], [[3.0, 2.0], [1.0, 2.0]]], device="cuda")
+    for eps, want in ((0.0, {(0, 0): (0.5, -5.5), (0, 1): (-1.0, -2.0), (1, 0): (-5.5, 0.5)}),
+                      (0.25, {(1, 1): (-1.0, -1.0)}),
+                      (3.0, {(0, 0): (1.75, -10.25), (1, 0): (-10.25, 1.75)})):
+        xt = x.clone().requires_grad_()
+        pl.LayerNormV3Func.apply(xt, eps).backward(torch.ones_like(x))
+        got = xt.grad.cpu().numpy()
+        for (n, m), chans in want.items():
+            np.testing.assert_allclose(got[n, :, m], np.array(chans), rtol=2e-6, err_msg=str((eps, n, m)))
+
+
 def test_large_common_offset_keeps_accuracy(pl):
     x = synth.normal(122, 1, (2, 64, 256), 1000.0, 0.5)
     out = pl.LayerNormV3Func.apply(torch.from_numpy(x).cuda(), 1e-6).cpu().numpy()
