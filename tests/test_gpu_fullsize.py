@@ -81,6 +81,47 @@ def test_channel_softmax_losses_full_size(pl, name):
     assert abs(total.item() - ref_total) <= 1e-5 * abs(ref_total)
 
 
+@pytest.mark.parametrize("kind,shape", [("lsr", (6, 19, 769, 769)), ("lmargin", (9, 19, 513, 513)), ("lsr", (3, 21, 1023, 1025))])
+def test_odd_crops_full_size(pl, kind, shape):
+    """fp32 channel planes of odd length take tiles per image with four pixels per lane (every image ends in a
+    partly filled lane, every plane starts at another offset into a cache line): the same properties as above at
+    crop sizes segmentation trains on, the oracle on the last image, and no dependence on the batch position."""
+    x = synth.normal(31, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(31, shape[:1] + shape[2:], shape[1], 255, 0.05)
+    xt = torch.from_numpy(x).cuda().requires_grad_()
+    yt = torch.from_numpy(y).cuda()
+    if kind == "lsr":
+        make = lambda red: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=255)
+        o_fwd = lambda a, b: oracle.lsr_forward(a, b, 255, 0.1)
+        o_bwd = lambda a, b, g: oracle.lsr_backward(a, b, 255, 0.1, g)
+    else:
+        make = lambda red: pl.LargeMarginSoftmaxV3(lam=0.3, reduction=red, ignore_index=255)
+        o_fwd = lambda a, b: oracle.lmargin_forward(a, b, 0.3, 255)
+        o_bwd = lambda a, b, g: oracle.lmargin_backward(a, b, 0.3, 255, g)
+    n_valid = int((y != 255).sum())
+    mean = make("mean")(xt, yt)
+    mean.backward()
+    g_mean = xt.grad.clone()
+    xt.grad = None
+    per = make("none")(xt, yt)
+    per.sum().backward()
+    g_sum = xt.grad.clone()
+    assert abs(mean.item() - per.double().sum().item() / n_valid) <= 1e-6 * abs(mean.item())
+    ign = yt == 255
+    assert (per[ign] == 0).all() and (per[~ign] > 0).all()
+    assert (g_sum.permute(0, 2, 3, 1)[ign] == 0).all()
+    assert g_sum.sum(dim=1).abs().max().item() < 1e-5
+    assert (g_mean * n_valid - g_sum).abs().max().item() < 1e-5
+    k = shape[0] - 1                                # the last image: its last lane is the last of the tensor
+    want = o_fwd(x[k:k + 1], y[k:k + 1])
+    got = per[k:k + 1].detach().cpu().numpy()
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6)
+    err = np.abs(g_sum[k:k + 1].cpu().numpy() - o_bwd(x[k:k + 1], y[k:k + 1], None)).max()
+    assert err <= 1e-5, err
+    alone = make("none")(xt[k:k + 1].detach().contiguous(), yt[k:k + 1].contiguous())
+    assert torch.equal(alone, per[k:k + 1].detach())
+
+
 def test_focal_full_size(pl):
     w = synth.workload("cfg3")
     x, y = w["logits"], w["labels"]
