@@ -522,8 +522,21 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true);
-        if (shape == Shape::Split) {
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true, true);
+        if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
+            constexpr int VD = VT / 2;
+            const unsigned grid = split_grid<VD>(P);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
+            switch (split_slots_deep(dimsize)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        hipLaunchKernelGGL((ohem_scores_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, ce, \
+                           P, m_size, C, ignore_index, run, tables);                                                  \
+        break;
+                PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+            }
+        } else if (shape == Shape::Split) {
             const unsigned grid = split_grid<VT>(P);
             const unsigned run = xcd_run_for(sizeof(T), m_size);
             switch (split_slots(dimsize)) {

@@ -698,8 +698,26 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
     constexpr bool kHasSplit = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);
     const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
-                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit);
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit, kHasSplit);
     if constexpr (kHasSplit) {
+        if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
+            constexpr int VD = VT / 2;
+            const unsigned grid = split_grid<VD>(p.P);
+            switch (split_slots_deep(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (Kind == kTaylorCeFwd)                                                                           \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VD, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+                               loss, part, p);                                                                        \
+        else                                                                                                          \
+            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
+                               p);                                                                                    \
+        break;
+                PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+            }
+            return grid;
+        }
         if (shape == Shape::Split) {
             const unsigned grid = split_grid<VT>(p.P);
             switch (split_slots(p.C)) {

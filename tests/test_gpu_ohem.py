@@ -54,6 +54,11 @@ SCORE_CASES = [
     ((2, 65, 8, 8), 255, 0.1),
     ((1, 133, 8, 8), 255, 0.1),
     ((1, 171, 8, 8), 255, 0.1),
+    ((2, 257, 8, 8), 255, 0.1),          # 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
+    ((1, 300, 9, 8), 255, 0.1),
+    ((1, 449, 8, 8), -100, 0.2),
+    ((1, 512, 8, 9), 255, 0.1),
+    ((1, 513, 8, 8), 255, 0.1),          # one channel more: a lane per pixel
     ((2, 19, 16, 16), 255, 1.0),         # everything ignored
 ]
 
