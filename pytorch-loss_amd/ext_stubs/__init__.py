@@ -1,7 +1,9 @@
-"""Stand-ins for the reference's four pybind11 extension modules, bound to libpytorch_loss_hip.so.
+"""Stand-ins for the reference's pybind11 extension modules of the fused-loss path and the ops next to
+it, bound to libpytorch_loss_hip.so.
 
 The reference's Python files import one CUDA extension per op at module level (`import lsr_cpp`,
-pytorch_loss/label_smooth.py:125; `focal_cpp`, `large_margin_cpp`, `lovasz_softmax_cpp` likewise).
+pytorch_loss/label_smooth.py:125; `focal_cpp`, `large_margin_cpp`, `lovasz_softmax_cpp`, `ohem_cpp`,
+`one_hot_cpp`, `taylor_softmax_cpp`, `soft_dice_cpp`, `layer_norm_cpp` likewise; setup.py:13-45 names them).
 Each module here carries the same function names with the same positional arguments and return
 values as the extension it replaces, so those files run unchanged once `install()` has put the
 stand-ins into `sys.modules` (or this directory is on `sys.path` ahead of the built extensions):
@@ -16,7 +18,8 @@ They are plain ctypes over the C ABI of include/pytorch_loss_hip.h and use nothi
 import importlib
 import sys
 
-NAMES = ("lsr_cpp", "focal_cpp", "large_margin_cpp", "lovasz_softmax_cpp")
+NAMES = ("lsr_cpp", "focal_cpp", "large_margin_cpp", "lovasz_softmax_cpp",
+         "ohem_cpp", "one_hot_cpp", "taylor_softmax_cpp", "soft_dice_cpp", "layer_norm_cpp")
 
 
 def install():

@@ -1,4 +1,4 @@
-"""What the four stand-in modules share: the loaded library, element-type tags, shape flattening
+"""What the stand-in modules share: the loaded library, element-type tags, shape flattening
 and the mapping of return codes to RuntimeError (the reference raises through AT_ERROR / AT_ASSERTM)."""
 import ctypes
 import os

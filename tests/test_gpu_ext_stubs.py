@@ -1,9 +1,12 @@
-"""The binding a maintainer of the reference would add: stand-in modules named like the reference's four
+"""The binding a maintainer of the reference would add: stand-in modules named like the reference's
 extensions (pytorch-loss_amd/ext_stubs), registered under those names and called with the extensions' exact
 signatures (csrc/lsr_kernel.cu:319-322, csrc/focal_kernel.cu:337-341, csrc/large_margin_kernel.cu:834-838,
-csrc/lovasz_softmax.cu:799-802), the way the reference's autograd Functions call them
+csrc/lovasz_softmax.cu:799-802; the ops next to the path: csrc/ohem_label_kernel.cu:279-281,
+csrc/one_hot_kernel.cu:351-353, csrc/taylor_softmax.cu:419-422, csrc/soft_dice_kernel_v2.cu:434-437,
+csrc/layer_norm.cu:390-393), the way the reference's autograd Functions call them
 (pytorch_loss/label_smooth.py:131-145, focal_loss.py:129-171, large_margin_softmax.py:146-193,
-pytorch_loss/lovasz_softmax.py:75-91). Results against the CPU oracle to the usual bars."""
+pytorch_loss/lovasz_softmax.py:75-91, ohem_loss.py:24, one_hot.py:54, taylor_softmax.py:25-34,
+soft_dice_loss.py:153-164, layer_norm.py:150-160). Results against the CPU oracle to the usual bars."""
 import sys
 
 import numpy as np
@@ -120,3 +123,90 @@ def test_lovasz_softmax_cpp(ext):
     with pytest.raises(RuntimeError, match="512"):
         lovasz_softmax_cpp.lovasz_softmax_forward(torch.zeros((1, 512, 2), device="cuda"),
                                                   torch.zeros((1, 2), dtype=torch.int64, device="cuda"), 255)
+
+
+def test_neighbouring_modules_are_importable_under_the_reference_names(ext):
+    import layer_norm_cpp
+    import ohem_cpp
+    import one_hot_cpp
+    import soft_dice_cpp
+    import taylor_softmax_cpp
+    assert ohem_cpp is ext["ohem_cpp"] and callable(ohem_cpp.score_ohem_label) and callable(one_hot_cpp.label_one_hot)
+    assert {"taylor_softmax_forward", "taylor_softmax_backward"} <= set(dir(taylor_softmax_cpp))
+    assert {"soft_dice_forward", "soft_dice_backward"} <= set(dir(soft_dice_cpp))
+    assert {"layer_norm_forward", "layer_norm_backward"} <= set(dir(layer_norm_cpp))
+
+
+@pytest.mark.parametrize("shape", [(2, 19, 32, 32), (3, 7, 5, 9), (50, 10)])
+def test_ohem_cpp(ext, shape):
+    import ohem_cpp
+    x, y = seg(95, shape, 255)
+    xt, yt = dev(x), dev(y)
+    n_min = y.size // 8
+    got = ohem_cpp.score_ohem_label(xt, yt, 255, 0.7, n_min)               # ohem_loss.py:24
+    assert got.shape == yt.shape and got.dtype == torch.int64 and torch.equal(yt, dev(y))
+    s = oracle.ohem_scores(x, y, 255)
+    want = oracle.ohem_select(s, y, 255, 0.7, n_min)
+    differ = got.cpu().numpy() != want
+    flat = np.sort(s.ravel())
+    near = (np.abs(s - np.float32(0.7)) <= 2e-6) | (np.abs(s - flat[n_min - 1]) <= 2e-6)
+    assert not (differ & ~near).any(), int(differ.sum())
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        ohem_cpp.score_ohem_label(xt.cpu(), yt.cpu(), 255, 0.7, n_min)
+
+
+def test_one_hot_cpp(ext):
+    import one_hot_cpp
+    y = synth.seg_labels(96, (3, 9, 11), 19, 255, 0.1)
+    got = one_hot_cpp.label_one_hot(dev(y), 255, 0.1, 19)                  # one_hot.py:54
+    assert got.shape == (3, 19, 9, 11) and got.dtype == torch.float32
+    assert np.array_equal(got.cpu().numpy(), oracle.onehot(y, 19, 0.1, 255))
+    with pytest.raises(RuntimeError, match="less than min_len"):
+        one_hot_cpp.label_one_hot(dev(y), 255, 0.1, 10)
+    with pytest.raises(RuntimeError, match="only supports gpu mode"):
+        one_hot_cpp.label_one_hot(torch.from_numpy(y), 255, 0.1, 19)
+
+
+@pytest.mark.parametrize("use_log", [False, True])
+@pytest.mark.parametrize("shape,dim", [((2, 19, 16, 17), 1), ((30, 100), 1), ((4, 6, 10), 2)])
+def test_taylor_softmax_cpp(ext, shape, dim, use_log):
+    import taylor_softmax_cpp
+    x = synth.normal(97, 1, shape, 0.0, 1.0)
+    g = synth.normal(97, 2, shape, 0.0, 1.0)
+    out = taylor_softmax_cpp.taylor_softmax_forward(dev(x), dim, 4, use_log)          # taylor_softmax.py:25
+    want = oracle.taylor_forward(x.astype(np.float64), dim, 4, use_log)
+    assert out.shape == x.shape and np.abs(out.cpu().numpy() - want).max() <= 1e-5
+    grad = taylor_softmax_cpp.taylor_softmax_backward(dev(g), dev(x), dim, 4, use_log)   # taylor_softmax.py:34
+    want_g = oracle.taylor_backward(g.astype(np.float64), x.astype(np.float64), dim, 4, use_log)
+    assert np.abs(grad.cpu().numpy() - want_g).max() <= 1e-5 * max(1.0, np.abs(want_g).max())
+
+
+@pytest.mark.parametrize("p,smooth", [(1.0, 1.0), (2.0, 0.5)])
+def test_soft_dice_cpp(ext, p, smooth):
+    import soft_dice_cpp
+    n, length = 5, 3001
+    x = synth.normal(98, 1, (n, length), 0.0, 2.0)
+    y = synth.uniform01(98, 2, n * length).reshape(n, length).astype(np.float32)        # soft labels: q^p + y shows
+    go = synth.normal(98, 3, (n,), 0.5, 1.0)
+    loss = soft_dice_cpp.soft_dice_forward(dev(x), dev(y), p, smooth)                   # soft_dice_loss.py:153
+    want, stats = oracle.soft_dice_forward(x.astype(np.float64), y.astype(np.float64), p, smooth)
+    assert loss.shape == (n,) and np.abs(loss.cpu().numpy() - want).max() <= 1e-5
+    grad = soft_dice_cpp.soft_dice_backward(dev(go), dev(x), dev(y), p, smooth)          # soft_dice_loss.py:164
+    want_g = oracle.soft_dice_backward(go.astype(np.float64), x.astype(np.float64), y.astype(np.float64), stats, p)
+    assert np.abs(grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max() + 1e-12
+
+
+def test_layer_norm_cpp(ext):
+    import layer_norm_cpp
+    shape = (2, 48, 130)
+    x = synth.normal(99, 1, shape, 0.3, 1.5)
+    g = synth.normal(99, 2, shape, 0.0, 1.0)
+    out = layer_norm_cpp.layer_norm_forward(dev(x), 1e-6)                               # layer_norm.py:150
+    assert np.abs(out.cpu().numpy() - oracle.layer_norm_forward(x.astype(np.float64), 1e-6)).max() <= 1e-5
+    grad = layer_norm_cpp.layer_norm_backward(dev(g), dev(x), 1e-6)                     # layer_norm.py:160
+    want_g = oracle.layer_norm_backward(g.astype(np.float64), x.astype(np.float64), 1e-6)
+    assert np.abs(grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max()
+    # the hand-worked values of csrc/layer_norm.cu:214 for the pixel (1, 3) at eps = 0: +1/2 g and -11/2 g
+    two = layer_norm_cpp.layer_norm_backward(torch.ones(1, 2, 1, device="cuda"),
+                                             torch.tensor([[[1.0], [3.0]]], device="cuda"), 0.0)
+    np.testing.assert_allclose(two.cpu().numpy().ravel(), [0.5, -5.5], rtol=2e-6)
