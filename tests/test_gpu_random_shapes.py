@@ -1,12 +1,15 @@
-"""Seeded sweep over small random shapes: every op against the CPU oracle on sizes nobody picked
-by hand (odd extents, one channel, one pixel, tiles that end mid-wave, channel counts on both
-sides of every kernel-shape boundary). Same tolerances as the hand-picked parity tests."""
+"""A seeded sweep over shapes nobody picked by hand: every launch shape has its boundaries in the tables of
+test_gpu_parity.py; this walks random points between them (channel counts 1..600, odd and even planes on both
+sides of the 4096-pixel limit of the per-image form, (N, C) rows up to 6000, all three storage types, the three
+ignore conventions) for the four channel-softmax losses and the OHEM scores, against the CPU oracle to the usual bars."""
 import numpy as np
 import pytest
 import torch
 
 import oracle
 from oracle import synth
+
+from .test_gpu_dtypes import ULP_REL, close_grad_stored
 from .test_gpu_parity import close_grad, close_loss, dev, seg_inputs
 
 pytestmark = pytest.mark.gpu
@@ -20,109 +23,118 @@ def pl():
     return pytorch_loss
 
 
-def _shapes(seed, count, max_c, max_m):
-    rng = np.random.default_rng(seed)
-    out = []
-    for _ in range(count):
-        n = int(rng.integers(1, 4))
-        c = int(rng.choice([1, 2, 3, int(rng.integers(4, max_c + 1))]))
-        m = int(rng.choice([1, 2, int(rng.integers(3, 70)), int(rng.integers(70, max_m + 1))]))
-        out.append((n, c, m))
-    return out
+def _draw(seed):
+    r = np.random.RandomState(1000 + seed)
+    kind = ("lsr", "lmargin", "taylor", "ohem")[seed % 4]
+    family = r.randint(5)
+    if family == 0:            # segmentation, channels in registers
+        shape = (int(r.randint(1, 4)), int(r.randint(1, 33)), int(r.randint(1, 70)), int(r.randint(1, 70)))
+    elif family == 1:          # fp32 planes around the per-image form: odd lengths of 4096 pixels or more, C <= 24 and just above
+        h = int(r.randint(60, 100)) | 1
+        w = int(r.randint(64, 100)) | 1
+        shape = (int(r.randint(1, 4)), int(r.randint(2, 27)), h, w)
+    elif family == 2:          # channels shared out over the wavefronts of a block (33..512) and a lane per pixel beyond
+        shape = (int(r.randint(1, 3)), int(r.randint(33, 600)), int(r.randint(1, 24)), int(r.randint(1, 24)))
+    elif family == 3:          # (N, C) rows: a wavefront or a block per row
+        shape = (int(r.randint(1, 40)), int(r.choice([r.randint(1, 33), r.randint(33, 2049), r.randint(2049, 6000)])))
+    else:                      # 5-D and 3-D inputs
+        shape = (int(r.randint(1, 3)), int(r.randint(2, 80))) + tuple(int(v) for v in r.randint(1, 9, size=int(r.choice([1, 3]))))
+    ignore = int(r.choice([255, -100, 0]))
+    frac = float(r.choice([0.0, 0.1, 0.5]))
+    dt = (torch.float32, torch.float32, torch.bfloat16, torch.float16)[int(r.randint(4))]
+    return kind, shape, ignore, frac, dt
 
 
-@pytest.mark.parametrize("shape", _shapes(1, 24, 40, 700))
-def test_pixel_losses(pl, shape):
-    n, c, m = shape
-    x, y = seg_inputs(200 + n * c * m, (n, c, m), 255, 0.1)
+@pytest.mark.parametrize("seed", range(160))
+def test_random_shape(pl, seed):
+    from pytorch_loss import _native
+    kind, shape, ignore, frac, dt = _draw(seed)
+    if kind == "lmargin" and shape[1] < 2:
+        shape = (shape[0], 2) + shape[2:]           # 1 / (C - 1)
+    x, y = seg_inputs(300 + seed, shape, ignore, frac)
+    xt = dev(x).to(dt)
+    xr = xt.float().cpu().numpy()                   # what the kernels see, widened
     yt = dev(y)
-    go = synth.normal(201, 3, y.shape, 0.0, 1.0)
-    for name, fn, fwd, bwd in (
-            ("lsr", lambda t: pl.LSRCrossEntropyFunctionV3.apply(t, yt, 0.1, 255),
-             lambda: oracle.lsr_forward(x, y, 255, 0.1), lambda: oracle.lsr_backward(x, y, 255, 0.1, go)),
-            ("lmargin", lambda t: pl.LargeMarginSoftmaxFuncV3.apply(t, yt, 0.3, 255),
-             lambda: oracle.lmargin_forward(x, y, 0.3, 255), lambda: oracle.lmargin_backward(x, y, 0.3, 255, go)),
-            ("taylor", lambda t: pl.TaylorCrossEntropyFunctionV3.apply(t, yt, 4, 255, "none"),
-             lambda: oracle.taylor_ce(x, y, 4, 255), lambda: oracle.taylor_ce_backward(x, y, 4, 255, go))):
-        if c == 1 and name == "lmargin":
-            continue    # the margin term carries 1 / (C - 1) (csrc/large_margin_kernel.cu:100): undefined for one class
-        xt = dev(x).requires_grad_()
-        out = fn(xt)
-        if c == 1:      # a single class: every loss is exactly 0; the kernels' exp2/log2 pair leaves ~5e-8
-            assert np.abs(out.detach().cpu().numpy() - fwd()).max() <= 1e-6
+    what = "%s %s %s ignore=%d" % (kind, shape, str(dt)[6:], ignore)
+    if kind == "ohem":
+        got = _native.ohem_scores(xt, yt, ignore).cpu().numpy()
+        assert np.abs(got - oracle.ohem_scores(xr, y, ignore)).max() <= 1e-6, what
+        return
+    xt.requires_grad_()
+    if kind == "lsr":
+        losses = pl.LSRCrossEntropyFunctionV3.apply(xt, yt, 0.1, ignore)
+        want = oracle.lsr_forward(xr, y, ignore, 0.1)
+        grad_of = lambda g: oracle.lsr_backward(xr, y, ignore, 0.1, g)
+    elif kind == "lmargin":
+        losses = pl.LargeMarginSoftmaxFuncV3.apply(xt, yt, 0.3, ignore)
+        want = oracle.lmargin_forward(xr, y, 0.3, ignore)
+        grad_of = lambda g: oracle.lmargin_backward(xr, y, 0.3, ignore, g)
+    else:
+        losses = pl.TaylorCrossEntropyFunctionV3.apply(xt, yt, 4, ignore, "none")
+        want = oracle.taylor_ce(xr.astype(np.float64), y, 4, ignore)
+        grad_of = lambda g: oracle.taylor_ce_backward(xr.astype(np.float64), y, 4, ignore, g.astype(np.float64))
+    assert losses.shape == yt.shape, what
+    got = losses.detach().float().cpu().numpy()
+    if dt == torch.float32:
+        close_loss(got, want, what)
+    else:                                           # losses come back in the storage type: one rounding of it
+        assert np.all(np.abs(got - want) <= ULP_REL[dt] * np.abs(want) + 1e-6), what
+    assert (got[y == ignore] == 0).all(), what
+    go = synth.normal(300 + seed, 3, y.shape, 0.0, 1.0)
+    losses.backward(dev(go).to(losses.dtype))
+    go_seen = dev(go).to(losses.dtype).float().cpu().numpy()
+    want_g = np.asarray(grad_of(go_seen))
+    if dt == torch.float32:
+        if kind == "taylor":                        # gradients through log f grow where f comes close to 0
+            err = np.abs(xt.grad.cpu().numpy() - want_g).max() if want_g.size else 0.0
+            assert err <= 1e-5 * max(1.0, np.abs(want_g).max()), (what, err)
         else:
-            close_loss(out.detach().cpu().numpy(), fwd(), "%s %s" % (name, shape))
-        out.backward(dev(go))
-        if c == 1:      # and every gradient is exactly 0: what is left on either side is rounding
-            assert np.abs(xt.grad.cpu().numpy() - bwd()).max() <= 1e-5
-        else:
-            close_grad(xt.grad.cpu().numpy(), bwd(), "%s %s" % (name, shape))
+            close_grad(xt.grad.cpu().numpy(), want_g, what)
+    else:
+        close_grad_stored(xt.grad, want_g, dt, what)
+    g = xt.grad.float().cpu().numpy()
+    assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all(), what
 
 
-@pytest.mark.parametrize("shape", _shapes(2, 16, 24, 500))
-def test_lovasz_and_relabelling(pl, shape):
-    n, c, m = shape
-    x, y = seg_inputs(300 + n * c * m, (n, c, m), 255, 0.1)
-    xt, yt = dev(x).requires_grad_(), dev(y)
-    losses = pl.LovaszSoftmaxFunctionV3.apply(xt, yt, 255)
-    want, want_jacc = oracle.lovasz_forward(x.astype(np.float64), y, 255)
-    assert np.abs(losses.detach().cpu().numpy() - want).max() <= 1e-5 * max(1e-30, np.abs(want).max())
-    n_min = max(1, y.size // 8)
-    got = pl.score_ohem_label(xt.detach(), yt, 255, 0.4, n_min).cpu().numpy()
-    scores = oracle.ohem_scores(x, y, 255)
-    # the selection is exact on given scores; scores themselves may differ in the last bit, so compare
-    # wherever no score sits within 1e-6 of the threshold or of the n_min-th smallest score
-    order = np.sort(scores.reshape(-1))
-    cut = order[min(n_min, order.size) - 1]
-    sure = (np.abs(scores - 0.4) > 1e-6) & (np.abs(scores - cut) > 1e-6)
-    want_lab = oracle.ohem_score_label(x, y, 255, 0.4, n_min)
-    assert np.array_equal(got[sure], want_lab[sure])
-    onehot = pl.OnehotEncoder(c, lb_smooth=0.1, ignore_idx=255)(yt).cpu().numpy()
-    assert np.array_equal(onehot, oracle.onehot(y, c, 0.1, 255))
-
-
-@pytest.mark.parametrize("shape", _shapes(3, 24, 150, 400))
-def test_layer_norm_taylor_softmax(pl, shape):
-    x = synth.normal(400 + sum(shape), 1, shape, 0.2, 1.5)
-    g = synth.normal(401, 2, shape, 0.0, 1.0)
-    xt = dev(x).requires_grad_()
-    out = pl.LayerNormV3Func.apply(xt, 1e-5)
-    if shape[1] > 1:
-        # fp32 carries x - mean to about one spacing of |x|, and the output multiplies that by
-        # 1/sqrt(var + eps), which is large where the channels of a pixel nearly coincide
-        rstd = 1.0 / np.sqrt(x.astype(np.float64).var(axis=1) + 1e-5)
-        bound = 1e-5 + 2.4e-7 * np.abs(x).max() * rstd.max()
-        assert np.abs(out.detach().cpu().numpy() - oracle.layer_norm_forward(x.astype(np.float64), 1e-5)).max() <= bound
-    out.backward(dev(g))
-    want = oracle.layer_norm_backward(g.astype(np.float64), x.astype(np.float64), 1e-5)
-    assert np.abs(xt.grad.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max() + 1e-12
-    for use_log, mod in ((False, pl.TaylorSoftmaxV3(dim=1, n=2)), (True, pl.LogTaylorSoftmaxV3(dim=1, n=2))):
-        xt = dev(x).requires_grad_()
-        out = mod(xt)
-        want = oracle.taylor_forward(x.astype(np.float64), 1, 2, use_log)
-        assert np.abs(out.detach().cpu().numpy() - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
-        out.backward(dev(g))
-        want_g = oracle.taylor_backward(g.astype(np.float64), x.astype(np.float64), 1, 2, use_log)
-        assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * max(1.0, np.abs(want_g).max())
-
-
-@pytest.mark.parametrize("shape", _shapes(4, 16, 12, 3000))
-def test_elementwise_ops(pl, shape):
-    x = synth.normal(500 + sum(shape), 1, shape, -1.0, 1.5)
-    y = synth.bernoulli(501, 2, shape, 0.25).astype(np.float32)
-    go = synth.normal(502, 3, shape, 0.0, 1.0)
-    xt = dev(x).requires_grad_()
-    out = pl.FocalSigmoidLossFuncV3.apply(xt, dev(y), 0.25, 2)
-    close_loss(out.detach().cpu().numpy(), oracle.focal_forward(x, y, 0.25, 2), "focal %s" % (shape,))
-    out.backward(dev(go))
-    close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, 0.25, 2, go), "focal %s" % (shape,))
-    rows = x.reshape(shape[0], -1)
-    xt = dev(rows).requires_grad_()
-    loss = pl.SoftDiceLossV3Func.apply(xt, dev(y.reshape(shape[0], -1)), 2, 0.5)
-    want, stats = oracle.soft_dice_forward(rows.astype(np.float64), y.reshape(shape[0], -1).astype(np.float64), 2, 0.5)
-    assert np.abs(loss.detach().cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max() + 1e-7
-    gr = synth.normal(503, 4, (shape[0],), 0.5, 1.0)
-    loss.backward(dev(gr))
-    want_g = oracle.soft_dice_backward(gr.astype(np.float64), rows.astype(np.float64),
-                                       y.reshape(shape[0], -1).astype(np.float64), stats, 2)
-    assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max() + 1e-12
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shape_lovasz(pl, seed):
+    """The sort pipeline at random row lengths and class counts (tiles that end anywhere, rows shorter than a
+    tile, classes without positives, one to three storage types): loss per class against the fp64 restatement,
+    Jaccard differences mostly bit-equal to the fp32 one, exact zeros at ignored pixels, and the gradient to the
+    bound that near-ties allow."""
+    from pytorch_loss import _native
+    r = np.random.RandomState(5000 + seed)
+    shape = (int(r.randint(1, 4)), int(r.randint(1, 41)), int(r.randint(1, 90)), int(r.randint(1, 90)))
+    ignore = int(r.choice([255, -100]))
+    frac = float(r.choice([0.0, 0.1, 0.6]))
+    scale = float(r.choice([0.5, 2.0, 6.0]))
+    dt = (torch.float32, torch.float32, torch.bfloat16)[int(r.randint(3))]
+    x = synth.normal(400 + seed, 1, shape, 0.0, scale)
+    y = synth.seg_labels(400 + seed, shape[:1] + shape[2:], shape[1], ignore, frac)
+    xt = dev(x).to(dt)
+    xr = xt.float().cpu().numpy()
+    what = "lovasz %s %s ignore=%d scale=%g" % (shape, str(dt)[6:], ignore, scale)
+    losses, jacc = _native.lovasz_forward(xt, dev(y), ignore)
+    jacc = jacc.cpu().numpy()
+    l64, j64 = oracle.lovasz_forward(xr.astype(np.float64), y, ignore)
+    rtol = 3e-4 if scale > 2 else 1e-5              # confident logits: 1 - p carries p's fp32 rounding enlarged
+    if dt != torch.float32:
+        rtol += ULP_REL[dt]                         # the losses come back in the storage type
+    np.testing.assert_allclose(losses.float().cpu().numpy(), l64, rtol=rtol, atol=1e-7, err_msg=what)
+    assert (jacc[:, y.reshape(-1) == ignore] == 0).all(), what
+    if (y != ignore).any():
+        np.testing.assert_allclose(jacc.sum(axis=1, dtype=np.float64), 1.0, rtol=1e-4, err_msg=what)
+    _, j32 = oracle.lovasz_forward(xr, y, ignore)
+    assert (jacc.view(np.uint32) == j32.view(np.uint32)).mean() > 0.99, what
+    xt.requires_grad_()
+    out = pl.LovaszSoftmaxFunctionV3.apply(xt, dev(y), ignore)
+    w = synth.normal(400 + seed, 4, (shape[1],), 0.5, 1.0)
+    out.backward(dev(w).to(out.dtype))
+    w_seen = dev(w).to(out.dtype).float().cpu().numpy().astype(np.float64)
+    want_g = oracle.lovasz_backward(w_seen, xr.astype(np.float64), y, j64, ignore)
+    g = xt.grad.float().cpu().numpy()
+    bound = max(1e-5, 2e-3 * np.abs(j64).max() * np.abs(w_seen).max())
+    if dt != torch.float32:
+        bound += ULP_REL[dt] * np.abs(want_g).max()
+    assert np.abs(g - want_g).max() <= bound, (what, np.abs(g - want_g).max(), bound)
+    assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all(), what
