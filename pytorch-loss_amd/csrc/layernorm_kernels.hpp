@@ -143,7 +143,7 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
 }
 
 // Any C: G lanes share one slice and stride over it (G = 64: a wavefront per contiguous row;
-// G = 1: a lane per slice). Statistics from sums shifted by the slice's first element, which keeps
+// G = 1: a lane per slice). Statistics from sums shifted by the mean of the slice's first elements, which keeps
 // the one-pass variance well conditioned; the second sweep re-reads the slice through cache.
 template <class T, int G, bool Bwd>
 __global__ __launch_bounds__(256) void ln_group(const T *__restrict__ x, const T *__restrict__ g, T *__restrict__ out,
@@ -158,14 +158,33 @@ __global__ __launch_bounds__(256) void ln_group(const T *__restrict__ x, const T
         const int64_t pc = live ? pix : 0;
         const int64_t n = pc / p.m_size;
         const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size;
-        const float shift = load_one(x + base);
-        float s1 = 0.f, s2 = 0.f;
-#pragma unroll 8
-        for (int j = sub; j < p.C; j += G) {          // unrolled: eight loads in flight per lane
-            const float d = load_one(x + base + (int64_t)j * p.m_size) - shift;
-            s1 += d;
-            s2 = __builtin_fmaf(d, d, s2);
+        // The shift is the mean of the slice's first (up to) 8 elements: a single element can sit several standard
+        // deviations from the mean, and E[d^2] - E[d]^2 then cancels digits (shifted by its first element, a slice
+        // of 1317 channels missed 1e-5 by a factor of 4). Four independent partial sums per lane keep the rounding
+        // of the long sums down and eight loads in flight.
+        const int n_shift = p.C < 8 ? p.C : 8;
+        float shift = 0.f;
+        for (int j = 0; j < n_shift; ++j) shift += load_one(x + base + (int64_t)j * p.m_size);
+        shift *= 1.f / (float)n_shift;
+        float a1[4] = {0.f, 0.f, 0.f, 0.f}, a2[4] = {0.f, 0.f, 0.f, 0.f};
+        int j = sub;
+#pragma unroll 2
+        for (; j + 3 * G < p.C; j += 4 * G) {
+            float d[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) d[u] = load_one(x + base + (int64_t)(j + u * G) * p.m_size) - shift;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a1[u] += d[u];
+                a2[u] = __builtin_fmaf(d[u], d[u], a2[u]);
+            }
         }
+        for (; j < p.C; j += G) {
+            const float d = load_one(x + base + (int64_t)j * p.m_size) - shift;
+            a1[0] += d;
+            a2[0] = __builtin_fmaf(d, d, a2[0]);
+        }
+        float s1 = (a1[0] + a1[1]) + (a1[2] + a1[3]), s2 = (a2[0] + a2[1]) + (a2[2] + a2[3]);
         s1 = group_reduce<G>(s1, OpSum());
         s2 = group_reduce<G>(s2, OpSum());
         const float dm = s1 * inv_c;

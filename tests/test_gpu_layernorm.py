@@ -59,6 +59,17 @@ def test_backward_known_answers(pl):
             np.testing.assert_allclose(got[n, :, m], np.array(chans), rtol=2e-6, err_msg=str((eps, n, m)))
 
 
+@pytest.mark.parametrize("shape", [(3, 1317, 57), (2, 1500, 1), (4, 3000, 1), (1, 2048, 33)])
+def test_long_slices_with_an_outlying_first_channel(pl, shape):
+    """More than 1024 channels, and (N, C) rows: one pass over the slice with shifted sums. A first channel far from
+    the slice's mean must not cost accuracy (the shift is the mean of the first few channels, not the first one)."""
+    x = synth.normal(123, 1, shape, 0.3, 1.5)
+    x[:, 0, :] += 12.0
+    out = pl.LayerNormV3Func.apply(torch.from_numpy(x).cuda(), 1e-6).cpu().numpy()
+    want = oracle.layer_norm_forward(x.astype(np.float64), 1e-6)
+    assert np.abs(out - want).max() <= 1e-5, np.abs(out - want).max()
+
+
 def test_large_common_offset_keeps_accuracy(pl):
     x = synth.normal(122, 1, (2, 64, 256), 1000.0, 0.5)
     out = pl.LayerNormV3Func.apply(torch.from_numpy(x).cuda(), 1e-6).cpu().numpy()

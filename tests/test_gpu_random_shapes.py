@@ -138,3 +138,63 @@ def test_random_shape_lovasz(pl, seed):
         bound += ULP_REL[dt] * np.abs(want_g).max()
     assert np.abs(g - want_g).max() <= bound, (what, np.abs(g - want_g).max(), bound)
     assert (g[np.broadcast_to(np.expand_dims(y == ignore, 1), g.shape)] == 0).all(), what
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_shape_neighbouring_ops(pl, seed):
+    """Focal, Taylor softmax, soft dice and layer norm at random sizes (element counts that end anywhere inside a
+    vector, a wavefront or a block; channel counts on both sides of every launch shape of the layer norm)."""
+    r = np.random.RandomState(7000 + seed)
+    kind = ("focal", "taylor_sm", "dice", "layernorm")[seed % 4]
+    if kind == "focal":
+        shape = tuple(int(v) for v in r.randint(1, 40, size=int(r.randint(1, 5))))
+        x = synth.normal(500 + seed, 1, shape, -1.0, 2.0)
+        if seed % 8 < 4:
+            y = synth.bernoulli(500 + seed, 2, shape, 0.2).astype(np.float32)
+        else:
+            y = synth.uniform01(500 + seed, 2, int(np.prod(shape))).reshape(shape).astype(np.float32)
+        alpha, gamma = float(r.choice([0.25, 0.6])), float(r.choice([0.0, 1.5, 2.0]))
+        xt = dev(x).requires_grad_()
+        loss = pl.FocalSigmoidLossFuncV3.apply(xt, dev(y), alpha, gamma)
+        close_loss(loss.detach().cpu().numpy(), oracle.focal_forward(x, y, alpha, gamma), "focal %s" % (shape,))
+        go = synth.normal(500 + seed, 3, shape, 0.0, 1.0)
+        loss.backward(dev(go))
+        close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, alpha, gamma, go), "focal %s" % (shape,))
+    elif kind == "taylor_sm":
+        shape = (int(r.randint(1, 4)), int(r.choice([r.randint(1, 33), r.randint(33, 300), r.randint(300, 3000)])),
+                 int(r.choice([1, r.randint(1, 70)])))
+        order, use_log = int(r.choice([2, 4, 6])), bool(r.randint(2))
+        x = synth.normal(500 + seed, 1, shape, 0.0, 1.0)
+        g = synth.normal(500 + seed, 2, shape, 0.0, 1.0)
+        xt = dev(x).requires_grad_()
+        out = pl.TaylorSoftmaxFunc.apply(xt, 1, order, use_log)
+        want = oracle.taylor_forward(x.astype(np.float64), 1, order, use_log)
+        assert np.abs(out.detach().cpu().numpy() - want).max() <= 1e-5 * max(1.0, np.abs(want).max()), shape
+        out.backward(dev(g))
+        want_g = oracle.taylor_backward(g.astype(np.float64), x.astype(np.float64), 1, order, use_log)
+        assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * max(1.0, np.abs(want_g).max()), shape
+    elif kind == "dice":
+        n, length = int(r.randint(1, 9)), int(r.choice([r.randint(1, 100), r.randint(100, 70000)]))
+        p, smooth = float(r.choice([1.0, 2.0, 1.5])), float(r.choice([1.0, 0.1]))
+        x = synth.normal(500 + seed, 1, (n, length), 0.0, 2.0)
+        y = synth.uniform01(500 + seed, 2, n * length).reshape(n, length).astype(np.float32)
+        xt = dev(x).requires_grad_()
+        loss = pl.SoftDiceLossV3Func.apply(xt, dev(y), p, smooth)
+        want, stats = oracle.soft_dice_forward(x.astype(np.float64), y.astype(np.float64), p, smooth)
+        assert np.abs(loss.detach().cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max() + 1e-7, (n, length)
+        go = synth.normal(500 + seed, 3, (n,), 0.5, 1.0)
+        loss.backward(dev(go))
+        want_g = oracle.soft_dice_backward(go.astype(np.float64), x.astype(np.float64), y.astype(np.float64), stats, p)
+        assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max() + 1e-12, (n, length)
+    else:
+        shape = (int(r.randint(1, 4)), int(r.choice([r.randint(1, 33), r.randint(33, 513), r.randint(513, 1500)])),
+                 int(r.choice([1, r.randint(1, 200)])))
+        x = synth.normal(500 + seed, 1, shape, 0.3, 1.5)
+        g = synth.normal(500 + seed, 2, shape, 0.0, 1.0)
+        xt = dev(x).requires_grad_()
+        out = pl.LayerNormV3Func.apply(xt, 1e-6)
+        if shape[1] > 1:
+            assert np.abs(out.detach().cpu().numpy() - oracle.layer_norm_forward(x.astype(np.float64), 1e-6)).max() <= 1e-5, shape
+        out.backward(dev(g))
+        want_g = oracle.layer_norm_backward(g.astype(np.float64), x.astype(np.float64), 1e-6)
+        assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max(), shape
