@@ -198,3 +198,62 @@ def test_random_shape_neighbouring_ops(pl, seed):
         out.backward(dev(g))
         want_g = oracle.layer_norm_backward(g.astype(np.float64), x.astype(np.float64), 1e-6)
         assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max(), shape
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_shape_module_reductions(pl, seed):
+    """'mean' / 'sum' of the modules (per-block partials inside the forward kernel, a fixed-order finish, the
+    upstream scalar and 1 / n_valid folded into the backward) at random shapes large enough for many blocks, on every
+    launch shape: loss and gradient against the oracle's reduction of its per-pixel values."""
+    r = np.random.RandomState(9000 + seed)
+    kind = ("lsr", "lmargin", "taylor", "ohem_ce")[seed % 4]
+    family = r.randint(4)
+    if family == 0:
+        shape = (int(r.randint(1, 5)), int(r.randint(2, 33)), int(r.randint(20, 200)), int(r.randint(20, 200)))
+    elif family == 1:          # odd planes: the per-image form for fp32
+        shape = (int(r.randint(1, 5)), int(r.randint(2, 25)), int(r.randint(64, 160)) | 1, int(r.randint(64, 160)) | 1)
+    elif family == 2:
+        shape = (int(r.randint(1, 3)), int(r.randint(33, 520)), int(r.randint(8, 40)), int(r.randint(8, 40)))
+    else:
+        shape = (int(r.randint(100, 3000)), int(r.choice([r.randint(2, 33), r.randint(33, 1200)])))
+    ignore = int(r.choice([255, -100]))
+    reduction = ("mean", "sum")[int(r.randint(2))]
+    dt = (torch.float32, torch.float32, torch.bfloat16)[int(r.randint(3))]
+    x, y = seg_inputs(600 + seed, shape, ignore, 0.1)
+    xt = dev(x).to(dt)
+    xr = xt.float().cpu().numpy()
+    xt.requires_grad_()
+    yt = dev(y)
+    what = "%s %s %s %s" % (kind, shape, reduction, str(dt)[6:])
+    n_valid = int((y != ignore).sum())
+    if kind == "lsr":
+        crit = pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=reduction, ignore_index=ignore)
+        per = oracle.lsr_forward(xr.astype(np.float64), y, ignore, 0.1)
+        grad_of = lambda g: oracle.lsr_backward(xr, y, ignore, 0.1, g)
+    elif kind == "lmargin":
+        crit = pl.LargeMarginSoftmaxV3(lam=0.3, reduction=reduction, ignore_index=ignore)
+        per = oracle.lmargin_forward(xr.astype(np.float64), y, 0.3, ignore)
+        grad_of = lambda g: oracle.lmargin_backward(xr, y, 0.3, ignore, g)
+    elif kind == "taylor":
+        crit = pl.TaylorCrossEntropyLossV3(n=4, ignore_index=ignore, reduction=reduction)
+        per = oracle.taylor_ce(xr.astype(np.float64), y, 4, ignore)
+        grad_of = lambda g: oracle.taylor_ce_backward(xr.astype(np.float64), y, 4, ignore, g)
+    else:
+        # OhemCELoss with a threshold no score exceeds keeps every label: plain cross entropy, mean over the valid pixels
+        crit = pl.OhemCELoss(score_thresh=2.0, n_min=1, ignore_index=ignore)
+        reduction = "mean"
+        per = oracle.lsr_forward(xr.astype(np.float64), y, ignore, 0.0)
+        grad_of = lambda g: oracle.lsr_backward(xr, y, ignore, 0.0, g)
+    loss = crit(xt, yt)
+    assert loss.dim() == 0, what
+    want = per.sum(dtype=np.float64) / (n_valid if reduction == "mean" else 1)
+    rtol = 1e-5 + (ULP_REL[dt] if dt != torch.float32 else 0.0)
+    assert abs(loss.item() - want) <= rtol * abs(want), (what, loss.item(), want)
+    loss.backward()
+    scale = np.float32(1.0 / n_valid) if reduction == "mean" else np.float32(1.0)
+    want_g = np.asarray(grad_of(np.full(y.shape, scale, dtype=np.float32)))
+    if dt == torch.float32:
+        err = np.abs(xt.grad.cpu().numpy() - want_g).max()
+        assert err <= 2e-5 * np.abs(want_g).max() + 1e-12, (what, err, np.abs(want_g).max())
+    else:
+        close_grad_stored(xt.grad, want_g, dt, what)
