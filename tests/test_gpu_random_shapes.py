@@ -267,3 +267,69 @@ def test_random_shape_module_reductions(pl, seed):
         assert err <= 2e-5 * np.abs(want_g).max() + 1e-12, (what, err, np.abs(want_g).max())
     else:
         close_grad_stored(xt.grad, want_g, dt, what)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_shape_fused_variants(pl, seed):
+    """The forward+backward-in-one-pass Functions (focal, large margin with its valid count) and the OHEM modules
+    (relabelling and loss in one forward pass) at random shapes: against the oracle, and the OHEM losses against the
+    composition of the separately tested relabelling with the plain loss on the new labels."""
+    from pytorch_loss import _native
+    r = np.random.RandomState(11000 + seed)
+    kind = ("focal_fb", "lmargin_fb", "ohem_ce", "ohem_lm")[seed % 4]
+    if kind == "focal_fb":
+        shape = tuple(int(v) for v in r.randint(1, 50, size=int(r.randint(1, 5))))
+        x = synth.normal(800 + seed, 1, shape, -1.0, 2.0)
+        y = synth.bernoulli(800 + seed, 2, shape, 0.3).astype(np.float32)
+        alpha, gamma = float(r.choice([0.25, 0.5])), float(r.choice([0.0, 1.0, 2.0, 3.0]))
+        xt = dev(x).requires_grad_()
+        loss = pl.FocalSigmoidLossFuncV3FB.apply(xt, dev(y), alpha, gamma)
+        close_loss(loss.detach().cpu().numpy(), oracle.focal_forward(x, y, alpha, gamma), "focal fb %s" % (shape,))
+        go = synth.normal(800 + seed, 3, shape, 0.0, 1.0)
+        loss.backward(dev(go))
+        close_grad(xt.grad.cpu().numpy(), oracle.focal_backward(x, y, alpha, gamma, go), "focal fb %s" % (shape,))
+        return
+    family = r.randint(3)
+    if family == 0:
+        shape = (int(r.randint(1, 4)), int(r.randint(2, 33)), int(r.randint(1, 90)), int(r.randint(1, 90)))
+    elif family == 1:
+        shape = (int(r.randint(1, 3)), int(r.randint(33, 520)), int(r.randint(8, 24)), int(r.randint(8, 24)))
+    else:
+        shape = (int(r.randint(16, 600)), int(r.choice([r.randint(2, 33), r.randint(33, 3000)])))
+    ignore = int(r.choice([255, -100]))
+    x, y = seg_inputs(800 + seed, shape, ignore, 0.1)
+    x = x * np.float32(r.choice([1.0, 2.0]))
+    xt = dev(x).requires_grad_()
+    yt = dev(y)
+    what = "%s %s ignore=%d" % (kind, shape, ignore)
+    if kind == "lmargin_fb":
+        losses, cnt = pl.LargeMarginSoftmaxFuncV3FB.apply(xt, yt, 0.3, ignore)
+        assert cnt.dtype == torch.int64 and int(cnt.item()) == int((y != ignore).sum()), what
+        close_loss(losses.detach().cpu().numpy(), oracle.lmargin_forward(x, y, 0.3, ignore), what)
+        go = synth.normal(800 + seed, 3, y.shape, 0.0, 1.0)
+        losses.backward(dev(go))
+        close_grad(xt.grad.cpu().numpy(), oracle.lmargin_backward(x, y, 0.3, ignore, go), what)
+        return
+    thresh = float(r.choice([0.3, 0.7, 0.9]))
+    n_min = int(y.size // int(r.choice([4, 16, 64]))) + 1
+    crit = (pl.OhemCELoss if kind == "ohem_ce" else pl.OhemLargeMarginLoss)(thresh, n_min, ignore)
+    loss = crit(xt, yt)
+    new = _native.ohem_score_label(xt.detach(), yt, ignore, thresh, n_min).cpu().numpy()
+    assert np.array_equal(yt.cpu().numpy(), y), what
+    n_valid = int((new != ignore).sum())
+    assert n_valid >= min(n_min, int((y != ignore).sum())) - 0, what
+    if kind == "ohem_ce":
+        per = oracle.lsr_forward(x.astype(np.float64), new, ignore, 0.0)
+        grad_of = lambda g: oracle.lsr_backward(x, new, ignore, 0.0, g)
+    else:
+        per = oracle.lmargin_forward(x.astype(np.float64), new, 0.3, ignore)
+        grad_of = lambda g: oracle.lmargin_backward(x, new, 0.3, ignore, g)
+    want = per.sum(dtype=np.float64) / max(n_valid, 1)
+    if n_valid == 0:
+        assert np.isnan(loss.item()), what
+        return
+    assert abs(loss.item() - want) <= 1e-5 * abs(want), (what, loss.item(), want)
+    loss.backward()
+    want_g = np.asarray(grad_of(np.full(y.shape, np.float32(1.0 / n_valid), dtype=np.float32)))
+    err = np.abs(xt.grad.cpu().numpy() - want_g).max()
+    assert err <= 2e-5 * np.abs(want_g).max() + 1e-12, (what, err)
