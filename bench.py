@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|lsr_vocab|lmargin_rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|focal_seg|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|lsr_vocab|lmargin_rows]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -73,6 +73,9 @@ WORKLOADS = {
                      "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lsr_c300": dict(base="lsr", shape=(8, 300, 256, 256), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8,300,256,256), "
                      "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
+    # the focal loss at the segmentation shape of the other two losses (the shape the >= 70 % target is stated on)
+    "focal_seg": dict(base="focal", shape=(8, 19, 1024, 1024), desc="FocalLossV3 fwd+bwd, fp32 logits/labels (8,19,1024,1024), "
+                      "Bernoulli(0.02) labels, alpha=0.25 gamma=2, mean"),
     # crops of odd size: every channel plane starts at another offset into a cache line (tiles per image, 4 pixels per lane)
     "lsr_crop769": dict(base="lsr", shape=(16, 19, 769, 769), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (16,19,769,769), "
                         "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
