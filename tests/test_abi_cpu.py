@@ -275,3 +275,46 @@ def test_taylor_orders_are_checked_at_construction():
         with pytest.raises(AssertionError):
             pl.TaylorCrossEntropyLossV3(n=bad)
     assert pl.TaylorCrossEntropyLossV3(n=4).n == 4 and pl.LogTaylorSoftmaxV3(n=2).n == 2
+
+
+def test_extension_stand_ins_load_and_refuse_cpu_tensors():
+    """The ctypes stand-ins for the reference's extension modules bind every entry point they use at import time
+    (a misspelt or missing symbol fails here, without a GPU) and raise the extensions' own error for CPU tensors."""
+    import sys
+    import torch
+    import ext_stubs
+    saved = {n: sys.modules.get(n) for n in ext_stubs.NAMES}
+    try:
+        mods = ext_stubs.install()
+        assert set(mods) == {"lsr_cpp", "focal_cpp", "large_margin_cpp", "lovasz_softmax_cpp", "ohem_cpp", "one_hot_cpp",
+                             "taylor_softmax_cpp", "soft_dice_cpp", "layer_norm_cpp"}
+        x = torch.zeros(2, 3, 4)
+        y = torch.zeros(2, 4, dtype=torch.int64)
+        calls = [
+            lambda: mods["lsr_cpp"].lsr_forward(x, y, 255, 0.1),
+            lambda: mods["lsr_cpp"].lsr_backward(x, y, 255, 0.1),
+            lambda: mods["focal_cpp"].focalloss_forward(x, x, 2.0, 0.25),
+            lambda: mods["focal_cpp"].focalloss_backward(x, x, 2.0, 0.25),
+            lambda: mods["focal_cpp"].focalloss_forward_backward(x, x, 2.0, 0.25),
+            lambda: mods["large_margin_cpp"].l_margin_forward(x, y, 0.3, 255),
+            lambda: mods["large_margin_cpp"].l_margin_backward(x, y, 0.3, 255),
+            lambda: mods["large_margin_cpp"].l_margin_forward_backward(x, y, 0.3, 255),
+            lambda: mods["lovasz_softmax_cpp"].lovasz_softmax_forward(x, y, 255),
+            lambda: mods["ohem_cpp"].score_ohem_label(x, y, 255, 0.7, 2),
+            lambda: mods["one_hot_cpp"].label_one_hot(y, 255, 0.1, 3),
+            lambda: mods["taylor_softmax_cpp"].taylor_softmax_forward(x, 1, 2, False),
+            lambda: mods["taylor_softmax_cpp"].taylor_softmax_backward(x, x, 1, 2, False),
+            lambda: mods["soft_dice_cpp"].soft_dice_forward(x[0], x[0], 1.0, 1.0),
+            lambda: mods["soft_dice_cpp"].soft_dice_backward(torch.ones(3), x[0], x[0], 1.0, 1.0),
+            lambda: mods["layer_norm_cpp"].layer_norm_forward(x, 1e-6),
+            lambda: mods["layer_norm_cpp"].layer_norm_backward(x, x, 1e-6),
+        ]
+        for call in calls:
+            with pytest.raises(RuntimeError, match="only supports gpu mode"):
+                call()
+    finally:
+        for n, m in saved.items():
+            if m is None:
+                sys.modules.pop(n, None)
+            else:
+                sys.modules[n] = m
