@@ -193,6 +193,8 @@ int plh_lmargin_forward_backward(const void *logits, int32_t dtype, const int64_
  * workspace: scratch device memory of at least plh_lovasz_workspace_bytes() bytes,
  *         256-byte aligned, owned by the caller; contents are undefined afterwards.
  * Limits: dimsize < 512 and n_size*dimsize*m_size < 2^31 (csrc/lovasz_softmax.cu:664-665).
+ * With PLH_LOVASZ_SCAN=lookback in the environment (read by both functions at every call) the sort passes run
+ * their decoupled look-back variant, which needs a larger workspace; results are identical, the default is faster.
  */
 int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size);
 

@@ -32,6 +32,9 @@
 // A 4096-key tile is handled by 512 threads with 8 keys each; neighbouring tiles of a class row run
 // on the same XCD (sort_tile) so that the sectors they share merge in one L2.
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
+#include <cstdlib>
+#include <cstring>
+
 #include "plh_common.hpp"
 
 namespace plh {
@@ -220,6 +223,12 @@ struct SortArgs {
     int tiles;                   // ceil(P / kSortTile)
     int tiles_pad;               // tiles rounded up to a multiple of kSortWaves: row length of the tile tables
     int pass;                    // 0, 1, 2: scatter pass; the last (fused) pass of a class is passes - 1
+    // decoupled look-back variant only (see lov_look_back): this pass's tile descriptors [C][tiles][kRadix] (64-bit
+    // ones in the last pass), its per-class ticket counters and the word that a timed-out wait sets
+    uint32_t *desc;
+    unsigned long long *desc_wide;
+    uint32_t *tickets;
+    uint32_t *timed_out;
 };
 
 // The digits of a class. Keys that take part in a class's sort are below 2^bits (bits from the
@@ -541,6 +550,117 @@ __global__ __launch_bounds__(256) void lov_row_scan(uint32_t *table0, uint32_t *
     if (threadIdx.x == 0) totals[rid] = carry;
 }
 
+// ---- the decoupled look-back variant of the passes (opt-in: PLH_LOVASZ_SCAN=lookback) -------------------
+// Instead of a histogram kernel and a row scan in front of every pass, a tile learns how many keys of each digit
+// the tiles before it hold by walking back over their descriptors: every tile publishes, per digit, first its own
+// count ("aggregate") and, once it knows the sum over all its predecessors, the inclusive sum ("prefix"); a walk
+// adds aggregates until it meets a prefix. The count travels in the same word as the state, so plain device-scope
+// atomic loads and stores carry it (no fence). Tiles are handed out by a ticket counter per class, in the order
+// in which blocks start, so every predecessor of a waiting block is resident and gets to publish: the waits end.
+// They are bounded all the same; a wait that runs out sets `timed_out`, which turns the class losses into NaN.
+// The digit totals of all passes come from one pass over the keys up front (lov_hist_all, lov_hist_reduce).
+constexpr uint32_t kDescAggregate = 1u << 30, kDescPrefix = 2u << 30, kDescValue = (1u << 30) - 1u;
+constexpr int kLookBackSpins = 1 << 22;
+
+__device__ __forceinline__ uint32_t lov_look_back(uint32_t *desc_row, int tile, int d, uint32_t mine, uint32_t *timed_out) {
+    uint32_t *me = desc_row + (int64_t)tile * kRadix + d;
+    __hip_atomic_store(me, kDescAggregate | mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t before = 0;
+    for (int t = tile - 1; t >= 0; --t) {
+        const uint32_t *at = desc_row + (int64_t)t * kRadix + d;
+        uint32_t v = 0;
+        for (int spin = 0; spin < kLookBackSpins; ++spin) {
+            v = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v >> 30) break;
+        }
+        if ((v >> 30) == 0) {
+            *timed_out = 1u;
+            break;
+        }
+        before += v & kDescValue;
+        if ((v >> 30) == 2u) break;
+    }
+    __hip_atomic_store(me, kDescPrefix | (before + mine), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return before;
+}
+
+// The same for two counts at once (keys and positives of the last pass): state in bits 62-63, positives in
+// bits 31-61, keys in bits 0-30.
+constexpr unsigned long long kWideAggregate = 1ull << 62, kWidePrefix = 2ull << 62, kWideField = (1ull << 31) - 1ull;
+__device__ __forceinline__ void lov_look_back2(unsigned long long *desc_row, int tile, int d, uint32_t mine, uint32_t mine_hot,
+                                               uint32_t &before, uint32_t &before_hot, uint32_t *timed_out) {
+    unsigned long long *me = desc_row + (int64_t)tile * kRadix + d;
+    __hip_atomic_store(me, kWideAggregate | ((unsigned long long)mine_hot << 31) | mine, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    unsigned long long sum = 0;         // both fields at once: neither can carry into the other (counts stay below 2^31)
+    for (int t = tile - 1; t >= 0; --t) {
+        const unsigned long long *at = desc_row + (int64_t)t * kRadix + d;
+        unsigned long long v = 0;
+        for (int spin = 0; spin < kLookBackSpins; ++spin) {
+            v = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v >> 62) break;
+        }
+        if ((v >> 62) == 0) {
+            *timed_out = 1u;
+            break;
+        }
+        sum += v & ((1ull << 62) - 1ull);
+        if ((v >> 62) == 2ull) break;
+    }
+    before = (uint32_t)(sum & kWideField);
+    before_hot = (uint32_t)((sum >> 31) & kWideField);
+    __hip_atomic_store(me, kWidePrefix | ((unsigned long long)(before_hot + mine_hot) << 31) | (before + mine),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The tile of a block in the look-back variant: the next ticket of its class.
+__device__ __forceinline__ int lov_take_ticket(uint32_t *tickets, int c) {
+    __shared__ int ticket;
+    if (threadIdx.x == 0) ticket = (int)atomicAdd(&tickets[c], 1u);
+    __syncthreads();
+    return ticket;
+}
+
+// Digit counts of every pass of a class in one sweep over its keys: a block per two tiles, tables per pass in LDS,
+// one table set per block in `partial` [C][blocks][kHistTables][kRadix]; slot p < 3 = scatter pass p, slot 3 = the
+// class's last pass, slot 4 = the positives of the last pass.
+constexpr int kHistTables = 5;
+__global__ __launch_bounds__(kSortThreads) void lov_hist_all(const SortArgs a, uint32_t *__restrict__ partial, int blocks) {
+    __shared__ uint32_t counts[kHistTables][kRadix];
+    const int c = blockIdx.y;
+    for (int i = threadIdx.x; i < kHistTables * kRadix; i += kSortThreads) (&counts[0][0])[i] = 0;
+    __syncthreads();
+    const uint32_t bits = a.key_bits[c];
+    const int np = digit_plan(bits, 0).passes;
+    const uint32_t limit = keep_limit(a, c);
+    const int begin = blockIdx.x * (2 * kSortTile);
+    const uint32_t *kin = a.keys_in + (int64_t)c * a.P;
+    for (int i = begin + threadIdx.x; i < min(a.P, begin + 2 * kSortTile); i += kSortThreads) {
+        const uint32_t key = kin[i];
+        if (!keep_key(key, limit)) continue;
+        for (int p = 0; p < np; ++p) {
+            const DigitPlan dp = digit_plan(bits, p);
+            const uint32_t digit = (key >> dp.shift) & dp.mask;
+            const int slot = (p == np - 1) ? 3 : p;
+            atomicAdd(&counts[slot][digit], 1u);
+            if (p == np - 1 && (key >> 31)) atomicAdd(&counts[4][digit], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t *out = partial + ((int64_t)c * blocks + blockIdx.x) * (kHistTables * kRadix);
+    for (int i = threadIdx.x; i < kHistTables * kRadix; i += kSortThreads) out[i] = (&counts[0][0])[i];
+}
+
+// totals[slot][C][kRadix] = sum over the blocks' tables.
+__global__ __launch_bounds__(kRadix) void lov_hist_reduce(const uint32_t *__restrict__ partial, int blocks, int C,
+                                                          uint32_t *__restrict__ totals) {
+    const int c = blockIdx.y, slot = blockIdx.x, d = threadIdx.x;
+    uint32_t sum = 0;
+    for (int b = 0; b < blocks; ++b) sum += partial[(((int64_t)c * blocks + b) * kHistTables + slot) * kRadix + d];
+    totals[((int64_t)slot * C + c) * kRadix + d] = sum;
+}
+
+template <bool LookBack>
 __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t s_keys[kSortTile];
     __shared__ uint32_t s_vals[kSortTile];
@@ -552,10 +672,11 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     __shared__ uint32_t out_base[kRadix];             // global minus local position of each digit's run in this tile
     __shared__ uint32_t scan_tmp[2 * kSortWaves];
 
-    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
+    const int c = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const DigitPlan dp = digit_plan(a.key_bits[c], a.pass);
     if (a.pass >= dp.passes - 1) return;        // block-uniform: this class has fewer scatter passes
+    const int tile = LookBack ? lov_take_ticket(a.tickets, c) : sort_tile(row_items(a, c));
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
     if (count <= 0) return;                     // block-uniform: the row ends before this tile
@@ -579,7 +700,9 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
     uint32_t dtot = 0, tile_before = 0;         // thread d < kRadix: digit d's total in the row, and in the tiles before this one
     if (threadIdx.x < kRadix) {
         dtot = a.digit_total[(int64_t)c * kRadix + threadIdx.x];
-        if (threadIdx.x <= dp.mask) tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile];
+        if constexpr (!LookBack) {
+            if (threadIdx.x <= dp.mask) tile_before = a.tile_hist[((int64_t)c * kRadix + threadIdx.x) * a.tiles_pad + tile];
+        }
     }
     for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) reinterpret_cast<uint32_t *>(&counts[0][0])[i] = 0;
     __syncthreads();
@@ -629,6 +752,10 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
                 run += t;
             }
             mine = run;
+            if constexpr (LookBack) {
+                if (d <= (int)dp.mask)
+                    tile_before = lov_look_back(a.desc + (int64_t)c * a.tiles * kRadix, tile, d, mine, a.timed_out);
+            }
         }
         uint32_t row_total, local_start, global_start;
         block_excl_scan2(mine, dtot, scan_tmp, local_start, n_local, global_start, row_total);
@@ -682,7 +809,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_scatter(const SortArgs a) {
 constexpr int kMinRegionBits = 13, kMaxRegionBits = 15;
 constexpr int kMaxRegions = 1024;             // per class row; larger rows take the direct scatter
 
-template <bool Binned>
+template <bool Binned, bool LookBack = false>
 __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, float *__restrict__ jacc,
                                                           float *__restrict__ tile_loss,
                                                           uint32_t *__restrict__ cursors, int regions, int region_bits) {
@@ -698,7 +825,7 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
     __shared__ uint32_t scan_tmp[2 * kSortWaves];
     __shared__ float wave_loss[kSortWaves];
 
-    const int c = blockIdx.y, tile = sort_tile(row_items(a, c));
+    const int c = blockIdx.y, tile = LookBack ? lov_take_ticket(a.tickets, c) : sort_tile(row_items(a, c));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int begin = tile * kSortTile;
     const int count = min(kSortTile, row_items(a, c) - begin);
@@ -728,9 +855,11 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
         const int64_t at = (int64_t)c * kRadix + threadIdx.x;
         dtot = a.digit_total[at];
         htot = a.hot_total[at];
-        if (threadIdx.x <= dp.mask) {
-            tile_before = a.tile_hist[at * a.tiles_pad + tile];
-            hot_before = a.tile_hot[at * a.tiles_pad + tile];
+        if constexpr (!LookBack) {
+            if (threadIdx.x <= dp.mask) {
+                tile_before = a.tile_hist[at * a.tiles_pad + tile];
+                hot_before = a.tile_hot[at * a.tiles_pad + tile];
+            }
         }
     }
     for (int i = threadIdx.x; i < kSortWaves * kRadix / 2; i += kSortThreads) {
@@ -789,6 +918,11 @@ __global__ __launch_bounds__(kSortThreads) void lov_final(const SortArgs a, floa
                 counts_hot[w][d] = (uint16_t)run_hot;
                 run += t;
                 run_hot += th;
+            }
+            if constexpr (LookBack) {
+                if (d <= (int)dp.mask)
+                    lov_look_back2(a.desc_wide + (int64_t)c * a.tiles * kRadix, tile, d, run, run_hot, tile_before, hot_before,
+                                   a.timed_out);
             }
         }
         uint32_t total, global_start, hot_start;
@@ -899,6 +1033,7 @@ __global__ __launch_bounds__(kUnbinThreads) void lov_unbin(float *__restrict__ j
     if (threadIdx.x == 0) {
         float total = 0.f;
         for (int w = 0; w < kUnbinThreads / 64; ++w) total += sorted[w];
+        if (a.timed_out && *a.timed_out) total = __builtin_nanf("");        // look-back variant: a wait ran out
         losses[c] = total;
     }
 }
@@ -1013,7 +1148,17 @@ struct LovaszPlan {
     int region_bits;        // log2 of the pixels per region
     int64_t off_keys_a, off_keys_c, off_vals_a, off_vals_b, off_hist, off_hot, off_digit_total, off_hot_total,
         off_tile_loss, off_cursors, off_class, off_block_max, bytes;
+    // look-back variant: tickets + time-out word + descriptors (cleared per call), totals, per-block tables
+    bool look_back;
+    int hist_blocks;
+    int64_t off_lb_clear, lb_clear_bytes, off_lb_totals, off_lb_partial;
 };
+
+// PLH_LOVASZ_SCAN=lookback selects the decoupled look-back variant of the sort passes (read at every call).
+static bool look_back_selected() {
+    const char *v = getenv("PLH_LOVASZ_SCAN");
+    return v && strcmp(v, "lookback") == 0;
+}
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
@@ -1044,6 +1189,15 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
     pl.off_class = off;       off += round_up(4 * dimsize * 4, 256);      // pos_max[C], kept[C], all_min[C], key_bits[C]
     pl.off_block_max = off;   off += round_up(4 * dimsize * ceil_div(pl.P, 256), 256);   // [key blocks][C]
+    pl.look_back = look_back_selected() && pl.regions > 0;
+    pl.hist_blocks = (int)ceil_div(pl.tiles, 2);
+    if (pl.look_back) {
+        // [4 passes][C] tickets + 1 word, 3 x [C][tiles][kRadix] u32 descriptors, [C][tiles][kRadix] u64 ones
+        pl.lb_clear_bytes = round_up(4 * (4 * dimsize + 1), 256) + (int64_t)(3 * 4 + 8) * dimsize * pl.tiles * kRadix;
+        pl.off_lb_clear = off;    off += round_up(pl.lb_clear_bytes, 256);
+        pl.off_lb_totals = off;   off += round_up(4 * (int64_t)kHistTables * dimsize * kRadix, 256);
+        pl.off_lb_partial = off;  off += round_up(4 * (int64_t)dimsize * pl.hist_blocks * kHistTables * kRadix, 256);
+    }
     pl.bytes = off;
     return PLH_OK;
 }
@@ -1135,6 +1289,10 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     // a histogram block counts two tiles; lov_row_scan reads the live tiles in whole groups of kSortWaves
     const dim3 hist_grid((unsigned)round_up(ceil_div(pl.tiles, 2), kSortWaves / 2), (unsigned)C);
     SortArgs a;
+    a.desc = nullptr;
+    a.desc_wide = nullptr;
+    a.tickets = nullptr;
+    a.timed_out = nullptr;
     a.keys_alt = nullptr;
     a.vals_alt = nullptr;
     a.tile_hist = hist;
@@ -1145,6 +1303,23 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     a.P = (int)pl.P;
     a.tiles = pl.tiles;
     a.tiles_pad = pl.tiles_pad;
+    uint32_t *lb_words = pl.look_back ? reinterpret_cast<uint32_t *>(ws + pl.off_lb_clear) : nullptr;
+    uint32_t *lb_desc = pl.look_back ? reinterpret_cast<uint32_t *>(ws + pl.off_lb_clear + round_up(4 * (4 * C + 1), 256)) : nullptr;
+    uint32_t *lb_totals = pl.look_back ? reinterpret_cast<uint32_t *>(ws + pl.off_lb_totals) : nullptr;
+    if (pl.look_back) {
+        // tickets, time-out word and descriptors start at zero; digit totals of every pass from one sweep over the keys
+        hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, reinterpret_cast<float *>(lb_words),
+                           pl.lb_clear_bytes / 4);
+        uint32_t *partial = reinterpret_cast<uint32_t *>(ws + pl.off_lb_partial);
+        a.keys_in = keys_0;
+        a.pos_max = pos_max;
+        a.all_min = all_min;
+        hipLaunchKernelGGL(lov_hist_all, dim3((unsigned)pl.hist_blocks, (unsigned)C), dim3(kSortThreads), 0, st, a, partial,
+                           pl.hist_blocks);
+        hipLaunchKernelGGL(lov_hist_reduce, dim3(kHistTables, (unsigned)C), dim3(kRadix), 0, st, partial, pl.hist_blocks, C,
+                           lb_totals);
+        a.timed_out = lb_words + 4 * C;
+    }
     for (int pass = 0; pass < 3; ++pass) {
         a.keys_in = pass == 0 ? keys_0 : (pass == 1 ? keys_a : keys_c);
         a.vals_in = pass == 0 ? nullptr : (pass == 1 ? vals_a : vals_b);
@@ -1155,10 +1330,17 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         a.all_min = (pass == 0) ? all_min : nullptr;
         a.kept_in = (pass == 0) ? nullptr : kept;
         a.kept_out = (pass == 0) ? kept : nullptr;
+        if (pl.look_back) {
+            a.digit_total = lb_totals + (int64_t)pass * C * kRadix;
+            a.desc = lb_desc + (int64_t)pass * C * pl.tiles * kRadix;
+            a.tickets = lb_words + pass * C;
+            hipLaunchKernelGGL(lov_scatter<true>, tile_grid, dim3(kSortThreads), 0, st, a);
+            continue;
+        }
         hipLaunchKernelGGL(lov_tile_hist<false>, hist_grid, dim3(kSortThreads), 0, st, a);
         hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 1), dim3(256), 0, st, hist, digit_total, hot,
                            hot_total, pl.tiles_pad, key_bits, pass, a.kept_in, (int)pl.P);
-        hipLaunchKernelGGL(lov_scatter, tile_grid, dim3(kSortThreads), 0, st, a);
+        hipLaunchKernelGGL(lov_scatter<false>, tile_grid, dim3(kSortThreads), 0, st, a);
     }
 
     // 3. last pass (the top digit of the class; bit 31 is never part of a digit) fused with the Jaccard
@@ -1174,15 +1356,26 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
     a.all_min = nullptr;
     a.kept_in = kept;
     a.kept_out = nullptr;
-    hipLaunchKernelGGL(lov_tile_hist<true>, hist_grid, dim3(kSortThreads), 0, st, a);
-    hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
-                       pl.tiles_pad, key_bits, kLastPass, kept, (int)pl.P);
+    if (pl.look_back) {
+        a.digit_total = lb_totals + (int64_t)3 * C * kRadix;
+        a.hot_total = lb_totals + (int64_t)4 * C * kRadix;
+        a.desc_wide = reinterpret_cast<unsigned long long *>(lb_desc + (int64_t)3 * C * pl.tiles * kRadix);
+        a.tickets = lb_words + 3 * C;
+    } else {
+        hipLaunchKernelGGL(lov_tile_hist<true>, hist_grid, dim3(kSortThreads), 0, st, a);
+        hipLaunchKernelGGL(lov_row_scan, dim3(kRadix, (unsigned)C, 2), dim3(256), 0, st, hist, digit_total, hot, hot_total,
+                           pl.tiles_pad, key_bits, kLastPass, kept, (int)pl.P);
+    }
     if (pl.regions > 0) {
         uint32_t *cursors = reinterpret_cast<uint32_t *>(ws + pl.off_cursors);      // zeroed by lov_class_max
         // the value buffer that a class's last pass does not read receives the pixel offsets that go with
         // the staged values
-        hipLaunchKernelGGL(lov_final<true>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, cursors,
-                           pl.regions, pl.region_bits);
+        if (pl.look_back)
+            hipLaunchKernelGGL((lov_final<true, true>), tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, cursors,
+                               pl.regions, pl.region_bits);
+        else
+            hipLaunchKernelGGL((lov_final<true, false>), tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, cursors,
+                               pl.regions, pl.region_bits);
         const dim3 unbin_grid((unsigned)pl.regions, (unsigned)C);
         switch (pl.region_bits) {
 #define PLH_UNBIN(B)                                                                                                  \
@@ -1197,7 +1390,7 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         // direct scatter: the pixels whose keys stayed out of the sort are not written, so clear first
         // (jacc stopped being a key buffer when the first pass read it)
         hipLaunchKernelGGL(lov_zero_f32, dim3(4096), dim3(256), 0, st, jacc, pl.E);
-        hipLaunchKernelGGL(lov_final<false>, tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, 0, 0);
+        hipLaunchKernelGGL((lov_final<false, false>), tile_grid, dim3(kSortThreads), 0, st, a, jacc, tile_loss, nullptr, 0, 0);
         hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     }
     return check_launch();
