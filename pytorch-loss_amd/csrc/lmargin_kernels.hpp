@@ -56,10 +56,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     float go[V];
     if constexpr (WantGrad) at.upstream(up, go);
 
-    // Four pixels per lane: a pixel's gradient takes the place of its logits in the slice as soon as it
+    // Four fp32 pixels per lane: a pixel's gradient takes the place of its logits in the slice as soon as it
     // is formed, and the pixels are worked through one after the other (no second array, no four
-    // pixels' intermediates alive at once).
-    constexpr bool kInPlace = (Form == kPerImage);
+    // pixels' intermediates alive at once). 16-bit pixels share dwords in pairs and keep the second array.
+    constexpr bool kInPlace = (Form == kPerImage) && sizeof(T) == 4;
     float out[V], score[V];
     float g[(WantGrad && !kInPlace) ? CP : 1][V];
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
@@ -759,18 +759,20 @@ static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, 
     return grid;
 }
 
-// fp32 NCHW whose channel planes have odd length: the per-image form, four pixels per lane.
-template <bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-static unsigned launch_image(const float *x, const int64_t *lab, const Upstream &up, float *loss, float *grad,
+// NCHW whose channel planes start on element boundaries only (odd lengths): the per-image form, four
+// pixels per lane.
+template <class T, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+static unsigned launch_image(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                              unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
-        hipLaunchKernelGGL((lm_regs<float, 4 * K, 4, kPerImage, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
-                           dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                           \
+        if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                             \
+            hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
+                               dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                       \
         break;
-        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
     return grid;
@@ -826,11 +828,9 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             blocks = launch_regs<T, V, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::RegsOne:
-            if constexpr (std::is_same<T, float>::value) {
-                if (image_form_pays(p.C, p.m_size)) {
-                    blocks = launch_image<WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
-                    break;
-                }
+            if (image_form_pays<T>(p.C, p.m_size)) {
+                blocks = launch_image<T, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+                break;
             }
             blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;

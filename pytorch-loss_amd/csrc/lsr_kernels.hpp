@@ -786,33 +786,37 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
     }
 }
 
-// fp32 NCHW whose channel planes have odd length: the per-image form, four pixels per lane.
-template <bool Reduce>
-static unsigned launch_fwd_image(const float *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
+// NCHW whose channel planes start on element boundaries only (odd lengths): the per-image form, four
+// pixels per lane.
+template <class T, bool Reduce>
+static unsigned launch_fwd_image(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                  hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                               \
     case K:                                                                                                       \
-        hipLaunchKernelGGL((lsr_fwd_regs<float, 4 * K, 4, kPerImage, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
-                           st, x, lab, loss, part, p);                                                            \
+        if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                          \
+            hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, 4, kPerImage, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
+                               st, x, lab, loss, part, p);                                                        \
         break;
-        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
     return grid;
 }
 
-static void launch_bwd_image(const float *x, const int64_t *lab, const Upstream &up, float *grad, const LsrParams &p,
+template <class T>
+static void launch_bwd_image(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
                              hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                              \
     case K:                                                                                                      \
-        hipLaunchKernelGGL((lsr_bwd_regs<float, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                           lab, up, grad, p);                                                                    \
+        if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                         \
+            hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
+                               lab, up, grad, p);                                                                \
         break;
-        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6)
+        PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
 }
@@ -825,9 +829,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::RegsOne:
-            if constexpr (std::is_same<T, float>::value) {
-                if (image_form_pays(p.C, p.m_size)) return launch_fwd_image<Reduce>(logits, labels, losses, part, p, st);
-            }
+            if (image_form_pays<T>(p.C, p.m_size)) return launch_fwd_image<T, Reduce>(logits, labels, losses, part, p, st);
             return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
@@ -867,11 +869,9 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::RegsOne:
-            if constexpr (std::is_same<T, float>::value) {
-                if (image_form_pays(p.C, p.m_size)) {
-                    launch_bwd_image(logits, labels, up, grad_logits, p, st);
-                    break;
-                }
+            if (image_form_pays<T>(p.C, p.m_size)) {
+                launch_bwd_image<T>(logits, labels, up, grad_logits, p, st);
+                break;
             }
             launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st);
             break;

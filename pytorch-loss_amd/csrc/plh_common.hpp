@@ -294,6 +294,8 @@ template <> struct Pack<float, 4> {
     static __device__ __forceinline__ void store(float *p, Raw r) {
         __builtin_nontemporal_store(plh_u4w_a4{r.x, r.y, r.z, r.w}, reinterpret_cast<plh_u4w_a4 *>(p));
     }
+    static __device__ __forceinline__ Raw load_unaligned(const float *p) { return load(p); }
+    static __device__ __forceinline__ void store_unaligned(float *p, Raw r) { store(p, r); }
     static __device__ __forceinline__ float get(Raw r, int k) { return bits_f32(k == 0 ? r.x : (k == 1 ? r.y : (k == 2 ? r.z : r.w))); }
     static __device__ __forceinline__ Raw put(const float (&g)[4]) {
         return Raw{f32_bits(g[0]), f32_bits(g[1]), f32_bits(g[2]), f32_bits(g[3])};
@@ -336,6 +338,7 @@ __device__ __forceinline__ float widen_hi(unsigned d, f16) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(d >> 16));
 }
 
+typedef unsigned plh_u2_a2 __attribute__((ext_vector_type(2), aligned(2)));
 template <class T> struct Pack<T, 4> {          // T = f16 or bf16
     typedef plh_u2 Raw;
     static __device__ __forceinline__ Raw load(const T *p) {
@@ -343,6 +346,14 @@ template <class T> struct Pack<T, 4> {          // T = f16 or bf16
     }
     static __device__ __forceinline__ void store(T *p, Raw r) {
         __builtin_nontemporal_store(r, reinterpret_cast<plh_u2 *>(p));
+    }
+    // the same 8 bytes from any element boundary (the per-image form on channel planes of odd length)
+    static __device__ __forceinline__ Raw load_unaligned(const T *p) {
+        const plh_u2_a2 t = __builtin_nontemporal_load(reinterpret_cast<const plh_u2_a2 *>(p));
+        return Raw{t.x, t.y};
+    }
+    static __device__ __forceinline__ void store_unaligned(T *p, Raw r) {
+        __builtin_nontemporal_store(plh_u2_a2{r.x, r.y}, reinterpret_cast<plh_u2_a2 *>(p));
     }
     static __device__ __forceinline__ float get(Raw r, int k) {
         const unsigned d = k < 2 ? r.x : r.y;
@@ -573,9 +584,10 @@ __device__ __forceinline__ plh_u4 rows_gather16(const Word *tile, int e) {
 //              (images) x (tiles per image), a lane takes V consecutive pixels of ONE image and the last
 //              lane of an image may hold fewer (`nv`); its accesses then go pixel by pixel, and the pixels
 //              it does not have read as ignored. Channel planes of odd length (513 x 513, 769 x 769 crops)
-//              start on 4-byte boundaries only, which would leave one pixel per lane and 256-byte runs of
-//              which every third cache line is shared with a neighbour; V = 4 with 16-byte accesses on
-//              4-byte boundaries makes that every ninth.
+//              start on element boundaries only, which would leave one pixel per lane and runs of 256 (fp32)
+//              or 128 bytes (16-bit) that share their first and last cache line with a neighbour; V = 4 with
+//              16-byte (fp32) or 8-byte (16-bit) accesses on element boundaries makes the runs 1 KiB and
+//              512 bytes (the hardware takes such accesses; the vector types of Pack<T, 4> say so).
 constexpr int kGeneral = 0, kUniform = 1, kPerImage = 2;
 
 // Grid of the per-image form.
@@ -585,9 +597,11 @@ inline unsigned image_grid(int64_t n_size, int64_t m_size) {
 }
 
 // Where the host picks it over one pixel per lane: planes long enough that the partly filled last
-// block of every image is a small share, and slices that four pixels per lane still keep in registers.
-constexpr int kImageFormMaxChannels = 24;
-inline bool image_form_pays(int C, int64_t m_size) { return C <= kImageFormMaxChannels && m_size >= 4096; }
+// block of every image is a small share, and slices that four pixels per lane still keep in registers
+// (a 16-bit slice takes half the registers of an fp32 one).
+template <class T> constexpr int kImageFormMaxChannels = sizeof(T) == 4 ? 24 : 32;
+template <class T>
+inline bool image_form_pays(int C, int64_t m_size) { return C <= kImageFormMaxChannels<T> && m_size >= 4096; }
 
 template <int V, int Form>
 struct PixelRef {
@@ -803,7 +817,10 @@ struct PixelRef {
             }
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (chan_ok<CP>(j, C)) raw[j] = Pack<T, V>::load(chan(t, j, m_size));
+                if (chan_ok<CP>(j, C)) {
+                    if constexpr (Form == kPerImage) raw[j] = Pack<T, V>::load_unaligned(chan(t, j, m_size));
+                    else raw[j] = Pack<T, V>::load(chan(t, j, m_size));
+                }
         }
     }
     template <class T, int CP>
@@ -837,7 +854,10 @@ struct PixelRef {
             }
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (chan_ok<CP>(j, C)) Pack<T, V>::store(chan(t, j, m_size), raw[j]);
+                if (chan_ok<CP>(j, C)) {
+                    if constexpr (Form == kPerImage) Pack<T, V>::store_unaligned(chan(t, j, m_size), raw[j]);
+                    else Pack<T, V>::store(chan(t, j, m_size), raw[j]);
+                }
         }
     }
 };

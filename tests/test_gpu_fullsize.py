@@ -122,6 +122,48 @@ def test_odd_crops_full_size(pl, kind, shape):
     assert torch.equal(alone, per[k:k + 1].detach())
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("kind,shape", [("lsr", (6, 19, 769, 769)), ("lmargin", (9, 19, 513, 513))])
+def test_odd_crops_full_size_16bit(pl, kind, shape, dt):
+    """The same crops with 16-bit logits (tiles per image, four pixels per lane, 8-byte accesses that start on
+    2-byte boundaries): exact zeros at ignored pixels, 'mean' against the per-pixel losses, the oracle on the
+    stored values of the last image to one step of the storage type, no dependence on the batch position."""
+    x = synth.normal(33, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(33, shape[:1] + shape[2:], shape[1], 255, 0.05)
+    xt = torch.from_numpy(x).cuda().to(dt).requires_grad_()
+    yt = torch.from_numpy(y).cuda()
+    k = shape[0] - 1
+    xr = xt[k:k + 1].detach().float().cpu().numpy()
+    if kind == "lsr":
+        make = lambda red: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=255)
+        want = oracle.lsr_forward(xr, y[k:k + 1], 255, 0.1)
+        want_g = oracle.lsr_backward(xr, y[k:k + 1], 255, 0.1, None)
+    else:
+        make = lambda red: pl.LargeMarginSoftmaxV3(lam=0.3, reduction=red, ignore_index=255)
+        want = oracle.lmargin_forward(xr, y[k:k + 1], 0.3, 255)
+        want_g = oracle.lmargin_backward(xr, y[k:k + 1], 0.3, 255, None)
+    n_valid = int((y != 255).sum())
+    with torch.autocast("cuda", dtype=dt):
+        mean = make("mean")(xt, yt)
+        per = make("none")(xt, yt)
+    assert per.dtype == torch.float32 and mean.dtype == torch.float32
+    per.sum().backward()
+    g_sum = xt.grad
+    assert g_sum.dtype == dt
+    assert abs(mean.item() - per.double().sum().item() / n_valid) <= 1e-6 * abs(mean.item())
+    ign = yt == 255
+    assert (per[ign] == 0).all() and (per[~ign] > 0).all()
+    assert (g_sum.permute(0, 2, 3, 1)[ign] == 0).all()
+    got = per[k:k + 1].detach().cpu().numpy()
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6)
+    ulp = 2.0 ** -10 if dt == torch.float16 else 2.0 ** -7      # one step of the storage type
+    got_g = g_sum[k:k + 1].float().cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got_g - want_g) <= ulp * np.abs(want_g) + 1e-6)    # + fp32 arithmetic on values of order one
+    with torch.autocast("cuda", dtype=dt):
+        alone = make("none")(xt[k:k + 1].detach().contiguous(), yt[k:k + 1].contiguous())
+    assert torch.equal(alone, per[k:k + 1].detach())
+
+
 def test_focal_full_size(pl):
     w = synth.workload("cfg3")
     x, y = w["logits"], w["labels"]

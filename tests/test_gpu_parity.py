@@ -114,6 +114,8 @@ SEG_CASES = [
     ((2, 24, 4097, 1), 255, 0.1),                   #   1 or 3 pixels; the widest slice that takes this form,
     ((1, 25, 65, 65), 255, 0.1),                    #   one channel more and one pixel fewer than its limits
     ((2, 24, 63, 65), 255, 0.1),
+    ((2, 32, 65, 65), 255, 0.1),                    # 16-bit slices take that form up to 32 channels (8-byte accesses
+    ((1, 29, 67, 63), -100, 0.1),                   #   on 2-byte boundaries); fp32 keeps one pixel per lane here
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
