@@ -36,7 +36,7 @@ __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)(
 
 // ------------------------------------------------------------------ scores ----
 
-template <class T, int CP, int V, bool Uniform>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                               float *__restrict__ scores, float *__restrict__ ce,
                                                               int64_t P, int64_t m_size, int C, int64_t ignore,
@@ -44,12 +44,12 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
     // the selection's tables start at zero; the kernels that fill them are launched after this one
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kRegsBlock) tables[i] = 0;
-    const PixelRef<V, Uniform> at(P, m_size, C, xcd_run);
+    const PixelRef<V, Form> at(P, m_size, C, xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, C, m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, ignore, lb);
     float out[V], loss[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
@@ -74,8 +74,8 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
         loss[k] = (tgt < 0) ? 0.f : __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, mx - x_y);
     }
     // the selection kernels read both back several times: leave them to the caches
-    store_vec_cached<V>(scores + at.pix, out);
-    if (ce) store_vec_cached<V>(ce + at.pix, loss);
+    at.store_f32_cached(scores, out);
+    if (ce) at.store_f32_cached(ce, loss);
 }
 
 // 33..256 channels in NCHW (SplitSlice): per wavefront the maximum, the exponential sum and the target's
@@ -551,17 +551,23 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         } else if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
             const bool vec = (shape == Shape::RegsVec);
             const bool uni = vec && tiles_are_uniform(m_size, VT, sizeof(T));
-            const unsigned grid = vec ? regs_grid<VT>(P) : regs_grid<1>(P);
+            // planes that start on element boundaries only: tiles per image, four pixels per lane
+            const bool image = !vec && image_form_pays<T>(C, m_size);
+            const unsigned grid = vec ? regs_grid<VT>(P) : (image ? image_grid<4>(n_size, m_size) : regs_grid<1>(P));
             const unsigned run = xcd_run_for(sizeof(T), m_size);
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
-        if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, true>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                                    labels, scores, ce, P, m_size, C, ignore_index, run, tables);                     \
-        else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, false>), dim3(grid), dim3(kRegsBlock), 0,    \
+        if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kUniform>), dim3(grid), dim3(kRegsBlock), 0, st,  \
+                                    x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);                  \
+        else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, \
                                          st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);         \
-        else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, false>), dim3(grid), dim3(kRegsBlock), 0, st, x,       \
-                                labels, scores, ce, P, m_size, C, ignore_index, run, tables);                         \
+        else if (image) {                                                                                             \
+            if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                          \
+                hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st,   \
+                                   x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);                   \
+        } else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x,  \
+                                  labels, scores, ce, P, m_size, C, ignore_index, run, tables);                       \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

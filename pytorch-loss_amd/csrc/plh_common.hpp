@@ -408,6 +408,7 @@ template <class T> struct Pack<T, 1> {          // T = f16 or bf16
 // the second evaluation costs instructions).
 __device__ __forceinline__ void forget_origin(unsigned &r) { asm volatile("" : "+v"(r)); }
 __device__ __forceinline__ void forget_origin(plh_u2 &r) { asm volatile("" : "+v"(r.x), "+v"(r.y)); }
+__device__ __forceinline__ void forget_origin(plh_u4w &r) { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
 
 // A regs kernel is instantiated for CP = channels rounded up to a multiple of 4, and launched only
 // for CP-3 <= C <= CP: the first CP-3 channel slots always exist, the last three are checked.
@@ -597,11 +598,12 @@ inline unsigned image_grid(int64_t n_size, int64_t m_size) {
 }
 
 // Where the host picks it over one pixel per lane: planes long enough that the partly filled last
-// block of every image is a small share, and slices that four pixels per lane still keep in registers
-// (a 16-bit slice takes half the registers of an fp32 one).
-template <class T> constexpr int kImageFormMaxChannels = sizeof(T) == 4 ? 24 : 32;
-template <class T>
-inline bool image_form_pays(int C, int64_t m_size) { return C <= kImageFormMaxChannels<T> && m_size >= 4096; }
+// block of every image is a small share, and slices that four pixels per lane still keep in registers:
+// 96 dwords for all the slices a kernel holds (a 16-bit slice takes half the registers of an fp32 one).
+template <class T, int Slices = 1>
+constexpr int kImageFormMaxChannels = (96 / (Slices * (int)sizeof(T)) < kMaxRegsChannels) ? 96 / (Slices * (int)sizeof(T)) : kMaxRegsChannels;
+template <class T, int Slices = 1>
+inline bool image_form_pays(int C, int64_t m_size) { return C <= kImageFormMaxChannels<T, Slices> && m_size >= 4096; }
 
 template <int V, int Form>
 struct PixelRef {

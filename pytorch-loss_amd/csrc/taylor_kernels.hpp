@@ -66,10 +66,10 @@ __device__ __forceinline__ void taylor_pair(float x, int order, float &f, float 
 
 // ---------------------------------------------------------------- regs ----
 
-template <class T, int CP, int V, bool Uniform>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restrict__ x, T *__restrict__ out,
                                                              const TaylorParams p) {
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
@@ -103,10 +103,10 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
     at.store_slice(out, p.C, p.m_size, raw);
 }
 
-template <class T, int CP, int V, bool Uniform>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restrict__ g, const T *__restrict__ x,
                                                              T *__restrict__ gx, const TaylorParams p) {
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP], graw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
@@ -153,17 +153,17 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
 }
 
 // Cross entropy on the log form: loss per pixel (fp32), and its gradient with the upstream folded in.
-template <class T, int CP, int V, bool Uniform, bool Reduce>
+template <class T, int CP, int V, int Form, bool Reduce>
 __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 float *__restrict__ loss, Partials part,
                                                                 const TaylorParams p) {
     __shared__ float red[4];
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     float out[V];
     float mine = 0.f;
     int cnt = 0;
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
         mine += out[k];
         cnt += (at.live && !ign) ? 1 : 0;
     }
-    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if (at.live && loss) at.store_f32(loss, out);
     if constexpr (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);
@@ -196,18 +196,18 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
     }
 }
 
-template <class T, int CP, int V, bool Uniform>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 const Upstream up, T *__restrict__ gx,
                                                                 const TaylorParams p) {
-    const PixelRef<V, Uniform> at(p.P, p.m_size, p.C, p.xcd_run);
+    const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     float go[V];
-    load_upstream<V>(up, at.pix, go);
+    at.upstream(up, go);
     // first per pixel (sum of the series, the target's term), then channel by channel so that only one
     // packed result is live at a time
     unsigned keep[V];
@@ -740,7 +740,11 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
         const bool vec = (shape == Shape::RegsVec) && g_ok;
         const bool uni = vec && tiles_are_uniform(p.m_size, VT, sizeof(T));
-        const unsigned grid = vec ? regs_grid<VT>(p.P) : regs_grid<1>(p.P);
+        // planes that start on element boundaries only: tiles per image, four pixels per lane (the softmax
+        // backward holds two slices, so half the channels)
+        constexpr int kSlices = (Kind == kTaylorBwd) ? 2 : 1;
+        const bool image = !vec && image_form_pays<T, kSlices>(p.C, p.m_size);
+        const unsigned grid = vec ? regs_grid<VT>(p.P) : (image ? image_grid<4>(p.P / p.m_size, p.m_size) : regs_grid<1>(p.P));
 #define PLH_GO(CPV, VV, UU)                                                                                          \
     do {                                                                                                             \
         if constexpr (Kind == kTaylorFwd)                                                                            \
@@ -755,11 +759,14 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                                up, out, p);                                                                          \
     } while (0)
         switch ((p.C + 3) / 4) {
-#define PLH_CASE(K)                       \
-    case K:                               \
-        if (uni) PLH_GO(4 * K, VT, true); \
-        else if (vec) PLH_GO(4 * K, VT, false); \
-        else PLH_GO(4 * K, 1, false);     \
+#define PLH_CASE(K)                                                    \
+    case K:                                                            \
+        if (uni) PLH_GO(4 * K, VT, kUniform);                          \
+        else if (vec) PLH_GO(4 * K, VT, kGeneral);                     \
+        else if (image) {                                              \
+            if constexpr (4 * K <= kImageFormMaxChannels<T, kSlices>)  \
+                PLH_GO(4 * K, 4, kPerImage);                           \
+        } else PLH_GO(4 * K, 1, kGeneral);                             \
         break;
             PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE

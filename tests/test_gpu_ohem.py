@@ -59,6 +59,11 @@ SCORE_CASES = [
     ((1, 449, 8, 8), -100, 0.2),
     ((1, 512, 8, 9), 255, 0.1),
     ((1, 513, 8, 8), 255, 0.1),          # one channel more: a lane per pixel
+    ((2, 19, 65, 65), 255, 0.05),        # planes of odd length, 4096 pixels or more: tiles per image, four pixels
+    ((3, 5, 71, 61), -100, 0.1),         #   per lane, the last lane of an image with 1 or 3 pixels; the widest
+    ((2, 24, 4097, 1), 255, 0.1),        #   slices that take this form (24 channels fp32, 32 for 16-bit logits)
+    ((2, 32, 65, 65), 255, 0.1),
+    ((1, 25, 63, 65), 255, 0.1),
     ((2, 19, 16, 16), 255, 1.0),         # everything ignored
 ]
 

@@ -35,6 +35,10 @@ CASES = [
     ((2, 2056), 1),                              # beyond the register rows: a block per row
     ((3, 4099), 1),                              #   odd length: element by element
     ((2, 30000), -1),                            #   1024-thread blocks
+    ((2, 19, 65, 65), 1),                        # planes of odd length, 4096 pixels or more: tiles per image, four
+    ((2, 11, 67, 63), 1),                        #   pixels per lane where the slices fit (the backward holds two:
+    ((1, 24, 4097, 1), 1),                       #   12 channels fp32, 24 for 16-bit elements; the forward one: 24 / 32)
+    ((2, 25, 65, 65), 1),
 ]
 
 
@@ -73,7 +77,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-11:])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-15:])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
@@ -156,8 +160,9 @@ def test_cross_entropy_equals_the_reference_composition(pl):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-def test_cross_entropy_16bit(pl, dt):
-    x, y = seg_inputs(106, (2, 19, 32, 32), 255, 0.1)
+@pytest.mark.parametrize("shape", [(2, 19, 32, 32), (2, 19, 65, 65), (2, 32, 63, 65), (1, 33, 65, 65)])
+def test_cross_entropy_16bit(pl, dt, shape):
+    x, y = seg_inputs(106, shape, 255, 0.1)
     xt = dev(x * 0.5).to(dt).requires_grad_()
     xr = xt.detach().float().cpu().numpy().astype(np.float64)
     with torch.autocast("cuda", dtype=dt):
