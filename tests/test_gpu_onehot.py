@@ -21,6 +21,8 @@ CASES = [
     ((2, 5, 7), 227),
     ((1, 2, 3, 4), 64),
     ((4, 1024, 256), 19),
+    ((2, 1028, 1024), 3),                        # planes of more than 2^20 pixels go chunk by chunk, the last one short
+    ((1, 2048, 1025), 5),                        #   (2 and 3 chunks)
 ]
 
 
