@@ -320,12 +320,20 @@ __device__ __forceinline__ void hist_add(uint32_t *bins, float s, uint32_t high_
 // block resolves first. (A device-wide "last block resolves it" would need a release fence in every
 // block, which costs more than this redundant scan of 1024 counts on a GPU whose XCDs have separate
 // L2s; so does a launch of its own.)
+// Once the digits resolved so far put the n_min-th smallest score at or below the threshold whatever its
+// remaining digits are, the rule is "drop what lies above the threshold" and nothing finer is needed: the
+// later passes leave their histograms empty (every block returns before it reads a score), the digits they
+// resolve from those come out as 0, and the key that ohem_ties publishes stays below the threshold.
 __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ scores, OhemTables tb, int P, int pass,
-                                                 uint32_t n_min, int vec) {
+                                                 uint32_t n_min, float thresh, int vec) {
     __shared__ uint32_t bins[kOhemBins];
     __shared__ uint32_t scan[260];
     for (int i = threadIdx.x; i < kOhemBins; i += 256) bins[i] = 0;
     const uint32_t prefix = pass == 0 ? 0u : ohem_resolve_digit(tb, pass - 1, n_min, scan, blockIdx.x == 0);
+    if (pass > 0) {
+        const uint32_t largest = prefix | ((1u << (30 - 10 * pass)) - 1u);      // block-uniform
+        if (__builtin_bit_cast(float, largest) <= thresh) return;
+    }
     __syncthreads();
     const uint32_t high_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (30 - 10 * pass));
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
@@ -631,7 +639,7 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         // addresses: 512 blocks (two per compute unit) measured 30 us faster than 2048 on 8 M scores
         const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
         for (int pass = 0; pass < 3; ++pass)
-            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, vec);
+            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, score_thresh, vec);
         hipLaunchKernelGGL(ohem_ties, dim3(kTieRuns / 4), dim3(256), 0, st, scores, tb, Pi, (int)tiles, k, score_thresh, vec);
     }
     hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, (int)tiles, k,
