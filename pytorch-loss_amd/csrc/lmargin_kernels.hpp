@@ -835,7 +835,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::Wave:
-            if (p.C <= kWaveRowCap) {
+            if (p.C <= wrow_cap<T>(wrow_wide<T>(x, WantGrad ? grad : nullptr, p.C))) {
                 const T *wrow_grad = WantGrad ? grad : nullptr;
 #define PLH_GO(NI, W, G)                                                                                           \
     do {                                                                                                           \

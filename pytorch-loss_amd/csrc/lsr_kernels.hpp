@@ -834,9 +834,9 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
-            if (p.C > kWaveRowCap) {
+            if (p.C > wrow_cap<T>(wrow_wide<T>(logits, nullptr, p.C))) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, logits, labels, losses, part, p,
+                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
@@ -878,13 +878,16 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::SplitDeep: launch_bwd_split<T, V / 2>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
-            if (p.C > kWaveRowCap) {
+            if (p.C > wrow_cap<T>(wrow_wide<T>(logits, grad_logits, p.C))) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
                 // chunks a row can have at most, and the threads that share them: 256 while 16 chunks per thread do
                 const int chunks = p.C / RowChunk<T>::kLen + 1;
                 const int threads = chunks <= kRowBlockShort * 16 ? kRowBlockShort : kRowBlock;
                 const int per = (chunks + threads - 1) / threads;
-                if (row_chunks_ok<T>(logits, grad_logits, p.C) && per <= 16) {
+                // 16 chunks per thread only in the 256-thread blocks: with 1024 threads they leave one block per
+                // compute unit and lose to the two sweeps below (fp32 (4096, 50257) 0.641 against 0.365 ms,
+                // (6144, 40000) 0.849 against 0.419; bf16 (2048, 128256) 0.276 against 0.246)
+                if (row_chunks_ok<T>(logits, grad_logits, p.C) && per <= (threads == kRowBlockShort ? 16 : 8)) {
                     if (per <= 4)
                         hipLaunchKernelGGL((lsr_bwd_rowregs<T, 4>), dim3(grid), dim3(threads), 0, st, logits, labels, up,
                                            grad_logits, p);

@@ -580,7 +580,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
-        } else if (shape == Shape::Wave && C <= kWaveRowCap) {
+        } else if (shape == Shape::Wave && C <= wrow_cap<T>(wrow_wide<T>(x, nullptr, C))) {
 #define PLH_GO(NI, W, G)                                                                                            \
     hipLaunchKernelGGL((ohem_scores_wrow<T, NI, W, G>), dim3(group_grid(P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
                        st, x, labels, scores, ce, P, C, ignore_index, tables)
@@ -588,7 +588,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #undef PLH_GO
         } else if (shape == Shape::Wave) {
             const unsigned grid = (unsigned)(P < 1 ? 1 : (P < kMinPartialSlots ? P : kMinPartialSlots));
-            hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(row_threads_for(C)), 0, st, x, labels, scores, ce, P, C,
+            hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(row_threads_for_sweep<T>(C)), 0, st, x, labels, scores, ce, P, C,
                                ignore_index, tables, row_chunks_ok<T>(x, nullptr, C));
         } else {
             hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,

@@ -1111,6 +1111,11 @@ struct WaveRowAt {
 // moved in 16-byte chunks when every row starts on a 16-byte boundary.
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
+// 16-bit rows that move in chunks go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the same 64
+// registers as an fp32 row of 2048); a block per row spends most of such a short row's time in its barriers
+// (bf16 LSR forward at (65536, 4096): 45 % of peak).
+template <class T>
+inline int wrow_cap(bool wide) { return (wide && sizeof(T) == 2) ? 2 * kWaveRowCap : kWaveRowCap; }
 
 template <class T>
 static bool wrow_wide(const T *x, const T *grad, int C) {
@@ -1145,10 +1150,8 @@ static int wrow_steps(int C, bool wide, int lanes) {
                 case 2: LAUNCH(2, true, 64); break;              /* chunks only */      \
                 case 4: LAUNCH(4, true, 64); break;              /* chunks only */      \
                 case 8:                                                                  \
-                    if constexpr (RowChunk<T>::kLen == 4) {                              \
-                        if (wrow_is_wide) { LAUNCH(8, true, 64); break; }                \
-                    }                                                                    \
-                    LAUNCH(8, false, 64);   /* 16-bit chunks never need 8 steps */       \
+                    if (wrow_is_wide) { LAUNCH(8, true, 64); break; }                    \
+                    LAUNCH(8, false, 64);                                                \
                     break;                                                               \
                 case 16: LAUNCH(16, false, 64); break;                                   \
                 default: LAUNCH(32, false, 64); break;                                   \
@@ -1167,6 +1170,12 @@ constexpr int kRowShortMax = 24576;  // lane where there was one, a quarter of t
                                      // Measured fp32 LSR fwd+bwd, 256 against 1024 threads: (16384, 4096) 0.153 / 0.223 ms,
                                      // (8192, 16384) 0.339 / 0.355, (4096, 21841) 0.230 / 0.228, (8192, 32000) 0.679 / 0.605
 inline int row_threads_for(int C, int short_max = kRowShortMax) { return C <= short_max ? kRowBlockShort : kRowBlock; }
+// The same limit for a forward sweep, by the bytes of a row (112 KiB): what decides is how long a block's loads are
+// in flight against the reduction that follows them, and a 16-bit row of 32000 or 50257 elements is a short one.
+// Measured bf16 forward, 256 against 1024 threads: LSR (8192, 32000) 0.106 / 0.142 ms, (4096, 50257) 0.085 / 0.091,
+// (2048, 128256) 0.106 / 0.100; Taylor cross entropy (8192, 32000) 0.113 / 0.164 (its backward 0.263 / 0.420).
+template <class T>
+inline int row_threads_for_sweep(int C) { return (int64_t)C * (int64_t)sizeof(T) <= 112 * 1024 ? kRowBlockShort : kRowBlock; }
 __device__ __forceinline__ int row_threads() { return (int)blockDim.x; }      // either of the two
 
 struct RowStats { float m, s, sx; };

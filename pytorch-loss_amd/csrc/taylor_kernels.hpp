@@ -775,10 +775,14 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         return grid;
     }
     if (p.m_size == 1) {
-        if (p.C <= kWaveRowCap) {
+        const bool wide = wrow_wide<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C) &&
+                          !(Kind == kTaylorBwd && misaligned(g, 16));
+        // the backwards keep the 2048-element limit: the softmax backward holds two rows in registers, and the
+        // cross-entropy backward with 64 registers of row ran at a third of its two-sweep form (bf16 (65536, 4096):
+        // 0.782 against 0.304 ms)
+        constexpr bool kForward = (Kind == kTaylorFwd || Kind == kTaylorCeFwd);
+        if (p.C <= (kForward ? wrow_cap<T>(wide) : kWaveRowCap)) {
             unsigned grid = 0;
-            const bool wide = wrow_wide<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C) &&
-                              !(Kind == kTaylorBwd && misaligned(g, 16));
 #define PLH_GO(NI, W, G)                                                                                          \
     do {                                                                                                          \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                      \
@@ -791,11 +795,11 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         }
         const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
         if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
-            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, x, lab, up, out, loss,
+            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, lab, up, out, loss,
                                part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
         } else {
             const int vec = row_chunks_ok<T>(x, out, p.C) && !(Kind == kTaylorBwd && misaligned(g, 16));
-            hipLaunchKernelGGL((taylor_sm_row<T, Kind>), dim3(grid), dim3(row_threads_for(p.C)), 0, st, x, g, out, p, vec);
+            hipLaunchKernelGGL((taylor_sm_row<T, Kind>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, g, out, p, vec);
         }
         return grid;
     }

@@ -83,10 +83,13 @@ SEG_CASES = [
     ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
     ((2, 2048), 255, 0.0),
     ((2, 2049), -100, 0.0),                         # one channel more: staged or swept rows
+    ((4, 3000), -100, 0.1),                         # 16-bit rows in whole chunks stay in a wavefront's registers up to
+    ((3, 4096), 255, 0.1),                          #   4096 elements (8 steps of 8); fp32 rows take a block per row
     ((3, 4100), 255, 0.0),                          # row longer than the LDS staging buffer
     ((5, 4104), 255, 0.2),                          # ... a multiple of 8 elements: 16-byte chunks for 16-bit rows too
     ((2, 4099), -100, 0.0),                         # ... an odd length: element by element
     ((3, 50000), 255, 0.3),                         # a vocabulary
+    ((2, 60000), 255, 0.0),                         #   one whose 16-bit rows exceed the 256-thread blocks' 112 KiB as well
     ((2, 33, 6, 7), 255, 0.2),                      # deep channel dim in NCHW: one lane per pixel
     ((2, 227, 5, 5), 255, 0.1),
     ((1, 64, 2, 3, 4), 0, 0.3),                     # 5-D input, ignore_index inside the class range
