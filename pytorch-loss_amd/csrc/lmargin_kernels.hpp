@@ -478,13 +478,13 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 // (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
 // sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group.
 
-template <class T, int NI, bool Wide, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G>
+template <class T, int NI, int LP, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G>
 __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
                                                const LmParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
     const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
@@ -493,7 +493,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         const bool live = r0 + at.grp < p.P;
         const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide, G> r;
+        WaveRow<T, NI, LP, G> r;
         r.load(xs, p.C, lane);
         const int64_t lb = lab[row];
         const bool ign = (lb == p.ignore);
@@ -558,8 +558,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             if constexpr (WantGrad) {
                 if (ok && live) {
                     T *gs = grad + row * p.C + e0;
-                    if constexpr (Wide) RowChunk<T>::store(gs, g);
-                    else store_one(gs, g[0]);
+                    RowPiece<T, L>::store(gs, g);
                 }
             }
         }
@@ -835,15 +834,14 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::Wave:
-            if (p.C <= wrow_cap<T>(wrow_wide<T>(x, WantGrad ? grad : nullptr, p.C))) {
-                const T *wrow_grad = WantGrad ? grad : nullptr;
+            if (p.C <= wrow_cap<T>(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C))) {
 #define PLH_GO(NI, W, G)                                                                                           \
     do {                                                                                                           \
         blocks = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                     \
         hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G>), dim3(blocks), dim3(256), 0, \
                            st, x, lab, up, loss, grad, cnt, part, p);                                              \
     } while (0)
-                PLH_WROW_DISPATCH(x, wrow_grad, p.C, PLH_GO);
+                PLH_WROW_DISPATCH(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C), p.C, PLH_GO);
 #undef PLH_GO
                 break;
             }

@@ -425,11 +425,11 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 // 16 bytes per lane and step where the rows allow it, else one element), so the row is read once and
 // every load of the row is in flight before the first one is used. Four rows per block at a time.
 
-template <class T, int NI, bool Wide, bool Reduce, int G>
+template <class T, int NI, int LP, bool Reduce, int G>
 __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     float *__restrict__ loss, Partials part, const LsrParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
     float mine = 0.f, cnt = 0.f;
     const float fc = (float)p.C;
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
         const bool live = r0 + at.grp < p.P;
         const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide, G> r;
+        WaveRow<T, NI, LP, G> r;
         r.load(xs, p.C, at.sub);
         const float mx = r.max();
         float s = 0.f, d = 0.f;
@@ -475,17 +475,17 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
     }
 }
 
-template <class T, int NI, bool Wide, int G>
+template <class T, int NI, int LP, int G>
 __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, T *__restrict__ grad, const LsrParams p) {
-    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
     for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
         const bool live = r0 + at.grp < p.P;
         const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
         T *gs = grad + row * p.C;
-        WaveRow<T, NI, Wide, G> r;
+        WaveRow<T, NI, LP, G> r;
         r.load(xs, p.C, at.sub);
         const int64_t lb = lab[row];
         float go[1];
@@ -511,8 +511,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
                 float g[L];
 #pragma unroll
                 for (int l = 0; l < L; ++l) g[l] = __builtin_fmaf(r.v[i][l], scale, (e0 + l == tgt) ? n_pos : n_neg);
-                if constexpr (Wide) RowChunk<T>::store(gs + e0, g);
-                else store_one(gs + e0, g[0]);
+                RowPiece<T, L>::store(gs + e0, g);
             }
         }
     }
@@ -834,21 +833,21 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
-            if (p.C > wrow_cap<T>(wrow_wide<T>(logits, nullptr, p.C))) {
+            const int piece = wrow_piece<T>(logits, nullptr, p.C);
+            if (p.C > wrow_cap<T>(piece)) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
                 hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
             unsigned grid = 0;
-            const T *wrow_grad = nullptr;
 #define PLH_GO(NI, W, G)                                                                                            \
     do {                                                                                                            \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                        \
         hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce, G>), dim3(grid), dim3(256), 0, st, logits, labels, losses, \
                            part, p);                                                                                \
     } while (0)
-            PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
+            PLH_WROW_DISPATCH(piece, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
         }
@@ -878,7 +877,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::SplitDeep: launch_bwd_split<T, V / 2>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
-            if (p.C > wrow_cap<T>(wrow_wide<T>(logits, grad_logits, p.C))) {
+            if (p.C > wrow_cap<T>(wrow_piece<T>(logits, grad_logits, p.C))) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
                 // chunks a row can have at most, and the threads that share them: 256 while 16 chunks per thread do
                 const int chunks = p.C / RowChunk<T>::kLen + 1;
@@ -904,11 +903,10 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                 break;
             }
             {
-                const T *wrow_grad = grad_logits;
 #define PLH_GO(NI, W, G)                                                                                          \
     hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
                        st, logits, labels, up, grad_logits, p)
-                PLH_WROW_DISPATCH(logits, wrow_grad, p.C, PLH_GO);
+                PLH_WROW_DISPATCH(wrow_piece<T>(logits, grad_logits, p.C), p.C, PLH_GO);
 #undef PLH_GO
             }
             break;

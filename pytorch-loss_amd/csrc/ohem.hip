@@ -170,13 +170,13 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
 
 // (N, C) inputs with 33..2048 channels: a wavefront per row, the row in its registers (one read of HBM,
 // every access a contiguous run), where the lane-per-pixel kernel would have each lane walk its own row.
-template <class T, int NI, bool Wide, int G>
+template <class T, int NI, int LP, int G>
 __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         float *__restrict__ scores, float *__restrict__ ce, int64_t P,
                                                         int C, int64_t ignore, uint32_t *__restrict__ tables) {
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += 256) tables[i] = 0;
-    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
     for (int64_t r0 = at.start; r0 < P; r0 += at.stride) {   // wave-uniform
         const bool live = r0 + at.grp < P;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x,
             }
         }
         const T *xs = x + row * C;
-        WaveRow<T, NI, Wide, G> r;
+        WaveRow<T, NI, LP, G> r;
         r.load(xs, C, at.sub);
         const float mx = r.max();
         float s = 0.f;
@@ -580,11 +580,11 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
             }
-        } else if (shape == Shape::Wave && C <= wrow_cap<T>(wrow_wide<T>(x, nullptr, C))) {
+        } else if (shape == Shape::Wave && C <= wrow_cap<T>(wrow_piece<T>(x, (const T *)nullptr, C))) {
 #define PLH_GO(NI, W, G)                                                                                            \
     hipLaunchKernelGGL((ohem_scores_wrow<T, NI, W, G>), dim3(group_grid(P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
                        st, x, labels, scores, ce, P, C, ignore_index, tables)
-            PLH_WROW_DISPATCH(x, (const T *)nullptr, C, PLH_GO);
+            PLH_WROW_DISPATCH(wrow_piece<T>(x, (const T *)nullptr, C), C, PLH_GO);
 #undef PLH_GO
         } else if (shape == Shape::Wave) {
             const unsigned grid = (unsigned)(P < 1 ? 1 : (P < kMinPartialSlots ? P : kMinPartialSlots));

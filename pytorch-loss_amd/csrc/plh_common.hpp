@@ -1055,24 +1055,57 @@ template <class T> struct RowChunk {             // T = f16 or bf16
     }
 };
 
+// ---- pieces of a contiguous row: L elements of 2 .. 16 bytes together, at an address aligned to their size ----
+template <class T, int L> struct RowPiece {
+    static_assert(L * sizeof(T) <= 16 && (L & (L - 1)) == 0, "pieces of 1, 2, 4 or 8 elements, 16 bytes at most");
+    static __device__ __forceinline__ void load(const T *p, float (&v)[L]) {
+        if constexpr (L == RowChunk<T>::kLen) {
+            RowChunk<T>::load(p, v);
+        } else if constexpr (L == 1) {
+            v[0] = load_one(p);
+        } else if constexpr (sizeof(T) == 4) {                   // two fp32
+            const plh_f2 t = *reinterpret_cast<const plh_f2 *>(p);
+            v[0] = t.x; v[1] = t.y;
+        } else if constexpr (L == 2) {                           // two 16-bit elements: one dword
+            const unsigned d = *reinterpret_cast<const unsigned *>(p);
+            v[0] = widen_lo(d, T{}); v[1] = widen_hi(d, T{});
+        } else {                                                 // four 16-bit elements
+            const plh_u2 t = *reinterpret_cast<const plh_u2 *>(p);
+            v[0] = widen_lo(t.x, T{}); v[1] = widen_hi(t.x, T{});
+            v[2] = widen_lo(t.y, T{}); v[3] = widen_hi(t.y, T{});
+        }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&v)[L]) {
+        if constexpr (L == RowChunk<T>::kLen) {
+            RowChunk<T>::store(p, v);
+        } else if constexpr (L == 1) {
+            store_one(p, v[0]);
+        } else if constexpr (sizeof(T) == 4) {       // short pieces go through the cache: a wavefront's stores
+            *reinterpret_cast<plh_f2 *>(p) = plh_f2{v[0], v[1]};         // of one step cover parts of lines, which
+        } else if constexpr (L == 2) {                                   // the next steps complete there
+            *reinterpret_cast<unsigned *>(p) = narrow2(v[0], v[1], T{});
+        } else {
+            *reinterpret_cast<plh_u2 *>(p) = plh_u2{narrow2(v[0], v[1], T{}), narrow2(v[2], v[3], T{})};
+        }
+    }
+};
+
 // ---- a wavefront holds rows of an (N, C) input in registers --------------------------------
 // G lanes share a row (G = 64: one row per wavefront; G = 16: four short rows per wavefront, so that a
-// wavefront still has a few KB in flight), NI steps of G lanes, 16 bytes per lane and step where the rows
-// allow it, else one element: a row is read once and every load of it is in flight before the first one
-// is used.
-template <class T, int NI, bool Wide, int G = 64>
+// wavefront still has a few KB in flight), NI steps of G lanes, a piece of L elements per lane and step
+// (16 bytes where the rows allow it; rows whose length in bytes is only a multiple of 8, 4 or 2 move in
+// pieces of that size): a row is read once and every load of it is in flight before the first one is used.
+template <class T, int NI, int L_, int G = 64>
 struct WaveRow {
-    static constexpr int L = Wide ? RowChunk<T>::kLen : 1;
+    static constexpr int L = L_;
     float v[NI][L];
     // `sub` = lane within the row's group; elements beyond the row read as -inf (and are never stored)
     __device__ __forceinline__ void load(const T *xs, int C, int sub) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int e0 = (sub + G * i) * L;
-            const bool ok = e0 < C;                   // rows moved in chunks hold a whole number of them
-            const T *at = xs + (ok ? e0 : 0);
-            if constexpr (Wide) RowChunk<T>::load(at, v[i]);
-            else v[i][0] = load_one(at);
+            const bool ok = e0 < C;                   // a row holds a whole number of pieces
+            RowPiece<T, L>::load(xs + (ok ? e0 : 0), v[i]);
 #pragma unroll
             for (int l = 0; l < L; ++l) v[i][l] = ok ? v[i][l] : -INFINITY;
         }
@@ -1104,61 +1137,57 @@ struct WaveRowAt {
     }
 };
 
-// Lanes per row and steps for a row of C elements. Rows of up to 256 elements get 16 lanes (at most 16
-// elements per lane); longer ones a whole wavefront. Instantiated sizes -- 16 lanes: 2 or 4 steps of
-// 16-byte chunks (4 only for fp32, whose chunks hold 4 elements), 4, 8 or 16 steps of single elements;
-// 64 lanes: 2, 4 or 8 steps of chunks (8 only for fp32), 8, 16 or 32 steps of single elements. Rows can be
-// moved in 16-byte chunks when every row starts on a 16-byte boundary.
+// Lanes per row, piece length and steps for a row of C elements. Rows of up to 256 elements get 16 lanes,
+// longer ones a whole wavefront. The piece is the largest of 16, 8, 4, 2 bytes that divides the row's bytes
+// and that every tensor involved is aligned to. Instantiated steps -- 16 lanes: 4, 8, 16 single elements,
+// 2, 4, 8 pieces of two, 2, 4 of four, 2 of eight; 64 lanes: 8, 16, 32 single elements, 4, 8, 16 pieces of
+// two, 2, 4, 8 of four or eight.
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
-// 16-bit rows that move in chunks go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the same 64
-// registers as an fp32 row of 2048); a block per row spends most of such a short row's time in its barriers
-// (bf16 LSR forward at (65536, 4096): 45 % of peak).
+// 16-bit rows that move in 16-byte pieces go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the
+// same 64 registers as an fp32 row of 2048); a block per row spends most of such a short row's time in its
+// barriers (bf16 LSR forward at (65536, 4096): 45 % of peak).
 template <class T>
-inline int wrow_cap(bool wide) { return (wide && sizeof(T) == 2) ? 2 * kWaveRowCap : kWaveRowCap; }
+inline int wrow_cap(int piece) { return piece == 8 ? 2 * kWaveRowCap : kWaveRowCap; }
 
 template <class T>
-static bool wrow_wide(const T *x, const T *grad, int C) {
-    return C % RowChunk<T>::kLen == 0 && !misaligned(x, 16) && !(grad && misaligned(grad, 16));
+static int wrow_piece(const T *x, const T *second, int C, const T *third = nullptr) {
+    int len = RowChunk<T>::kLen;
+    while (len > 1 && (C % len != 0 || misaligned(x, len * sizeof(T)) || (second && misaligned(second, len * sizeof(T))) ||
+                       (third && misaligned(third, len * sizeof(T)))))
+        len /= 2;
+    return len;
 }
 template <class T>
-static int wrow_steps(int C, bool wide, int lanes) {
-    const int per = lanes * (wide ? RowChunk<T>::kLen : 1);
+static int wrow_steps(int C, int piece, int lanes) {
+    const int per = lanes * piece;
     const int need = (C + per - 1) / per;
-    int steps = wide ? 2 : (lanes == 16 ? 4 : 8);      // the smallest instantiated size of each kind
+    int steps = piece == 1 ? (lanes == 16 ? 4 : 8) : (piece == 2 && lanes == 64 ? 4 : 2);   // the smallest instantiated sizes
     while (steps < need) steps *= 2;
     return steps;
 }
-// LAUNCH(NI, Wide, G) launches the kernel instance; its grid is group_grid(rows, WaveRowAt<G>::kRowsPerBlock).
-#define PLH_WROW_DISPATCH_WIDE(WIDE, C, LAUNCH)                                          \
+// LAUNCH(NI, L, G) launches the kernel instance; its grid is group_grid(rows, WaveRowAt<G>::kRowsPerBlock).
+#define PLH_WROW_STEPS3(PIECE, LANES, C, A, B, D, LAUNCH)                                \
+    switch (wrow_steps<T>(C, PIECE, LANES)) {                                            \
+        case A: LAUNCH(A, PIECE, LANES); break;                                          \
+        case B: LAUNCH(B, PIECE, LANES); break;                                          \
+        default: LAUNCH(D, PIECE, LANES); break;                                         \
+    }
+#define PLH_WROW_DISPATCH(PIECE, C, LAUNCH)                                              \
     do {                                                                                 \
-        const bool wrow_is_wide = (WIDE);                                                \
+        const int wrow_len = (PIECE);                                                    \
         if ((C) <= kWaveRowShort) {                                                      \
-            switch (wrow_steps<T>(C, wrow_is_wide, 16)) {                                \
-                case 2: LAUNCH(2, true, 16); break;              /* chunks only */      \
-                case 4:                                                                  \
-                    if constexpr (RowChunk<T>::kLen == 4) {                              \
-                        if (wrow_is_wide) { LAUNCH(4, true, 16); break; }                \
-                    }                                                                    \
-                    LAUNCH(4, false, 16);   /* 16-bit chunks never need 4 steps here */  \
-                    break;                                                               \
-                case 8: LAUNCH(8, false, 16); break;                                     \
-                default: LAUNCH(16, false, 16); break;                                   \
-            }                                                                            \
+            if (wrow_len == 1) { PLH_WROW_STEPS3(1, 16, C, 4, 8, 16, LAUNCH) }           \
+            else if (wrow_len == 2) { PLH_WROW_STEPS3(2, 16, C, 2, 4, 8, LAUNCH) }       \
+            else if (wrow_len == 4) { PLH_WROW_STEPS3(4, 16, C, 2, 4, 4, LAUNCH) }       \
+            else if constexpr (RowChunk<T>::kLen == 8) { LAUNCH(2, 8, 16); }             \
         } else {                                                                         \
-            switch (wrow_steps<T>(C, wrow_is_wide, 64)) {                                \
-                case 2: LAUNCH(2, true, 64); break;              /* chunks only */      \
-                case 4: LAUNCH(4, true, 64); break;              /* chunks only */      \
-                case 8:                                                                  \
-                    if (wrow_is_wide) { LAUNCH(8, true, 64); break; }                    \
-                    LAUNCH(8, false, 64);                                                \
-                    break;                                                               \
-                case 16: LAUNCH(16, false, 64); break;                                   \
-                default: LAUNCH(32, false, 64); break;                                   \
-            }                                                                            \
+            if (wrow_len == 1) { PLH_WROW_STEPS3(1, 64, C, 8, 16, 32, LAUNCH) }          \
+            else if (wrow_len == 2) { PLH_WROW_STEPS3(2, 64, C, 4, 8, 16, LAUNCH) }      \
+            else if (wrow_len == 4) { PLH_WROW_STEPS3(4, 64, C, 2, 4, 8, LAUNCH) }       \
+            else if constexpr (RowChunk<T>::kLen == 8) { PLH_WROW_STEPS3(8, 64, C, 2, 4, 8, LAUNCH) } \
         }                                                                                \
     } while (0)
-#define PLH_WROW_DISPATCH(X, GRAD, C, LAUNCH) PLH_WROW_DISPATCH_WIDE(wrow_wide<T>(X, GRAD, C), C, LAUNCH)
 
 // ---- a block per row: rows longer than a wavefront's registers (a vocabulary) ------------------
 // One block of 1024 (or, for shorter rows, 256) threads per row at a time, 16-byte loads, four of them in flight per lane, and running

@@ -479,13 +479,13 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
 // upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
 // the group kernel.
 
-template <class T, int NI, bool Wide, int Kind, bool Reduce, int G>
+template <class T, int NI, int LP, int Kind, bool Reduce, int G>
 __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
                                                    const int64_t *__restrict__ lab, const Upstream up,
                                                    T *__restrict__ out, float *__restrict__ loss, Partials part,
                                                    const TaylorParams p) {
     __shared__ float red[4];
-    constexpr int L = WaveRow<T, NI, Wide, G>::L;
+    constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
     const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
@@ -493,9 +493,9 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
         const bool live = r0 + at.grp < p.P;
         const int64_t row = live ? r0 + at.grp : p.P - 1;
         const T *xs = x + row * p.C;
-        WaveRow<T, NI, Wide, G> r;
+        WaveRow<T, NI, LP, G> r;
         r.load(xs, p.C, lane);
-        WaveRow<T, (Kind == kTaylorBwd) ? NI : 1, Wide, G> rg;
+        WaveRow<T, (Kind == kTaylorBwd) ? NI : 1, LP, G> rg;
         if constexpr (Kind == kTaylorBwd) rg.load(g + row * p.C, p.C, lane);
         float s = 0.f, dot = 0.f;
 #pragma unroll
@@ -559,8 +559,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 }
                 if (e0 < p.C && live) {
                     T *dst = out + row * p.C + e0;
-                    if constexpr (Wide) RowChunk<T>::store(dst, o);
-                    else store_one(dst, o[0]);
+                    RowPiece<T, L>::store(dst, o);
                 }
             }
         }
@@ -775,13 +774,13 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         return grid;
     }
     if (p.m_size == 1) {
-        const bool wide = wrow_wide<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C) &&
-                          !(Kind == kTaylorBwd && misaligned(g, 16));
+        const int piece = wrow_piece<T>(x, (Kind == kTaylorCeFwd) ? (const T *)nullptr : (const T *)out, p.C,
+                                        (Kind == kTaylorBwd) ? g : (const T *)nullptr);
         // the backwards keep the 2048-element limit: the softmax backward holds two rows in registers, and the
         // cross-entropy backward with 64 registers of row ran at a third of its two-sweep form (bf16 (65536, 4096):
         // 0.782 against 0.304 ms)
         constexpr bool kForward = (Kind == kTaylorFwd || Kind == kTaylorCeFwd);
-        if (p.C <= (kForward ? wrow_cap<T>(wide) : kWaveRowCap)) {
+        if (p.C <= (kForward ? wrow_cap<T>(piece) : kWaveRowCap)) {
             unsigned grid = 0;
 #define PLH_GO(NI, W, G)                                                                                          \
     do {                                                                                                          \
@@ -789,7 +788,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
                            loss, part, p);                                                                        \
     } while (0)
-            PLH_WROW_DISPATCH_WIDE(wide, p.C, PLH_GO);
+            PLH_WROW_DISPATCH(piece, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
         }

@@ -82,6 +82,11 @@ SEG_CASES = [
     ((4, 1001), -100, 0.1),
     ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
     ((2, 2048), 255, 0.0),
+    ((7, 150), 255, 0.1),                           #   lengths that are a multiple of 2 but not of 4 (and of 4 but not of 8):
+    ((5, 34), -100, 0.1),                           #   pieces of two fp32 elements, of two or four 16-bit ones
+    ((3, 1002), 255, 0.1),
+    ((4, 2046), -100, 0.0),
+    ((6, 300), 255, 0.1),
     ((2, 2049), -100, 0.0),                         # one channel more: staged or swept rows
     ((4, 3000), -100, 0.1),                         # 16-bit rows in whole chunks stay in a wavefront's registers up to
     ((3, 4096), 255, 0.1),                          #   4096 elements (8 steps of 8); fp32 rows take a block per row
