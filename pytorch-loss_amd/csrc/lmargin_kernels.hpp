@@ -197,8 +197,8 @@ struct LmSplitStats {
     float m_no, s_no, sum_qt, sum_t, x_y;
 };
 
-template <class T, int KW, int V, bool WantSumT>
-__device__ __forceinline__ void lm_split_parts(const SplitSlice<T, V, KW> &at, const typename Pack<T, V>::Raw (&raw)[KW],
+template <class T, int KW, int V, bool WantSumT, class Slice>
+__device__ __forceinline__ void lm_split_parts(const Slice &at, const typename Pack<T, V>::Raw (&raw)[KW],
                                                int k, int rel, float (*parts)[kSplitWaves][kWave * V], int q, int wave) {
     float xv[KW];
     float mx = -INFINITY, x_y = -INFINITY;
@@ -258,14 +258,14 @@ __device__ __forceinline__ LmSplitStats<V> lm_split_combine(float (*parts)[kSpli
     return r;
 }
 
-template <class T, int KW, int V, bool Reduce>
+template <class T, int KW, int V, bool Reduce, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            float *__restrict__ loss, Partials part, const LmParams p) {
     __shared__ float parts[6][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     if (at.here > 0) {                                  // wave-uniform
         typename Pack<T, V>::Raw raw[KW];
         at.load(x, p.C, p.m_size, raw);
@@ -301,8 +301,8 @@ __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict_
         mine += out[k];
         cnt += valid ? 1 : 0;
     }
-    if (at.live && loss) store_vec<V>(loss + at.pix, out);
-    if (at.live && p.scores) store_vec_cached<V>(p.scores + at.pix, score);
+    if (at.live && loss) at.store_f32(loss, out);
+    if (at.live && p.scores) at.template store_f32<true>(p.scores, score);
     if constexpr (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());
@@ -313,20 +313,20 @@ __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict_
     }
 }
 
-template <class T, int KW, int V>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lm_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            const Upstream up, T *__restrict__ grad, const LmParams p) {
     __shared__ float parts[4][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
     typename PK::Raw raw[KW];
     int64_t lb[V];
     float go[V];
     if (at.here > 0) {                                  // wave-uniform
         at.load(x, p.C, p.m_size, raw);
-        load_labels<V>(lab + at.pix, lb);
-        load_upstream<V>(up, at.pix, go);
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             bool ign;
@@ -787,7 +787,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
     // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
     constexpr bool kHasSplit = !(WantLoss && WantGrad);
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
-                       second_f32, kHasSplit, kHasSplit)) {
+                       second_f32, kHasSplit, kHasSplit, kHasSplit)) {
         case Shape::SplitDeep:
             if constexpr (kHasSplit) {
                 constexpr int VD = V / 2;
@@ -817,6 +817,24 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
                                part, p);                                                                              \
         else                                                                                                          \
             hipLaunchKernelGGL((lm_bwd_split<T, KW, V>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
+        break;
+                    PLH_SPLIT_SLOT_CASES
+#undef PLH_CASE
+                }
+            }
+            break;
+        case Shape::SplitImage:                // tiles per image: channel planes that start on element boundaries only
+            if constexpr (kHasSplit) {
+                blocks = split_image_grid<V>(p.P / p.m_size, p.m_size);
+                switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (WantLoss)                                                                                       \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, V, Reduce, true>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, \
+                               loss, part, p);                                                                        \
+        else                                                                                                          \
+            hipLaunchKernelGGL((lm_bwd_split<T, KW, V, true>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up,    \
+                               grad, p);                                                                              \
         break;
                     PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE

@@ -156,15 +156,15 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 //   backward  (c_w, s_w) in the base-2 domain, c_w = fl(m_w log2e), s_w = sum_j 2^(x_j log2e - c_w); every
 //             wavefront then evaluates 2^(x_j log2e - max_w c_w) / sum_w s_w 2^(c_w - max c) for its channels.
 
-template <class T, int KW, int V, bool Reduce>
+template <class T, int KW, int V, bool Reduce, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                             float *__restrict__ loss, Partials part,
                                                             const LsrParams p) {
     __shared__ float parts[4][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     if (at.here > 0) {                                  // wave-uniform
         typename Pack<T, V>::Raw raw[KW];
         at.load(x, p.C, p.m_size, raw);
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
         mine += out[k];
         cnt += valid ? 1 : 0;
     }
-    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if (at.live && loss) at.store_f32(loss, out);
     if constexpr (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());      // at most 256 per block: exact in fp32
@@ -236,21 +236,21 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
     }
 }
 
-template <class T, int KW, int V>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lsr_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                             const Upstream up, T *__restrict__ grad,
                                                             const LsrParams p) {
     __shared__ float parts[2][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
     typename PK::Raw raw[KW];
     int64_t lb[V];
     float go[V];
     if (at.here > 0) {                                  // wave-uniform
         at.load(x, p.C, p.m_size, raw);
-        load_labels<V>(lab + at.pix, lb);
-        load_upstream<V>(up, at.pix, go);
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float xv[KW];
@@ -422,7 +422,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 
 // ------------------------------------------------- wavefront per row, in registers ----
 // (N, C) inputs with 33..2048 channels: a wavefront holds a whole row in registers (NI steps of 64 lanes,
-// 16 bytes per lane and step where the rows allow it, else one element), so the row is read once and
+// 16 bytes per lane and step where the rows allow it, else pieces of 8, 4 or 2 bytes), so the row is read once and
 // every load of the row is in flight before the first one is used. Four rows per block at a time.
 
 template <class T, int NI, int LP, bool Reduce, int G>
@@ -732,9 +732,38 @@ static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, 
     }
 }
 
+// `image`: tiles per image (channel planes that start on element boundaries only)
 template <class T, int V, bool Reduce>
 static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
-                                 hipStream_t st) {
+                                 hipStream_t st, bool image = false) {
+    if constexpr (V == ElemTraits<T>::kVec) if (image) {      // the deep form (V / 2) has no such variant
+        if constexpr (sizeof(T) == 4) {
+            if (split_image_wide(p.C)) {       // four fp32 pixels per lane
+                const unsigned grid = split_image_grid<4>(p.P / p.m_size, p.m_size);
+                switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, 4, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+                           loss, part, p);                                                                        \
+        break;
+                    PLH_CASE(16) PLH_CASE(20)
+#undef PLH_CASE
+                }
+                return grid;
+            }
+        }
+        const unsigned grid = split_image_grid<V>(p.P / p.m_size, p.m_size);
+        switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+                           loss, part, p);                                                                        \
+        break;
+            PLH_SPLIT_SLOT_CASES
+#undef PLH_CASE
+        }
+        return grid;
+    }
     const unsigned grid = split_grid<V>(p.P);
     if constexpr (V < ElemTraits<T>::kVec) {        // the deep form
         switch (split_slots_deep(p.C)) {
@@ -762,7 +791,35 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
 
 template <class T, int V>
 static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
-                             hipStream_t st) {
+                             hipStream_t st, bool image = false) {
+    if constexpr (V == ElemTraits<T>::kVec) if (image) {      // the deep form (V / 2) has no such variant
+        if constexpr (sizeof(T) == 4) {
+            if (split_image_wide(p.C)) {       // four fp32 pixels per lane
+                const unsigned grid = split_image_grid<4>(p.P / p.m_size, p.m_size);
+                switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_bwd_split<T, KW, 4, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, grad, \
+                           p);                                                                                    \
+        break;
+                    PLH_CASE(16) PLH_CASE(20)
+#undef PLH_CASE
+                }
+                return;
+            }
+        }
+        const unsigned grid = split_image_grid<V>(p.P / p.m_size, p.m_size);
+        switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                              \
+    case KW:                                                                                                      \
+        hipLaunchKernelGGL((lsr_bwd_split<T, KW, V, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, grad, \
+                           p);                                                                                    \
+        break;
+            PLH_SPLIT_SLOT_CASES
+#undef PLH_CASE
+        }
+        return;
+    }
     const unsigned grid = split_grid<V>(p.P);
     if constexpr (V < ElemTraits<T>::kVec) {        // the deep form
         switch (split_slots_deep(p.C)) {
@@ -825,12 +882,13 @@ template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
                         hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true, true)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) return launch_fwd_image<T, Reduce>(logits, labels, losses, part, p, st);
             return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::SplitImage: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st, true);
         case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
             const int piece = wrow_piece<T>(logits, nullptr, p.C);
@@ -865,7 +923,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true, true)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) {
@@ -875,6 +933,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
             launch_bwd_regs<T, 1>(logits, labels, up, grad_logits, p, st);
             break;
         case Shape::Split: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st); break;
+        case Shape::SplitImage: launch_bwd_split<T, V>(logits, labels, up, grad_logits, p, st, true); break;
         case Shape::SplitDeep: launch_bwd_split<T, V / 2>(logits, labels, up, grad_logits, p, st); break;
         case Shape::Wave:
             if (p.C > wrow_cap<T>(wrow_piece<T>(logits, grad_logits, p.C))) {

@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
 
 // 33..256 channels in NCHW (SplitSlice): per wavefront the maximum, the exponential sum and the target's
 // logit of its channels; wavefront 0 combines them into the pixel's score and cross entropy.
-template <class T, int KW, int V>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 float *__restrict__ scores, float *__restrict__ ce,
                                                                 int64_t P, int64_t m_size, int C, int64_t ignore,
@@ -89,9 +89,9 @@ __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__rest
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kSplitBlock) tables[i] = 0;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(P, m_size, C, xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(P, m_size, C, xcd_run);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, ignore, lb);
     if (at.here > 0) {                                  // wave-uniform
         typename Pack<T, V>::Raw raw[KW];
         at.load(x, C, m_size, raw);
@@ -135,8 +135,8 @@ __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__rest
         out[k] = (tgt < 0) ? 1.f : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
         loss[k] = (tgt < 0) ? 0.f : fast_log(S) + (M - x_y);
     }
-    store_vec_cached<V>(scores + at.pix, out);
-    if (ce) store_vec_cached<V>(ce + at.pix, loss);
+    at.template store_f32<true>(scores, out);
+    if (ce) at.template store_f32<true>(ce, loss);
 }
 
 // Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).
@@ -530,7 +530,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true, true);
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true, true, true);
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
             const unsigned grid = split_grid<VD>(P);
@@ -542,6 +542,18 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
                            P, m_size, C, ignore_index, run, tables);                                                  \
         break;
                 PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+            }
+        } else if (shape == Shape::SplitImage) {    // tiles per image: channel planes that start on element boundaries only
+            const unsigned grid = split_image_grid<VT>(n_size, m_size);
+            const unsigned run = xcd_run_for(sizeof(T), m_size);
+            switch (split_slots(dimsize)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        hipLaunchKernelGGL((ohem_scores_split<T, KW, VT, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, \
+                           ce, P, m_size, C, ignore_index, run, tables);                                              \
+        break;
+                PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
             }
         } else if (shape == Shape::Split) {

@@ -6,15 +6,15 @@
 //             a wavefront is one contiguous 64*V*4-byte run, logits are read from HBM
 //             exactly once and no cross-lane traffic is needed. (N, C) inputs with C <= 32
 //             take the same kernels; a wavefront moves its 64 rows through a private LDS tile.
-//   "split" : 33..256 channels in NCHW. The regs shape with the slice of a pixel shared out
+//   "split" : 33..512 channels in NCHW. The regs shape with the slice of a pixel shared out
 //             over the 8 wavefronts of a block; per-wavefront statistics meet in LDS.
-//   "wrow"  : (N, C) rows of 33..2048 elements held in the registers of the 64 (or 16) lanes
-//             that share a row; every sweep after the first runs on registers.
+//   "wrow"  : (N, C) rows of 33..2048 elements (4096 for 16-bit rows in 16-byte pieces) held in the
+//             registers of the 64 (or 16) lanes that share a row; every sweep after the first runs on registers.
 //   "row"   : (N, C) rows longer than that (every loss, the OHEM scores and the Taylor ops): a
 //             block per row, 16-byte chunks, running statistics that are rescaled when the
 //             maximum moves, a second sweep from cache where a gradient is written.
 //   "group" : everything else. G = 64: a wavefront per row striding over its channels (layer norm
-//             on long rows); G = 1: a lane per pixel for more than 256 channels in NCHW, channel
+//             on long rows); G = 1: a lane per pixel for more than 512 channels in NCHW, channel
 //             loop through the caches. Reductions inside a group use DPP/swizzle; nothing is
 //             staged in LDS.
 #pragma once
@@ -77,7 +77,7 @@ inline int check_gout(const void *gout, int64_t stride) {
 // (see "the split launch shape" below); only for kernels that have that form (`with_split`).
 // SplitDeep: the split shape with half the pixels per lane (4 bytes per lane and channel) and up to 64
 // channel slots per wavefront, for 257..512 channels; only for kernels that have it (`with_deep`).
-enum class Shape { RegsVec, RegsOne, Split, SplitDeep, Wave, Lane };
+enum class Shape { RegsVec, RegsOne, Split, SplitImage, SplitDeep, Wave, Lane };
 
 constexpr int kMaxRegsChannels = 32;
 constexpr int kSplitWaves = 8;
@@ -87,7 +87,7 @@ constexpr int kMaxDeepChannels = kMaxDeepSlots * kSplitWaves;
 
 inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, const void *typed0, const void *typed1,
                         const void *labels, const void *f32a, const void *f32b, bool with_split = false,
-                        bool with_deep = false) {
+                        bool with_deep = false, bool with_image = false) {
     auto fits = [&](int v) {
         return (m_size % v == 0) && !(typed0 && misaligned(typed0, v * elem)) &&
                !(typed1 && misaligned(typed1, v * elem)) && !(f32a && misaligned(f32a, v * 4)) &&
@@ -96,6 +96,9 @@ inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, con
     const bool vec = fits(V) && !(labels && misaligned(labels, 16));
     if (dimsize <= kMaxRegsChannels) return vec ? Shape::RegsVec : Shape::RegsOne;
     if (with_split && vec && dimsize <= kMaxSplitChannels && m_size >= 64) return Shape::Split;
+    // planes that start on element boundaries only (odd lengths) and are long enough that the partly filled
+    // last block of every image is a small share: the split shape in tiles per image
+    if (with_image && !vec && dimsize <= kMaxSplitChannels && m_size >= 4096) return Shape::SplitImage;
     if (with_deep && dimsize > kMaxSplitChannels && dimsize <= kMaxDeepChannels && m_size >= 64 && fits(V / 2))
         return Shape::SplitDeep;
     return m_size == 1 ? Shape::Wave : Shape::Lane;
@@ -258,6 +261,9 @@ __device__ __forceinline__ unsigned f32_bits(float v) { return __builtin_bit_cas
 __device__ __forceinline__ float bits_f32(unsigned v) { return __builtin_bit_cast(float, v); }
 
 template <class T, int V> struct Pack;
+typedef unsigned plh_u2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef float plh_f2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef long long plh_l2_a8 __attribute__((ext_vector_type(2), aligned(8)));
 
 template <> struct Pack<float, 2> {
     typedef plh_u2 Raw;
@@ -266,6 +272,14 @@ template <> struct Pack<float, 2> {
     }
     static __device__ __forceinline__ void store(float *p, Raw r) {
         __builtin_nontemporal_store(r, reinterpret_cast<plh_u2 *>(p));
+    }
+    // the same 8 bytes from any element boundary (tiles per image on channel planes of odd length)
+    static __device__ __forceinline__ Raw load_unaligned(const float *p) {
+        const plh_u2_a4 t = __builtin_nontemporal_load(reinterpret_cast<const plh_u2_a4 *>(p));
+        return Raw{t.x, t.y};
+    }
+    static __device__ __forceinline__ void store_unaligned(float *p, Raw r) {
+        __builtin_nontemporal_store(plh_u2_a4{r.x, r.y}, reinterpret_cast<plh_u2_a4 *>(p));
     }
     static __device__ __forceinline__ float get(Raw r, int k) { return bits_f32(k == 0 ? r.x : r.y); }
     static __device__ __forceinline__ Raw put(const float (&g)[2]) { return Raw{f32_bits(g[0]), f32_bits(g[1])}; }
@@ -284,7 +298,6 @@ template <> struct Pack<float, 2> {
 typedef unsigned plh_u4w __attribute__((ext_vector_type(4)));
 typedef unsigned plh_u4w_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef float plh_f4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-typedef long long plh_l2_a8 __attribute__((ext_vector_type(2), aligned(8)));
 template <> struct Pack<float, 4> {
     typedef plh_u4w Raw;
     static __device__ __forceinline__ Raw load(const float *p) {
@@ -893,6 +906,10 @@ inline int split_slots(int64_t dimsize) {
     const int kw = (per + 3) / 4 * 4;
     return kw < 8 ? 8 : kw;
 }
+// fp32 slices of 16 or 20 slots per wavefront (97..160 channels) take four pixels per lane in the tiles-per-image
+// form of the LSR kernels: 1 KiB runs, 80 registers of slice. Measured fwd+bwd on (8,150,513,513): 0.951 -> 0.824 ms;
+// with 8 slots (40 and 60 channels) it changed nothing or lost (0.282 -> 0.303 ms on (8,40,481,641)).
+inline bool split_image_wide(int64_t dimsize) { return split_slots(dimsize) == 16 || split_slots(dimsize) == 20; }
 // The deep form (257..512 channels): 40, 48, 56 or 64 slots per wavefront.
 #define PLH_SPLIT_DEEP_CASES PLH_CASE(40) PLH_CASE(48) PLH_CASE(56) PLH_CASE(64)
 inline int split_slots_deep(int64_t dimsize) {
@@ -901,20 +918,44 @@ inline int split_slots_deep(int64_t dimsize) {
     return kw < 40 ? 40 : kw;
 }
 
-template <class T, int V, int KW>
+// `PerImage`: tiles that never straddle two images (grid = images x tiles per image, split_image_grid), for channel
+// planes that start on element boundaries only (odd lengths: 513 x 513 crops with 150 classes): a lane's V pixels
+// are moved with accesses of the same width from element boundaries, the last lane of an image may hold fewer
+// (`nv`) and then goes pixel by pixel; the pixels it lacks read as ignored and are never stored.
+template <int V>
+inline unsigned split_image_grid(int64_t n_size, int64_t m_size) {
+    return (unsigned)(n_size * ceil_div(m_size, (int64_t)kWave * V));
+}
+
+template <class T, int V, int KW, bool PerImage = false>
 struct SplitSlice {
     int64_t pix;      // first of this lane's V pixels (0 for a lane beyond the end: it still loads, never stores)
     int64_t base;     // element offset of (image, channel 0, pix)
     int first;        // first channel of this wavefront
     int here;         // channels of this wavefront that exist (0..KW), wave-uniform
+    int nv;           // pixels this lane has (V, or fewer in the last lane of an image)
     bool live;
 
     __device__ __forceinline__ SplitSlice(int64_t P, int64_t m_size, int C, unsigned xcd_run) {
-        const int64_t want = (tile_of_block(xcd_run) * kWave + (threadIdx.x & 63)) * V;
-        live = want < P;
-        pix = live ? want : 0;
-        const int64_t n = pix / m_size;
-        base = pix + n * (int64_t)(C - 1) * m_size;
+        if constexpr (PerImage) {
+            const int64_t tiles = ceil_div_dev(m_size, (int64_t)kWave * V);
+            const int64_t b = tile_of_block(xcd_run);
+            const int64_t n = b / tiles;                        // block-uniform
+            const int64_t local = ((b - n * tiles) * kWave + (threadIdx.x & 63)) * V;
+            const int64_t left = m_size - local;
+            nv = left >= V ? V : (left > 0 ? (int)left : 0);
+            live = nv > 0;
+            const int64_t safe = live ? local : 0;
+            pix = n * m_size + safe;
+            base = n * (int64_t)C * m_size + safe;
+        } else {
+            const int64_t want = (tile_of_block(xcd_run) * kWave + (threadIdx.x & 63)) * V;
+            live = want < P;
+            nv = V;
+            pix = live ? want : 0;
+            const int64_t n = pix / m_size;
+            base = pix + n * (int64_t)(C - 1) * m_size;
+        }
         first = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * KW;
         const int left = C - first;
         here = left < 0 ? 0 : (left > KW ? KW : left);
@@ -922,16 +963,91 @@ struct SplitSlice {
     // Slot i holds channel min(first + i, C - 1): a slot beyond the last channel repeats it, so that no
     // load sits behind a branch; what is computed from such a slot is masked by the caller (i < here).
     __device__ __forceinline__ void load(const T *t, int C, int64_t m_size, typename Pack<T, V>::Raw (&raw)[KW]) const {
+        if constexpr (PerImage) {
+            if (nv < V) {                           // the last lane of an image (or a lane beyond it: zeros)
+#pragma unroll
+                for (int i = 0; i < KW; ++i) {
+                    const int j = (first + i < C) ? first + i : C - 1;
+                    float one[V];
+#pragma unroll
+                    for (int k = 0; k < V; ++k) one[k] = k < nv ? load_one(t + (base + (int64_t)j * m_size) + k) : 0.f;
+                    raw[i] = Pack<T, V>::put(one);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < KW; ++i) {
             const int j = (first + i < C) ? first + i : C - 1;
-            raw[i] = Pack<T, V>::load(t + (base + (int64_t)j * m_size));
+            if constexpr (PerImage) raw[i] = Pack<T, V>::load_unaligned(t + (base + (int64_t)j * m_size));
+            else raw[i] = Pack<T, V>::load(t + (base + (int64_t)j * m_size));
         }
     }
     __device__ __forceinline__ void store(T *t, int64_t m_size, const typename Pack<T, V>::Raw (&raw)[KW]) const {
+        if constexpr (PerImage) {
+            if (nv < V) {
+#pragma unroll
+                for (int i = 0; i < KW; ++i)
+                    if (i < here) {
+#pragma unroll
+                        for (int k = 0; k < V; ++k)
+                            if (k < nv) store_one(t + (base + (int64_t)(first + i) * m_size) + k, Pack<T, V>::get(raw[i], k));
+                    }
+                return;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < KW; ++i)
-            if (i < here) Pack<T, V>::store(t + (base + (int64_t)(first + i) * m_size), raw[i]);
+            if (i < here) {
+                if constexpr (PerImage) Pack<T, V>::store_unaligned(t + (base + (int64_t)(first + i) * m_size), raw[i]);
+                else Pack<T, V>::store(t + (base + (int64_t)(first + i) * m_size), raw[i]);
+            }
+    }
+    // Labels, per-pixel fp32 outputs and the upstream gradient of this lane's pixels.
+    __device__ __forceinline__ void labels(const int64_t *lab, int64_t ignore, int64_t (&lb)[V]) const {
+        if constexpr (PerImage) {
+            if (nv == V) {
+#pragma unroll
+                for (int k = 0; k < V; k += 2) {
+                    const plh_l2_a8 t = __builtin_nontemporal_load(reinterpret_cast<const plh_l2_a8 *>(lab + pix + k));
+                    lb[k] = t.x; lb[k + 1] = t.y;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; ++k) lb[k] = k < nv ? lab[pix + k] : ignore;
+            }
+        } else {
+            load_labels<V>(lab + pix, lb);
+        }
+    }
+    template <bool Cached = false>
+    __device__ __forceinline__ void store_f32(float *out, const float (&v)[V]) const {
+        if constexpr (PerImage) {
+            if (nv == V) {
+#pragma unroll
+                for (int k = 0; k < V; k += 2) {
+                    if constexpr (Cached) *reinterpret_cast<plh_f2_a4 *>(out + pix + k) = plh_f2_a4{v[k], v[k + 1]};
+                    else __builtin_nontemporal_store(plh_f2_a4{v[k], v[k + 1]}, reinterpret_cast<plh_f2_a4 *>(out + pix + k));
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < V; ++k)
+                    if (k < nv) out[pix + k] = v[k];
+            }
+        } else {
+            if constexpr (Cached) store_vec_cached<V>(out + pix, v);
+            else store_vec<V>(out + pix, v);
+        }
+    }
+    __device__ __forceinline__ void upstream(const Upstream &up, float (&go)[V]) const {
+        if constexpr (PerImage) {
+            if (up.gout != nullptr && up.stride != 0) {
+#pragma unroll
+                for (int k = 0; k < V; ++k) go[k] = k < nv ? up.gout[pix + k] : 0.f;
+                return;
+            }
+        }
+        load_upstream<V>(up, pix, go);
     }
 };
 

@@ -255,15 +255,15 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
 // Cross entropy for 33..256 channels in NCHW (SplitSlice). The series needs no maximum, so the parts of
 // a pixel are just each wavefront's sum of the series and the target's term if it is held there.
 
-template <class T, int KW, int V, bool Reduce>
+template <class T, int KW, int V, bool Reduce, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                   float *__restrict__ loss, Partials part,
                                                                   const TaylorParams p) {
     __shared__ float parts[2][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     int64_t lb[V];
-    load_labels<V>(lab + at.pix, lb);
+    at.labels(lab, p.ignore, lb);
     if (at.here > 0) {                                  // wave-uniform
         typename Pack<T, V>::Raw raw[KW];
         at.load(x, p.C, p.m_size, raw);
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
         mine += out[k];
         cnt += (at.live && !ign) ? 1 : 0;
     }
-    if (at.live && loss) store_vec<V>(loss + at.pix, out);
+    if (at.live && loss) at.store_f32(loss, out);
     if constexpr (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());
@@ -314,13 +314,13 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
     }
 }
 
-template <class T, int KW, int V>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                   const Upstream up, T *__restrict__ gx,
                                                                   const TaylorParams p) {
     __shared__ float parts[2][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const SplitSlice<T, V, KW> at(p.P, p.m_size, p.C, p.xcd_run);
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     typename Pack<T, V>::Raw raw[KW];
     int64_t lb[V];
     float go[V];
@@ -328,8 +328,8 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
     unsigned keep[V];
     if (at.here > 0) {                                  // wave-uniform
         at.load(x, p.C, p.m_size, raw);
-        load_labels<V>(lab + at.pix, lb);
-        load_upstream<V>(up, at.pix, go);
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             bool ign;
@@ -697,7 +697,8 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
     constexpr bool kHasSplit = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);
     const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
-                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit, kHasSplit);
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit, kHasSplit,
+                                   kHasSplit);
     if constexpr (kHasSplit) {
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
@@ -713,6 +714,23 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                                p);                                                                                    \
         break;
                 PLH_SPLIT_DEEP_CASES
+#undef PLH_CASE
+            }
+            return grid;
+        }
+        if (shape == Shape::SplitImage) {           // tiles per image: channel planes that start on element boundaries only
+            const unsigned grid = split_image_grid<VT>(p.P / p.m_size, p.m_size);
+            switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                                                                                                  \
+    case KW:                                                                                                          \
+        if constexpr (Kind == kTaylorCeFwd)                                                                           \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
+                               lab, loss, part, p);                                                                   \
+        else                                                                                                          \
+            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, \
+                               out, p);                                                                               \
+        break;
+                PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
             }
             return grid;

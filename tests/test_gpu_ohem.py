@@ -64,6 +64,9 @@ SCORE_CASES = [
     ((2, 24, 4097, 1), 255, 0.1),        #   slices that take this form (24 channels fp32, 32 for 16-bit logits)
     ((2, 32, 65, 65), 255, 0.1),
     ((1, 25, 63, 65), 255, 0.1),
+    ((2, 150, 65, 65), 255, 0.05),       # 33..256 channels on such planes: the split shape in tiles per image
+    ((1, 33, 67, 63), -100, 0.1),
+    ((1, 256, 4097, 1), 255, 0.1),
     ((2, 19, 16, 16), 255, 1.0),         # everything ignored
 ]
 

@@ -73,8 +73,8 @@ SEG_CASES = [
     ((33, 100), -100, 0.1),                         # (N, C): one wavefront per row
     ((5, 1000), 255, 0.3),
     ((9, 77), -100, 0.1),                           # ... rows of 33..2048 channels sit in a wavefront's registers:
-    ((6, 501), 255, 0.2),                           #   2 .. 32 steps, element by element for odd lengths,
-    ((7, 201), 255, 0.1),
+    ((6, 501), 255, 0.2),                           #   2 .. 32 steps, element by element for odd lengths (in pieces of
+    ((7, 201), 255, 0.1),                           #   8, 4 or 2 bytes when only those divide a row's bytes),
     ((70, 33), -100, 0.1),                          #   rows of up to 256 channels: four rows per wavefront,
     ((21, 136), 255, 0.1),                          #   the last wavefront partly filled
     ((3, 256), 255, 0.0),
@@ -124,6 +124,13 @@ SEG_CASES = [
     ((2, 24, 63, 65), 255, 0.1),
     ((2, 32, 65, 65), 255, 0.1),                    # 16-bit slices take that form up to 32 channels (8-byte accesses
     ((1, 29, 67, 63), -100, 0.1),                   #   on 2-byte boundaries); fp32 keeps one pixel per lane here
+    ((2, 150, 65, 65), 255, 0.05),                  # 33..256 channels on planes of odd length, 4096 pixels or more: the
+    ((1, 33, 67, 63), -100, 0.1),                   #   split shape in tiles per image; the last lane of an image holds
+    ((2, 256, 4097, 1), 255, 0.1),                  #   1, 2 or 3 pixels; both ends of the channel range
+    ((3, 60, 65, 63), 255, 0.1),
+    ((2, 100, 65, 65), -100, 0.1),                  #   97..160 channels: four fp32 pixels per lane in the LSR kernels
+    ((1, 160, 71, 61), 255, 0.1),
+    ((1, 257, 65, 65), 255, 0.1),                   #   one channel more: a lane per pixel
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
