@@ -23,6 +23,10 @@ CASES = [
     ((4, 1024, 256), 19),
     ((2, 1028, 1024), 3),                        # planes of more than 2^20 pixels go chunk by chunk, the last one short
     ((1, 2048, 1025), 5),                        #   (2 and 3 chunks)
+    ((3, 65, 65), 19),                           # planes of odd length: 16-byte stores from 4-byte boundaries, the last
+    ((2, 513, 513), 4),                          #   lane of a plane with 1 .. 3 pixels
+    ((5, 257), 40),
+    ((2, 1023, 2), 7),
 ]
 
 
