@@ -34,7 +34,8 @@ def shifted(a, dt=None, by=1):
     return view
 
 
-SHAPES = [(2, 19, 32, 32), (2, 19, 65, 65), (2, 40, 16, 16), (1, 300, 8, 8), (37, 100), (5, 4104), (2, 50001), (300, 19)]
+SHAPES = [(2, 19, 32, 32), (2, 19, 65, 65), (2, 40, 16, 16), (2, 40, 64, 64), (1, 150, 65, 63), (1, 300, 8, 8), (37, 100), (5, 4104),
+          (2, 50001), (300, 19)]
 
 
 @pytest.mark.parametrize("which", ["logits", "labels", "both"])
