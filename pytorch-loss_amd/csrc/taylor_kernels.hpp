@@ -380,6 +380,118 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
     at.store(gx, p.m_size, raw);
 }
 
+// The softmax / log-softmax themselves for 33..256 channels in NCHW (SplitSlice): the parts of a pixel are each
+// wavefront's sum of the series and, in the backward, of its products with the upstream gradient; every wavefront
+// then finishes its own channels. The backward holds two slices (logits and upstream) per wavefront.
+template <class T, int KW, int V, bool PerImage = false>
+__global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__restrict__ x, T *__restrict__ out,
+                                                                  const TaylorParams p) {
+    __shared__ float parts[kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
+    using PK = Pack<T, V>;
+    typename PK::Raw raw[KW];
+    if (at.here > 0) {                                  // wave-uniform
+        at.load(x, p.C, p.m_size, raw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                float f, df;
+                taylor_pair(PK::get(raw[i], k), p.order, f, df);
+                s += (i < at.here) ? f : 0.f;
+            }
+            parts[wave][lane * V + k] = s;
+        }
+    }
+    __syncthreads();
+    if (at.here == 0 || !at.live) return;
+    const int used = (p.C + KW - 1) / KW;
+    float inv[V], ls[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f;
+        for (int w = 0; w < used; ++w) s += parts[w][lane * V + k];
+        inv[k] = 1.f / s;
+        ls[k] = logf(s);
+    }
+#pragma unroll
+    for (int i = 0; i < KW; ++i) forget_origin(raw[i]);
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        float r[V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float f, df;
+            taylor_pair(PK::get(raw[i], k), p.order, f, df);
+            r[k] = p.use_log ? logf(f) - ls[k] : f * inv[k];
+        }
+        raw[i] = PK::put(r);
+    }
+    at.store(out, p.m_size, raw);
+}
+
+template <class T, int KW, int V, bool PerImage = false>
+__global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__restrict__ g, const T *__restrict__ x,
+                                                                  T *__restrict__ gx, const TaylorParams p) {
+    __shared__ float parts[2][kSplitWaves][kWave * V];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
+    using PK = Pack<T, V>;
+    typename PK::Raw raw[KW], graw[KW];
+    if (at.here > 0) {                                  // wave-uniform
+        at.load(x, p.C, p.m_size, raw);
+        at.load(g, p.C, p.m_size, graw);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float s = 0.f, dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                float f, df;
+                taylor_pair(PK::get(raw[i], k), p.order, f, df);
+                const float gj = PK::get(graw[i], k);
+                s += (i < at.here) ? f : 0.f;
+                dot += (i < at.here) ? (p.use_log ? gj : f * gj) : 0.f;
+            }
+            parts[0][wave][lane * V + k] = s;
+            parts[1][wave][lane * V + k] = dot;
+        }
+    }
+    __syncthreads();
+    if (at.here == 0 || !at.live) return;
+    const int used = (p.C + KW - 1) / KW;
+    float inv[V], mid[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        float s = 0.f, dot = 0.f;
+        for (int w = 0; w < used; ++w) {
+            s += parts[0][w][lane * V + k];
+            dot += parts[1][w][lane * V + k];
+        }
+        inv[k] = 1.f / s;
+        mid[k] = p.use_log ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
+    }
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        forget_origin(raw[i]);
+        forget_origin(graw[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+        float r[V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+            float f, df;
+            taylor_pair(PK::get(raw[i], k), p.order, f, df);
+            const float gj = PK::get(graw[i], k);
+            r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
+        }
+        raw[i] = PK::put(r);
+    }
+    at.store(gx, p.m_size, raw);
+}
+
 // --------------------------------------------------------------- group ----
 // Any dimsize: G lanes share one slice and stride over it (launched with G = 1: a lane per slice, for what
 // no other shape takes). The series is re-evaluated in each sweep; re-reads hit cache.
@@ -695,11 +807,11 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                        const TaylorParams &p, hipStream_t st) {
     constexpr int VT = ElemTraits<T>::kVec;
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
-    constexpr bool kHasSplit = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);
+    constexpr bool kIsCe = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);       // the deep split form is theirs only
     const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
-                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, kHasSplit, kHasSplit,
-                                   kHasSplit);
-    if constexpr (kHasSplit) {
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true);
+    const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
+    if constexpr (kIsCe) {
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
             const unsigned grid = split_grid<VD>(p.P);
@@ -718,42 +830,37 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
             }
             return grid;
         }
-        if (shape == Shape::SplitImage) {           // tiles per image: channel planes that start on element boundaries only
-            const unsigned grid = split_image_grid<VT>(p.P / p.m_size, p.m_size);
-            switch (split_slots(p.C)) {
-#define PLH_CASE(KW)                                                                                                  \
-    case KW:                                                                                                          \
-        if constexpr (Kind == kTaylorCeFwd)                                                                           \
-            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
+    }
+    // 33..256 channels in NCHW; in tiles per image where the planes start on element boundaries only (or the
+    // upstream tensor of the softmax backward does)
+    const bool image = shape == Shape::SplitImage || (shape == Shape::Split && !g_ok && p.m_size >= 4096);
+    if (image || (shape == Shape::Split && g_ok)) {
+        const unsigned grid = image ? split_image_grid<VT>(p.P / p.m_size, p.m_size) : split_grid<VT>(p.P);
+#define PLH_GO(KW, IMG)                                                                                               \
+    do {                                                                                                              \
+        if constexpr (Kind == kTaylorFwd)                                                                             \
+            hipLaunchKernelGGL((taylor_sm_fwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, out, p); \
+        else if constexpr (Kind == kTaylorBwd)                                                                        \
+            hipLaunchKernelGGL((taylor_sm_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, g, x, out, p); \
+        else if constexpr (Kind == kTaylorCeFwd)                                                                      \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
                                lab, loss, part, p);                                                                   \
         else                                                                                                          \
-            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, \
+            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, \
                                out, p);                                                                               \
+    } while (0)
+        switch (split_slots(p.C)) {
+#define PLH_CASE(KW)                   \
+    case KW:                           \
+        if (image) PLH_GO(KW, true);   \
+        else PLH_GO(KW, false);        \
         break;
-                PLH_SPLIT_SLOT_CASES
+            PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
-            }
-            return grid;
+#undef PLH_GO
         }
-        if (shape == Shape::Split) {
-            const unsigned grid = split_grid<VT>(p.P);
-            switch (split_slots(p.C)) {
-#define PLH_CASE(KW)                                                                                                  \
-    case KW:                                                                                                          \
-        if constexpr (Kind == kTaylorCeFwd)                                                                           \
-            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
-                               loss, part, p);                                                                        \
-        else                                                                                                          \
-            hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
-                               p);                                                                                    \
-        break;
-                PLH_SPLIT_SLOT_CASES
-#undef PLH_CASE
-            }
-            return grid;
-        }
+        return grid;
     }
-    const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
     if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
         const bool vec = (shape == Shape::RegsVec) && g_ok;
         const bool uni = vec && tiles_are_uniform(p.m_size, VT, sizeof(T));

@@ -39,6 +39,11 @@ CASES = [
     ((2, 11, 67, 63), 1),                        #   pixels per lane where the slices fit (the backward holds two:
     ((1, 24, 4097, 1), 1),                       #   12 channels fp32, 24 for 16-bit elements; the forward one: 24 / 32)
     ((2, 25, 65, 65), 1),
+    ((2, 40, 16, 16), 1),                        # 33..256 channels, 64 pixels or more per image: the channels of a
+    ((1, 150, 12, 16), 1),                       #   pixel shared out over the wavefronts of a block
+    ((2, 256, 8, 8), 1),
+    ((2, 60, 65, 65), 1),                        #   the same on planes of odd length: tiles per image
+    ((1, 33, 67, 63), 1),
 ]
 
 
@@ -77,7 +82,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-15:])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-20:])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
