@@ -25,13 +25,22 @@ __device__ __forceinline__ float sigmoid_fast(float x) {
     return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-x * kLog2e));
 }
 
+// Vec: rows that start on 16-byte boundaries and hold a whole number of 4-element groups. Otherwise (rows of odd
+// length: a 513 x 513 crop per sample) a group is still moved in one access, from an element boundary (the
+// hardware takes such accesses, the types of Pack<T, 4> say so); only a row's last group goes element by element.
 template <class T, bool Vec>
 __device__ __forceinline__ void dice_load(const T *row, int64_t i, int64_t L, float (&v)[kDicePerThread]) {
     if constexpr (Vec) {
         load_vec<kDicePerThread>(row + i, v);
     } else {
+        if (i + kDicePerThread <= L) {
+            const typename Pack<T, 4>::Raw raw = Pack<T, 4>::load_unaligned(row + i);
 #pragma unroll
-        for (int k = 0; k < kDicePerThread; ++k) v[k] = (i + k < L) ? load_one(row + i + k) : 0.f;
+            for (int k = 0; k < kDicePerThread; ++k) v[k] = Pack<T, 4>::get(raw, k);
+        } else {
+#pragma unroll
+            for (int k = 0; k < kDicePerThread; ++k) v[k] = (i + k < L) ? load_one(row + i + k) : 0.f;
+        }
     }
 }
 
@@ -116,25 +125,39 @@ __global__ __launch_bounds__(kDiceBlock) void dice_backward(const float *__restr
     const int64_t off = (int64_t)blockIdx.y * L;
     const float numer = stats[2 * blockIdx.y], denor = stats[2 * blockIdx.y + 1], g = gout[blockIdx.y];
     const float c1 = g * p * numer / (denor * denor), c2 = g * 2.f / denor;
-    for (int64_t i = ((int64_t)blockIdx.x * kDiceBlock + threadIdx.x) * kDicePerThread; i < L;
+    auto grad_of = [&](float xv, float yv) {
+        const float q = sigmoid_fast(xv);
+        const float w = q * (1.f - q);
+        // p q^p (1-q) numer/denor^2 - 2 y q (1-q)/denor, with q^p (1-q) = q^(p-1) * q(1-q)
+        const float qp1 = mode == 1 ? 1.f : (mode == 2 ? q : powf(q, p - 1.f));
+        return w * (c1 * qp1 - c2 * yv);
+    };
+    // Rows that start on element boundaries only: the elements up to the gradient row's first 128-byte line are
+    // written one by one by the row's first block; from there on a wavefront's stores are whole lines.
+    int64_t head = 0;
+    if constexpr (!Vec) {
+        const int64_t to_line = (int64_t)((128u - (unsigned)(reinterpret_cast<uintptr_t>(gx + off) & 127u)) & 127u) / (int64_t)sizeof(T);
+        head = to_line < L ? to_line : L;
+        if (blockIdx.x == 0 && (int64_t)threadIdx.x < head)
+            store_one(gx + off + threadIdx.x, grad_of(load_one(x + off + threadIdx.x), load_one(y + off + threadIdx.x)));
+    }
+    for (int64_t i = head + ((int64_t)blockIdx.x * kDiceBlock + threadIdx.x) * kDicePerThread; i < L;
          i += (int64_t)gridDim.x * kDiceTile) {
         float xv[kDicePerThread], yv[kDicePerThread], r[kDicePerThread];
         dice_load<T, Vec>(x + off, i, L, xv);
         dice_load<T, Vec>(y + off, i, L, yv);
 #pragma unroll
-        for (int k = 0; k < kDicePerThread; ++k) {
-            const float q = sigmoid_fast(xv[k]);
-            const float w = q * (1.f - q);
-            // p q^p (1-q) numer/denor^2 - 2 y q (1-q)/denor, with q^p (1-q) = q^(p-1) * q(1-q)
-            const float qp1 = mode == 1 ? 1.f : (mode == 2 ? q : powf(q, p - 1.f));
-            r[k] = w * (c1 * qp1 - c2 * yv[k]);
-        }
+        for (int k = 0; k < kDicePerThread; ++k) r[k] = grad_of(xv[k], yv[k]);
         if constexpr (Vec) {
             store_vec<kDicePerThread>(gx + off + i, r);
         } else {
+            if (i + kDicePerThread <= L) {
+                Pack<T, 4>::store_unaligned(gx + off + i, Pack<T, 4>::put(r));
+            } else {
 #pragma unroll
-            for (int k = 0; k < kDicePerThread; ++k)
-                if (i + k < L) store_one(gx + off + i + k, r[k]);
+                for (int k = 0; k < kDicePerThread; ++k)
+                    if (i + k < L) store_one(gx + off + i + k, r[k]);
+            }
         }
     }
 }

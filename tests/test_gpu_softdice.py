@@ -28,7 +28,7 @@ def _inputs(seed, n, length, soft=False):
     return x, y
 
 
-CASES = [(1, 1), (1, 1000), (4, 37), (3, 4096), (7, 1023), (2, 100_003), (64, 512), (1, 2_000_000)]
+CASES = [(1, 1), (1, 1000), (4, 37), (3, 4096), (7, 1023), (2, 100_003), (64, 512), (1, 2_000_000), (3, 513 * 513), (5, 4099), (6, 2)]
 
 
 @pytest.mark.parametrize("n,length", CASES)
