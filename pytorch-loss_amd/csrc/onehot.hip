@@ -58,6 +58,7 @@ __global__ __launch_bounds__(kRegsBlock) void onehot_regs(const int64_t *__restr
 // re-reads are the 8 MiB (1 MiB per XCD) that the pass before it left in the second-level caches: whole planes of
 // 2048 x 2048 pixels ran at 3.4 TB/s.
 constexpr int64_t kOnehotChunk = (int64_t)1 << 20;
+template <bool Lines>      // Lines: every output plane starts on a 128-byte line and holds whole groups of four
 __global__ __launch_bounds__(kRegsBlock) void onehot_plane(const int64_t *__restrict__ lab, float *__restrict__ out,
                                                           int32_t *__restrict__ flags, int64_t m_size, int C,
                                                           int chunks, int64_t chunk, int64_t ignore, float lb_pos,
@@ -71,16 +72,24 @@ __global__ __launch_bounds__(kRegsBlock) void onehot_plane(const int64_t *__rest
     // a plane may hold fewer than four pixels and goes pixel by pixel.
     const int64_t *lplane = lab + (int64_t)n * m_size;
     float *oplane = out + ((int64_t)n * C + j) * m_size;
-    const int64_t to_line = (int64_t)((128u - (unsigned)(reinterpret_cast<uintptr_t>(oplane) & 127u)) & 127u) / 4;
-    const int64_t head = to_line < m_size ? to_line : m_size;
+    int64_t head = 0;
+    if constexpr (!Lines) {
+        const int64_t to_line = (int64_t)((128u - (unsigned)(reinterpret_cast<uintptr_t>(oplane) & 127u)) & 127u) / 4;
+        head = to_line < m_size ? to_line : m_size;
+    }
     auto encode = [&](int64_t label) { return (label == ignore) ? 0.f : ((label == j) ? lb_pos : lb_neg); };
     int64_t seen[5] = {ignore, ignore, ignore, ignore, ignore};      // this lane's labels, for the range check below
-    if (q == 0 && blockIdx.x == 0 && (int64_t)threadIdx.x < head) {
-        seen[4] = lplane[threadIdx.x];
-        oplane[threadIdx.x] = encode(seen[4]);
+    if constexpr (!Lines) {
+        if (q == 0 && blockIdx.x == 0 && (int64_t)threadIdx.x < head) {
+            seen[4] = lplane[threadIdx.x];
+            oplane[threadIdx.x] = encode(seen[4]);
+        }
     }
     const int64_t m = head + (int64_t)q * chunk + ((int64_t)blockIdx.x * kRegsBlock + threadIdx.x) * 4;
-    if (m + 4 <= m_size) {
+    if constexpr (Lines) {
+        if (m >= m_size) return;
+    }
+    if (Lines || m + 4 <= m_size) {
         const plh_l2_a8 a = *reinterpret_cast<const plh_l2_a8 *>(lplane + m);
         const plh_l2_a8 b = *reinterpret_cast<const plh_l2_a8 *>(lplane + m + 2);
         seen[0] = a.x; seen[1] = a.y; seen[2] = b.x; seen[3] = b.y;
@@ -155,9 +164,13 @@ extern "C" int plh_onehot(const int64_t *labels, float *one_hot, int32_t *range_
         // XCD, and its labels that XCD's L2, in every channel pass. Planes of 977 or 258 tiles ran at 35-42 % of peak
         // (every channel pass fetched the labels from memory again) where planes of 1024 tiles ran at 90 %.
         const int64_t chunk = ceil_div(ceil_div(m_size, chunks), 8192) * 8192;
-        hipLaunchKernelGGL(onehot_plane, dim3((unsigned)(chunk / 1024), (unsigned)dimsize, (unsigned)(n_size * chunks)),
-                           dim3(kRegsBlock), 0, st, labels, one_hot, range_flags, m_size, C, (int)chunks, chunk,
-                           ignore_index, lb_pos, lb_neg);
+        const dim3 grid((unsigned)(chunk / 1024), (unsigned)dimsize, (unsigned)(n_size * chunks));
+        if (m_size % 32 == 0 && !misaligned(one_hot, 128))
+            hipLaunchKernelGGL(onehot_plane<true>, grid, dim3(kRegsBlock), 0, st, labels, one_hot, range_flags, m_size, C,
+                               (int)chunks, chunk, ignore_index, lb_pos, lb_neg);
+        else
+            hipLaunchKernelGGL(onehot_plane<false>, grid, dim3(kRegsBlock), 0, st, labels, one_hot, range_flags, m_size, C,
+                               (int)chunks, chunk, ignore_index, lb_pos, lb_neg);
         return check_launch();
     }
     if (shape == Shape::RegsVec || shape == Shape::RegsOne) {
