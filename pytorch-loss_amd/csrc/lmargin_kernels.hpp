@@ -787,7 +787,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
     // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
     constexpr bool kHasSplit = !(WantLoss && WantGrad);
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
-                       second_f32, kHasSplit, kHasSplit, kHasSplit)) {
+                       second_f32, kHasSplit, kHasSplit, kHasSplit, kImageFormMaxChannels<T>)) {
         case Shape::SplitDeep:
             if constexpr (kHasSplit) {
                 constexpr int VD = V / 2;

@@ -882,7 +882,8 @@ template <class T, bool Reduce>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
                         hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true, true,
+                       kImageFormMaxChannels<T>)) {
         case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) return launch_fwd_image<T, Reduce>(logits, labels, losses, part, p, st);
@@ -923,7 +924,8 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
-    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true, true)) {
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true, true,
+                       kImageFormMaxChannels<T>)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) {

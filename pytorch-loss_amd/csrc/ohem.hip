@@ -530,7 +530,8 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
         constexpr int VT = ElemTraits<T>::kVec;
-        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true, true, true);
+        const Shape shape = pick_shape(dimsize, m_size, VT, sizeof(T), x, nullptr, labels, scores, ce, true, true, true,
+                                       kImageFormMaxChannels<T>);
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
             const unsigned grid = split_grid<VD>(P);

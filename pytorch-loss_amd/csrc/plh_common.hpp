@@ -87,13 +87,19 @@ constexpr int kMaxDeepChannels = kMaxDeepSlots * kSplitWaves;
 
 inline Shape pick_shape(int64_t dimsize, int64_t m_size, int V, size_t elem, const void *typed0, const void *typed1,
                         const void *labels, const void *f32a, const void *f32b, bool with_split = false,
-                        bool with_deep = false, bool with_image = false) {
+                        bool with_deep = false, bool with_image = false, int regs_image_max = 0) {
     auto fits = [&](int v) {
         return (m_size % v == 0) && !(typed0 && misaligned(typed0, v * elem)) &&
                !(typed1 && misaligned(typed1, v * elem)) && !(f32a && misaligned(f32a, v * 4)) &&
                !(f32b && misaligned(f32b, v * 4)) && !(labels && misaligned(labels, v > 1 ? 16 : 8));
     };
-    const bool vec = fits(V) && !(labels && misaligned(labels, 16));
+    bool vec = fits(V) && !(labels && misaligned(labels, 16));
+    // Planes that do not start on 128-byte lines (1022 x 1022, 510 x 510) take the tiles-per-image forms as the
+    // odd ones do, where the caller has them for this channel count: fp32 LSR fwd+bwd (8,19,1022,1022)
+    // 0.433 -> 0.395 ms, (8,150,510,510) 0.947 -> 0.834 ms against 8-byte accesses whose runs straddle lines.
+    if (with_image && m_size >= 4096 && (m_size * (int64_t)elem) % 128 != 0 &&
+        (dimsize > kMaxRegsChannels || dimsize <= regs_image_max))
+        vec = false;
     if (dimsize <= kMaxRegsChannels) return vec ? Shape::RegsVec : Shape::RegsOne;
     if (with_split && vec && dimsize <= kMaxSplitChannels && m_size >= 64) return Shape::Split;
     // planes that start on element boundaries only (odd lengths) and are long enough that the partly filled

@@ -809,7 +809,8 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
     constexpr bool kIsCe = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);       // the deep split form is theirs only
     const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
-                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true);
+                                   lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true,
+                                   kImageFormMaxChannels<T, (Kind == kTaylorBwd) ? 2 : 1>);
     const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
     if constexpr (kIsCe) {
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane

@@ -131,6 +131,9 @@ SEG_CASES = [
     ((2, 100, 65, 65), -100, 0.1),                  #   97..160 channels: four fp32 pixels per lane in the LSR kernels
     ((1, 160, 71, 61), 255, 0.1),
     ((1, 257, 65, 65), 255, 0.1),                   #   one channel more: a lane per pixel
+    ((2, 19, 66, 66), 255, 0.1),                    # planes of even length that do not start on 128-byte lines take
+    ((2, 60, 66, 66), -100, 0.1),                   #   the tiles-per-image forms as well (4356 pixels: 17424 or 8712 bytes)
+    ((1, 28, 66, 66), 255, 0.1),                    #   ... but not where that form does not reach (28 channels in fp32)
     ((2, 19, 16, 16), 255, 1.0),                    # everything ignored
 ]
 
