@@ -29,28 +29,71 @@ constexpr int kLnBlock = 256;
 // KW = channel slots per wave (>= the channels it holds), V = pixels per lane, WS = waves sharing a
 // pixel group (1: each of a block's four waves has its own group and all channels; 4 or 8: the block
 // is WS waves with 1/WS of the channels each).
-template <class T, int KW, int V, int WS, bool Bwd>
+// PerImage: pixel groups that never straddle two images (groups = images x groups per image), for channel planes
+// that start on element boundaries only (odd lengths): a lane's V pixels are moved with accesses of the same
+// width from element boundaries; the last lane of an image may hold fewer and goes pixel by pixel.
+template <class T, int KW, int V, int WS, bool Bwd, bool PerImage = false>
 __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *__restrict__ x, const T *__restrict__ g,
                                                     T *__restrict__ out, const LnParams p) {
     using PK = Pack<T, V>;
     __shared__ float ex[WS][2][V][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t group = WS > 1 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
-    const int64_t pix = (group * 64 + lane) * V;
-    const bool live = pix < p.P;
-    const int64_t pc = live ? pix : 0;                 // dead lanes read pixel 0 and store nothing
-    const int64_t n = pc / p.m_size;
+    bool live;
+    int nv = V;                                        // pixels this lane has
+    int64_t pc, n;
+    if constexpr (PerImage) {
+        const int64_t per_image = ceil_div_dev(p.m_size, (int64_t)64 * V);
+        n = group / per_image;
+        const int64_t local = ((group - n * per_image) * 64 + lane) * V;
+        const int64_t left = p.m_size - local;
+        nv = left >= V ? V : (left > 0 ? (int)left : 0);
+        live = nv > 0 && n * p.m_size < p.P;
+        if (!live) { n = 0; nv = V; }                  // dead lanes read pixel 0 and store nothing
+        pc = live ? n * p.m_size + local : 0;
+    } else {
+        const int64_t pix = (group * 64 + lane) * V;
+        live = pix < p.P;
+        pc = live ? pix : 0;                           // dead lanes read pixel 0 and store nothing
+        n = pc / p.m_size;
+    }
     const int c0 = WS > 1 ? wave * p.per_wave : 0;
     int cnt = WS > 1 ? p.C - c0 : p.C;
     cnt = cnt < 1 ? 1 : (WS > 1 && cnt > p.per_wave ? p.per_wave : cnt);   // a split always leaves every wave >= 1 channel
     cnt = __builtin_amdgcn_readfirstlane(cnt);
     const int64_t base = pc + n * (int64_t)(p.C - 1) * p.m_size + (int64_t)c0 * p.m_size;
+    auto fetch = [&](const T *at) {
+        if constexpr (PerImage) {
+            if (nv < V) {
+                float one[V];
+#pragma unroll
+                for (int k = 0; k < V; ++k) one[k] = k < nv ? load_one(at + k) : 0.f;
+                return PK::put(one);
+            }
+            return PK::load_unaligned(at);
+        } else {
+            return PK::load(at);
+        }
+    };
+    auto put_back = [&](T *at, const float (&r)[V]) {
+        if constexpr (PerImage) {
+            if (nv < V) {
+#pragma unroll
+                for (int k = 0; k < V; ++k)
+                    if (k < nv) store_one(at + k, r[k]);
+                return;
+            }
+            PK::store_unaligned(at, PK::put(r));
+        } else {
+            PK::store(at, PK::put(r));
+        }
+    };
 
     // Slots past the wave's last channel re-read that channel (same address, served by cache) and are
     // weighted out of the sums: straight-line code, no per-slot control flow.
     typename PK::Raw raw[KW];
 #pragma unroll
-    for (int j = 0; j < KW; ++j) raw[j] = PK::load(x + base + (int64_t)(j < cnt ? j : cnt - 1) * p.m_size);
+    for (int j = 0; j < KW; ++j) raw[j] = fetch(x + base + (int64_t)(j < cnt ? j : cnt - 1) * p.m_size);
 
     const float inv_c = 1.f / (float)p.C;
     float mean[V], v[V];
@@ -117,7 +160,7 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
             float r[V];
 #pragma unroll
             for (int k = 0; k < V; ++k) r[k] = (PK::get(raw[j], k) - mean[k]) * rstd[k];
-            if (live && j < cnt) PK::store(out + base + (int64_t)j * p.m_size, PK::put(r));
+            if (live && j < cnt) put_back(out + base + (int64_t)j * p.m_size, r);
         }
     } else {
         constexpr int kChunk = KW < 8 ? KW : 8;        // gradient slices in flight per trip
@@ -126,7 +169,7 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
             typename PK::Raw graw[kChunk];
 #pragma unroll
             for (int jj = 0; jj < kChunk; ++jj)
-                graw[jj] = PK::load(g + base + (int64_t)(j0 + jj < cnt ? j0 + jj : cnt - 1) * p.m_size);
+                graw[jj] = fetch(g + base + (int64_t)(j0 + jj < cnt ? j0 + jj : cnt - 1) * p.m_size);
 #pragma unroll
             for (int jj = 0; jj < kChunk; ++jj) {
                 float r[V];
@@ -136,7 +179,7 @@ __global__ __launch_bounds__(WS > 4 ? 64 * WS : kLnBlock) void ln_regs(const T *
                     const float inner = __builtin_fmaf((val - mean[k]) * (val - inv_c), mv[k], inv_c);
                     r[k] = -rstd[k] * inner * PK::get(graw[jj], k);
                 }
-                if (live && j0 + jj < cnt) PK::store(out + base + (int64_t)(j0 + jj) * p.m_size, PK::put(r));
+                if (live && j0 + jj < cnt) put_back(out + base + (int64_t)(j0 + jj) * p.m_size, r);
             }
         }
     }
@@ -231,12 +274,17 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
     }
     const bool vec = dimsize <= 768 && m_size % VT == 0 && !misaligned(x, VT * sizeof(T)) &&
                      !misaligned(out, VT * sizeof(T)) && !(Bwd && misaligned(g, VT * sizeof(T)));
-    const int64_t groups = ceil_div(p.P, 64 * (vec ? VT : 1));
+    // planes that start on element boundaries only (odd lengths, misaligned tensors) and are long enough that
+    // the partly filled last group of every image is a small share: the same pixels per lane in groups per image
+    const bool image = !vec && dimsize <= 768 && m_size >= 4096;
+    const int64_t groups = image ? n_size * ceil_div(m_size, 64 * VT) : ceil_div(p.P, 64 * (vec ? VT : 1));
     const unsigned grid = (unsigned)(ws > 1 ? groups : ceil_div(groups, 4));
     const int slots = p.per_wave;
 #define PLH_LN(KW, VV, WS) \
     hipLaunchKernelGGL((ln_regs<T, KW, VV, WS, Bwd>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
-#define PLH_LN_V(KW, WS) do { if (vec) PLH_LN(KW, VT, WS); else PLH_LN(KW, 1, WS); } while (0)
+#define PLH_LN_IMAGE(KW, WS) \
+    hipLaunchKernelGGL((ln_regs<T, KW, VT, WS, Bwd, true>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
+#define PLH_LN_V(KW, WS) do { if (vec) PLH_LN(KW, VT, WS); else if (image) PLH_LN_IMAGE(KW, WS); else PLH_LN(KW, 1, WS); } while (0)
     // Slot counts in steps of about 1.5x: a wave whose channels fall short of its slots re-reads its last
     // channel for the rest, and at 12 channels in 16 slots that cost a third of the bandwidth.
     if (ws == 1) {
@@ -257,6 +305,7 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
     else if (slots <= 96) PLH_LN_V(96, 8);             // C <= 768
     else PLH_LN(128, 1, 8);                            // 768 < C <= 1024: one pixel per lane
 #undef PLH_LN_V
+#undef PLH_LN_IMAGE
 #undef PLH_LN
 }
 

@@ -24,7 +24,9 @@ def pl():
 # and the two-sweep kernel (C > 1024)
 SHAPES = [(2, 1, 64), (2, 3, 130), (2, 8, 64), (1, 19, 1000), (2, 32, 66), (2, 33, 64), (1, 64, 300), (2, 65, 128),
           (1, 100, 77), (1, 128, 256), (1, 200, 64), (1, 256, 130), (1, 384, 64), (1, 512, 128), (1, 513, 64),
-          (1, 768, 70), (1, 1024, 64), (1, 1025, 40), (5, 96, 1), (3, 2000, 1), (2, 64, 49), (3, 40, 3)]
+          (1, 768, 70), (1, 1024, 64), (1, 1025, 40), (5, 96, 1), (3, 2000, 1), (2, 64, 49), (3, 40, 3),
+          # planes of odd length, 4096 pixels or more: pixel groups per image, the last lane of an image with 1 .. 3 pixels
+          (2, 19, 4225), (3, 64, 4097), (2, 100, 4099), (1, 768, 4098), (2, 40, 4331)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
