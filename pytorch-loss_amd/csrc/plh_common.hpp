@@ -1341,6 +1341,10 @@ static int wrow_steps(int C, int piece, int lanes) {
     const int need = (C + per - 1) / per;
     int steps = piece == 1 ? (lanes == 16 ? 4 : 8) : (piece == 2 && lanes == 64 ? 4 : 2);   // the smallest instantiated sizes
     while (steps < need) steps *= 2;
+    // 129..160 elements in short pieces (150 classes, channels last) would fill 5 of 8 or 10 of 16 steps: they have
+    // instances of their own
+    if (lanes == 16 && piece == 2 && need == 5) return 5;
+    if (lanes == 16 && piece == 1 && (need == 9 || need == 10)) return 10;
     return steps;
 }
 // LAUNCH(NI, L, G) launches the kernel instance; its grid is group_grid(rows, WaveRowAt<G>::kRowsPerBlock).
@@ -1354,8 +1358,13 @@ static int wrow_steps(int C, int piece, int lanes) {
     do {                                                                                 \
         const int wrow_len = (PIECE);                                                    \
         if ((C) <= kWaveRowShort) {                                                      \
-            if (wrow_len == 1) { PLH_WROW_STEPS3(1, 16, C, 4, 8, 16, LAUNCH) }           \
-            else if (wrow_len == 2) { PLH_WROW_STEPS3(2, 16, C, 2, 4, 8, LAUNCH) }       \
+            if (wrow_len == 1) {                                                         \
+                if (wrow_steps<T>(C, 1, 16) == 10) LAUNCH(10, 1, 16);                    \
+                else { PLH_WROW_STEPS3(1, 16, C, 4, 8, 16, LAUNCH) }                     \
+            } else if (wrow_len == 2) {                                                  \
+                if (wrow_steps<T>(C, 2, 16) == 5) LAUNCH(5, 2, 16);                      \
+                else { PLH_WROW_STEPS3(2, 16, C, 2, 4, 8, LAUNCH) }                      \
+            }                                                                            \
             else if (wrow_len == 4) { PLH_WROW_STEPS3(4, 16, C, 2, 4, 4, LAUNCH) }       \
             else if constexpr (RowChunk<T>::kLen == 8) { LAUNCH(2, 8, 16); }             \
         } else {                                                                         \

@@ -87,6 +87,9 @@ SEG_CASES = [
     ((3, 1002), 255, 0.1),
     ((4, 2046), -100, 0.0),
     ((6, 300), 255, 0.1),
+    ((9, 151), 255, 0.1),                           #   129..160 elements in short pieces: 5 steps of two, 10 of one
+    ((5, 130), -100, 0.1),
+    ((7, 143), 255, 0.1),
     ((2, 2049), -100, 0.0),                         # one channel more: staged or swept rows
     ((4, 3000), -100, 0.1),                         # 16-bit rows in whole chunks stay in a wavefront's registers up to
     ((3, 4096), 255, 0.1),                          #   4096 elements (8 steps of 8); fp32 rows take a block per row
