@@ -485,6 +485,8 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                                                const LmParams p) {
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
+    using Span = WaveRowSpan<T, L, G>;
+    T *tile = Span::tile();
     const WaveRowAt<G> at;
     const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
@@ -557,10 +559,14 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             }
             if constexpr (WantGrad) {
                 if (ok && live) {
-                    T *gs = grad + row * p.C + e0;
-                    RowPiece<T, L>::store(gs, g);
+                    if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, g);
+                    else RowPiece<T, L>::store(grad + row * p.C + e0, g);
                 }
             }
+        }
+        if constexpr (WantGrad && Span::kUse) {
+            const int64_t left = p.P - r0;
+            Span::flush(tile, grad + r0 * p.C, left < Span::kRows ? (int)left : Span::kRows, p.C);
         }
         if constexpr (WantLoss) {
             acc = group_reduce<G>(acc, OpSum());

@@ -479,6 +479,8 @@ template <class T, int NI, int LP, int G>
 __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, T *__restrict__ grad, const LsrParams p) {
     constexpr int L = WaveRow<T, NI, LP, G>::L;
+    using Span = WaveRowSpan<T, L, G>;
+    T *tile = Span::tile();
     const WaveRowAt<G> at;
     for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
         const bool live = r0 + at.grp < p.P;
@@ -511,8 +513,13 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
                 float g[L];
 #pragma unroll
                 for (int l = 0; l < L; ++l) g[l] = __builtin_fmaf(r.v[i][l], scale, (e0 + l == tgt) ? n_pos : n_neg);
-                RowPiece<T, L>::store(gs + e0, g);
+                if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, g);
+                else RowPiece<T, L>::store(gs + e0, g);
             }
+        }
+        if constexpr (Span::kUse) {
+            const int64_t left = p.P - r0;
+            Span::flush(tile, grad + r0 * p.C, left < Span::kRows ? (int)left : Span::kRows, p.C);
         }
     }
 }

@@ -306,6 +306,7 @@ template <> struct Pack<float, 2> {
 // a lane's 16 bytes start on a 4-byte boundary; the hardware takes such accesses, the types say so).
 typedef unsigned plh_u4w __attribute__((ext_vector_type(4)));
 typedef unsigned plh_u4w_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned plh_u4_a2 __attribute__((ext_vector_type(4), aligned(2)));
 typedef float plh_f4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 template <> struct Pack<float, 4> {
     typedef plh_u4w Raw;
@@ -1311,6 +1312,51 @@ struct WaveRowAt {
         grp = lane / G;
         start = ((int64_t)blockIdx.x * 4 + wave) * kRowsPerWave;
         stride = (int64_t)gridDim.x * kRowsPerBlock;
+    }
+};
+
+// Results of a wavefront's short rows written as one run. With 16 lanes per row and pieces shorter than 16 bytes a
+// step's stores are four separate segments of 32..128 bytes; the four rows of a round are contiguous in memory, so
+// they are gathered in LDS (as stored: T) and leave as 16-byte pieces of one run of 4*C elements, whose lines are
+// whole except the run's first and last.
+constexpr int kWaveRowShortElems = 256;       // = kWaveRowShort below: the longest row that 16 lanes share
+template <class T, int L, int G>
+struct WaveRowSpan {
+    static constexpr bool kUse = (G == 16 && L < RowChunk<T>::kLen);
+    static constexpr int kRows = 64 / G;
+    static __device__ __forceinline__ T *tile() {
+        __shared__ __attribute__((aligned(16))) T buf[4][kUse ? kRows * kWaveRowShortElems : 8];
+        return buf[threadIdx.x >> 6];
+    }
+    // the piece of step i of lane (grp, sub) into the tile
+    static __device__ __forceinline__ void stage(T *tile, int C, int grp, int e0, const float (&g)[L]) {
+        T *at = tile + grp * C + e0;
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int l = 0; l < L; ++l) reinterpret_cast<float *>(at)[l] = g[l];
+        } else if constexpr (L == 1) {
+            store_one(at, g[0]);
+        } else {
+#pragma unroll
+            for (int l = 0; l < L; l += 2) *reinterpret_cast<unsigned *>(at + l) = narrow2(g[l], g[l + 1], T{});
+        }
+    }
+    // the rows of the round (`rows` of them, from `dst` on) out of the tile; all 64 lanes call it
+    static __device__ __forceinline__ void flush(const T *tile, T *dst, int rows, int C) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int kPer = 16 / (int)sizeof(T);
+        typedef typename std::conditional<sizeof(T) == 4, plh_u4w_a4, plh_u4_a2>::type Piece;   // 16 bytes from an element boundary
+        const int lane = threadIdx.x & 63, n = rows * C;
+        const plh_u4 *tile4 = reinterpret_cast<const plh_u4 *>(tile);
+        for (int c = lane; c < n / kPer; c += 64) {
+            const plh_u4 v = tile4[c];
+            __builtin_nontemporal_store(Piece{v.x, v.y, v.z, v.w}, reinterpret_cast<Piece *>(dst + c * kPer));
+        }
+        const int done = n / kPer * kPer;
+        if (lane < n - done) dst[done + lane] = tile[done + lane];
+        __builtin_amdgcn_wave_barrier();        // the tile is free again only when every lane has read its pieces
     }
 };
 

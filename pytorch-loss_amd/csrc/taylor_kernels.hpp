@@ -598,6 +598,8 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                                                    const TaylorParams p) {
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
+    using Span = WaveRowSpan<T, L, G>;
+    T *tile = Span::tile();
     const WaveRowAt<G> at;
     const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
@@ -670,9 +672,13 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                     }
                 }
                 if (e0 < p.C && live) {
-                    T *dst = out + row * p.C + e0;
-                    RowPiece<T, L>::store(dst, o);
+                    if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, o);
+                    else RowPiece<T, L>::store(out + row * p.C + e0, o);
                 }
+            }
+            if constexpr (Span::kUse) {
+                const int64_t left = p.P - r0;
+                Span::flush(tile, out + r0 * p.C, left < Span::kRows ? (int)left : Span::kRows, p.C);
             }
         }
     }
