@@ -565,13 +565,16 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
                 float go[1];
                 load_upstream<1>(up, pc, go);
                 const float gk = has_y ? go[0] : 0.f;
+                // f' times one of two factors per pixel: the division by f(x_y) happens once, not per channel
+                float f_y = 1.f, df_y;
+                if (has_y) taylor_pair(load_one(xs + lb * p.m_size), p.order, f_y, df_y);
+                const float cold = inv * gk, hot = cold - gk / f_y;
                 if (live)
 #pragma unroll kGroupUnroll<G>
                     for (int j = sub; j < p.C; j += G) {
                         float f, df;
                         taylor_pair(load_one(xs + (int64_t)j * p.m_size), p.order, f, df);
-                        store_one(out + base + (int64_t)j * p.m_size,
-                                  has_y ? df * inv * gk - ((lb == j) ? df / f * gk : 0.f) : 0.f);
+                        store_one(out + base + (int64_t)j * p.m_size, has_y ? df * ((lb == j) ? hot : cold) : 0.f);
                     }
             }
         }
@@ -644,14 +647,17 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
             const float ls = logf(s);
             const float mid = p.use_log ? dot * inv : dot * inv * inv;
             int tgt = -1;
-            float gk = 0.f;
+            float cold = 0.f, hot = 0.f;        // cross entropy: f' times one of these, see taylor_group
             if constexpr (Kind == kTaylorCeBwd) {
                 const int64_t lb = lab[row];
                 float go[1];
                 load_upstream<1>(up, row, go);
                 if (lb != p.ignore && lb >= 0 && lb < p.C) {
                     tgt = (int)lb;
-                    gk = go[0];
+                    float f_y, df_y;
+                    taylor_pair(load_one(xs + lb), p.order, f_y, df_y);
+                    cold = inv * go[0];
+                    hot = cold - go[0] / f_y;
                 }
             }
 #pragma unroll
@@ -668,7 +674,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                         const float gj = rg.v[i][l];
                         o[l] = p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
                     } else {
-                        o[l] = (tgt >= 0) ? df * inv * gk - ((e0 + l == tgt) ? df / f * gk : 0.f) : 0.f;
+                        o[l] = (tgt >= 0) ? df * ((e0 + l == tgt) ? hot : cold) : 0.f;
                     }
                 }
                 if (e0 < p.C && live) {
@@ -791,10 +797,13 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
             const float gk = has_y ? go[0] : 0.f;
             const float inv = 1.f / s;
             const int tgt = has_y ? (int)lb : -1;
+            float f_y = 1.f, df_y;
+            if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df_y);
+            const float cold = inv * gk, hot = cold - gk / f_y;          // see taylor_group
             row_map<T>(xs, out + row * p.C, p.C, vec != 0, [&](float v, int j) {
                 float f, df;
                 taylor_pair(v, p.order, f, df);
-                return has_y ? df * inv * gk - ((j == tgt) ? df / f * gk : 0.f) : 0.f;
+                return has_y ? df * ((j == tgt) ? hot : cold) : 0.f;
             });
         }
     }
