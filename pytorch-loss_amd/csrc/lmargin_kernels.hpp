@@ -503,34 +503,44 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         float go[1] = {1.f};
         if constexpr (WantGrad) load_upstream<1>(up, row, go);
 
-        float m_no = -INFINITY, x_y = -INFINITY;
+        // The target leaves the row: with -inf in its slot, as in the slots beyond the row, the sweeps over
+        // "the other channels" need no mask of their own (exp gives 0, the linear terms test for -inf).
+        const float x_y = (tgt >= 0) ? load_one(xs + tgt) : -INFINITY;
+        float m_no = -INFINITY;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int l = 0; l < L; ++l) {
-                const float t = r.v[i][l];              // -inf beyond the row
                 const bool hot = ((lane + G * i) * L + l == tgt);
-                x_y = hot ? t : x_y;
-                m_no = hot ? m_no : fmaxf(m_no, t);
+                r.v[i][l] = hot ? -INFINITY : r.v[i][l];
+                m_no = fmaxf(m_no, r.v[i][l]);
             }
         m_no = group_reduce<G>(m_no, OpMax());
-        x_y = group_reduce<G>(x_y, OpMax());
         const float m_all = fmaxf(m_no, x_y);
-        float s_no = 0.f, sum_ex = 0.f;
+        // Without gradients the margin term needs no third sweep: with d = x - m_no over the channels other
+        // than the target, sum (q - coeff) (d - lse_no) = (sum e d) / s_no - lse_no - coeff (sum d - n lse_no).
+        constexpr bool kClosed = WantLoss && !WantGrad;
+        float s_no = 0.f, sum_ex = 0.f, sum_d = 0.f;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const bool ok = (lane + G * i) * L < p.C;
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 const float t = r.v[i][l];
-                const bool hot = ((lane + G * i) * L + l == tgt);
-                const float e = hot ? 0.f : fast_exp(t - m_no);
+                const float d = t - m_no;
+                const float e = fast_exp(d);
+                const bool in = d > -INFINITY;
                 s_no += e;
-                sum_ex += ok ? e * t : 0.f;
+                if constexpr (kClosed) {
+                    const float dz = in ? d : 0.f;
+                    sum_ex = __builtin_fmaf(e, dz, sum_ex);
+                    sum_d += dz;
+                } else {
+                    sum_ex = __builtin_fmaf(e, in ? t : 0.f, sum_ex);
+                }
             }
-        }
         s_no = group_reduce<G>(s_no, OpSum());
         sum_ex = group_reduce<G>(sum_ex, OpSum());
+        if constexpr (kClosed) sum_d = group_reduce<G>(sum_d, OpSum());
         const float t_all = fast_exp(m_no - m_all);
         const float e_y = fast_exp(x_y - m_all);
         const float s_all = s_no * t_all + e_y;
@@ -539,8 +549,12 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         const float lse_no = logf(s_no);
         const float g_hot = (e_y * inv_all - 1.f) * go[0];
         float acc = 0.f;
+        if constexpr (kClosed) {
+            const float n_no = (float)(p.C - (tgt >= 0 ? 1 : 0));
+            acc = p.half_lam * (sum_ex * inv_no - lse_no - p.coeff * (sum_d - n_no * lse_no));
+        }
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = 0; i < (kClosed ? 0 : NI); ++i) {
             const int e0 = (lane + G * i) * L;
             const bool ok = e0 < p.C;
             float g[L];
@@ -569,7 +583,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             Span::flush(tile, grad + r0 * p.C, left < Span::kRows ? (int)left : Span::kRows, p.C);
         }
         if constexpr (WantLoss) {
-            acc = group_reduce<G>(acc, OpSum());
+            if constexpr (!kClosed) acc = group_reduce<G>(acc, OpSum());
             acc += -(x_y - m_all) + logf(s_all);
             if (lane == 0 && live) {
                 if (loss) loss[row] = ign ? 0.f : acc;
