@@ -478,7 +478,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 // (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
 // sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group.
 
-template <class T, int NI, int LP, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G>
+template <class T, int NI, int LP, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
@@ -574,7 +574,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             if constexpr (WantGrad) {
                 if (ok && live) {
                     if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, g);
-                    else RowPiece<T, L>::store(grad + row * p.C + e0, g);
+                    else RowPiece<T, L>::template store<Cached>(grad + row * p.C + e0, g);
                 }
             }
         }
@@ -876,6 +876,13 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
 #define PLH_GO(NI, W, G)                                                                                           \
     do {                                                                                                           \
         blocks = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                     \
+        if constexpr (WantGrad && wrow_cached_form<T>(W, G)) {                                                     \
+            if (wrow_rows_end_inside_lines<T>(p.C)) {                                                              \
+                hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G, true>), dim3(blocks), \
+                                   dim3(256), 0, st, x, lab, up, loss, grad, cnt, part, p);                        \
+                break;                                                                                             \
+            }                                                                                                      \
+        }                                                                                                          \
         hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G>), dim3(blocks), dim3(256), 0, \
                            st, x, lab, up, loss, grad, cnt, part, p);                                              \
     } while (0)

@@ -475,7 +475,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
     }
 }
 
-template <class T, int NI, int LP, int G>
+template <class T, int NI, int LP, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, T *__restrict__ grad, const LsrParams p) {
     constexpr int L = WaveRow<T, NI, LP, G>::L;
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
 #pragma unroll
                 for (int l = 0; l < L; ++l) g[l] = __builtin_fmaf(r.v[i][l], scale, (e0 + l == tgt) ? n_pos : n_neg);
                 if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, g);
-                else RowPiece<T, L>::store(gs + e0, g);
+                else RowPiece<T, L>::template store<Cached>(gs + e0, g);
             }
         }
         if constexpr (Span::kUse) {
@@ -971,9 +971,18 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                 break;
             }
             {
-#define PLH_GO(NI, W, G)                                                                                          \
-    hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
-                       st, logits, labels, up, grad_logits, p)
+#define PLH_GO(NI, W, G)                                                                                           \
+    do {                                                                                                           \
+        if constexpr (wrow_cached_form<T>(W, G)) {                                                                 \
+            if (wrow_rows_end_inside_lines<T>(p.C)) {                                                              \
+                hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G, true>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), \
+                                   dim3(256), 0, st, logits, labels, up, grad_logits, p);                          \
+                break;                                                                                             \
+            }                                                                                                      \
+        }                                                                                                          \
+        hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
+                           st, logits, labels, up, grad_logits, p);                                                \
+    } while (0)
                 PLH_WROW_DISPATCH(wrow_piece<T>(logits, grad_logits, p.C), p.C, PLH_GO);
 #undef PLH_GO
             }

@@ -1214,6 +1214,9 @@ template <> struct RowChunk<float> {
     static __device__ __forceinline__ void store(float *p, const float (&v)[4]) {
         __builtin_nontemporal_store(plh_f4{v[0], v[1], v[2], v[3]}, reinterpret_cast<plh_f4 *>(p));
     }
+    static __device__ __forceinline__ void store_cached(float *p, const float (&v)[4]) {
+        *reinterpret_cast<plh_f4 *>(p) = plh_f4{v[0], v[1], v[2], v[3]};
+    }
 };
 template <class T> struct RowChunk {             // T = f16 or bf16
     static constexpr int kLen = 8;
@@ -1230,6 +1233,10 @@ template <class T> struct RowChunk {             // T = f16 or bf16
         const plh_u4 t = {narrow2(v[0], v[1], T{}), narrow2(v[2], v[3], T{}), narrow2(v[4], v[5], T{}),
                           narrow2(v[6], v[7], T{})};
         __builtin_nontemporal_store(t, reinterpret_cast<plh_u4 *>(p));
+    }
+    static __device__ __forceinline__ void store_cached(T *p, const float (&v)[8]) {
+        *reinterpret_cast<plh_u4 *>(p) = plh_u4{narrow2(v[0], v[1], T{}), narrow2(v[2], v[3], T{}),
+                                                 narrow2(v[4], v[5], T{}), narrow2(v[6], v[7], T{})};
     }
 };
 
@@ -1265,6 +1272,15 @@ template <class T, int L> struct RowPiece {
         } else {
             *reinterpret_cast<plh_u2 *>(p) = plh_u2{narrow2(v[0], v[1], T{}), narrow2(v[2], v[3], T{})};
         }
+    }
+    // Cached: 16-byte pieces through the cache as well -- for short rows that end inside a line,
+    // four to a wavefront: (1 M, 200) LSR backward fp32 0.370 -> 0.315 ms, bf16 0.201 -> 0.154 ms; with a wavefront
+    // per row it made no difference. A compile-time choice: with both kinds of store in one kernel behind a
+    // wave-uniform branch the aligned rows lost 10-15 %.
+    template <bool Cached>
+    static __device__ __forceinline__ void store(T *p, const float (&v)[L]) {
+        if constexpr (L == RowChunk<T>::kLen && Cached) RowChunk<T>::store_cached(p, v);
+        else store(p, v);
     }
 };
 
@@ -1364,7 +1380,8 @@ struct WaveRowSpan {
 // longer ones a whole wavefront. The piece is the largest of 16, 8, 4, 2 bytes that divides the row's bytes
 // and that every tensor involved is aligned to. Instantiated steps -- 16 lanes: 4, 8, 16 single elements,
 // 2, 4, 8 pieces of two, 2, 4 of four, 2 of eight; 64 lanes: 8, 16, 32 single elements, 4, 8, 16 pieces of
-// two, 2, 4, 8 of four or eight.
+// two, 2, 4, 8 of four or eight. 16-bit rows of 257..512 elements in 16-byte pieces also get 16 lanes (4 steps: the
+// same KiB per row as 256 fp32 elements; a whole wavefront for 528 bytes left the bf16 LSR backward at 39 % of peak).
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
 // 16-bit rows that move in 16-byte pieces go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the
@@ -1393,6 +1410,12 @@ static int wrow_steps(int C, int piece, int lanes) {
     if (lanes == 16 && piece == 1 && (need == 9 || need == 10)) return 10;
     return steps;
 }
+// Kernels that write a row of results have a second instance for short rows in 16-byte pieces whose ends fall inside
+// 128-byte lines (RowPiece::store<true>): which (piece, lanes) have it, and which rows take it.
+template <class T>
+constexpr bool wrow_cached_form(int piece, int lanes) { return lanes == 16 && piece == RowChunk<T>::kLen; }
+template <class T>
+inline bool wrow_rows_end_inside_lines(int C) { return (C * (int)sizeof(T)) % 128 != 0; }
 // LAUNCH(NI, L, G) launches the kernel instance; its grid is group_grid(rows, WaveRowAt<G>::kRowsPerBlock).
 #define PLH_WROW_STEPS3(PIECE, LANES, C, A, B, D, LAUNCH)                                \
     switch (wrow_steps<T>(C, PIECE, LANES)) {                                            \
@@ -1403,6 +1426,12 @@ static int wrow_steps(int C, int piece, int lanes) {
 #define PLH_WROW_DISPATCH(PIECE, C, LAUNCH)                                              \
     do {                                                                                 \
         const int wrow_len = (PIECE);                                                    \
+        if constexpr (RowChunk<T>::kLen == 8) {                                          \
+            if (wrow_len == 8 && (C) > kWaveRowShort && (C) <= 2 * kWaveRowShort) {      \
+                LAUNCH(4, 8, 16);                                                        \
+                break;                                                                   \
+            }                                                                            \
+        }                                                                                \
         if ((C) <= kWaveRowShort) {                                                      \
             if (wrow_len == 1) {                                                         \
                 if (wrow_steps<T>(C, 1, 16) == 10) LAUNCH(10, 1, 16);                    \

@@ -594,7 +594,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
 // upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
 // the group kernel.
 
-template <class T, int NI, int LP, int Kind, bool Reduce, int G>
+template <class T, int NI, int LP, int Kind, bool Reduce, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
                                                    const int64_t *__restrict__ lab, const Upstream up,
                                                    T *__restrict__ out, float *__restrict__ loss, Partials part,
@@ -679,7 +679,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 }
                 if (e0 < p.C && live) {
                     if constexpr (Span::kUse) Span::stage(tile, p.C, at.grp, e0, o);
-                    else RowPiece<T, L>::store(out + row * p.C + e0, o);
+                    else RowPiece<T, L>::template store<Cached>(out + row * p.C + e0, o);
                 }
             }
             if constexpr (Span::kUse) {
@@ -926,6 +926,13 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
 #define PLH_GO(NI, W, G)                                                                                          \
     do {                                                                                                          \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                      \
+        if constexpr (Kind != kTaylorCeFwd && wrow_cached_form<T>(W, G)) {                                        \
+            if (wrow_rows_end_inside_lines<T>(p.C)) {                                                             \
+                hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G, true>), dim3(grid), dim3(256), 0, st, x, g, \
+                                   lab, up, out, loss, part, p);                                                  \
+                break;                                                                                            \
+            }                                                                                                     \
+        }                                                                                                         \
         hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
                            loss, part, p);                                                                        \
     } while (0)

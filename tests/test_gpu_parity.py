@@ -79,6 +79,9 @@ SEG_CASES = [
     ((21, 136), 255, 0.1),                          #   the last wavefront partly filled
     ((3, 256), 255, 0.0),
     ((5, 260), 255, 0.2),
+    ((9, 264), 255, 0.1),                           #   16-bit rows of 257..512 elements in whole chunks: 16 lanes too
+    ((6, 512), -100, 0.1),
+    ((5, 200), 255, 0.1),                           #   short rows in whole chunks that end inside a 128-byte line
     ((4, 1001), -100, 0.1),
     ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
     ((2, 2048), 255, 0.0),

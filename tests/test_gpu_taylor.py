@@ -30,6 +30,9 @@ CASES = [
     ((70, 33), 1),
     ((21, 136), 1),
     ((5, 260), 1),
+    ((9, 264), 1),                               #   16-bit rows of 257..512 elements in whole chunks: 16 lanes, 4 steps
+    ((6, 512), 1),
+    ((5, 200), 1),                               #   short rows in whole chunks that end inside a 128-byte line
     ((4, 1001), 1),
     ((5, 1544), 1),
     ((2, 2056), 1),                              # beyond the register rows: a block per row
@@ -82,7 +85,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-20:])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-23:])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
