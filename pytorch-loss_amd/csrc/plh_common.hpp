@@ -574,7 +574,6 @@ inline unsigned regs_grid(int64_t pixels) { return (unsigned)ceil_div(ceil_div(p
 //              through LDS with consecutive lanes on consecutive addresses, and every lane then picks its
 //              row out of LDS; stores go the same way back. The LDS index is skewed by one word per 32
 //              (e + e/32), which keeps the row reads of 64 lanes off a common bank for every C.
-constexpr int kRowsTileWords = 64 * kMaxRegsChannels + 64 * kMaxRegsChannels / 32 + 8;
 __device__ __forceinline__ int rows_skew(int e) { return e + (e >> 5); }
 
 typedef unsigned plh_u4 __attribute__((ext_vector_type(4)));
@@ -745,16 +744,19 @@ struct PixelRef {
         load_upstream<V>(up, pix, go);
     }
 
-    template <class T>
+    // A wavefront's tile holds 64 rows of the kernel's channel count, skewed: 5.3 KB for 20 fp32 channels rather than
+    // the 8.5 KB of 32, so that LDS does not hold the blocks per CU below what the registers allow.
+    template <class T, int CP>
     static __device__ __forceinline__ typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type *rows_tile() {
         typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
-        __shared__ __attribute__((aligned(16))) Word tile[kRegsBlock / 64][kRowsTileWords];     // rows of 8480 / 4240 bytes
+        constexpr int kChan = CP < kMaxRegsChannels ? CP : kMaxRegsChannels;
+        __shared__ __attribute__((aligned(16))) Word tile[kRegsBlock / 64][64 * kChan + 64 * kChan / 32 + 8];
         return tile[threadIdx.x >> 6];
     }
     template <class T, int CP>
     __device__ __forceinline__ void rows_load(const T *t, int C, unsigned (&raw)[CP]) const {
         typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
-        Word *tile = rows_tile<T>();
+        Word *tile = rows_tile<T, CP>();
         const int lane = threadIdx.x & 63;
         const Word *src = reinterpret_cast<const Word *>(t) + wave_first * C;
         const int n = rows_here * C;
@@ -812,7 +814,7 @@ struct PixelRef {
     template <class T, int CP>
     __device__ __forceinline__ void rows_store(T *t, int C, const unsigned (&raw)[CP]) const {
         typedef typename std::conditional<sizeof(T) == 4, unsigned, unsigned short>::type Word;
-        Word *tile = rows_tile<T>();
+        Word *tile = rows_tile<T, CP>();
         const int lane = threadIdx.x & 63;
         const bool plain = (C & 1) && rows_here == 64 && (reinterpret_cast<uintptr_t>(t) & 15) == 0;   // as in rows_load
         if (plain) {
