@@ -49,12 +49,21 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     const bool live = at.live;
     if (!Reduce && !live) return;
 
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, p.C, p.m_size, raw);
+    // labels (and the upstream gradient) before the slice, except in the one-pixel-per-lane backwards on 16-bit
+    // elements (see lsr_bwd_regs)
+    constexpr bool kLabelsFirst = !(sizeof(T) == 2 && V == 1 && WantGrad);
     int64_t lb[V];
-    at.labels(lab, p.ignore, lb);
     float go[V];
-    if constexpr (WantGrad) at.upstream(up, go);
+    typename Pack<T, V>::Raw raw[CP];
+    if constexpr (kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        if constexpr (WantGrad) at.upstream(up, go);
+    }
+    at.load_slice(x, p.C, p.m_size, raw);
+    if constexpr (!kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        if constexpr (WantGrad) at.upstream(up, go);
+    }
 
     // Four fp32 pixels per lane: a pixel's gradient takes the place of its logits in the slice as soon as it
     // is formed, and the pixels are worked through one after the other (no second array, no four

@@ -43,10 +43,11 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
 
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, p.C, p.m_size, raw);
+    // labels (and the upstream gradient) first: in the rows form the slice arrives through LDS behind a wait
     int64_t lb[V];
     at.labels(lab, p.ignore, lb);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
 
     float out[V];
     float mine = 0.f;
@@ -97,12 +98,23 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
 
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, p.C, p.m_size, raw);
+    // Labels and the upstream gradient are asked for before the slice: in the rows form the slice arrives through
+    // LDS behind a wait, and the block-uniform forms gain as well (fp32 (8,19,1024,1024) backward 0.2305 -> 0.227 ms,
+    // bf16 forward 0.0726 -> 0.0655 ms). The one-pixel-per-lane backwards on 16-bit elements keep the old order:
+    // their rows form lost 4-9 % with the new one ((4 M, 32) bf16 0.111 -> 0.121 ms).
+    constexpr bool kLabelsFirst = !(sizeof(T) == 2 && V == 1);
     int64_t lb[V];
-    at.labels(lab, p.ignore, lb);
     float go[V];
-    at.upstream(up, go);
+    typename Pack<T, V>::Raw raw[CP];
+    if constexpr (kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
+    }
+    at.load_slice(x, p.C, p.m_size, raw);
+    if constexpr (!kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
+    }
 
     // The gradient of a pixel replaces its logits in the slice as soon as they are no longer needed
     // (one pixel at a time for fp32, two for 16-bit elements, which share a dword): no second array.

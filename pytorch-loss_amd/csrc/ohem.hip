@@ -46,10 +46,11 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kRegsBlock) tables[i] = 0;
     const PixelRef<V, Form> at(P, m_size, C, xcd_run);
     if (!at.live) return;
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, C, m_size, raw);
+    // labels (and the upstream gradient) first: in the rows form the slice arrives through LDS behind a wait
     int64_t lb[V];
     at.labels(lab, ignore, lb);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, C, m_size, raw);
     float out[V], loss[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {

@@ -160,10 +160,11 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
     __shared__ float red[4];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, p.C, p.m_size, raw);
+    // labels (and the upstream gradient) first: in the rows form the slice arrives through LDS behind a wait
     int64_t lb[V];
     at.labels(lab, p.ignore, lb);
+    typename Pack<T, V>::Raw raw[CP];
+    at.load_slice(x, p.C, p.m_size, raw);
     float out[V];
     float mine = 0.f;
     int cnt = 0;
@@ -202,12 +203,21 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
                                                                 const TaylorParams p) {
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
-    typename Pack<T, V>::Raw raw[CP];
-    at.load_slice(x, p.C, p.m_size, raw);
+    // labels and the upstream gradient before the slice, except in the one-pixel-per-lane form on 16-bit elements
+    // (see lsr_bwd_regs)
+    constexpr bool kLabelsFirst = !(sizeof(T) == 2 && V == 1);
     int64_t lb[V];
-    at.labels(lab, p.ignore, lb);
     float go[V];
-    at.upstream(up, go);
+    typename Pack<T, V>::Raw raw[CP];
+    if constexpr (kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
+    }
+    at.load_slice(x, p.C, p.m_size, raw);
+    if constexpr (!kLabelsFirst) {
+        at.labels(lab, p.ignore, lb);
+        at.upstream(up, go);
+    }
     // first per pixel (sum of the series, the target's term), then channel by channel so that only one
     // packed result is live at a time
     unsigned keep[V];
