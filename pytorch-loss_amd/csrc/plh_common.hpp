@@ -1382,8 +1382,9 @@ struct WaveRowSpan {
 // longer ones a whole wavefront. The piece is the largest of 16, 8, 4, 2 bytes that divides the row's bytes
 // and that every tensor involved is aligned to. Instantiated steps -- 16 lanes: 4, 8, 16 single elements,
 // 2, 4, 8 pieces of two, 2, 4 of four, 2 of eight; 64 lanes: 8, 16, 32 single elements, 4, 8, 16 pieces of
-// two, 2, 4, 8 of four or eight. 16-bit rows of 257..512 elements in 16-byte pieces also get 16 lanes (4 steps: the
-// same KiB per row as 256 fp32 elements; a whole wavefront for 528 bytes left the bf16 LSR backward at 39 % of peak).
+// two, 2, 4, 8 of four or eight. Rows of 257..512 elements in 16-byte pieces also get 16 lanes (4 steps of eight
+// 16-bit elements, 8 steps of four fp32 ones; a whole wavefront for 528 bytes left the bf16 LSR backward at 39 % of
+// peak).
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
 // 16-bit rows that move in 16-byte pieces go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the
@@ -1428,11 +1429,10 @@ inline bool wrow_rows_end_inside_lines(int C) { return (C * (int)sizeof(T)) % 12
 #define PLH_WROW_DISPATCH(PIECE, C, LAUNCH)                                              \
     do {                                                                                 \
         const int wrow_len = (PIECE);                                                    \
-        if constexpr (RowChunk<T>::kLen == 8) {                                          \
-            if (wrow_len == 8 && (C) > kWaveRowShort && (C) <= 2 * kWaveRowShort) {      \
-                LAUNCH(4, 8, 16);                                                        \
-                break;                                                                   \
-            }                                                                            \
+        if (wrow_len == RowChunk<T>::kLen && (C) > kWaveRowShort && (C) <= 2 * kWaveRowShort) { \
+            if constexpr (RowChunk<T>::kLen == 8) LAUNCH(4, 8, 16);                      \
+            else LAUNCH(8, 4, 16);                                                       \
+            break;                                                                       \
         }                                                                                \
         if ((C) <= kWaveRowShort) {                                                      \
             if (wrow_len == 1) {                                                         \
