@@ -494,7 +494,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                                                const LmParams p) {
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
-    using Span = WaveRowSpan<T, L, G>;
+    using Span = WaveRowSpan<T, L, G, NI>;
     T *tile = Span::tile();
     const WaveRowAt<G> at;
     const int lane = at.sub;
@@ -895,7 +895,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
         hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G>), dim3(blocks), dim3(256), 0, \
                            st, x, lab, up, loss, grad, cnt, part, p);                                              \
     } while (0)
-                PLH_WROW_DISPATCH(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C), p.C, PLH_GO);
+                PLH_WROW_DISPATCH_IF(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C), p.C, PLH_GO, (WantGrad ? 1 : 2));
 #undef PLH_GO
                 break;
             }

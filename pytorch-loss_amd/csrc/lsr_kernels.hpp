@@ -491,7 +491,7 @@ template <class T, int NI, int LP, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, T *__restrict__ grad, const LsrParams p) {
     constexpr int L = WaveRow<T, NI, LP, G>::L;
-    using Span = WaveRowSpan<T, L, G>;
+    using Span = WaveRowSpan<T, L, G, NI>;
     T *tile = Span::tile();
     const WaveRowAt<G> at;
     for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
@@ -995,7 +995,7 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         hipLaunchKernelGGL((lsr_bwd_wrow<T, NI, W, G>), dim3(group_grid(p.P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
                            st, logits, labels, up, grad_logits, p);                                                \
     } while (0)
-                PLH_WROW_DISPATCH(wrow_piece<T>(logits, grad_logits, p.C), p.C, PLH_GO);
+                PLH_WROW_DISPATCH_IF(wrow_piece<T>(logits, grad_logits, p.C), p.C, PLH_GO, 1);
 #undef PLH_GO
             }
             break;

@@ -1337,13 +1337,13 @@ struct WaveRowAt {
 // step's stores are four separate segments of 32..128 bytes; the four rows of a round are contiguous in memory, so
 // they are gathered in LDS (as stored: T) and leave as 16-byte pieces of one run of 4*C elements, whose lines are
 // whole except the run's first and last.
-constexpr int kWaveRowShortElems = 256;       // = kWaveRowShort below: the longest row that 16 lanes share
-template <class T, int L, int G>
+template <class T, int L, int G, int NI>
 struct WaveRowSpan {
     static constexpr bool kUse = (G == 16 && L < RowChunk<T>::kLen);
     static constexpr int kRows = 64 / G;
+    static constexpr int kRowSlots = G * NI * L;         // the longest row this instance holds (a multiple of 16 elements)
     static __device__ __forceinline__ T *tile() {
-        __shared__ __attribute__((aligned(16))) T buf[4][kUse ? kRows * kWaveRowShortElems : 8];
+        __shared__ __attribute__((aligned(16))) T buf[4][kUse ? kRows * kRowSlots : 8];
         return buf[threadIdx.x >> 6];
     }
     // the piece of step i of lane (grp, sub) into the tile
@@ -1382,9 +1382,9 @@ struct WaveRowSpan {
 // longer ones a whole wavefront. The piece is the largest of 16, 8, 4, 2 bytes that divides the row's bytes
 // and that every tensor involved is aligned to. Instantiated steps -- 16 lanes: 4, 8, 16 single elements,
 // 2, 4, 8 pieces of two, 2, 4 of four, 2 of eight; 64 lanes: 8, 16, 32 single elements, 4, 8, 16 pieces of
-// two, 2, 4, 8 of four or eight. Rows of 257..512 elements in 16-byte pieces also get 16 lanes (4 steps of eight
-// 16-bit elements, 8 steps of four fp32 ones; a whole wavefront for 528 bytes left the bf16 LSR backward at 39 % of
-// peak).
+// two, 2, 4, 8 of four or eight. Rows of 257..512 elements also get 16 lanes (32 slots per lane: 4 steps of eight,
+// 8 of four, 16 of two or 32 single elements; a whole wavefront per row takes a power-of-two number of steps, and for
+// 528 bytes it left the bf16 LSR backward at 39 % of peak).
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
 // 16-bit rows that move in 16-byte pieces go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the
@@ -1426,13 +1426,38 @@ inline bool wrow_rows_end_inside_lines(int C) { return (C * (int)sizeof(T)) % 12
         case B: LAUNCH(B, PIECE, LANES); break;                                          \
         default: LAUNCH(D, PIECE, LANES); break;                                         \
     }
-#define PLH_WROW_DISPATCH(PIECE, C, LAUNCH)                                              \
+// WIDE_SHORT (a constant expression): which rows of 257..512 elements in pieces shorter than 16 bytes take the 16-lane
+// form too -- 2: all (the forwards), 1: not those of single elements (kernels that write a row: 32 staged steps per
+// lane lose to the wavefront per row, bf16 (512 K, 301) large-margin backward 0.255 -> 0.363 ms), 0: none (the Taylor
+// backwards: bf16 (512 K, 300) cross-entropy backward 0.255 -> 0.293 ms with it).
+#define PLH_WROW_DISPATCH(PIECE, C, LAUNCH) PLH_WROW_DISPATCH_IF(PIECE, C, LAUNCH, 2)
+#define PLH_WROW_DISPATCH_IF(PIECE, C, LAUNCH, WIDE_SHORT)                               \
     do {                                                                                 \
         const int wrow_len = (PIECE);                                                    \
-        if (wrow_len == RowChunk<T>::kLen && (C) > kWaveRowShort && (C) <= 2 * kWaveRowShort) { \
-            if constexpr (RowChunk<T>::kLen == 8) LAUNCH(4, 8, 16);                      \
-            else LAUNCH(8, 4, 16);                                                       \
-            break;                                                                       \
+        if ((C) > kWaveRowShort && (C) <= 2 * kWaveRowShort) {                           \
+            if (wrow_len == RowChunk<T>::kLen) {                                         \
+                if constexpr (RowChunk<T>::kLen == 8) LAUNCH(4, 8, 16);                  \
+                else LAUNCH(8, 4, 16);                                                   \
+                break;                                                                   \
+            }                                                                            \
+            if constexpr ((WIDE_SHORT) == 2) {                                           \
+                if (wrow_len == 1) {                                                     \
+                    LAUNCH(32, 1, 16);                                                   \
+                    break;                                                               \
+                }                                                                        \
+            }                                                                            \
+            if constexpr ((WIDE_SHORT) >= 1) {                                           \
+                if (wrow_len == 2) {                                                     \
+                    LAUNCH(16, 2, 16);                                                   \
+                    break;                                                               \
+                }                                                                        \
+                if constexpr (RowChunk<T>::kLen == 8) {                                  \
+                    if (wrow_len == 4) {                                                 \
+                        LAUNCH(8, 4, 16);                                                \
+                        break;                                                           \
+                    }                                                                    \
+                }                                                                        \
+            }                                                                            \
         }                                                                                \
         if ((C) <= kWaveRowShort) {                                                      \
             if (wrow_len == 1) {                                                         \

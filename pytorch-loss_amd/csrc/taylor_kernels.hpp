@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                                                    const TaylorParams p) {
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
-    using Span = WaveRowSpan<T, L, G>;
+    using Span = WaveRowSpan<T, L, G, NI>;
     T *tile = Span::tile();
     const WaveRowAt<G> at;
     const int lane = at.sub;
@@ -946,7 +946,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
                            loss, part, p);                                                                        \
     } while (0)
-            PLH_WROW_DISPATCH(piece, p.C, PLH_GO);
+            PLH_WROW_DISPATCH_IF(piece, p.C, PLH_GO, (kForward ? 2 : 0));
 #undef PLH_GO
             return grid;
         }

@@ -39,7 +39,8 @@ SCORE_CASES = [
     ((70, 33), -100, 0.1),
     ((21, 136), 255, 0.1),
     ((5, 260), 255, 0.2),
-    ((9, 264), 255, 0.1),                  # 16-bit rows of 257..512 elements in whole chunks: 16 lanes per row
+    ((9, 264), 255, 0.1),                  # rows of 257..512 elements: 16 lanes per row
+    ((7, 301), 255, 0.1),
     ((4, 1001), -100, 0.1),
     ((5, 1544), 255, 0.1),
     ((3, 2047), 255, 0.1),

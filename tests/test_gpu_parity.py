@@ -82,6 +82,9 @@ SEG_CASES = [
     ((9, 264), 255, 0.1),                           #   16-bit rows of 257..512 elements in whole chunks: 16 lanes too
     ((6, 512), -100, 0.1),
     ((5, 200), 255, 0.1),                           #   short rows in whole chunks that end inside a 128-byte line
+    ((7, 301), 255, 0.1),                           #   257..512 elements in short pieces: 16 lanes, 32 single elements,
+    ((5, 258), -100, 0.1),                          #   16 pieces of two, 8 of four (16-bit 300 and 500)
+    ((4, 500), 255, 0.1),
     ((4, 1001), -100, 0.1),
     ((3, 2047), 255, 0.1),                          #   16-byte chunks otherwise
     ((2, 2048), 255, 0.0),

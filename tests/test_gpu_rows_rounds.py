@@ -30,7 +30,7 @@ def _slices(rows):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("classes", [150, 151, 130, 34, 200, 256, 264, 512, 1000, 1001])
+@pytest.mark.parametrize("classes", [150, 151, 130, 34, 200, 256, 264, 300, 301, 512, 1000, 1001])
 @pytest.mark.parametrize("loss", ["lsr", "lmargin", "taylor"])
 def test_many_short_rows_equal_their_slices(pl, loss, classes, dtype):
     gen = torch.Generator(device="cuda")

@@ -33,6 +33,8 @@ CASES = [
     ((9, 264), 1),                               #   16-bit rows of 257..512 elements in whole chunks: 16 lanes, 4 steps
     ((6, 512), 1),
     ((5, 200), 1),                               #   short rows in whole chunks that end inside a 128-byte line
+    ((7, 301), 1),                               #   257..512 elements in short pieces: 16 lanes, 32 single elements
+    ((5, 258), 1),                               #   ... 16 pieces of two
     ((4, 1001), 1),
     ((5, 1544), 1),
     ((2, 2056), 1),                              # beyond the register rows: a block per row
@@ -85,7 +87,7 @@ def test_function_matches_oracle(pl, shape, dim, order, use_log):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-23:])
+@pytest.mark.parametrize("shape,dim", CASES[:7] + CASES[-25:])
 def test_function_16bit(pl, shape, dim, dt):
     x = synth.normal(102, 1, shape, 0.0, 1.0)
     g = synth.normal(102, 2, shape, 0.0, 1.0)
