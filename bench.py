@@ -453,12 +453,20 @@ def copy_ceiling(device, nbytes=1 << 30):
     return round(2 * nbytes / (ms * 1e-3) / 1e9, 1)
 
 
-def cpu_baseline(name, shape):
+def cpu_threads():
+    """Host threads of the CPU leg. A one-GPU box hands a job 16 host threads whatever os.cpu_count() shows
+    (OMP_NUM_THREADS=16 is exported there), so that is the count used and stated; without the variable, every core
+    up to 16."""
+    return int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+
+
+def cpu_baseline(name, shape, spot_check=True):
     """Pure-torch restatement of the reference's V2 (V1 for Lovasz) path on the host cores, on a
-    bounded sample: one image of the batch, scaled to the whole batch."""
+    bounded sample: one image of the batch, scaled to the whole batch (Lovasz: the whole batch, once warm and
+    twice timed, since its per-class sort runs over all images together)."""
     import torch
     from oracle import synth, torch_ref
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    cores = cpu_threads()
     torch.set_num_threads(cores)
     if name == "layernorm":
         g = torch.Generator().manual_seed(15)
@@ -471,7 +479,8 @@ def cpu_baseline(name, shape):
         labels = (torch.rand(logits.shape, generator=g) < 0.3).float()
         return _time_cpu(name, shape, cores, lambda: torch_ref.soft_dice(logits, labels, 1, 1.0), logits)
     cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2", "taylor": "cfg2"}[name]
-    w = synth.workload(cfg, batch=1)
+    whole = name == "lovasz"
+    w = synth.workload(cfg) if whole else synth.workload(cfg, batch=1)
     logits = torch.from_numpy(w["logits"]).requires_grad_()
     labels = torch.from_numpy(w["labels"])
     fn = {"lsr": lambda: torch_ref.lsr(logits, labels, 0.1, "mean", 255),
@@ -480,35 +489,38 @@ def cpu_baseline(name, shape):
           "lovasz": lambda: torch_ref.lovasz(logits, labels, "mean", 255),
           "ohem": lambda: torch_ref.ohem_ce(logits, labels, 0.7, None, 255),
           "taylor": lambda: torch_ref.taylor_ce(logits, labels, 4, "mean", 255)}[name]
-    res = _time_cpu(name, shape, cores, fn, logits)
-    # the same image through the HIP module: the two losses are printed side by side
+    res = _time_cpu(name, shape, cores, fn, logits, whole=whole)
+    if not spot_check:
+        return res
+    # the same input through the HIP module: the two losses are printed side by side
     try:
         with torch.no_grad():
             want = float(fn().item())
         got = float(make_criterion(name)(logits.detach().to("cuda:0"), labels.to("cuda:0")).item())
-        res["parity_spot_check"] = {"what": "loss of image 0 of the workload: HIP module on cuda:0 against the CPU restatement",
+        res["parity_spot_check"] = {"what": "loss of the CPU leg's input: HIP module on cuda:0 against the CPU restatement",
                                     "hip": got, "cpu": want, "rel_err": abs(got - want) / max(abs(want), 1e-30)}
     except Exception as e:
         res["parity_spot_check"] = {"error": "%s: %s" % (type(e).__name__, e)}
     return res
 
 
-def _time_cpu(name, shape, cores, fn, logits):
+def _time_cpu(name, shape, cores, fn, logits, whole=False):
     times = []
-    for i in range(4):
+    for i in range(3 if whole else 4):
         logits.grad = None
         t0 = time.perf_counter()
         fn().backward()
         t1 = time.perf_counter()
         if i:
             times.append((t1 - t0) * 1e3)
-    scale = shape[0]
+    scale = 1 if whole else shape[0]
     ms_full = statistics.median(times) * scale
     fwd, bwd = algorithmic_bytes(name, shape)
+    sample = ("the whole batch, fwd+bwd, median of %d" % len(times)) if whole else (
+        "1 of %d images of the workload, fwd+bwd, median of %d, time scaled x%d" % (scale, len(times), scale))
     return {"value": round((fwd + bwd) / (ms_full * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "ms_per_step": round(ms_full, 2),
-            "sample": "oracle/torch_ref.py (pure-torch restatement of the reference's V2/V1 CPU path) on 1 of %d "
-                      "images of the workload, fwd+bwd, median of 3, time scaled x%d" % (scale, scale)}
+            "ms_per_step": round(ms_full, 2), "os_cpu_count": os.cpu_count(),
+            "sample": "oracle/torch_ref.py (pure-torch restatement of the reference's V2/V1 CPU path) on " + sample}
 
 
 def run_onehot(steps, warmup, device):
@@ -616,6 +628,41 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
     return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist, function_level=func)
 
 
+TARGETS = ("lsr", "lmargin", "focal", "focal_seg", "lovasz")
+
+
+def targets_block(headline, main_res, others, headline_cpu, with_cpu):
+    """LSR, large margin, focal (at its own shape and at the segmentation shape) and Lovasz in one short object:
+    eager module step (ms), the same step replayed from a HIP graph (graph_ms), the bytes the step has to move and the
+    fraction of the 8 TB/s peak that makes (frac), forward / backward entry points alone (fwd_ms, bwd_ms), and the CPU
+    restatement of the reference's V2 (Lovasz: V1) path on the host threads (cpu: ms per step, GB/s of the
+    Function-level bytes, threads, relative difference of its loss from the HIP module's on the same input)."""
+    out = {"unit": "ms", "peak_GBps": HBM_PEAK_GBPS}
+    for t in TARGETS:
+        if t == headline:
+            ms, nbytes, step_ms, kern = main_res["ms_per_step"], main_res["bytes"], main_res["step_ms"], main_res["roofline"]
+        else:
+            o = others.get(t)
+            if not o or "error" in o:
+                out[t] = {"error": (o or {}).get("error", "not run")}
+                continue
+            ms, nbytes, step_ms, kern = o["ms_per_step"], o["algorithmic_bytes_per_step"], o["step_ms"], o["kernels"]
+        e = {"ms": round(ms, 4), "graph_ms": (step_ms.get("graph") or {}).get("ms"), "bytes": nbytes,
+             "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+             "fwd_ms": (kern.get("forward") or {}).get("ms"), "bwd_ms": (kern.get("backward") or {}).get("ms")}
+        if with_cpu and "base" not in WORKLOADS[t]:
+            try:
+                c = headline_cpu if (t == headline and headline_cpu and "error" not in headline_cpu) else \
+                    cpu_baseline(t, WORKLOADS[t]["shape"])
+                rel = c.get("parity_spot_check", {}).get("rel_err")
+                e["cpu"] = {"ms": c["ms_per_step"], "GB/s": c["value"], "threads": c["cores"],
+                            "rel_err": None if rel is None else float("%.2g" % rel)}
+            except Exception as ex:
+                e["cpu"] = {"error": "%s: %s" % (type(ex).__name__, ex)}
+        out[t] = e
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -699,6 +746,9 @@ def main():
             line["cpu_baseline"] = cpu_baseline(name, WORKLOADS[name]["shape"])
         except Exception as e:
             line["cpu_baseline"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    # Last key of the line, and short: the configurations the metric names, side by side. A record that keeps
+    # only the end of a long line still holds all of them.
+    line["targets"] = targets_block(name, main_res, others, line.get("cpu_baseline"), not args.no_cpu_baseline)
     print(json.dumps(line), flush=True)
 
 

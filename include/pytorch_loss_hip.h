@@ -12,8 +12,8 @@
  *     same way, csrc/lsr_kernel.cu:199-202); integer labels are int64 (n_size, m_size);
  *   - `stream` is a hipStream_t (NULL = the default stream); launches are
  *     asynchronous and the library never synchronises, allocates or frees
- *     device memory, and keeps no state between calls (re-entrant; the one exception,
- *     plh_lsr_forward_reduced_static, says so);
+ *     device memory, reads no environment variable and keeps no state between calls
+ *     (re-entrant; the one exception, plh_lsr_forward_reduced_static, says so);
  *   - the caller sets the current device to the one that owns the pointers;
  *   - return value: PLH_OK (0), a negative PLH_ERR_* for rejected arguments
  *     (nothing was launched), or a positive hipError_t from the launch;
@@ -107,7 +107,8 @@ int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *la
  * counterpart in the reference. Same arguments and results as plh_lsr_forward_reduced, without the
  * workspace: the per-block partials live in a 2 MiB device array that is part of the library's
  * code object (each GPU that the library runs on holds its own copy until the process ends); its
- * address is looked up on the first call on each device. The call allocates and frees nothing.
+ * address is looked up on the first call on each device (hipGetSymbolAddress, under a mutex: make that
+ * first call outside a stream capture). The call allocates and frees nothing.
  * Limit: n_size * m_size <= 2^24 pixels, else PLH_ERR_BAD_SIZE. All calls on one GPU share the one
  * array: calls that overlap on one GPU (different streams or threads) race; calls on one stream
  * are ordered and need no clearing in between.
@@ -193,8 +194,6 @@ int plh_lmargin_forward_backward(const void *logits, int32_t dtype, const int64_
  * workspace: scratch device memory of at least plh_lovasz_workspace_bytes() bytes,
  *         256-byte aligned, owned by the caller; contents are undefined afterwards.
  * Limits: dimsize < 512 and n_size*dimsize*m_size < 2^31 (csrc/lovasz_softmax.cu:664-665).
- * With PLH_LOVASZ_SCAN=lookback in the environment (read by both functions at every call) the sort passes run
- * their decoupled look-back variant, which needs a larger workspace; results are identical, the default is faster.
  */
 int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size);
 
@@ -203,6 +202,19 @@ int plh_lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels,
                        void *workspace, int64_t workspace_bytes,
                        int64_t n_size, int64_t dimsize, int64_t m_size,
                        int64_t ignore_index, void *stream);
+
+/* The same forward with the sort passes in their decoupled look-back form (tile descriptors and chained waits instead
+ * of a histogram kernel and a row scan in front of every pass; no counterpart in the reference, whose scan is
+ * csrc/cumsum.hpp:82-108). Results are those of plh_lovasz_forward bit for bit; it needs the larger workspace that
+ * plh_lovasz_lookback_workspace_bytes() names, n_size*m_size < 2^30, and is the slower of the two on MI355X: it is
+ * kept to be measured against the default. */
+int64_t plh_lovasz_lookback_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size);
+
+int plh_lovasz_forward_lookback(const void *logits, int32_t dtype, const int64_t *labels,
+                                float *losses, float *jacc,
+                                void *workspace, int64_t workspace_bytes,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t ignore_index, void *stream);
 
 int plh_lovasz_backward(const float *grad_output, const void *logits, int32_t dtype, const int64_t *labels,
                         const float *jacc, void *grad_logits,

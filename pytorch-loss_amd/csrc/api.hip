@@ -1,7 +1,5 @@
 // Library-level entry points: ABI version, error text, and the plain copy kernel
 // used to calibrate byte counters and to measure achievable copy bandwidth.
-#include <stdlib.h>
-
 #include "plh_common.hpp"
 
 namespace plh {
@@ -24,13 +22,7 @@ __global__ __launch_bounds__(256) void stream_copy_scalar(const float *__restric
 // 64..288 lose 3..20 % on several shapes. The one systematic exception: fp32 logits whose channel
 // plane is a multiple of 4 MiB (1024x1024, 2048x1024) run 3 % faster with runs of 1024 tiles, which
 // costs 16-bit logits of the same shapes up to 13 %, hence the element-size condition.
-// PLH_XCD_RUN=<tiles> in the environment overrides the choice (read once; a tuning aid).
 unsigned xcd_run_for(size_t elem_bytes, int64_t m_size) {
-    static const long forced = [] {
-        const char *e = getenv("PLH_XCD_RUN");
-        return e ? strtol(e, nullptr, 10) : 0L;
-    }();
-    if (forced > 0) return (unsigned)forced;
     if (elem_bytes == 4 && m_size > 0 && (m_size * 4) % ((int64_t)4 << 20) == 0) return 1024u;
     return 32u;
 }

@@ -530,6 +530,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         // than the target, sum (q - coeff) (d - lse_no) = (sum e d) / s_no - lse_no - coeff (sum d - n lse_no).
         constexpr bool kClosed = WantLoss && !WantGrad;
         float s_no = 0.f, sum_ex = 0.f, sum_d = 0.f;
+        int finite_slots = 0;                   // wave-uniform: slots of the wavefront's rows that hold a finite logit
 #pragma unroll
         for (int i = 0; i < NI; ++i)
 #pragma unroll
@@ -543,6 +544,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                     const float dz = in ? d : 0.f;
                     sum_ex = __builtin_fmaf(e, dz, sum_ex);
                     sum_d += dz;
+                    finite_slots += __builtin_popcountll(__builtin_amdgcn_ballot_w64(in));   // scalar unit: the vote exists already
                 } else {
                     sum_ex = __builtin_fmaf(e, in ? t : 0.f, sum_ex);
                 }
@@ -558,12 +560,21 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
         const float lse_no = logf(s_no);
         const float g_hot = (e_y * inv_all - 1.f) * go[0];
         float acc = 0.f;
+        // The closed form counts every channel other than the target as a finite term. A row with a logit of -inf
+        // among them (a masked class) has a term (0 - coeff) * log 0 instead, which the sweep below evaluates as
+        // the kernels with gradients do; whether any row of this wavefront has one shows in the number of finite
+        // slots, which the votes above counted on the scalar unit.
+        bool closed = kClosed;
         if constexpr (kClosed) {
+            const int with_target = __builtin_popcountll(__builtin_amdgcn_ballot_w64(tgt >= 0)) / G;
+            closed = finite_slots == (kWave / G) * p.C - with_target;      // wave-uniform
             const float n_no = (float)(p.C - (tgt >= 0 ? 1 : 0));
             acc = p.half_lam * (sum_ex * inv_no - lse_no - p.coeff * (sum_d - n_no * lse_no));
+            if (!closed) acc = 0.f;
         }
+        if (!closed) {
 #pragma unroll
-        for (int i = 0; i < (kClosed ? 0 : NI); ++i) {
+        for (int i = 0; i < NI; ++i) {
             const int e0 = (lane + G * i) * L;
             const bool ok = e0 < p.C;
             float g[L];
@@ -587,12 +598,13 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                 }
             }
         }
+        }
         if constexpr (WantGrad && Span::kUse) {
             const int64_t left = p.P - r0;
             Span::flush(tile, grad + r0 * p.C, left < Span::kRows ? (int)left : Span::kRows, p.C);
         }
         if constexpr (WantLoss) {
-            if constexpr (!kClosed) acc = group_reduce<G>(acc, OpSum());
+            if (!closed) acc = group_reduce<G>(acc, OpSum());
             acc += -(x_y - m_all) + logf(s_all);
             if (lane == 0 && live) {
                 if (loss) loss[row] = ign ? 0.f : acc;
@@ -645,7 +657,10 @@ __device__ __forceinline__ void lm_row_absorb(const float (&v)[L], int idx0, int
         const bool hot = (idx0 + i == tgt);
         const float e = hot ? 0.f : fast_exp(v[i] - st.m);
         st.s += e;
-        st.ex += hot ? 0.f : e * v[i];
+        // e is 0 for the target and for a masked (-inf) logit: clamping the logit keeps 0 * -inf out of the sum,
+        // while the plain sum below still turns -inf, so that a masked class gives the (0 - coeff) * log 0 = +inf
+        // of the per-element form
+        st.ex = __builtin_fmaf(e, fmaxf(v[i], -3.0e38f), st.ex);
         st.sx += hot ? 0.f : v[i];
     }
 }

@@ -32,9 +32,6 @@
 // A 4096-key tile is handled by 512 threads with 8 keys each; neighbouring tiles of a class row run
 // on the same XCD (sort_tile) so that the sectors they share merge in one L2.
 // Equal errors keep pixel order (the sort is stable); the reference leaves tie order open.
-#include <cstdlib>
-#include <cstring>
-
 #include "plh_common.hpp"
 
 namespace plh {
@@ -550,7 +547,7 @@ __global__ __launch_bounds__(256) void lov_row_scan(uint32_t *table0, uint32_t *
     if (threadIdx.x == 0) totals[rid] = carry;
 }
 
-// ---- the decoupled look-back variant of the passes (opt-in: PLH_LOVASZ_SCAN=lookback) -------------------
+// ---- the decoupled look-back variant of the passes (plh_lovasz_forward_lookback) ------------------------
 // Instead of a histogram kernel and a row scan in front of every pass, a tile learns how many keys of each digit
 // the tiles before it hold by walking back over their descriptors: every tile publishes, per digit, first its own
 // count ("aggregate") and, once it knows the sum over all its predecessors, the inclusive sum ("prefix"); a walk
@@ -1154,15 +1151,9 @@ struct LovaszPlan {
     int64_t off_lb_clear, lb_clear_bytes, off_lb_totals, off_lb_partial;
 };
 
-// PLH_LOVASZ_SCAN=lookback selects the decoupled look-back variant of the sort passes (read at every call).
-static bool look_back_selected() {
-    const char *v = getenv("PLH_LOVASZ_SCAN");
-    return v && strcmp(v, "lookback") == 0;
-}
-
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
-static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan &pl) {
+static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan &pl, bool look_back = false) {
     if (n_size < 0 || dimsize < 0 || m_size < 0) return PLH_ERR_BAD_SIZE;
     if (dimsize >= 512) return PLH_ERR_TOO_MANY_CLASSES;
     const double numel = (double)n_size * (double)dimsize * (double)m_size;
@@ -1189,7 +1180,9 @@ static int make_plan(int64_t n_size, int64_t dimsize, int64_t m_size, LovaszPlan
     pl.off_cursors = off;     off += round_up(4 * dimsize * kMaxRegions, 256);
     pl.off_class = off;       off += round_up(4 * dimsize * 4, 256);      // pos_max[C], kept[C], all_min[C], key_bits[C]
     pl.off_block_max = off;   off += round_up(4 * dimsize * ceil_div(pl.P, 256), 256);   // [key blocks][C]
-    pl.look_back = look_back_selected() && pl.regions > 0;
+    // the look-back descriptors carry a count in 30 bits next to their 2 state bits
+    if (look_back && pl.P >= ((int64_t)1 << 30)) return PLH_ERR_BAD_SIZE;
+    pl.look_back = look_back && pl.regions > 0;
     pl.hist_blocks = (int)ceil_div(pl.tiles, 2);
     if (pl.look_back) {
         // [4 passes][C] tickets + 1 word, 3 x [C][tiles][kRadix] u32 descriptors, [C][tiles][kRadix] u64 ones
@@ -1212,13 +1205,18 @@ extern "C" int64_t plh_lovasz_workspace_bytes(int64_t n_size, int64_t dimsize, i
     return rc == PLH_OK ? pl.bytes : (int64_t)rc;
 }
 
-extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *jacc,
-                                  void *workspace, int64_t workspace_bytes,
-                                  int64_t n_size, int64_t dimsize, int64_t m_size,
-                                  int64_t ignore_index, void *stream) {
+extern "C" int64_t plh_lovasz_lookback_workspace_bytes(int64_t n_size, int64_t dimsize, int64_t m_size) {
+    LovaszPlan pl;
+    const int rc = make_plan(n_size, dimsize, m_size, pl, true);
+    return rc == PLH_OK ? pl.bytes : (int64_t)rc;
+}
+
+static int lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *jacc,
+                          void *workspace, int64_t workspace_bytes, int64_t n_size, int64_t dimsize, int64_t m_size,
+                          int64_t ignore_index, void *stream, bool look_back) {
     if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     LovaszPlan pl;
-    int rc = make_plan(n_size, dimsize, m_size, pl);
+    int rc = make_plan(n_size, dimsize, m_size, pl, look_back);
     if (rc != PLH_OK) return rc;
     if (pl.E == 0) return PLH_OK;
     if (!logits || !labels || !losses || !jacc) return PLH_ERR_NULL_POINTER;
@@ -1394,6 +1392,22 @@ extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64
         hipLaunchKernelGGL(lov_reduce_loss, dim3((unsigned)C), dim3(256), 0, st, tile_loss, losses, pl.tiles);
     }
     return check_launch();
+}
+
+extern "C" int plh_lovasz_forward(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *jacc,
+                                  void *workspace, int64_t workspace_bytes,
+                                  int64_t n_size, int64_t dimsize, int64_t m_size,
+                                  int64_t ignore_index, void *stream) {
+    return lovasz_forward(logits, dtype, labels, losses, jacc, workspace, workspace_bytes, n_size, dimsize, m_size,
+                          ignore_index, stream, false);
+}
+
+extern "C" int plh_lovasz_forward_lookback(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                                           float *jacc, void *workspace, int64_t workspace_bytes,
+                                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                                           int64_t ignore_index, void *stream) {
+    return lovasz_forward(logits, dtype, labels, losses, jacc, workspace, workspace_bytes, n_size, dimsize, m_size,
+                          ignore_index, stream, true);
 }
 
 extern "C" int plh_lovasz_backward(const float *grad_output, const void *logits, int32_t dtype, const int64_t *labels,

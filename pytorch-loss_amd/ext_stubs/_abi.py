@@ -56,3 +56,15 @@ def gpu_only(what, *tensors):
     for t in tensors:
         if not t.is_cuda:
             raise RuntimeError("this %s only supports gpu mode" % what)
+
+
+def labels(t, logits):
+    """The int64 labels of `logits` as the C ABI reads them: the reference takes them through
+    `labels.contiguous().data_ptr<int64_t>()` (e.g. csrc/lsr_kernel.cu:224), which raises for any other dtype;
+    a label tensor that is not (N, *) of the logits' (N, C, *) would be read out of bounds, so it raises too."""
+    if t.dtype != torch.int64:
+        raise RuntimeError("expected scalar type Long for the labels but found %s" % t.dtype)
+    n, _, m = dims(logits)
+    if t.numel() != n * m:
+        raise RuntimeError("labels of shape %s do not go with logits of shape %s" % (tuple(t.shape), tuple(logits.shape)))
+    return t.contiguous()

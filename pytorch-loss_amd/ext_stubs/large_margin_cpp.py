@@ -3,6 +3,7 @@ Python-side argument order (lam, ignore_index), as the reference's interface fun
 import torch
 
 from ._abi import F32, I32, I64, P, bind, check, dims, gpu_only, native, stream
+from ._abi import labels as int64_labels
 
 _fwd = bind("plh_lmargin_forward", [P, I32, P, P, I64, I64, I64, I64, F32, P])
 _bwd = bind("plh_lmargin_backward", [P, I32, P, P, I64, P, I64, I64, I64, I64, F32, P])
@@ -11,7 +12,7 @@ _fb = bind("plh_lmargin_forward_backward", [P, I32, P, P, P, P, I64, I64, I64, I
 
 def l_margin_forward(logits, labels, lam, ignore_index):
     gpu_only("large margin loss", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
     if x.numel():
         with torch.cuda.device_of(x):
@@ -21,7 +22,7 @@ def l_margin_forward(logits, labels, lam, ignore_index):
 
 def l_margin_backward(logits, labels, lam, ignore_index):
     gpu_only("large margin loss", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     grad = torch.empty_like(x)
     if x.numel():
         with torch.cuda.device_of(x):
@@ -32,7 +33,7 @@ def l_margin_backward(logits, labels, lam, ignore_index):
 def l_margin_forward_backward(logits, labels, lam, ignore_index):
     """-> (losses, dloss/dlogits, valid_cnt int64[1]), csrc/large_margin_kernel.cu:820-831."""
     gpu_only("large margin loss", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)
     grad = torch.empty_like(x)
     cnt = torch.zeros(1, dtype=torch.int64, device=x.device)

@@ -6,6 +6,7 @@ the caller for: plh_lovasz_workspace_bytes() bytes, allocated here through torch
 import torch
 
 from ._abi import I32, I64, P, bind, check, dims, gpu_only, native, stream
+from ._abi import labels as int64_labels
 
 _ws_bytes = bind("plh_lovasz_workspace_bytes", [I64, I64, I64], I64)
 _fwd = bind("plh_lovasz_forward", [P, I32, P, P, P, P, I64, I64, I64, I64, I64, P])
@@ -15,7 +16,7 @@ _bwd = bind("plh_lovasz_backward", [P, P, I32, P, P, P, I64, I64, I64, I64, P])
 def lovasz_softmax_forward(logits, labels, ignore_index):
     """-> (losses [C], jacc [C, P]), csrc/lovasz_softmax.cu:778-786."""
     gpu_only("lovasz softmax function", logits)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     n, c, m = dims(x)
     losses = torch.zeros(c, dtype=torch.float32, device=x.device)
     jacc = torch.zeros((c, n * m), dtype=torch.float32, device=x.device)
@@ -33,7 +34,7 @@ def lovasz_softmax_forward(logits, labels, ignore_index):
 def lovasz_softmax_backward(grad, logits, labels, jacc, ignore_index):
     """-> dloss/dlogits for the upstream gradient `grad` [C], csrc/lovasz_softmax.cu:788-797."""
     gpu_only("lovasz softmax function", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     out = torch.empty_like(x)
     go, dj = grad.float().contiguous(), jacc.float().contiguous()      # fp32 at the ABI
     if x.numel():

@@ -2,6 +2,7 @@
 import torch
 
 from ._abi import F32, I32, I64, P, bind, check, dims, gpu_only, native, stream
+from ._abi import labels as int64_labels
 
 _fwd = bind("plh_lsr_forward", [P, I32, P, P, I64, I64, I64, I64, F32, P])
 _bwd = bind("plh_lsr_backward", [P, I32, P, P, I64, P, I64, I64, I64, I64, F32, P])
@@ -10,7 +11,7 @@ _bwd = bind("plh_lsr_backward", [P, I32, P, P, I64, P, I64, I64, I64, I64, F32, 
 def lsr_forward(logits, labels, ignore_index, smooth):
     """csrc/lsr_kernel.cu:296-305 -> per-pixel losses, shape of `labels`, dtype of `logits`."""
     gpu_only("LSR loss", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     losses = torch.empty(lb.shape, dtype=torch.float32, device=x.device)     # losses are fp32 at the ABI
     if x.numel():
         with torch.cuda.device_of(x):
@@ -22,7 +23,7 @@ def lsr_backward(logits, labels, ignore_index, smooth):
     """csrc/lsr_kernel.cu:307-317 -> dloss/dlogits; pytorch_loss/label_smooth.py:144 then multiplies by
     the upstream gradient (a NULL grad_output asks the library for the reference's raw gradient)."""
     gpu_only("LSR loss", logits, labels)
-    (x, tag), lb = native(logits), labels.contiguous()
+    (x, tag), lb = native(logits), int64_labels(labels, logits)
     grad = torch.empty_like(x)
     if x.numel():
         with torch.cuda.device_of(x):

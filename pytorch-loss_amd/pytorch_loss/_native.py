@@ -47,6 +47,8 @@ _SIGNATURES = {
     "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_lovasz_lookback_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "plh_lovasz_forward_lookback": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "plh_ohem_workspace_bytes": (_i64, [_i64]),
     "plh_ohem_scores": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _p]),
@@ -418,18 +420,21 @@ def lovasz_args(logits, labels):
     return seg_args(logits, labels, "lovasz softmax function", "lovasz_softmax")
 
 
-def lovasz_forward(logits, labels, ignore_index, args=None):
-    """-> (losses[C], jacc[C, N*M] fp32)"""
+def lovasz_forward(logits, labels, ignore_index, args=None, look_back=False):
+    """-> (losses[C], jacc[C, N*M] fp32). look_back=True runs the sort passes in their decoupled look-back form
+    (same results bit for bit, slower; see plh_lovasz_forward_lookback)."""
     a = args or lovasz_args(logits, labels)
+    entry, sizer = (("plh_lovasz_forward_lookback", "plh_lovasz_lookback_workspace_bytes") if look_back
+                    else ("plh_lovasz_forward", "plh_lovasz_workspace_bytes"))
     losses = torch.empty((a.c,), dtype=torch.float32, device=a.x.device)
     jacc = torch.empty((a.c, a.n * a.m), dtype=torch.float32, device=a.x.device)
     if a.x.numel() == 0:
         return _back_to(losses.zero_(), _loss_dtype(a.dtype)), jacc
-    ws_bytes = int(load().plh_lovasz_workspace_bytes(a.n, a.c, a.m))
+    ws_bytes = int(getattr(load(), sizer)(a.n, a.c, a.m))
     if ws_bytes < 0:
         _check(ws_bytes)
     workspace = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=a.x.device)
-    _call(a.x, "plh_lovasz_forward", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(losses), _ptr(jacc), _ptr(workspace), ws_bytes,
           a.n, a.c, a.m, int(ignore_index))
     return _back_to(losses, _loss_dtype(a.dtype)), jacc
 

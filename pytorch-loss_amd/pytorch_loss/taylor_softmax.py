@@ -18,10 +18,15 @@ from . import _native
 
 
 def _even_order(n):
-    """The reference asserts on the order where it is given (taylor_softmax.py:89, 110, 132, 182). Its log
-    module and its cross entropy let n = 0 through their constructors (`assert n % 2 == 0`) and fail on it
-    in the first forward (`assert n % 2 == 0 and n > 0`, :36); here the constructor already refuses it."""
+    """What the reference asserts wherever the order is used (taylor_softmax.py:38, 50, 85)."""
     assert n % 2 == 0 and n > 0, "the order of the Taylor polynomial must be even and positive"
+    return n
+
+
+def _even(n):
+    """What the constructors of the reference's log module and cross entropy assert (taylor_softmax.py:131, 181):
+    an even order; n = 0 (or a negative even one) passes there and fails in the first forward, as it does here."""
+    assert n % 2 == 0, "the order of the Taylor polynomial must be even"
     return n
 
 
@@ -60,6 +65,10 @@ class LogTaylorSoftmaxV3(_TaylorAlongDim):
     """Usage as ``nn.LogSoftmax(dim)``."""
     use_log = True
 
+    def __init__(self, dim=1, n=2):
+        nn.Module.__init__(self)
+        self.dim, self.n = dim, _even(n)
+
 
 class TaylorCrossEntropyFunctionV3(torch.autograd.Function):
     """-log_taylor_softmax(logits)[label] per pixel, or its 'sum' / 'mean' over the non-ignored
@@ -84,7 +93,7 @@ class TaylorCrossEntropyLossV3(nn.Module):
 
     def __init__(self, n=2, ignore_index=-1, reduction='mean'):
         super().__init__()
-        self.n, self.ignore_index, self.reduction = _even_order(n), ignore_index, reduction
+        self.n, self.ignore_index, self.reduction = _even(n), ignore_index, reduction
 
     def forward(self, logits, labels):
-        return TaylorCrossEntropyFunctionV3.apply(logits, labels, self.n, self.ignore_index, self.reduction)
+        return TaylorCrossEntropyFunctionV3.apply(logits, labels, _even_order(self.n), self.ignore_index, self.reduction)

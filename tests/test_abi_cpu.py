@@ -266,15 +266,40 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
 
 
-def test_taylor_orders_are_checked_at_construction():
+def test_taylor_orders_are_checked_where_the_reference_checks_them():
+    """pytorch_loss/taylor_softmax.py: TaylorSoftmaxV3's constructor wants an even positive order (:85), the log
+    module's and the cross entropy's only an even one (:131, :181); those two refuse n = 0 in their first forward (:50)."""
     import pytorch_loss as pl
     for bad in (0, 3, -2):
-        for make in (pl.TaylorSoftmaxV3, pl.LogTaylorSoftmaxV3):
-            with pytest.raises(AssertionError):
-                make(dim=1, n=bad)
+        with pytest.raises(AssertionError):
+            pl.TaylorSoftmaxV3(dim=1, n=bad)
+    for bad in (3, -1):
+        with pytest.raises(AssertionError):
+            pl.LogTaylorSoftmaxV3(dim=1, n=bad)
         with pytest.raises(AssertionError):
             pl.TaylorCrossEntropyLossV3(n=bad)
+    x, y = torch.zeros(2, 3), torch.zeros(2, dtype=torch.int64)
+    with pytest.raises(AssertionError):
+        pl.LogTaylorSoftmaxV3(n=0)(x)
+    with pytest.raises(AssertionError):
+        pl.TaylorCrossEntropyLossV3(n=0)(x, y)
     assert pl.TaylorCrossEntropyLossV3(n=4).n == 4 and pl.LogTaylorSoftmaxV3(n=2).n == 2
+
+
+def test_extension_stand_ins_refuse_labels_the_abi_would_misread():
+    """The C ABI reads labels as int64, one per pixel: the stand-ins raise for another dtype (as the reference's
+    data_ptr<int64_t>() does) or another element count before any pointer is handed over."""
+    from ext_stubs import _abi
+    x = torch.zeros(2, 3, 4)
+    assert _abi.labels(torch.zeros(2, 4, dtype=torch.int64), x).dtype == torch.int64
+    assert _abi.labels(torch.zeros(4, 2, dtype=torch.int64).t(), x).is_contiguous()
+    for bad in (torch.zeros(2, 4, dtype=torch.int32), torch.zeros(2, 4, dtype=torch.uint8), torch.zeros(2, 4)):
+        with pytest.raises(RuntimeError, match="Long"):
+            _abi.labels(bad, x)
+    for bad in (torch.zeros(2, 3, dtype=torch.int64), torch.zeros(2, 3, 4, dtype=torch.int64)):
+        with pytest.raises(RuntimeError, match="do not go with"):
+            _abi.labels(bad, x)
+    assert _abi.labels(torch.zeros(5, dtype=torch.int64), torch.zeros(5, 7)).shape == (5,)
 
 
 def test_extension_stand_ins_load_and_refuse_cpu_tensors():

@@ -1,4 +1,4 @@
-"""The decoupled look-back variant of the Lovasz sort passes (PLH_LOVASZ_SCAN=lookback: tile descriptors and
+"""The decoupled look-back variant of the Lovasz sort passes (plh_lovasz_forward_lookback: tile descriptors and
 chained waits instead of a histogram kernel and a row scan in front of every pass) must give the results of the
 default passes bit for bit: same keys, same stable order, same Jaccard differences, same fixed-order loss sums."""
 import numpy as np
@@ -34,18 +34,16 @@ CASES = [
 
 
 @pytest.mark.parametrize("shape,scale,boost", CASES)
-def test_look_back_variant_is_bit_identical(native, monkeypatch, shape, scale, boost):
+def test_look_back_variant_is_bit_identical(native, shape, scale, boost):
     n_cls = shape[1]
     y = synth.seg_labels(61, shape[:1] + shape[2:], n_cls, 255, 0.1)
     x = synth.normal(61, 1, shape, 0.0, scale)
     if boost:
         x = x + np.float32(boost) * np.moveaxis(np.eye(n_cls, dtype=np.float32)[np.where(y == 255, 0, y)], -1, 1)
     xt, yt = dev(x), dev(y)
-    monkeypatch.delenv("PLH_LOVASZ_SCAN", raising=False)
     losses, jacc = native.lovasz_forward(xt, yt, 255)
-    monkeypatch.setenv("PLH_LOVASZ_SCAN", "lookback")
     for _ in range(2):                                  # twice: tickets and descriptors are cleared per call
-        losses_lb, jacc_lb = native.lovasz_forward(xt, yt, 255)
+        losses_lb, jacc_lb = native.lovasz_forward(xt, yt, 255, look_back=True)
         assert not torch.isnan(losses_lb).any()
         assert torch.equal(losses_lb, losses)
         assert torch.equal(jacc_lb.view(torch.int32), jacc.view(torch.int32))

@@ -198,10 +198,24 @@ def test_lsr_module_reductions(pl, reduction, smooth):
 def test_fused_reductions_on_every_execution_shape(pl, kind, shape, ignore, frac):
     """'mean' / 'sum' come from per-block partials inside the forward kernel: every launch shape
     (registers, wavefront per row, lane per pixel, ragged tails) must agree with the unreduced path."""
-    if frac >= 1.0:
-        pytest.skip("all ignored: covered by the NaN test")
     x, y = seg_inputs(25, shape, ignore, frac)
     yt = dev(y)
+    if frac >= 1.0:
+        # every pixel ignored: 'sum' is an exact 0 with an exactly zero gradient, 'mean' is 0 / 0 = NaN, as in the
+        # reference's modules (pytorch_loss/label_smooth.py:169-170, pytorch_loss/large_margin_softmax.py:170-171)
+        assert int((y != ignore).sum()) == 0
+        for red in ("sum", "mean"):
+            crit = (pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=ignore) if kind == "lsr"
+                    else pl.LargeMarginSoftmaxV3(lam=0.3, reduction=red, ignore_index=ignore))
+            xt = dev(x).requires_grad_()
+            out = crit(xt, yt)
+            if red == "sum":
+                assert out.item() == 0.0
+                out.backward()
+                assert xt.grad.abs().max().item() == 0.0
+            else:
+                assert torch.isnan(out).item()
+        return
     if kind == "lsr":
         make = lambda red: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=red, ignore_index=ignore)
         per = oracle.lsr_forward(x.astype(np.float64), y, ignore, 0.1)
@@ -573,6 +587,28 @@ def test_rows_with_masked_vocabulary_entries_stay_finite(pl, n_cls, masked):
     scores = _native.ohem_scores(xt, yt, 255).cpu().numpy()
     assert np.isfinite(scores).all()
     np.testing.assert_allclose(scores, oracle.ohem_scores(x, y, 255), rtol=2e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("shape", [(6, 100), (5, 300), (9, 1000), (6, 150), (4, 5000)])
+def test_large_margin_rows_with_a_masked_class(pl, shape):
+    """A logit of -inf among the classes other than the target: that class has q = 0 and the margin term
+    (0 - coeff) * log 0 = +inf (root large_margin_softmax.py:84-90, csrc/large_margin_kernel.cu:183-190). The
+    forward-only kernels of the (N, C) shapes take the margin term in closed form; a row with a masked class must
+    come out as it does from the kernels that also produce the gradient, and the rows around it must not notice."""
+    x = synth.normal(91, 1, shape, 0.0, 2.0)
+    y = synth.randint(91, 11, shape[:1], 0, shape[1])
+    y[0] = 255
+    masked_row = 2
+    col = (int(y[masked_row]) + 3) % shape[1]
+    x[masked_row, col] = -np.inf
+    want = oracle.lmargin_forward(x.astype(np.float64), y, 0.3, 255)
+    assert np.isposinf(want[masked_row]) and np.isfinite(np.delete(want, masked_row)).all()
+    xt, yt = dev(x), dev(y)
+    fwd = pl.LargeMarginSoftmaxFuncV3.apply(xt, yt, 0.3, 255).cpu().numpy()
+    both = pl.LargeMarginSoftmaxFuncV3FB.apply(xt.clone().requires_grad_(), yt, 0.3, 255)[0].detach().cpu().numpy()
+    for got, what in ((fwd, "forward"), (both, "forward+backward")):
+        assert np.isposinf(got[masked_row]), (what, got[masked_row])
+        close_loss(np.delete(got, masked_row), np.delete(want, masked_row), "masked class, " + what)
 
 
 def _prototype_logits(seed, shape, n_proto):

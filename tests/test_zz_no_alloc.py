@@ -73,3 +73,51 @@ def test_static_scratch_entry_point_rejects_oversize_and_bad_arguments():
     assert lib.plh_lsr_forward_reduced_static(p(x), 7, p(y), None, p(out), None, 1, 1, 2, 1, 255, 0.1, None) == -7
     assert lib.plh_lsr_forward_reduced_static(p(x), 0, p(y), None, None, None, 1, 2, 2, 2, 255, 0.1, None) == -1
     torch.cuda.synchronize()
+
+
+def test_static_scratch_entry_point_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point is for: the device's free memory is the same before and after its calls (the first call
+    on a device, which looks the scratch array's address up, has happened by then), and a call captured in a HIP
+    graph replays to the bits of the eager call, with eager work between the replays."""
+    from pytorch_loss import _native
+    lib = _native.load()
+    dev = torch.device("cuda:0")
+    shape, ignore = (3, 19, 96, 80), 255
+    x_np = synth.normal(47, 1, shape, 0.0, 2.0)
+    y_np = synth.seg_labels(47, shape[:1] + shape[2:], shape[1], ignore, 0.1)
+    x, y = torch.from_numpy(x_np).to(dev), torch.from_numpy(y_np).to(dev)
+    n, c, m = shape[0], shape[1], shape[2] * shape[3]
+    loss = torch.zeros(1, device=dev)
+    cnt = torch.zeros(1, dtype=torch.int64, device=dev)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def call(stream):
+        rc = lib.plh_lsr_forward_reduced_static(p(x), 0, p(y), None, p(loss), p(cnt), 1, n, c, m, ignore, 0.1,
+                                                ctypes.c_void_p(stream))
+        assert rc == 0, rc
+
+    call(torch.cuda.current_stream().cuda_stream)            # first call on the device: outside any capture
+    torch.cuda.synchronize()
+    want = (loss.clone(), cnt.clone())
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(5):
+        call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(loss, want[0]) and torch.equal(cnt, want[1])
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream().cuda_stream)
+    for i in range(3):
+        loss.fill_(-1.0)
+        cnt.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(loss, want[0]) and torch.equal(cnt, want[1]), i
+        # eager work between the replays, on the same scratch array (a smaller input)
+        small = _run(lib, "plh_lsr_forward_reduced_static", x[:1].contiguous(), y[:1].contiguous(), ignore, 0.1, 1, False)
+        assert small[1] == int((y_np[:1] != ignore).sum())
+    per = oracle.lsr_forward(x_np.astype(np.float64), y_np, ignore, 0.1)
+    ref = per.sum() / int((y_np != ignore).sum())
+    assert abs(float(want[0].item()) - ref) <= 1e-5 * abs(ref)
