@@ -1,6 +1,5 @@
 // Large-margin softmax cross entropy for gfx950: the C entry points. The kernels live in
-// lmargin_kernels.hpp and are compiled once per element type (lmargin_f32.hip, lmargin_f16.hip,
-// lmargin_bf16.hip).
+// lmargin_kernels.hpp and are compiled per element type and direction (lmargin_f32_fwd.hip, ...).
 #include "lmargin_kernels.hpp"
 
 namespace plh {
@@ -8,6 +7,19 @@ namespace plh {
 PLH_LM_EXTERN(float)
 PLH_LM_EXTERN(f16)
 PLH_LM_EXTERN(bf16)
+
+// The partial sums (part.sum) and the count of valid pixels (cnt) are produced when their pointers are given: the
+// kernels test the pointers, so the reduced forward shares its kernels with the plain one.
+template <class T>
+static unsigned lmargin_run_typed(int variant, const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
+                                  unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
+    switch (variant) {
+        case kLmForward:
+        case kLmForwardReduced: return launch_typed<T, true, false>(x, lab, up, loss, grad, cnt, part, p, st);
+        case kLmBackward: return launch_typed<T, false, true>(x, lab, up, loss, grad, cnt, part, p, st);
+        default: return launch_typed<T, true, true>(x, lab, up, loss, grad, cnt, part, p, st);
+    }
+}
 
 // Launches one direction (or the fused pair). blocks_out: blocks that wrote partials (Reduce only).
 static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,

@@ -38,12 +38,17 @@ struct LmParams {
 // log2(s_no), sum q_j u_j and the rebuilt full sum.
 constexpr float kLmMasked = -1e30f;
 
-template <class T, int CP, int V, int Form, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, int CP, int V, int Form, bool WantLoss, bool WantGrad>
 __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                      const Upstream up,
                                                      float *__restrict__ loss, T *__restrict__ grad,
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
+    // only the plain forward leaves partial sums, so the other combinations carry no code for them
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     const bool live = at.live;
@@ -160,7 +165,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                     }
                 }
         }
-        if constexpr (WantCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
+        if constexpr (kMayCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
         if constexpr (kInPlace) __builtin_amdgcn_sched_barrier(0);
     }
     if (live) {
@@ -178,11 +183,11 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             at.store_slice(grad, p.C, p.m_size, raw);
         }
     }
-    if constexpr (WantCount) {
+    if (WantCount) {
         // lanes leave only at the tail of the grid, so lane 0 of a wave with work is alive
         if ((threadIdx.x & 63) == 0) atomicAdd(valid_cnt, (unsigned long long)n_valid);
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);
         if (threadIdx.x == 0) {
@@ -267,9 +272,10 @@ __device__ __forceinline__ LmSplitStats<V> lm_split_combine(float (*parts)[kSpli
     return r;
 }
 
-template <class T, int KW, int V, bool Reduce, bool PerImage = false>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            float *__restrict__ loss, Partials part, const LmParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float parts[6][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
@@ -312,7 +318,7 @@ __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict_
     }
     if (at.live && loss) at.store_f32(loss, out);
     if (at.live && p.scores) at.template store_f32<true>(p.scores, score);
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());
         if (lane == 0) {
@@ -391,12 +397,17 @@ __global__ __launch_bounds__(kSplitBlock) void lm_bwd_split(const T *__restrict_
 // G lanes per pixel, striding over its channels; three sweeps, the later ones re-reading what the first
 // pulled into cache. Launched with G = 1: a lane per pixel, for channel counts no other shape takes.
 
-template <class T, int G, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, int G, bool WantLoss, bool WantGrad>
 __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                 const Upstream up,
                                                 float *__restrict__ loss, T *__restrict__ grad,
                                                 unsigned long long *__restrict__ valid_cnt, Partials part,
                                                 const LmParams p) {
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
+    // only the plain forward leaves partial sums, so the other combinations carry no code for them
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    const bool Reduce = kMayReduce && part.sum != nullptr;
     constexpr int kPix = 256 / G;
     __shared__ float red[4];
     float mine = 0.f, cnt = 0.f;
@@ -467,13 +478,13 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
             }
         }
         // every lane of the wave is inside the loop, so the ballot sees the whole wave
-        if constexpr (WantCount)
+        if constexpr (kMayCount)
             n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && sub == 0 && !ign));
     }
-    if constexpr (WantCount) {
+    if (WantCount) {
         if ((threadIdx.x & 63) == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);
         if (threadIdx.x == 0) {
@@ -487,11 +498,16 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
 // (N, C) inputs with 33..2048 channels: the row sits in the wavefront's registers (WaveRow), so the three
 // sweeps of the group kernel (maxima, sums, terms) read HBM once. Same arithmetic as lm_group.
 
-template <class T, int NI, int LP, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce, int G, bool Cached = false>
+template <class T, int NI, int LP, bool WantLoss, bool WantGrad, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
                                                const LmParams p) {
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
+    // only the plain forward leaves partial sums, so the other combinations carry no code for them
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
     using Span = WaveRowSpan<T, L, G, NI>;
@@ -613,12 +629,12 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                 cnt += ign ? 0.f : 1.f;
             }
         }
-        if constexpr (WantCount) n_valid += (lane == 0 && live && !ign) ? 1 : 0;
+        if constexpr (kMayCount) n_valid += (lane == 0 && live && !ign) ? 1 : 0;
     }
-    if constexpr (WantCount) {
+    if (WantCount) {
         if (lane == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);
         if (threadIdx.x == 0) {
@@ -701,11 +717,16 @@ __device__ __forceinline__ LmRowStats lm_row_sweep(const T *xs, int C, int tgt, 
     return r;
 }
 
-template <class T, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, bool WantLoss, bool WantGrad>
 __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
                                                     const LmParams p, int vec) {
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
+    // only the plain forward leaves partial sums, so the other combinations carry no code for them
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[kRowBlock / 64];
     constexpr int L = RowChunk<T>::kLen;
     float mine = 0.f;
@@ -737,7 +758,7 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                 cnt += ign ? 0 : 1;
             }
         }
-        if constexpr (WantCount) n_valid += (threadIdx.x == 0 && !ign) ? 1 : 0;
+        if constexpr (kMayCount) n_valid += (threadIdx.x == 0 && !ign) ? 1 : 0;
         if constexpr (WantGrad) {
             float go[1];
             load_upstream<1>(up, row, go);
@@ -763,10 +784,10 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
             for (int j = sp.tail_from + threadIdx.x; j < p.C; j += row_threads()) store_one(gs + j, one(load_one(xs + j), j));
         }
     }
-    if constexpr (WantCount) {
+    if (WantCount) {
         if (threadIdx.x == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
@@ -778,7 +799,7 @@ static __global__ void lm_zero_count(unsigned long long *cnt) { *cnt = 0; }
 
 // ------------------------------------------------------------ dispatch ----
 
-template <class T, int V, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, int V, bool WantLoss, bool WantGrad>
 static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                             unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
@@ -788,12 +809,12 @@ static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, 
     case K:                                                                                                          \
         if constexpr (V * sizeof(T) == 8) {                                                                          \
             if (uni) {                                                                                               \
-                hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kUniform, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),  \
+                hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kUniform, WantLoss, WantGrad>), dim3(grid),  \
                                    dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                   \
                 break;                                                                                               \
             }                                                                                                        \
         }                                                                                                            \
-        hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kGeneral, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid),         \
+        hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kGeneral, WantLoss, WantGrad>), dim3(grid),         \
                            dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                           \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -804,7 +825,7 @@ static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, 
 
 // NCHW whose channel planes start on element boundaries only (odd lengths): the per-image form, four
 // pixels per lane.
-template <class T, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
+template <class T, bool WantLoss, bool WantGrad>
 static unsigned launch_image(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                              unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
@@ -812,7 +833,7 @@ static unsigned launch_image(const T *x, const int64_t *lab, const Upstream &up,
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
         if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                             \
-            hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, WantLoss, WantGrad, WantCount, Reduce>), dim3(grid), \
+            hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, WantLoss, WantGrad>), dim3(grid), \
                                dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                       \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -821,8 +842,8 @@ static unsigned launch_image(const T *x, const int64_t *lab, const Upstream &up,
     return grid;
 }
 
-template <class T, bool WantLoss, bool WantGrad, bool WantCount, bool Reduce>
-static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
+template <class T, bool WantLoss, bool WantGrad>
+unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                              unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
@@ -840,7 +861,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         if constexpr (WantLoss)                                                                                       \
-            hipLaunchKernelGGL((lm_fwd_split<T, KW, VD, Reduce>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, VD>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
                                part, p);                                                                              \
         else                                                                                                          \
             hipLaunchKernelGGL((lm_bwd_split<T, KW, VD>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
@@ -857,7 +878,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         if constexpr (WantLoss)                                                                                       \
-            hipLaunchKernelGGL((lm_fwd_split<T, KW, V, Reduce>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, V>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, loss, \
                                part, p);                                                                              \
         else                                                                                                          \
             hipLaunchKernelGGL((lm_bwd_split<T, KW, V>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up, grad, p); \
@@ -874,7 +895,7 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         if constexpr (WantLoss)                                                                                       \
-            hipLaunchKernelGGL((lm_fwd_split<T, KW, V, Reduce, true>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, \
+            hipLaunchKernelGGL((lm_fwd_split<T, KW, V, true>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, \
                                loss, part, p);                                                                        \
         else                                                                                                          \
             hipLaunchKernelGGL((lm_bwd_split<T, KW, V, true>), dim3(blocks), dim3(kSplitBlock), 0, st, x, lab, up,    \
@@ -886,14 +907,14 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
             }
             break;
         case Shape::RegsVec:
-            blocks = launch_regs<T, V, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+            blocks = launch_regs<T, V, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) {
-                blocks = launch_image<T, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+                blocks = launch_image<T, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
                 break;
             }
-            blocks = launch_regs<T, 1, WantLoss, WantGrad, WantCount, Reduce>(x, lab, up, loss, grad, cnt, part, p, st);
+            blocks = launch_regs<T, 1, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
             break;
         case Shape::Wave:
             if (p.C <= wrow_cap<T>(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C))) {
@@ -902,12 +923,12 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
         blocks = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                     \
         if constexpr (WantGrad && wrow_cached_form<T>(W, G)) {                                                     \
             if (wrow_rows_end_inside_lines<T>(p.C)) {                                                              \
-                hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G, true>), dim3(blocks), \
+                hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, G, true>), dim3(blocks), \
                                    dim3(256), 0, st, x, lab, up, loss, grad, cnt, part, p);                        \
                 break;                                                                                             \
             }                                                                                                      \
         }                                                                                                          \
-        hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, WantCount, Reduce, G>), dim3(blocks), dim3(256), 0, \
+        hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, G>), dim3(blocks), dim3(256), 0, \
                            st, x, lab, up, loss, grad, cnt, part, p);                                              \
     } while (0)
                 PLH_WROW_DISPATCH_IF(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C), p.C, PLH_GO, (WantGrad ? 1 : 2));
@@ -915,38 +936,31 @@ static unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up,
                 break;
             }
             blocks = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0, st,
+            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0, st,
                                x, lab, up, loss, grad, cnt, part, p, row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C));
             break;
         case Shape::Lane:
             blocks = group_grid(p.P, 256);
-            hipLaunchKernelGGL((lm_group<T, 1, WantLoss, WantGrad, WantCount, Reduce>), dim3(blocks), dim3(256), 0, st,
+            hipLaunchKernelGGL((lm_group<T, 1, WantLoss, WantGrad>), dim3(blocks), dim3(256), 0, st,
                                x, lab, up, loss, grad, cnt, part, p);
             break;
     }
     return blocks;
 }
 
-// Per-dtype entry into the kernels of this header: `variant` picks one of the four combinations the
-// entry points use. Explicitly instantiated in lmargin_f32.hip, lmargin_f16.hip and lmargin_bf16.hip
-// so that the three element types compile in parallel.
+// Per-dtype entries into the kernels of this header. The entry points use three combinations of (loss, gradient):
+// forward (plain or with partial sums), backward, and the fused pair (with the count of valid pixels); each is
+// explicitly instantiated per element type in a translation unit of its own (lmargin_f32_fwd.hip, lmargin_f32_bwd.hip,
+// lmargin_f32_both.hip, ...) so that the nine parts compile in parallel.
 enum LmVariant { kLmForward = 0, kLmForwardReduced = 1, kLmBackward = 2, kLmForwardBackwardCount = 3 };
 
-template <class T>
-unsigned lmargin_run_typed(int variant, const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
-                           unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
-    switch (variant) {
-        case kLmForward: return launch_typed<T, true, false, false, false>(x, lab, up, loss, grad, cnt, part, p, st);
-        case kLmForwardReduced: return launch_typed<T, true, false, false, true>(x, lab, up, loss, grad, cnt, part, p, st);
-        case kLmBackward: return launch_typed<T, false, true, false, false>(x, lab, up, loss, grad, cnt, part, p, st);
-        default: return launch_typed<T, true, true, true, false>(x, lab, up, loss, grad, cnt, part, p, st);
-    }
-}
-
-#define PLH_LM_SIGNATURE(T)                                                                                        \
-    unsigned lmargin_run_typed<T>(int, const T *, const int64_t *, const Upstream &, float *, T *, unsigned long long *, \
-                                  Partials, const LmParams &, hipStream_t);
-#define PLH_LM_EXTERN(T) extern template PLH_LM_SIGNATURE(T)
-#define PLH_LM_INSTANTIATE(T) template PLH_LM_SIGNATURE(T)
+#define PLH_LM_SIGNATURE(T, L, G)                                                                                    \
+    unsigned launch_typed<T, L, G>(const T *, const int64_t *, const Upstream &, float *, T *, unsigned long long *, \
+                                   Partials, const LmParams &, hipStream_t);
+#define PLH_LM_EXTERN(T)                              \
+    extern template PLH_LM_SIGNATURE(T, true, false)  \
+    extern template PLH_LM_SIGNATURE(T, false, true)  \
+    extern template PLH_LM_SIGNATURE(T, true, true)
+#define PLH_LM_INSTANTIATE(T, L, G) template PLH_LM_SIGNATURE(T, L, G)
 
 }  // namespace plh

@@ -1,0 +1,5 @@
+// LSR forward kernels for bf16 logits (one translation unit per element type and direction).
+#include "lsr_kernels.hpp"
+namespace plh {
+PLH_LSR_INSTANTIATE_FWD(bf16)
+}

@@ -34,11 +34,12 @@ struct LsrParams {
 // exp(x - mx) is evaluated as exp2(fma(x, log2e, -c)) with c = fl(mx * log2e); what the rounding
 // of c left out, r = mx*log2e - c (exact, one fma), scales every term by 2^r and is taken back
 // out of log2(sum).
-template <class T, int CP, int V, int Form, bool Reduce>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           float *__restrict__ loss, Partials part,
                                                           const LsrParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
         cnt += valid ? 1 : 0;
     }
     if (at.live && loss) at.store_f32(loss, out);
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);   // at most 1024 per block: exact in fp32
         if (threadIdx.x == 0) {
@@ -168,10 +169,11 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 //   backward  (c_w, s_w) in the base-2 domain, c_w = fl(m_w log2e), s_w = sum_j 2^(x_j log2e - c_w); every
 //             wavefront then evaluates 2^(x_j log2e - max_w c_w) / sum_w s_w 2^(c_w - max c) for its channels.
 
-template <class T, int KW, int V, bool Reduce, bool PerImage = false>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                             float *__restrict__ loss, Partials part,
                                                             const LsrParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float parts[4][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
         cnt += valid ? 1 : 0;
     }
     if (at.live && loss) at.store_f32(loss, out);
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());      // at most 256 per block: exact in fp32
         if (lane == 0) {
@@ -323,11 +325,12 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_bwd_split(const T *__restrict
 // G lanes per pixel, striding over its channels and re-reading global memory in each sweep (the
 // preceding sweep has just pulled the slice into cache). Launched with G = 1: a lane per pixel.
 
-template <class T, int G, bool Reduce>
+template <class T, int G>
 __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
                                                      const int64_t *__restrict__ lab,
                                                      float *__restrict__ loss, Partials part,
                                                      const LsrParams p) {
+    const bool Reduce = part.sum != nullptr;
     constexpr int kPix = 256 / G;
     __shared__ float red[4];
     const int sub = threadIdx.x % G;
@@ -373,7 +376,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
             cnt += valid ? 1.f : 0.f;
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);     // exact while a block sees < 2^24 pixels
         if (threadIdx.x == 0) {
@@ -437,9 +440,10 @@ __global__ __launch_bounds__(256) void lsr_bwd_group(const T *__restrict__ x,
 // 16 bytes per lane and step where the rows allow it, else pieces of 8, 4 or 2 bytes), so the row is read once and
 // every load of the row is in flight before the first one is used. Four rows per block at a time.
 
-template <class T, int NI, int LP, bool Reduce, int G>
+template <class T, int NI, int LP, int G>
 __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     float *__restrict__ loss, Partials part, const LsrParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
     const WaveRowAt<G> at;
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
             cnt += ign ? 0.f : 1.f;
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);
         if (threadIdx.x == 0) {
@@ -542,9 +546,10 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
 // that is rescaled when the maximum moves, so the forward reads the row once; the backward reads it a
 // second time (from cache for all but the longest rows) to write the gradient.
 
-template <class T, bool Reduce>
+template <class T>
 __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                    float *__restrict__ loss, Partials part, const LsrParams p, int vec) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float red[kRowBlock / 64];
     float mine = 0.f;
     int cnt = 0;
@@ -566,7 +571,7 @@ __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x
             cnt += ign ? 0 : 1;
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
@@ -704,7 +709,7 @@ inline LsrParams make_params(int64_t n_size, int64_t dimsize, int64_t m_size, in
     return p;
 }
 
-template <class T, int V, bool Reduce>
+template <class T, int V>
 static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                 hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
@@ -714,12 +719,12 @@ static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Par
     case K:                                                                                                       \
         if constexpr (V * sizeof(T) == 8) {                                                                       \
             if (uni) {                                                                                            \
-                hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kUniform, Reduce>), dim3(grid), dim3(kRegsBlock), 0,    \
+                hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kUniform>), dim3(grid), dim3(kRegsBlock), 0,    \
                                    st, x, lab, loss, part, p);                                                    \
                 break;                                                                                            \
             }                                                                                                     \
         }                                                                                                         \
-        hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kGeneral, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
+        hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, V, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
                            lab, loss, part, p);                                                                   \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -752,7 +757,7 @@ static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, 
 }
 
 // `image`: tiles per image (channel planes that start on element boundaries only)
-template <class T, int V, bool Reduce>
+template <class T, int V>
 static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                  hipStream_t st, bool image = false) {
     if constexpr (V == ElemTraits<T>::kVec) if (image) {      // the deep form (V / 2) has no such variant
@@ -762,7 +767,7 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
                 switch (split_slots(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
-        hipLaunchKernelGGL((lsr_fwd_split<T, KW, 4, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, 4, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
                            loss, part, p);                                                                        \
         break;
                     PLH_CASE(16) PLH_CASE(20)
@@ -775,7 +780,7 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
         switch (split_slots(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
-        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
                            loss, part, p);                                                                        \
         break;
             PLH_SPLIT_SLOT_CASES
@@ -788,7 +793,7 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
         switch (split_slots_deep(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
-        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
                            part, p);                                                                              \
         break;
             PLH_SPLIT_DEEP_CASES
@@ -799,7 +804,7 @@ static unsigned launch_fwd_split(const T *x, const int64_t *lab, float *loss, Pa
     switch (split_slots(p.C)) {
 #define PLH_CASE(KW)                                                                                              \
     case KW:                                                                                                      \
-        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
+        hipLaunchKernelGGL((lsr_fwd_split<T, KW, V>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, loss, \
                            part, p);                                                                              \
         break;
         PLH_SPLIT_SLOT_CASES
@@ -863,7 +868,7 @@ static void launch_bwd_split(const T *x, const int64_t *lab, const Upstream &up,
 
 // NCHW whose channel planes start on element boundaries only (odd lengths): the per-image form, four
 // pixels per lane.
-template <class T, bool Reduce>
+template <class T>
 static unsigned launch_fwd_image(const T *x, const int64_t *lab, float *loss, Partials part, const LsrParams &p,
                                  hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
@@ -871,7 +876,7 @@ static unsigned launch_fwd_image(const T *x, const int64_t *lab, float *loss, Pa
 #define PLH_CASE(K)                                                                                               \
     case K:                                                                                                       \
         if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                          \
-            hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, 4, kPerImage, Reduce>), dim3(grid), dim3(kRegsBlock), 0,   \
+            hipLaunchKernelGGL((lsr_fwd_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0,   \
                                st, x, lab, loss, part, p);                                                        \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
@@ -897,24 +902,24 @@ static void launch_bwd_image(const T *x, const int64_t *lab, const Upstream &up,
 }
 
 // Launches the forward; returns the number of blocks that wrote partials.
-template <class T, bool Reduce>
+template <class T>
 static unsigned forward_shape(const T *logits, const int64_t *labels, float *losses, Partials part, const LsrParams &p,
                         hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, nullptr, labels, losses, nullptr, true, true, true,
                        kImageFormMaxChannels<T>)) {
-        case Shape::RegsVec: return launch_fwd_regs<T, V, Reduce>(logits, labels, losses, part, p, st);
+        case Shape::RegsVec: return launch_fwd_regs<T, V>(logits, labels, losses, part, p, st);
         case Shape::RegsOne:
-            if (image_form_pays<T>(p.C, p.m_size)) return launch_fwd_image<T, Reduce>(logits, labels, losses, part, p, st);
-            return launch_fwd_regs<T, 1, Reduce>(logits, labels, losses, part, p, st);
-        case Shape::Split: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st);
-        case Shape::SplitImage: return launch_fwd_split<T, V, Reduce>(logits, labels, losses, part, p, st, true);
-        case Shape::SplitDeep: return launch_fwd_split<T, V / 2, Reduce>(logits, labels, losses, part, p, st);
+            if (image_form_pays<T>(p.C, p.m_size)) return launch_fwd_image<T>(logits, labels, losses, part, p, st);
+            return launch_fwd_regs<T, 1>(logits, labels, losses, part, p, st);
+        case Shape::Split: return launch_fwd_split<T, V>(logits, labels, losses, part, p, st);
+        case Shape::SplitImage: return launch_fwd_split<T, V>(logits, labels, losses, part, p, st, true);
+        case Shape::SplitDeep: return launch_fwd_split<T, V / 2>(logits, labels, losses, part, p, st);
         case Shape::Wave: {
             const int piece = wrow_piece<T>(logits, nullptr, p.C);
             if (p.C > wrow_cap<T>(piece)) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_fwd_row<T, Reduce>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels, losses, part, p,
+                hipLaunchKernelGGL((lsr_fwd_row<T>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels, losses, part, p,
                                    row_chunks_ok<T>(logits, nullptr, p.C));
                 return grid;
             }
@@ -922,7 +927,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
 #define PLH_GO(NI, W, G)                                                                                            \
     do {                                                                                                            \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                        \
-        hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, Reduce, G>), dim3(grid), dim3(256), 0, st, logits, labels, losses, \
+        hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, G>), dim3(grid), dim3(256), 0, st, logits, labels, losses, \
                            part, p);                                                                                \
     } while (0)
             PLH_WROW_DISPATCH(piece, p.C, PLH_GO);
@@ -931,7 +936,7 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
         }
         case Shape::Lane: {
             const unsigned grid = group_grid(p.P, 256);
-            hipLaunchKernelGGL((lsr_fwd_group<T, 1, Reduce>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
+            hipLaunchKernelGGL((lsr_fwd_group<T, 1>), dim3(grid), dim3(256), 0, st, logits, labels, losses, part, p);
             return grid;
         }
     }
@@ -1006,24 +1011,26 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
     }
 }
 
-// Per-dtype entry into the kernels of this header; explicitly instantiated in lsr_f32.hip,
-// lsr_f16.hip and lsr_bf16.hip so that the three element types compile in parallel.
+// Per-dtype entries into the kernels of this header; explicitly instantiated per element type and direction
+// (lsr_f32_fwd.hip, lsr_f32_bwd.hip, ...) so that the six parts compile in parallel.
 template <class T>
 unsigned lsr_forward_typed(const T *logits, const int64_t *labels, float *losses, Partials part, bool reduce,
                            const LsrParams &p, hipStream_t st) {
-    return reduce ? forward_shape<T, true>(logits, labels, losses, part, p, st)
-                  : forward_shape<T, false>(logits, labels, losses, part, p, st);
+    if (!reduce) part = Partials{nullptr, nullptr};      // the kernels leave partial sums where they are given a place
+    return forward_shape<T>(logits, labels, losses, part, p, st);
 }
 
-#define PLH_LSR_EXTERN(T)                                                                                           \
-    extern template unsigned lsr_forward_typed<T>(const T *, const int64_t *, float *, Partials, bool,              \
-                                                  const LsrParams &, hipStream_t);                                  \
-    extern template void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, \
-                                               hipStream_t);
+#define PLH_LSR_FWD_SIGNATURE(T)                                                                                    \
+    unsigned lsr_forward_typed<T>(const T *, const int64_t *, float *, Partials, bool, const LsrParams &, hipStream_t);
+#define PLH_LSR_BWD_SIGNATURE(T)                                                                                    \
+    void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, hipStream_t);
 
-#define PLH_LSR_INSTANTIATE(T)                                                                                      \
-    template unsigned lsr_forward_typed<T>(const T *, const int64_t *, float *, Partials, bool, const LsrParams &,  \
-                                           hipStream_t);                                                            \
-    template void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, hipStream_t);
+#define PLH_LSR_EXTERN(T)                  \
+    extern template PLH_LSR_FWD_SIGNATURE(T) \
+    extern template PLH_LSR_BWD_SIGNATURE(T)
+
+// one translation unit per element type and direction (lsr_<type>_fwd.hip, lsr_<type>_bwd.hip)
+#define PLH_LSR_INSTANTIATE_FWD(T) template PLH_LSR_FWD_SIGNATURE(T)
+#define PLH_LSR_INSTANTIATE_BWD(T) template PLH_LSR_BWD_SIGNATURE(T)
 
 }  // namespace plh

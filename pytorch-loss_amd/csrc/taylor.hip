@@ -1,6 +1,5 @@
 // Taylor softmax and the cross entropy on its logarithm: the C entry points. Kernels live in
-// taylor_kernels.hpp and are compiled once per element type (taylor_f32.hip, taylor_f16.hip,
-// taylor_bf16.hip).
+// taylor_kernels.hpp and are compiled per element type and kind (taylor_f32_fwd.hip, ...).
 #include "taylor_kernels.hpp"
 
 namespace plh {
@@ -8,6 +7,17 @@ namespace plh {
 PLH_TAYLOR_EXTERN(float)
 PLH_TAYLOR_EXTERN(f16)
 PLH_TAYLOR_EXTERN(bf16)
+
+template <class T>
+static unsigned taylor_run_typed(int kind, const T *x, const T *g, const int64_t *lab, const Upstream &up, T *out,
+                                 float *loss, Partials part, const TaylorParams &p, hipStream_t st) {
+    switch (kind) {
+        case kTaylorFwd: return taylor_launch<T, kTaylorFwd>(x, g, lab, up, out, loss, part, p, st);
+        case kTaylorBwd: return taylor_launch<T, kTaylorBwd>(x, g, lab, up, out, loss, part, p, st);
+        case kTaylorCeFwd: return taylor_launch<T, kTaylorCeFwd>(x, g, lab, up, out, loss, part, p, st);
+        default: return taylor_launch<T, kTaylorCeBwd>(x, g, lab, up, out, loss, part, p, st);
+    }
+}
 
 // Size and pointer checks of the label-free entry points: `in` and `out` hold elem-byte elements.
 static int check_pair(const void *in, const void *out, int64_t n_size, int64_t dimsize, int64_t m_size, size_t elem) {
@@ -31,12 +41,12 @@ static TaylorParams make_taylor(int64_t n_size, int64_t dimsize, int64_t m_size,
     return p;
 }
 
-static unsigned run(int kind, bool reduce, int32_t dtype, const void *x, const void *g, const int64_t *lab,
+static unsigned run(int kind, int32_t dtype, const void *x, const void *g, const int64_t *lab,
                     const Upstream &up, void *out, float *loss, Partials part, const TaylorParams &p, hipStream_t st) {
     unsigned blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
-        blocks = taylor_run_typed<T>(kind, reduce, static_cast<const T *>(x), static_cast<const T *>(g), lab, up,
+        blocks = taylor_run_typed<T>(kind, static_cast<const T *>(x), static_cast<const T *>(g), lab, up,
                                      static_cast<T *>(out), loss, part, p, st);
     });
     return blocks;
@@ -59,7 +69,7 @@ extern "C" int plh_taylor_softmax_forward(const void *feat, int32_t dtype, void 
     rc = check_pair(feat, out, n_size, dimsize, m_size, es);
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
-    run(kTaylorFwd, false, dtype, feat, nullptr, nullptr, kUnit, out, nullptr, kNone,
+    run(kTaylorFwd, dtype, feat, nullptr, nullptr, kUnit, out, nullptr, kNone,
         make_taylor(n_size, dimsize, m_size, order, use_log, 0, es), (hipStream_t)stream);
     return check_launch();
 }
@@ -76,7 +86,7 @@ extern "C" int plh_taylor_softmax_backward(const void *grad_output, const void *
     if (n_size * dimsize * m_size == 0) return PLH_OK;
     if (!grad_output) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_output, es)) return PLH_ERR_MISALIGNED;
-    run(kTaylorBwd, false, dtype, feat, grad_output, nullptr, kUnit, grad_feat, nullptr, kNone,
+    run(kTaylorBwd, dtype, feat, grad_output, nullptr, kUnit, grad_feat, nullptr, kNone,
         make_taylor(n_size, dimsize, m_size, order, use_log, 0, es), (hipStream_t)stream);
     return check_launch();
 }
@@ -104,7 +114,7 @@ extern "C" int plh_taylor_ce_forward(const void *logits, int32_t dtype, const in
     hipStream_t st = (hipStream_t)stream;
     unsigned blocks = 0;
     if (n_size * dimsize * m_size != 0)
-        blocks = run(kTaylorCeFwd, reduce, dtype, logits, nullptr, labels, kUnit, nullptr, losses, part,
+        blocks = run(kTaylorCeFwd, dtype, logits, nullptr, labels, kUnit, nullptr, losses, part,
                      make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es), st);
     if (reduce) finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
     return check_launch();
@@ -126,7 +136,7 @@ extern "C" int plh_taylor_ce_backward(const void *logits, int32_t dtype, const i
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
     const Upstream up{grad_output, grad_output_stride, divide_by, scale};
-    run(kTaylorCeBwd, false, dtype, logits, nullptr, labels, up, grad_logits, nullptr, kNone,
+    run(kTaylorCeBwd, dtype, logits, nullptr, labels, up, grad_logits, nullptr, kNone,
         make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es), (hipStream_t)stream);
     return check_launch();
 }

@@ -1,0 +1,5 @@
+// Taylor cross-entropy backward kernels for bf16 elements (see taylor_kernels.hpp).
+#include "taylor_kernels.hpp"
+namespace plh {
+PLH_TAYLOR_INSTANTIATE(bf16, kTaylorCeBwd)
+}

@@ -40,18 +40,26 @@ struct InvFactorials {
 __device__ constexpr InvFactorials kInvFact{};
 
 // f of order n (>= 2) and, as a by-product, of order n-1 (its derivative). The orders in common use
-// (2 and 4; `order` is uniform, so the branch is scalar) are evaluated in nested form, everything
-// else term by term upwards like the reference's recurrence (csrc/taylor_softmax.cu:24-33).
-__device__ __forceinline__ void taylor_pair(float x, int order, float &f, float &df) {
+// (2, the modules' default, and 4; `order` is uniform, so the branch is scalar) are evaluated in nested form.
+// The kernels that keep a slice or a row in registers are compiled for these two orders only (taylor_pair24):
+// every evaluation is inlined into their unrolled sweeps, and a third, general form there made up a third of
+// the library's code for orders nobody trains with; higher orders take the kernels that walk the slice
+// (taylor_group, the block-per-row forms), which evaluate term by term upwards like the reference's
+// recurrence (csrc/taylor_softmax.cu:24-33).
+__device__ __forceinline__ void taylor_pair24(float x, int order, float &f, float &df) {
     if (order == 2) {
         df = 1.f + x;
         f = __builtin_fmaf(x * x, 0.5f, df);
         return;
     }
-    if (order == 4) {
-        const float x2 = x * x;
-        df = __builtin_fmaf(x, __builtin_fmaf(x, __builtin_fmaf(x, 1.f / 6.f, 0.5f), 1.f), 1.f);
-        f = __builtin_fmaf(x2 * x2, 1.f / 24.f, df);
+    const float x2 = x * x;
+    df = __builtin_fmaf(x, __builtin_fmaf(x, __builtin_fmaf(x, 1.f / 6.f, 0.5f), 1.f), 1.f);
+    f = __builtin_fmaf(x2 * x2, 1.f / 24.f, df);
+}
+
+__device__ __forceinline__ void taylor_pair(float x, int order, float &f, float &df) {
+    if (order <= 4) {
+        taylor_pair24(x, order, f, df);
         return;
     }
     float res = 1.f + x, prev = 1.f, mid = x;
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, p.C)) {
                     float f, df;
-                    taylor_pair(PK::get(raw[j], k), p.order, f, df);
+                    taylor_pair24(PK::get(raw[j], k), p.order, f, df);
                     y[j][kk] = f;
                     s += f;
                 }
@@ -121,7 +129,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
                 s += f;
                 dot += p.use_log ? gj : f * gj;
@@ -142,7 +150,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
                 r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
             }
@@ -153,10 +161,11 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
 }
 
 // Cross entropy on the log form: loss per pixel (fp32), and its gradient with the upstream folded in.
-template <class T, int CP, int V, int Form, bool Reduce>
+template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 float *__restrict__ loss, Partials part,
                                                                 const TaylorParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
@@ -177,7 +186,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 s += f;
                 f_y = (tgt == j) ? f : f_y;
             }
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
         cnt += (at.live && !ign) ? 1 : 0;
     }
     if (at.live && loss) at.store_f32(loss, out);
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);
         if (threadIdx.x == 0) {
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 s += f;
                 f_y = (tgt[k] == j) ? f : f_y;
             }
@@ -252,7 +261,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
                 r[k] = df * ((tgt[k] == j) ? hot[k] : scale[k]);
             }
             raw[j] = Pack<T, V>::put(r) & mask;
@@ -265,10 +274,11 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
 // Cross entropy for 33..256 channels in NCHW (SplitSlice). The series needs no maximum, so the parts of
 // a pixel are just each wavefront's sum of the series and the target's term if it is held there.
 
-template <class T, int KW, int V, bool Reduce, bool PerImage = false>
+template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                   float *__restrict__ loss, Partials part,
                                                                   const TaylorParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float parts[2][kSplitWaves][kWave * V];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
                 s += (i < at.here) ? f : 0.f;
                 f_y = (rel == i) ? f : f_y;
             }
@@ -314,7 +324,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
         cnt += (at.live && !ign) ? 1 : 0;
     }
     if (at.live && loss) at.store_f32(loss, out);
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = group_reduce<64>(mine, OpSum());
         const float bc = group_reduce<64>((float)cnt, OpSum());
         if (lane == 0) {
@@ -350,7 +360,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
                 s += (i < at.here) ? f : 0.f;
                 f_y = (rel[k] == i) ? f : f_y;
             }
@@ -382,7 +392,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair(Pack<T, V>::get(raw[i], k), p.order, f, df);
+            taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
             r[k] = df * ((rel[k] == i) ? hot[k] : scale[k]);
         }
         raw[i] = Pack<T, V>::put(r) & mask;
@@ -409,7 +419,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair(PK::get(raw[i], k), p.order, f, df);
+                taylor_pair24(PK::get(raw[i], k), p.order, f, df);
                 s += (i < at.here) ? f : 0.f;
             }
             parts[wave][lane * V + k] = s;
@@ -434,7 +444,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair(PK::get(raw[i], k), p.order, f, df);
+            taylor_pair24(PK::get(raw[i], k), p.order, f, df);
             r[k] = p.use_log ? logf(f) - ls[k] : f * inv[k];
         }
         raw[i] = PK::put(r);
@@ -459,7 +469,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair(PK::get(raw[i], k), p.order, f, df);
+                taylor_pair24(PK::get(raw[i], k), p.order, f, df);
                 const float gj = PK::get(graw[i], k);
                 s += (i < at.here) ? f : 0.f;
                 dot += (i < at.here) ? (p.use_log ? gj : f * gj) : 0.f;
@@ -493,7 +503,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair(PK::get(raw[i], k), p.order, f, df);
+            taylor_pair24(PK::get(raw[i], k), p.order, f, df);
             const float gj = PK::get(graw[i], k);
             r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
         }
@@ -508,11 +518,12 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
 
 enum TaylorKind { kTaylorFwd = 0, kTaylorBwd = 1, kTaylorCeFwd = 2, kTaylorCeBwd = 3 };
 
-template <class T, int G, int Kind, bool Reduce>
+template <class T, int G, int Kind>
 __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, const T *__restrict__ g,
                                                     const int64_t *__restrict__ lab, const Upstream up,
                                                     T *__restrict__ out, float *__restrict__ loss, Partials part,
                                                     const TaylorParams p) {
+    const bool Reduce = part.sum != nullptr;
     constexpr int kPix = 256 / G;
     __shared__ float red[4];
     const int sub = threadIdx.x % G, grp = threadIdx.x / G;
@@ -589,7 +600,7 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
             }
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);
         if (threadIdx.x == 0) {
@@ -604,11 +615,12 @@ __global__ __launch_bounds__(256) void taylor_group(const T *__restrict__ x, con
 // upstream gradients) sits in the wavefront's registers, so both sweeps read HBM once. Same arithmetic as
 // the group kernel.
 
-template <class T, int NI, int LP, int Kind, bool Reduce, int G, bool Cached = false>
+template <class T, int NI, int LP, int Kind, int G, bool Cached = false>
 __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, const T *__restrict__ g,
                                                    const int64_t *__restrict__ lab, const Upstream up,
                                                    T *__restrict__ out, float *__restrict__ loss, Partials part,
                                                    const TaylorParams p) {
+    const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
     using Span = WaveRowSpan<T, L, G, NI>;
@@ -631,7 +643,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 float f, df;
-                taylor_pair(r.v[i][l], p.order, f, df);
+                taylor_pair24(r.v[i][l], p.order, f, df);
                 s += ok ? f : 0.f;
                 if constexpr (Kind == kTaylorBwd) {
                     const float gj = rg.v[i][l];
@@ -647,7 +659,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 const int64_t lb = lab[row];
                 const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
                 float f_y = 1.f, df;
-                if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df);
+                if (has_y) taylor_pair24(load_one(xs + lb), p.order, f_y, df);
                 const float v = has_y ? logf(s) - logf(f_y) : 0.f;
                 if (loss) loss[row] = v;
                 mine += v;
@@ -665,7 +677,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 if (lb != p.ignore && lb >= 0 && lb < p.C) {
                     tgt = (int)lb;
                     float f_y, df_y;
-                    taylor_pair(load_one(xs + lb), p.order, f_y, df_y);
+                    taylor_pair24(load_one(xs + lb), p.order, f_y, df_y);
                     cold = inv * go[0];
                     hot = cold - go[0] / f_y;
                 }
@@ -677,7 +689,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
 #pragma unroll
                 for (int l = 0; l < L; ++l) {
                     float f, df;
-                    taylor_pair(r.v[i][l], p.order, f, df);
+                    taylor_pair24(r.v[i][l], p.order, f, df);
                     if constexpr (Kind == kTaylorFwd) {
                         o[l] = p.use_log ? logf(f) - ls : f * inv;
                     } else if constexpr (Kind == kTaylorBwd) {
@@ -698,7 +710,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
             }
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256(cnt, red);
         if (threadIdx.x == 0) {
@@ -772,11 +784,12 @@ __global__ __launch_bounds__(kRowBlock) void taylor_sm_row(const T *__restrict__
     }
 }
 
-template <class T, int Kind, bool Reduce>
+template <class T, int Kind>
 __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            const Upstream up, T *__restrict__ out,
                                                            float *__restrict__ loss, Partials part,
                                                            const TaylorParams p, int vec) {
+    const bool Reduce = part.sum != nullptr;
     static_assert(Kind == kTaylorCeFwd || Kind == kTaylorCeBwd, "cross entropy only");
     __shared__ float red[kRowBlock / 64];
     float mine = 0.f;
@@ -817,7 +830,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
             });
         }
     }
-    if constexpr (Reduce) {
+    if (Reduce) {
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
@@ -827,13 +840,14 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
 
 // ------------------------------------------------------------ dispatch ----
 
-template <class T, int Kind, bool Reduce>
+template <class T, int Kind>
 unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstream &up, T *out, float *loss, Partials part,
                        const TaylorParams &p, hipStream_t st) {
     constexpr int VT = ElemTraits<T>::kVec;
     const float *go_vec = (Kind == kTaylorCeBwd && up.gout && up.stride == 1) ? up.gout : nullptr;
     constexpr bool kIsCe = (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd);       // the deep split form is theirs only
-    const Shape shape = pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
+    const bool walk = p.order > 4;          // the register-resident forms are compiled for orders 2 and 4 (taylor_pair24)
+    const Shape shape = walk ? Shape::Lane : pick_shape(p.C, p.m_size, VT, sizeof(T), x, (Kind == kTaylorCeFwd) ? nullptr : (const void *)out,
                                    lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true,
                                    kImageFormMaxChannels<T, (Kind == kTaylorBwd) ? 2 : 1>);
     const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
@@ -845,7 +859,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         if constexpr (Kind == kTaylorCeFwd)                                                                           \
-            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VD, Reduce>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
                                loss, part, p);                                                                        \
         else                                                                                                          \
             hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
@@ -869,7 +883,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         else if constexpr (Kind == kTaylorBwd)                                                                        \
             hipLaunchKernelGGL((taylor_sm_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, g, x, out, p); \
         else if constexpr (Kind == kTaylorCeFwd)                                                                      \
-            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, Reduce, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
+            hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
                                lab, loss, part, p);                                                                   \
         else                                                                                                          \
             hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, \
@@ -902,7 +916,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         else if constexpr (Kind == kTaylorBwd)                                                                       \
             hipLaunchKernelGGL((taylor_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, g, x, out, p); \
         else if constexpr (Kind == kTaylorCeFwd)                                                                     \
-            hipLaunchKernelGGL((taylor_ce_fwd_regs<T, CPV, VV, UU, Reduce>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
+            hipLaunchKernelGGL((taylor_ce_fwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
                                lab, loss, part, p);                                                                  \
         else                                                                                                         \
             hipLaunchKernelGGL((taylor_ce_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab,    \
@@ -931,19 +945,19 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         // cross-entropy backward with 64 registers of row ran at a third of its two-sweep form (bf16 (65536, 4096):
         // 0.782 against 0.304 ms)
         constexpr bool kForward = (Kind == kTaylorFwd || Kind == kTaylorCeFwd);
-        if (p.C <= (kForward ? wrow_cap<T>(piece) : kWaveRowCap)) {
+        if (!walk && p.C <= (kForward ? wrow_cap<T>(piece) : kWaveRowCap)) {
             unsigned grid = 0;
 #define PLH_GO(NI, W, G)                                                                                          \
     do {                                                                                                          \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                      \
         if constexpr (Kind != kTaylorCeFwd && wrow_cached_form<T>(W, G)) {                                        \
             if (wrow_rows_end_inside_lines<T>(p.C)) {                                                             \
-                hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G, true>), dim3(grid), dim3(256), 0, st, x, g, \
+                hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, G, true>), dim3(grid), dim3(256), 0, st, x, g, \
                                    lab, up, out, loss, part, p);                                                  \
                 break;                                                                                            \
             }                                                                                                     \
         }                                                                                                         \
-        hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, Reduce, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
+        hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
                            loss, part, p);                                                                        \
     } while (0)
             PLH_WROW_DISPATCH_IF(piece, p.C, PLH_GO, (kForward ? 2 : 0));
@@ -952,7 +966,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         }
         const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
         if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
-            hipLaunchKernelGGL((taylor_ce_row<T, Kind, Reduce>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, lab, up, out, loss,
+            hipLaunchKernelGGL((taylor_ce_row<T, Kind>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, lab, up, out, loss,
                                part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
         } else {
             const int vec = row_chunks_ok<T>(x, out, p.C) && !(Kind == kTaylorBwd && misaligned(g, 16));
@@ -961,28 +975,20 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         return grid;
     }
     const unsigned grid = group_grid(p.P, 256);
-    hipLaunchKernelGGL((taylor_group<T, 1, Kind, Reduce>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss, part, p);
+    hipLaunchKernelGGL((taylor_group<T, 1, Kind>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, loss, part, p);
     return grid;
 }
 
-// Per-dtype entry, instantiated in taylor_f32.hip / taylor_f16.hip / taylor_bf16.hip.
-template <class T>
-unsigned taylor_run_typed(int kind, bool reduce, const T *x, const T *g, const int64_t *lab, const Upstream &up, T *out,
-                          float *loss, Partials part, const TaylorParams &p, hipStream_t st) {
-    switch (kind) {
-        case kTaylorFwd: return taylor_launch<T, kTaylorFwd, false>(x, g, lab, up, out, loss, part, p, st);
-        case kTaylorBwd: return taylor_launch<T, kTaylorBwd, false>(x, g, lab, up, out, loss, part, p, st);
-        case kTaylorCeFwd:
-            return reduce ? taylor_launch<T, kTaylorCeFwd, true>(x, g, lab, up, out, loss, part, p, st)
-                          : taylor_launch<T, kTaylorCeFwd, false>(x, g, lab, up, out, loss, part, p, st);
-        default: return taylor_launch<T, kTaylorCeBwd, false>(x, g, lab, up, out, loss, part, p, st);
-    }
-}
-
-#define PLH_TAYLOR_SIGNATURE(T)                                                                                       \
-    unsigned taylor_run_typed<T>(int, bool, const T *, const T *, const int64_t *, const Upstream &, T *, float *,    \
-                                 Partials, const TaylorParams &, hipStream_t);
-#define PLH_TAYLOR_EXTERN(T) extern template PLH_TAYLOR_SIGNATURE(T)
-#define PLH_TAYLOR_INSTANTIATE(T) template PLH_TAYLOR_SIGNATURE(T)
+// One translation unit per element type and kind (taylor_f32_fwd.hip, taylor_f32_bwd.hip, taylor_f32_cefwd.hip,
+// taylor_f32_cebwd.hip, ...) so that the twelve parts compile in parallel.
+#define PLH_TAYLOR_SIGNATURE(T, K)                                                                                    \
+    unsigned taylor_launch<T, K>(const T *, const T *, const int64_t *, const Upstream &, T *, float *, Partials,     \
+                                 const TaylorParams &, hipStream_t);
+#define PLH_TAYLOR_EXTERN(T)                              \
+    extern template PLH_TAYLOR_SIGNATURE(T, kTaylorFwd)   \
+    extern template PLH_TAYLOR_SIGNATURE(T, kTaylorBwd)   \
+    extern template PLH_TAYLOR_SIGNATURE(T, kTaylorCeFwd) \
+    extern template PLH_TAYLOR_SIGNATURE(T, kTaylorCeBwd)
+#define PLH_TAYLOR_INSTANTIATE(T, K) template PLH_TAYLOR_SIGNATURE(T, K)
 
 }  // namespace plh

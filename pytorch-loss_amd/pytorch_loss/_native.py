@@ -12,6 +12,7 @@ call raises, like the reference's AT_ERROR("... only supports gpu mode")
 """
 import ctypes
 import os
+import threading
 
 import torch
 
@@ -245,11 +246,33 @@ def _pixel_backward(entry, a, ignore_index, param, grad_output):
     return _back_to(grad, a.dtype)
 
 
+# Reduction workspaces (per-block partial sums of a fused 'mean' / 'sum') are kept per (device, stream, thread):
+# a forward writes its partials and its finishing kernel reads them on the same stream, so the next call on that
+# stream may use the same bytes, and a step costs one dictionary look-up where it cost an allocation and a call
+# into the library. Calls under stream capture allocate as before (their memory belongs to the graph's pool).
+_WS_BYTES = {}
+_WS_CACHE = {}
+
+
 def _reduce_workspace(units, device):
-    nbytes = int(load().plh_reduce_workspace_bytes(int(units)))
-    if nbytes < 0:
-        _check(nbytes)
-    return torch.empty((nbytes,), dtype=torch.uint8, device=device), nbytes
+    units = int(units)
+    nbytes = _WS_BYTES.get(units)
+    if nbytes is None:
+        nbytes = int(load().plh_reduce_workspace_bytes(units))
+        if nbytes < 0:
+            _check(nbytes)
+        if len(_WS_BYTES) < 4096:
+            _WS_BYTES[units] = nbytes
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if _raw_stream is None or torch.cuda.is_current_stream_capturing():
+        return torch.empty((nbytes,), dtype=torch.uint8, device=device), nbytes
+    key = (index, _raw_stream(index), threading.get_ident())
+    ws = _WS_CACHE.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if len(_WS_CACHE) >= 64:
+            _WS_CACHE.clear()
+        ws = _WS_CACHE[key] = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+    return ws, nbytes
 
 
 def _scalar_f32(t):
