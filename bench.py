@@ -114,7 +114,7 @@ def algorithmic_bytes(name, shape, dtype="f32"):
     E = numel(shape)
     P = E // shape[1]
     b = ELEM_BYTES[dtype]
-    if name == "ohem":     # forward: logits and labels in, new labels (and one loss) out; backward: logits, new labels, gradient
+    if name == "ohem":     # forward: logits and labels in, the selection (as new labels) and one loss out; backward: logits, labels, gradient
         return b * E + 8 * P + 8 * P, b * E + 8 * P + b * E
     if name in ("lsr", "lmargin", "taylor"):
         fwd = b * E + 8 * P + 4 * P
@@ -358,23 +358,23 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
     out = {}
     if name == "ohem":
         # forward = relabelling + mean cross entropy in one entry point; backward = cross-entropy gradient on the new labels
-        new_labels = torch.empty_like(labels)
+        kept = torch.empty(labels.numel(), dtype=torch.uint8, device=x.device)
         scratch = torch.empty((2, labels.numel()), dtype=torch.float32, device=x.device)
         loss = torch.empty((), dtype=torch.float32, device=x.device)
         n_valid = torch.empty((), dtype=torch.int64, device=x.device)
         grad = torch.empty_like(x)
         ws_bytes = int(lib.plh_ohem_ce_workspace_bytes(labels.numel()))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-        f = lambda: lib.plh_ohem_ce_forward(P(x), tag, P(labels), P(new_labels), P(scratch[0]), P(scratch[1]), P(loss),
-                                            P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.7, labels.numel() // 16, st())
-        b = lambda: lib.plh_lsr_backward_scaled(P(x), tag, P(new_labels), P(loss), 1.0, P(n_valid), P(grad), n, c, m, 255,
-                                                0.0, st())
+        f = lambda: lib.plh_ohem_ce_forward_kept(P(x), tag, P(labels), P(kept), P(scratch[0]), P(scratch[1]), P(loss),
+                                                 P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.7, labels.numel() // 16, st())
+        b = lambda: lib.plh_lsr_backward_kept(P(x), tag, P(labels), P(kept), P(loss), 1.0, P(n_valid), P(grad), n, c, m, 255,
+                                              0.0, st())
         # OhemLargeMarginLoss: the same pipeline behind the large-margin forward kernel, and that loss's gradient
-        fl = lambda: lib.plh_ohem_lmargin_forward(P(x), tag, P(labels), P(new_labels), P(scratch[0]), P(scratch[1]),
-                                                  P(loss), P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.3, 0.7,
-                                                  labels.numel() // 16, st())
-        bl = lambda: lib.plh_lmargin_backward_scaled(P(x), tag, P(new_labels), P(loss), 1.0, P(n_valid), P(grad), n, c, m,
-                                                     255, 0.3, st())
+        fl = lambda: lib.plh_ohem_lmargin_forward_kept(P(x), tag, P(labels), P(kept), P(scratch[0]), P(scratch[1]),
+                                                       P(loss), P(n_valid), P(ws), ws_bytes, n, c, m, 255, 0.3, 0.7,
+                                                       labels.numel() // 16, st())
+        bl = lambda: lib.plh_lmargin_backward_kept(P(x), tag, P(labels), P(kept), P(loss), 1.0, P(n_valid), P(grad), n, c, m,
+                                                   255, 0.3, st())
         assert f() == 0 and b() == 0 and fl() == 0 and bl() == 0
         for key, fn, nbytes in (("forward", f, fwd_bytes), ("backward", b, bwd_bytes),
                                 ("large_margin_forward", fl, fwd_bytes), ("large_margin_backward", bl, bwd_bytes)):

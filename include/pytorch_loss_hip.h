@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define PLH_ABI_VERSION 2
+#define PLH_ABI_VERSION 3
 
 #define PLH_OK 0
 #define PLH_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
@@ -284,6 +284,40 @@ int plh_ohem_lmargin_forward(const void *logits, int32_t dtype, const int64_t *l
                              void *workspace, int64_t workspace_bytes,
                              int64_t n_size, int64_t dimsize, int64_t m_size,
                              int64_t ignore_index, float lam, float score_thresh, int64_t n_min, void *stream);
+
+/* The two forwards above for callers that keep the selection as a mask rather than as new labels (no counterpart in
+ * the reference; what OhemCELoss / OhemLargeMarginLoss of this package call): `kept` receives one byte per pixel,
+ * 1 where the pixel keeps a label other than ignore_index and 0 elsewhere (4-byte aligned, n_size*m_size bytes). The
+ * relabelling pass then neither reads the labels again nor writes new ones (9 instead of 24 bytes per pixel).
+ * plh_lsr_backward_kept (smooth = 0) and plh_lmargin_backward_kept are the matching gradients: plh_*_backward_scaled
+ * on the ORIGINAL labels, with an upstream gradient of 0 for every pixel whose byte in `kept` is 0. Everything else
+ * as for plh_ohem_ce_forward / plh_ohem_lmargin_forward; `scores` holds 2 instead of 1 for pixels without a target.
+ */
+int plh_ohem_ce_forward_kept(const void *logits, int32_t dtype, const int64_t *labels,
+                             uint8_t *kept, float *scores, float *pixel_ce,
+                             float *loss_out, int64_t *n_valid_out,
+                             void *workspace, int64_t workspace_bytes,
+                             int64_t n_size, int64_t dimsize, int64_t m_size,
+                             int64_t ignore_index, float score_thresh, int64_t n_min, void *stream);
+
+int plh_ohem_lmargin_forward_kept(const void *logits, int32_t dtype, const int64_t *labels,
+                                  uint8_t *kept, float *scores, float *pixel_loss,
+                                  float *loss_out, int64_t *n_valid_out,
+                                  void *workspace, int64_t workspace_bytes,
+                                  int64_t n_size, int64_t dimsize, int64_t m_size,
+                                  int64_t ignore_index, float lam, float score_thresh, int64_t n_min, void *stream);
+
+int plh_lsr_backward_kept(const void *logits, int32_t dtype, const int64_t *labels, const uint8_t *kept,
+                          const float *grad_scalar, float scale, const int64_t *divide_by,
+                          void *grad_logits,
+                          int64_t n_size, int64_t dimsize, int64_t m_size,
+                          int64_t ignore_index, float smooth, void *stream);
+
+int plh_lmargin_backward_kept(const void *logits, int32_t dtype, const int64_t *labels, const uint8_t *kept,
+                              const float *grad_scalar, float scale, const int64_t *divide_by,
+                              void *grad_logits,
+                              int64_t n_size, int64_t dimsize, int64_t m_size,
+                              int64_t ignore_index, float lam, void *stream);
 
 /* ---- one-hot / label-smoothed targets -------------------------------------------------
  * Replaces one_hot_cpp.label_one_hot (csrc/one_hot_kernel.cu:265-350).

@@ -24,7 +24,8 @@ static unsigned lmargin_run_typed(int variant, const T *x, const int64_t *lab, c
 // Launches one direction (or the fused pair). blocks_out: blocks that wrote partials (Reduce only).
 static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,
                   int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
-                  int64_t m_size, int64_t ignore, float lam, void *stream, float *scores = nullptr) {
+                  int64_t m_size, int64_t ignore, float lam, void *stream, float *scores = nullptr,
+                  float no_target_score = 1.f) {
     const bool WantLoss = variant != kLmBackward, WantGrad = variant == kLmBackward || variant == kLmForwardBackwardCount;
     const bool WantCount = variant == kLmForwardBackwardCount, Reduce = variant == kLmForwardReduced;
     if (blocks_out) *blocks_out = 0;
@@ -52,6 +53,7 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     p.coeff = 1.f / (float)(dimsize - 1);            // csrc/large_margin_kernel.cu:404
     p.xcd_run = xcd_run_for(es, m_size);
     p.scores = scores;
+    p.no_target_score = no_target_score;
     unsigned blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
@@ -68,10 +70,10 @@ static const Partials kNoPartials{nullptr, nullptr};
 // pixel's score.
 int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
                                 int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
-                                hipStream_t stream) {
+                                hipStream_t stream, float no_target_score) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
     return launch(kLmForward, logits, dtype, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr, n_size, dimsize,
-                  m_size, ignore_index, lam, stream, scores);
+                  m_size, ignore_index, lam, stream, scores, no_target_score);
 }
 
 }  // namespace plh
@@ -124,6 +126,18 @@ extern "C" int plh_lmargin_backward_scaled(const void *logits, int32_t dtype, co
     if (n_size * dimsize * m_size != 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, divide_by, scale};
+    return launch(kLmBackward, logits, dtype, labels, up, nullptr, grad_logits, nullptr, kNoPartials,
+                                             nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
+}
+
+extern "C" int plh_lmargin_backward_kept(const void *logits, int32_t dtype, const int64_t *labels, const uint8_t *kept,
+                                         const float *grad_scalar, float scale, const int64_t *divide_by,
+                                         void *grad_logits,
+                                         int64_t n_size, int64_t dimsize, int64_t m_size,
+                                         int64_t ignore_index, float lam, void *stream) {
+    if (n_size * dimsize * m_size != 0 && (!grad_scalar || !kept)) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale, kept};
     return launch(kLmBackward, logits, dtype, labels, up, nullptr, grad_logits, nullptr, kNoPartials,
                                              nullptr, n_size, dimsize, m_size, ignore_index, lam, stream);
 }

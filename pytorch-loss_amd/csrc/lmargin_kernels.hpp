@@ -25,6 +25,8 @@ struct LmParams {
     float half_lam, coeff;
     unsigned xcd_run;   // tile permutation run length (xcd_run_for)
     float *scores;      // forward kernels: if set, also the softmax probability at the label per pixel
+    float no_target_score;   // what `scores` gets where a pixel has no target (ignored, label out of range): 1, as the
+                             // reference's score pass writes it, or a mark above 1 that the selection tells apart
                         // (1 for a pixel without a target), what the OHEM relabelling ranks
 };
 
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             const float margin = sum_qt - lse_no - p.coeff * (sum_t - others * lse_no);
             const float acc = p.half_lam * margin - (x_y - m_all) + fast_log(s_all);
             out[k] = (ign || !live) ? 0.f : acc;
-            score[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
+            score[k] = (tgt < 0) ? p.no_target_score : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
             // formed here: left to itself the compiler moves a pixel's whole reduction down to the guarded
             // stores at the end and keeps every pixel's exponentials alive until then
             asm volatile("" : "+v"(out[k]), "+v"(score[k]));
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict_
         const float acc = p.half_lam * margin - (st.x_y - m_all) + fast_log(s_all);
         const bool valid = at.live && !ign;
         out[k] = valid ? acc : 0.f;
-        score[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
+        score[k] = (tgt < 0) ? p.no_target_score : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
         mine += out[k];
         cnt += valid ? 1 : 0;
     }
@@ -472,7 +474,7 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
             acc += -(x_y - m_all) + logf(s_all);
             if (live && sub == 0) {
                 if (loss) loss[pix] = ign ? 0.f : acc;
-                if (p.scores) p.scores[pix] = (ign || lb < 0 || lb >= p.C) ? 1.f : fminf(e_y * inv_all, 1.f);
+                if (p.scores) p.scores[pix] = (ign || lb < 0 || lb >= p.C) ? p.no_target_score : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0.f : 1.f;
             }
@@ -624,7 +626,7 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             acc += -(x_y - m_all) + logf(s_all);
             if (lane == 0 && live) {
                 if (loss) loss[row] = ign ? 0.f : acc;
-                if (p.scores) p.scores[row] = (ign || tgt < 0) ? 1.f : fminf(e_y * inv_all, 1.f);
+                if (p.scores) p.scores[row] = (ign || tgt < 0) ? p.no_target_score : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0.f : 1.f;
             }
@@ -753,7 +755,7 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                 const float margin = p.half_lam * ((sum_qx - off) - p.coeff * (st.sx - n_no * off));
                 const float acc = margin - (x_y - m_all) + logf(s_all);
                 if (loss) loss[row] = ign ? 0.f : acc;
-                if (p.scores) p.scores[row] = (ign || tgt < 0) ? 1.f : fminf(e_y * inv_all, 1.f);
+                if (p.scores) p.scores[row] = (ign || tgt < 0) ? p.no_target_score : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0 : 1;
             }

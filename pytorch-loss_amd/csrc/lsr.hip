@@ -1,5 +1,5 @@
 // Label-smoothed softmax cross entropy for gfx950: the C entry points. The kernels live in
-// lsr_kernels.hpp and are compiled once per element type (lsr_f32.hip, lsr_f16.hip, lsr_bf16.hip).
+// lsr_kernels.hpp and are compiled per element type and direction (lsr_f32_fwd.hip, lsr_f32_bwd.hip, ...).
 #include <mutex>
 
 #include "lsr_kernels.hpp"
@@ -138,5 +138,16 @@ extern "C" int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const 
     if (n_size * dimsize * m_size != 0 && !grad_scalar) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, divide_by, scale};
+    return backward(logits, dtype, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream);
+}
+
+extern "C" int plh_lsr_backward_kept(const void *logits, int32_t dtype, const int64_t *labels, const uint8_t *kept,
+                                     const float *grad_scalar, float scale, const int64_t *divide_by,
+                                     void *grad_logits,
+                                     int64_t n_size, int64_t dimsize, int64_t m_size,
+                                     int64_t ignore_index, float smooth, void *stream) {
+    if (n_size * dimsize * m_size != 0 && (!grad_scalar || !kept)) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale, kept};
     return backward(logits, dtype, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream);
 }

@@ -35,12 +35,18 @@ __device__ __forceinline__ uint32_t score_key(float s) {
 __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)((key >> (20 - 10 * pass)) & 1023u); }
 
 // ------------------------------------------------------------------ scores ----
+// `none` is what a pixel without a target (ignored, or a label outside [0, C)) scores: 1, as the reference
+// writes it (csrc/ohem_label_kernel.cu:131-134), or kNoTargetMark for the forwards that hand their selection
+// on as a mask and have to tell such a pixel from a valid one that scores exactly 1 without reading the labels
+// again. Both sort last (score_key clamps at 1) and tie with each other in pixel order.
+constexpr float kNoTargetMark = 2.f;
+
 
 template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                               float *__restrict__ scores, float *__restrict__ ce,
                                                               int64_t P, int64_t m_size, int C, int64_t ignore,
-                                                              unsigned xcd_run, uint32_t *__restrict__ tables) {
+                                                              unsigned xcd_run, uint32_t *__restrict__ tables, float none) {
     // the selection's tables start at zero; the kernels that fill them are launched after this one
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kRegsBlock) tables[i] = 0;
@@ -70,7 +76,7 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
             }
         // ignored pixels score 1 (ohem_label_kernel.cu:131-134); so does a label outside [0, C),
         // which the reference leaves undefined
-        out[k] = (tgt < 0) ? 1.f : fminf(e_y * __builtin_amdgcn_rcpf(s), 1.f);
+        out[k] = (tgt < 0) ? none : fminf(e_y * __builtin_amdgcn_rcpf(s), 1.f);
         // the pixel's cross entropy from the same sums, exact also where the score underflows
         loss[k] = (tgt < 0) ? 0.f : __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, mx - x_y);
     }
@@ -85,7 +91,7 @@ template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 float *__restrict__ scores, float *__restrict__ ce,
                                                                 int64_t P, int64_t m_size, int C, int64_t ignore,
-                                                                unsigned xcd_run, uint32_t *__restrict__ tables) {
+                                                                unsigned xcd_run, uint32_t *__restrict__ tables, float none) {
     __shared__ float parts[3][kSplitWaves][kWave * V];
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kSplitBlock) tables[i] = 0;
@@ -133,7 +139,7 @@ __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__rest
             S = __builtin_fmaf(parts[1][w][q], fast_exp(parts[0][w][q] - M), S);
             x_y = fmaxf(x_y, parts[2][w][q]);
         }
-        out[k] = (tgt < 0) ? 1.f : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
+        out[k] = (tgt < 0) ? none : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
         loss[k] = (tgt < 0) ? 0.f : fast_log(S) + (M - x_y);
     }
     at.template store_f32<true>(scores, out);
@@ -145,13 +151,13 @@ template <class T>
 __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         float *__restrict__ scores, float *__restrict__ ce, int64_t P,
                                                         int64_t m_size, int C, int64_t ignore,
-                                                        uint32_t *__restrict__ tables) {
+                                                        uint32_t *__restrict__ tables, float none) {
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += 256) tables[i] = 0;
     for (int64_t pix = (int64_t)blockIdx.x * 256 + threadIdx.x; pix < P; pix += (int64_t)gridDim.x * 256) {
         const int64_t lb = lab[pix];
         if (lb == ignore || lb < 0 || lb >= C) {
-            scores[pix] = 1.f;
+            scores[pix] = none;
             if (ce) ce[pix] = 0.f;
             continue;
         }
@@ -174,7 +180,7 @@ __global__ __launch_bounds__(256) void ohem_scores_lane(const T *__restrict__ x,
 template <class T, int NI, int LP, int G>
 __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         float *__restrict__ scores, float *__restrict__ ce, int64_t P,
-                                                        int C, int64_t ignore, uint32_t *__restrict__ tables) {
+                                                        int C, int64_t ignore, uint32_t *__restrict__ tables, float none) {
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += 256) tables[i] = 0;
     constexpr int L = WaveRow<T, NI, LP, G>::L;
@@ -187,7 +193,7 @@ __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x,
         if constexpr (G == 64) {                              // the wavefront has one row: skip its loads
             if (no_target) {
                 if (at.sub == 0) {
-                    scores[row] = 1.f;
+                    scores[row] = none;
                     if (ce) ce[row] = 0.f;
                 }
                 continue;
@@ -205,7 +211,7 @@ __global__ __launch_bounds__(256) void ohem_scores_wrow(const T *__restrict__ x,
         s = group_reduce<G>(s, OpSum());
         if (at.sub == 0 && live) {
             const float x_y = load_one(xs + (no_target ? 0 : lb));
-            scores[row] = no_target ? 1.f : fminf(fast_exp(x_y - mx) / s, 1.f);
+            scores[row] = no_target ? none : fminf(fast_exp(x_y - mx) / s, 1.f);
             if (ce) ce[row] = no_target ? 0.f : logf(s) + (mx - x_y);
         }
     }
@@ -217,7 +223,7 @@ template <class T>
 __global__ __launch_bounds__(kRowBlock) void ohem_scores_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                              float *__restrict__ scores, float *__restrict__ ce,
                                                              int64_t P, int C, int64_t ignore,
-                                                             uint32_t *__restrict__ tables, int vec) {
+                                                             uint32_t *__restrict__ tables, int vec, float none) {
     __shared__ float red[kRowBlock / 64];
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += row_threads()) tables[i] = 0;
@@ -225,7 +231,7 @@ __global__ __launch_bounds__(kRowBlock) void ohem_scores_row(const T *__restrict
         const int64_t lb = lab[row];
         if (lb == ignore || lb < 0 || lb >= C) {
             if (threadIdx.x == 0) {
-                scores[row] = 1.f;
+                scores[row] = none;
                 if (ce) ce[row] = 0.f;
             }
             continue;
@@ -423,10 +429,13 @@ __global__ __launch_bounds__(256) void ohem_ties(const float *__restrict__ score
 // With `part`, the block also leaves the sum of `ce` over the pixels that keep a label other than
 // `ignore`, and their number: the mean cross entropy of the relabelled batch needs no further pass
 // over the logits.
+// With `kept`, the labels are neither read nor written: the kernel leaves one byte per pixel instead, 1 where
+// the pixel keeps a label other than `ignore` (pixels without a target carry kNoTargetMark as their score).
 __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ scores, const int64_t *__restrict__ lab,
                                                     int64_t *__restrict__ out, OhemTables tb, int P, int tiles, uint32_t n_min,
                                                     float thresh, int64_t ignore, int vec,
-                                                    const float *__restrict__ ce, Partials part) {
+                                                    const float *__restrict__ ce, Partials part,
+                                                    uint8_t *__restrict__ kept_out) {
     __shared__ uint32_t wave_ties[4], run_ties[4];
     __shared__ float red[4];
     const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
@@ -476,7 +485,18 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
         }
     }
     bool kept[4] = {false, false, false, false};
-    if (vec && base + 3 < P) {
+    if (kept_out) {                                     // uniform over the grid
+#pragma unroll
+        for (int k = 0; k < 4; ++k) kept[k] = base + k < P && !drop[k] && !(s[k] > 1.5f);
+        if (base + 3 < P) {
+            *reinterpret_cast<uint32_t *>(kept_out + base) =
+                (uint32_t)kept[0] | ((uint32_t)kept[1] << 8) | ((uint32_t)kept[2] << 16) | ((uint32_t)kept[3] << 24);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (base + k < P) kept_out[base + k] = kept[k] ? 1 : 0;
+        }
+    } else if (vec && base + 3 < P) {
         const plh_l2 *in2 = reinterpret_cast<const plh_l2 *>(lab + base);
         plh_l2 *out2 = reinterpret_cast<plh_l2 *>(out + base);
         plh_l2 a = __builtin_nontemporal_load(in2), b = __builtin_nontemporal_load(in2 + 1);
@@ -524,7 +544,7 @@ static int64_t ohem_tiles(int64_t P) { return ceil_div(P > 0 ? P : 1, kOhemTile)
 
 static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, float *ce,
                          int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st,
-                         uint32_t *tables = nullptr) {
+                         uint32_t *tables = nullptr, float none = 1.f) {
     const int64_t P = n_size * m_size;
     const int C = (int)dimsize;
     dispatch_dtype(dtype, [&](auto tag) {
@@ -541,7 +561,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         hipLaunchKernelGGL((ohem_scores_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, ce, \
-                           P, m_size, C, ignore_index, run, tables);                                                  \
+                           P, m_size, C, ignore_index, run, tables, none);                                                  \
         break;
                 PLH_SPLIT_DEEP_CASES
 #undef PLH_CASE
@@ -553,7 +573,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         hipLaunchKernelGGL((ohem_scores_split<T, KW, VT, true>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, \
-                           ce, P, m_size, C, ignore_index, run, tables);                                              \
+                           ce, P, m_size, C, ignore_index, run, tables, none);                                              \
         break;
                 PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
@@ -565,7 +585,7 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         hipLaunchKernelGGL((ohem_scores_split<T, KW, VT>), dim3(grid), dim3(kSplitBlock), 0, st, x, labels, scores, ce, \
-                           P, m_size, C, ignore_index, run, tables);                                                  \
+                           P, m_size, C, ignore_index, run, tables, none);                                                  \
         break;
                 PLH_SPLIT_SLOT_CASES
 #undef PLH_CASE
@@ -581,15 +601,15 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
         if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kUniform>), dim3(grid), dim3(kRegsBlock), 0, st,  \
-                                    x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);                  \
+                                    x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                  \
         else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, \
-                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);         \
+                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);         \
         else if (image) {                                                                                             \
             if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                          \
                 hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st,   \
-                                   x, labels, scores, ce, P, m_size, C, ignore_index, run, tables);                   \
+                                   x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                   \
         } else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x,  \
-                                  labels, scores, ce, P, m_size, C, ignore_index, run, tables);                       \
+                                  labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                       \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -597,16 +617,16 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
         } else if (shape == Shape::Wave && C <= wrow_cap<T>(wrow_piece<T>(x, (const T *)nullptr, C))) {
 #define PLH_GO(NI, W, G)                                                                                            \
     hipLaunchKernelGGL((ohem_scores_wrow<T, NI, W, G>), dim3(group_grid(P, WaveRowAt<G>::kRowsPerBlock)), dim3(256), 0, \
-                       st, x, labels, scores, ce, P, C, ignore_index, tables)
+                       st, x, labels, scores, ce, P, C, ignore_index, tables, none)
             PLH_WROW_DISPATCH(wrow_piece<T>(x, (const T *)nullptr, C), C, PLH_GO);
 #undef PLH_GO
         } else if (shape == Shape::Wave) {
             const unsigned grid = (unsigned)(P < 1 ? 1 : (P < kMinPartialSlots ? P : kMinPartialSlots));
             hipLaunchKernelGGL(ohem_scores_row<T>, dim3(grid), dim3(row_threads_for_sweep<T>(C)), 0, st, x, labels, scores, ce, P, C,
-                               ignore_index, tables, row_chunks_ok<T>(x, nullptr, C));
+                               ignore_index, tables, row_chunks_ok<T>(x, nullptr, C), none);
         } else {
             hipLaunchKernelGGL(ohem_scores_lane<T>, dim3(group_grid(P, 256)), dim3(256), 0, st, x, labels, scores, ce, P,
-                               m_size, C, ignore_index, tables);
+                               m_size, C, ignore_index, tables, none);
         }
     });
     return check_launch();
@@ -626,7 +646,7 @@ static int check_workspace(const void *workspace, int64_t workspace_bytes, int64
 static int launch_select(const float *scores, const int64_t *labels, int64_t *out_labels, void *workspace,
                          int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st,
                          const float *ce = nullptr, Partials part = Partials{nullptr, nullptr},
-                         bool tables_zeroed = false) {
+                         bool tables_zeroed = false, uint8_t *kept_out = nullptr) {
     if (n_min >= P && part.sum) {                // nothing is relabelled, the loss is still wanted
         n_min = 0;
         score_thresh = INFINITY;
@@ -645,7 +665,7 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
     const uint32_t k = n_min > 0 ? (uint32_t)n_min : 0u;
     const int Pi = (int)P;
     // 16-byte accesses when every tensor allows them (tile bases are multiples of 4 pixels)
-    const int vec = !misaligned(scores, 16) && !misaligned(labels, 16) && !misaligned(out_labels, 16);
+    const int vec = !misaligned(scores, 16) && (kept_out || (!misaligned(labels, 16) && !misaligned(out_labels, 16)));
     if (k > 0) {
         if (!tables_zeroed)     // the score kernel of the one-call entry points has done it
             hipLaunchKernelGGL(ohem_zero, dim3((kOhemZeroWords + 255) / 256), dim3(256), 0, st, tb.hist, kOhemZeroWords);
@@ -657,7 +677,7 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         hipLaunchKernelGGL(ohem_ties, dim3(kTieRuns / 4), dim3(256), 0, st, scores, tb, Pi, (int)tiles, k, score_thresh, vec);
     }
     hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, (int)tiles, k,
-                       score_thresh, ignore_index, vec, ce, part);
+                       score_thresh, ignore_index, vec, ce, part, kept_out);
     return check_launch();
 }
 
@@ -724,13 +744,17 @@ extern "C" int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels) {
 // The one-call forwards: scores and per-pixel loss in one pass over the logits (cross entropy: the
 // score kernel itself; large margin: that loss's forward kernel, which then also leaves the scores),
 // relabelling that adds up the kept pixels' losses, fixed-order finish.
+// With `kept` (and no out_labels) the selection leaves the byte mask that plh_lsr_backward_kept and
+// plh_lmargin_backward_kept read, instead of relabelled labels: the relabelling pass then neither reads the
+// labels nor writes new ones.
 static int ohem_loss_forward(bool large_margin, float lam, const void *logits, int32_t dtype, const int64_t *labels,
                              int64_t *out_labels, float *scores, float *pixel_loss, float *loss_out,
                              int64_t *n_valid_out, void *workspace, int64_t workspace_bytes, int64_t n_size,
                              int64_t dimsize, int64_t m_size, int64_t ignore_index, float score_thresh, int64_t n_min,
-                             void *stream) {
+                             void *stream, uint8_t *kept = nullptr) {
     if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
-    int rc = check_slice_args(logits, labels, out_labels, n_size, dimsize, m_size, dtype_size(dtype), 8);
+    int rc = kept ? check_slice_args(logits, labels, kept, n_size, dimsize, m_size, dtype_size(dtype), 4)
+                  : check_slice_args(logits, labels, out_labels, n_size, dimsize, m_size, dtype_size(dtype), 8);
     if (rc != PLH_OK) return rc;
     if (n_size * m_size > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
     if (!loss_out) return PLH_ERR_NULL_POINTER;
@@ -749,15 +773,16 @@ static int ohem_loss_forward(bool large_margin, float lam, const void *logits, i
     Partials part;
     part.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P));
     part.cnt = reinterpret_cast<int *>(part.sum + tiles);
+    const float none = kept ? kNoTargetMark : 1.f;
     if (large_margin)
         rc = lmargin_forward_with_scores(logits, dtype, labels, pixel_loss, scores, n_size, dimsize, m_size, ignore_index,
-                                         lam, st);
+                                         lam, st, none);
     else
         rc = launch_scores(logits, dtype, labels, scores, pixel_loss, n_size, dimsize, m_size, ignore_index, st,
-                           static_cast<uint32_t *>(workspace));
+                           static_cast<uint32_t *>(workspace), none);
     if (rc != PLH_OK) return rc;
     rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_loss, part,
-                       /*tables_zeroed=*/!large_margin);
+                       /*tables_zeroed=*/!large_margin, kept);
     if (rc != PLH_OK) return rc;
     finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
     return check_launch();
@@ -779,4 +804,26 @@ extern "C" int plh_ohem_lmargin_forward(const void *logits, int32_t dtype, const
                                         float lam, float score_thresh, int64_t n_min, void *stream) {
     return ohem_loss_forward(true, lam, logits, dtype, labels, out_labels, scores, pixel_loss, loss_out, n_valid_out,
                              workspace, workspace_bytes, n_size, dimsize, m_size, ignore_index, score_thresh, n_min, stream);
+}
+
+extern "C" int plh_ohem_ce_forward_kept(const void *logits, int32_t dtype, const int64_t *labels, uint8_t *kept,
+                                        float *scores, float *pixel_ce, float *loss_out, int64_t *n_valid_out,
+                                        void *workspace, int64_t workspace_bytes,
+                                        int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                        float score_thresh, int64_t n_min, void *stream) {
+    if (!kept && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
+    return ohem_loss_forward(false, 0.f, logits, dtype, labels, nullptr, scores, pixel_ce, loss_out, n_valid_out,
+                             workspace, workspace_bytes, n_size, dimsize, m_size, ignore_index, score_thresh, n_min, stream,
+                             kept);
+}
+
+extern "C" int plh_ohem_lmargin_forward_kept(const void *logits, int32_t dtype, const int64_t *labels, uint8_t *kept,
+                                             float *scores, float *pixel_loss, float *loss_out, int64_t *n_valid_out,
+                                             void *workspace, int64_t workspace_bytes,
+                                             int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index,
+                                             float lam, float score_thresh, int64_t n_min, void *stream) {
+    if (!kept && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
+    return ohem_loss_forward(true, lam, logits, dtype, labels, nullptr, scores, pixel_loss, loss_out, n_valid_out,
+                             workspace, workspace_bytes, n_size, dimsize, m_size, ignore_index, score_thresh, n_min, stream,
+                             kept);
 }

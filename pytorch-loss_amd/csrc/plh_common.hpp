@@ -476,10 +476,13 @@ struct Upstream {
     int64_t stride;             // 0 = one scalar, 1 = per loss element
     const int64_t *divide_by;   // nullptr = 1; device-resident count (e.g. the valid pixels of a 'mean')
     float scale;                // host-side factor
+    const uint8_t *keep;        // nullptr = every pixel; else one byte per pixel, 0 = the pixel takes no part (its
+                                // upstream gradient is 0): how the hard-example losses hand their selection on
 };
 
+// `have` = how many of the V pixels from i on exist (the per-image form's last lane of an image has fewer).
 template <int V>
-__device__ __forceinline__ void load_upstream(const Upstream &up, int64_t i, float (&out)[V]) {
+__device__ __forceinline__ void load_upstream(const Upstream &up, int64_t i, float (&out)[V], int have = V) {
     if (up.gout != nullptr && up.stride != 0) {
         load_vec<V>(up.gout + i, out);
         return;
@@ -488,6 +491,11 @@ __device__ __forceinline__ void load_upstream(const Upstream &up, int64_t i, flo
     if (up.divide_by) g = g / (float)(*up.divide_by);
 #pragma unroll
     for (int k = 0; k < V; ++k) out[k] = g;
+    if (up.keep) {                  // uniform
+#pragma unroll
+        for (int k = 0; k < V; ++k)
+            if (k < have && up.keep[i + k] == 0) out[k] = 0.f;
+    }
 }
 
 // ---- two-stage deterministic reduction of the losses ------------------------------
@@ -528,7 +536,7 @@ void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int
 // its label (1 where there is no target) into `scores`.
 int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
                                 int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
-                                hipStream_t stream);
+                                hipStream_t stream, float no_target_score = 1.f);
 
 // ---- the "regs" launch shape ---------------------------------------------------
 // 256 threads per block, V pixels per thread; block b of the grid owns the pixel tile
@@ -741,7 +749,7 @@ struct PixelRef {
                 return;
             }
         }
-        load_upstream<V>(up, pix, go);
+        load_upstream<V>(up, pix, go, nv);
     }
 
     // A wavefront's tile holds 64 rows of the kernel's channel count, skewed: 5.3 KB for 20 fp32 channels rather than
@@ -1111,7 +1119,7 @@ struct SplitSlice {
                 return;
             }
         }
-        load_upstream<V>(up, pix, go);
+        load_upstream<V>(up, pix, go, nv);
     }
 };
 

@@ -41,25 +41,32 @@ __device__ constexpr InvFactorials kInvFact{};
 
 // f of order n (>= 2) and, as a by-product, of order n-1 (its derivative). The orders in common use
 // (2, the modules' default, and 4; `order` is uniform, so the branch is scalar) are evaluated in nested form.
-// The kernels that keep a slice or a row in registers are compiled for these two orders only (taylor_pair24):
-// every evaluation is inlined into their unrolled sweeps, and a third, general form there made up a third of
-// the library's code for orders nobody trains with; higher orders take the kernels that walk the slice
+// The kernels that keep a slice or a row in registers are compiled for these two orders only (taylor_pair24, the
+// order a compile-time constant of a body that is chosen once per launch): every evaluation is inlined into their
+// unrolled sweeps, and a third, general form there made up a third of the library's code for orders nobody trains
+// with; higher orders take the kernels that walk the slice
 // (taylor_group, the block-per-row forms), which evaluate term by term upwards like the reference's
 // recurrence (csrc/taylor_softmax.cu:24-33).
-__device__ __forceinline__ void taylor_pair24(float x, int order, float &f, float &df) {
-    if (order == 2) {
+template <int ORD>
+__device__ __forceinline__ void taylor_pair24(float x, float &f, float &df) {
+    static_assert(ORD == 2 || ORD == 4, "the register-resident kernels are compiled for orders 2 and 4");
+    if constexpr (ORD == 2) {
         df = 1.f + x;
         f = __builtin_fmaf(x * x, 0.5f, df);
-        return;
+    } else {
+        const float x2 = x * x;
+        df = __builtin_fmaf(x, __builtin_fmaf(x, __builtin_fmaf(x, 1.f / 6.f, 0.5f), 1.f), 1.f);
+        f = __builtin_fmaf(x2 * x2, 1.f / 24.f, df);
     }
-    const float x2 = x * x;
-    df = __builtin_fmaf(x, __builtin_fmaf(x, __builtin_fmaf(x, 1.f / 6.f, 0.5f), 1.f), 1.f);
-    f = __builtin_fmaf(x2 * x2, 1.f / 24.f, df);
 }
 
 __device__ __forceinline__ void taylor_pair(float x, int order, float &f, float &df) {
-    if (order <= 4) {
-        taylor_pair24(x, order, f, df);
+    if (order == 2) {
+        taylor_pair24<2>(x, f, df);
+        return;
+    }
+    if (order == 4) {
+        taylor_pair24<4>(x, f, df);
         return;
     }
     float res = 1.f + x, prev = 1.f, mid = x;
@@ -77,6 +84,10 @@ __device__ __forceinline__ void taylor_pair(float x, int order, float &f, float 
 template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restrict__ x, T *__restrict__ out,
                                                              const TaylorParams p) {
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
@@ -95,7 +106,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, p.C)) {
                     float f, df;
-                    taylor_pair24(PK::get(raw[j], k), p.order, f, df);
+                    taylor_pair24<ORD>(PK::get(raw[j], k), f, df);
                     y[j][kk] = f;
                     s += f;
                 }
@@ -109,11 +120,18 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
             if (chan_ok<CP>(j, p.C)) PK::set(raw[j], k0 / PK::kStep, y[j]);
     }
     at.store_slice(out, p.C, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restrict__ g, const T *__restrict__ x,
                                                              T *__restrict__ gx, const TaylorParams p) {
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP], graw[CP];
@@ -129,7 +147,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
                 s += f;
                 dot += p.use_log ? gj : f * gj;
@@ -150,7 +168,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
                 r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
             }
@@ -158,6 +176,9 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
             forget_origin(raw[j]);      // packed here, channel by channel: nothing of the sweep waits for the stores
         }
     at.store_slice(gx, p.C, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 // Cross entropy on the log form: loss per pixel (fp32), and its gradient with the upstream folded in.
@@ -167,6 +188,10 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
                                                                 const TaylorParams p) {
     const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!Reduce && !at.live) return;
     // labels (and the upstream gradient) first: in the rows form the slice arrives through LDS behind a wait
@@ -186,7 +211,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 s += f;
                 f_y = (tgt == j) ? f : f_y;
             }
@@ -204,12 +229,19 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
             part.cnt[blockIdx.x] = (int)bc;
         }
     }
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                                 const Upstream up, T *__restrict__ gx,
                                                                 const TaylorParams p) {
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     // labels and the upstream gradient before the slice, except in the one-pixel-per-lane form on 16-bit elements
@@ -242,7 +274,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
         for (int j = 0; j < CP; ++j)
             if (chan_ok<CP>(j, p.C)) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 s += f;
                 f_y = (tgt[k] == j) ? f : f_y;
             }
@@ -261,13 +293,16 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_bwd_regs(const T *__rest
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[j], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 r[k] = df * ((tgt[k] == j) ? hot[k] : scale[k]);
             }
             raw[j] = Pack<T, V>::put(r) & mask;
             forget_origin(raw[j]);      // packed here, channel by channel: nothing of the sweep waits for the stores
         }
     at.store_slice(gx, p.C, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 // --------------------------------------------------------------- split ----
@@ -280,6 +315,10 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
                                                                   const TaylorParams p) {
     const bool Reduce = part.sum != nullptr;
     __shared__ float parts[2][kSplitWaves][kWave * V];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     int64_t lb[V];
@@ -295,7 +334,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[i], k), f, df);
                 s += (i < at.here) ? f : 0.f;
                 f_y = (rel == i) ? f : f_y;
             }
@@ -332,6 +371,9 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
             part.cnt[blockIdx.x] = (int)bc;
         }
     }
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 template <class T, int KW, int V, bool PerImage = false>
@@ -339,6 +381,10 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
                                                                   const Upstream up, T *__restrict__ gx,
                                                                   const TaylorParams p) {
     __shared__ float parts[2][kSplitWaves][kWave * V];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     typename Pack<T, V>::Raw raw[KW];
@@ -360,7 +406,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
+                taylor_pair24<ORD>(Pack<T, V>::get(raw[i], k), f, df);
                 s += (i < at.here) ? f : 0.f;
                 f_y = (rel[k] == i) ? f : f_y;
             }
@@ -392,12 +438,15 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_bwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair24(Pack<T, V>::get(raw[i], k), p.order, f, df);
+            taylor_pair24<ORD>(Pack<T, V>::get(raw[i], k), f, df);
             r[k] = df * ((rel[k] == i) ? hot[k] : scale[k]);
         }
         raw[i] = Pack<T, V>::put(r) & mask;
     }
     at.store(gx, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 // The softmax / log-softmax themselves for 33..256 channels in NCHW (SplitSlice): the parts of a pixel are each
@@ -407,6 +456,10 @@ template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__restrict__ x, T *__restrict__ out,
                                                                   const TaylorParams p) {
     __shared__ float parts[kSplitWaves][kWave * V];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
@@ -419,7 +472,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair24(PK::get(raw[i], k), p.order, f, df);
+                taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
                 s += (i < at.here) ? f : 0.f;
             }
             parts[wave][lane * V + k] = s;
@@ -444,18 +497,25 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair24(PK::get(raw[i], k), p.order, f, df);
+            taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
             r[k] = p.use_log ? logf(f) - ls[k] : f * inv[k];
         }
         raw[i] = PK::put(r);
     }
     at.store(out, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 template <class T, int KW, int V, bool PerImage = false>
 __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__restrict__ g, const T *__restrict__ x,
                                                                   T *__restrict__ gx, const TaylorParams p) {
     __shared__ float parts[2][kSplitWaves][kWave * V];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
@@ -469,7 +529,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
 #pragma unroll
             for (int i = 0; i < KW; ++i) {
                 float f, df;
-                taylor_pair24(PK::get(raw[i], k), p.order, f, df);
+                taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
                 const float gj = PK::get(graw[i], k);
                 s += (i < at.here) ? f : 0.f;
                 dot += (i < at.here) ? (p.use_log ? gj : f * gj) : 0.f;
@@ -503,13 +563,16 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
 #pragma unroll
         for (int k = 0; k < V; ++k) {
             float f, df;
-            taylor_pair24(PK::get(raw[i], k), p.order, f, df);
+            taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
             const float gj = PK::get(graw[i], k);
             r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
         }
         raw[i] = PK::put(r);
     }
     at.store(gx, p.m_size, raw);
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 // --------------------------------------------------------------- group ----
@@ -622,6 +685,10 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                                                    const TaylorParams p) {
     const bool Reduce = part.sum != nullptr;
     __shared__ float red[4];
+    // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
+    // evaluation of the series carries a test of its own
+    auto run = [&](auto order_tag) {
+    constexpr int ORD = decltype(order_tag)::value;
     constexpr int L = WaveRow<T, NI, LP, G>::L;
     using Span = WaveRowSpan<T, L, G, NI>;
     T *tile = Span::tile();
@@ -643,7 +710,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
 #pragma unroll
             for (int l = 0; l < L; ++l) {
                 float f, df;
-                taylor_pair24(r.v[i][l], p.order, f, df);
+                taylor_pair24<ORD>(r.v[i][l], f, df);
                 s += ok ? f : 0.f;
                 if constexpr (Kind == kTaylorBwd) {
                     const float gj = rg.v[i][l];
@@ -659,7 +726,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 const int64_t lb = lab[row];
                 const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
                 float f_y = 1.f, df;
-                if (has_y) taylor_pair24(load_one(xs + lb), p.order, f_y, df);
+                if (has_y) taylor_pair24<ORD>(load_one(xs + lb), f_y, df);
                 const float v = has_y ? logf(s) - logf(f_y) : 0.f;
                 if (loss) loss[row] = v;
                 mine += v;
@@ -677,7 +744,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 if (lb != p.ignore && lb >= 0 && lb < p.C) {
                     tgt = (int)lb;
                     float f_y, df_y;
-                    taylor_pair24(load_one(xs + lb), p.order, f_y, df_y);
+                    taylor_pair24<ORD>(load_one(xs + lb), f_y, df_y);
                     cold = inv * go[0];
                     hot = cold - go[0] / f_y;
                 }
@@ -689,7 +756,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
 #pragma unroll
                 for (int l = 0; l < L; ++l) {
                     float f, df;
-                    taylor_pair24(r.v[i][l], p.order, f, df);
+                    taylor_pair24<ORD>(r.v[i][l], f, df);
                     if constexpr (Kind == kTaylorFwd) {
                         o[l] = p.use_log ? logf(f) - ls : f * inv;
                     } else if constexpr (Kind == kTaylorBwd) {
@@ -718,6 +785,9 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
             part.cnt[blockIdx.x] = (int)bc;
         }
     }
+    };
+    if (p.order == 2) run(std::integral_constant<int, 2>());
+    else run(std::integral_constant<int, 4>());
 }
 
 // ------------------------------------------------------- a block per row ----

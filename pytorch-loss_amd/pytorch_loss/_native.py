@@ -18,7 +18,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpytorch_loss_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -60,6 +60,12 @@ _SIGNATURES = {
                                            _p]),
     "plh_ohem_lmargin_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32,
                                                 _f32, _i64, _p]),
+    "plh_ohem_ce_forward_kept": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f32,
+                                                _i64, _p]),
+    "plh_ohem_lmargin_forward_kept": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
+                                                     _f32, _f32, _i64, _p]),
+    "plh_lsr_backward_kept": (ctypes.c_int, [_p, _i32, _p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward_kept": (ctypes.c_int, [_p, _i32, _p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_taylor_softmax_forward": (ctypes.c_int, [_p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
@@ -529,28 +535,41 @@ def ohem_score_label(logits, labels, ignore_index, score_thresh, n_min):
 
 
 def ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min, lam=None):
-    """Relabelling and mean loss of what is left, with one pass over the logits: cross entropy, or
+    """Selection of the hard pixels and mean loss over them, with one pass over the logits: cross entropy, or
     the large-margin loss when `lam` is given.
-    -> (loss 0-dim, n_valid 0-dim int64, args whose labels are the NEW labels, for the backward)."""
+    -> (loss 0-dim, n_valid 0-dim int64, args, kept: one byte per pixel, 1 where the pixel takes part)."""
     a = ohem_args(logits, labels)
     dev = a.x.device
     n_pixels = a.n * a.m
     loss = torch.empty((), dtype=torch.float32, device=dev)
     n_valid = torch.empty((), dtype=torch.int64, device=dev)
-    new_labels = torch.empty_like(a.lb)
+    kept = torch.empty((max(n_pixels, 1),), dtype=torch.uint8, device=dev)
     scratch = torch.empty((2, max(n_pixels, 1)), dtype=torch.float32, device=dev)
     nbytes = int(load().plh_ohem_ce_workspace_bytes(n_pixels))
     if nbytes < 0:
         _check(nbytes)
     ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev)
-    head = (_ptr(a.x), a.tag, _ptr(a.lb), _ptr(new_labels), _ptr(scratch[0]), _ptr(scratch[1]), _ptr(loss), _ptr(n_valid),
+    head = (_ptr(a.x), a.tag, _ptr(a.lb), _ptr(kept), _ptr(scratch[0]), _ptr(scratch[1]), _ptr(loss), _ptr(n_valid),
             _ptr(ws), nbytes, a.n, a.c, a.m, int(ignore_index))
     if lam is None:
-        _call(a.x, "plh_ohem_ce_forward", *head, float(score_thresh), int(n_min))
+        _call(a.x, "plh_ohem_ce_forward_kept", *head, float(score_thresh), int(n_min))
     else:
-        _call(a.x, "plh_ohem_lmargin_forward", *head, float(lam), float(score_thresh), int(n_min))
-    a.lb = new_labels
-    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, a
+        _call(a.x, "plh_ohem_lmargin_forward_kept", *head, float(lam), float(score_thresh), int(n_min))
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, a, kept
+
+
+def ohem_backward(args, kept, ignore_index, grad_scalar, n_valid, lam=None):
+    """Gradient of the mean loss over the kept pixels: the cross-entropy (label smoothing 0) or large-margin
+    backward on the original labels, pixels whose byte in `kept` is 0 taking no part."""
+    a = args
+    grad = torch.empty_like(a.x)
+    if a.x.numel() == 0:
+        return _back_to(grad, a.dtype)
+    go = _scalar_f32(grad_scalar)
+    entry, param = ("plh_lsr_backward_kept", 0.0) if lam is None else ("plh_lmargin_backward_kept", float(lam))
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(kept), _ptr(go), 1.0, _ptr(n_valid), _ptr(grad), a.n, a.c, a.m,
+          int(ignore_index), param)
+    return _back_to(grad, a.dtype)
 
 
 # --------------------------------------------------------------- taylor ----

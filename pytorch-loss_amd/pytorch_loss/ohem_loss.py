@@ -5,8 +5,9 @@ easy pixels as ignored (``score_ohem_label``: beyond the ``n_min`` lowest-scorin
 pixel whose softmax probability at its label exceeds ``score_thresh`` gets ``ignore_index``),
 then take the mean loss over what is left.  ``OhemCELoss`` uses plain cross entropy (the reference calls
 ``nn.CrossEntropyLoss(ignore_index, reduction='mean')``, ohem_loss.py:20): the relabelling pass over
-the logits already has every pixel's cross entropy at hand, so the forward is that one pass, and
-the backward is the label-smoothed kernel with a smoothing factor of 0 on the new labels;
+the logits already has every pixel's cross entropy at hand, so the forward is that one pass (it keeps the
+selection as one byte per pixel instead of writing new labels), and the backward is the label-smoothed kernel
+with a smoothing factor of 0 on the original labels and that mask;
 ``OhemLargeMarginLoss`` uses ``LargeMarginSoftmaxV3`` (ohem_loss.py:33-45), whose forward kernel
 holds every pixel's softmax and so leaves the scores as well: again one pass over the logits.
 """
@@ -30,17 +31,14 @@ class _OhemLossFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, logits, labels, ignore_index, score_thresh, n_min, lam):
-        loss, n_valid, args = _native.ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min, lam)
-        ctx.vars = args, n_valid, ignore_index, lam
+        loss, n_valid, args, kept = _native.ohem_ce_forward(logits, labels, ignore_index, score_thresh, n_min, lam)
+        ctx.vars = args, kept, n_valid, ignore_index, lam
         return loss
 
     @staticmethod
     def backward(ctx, grad_output):
-        args, n_valid, ignore_index, lam = ctx.vars
-        if lam is None:
-            grad = _native.lsr_backward_scaled(None, None, ignore_index, 0.0, grad_output, n_valid, args=args)
-        else:
-            grad = _native.lmargin_backward_scaled(None, None, lam, ignore_index, grad_output, n_valid, args=args)
+        args, kept, n_valid, ignore_index, lam = ctx.vars
+        grad = _native.ohem_backward(args, kept, ignore_index, grad_output, n_valid, lam)
         return grad, None, None, None, None, None
 
 

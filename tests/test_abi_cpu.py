@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol(native):
         assert name in native._SIGNATURES, "binding lacks " + name
         assert len(native._SIGNATURES[name][1]) == n_args, name
     assert set(native._SIGNATURES) == set(decl)
-    assert lib.plh_abi_version() == 2
+    assert lib.plh_abi_version() == 3
 
 
 def test_error_strings(native):
@@ -148,6 +148,17 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, None, 0, 1, 4, 16, 255, 0.7, 1, None) == -5
     assert lib.plh_ohem_ce_forward(p, 0, p, p, p, p, p, p, wsp, 16, 1, 4, 16, 255, 0.7, 1, None) == -5
     # fused OHEM large margin: the same checks behind one more scalar
+    # the forwards that leave a byte mask instead of new labels, and the backwards that read it
+    assert lib.plh_ohem_ce_forward_kept(p, 4, p, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -7
+    assert lib.plh_ohem_ce_forward_kept(p, 0, p, None, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.7, 1, None) == -1
+    assert lib.plh_ohem_ce_forward_kept(p, 0, p, p, p, p, p, p, wsp, 16, 1, 4, 16, 255, 0.7, 1, None) == -5
+    assert lib.plh_ohem_lmargin_forward_kept(p, 0, p, None, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
+    assert lib.plh_ohem_lmargin_forward_kept(p, 0, p, p, p, p, p, p, None, 0, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -5
+    for back in (lib.plh_lsr_backward_kept, lib.plh_lmargin_backward_kept):
+        assert back(p, 0, p, None, p, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -1
+        assert back(p, 0, p, p, None, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -1
+        assert back(p, 5, p, p, p, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -7
+        assert back(None, 0, None, None, None, 1.0, None, None, 0, 4, 16, 255, 0.0, None) == 0
     assert lib.plh_ohem_lmargin_forward(p, 4, p, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -7
     assert lib.plh_ohem_lmargin_forward(p, 0, None, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
     assert lib.plh_ohem_lmargin_forward(p, 0, p, p, None, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1

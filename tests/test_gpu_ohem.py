@@ -244,3 +244,50 @@ def test_ohem_ce_fused_forward_edge_cases(native, case, which):
         two_step = pl.LargeMarginSoftmaxV3(ignore_index=255, reduction="mean")(
             xt.detach(), pl.score_ohem_label(xt, dev(y), 255, thresh, n_min))
         assert abs(two_step.item() - loss.item()) <= 1e-6 * abs(loss.item())
+
+
+@pytest.mark.parametrize("lam", [None, 0.3], ids=["ce", "lmargin"])
+@pytest.mark.parametrize("shape,scale,thresh,div", [
+    ((2, 19, 40, 52), 2.0, 0.7, 16),         # the n_min-th smallest score is below the threshold: "drop what exceeds it"
+    ((2, 19, 40, 52), 2.0, 1e-7, 2),         # ... above it: ranks among the ties decide
+    ((2, 5, 33, 31), 40.0, 0.7, 4),          # saturated softmaxes: valid pixels that score exactly 1, next to ignored ones
+    ((3, 7, 9, 11), 40.0, 2.0, 8),           # a threshold nothing exceeds: every valid pixel stays
+    ((500, 23), 3.0, 0.5, 16),
+    ((64, 300), 6.0, 0.5, 8),
+])
+def test_kept_mask_is_the_relabelling(native, shape, scale, thresh, div, lam):
+    """The forwards that hand their selection on as a byte mask: the mask is the relabelling of
+    plh_ohem_score_label bit for bit (kept = new label is not ignore_index), loss and count are those of the entry
+    points that write new labels, and the masked backward on the old labels is the backward on the new ones."""
+    x = synth.normal(131, 1, shape, 0.0, scale)
+    y = synth.seg_labels(131, shape[:1] + shape[2:], shape[1], 255, 0.1)
+    xt, yt = dev(x), dev(y)
+    n_min = y.size // div
+    loss, n_valid, args, kept = native.ohem_ce_forward(xt, yt, 255, thresh, n_min, lam)
+    new_labels = native.ohem_score_label(xt, yt, 255, thresh, n_min)
+    assert torch.equal(kept[:y.size].view(y.shape).bool(), new_labels != 255)
+    assert int(n_valid.item()) == int((new_labels != 255).sum().item())
+    assert np.array_equal(yt.cpu().numpy(), y)                        # the labels are left alone
+    lib = native.load()
+    P, st = native._ptr, native._stream
+    n, c = shape[0], shape[1]
+    m = x.size // (n * c)
+    scratch = torch.empty((2, y.size), device=xt.device)
+    ws = torch.empty(int(lib.plh_ohem_ce_workspace_bytes(y.size)), dtype=torch.uint8, device=xt.device)
+    out_labels = torch.empty_like(yt)
+    loss2 = torch.empty((), device=xt.device)
+    cnt2 = torch.empty((), dtype=torch.int64, device=xt.device)
+    head = (P(xt), 0, P(yt), P(out_labels), P(scratch[0]), P(scratch[1]), P(loss2), P(cnt2), P(ws), ws.numel(), n, c, m, 255)
+    rc = (lib.plh_ohem_ce_forward(*head, thresh, n_min, st()) if lam is None
+          else lib.plh_ohem_lmargin_forward(*head, lam, thresh, n_min, st()))
+    assert rc == 0
+    assert torch.equal(out_labels, new_labels) and int(cnt2.item()) == int(n_valid.item())
+    if int(n_valid.item()):
+        assert loss2.cpu().numpy().tobytes() == loss.float().cpu().numpy().tobytes()
+    one = torch.ones((), device=xt.device)
+    got = native.ohem_backward(args, kept, 255, one, n_valid, lam)
+    if lam is None:
+        want = native.lsr_backward_scaled(xt, new_labels, 255, 0.0, one, n_valid)
+    else:
+        want = native.lmargin_backward_scaled(xt, new_labels, lam, 255, one, n_valid)
+    assert torch.equal(got, want)               # -0.0 == 0.0: a dropped pixel's products may carry a sign
