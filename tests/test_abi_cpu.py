@@ -158,7 +158,6 @@ def test_arguments_are_rejected_before_any_launch(native):
         assert back(p, 0, p, None, p, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -1
         assert back(p, 0, p, p, None, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -1
         assert back(p, 5, p, p, p, 1.0, None, p, 1, 4, 16, 255, 0.0, None) == -7
-        assert back(None, 0, None, None, None, 1.0, None, None, 0, 4, 16, 255, 0.0, None) == 0
     assert lib.plh_ohem_lmargin_forward(p, 4, p, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -7
     assert lib.plh_ohem_lmargin_forward(p, 0, None, p, p, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
     assert lib.plh_ohem_lmargin_forward(p, 0, p, p, None, p, p, p, wsp, ce_need, 1, 4, 16, 255, 0.3, 0.7, 1, None) == -1
