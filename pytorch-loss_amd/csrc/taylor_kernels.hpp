@@ -86,8 +86,9 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
                                                              const TaylorParams p) {
     // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
     // evaluation of the series carries a test of its own
-    auto run = [&](auto order_tag) {
+    auto run = [&](auto order_tag, auto log_tag) {
     constexpr int ORD = decltype(order_tag)::value;
+    constexpr bool LOG = decltype(log_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP];
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
             const float inv = 1.f / s, ls = logf(s);
 #pragma unroll
             for (int j = 0; j < CP; ++j)
-                if (chan_ok<CP>(j, p.C)) y[j][kk] = p.use_log ? logf(y[j][kk]) - ls : y[j][kk] * inv;
+                if (chan_ok<CP>(j, p.C)) y[j][kk] = LOG ? logf(y[j][kk]) - ls : y[j][kk] * inv;
         }
 #pragma unroll
         for (int j = 0; j < CP; ++j)
@@ -121,8 +122,10 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_fwd_regs(const T *__restric
     }
     at.store_slice(out, p.C, p.m_size, raw);
     };
-    if (p.order == 2) run(std::integral_constant<int, 2>());
-    else run(std::integral_constant<int, 4>());
+    if (p.order == 2 && p.use_log) run(std::integral_constant<int, 2>(), std::true_type());
+    else if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+    else if (p.use_log) run(std::integral_constant<int, 4>(), std::true_type());
+    else run(std::integral_constant<int, 4>(), std::false_type());
 }
 
 template <class T, int CP, int V, int Form>
@@ -130,8 +133,9 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
                                                              T *__restrict__ gx, const TaylorParams p) {
     // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
     // evaluation of the series carries a test of its own
-    auto run = [&](auto order_tag) {
+    auto run = [&](auto order_tag, auto log_tag) {
     constexpr int ORD = decltype(order_tag)::value;
+    constexpr bool LOG = decltype(log_tag)::value;
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
     if (!at.live) return;
     typename Pack<T, V>::Raw raw[CP], graw[CP];
@@ -150,10 +154,10 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
                 taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
                 s += f;
-                dot += p.use_log ? gj : f * gj;
+                dot += LOG ? gj : f * gj;
             }
         inv[k] = 1.f / s;
-        mid[k] = p.use_log ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
+        mid[k] = LOG ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
     }
 #pragma unroll
     for (int j = 0; j < CP; ++j)
@@ -170,15 +174,17 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_bwd_regs(const T *__restric
                 float f, df;
                 taylor_pair24<ORD>(Pack<T, V>::get(raw[j], k), f, df);
                 const float gj = Pack<T, V>::get(graw[j], k);
-                r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
+                r[k] = LOG ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
             }
             raw[j] = Pack<T, V>::put(r);
             forget_origin(raw[j]);      // packed here, channel by channel: nothing of the sweep waits for the stores
         }
     at.store_slice(gx, p.C, p.m_size, raw);
     };
-    if (p.order == 2) run(std::integral_constant<int, 2>());
-    else run(std::integral_constant<int, 4>());
+    if (p.order == 2 && p.use_log) run(std::integral_constant<int, 2>(), std::true_type());
+    else if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+    else if (p.use_log) run(std::integral_constant<int, 4>(), std::true_type());
+    else run(std::integral_constant<int, 4>(), std::false_type());
 }
 
 // Cross entropy on the log form: loss per pixel (fp32), and its gradient with the upstream folded in.
@@ -458,8 +464,9 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
     __shared__ float parts[kSplitWaves][kWave * V];
     // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
     // evaluation of the series carries a test of its own
-    auto run = [&](auto order_tag) {
+    auto run = [&](auto order_tag, auto log_tag) {
     constexpr int ORD = decltype(order_tag)::value;
+    constexpr bool LOG = decltype(log_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
@@ -498,14 +505,16 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_fwd_split(const T *__re
         for (int k = 0; k < V; ++k) {
             float f, df;
             taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
-            r[k] = p.use_log ? logf(f) - ls[k] : f * inv[k];
+            r[k] = LOG ? logf(f) - ls[k] : f * inv[k];
         }
         raw[i] = PK::put(r);
     }
     at.store(out, p.m_size, raw);
     };
-    if (p.order == 2) run(std::integral_constant<int, 2>());
-    else run(std::integral_constant<int, 4>());
+    if (p.order == 2 && p.use_log) run(std::integral_constant<int, 2>(), std::true_type());
+    else if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+    else if (p.use_log) run(std::integral_constant<int, 4>(), std::true_type());
+    else run(std::integral_constant<int, 4>(), std::false_type());
 }
 
 template <class T, int KW, int V, bool PerImage = false>
@@ -514,8 +523,9 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
     __shared__ float parts[2][kSplitWaves][kWave * V];
     // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
     // evaluation of the series carries a test of its own
-    auto run = [&](auto order_tag) {
+    auto run = [&](auto order_tag, auto log_tag) {
     constexpr int ORD = decltype(order_tag)::value;
+    constexpr bool LOG = decltype(log_tag)::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const SplitSlice<T, V, KW, PerImage> at(p.P, p.m_size, p.C, p.xcd_run);
     using PK = Pack<T, V>;
@@ -532,7 +542,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
                 taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
                 const float gj = PK::get(graw[i], k);
                 s += (i < at.here) ? f : 0.f;
-                dot += (i < at.here) ? (p.use_log ? gj : f * gj) : 0.f;
+                dot += (i < at.here) ? (LOG ? gj : f * gj) : 0.f;
             }
             parts[0][wave][lane * V + k] = s;
             parts[1][wave][lane * V + k] = dot;
@@ -550,7 +560,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
             dot += parts[1][w][lane * V + k];
         }
         inv[k] = 1.f / s;
-        mid[k] = p.use_log ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
+        mid[k] = LOG ? dot * inv[k] : dot * inv[k] * inv[k];     // csrc/taylor_softmax.cu:163-173
     }
 #pragma unroll
     for (int i = 0; i < KW; ++i) {
@@ -565,14 +575,16 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_sm_bwd_split(const T *__re
             float f, df;
             taylor_pair24<ORD>(PK::get(raw[i], k), f, df);
             const float gj = PK::get(graw[i], k);
-            r[k] = p.use_log ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
+            r[k] = LOG ? df * (__builtin_amdgcn_rcpf(f) * gj - mid[k]) : df * (inv[k] * gj - mid[k]);
         }
         raw[i] = PK::put(r);
     }
     at.store(gx, p.m_size, raw);
     };
-    if (p.order == 2) run(std::integral_constant<int, 2>());
-    else run(std::integral_constant<int, 4>());
+    if (p.order == 2 && p.use_log) run(std::integral_constant<int, 2>(), std::true_type());
+    else if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+    else if (p.use_log) run(std::integral_constant<int, 4>(), std::true_type());
+    else run(std::integral_constant<int, 4>(), std::false_type());
 }
 
 // --------------------------------------------------------------- group ----
@@ -687,8 +699,9 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
     __shared__ float red[4];
     // the order is uniform over the grid: the body is compiled once per order and chosen here, so that no
     // evaluation of the series carries a test of its own
-    auto run = [&](auto order_tag) {
+    auto run = [&](auto order_tag, auto log_tag) {
     constexpr int ORD = decltype(order_tag)::value;
+    constexpr bool LOG = decltype(log_tag)::value;
     constexpr int L = WaveRow<T, NI, LP, G>::L;
     using Span = WaveRowSpan<T, L, G, NI>;
     T *tile = Span::tile();
@@ -714,7 +727,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 s += ok ? f : 0.f;
                 if constexpr (Kind == kTaylorBwd) {
                     const float gj = rg.v[i][l];
-                    dot += ok ? (p.use_log ? gj : f * gj) : 0.f;
+                    dot += ok ? (LOG ? gj : f * gj) : 0.f;
                 }
             }
         }
@@ -734,7 +747,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
             }
         } else {
             const float ls = logf(s);
-            const float mid = p.use_log ? dot * inv : dot * inv * inv;
+            const float mid = LOG ? dot * inv : dot * inv * inv;
             int tgt = -1;
             float cold = 0.f, hot = 0.f;        // cross entropy: f' times one of these, see taylor_group
             if constexpr (Kind == kTaylorCeBwd) {
@@ -758,10 +771,10 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                     float f, df;
                     taylor_pair24<ORD>(r.v[i][l], f, df);
                     if constexpr (Kind == kTaylorFwd) {
-                        o[l] = p.use_log ? logf(f) - ls : f * inv;
+                        o[l] = LOG ? logf(f) - ls : f * inv;
                     } else if constexpr (Kind == kTaylorBwd) {
                         const float gj = rg.v[i][l];
-                        o[l] = p.use_log ? df / f * gj - mid * df : df * inv * gj - df * mid;
+                        o[l] = LOG ? df / f * gj - mid * df : df * inv * gj - df * mid;
                     } else {
                         o[l] = (tgt >= 0) ? df * ((e0 + l == tgt) ? hot : cold) : 0.f;
                     }
@@ -786,8 +799,16 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
         }
     }
     };
-    if (p.order == 2) run(std::integral_constant<int, 2>());
-    else run(std::integral_constant<int, 4>());
+    // the logarithmic form is a matter of the softmax kinds only
+    if constexpr (Kind == kTaylorFwd || Kind == kTaylorBwd) {
+        if (p.order == 2 && p.use_log) run(std::integral_constant<int, 2>(), std::true_type());
+        else if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+        else if (p.use_log) run(std::integral_constant<int, 4>(), std::true_type());
+        else run(std::integral_constant<int, 4>(), std::false_type());
+    } else {
+        if (p.order == 2) run(std::integral_constant<int, 2>(), std::false_type());
+        else run(std::integral_constant<int, 4>(), std::false_type());
+    }
 }
 
 // ------------------------------------------------------- a block per row ----
