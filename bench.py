@@ -434,6 +434,14 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         sb = lambda: lib.plh_taylor_softmax_backward(P(y_out), P(x), tag, P(grad), n, c, m, 4, 1, st())
         assert sf() == 0 and sb() == 0
         legs += [("log_softmax_forward", sf, 2 * eb), ("log_softmax_backward", sb, 3 * eb)]
+    if name == "lovasz":
+        # the same forward with its sort passes in the decoupled look-back form (an entry point of its own)
+        lb_bytes = int(lib.plh_lovasz_lookback_workspace_bytes(n, c, m))
+        lb_ws = torch.empty(lb_bytes, dtype=torch.uint8, device=x.device)
+        lf = lambda: lib.plh_lovasz_forward_lookback(P(x), tag, P(labels), P(losses), P(jacc), P(lb_ws), lb_bytes, n, c, m,
+                                                     255, st())
+        assert lf() == 0
+        legs += [("forward_look_back", lf, fwd_bytes)]
     for key, fn, nbytes in legs:
         ms = time_kernel(fn)
         gbps = nbytes / (ms * 1e-3) / 1e9
@@ -480,9 +488,15 @@ def cpu_baseline(name, shape, spot_check=True):
         return _time_cpu(name, shape, cores, lambda: torch_ref.soft_dice(logits, labels, 1, 1.0), logits)
     cfg = {"lsr": "cfg2", "lmargin": "cfg4", "focal": "cfg3", "lovasz": "cfg5", "ohem": "cfg2", "taylor": "cfg2"}[name]
     whole = name == "lovasz"
-    w = synth.workload(cfg) if whole else synth.workload(cfg, batch=1)
-    logits = torch.from_numpy(w["logits"]).requires_grad_()
-    labels = torch.from_numpy(w["labels"])
+    if name == "focal" and (name, tuple(shape)) not in SYNTH_CONFIG:
+        # the focal loss at another shape (the segmentation one): one image of make_inputs' distribution
+        g = torch.Generator().manual_seed(15)
+        logits = (torch.randn((1,) + tuple(shape[1:]), generator=g) * 1.5 - 2.0).requires_grad_()
+        labels = (torch.rand(logits.shape, generator=g) < 0.02).float()
+    else:
+        w = synth.workload(cfg) if whole else synth.workload(cfg, batch=1)
+        logits = torch.from_numpy(w["logits"]).requires_grad_()
+        labels = torch.from_numpy(w["labels"])
     fn = {"lsr": lambda: torch_ref.lsr(logits, labels, 0.1, "mean", 255),
           "lmargin": lambda: torch_ref.lmargin(logits, labels, 0.3, "mean", 255),
           "focal": lambda: torch_ref.focal(logits, labels, 0.25, 2, "mean"),
@@ -652,10 +666,10 @@ def targets_block(headline, main_res, others, headline_cpu, with_cpu):
         e = {"ms": round(ms, 4), "graph_ms": (step_ms.get("graph") or {}).get("ms"), "bytes": nbytes,
              "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
              "fwd_ms": (kern.get("forward") or {}).get("ms"), "bwd_ms": (kern.get("backward") or {}).get("ms")}
-        if with_cpu and "base" not in WORKLOADS[t]:
+        if with_cpu:
             try:
                 c = headline_cpu if (t == headline and headline_cpu and "error" not in headline_cpu) else \
-                    cpu_baseline(t, WORKLOADS[t]["shape"])
+                    cpu_baseline(WORKLOADS[t].get("base", t), WORKLOADS[t]["shape"])
                 rel = c.get("parity_spot_check", {}).get("rel_err")
                 e["cpu"] = {"ms": c["ms_per_step"], "GB/s": c["value"], "threads": c["cores"],
                             "rel_err": None if rel is None else float("%.2g" % rel)}
