@@ -41,23 +41,61 @@ __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)(
 // again. Both sort last (score_key clamps at 1) and tie with each other in pixel order.
 constexpr float kNoTargetMark = 2.f;
 
+// What the score kernel of the cross-entropy forward leaves besides scores and losses, for the case that the threshold
+// rule decides the selection (at least n_min pixels score within the threshold, so "beyond the n_min lowest" holds
+// for every pixel above it): the byte mask and the per-block sums of that rule, and per block the number of pixels
+// whose score, capped at 1 like the selection's keys, lies within the threshold. The first histogram kernel adds those
+// numbers up; when they reach n_min it raises kEarlyFlag in the selection's state and every later kernel of the
+// selection returns at once (the finish then adds up these sums instead of the relabelling pass's).
+struct OhemEarly {
+    uint8_t *kept;      // [P]; nullptr: nothing of this is produced
+    float *sum;         // [blocks of the score kernel]
+    int *cnt;           // [blocks]
+    int *below;         // [blocks]
+    float thresh;
+};
+constexpr int kEarlyFlag = 8;       // index into OhemTables::state
+
+// One byte per pixel for this thread's V pixels (nv of them exist).
+template <int V>
+__device__ __forceinline__ void store_kept(uint8_t *kept, int64_t pix, int nv, const bool (&kp)[V]) {
+    typedef unsigned short u16_a1 __attribute__((aligned(1)));
+    typedef unsigned u32_a1 __attribute__((aligned(1)));
+    if (nv == V && V == 2) {
+        *reinterpret_cast<u16_a1 *>(kept + pix) = (unsigned short)((unsigned)kp[0] | ((unsigned)kp[V - 1] << 8));
+    } else if (nv == V && V == 4) {
+        *reinterpret_cast<u32_a1 *>(kept + pix) =
+            (unsigned)kp[0] | ((unsigned)kp[1 % V] << 8) | ((unsigned)kp[2 % V] << 16) | ((unsigned)kp[3 % V] << 24);
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k)
+            if (k < nv) kept[pix + k] = kp[k] ? 1 : 0;
+    }
+}
+
 
 template <class T, int CP, int V, int Form>
 __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                               float *__restrict__ scores, float *__restrict__ ce,
                                                               int64_t P, int64_t m_size, int C, int64_t ignore,
-                                                              unsigned xcd_run, uint32_t *__restrict__ tables, float none) {
+                                                              unsigned xcd_run, uint32_t *__restrict__ tables, float none,
+                                                              const OhemEarly ev) {
+    __shared__ float red[4];
+    const bool early = ev.kept != nullptr;              // uniform over the grid
     // the selection's tables start at zero; the kernels that fill them are launched after this one
     if (tables && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kOhemZeroWords; i += kRegsBlock) tables[i] = 0;
     const PixelRef<V, Form> at(P, m_size, C, xcd_run);
-    if (!at.live) return;
+    if (!early && !at.live) return;
     // labels (and the upstream gradient) first: in the rows form the slice arrives through LDS behind a wait
     int64_t lb[V];
     at.labels(lab, ignore, lb);
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, C, m_size, raw);
     float out[V], loss[V];
+    bool kp[V];
+    float kept_sum = 0.f;
+    int kept_cnt = 0, below_cnt = 0;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
@@ -79,10 +117,31 @@ __global__ __launch_bounds__(kRegsBlock) void ohem_scores_regs(const T *__restri
         out[k] = (tgt < 0) ? none : fminf(e_y * __builtin_amdgcn_rcpf(s), 1.f);
         // the pixel's cross entropy from the same sums, exact also where the score underflows
         loss[k] = (tgt < 0) ? 0.f : __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, mx - x_y);
+        if (early) {
+            const bool real = at.live && k < at.nv;
+            kp[k] = real && tgt >= 0 && !(out[k] > ev.thresh);
+            kept_sum += kp[k] ? loss[k] : 0.f;
+            kept_cnt += kp[k] ? 1 : 0;
+            below_cnt += (real && fminf(out[k], 1.f) <= ev.thresh) ? 1 : 0;      // fminf: a NaN score counts as 1
+        }
     }
-    // the selection kernels read both back several times: leave them to the caches
-    at.store_f32_cached(scores, out);
-    if (ce) at.store_f32_cached(ce, loss);
+    if (at.live) {
+        // the selection kernels read both back several times: leave them to the caches (in the threshold-rule case
+        // nothing reads them again; stores that bypass the caches measured the same there)
+        at.store_f32_cached(scores, out);
+        if (ce) at.store_f32_cached(ce, loss);
+    }
+    if (early) {
+        if (at.live) store_kept<V>(ev.kept, at.pix, at.nv, kp);
+        const float bs = block_sum_256(kept_sum, red);
+        const float bk = block_sum_256((float)kept_cnt, red);         // at most 1024 per block: exact in fp32
+        const float bb = block_sum_256((float)below_cnt, red);
+        if (threadIdx.x == 0) {
+            ev.sum[blockIdx.x] = bs;
+            ev.cnt[blockIdx.x] = (int)bk;
+            ev.below[blockIdx.x] = (int)bb;
+        }
+    }
 }
 
 // 33..256 channels in NCHW (SplitSlice): per wavefront the maximum, the exponential sum and the target's
@@ -332,9 +391,36 @@ __device__ __forceinline__ void hist_add(uint32_t *bins, float s, uint32_t high_
 // later passes leave their histograms empty (every block returns before it reads a score), the digits they
 // resolve from those come out as 0, and the key that ohem_ties publishes stays below the threshold.
 __global__ __launch_bounds__(256) void ohem_hist(const float *__restrict__ scores, OhemTables tb, int P, int pass,
-                                                 uint32_t n_min, float thresh, int vec) {
+                                                 uint32_t n_min, float thresh, int vec,
+                                                 const int *__restrict__ below, unsigned below_blocks) {
     __shared__ uint32_t bins[kOhemBins];
     __shared__ uint32_t scan[260];
+    if (pass > 0 && tb.state[kEarlyFlag]) return;            // uniform over the grid
+    if (pass == 0 && below) {
+        // the score kernel counted, per block, the pixels that score within the threshold: with n_min or more of them
+        // the threshold rule is the whole selection (every block adds the numbers up for itself, block 0 says so)
+        // (the array is 16-byte aligned: four 16-byte loads in flight per thread and trip)
+        __shared__ float red[4];
+        typedef int i4 __attribute__((ext_vector_type(4)));
+        int mine = 0;
+        const i4 *b4 = reinterpret_cast<const i4 *>(below);
+        const unsigned quads = below_blocks / 4;
+        for (unsigned i = threadIdx.x; i < quads; i += 1024) {
+            i4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = i + u * 256 < quads ? b4[i + u * 256] : i4{0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) mine += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        }
+        if (threadIdx.x < below_blocks - quads * 4) mine += below[quads * 4 + threadIdx.x];
+        // per thread at most 2^31 / 256 pixels, in whole numbers a float holds up to 2^24: sum as two halves
+        const float lo = block_sum_256((float)(mine & 0xFFFF), red), hi = block_sum_256((float)(mine >> 16), red);
+        const uint64_t total = (uint64_t)lo + ((uint64_t)hi << 16);
+        if (total >= n_min) {
+            if (blockIdx.x == 0 && threadIdx.x == 0) tb.state[kEarlyFlag] = 1;
+            return;
+        }
+    }
     for (int i = threadIdx.x; i < kOhemBins; i += 256) bins[i] = 0;
     const uint32_t prefix = pass == 0 ? 0u : ohem_resolve_digit(tb, pass - 1, n_min, scan, blockIdx.x == 0);
     if (pass > 0) {
@@ -403,6 +489,7 @@ __device__ __forceinline__ void load_tile_keys(const float *scores, int P, int b
 __global__ __launch_bounds__(256) void ohem_ties(const float *__restrict__ scores, OhemTables tb, int P, int tiles,
                                                  uint32_t n_min, float thresh, int vec) {
     __shared__ uint32_t scan[260];
+    if (tb.state[kEarlyFlag]) return;                           // uniform over the grid
     const uint32_t v = ohem_resolve_digit(tb, 2, n_min, scan, blockIdx.x == 0);
     if (!(__builtin_bit_cast(float, v) > thresh)) return;       // block-uniform
     const int lane = threadIdx.x & 63;
@@ -438,6 +525,7 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
                                                     uint8_t *__restrict__ kept_out) {
     __shared__ uint32_t wave_ties[4], run_ties[4];
     __shared__ float red[4];
+    if (n_min != 0 && tb.state[kEarlyFlag]) return;     // uniform over the grid: the score kernel has left mask and sums
     const int base = blockIdx.x * kOhemTile + threadIdx.x * 4;
     float s[4];
     uint32_t key[4];
@@ -530,6 +618,16 @@ __global__ __launch_bounds__(256) void ohem_relabel(const float *__restrict__ sc
     }
 }
 
+// The mean over the kept pixels from whichever pass produced the final sums: the score kernel's (threshold rule,
+// kEarlyFlag raised) or the relabelling pass's.
+__global__ __launch_bounds__(1024) void ohem_finish(const uint32_t *__restrict__ state, Partials early, unsigned early_blocks,
+                                                    Partials late, unsigned late_blocks, float *__restrict__ loss_out,
+                                                    int64_t *__restrict__ count_out) {
+    const bool e = state[kEarlyFlag] != 0;              // uniform
+    finish_block(e ? early.sum : late.sum, e ? early.cnt : late.cnt, e ? early_blocks : late_blocks, loss_out, count_out,
+                 kFinishMeanOverCount, 0);
+}
+
 __global__ void ohem_copy_labels(const int64_t *__restrict__ in, int64_t *__restrict__ out, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
         out[i] = in[i];
@@ -544,9 +642,14 @@ static int64_t ohem_tiles(int64_t P) { return ceil_div(P > 0 ? P : 1, kOhemTile)
 
 static int launch_scores(const void *logits, int32_t dtype, const int64_t *labels, float *scores, float *ce,
                          int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, hipStream_t st,
-                         uint32_t *tables = nullptr, float none = 1.f) {
+                         uint32_t *tables = nullptr, float none = 1.f, const OhemEarly *early = nullptr,
+                         unsigned *early_blocks = nullptr) {
+    // `early`: taken up by the kernels that keep a pixel's channels in a lane's registers; *early_blocks then is their
+    // grid (0: the launch shape produces none of it)
     const int64_t P = n_size * m_size;
     const int C = (int)dimsize;
+    const OhemEarly ev = early ? *early : OhemEarly{nullptr, nullptr, nullptr, nullptr, 0.f};
+    if (early_blocks) *early_blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         const T *x = static_cast<const T *>(logits);
@@ -597,19 +700,20 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
             const bool image = !vec && image_form_pays<T>(C, m_size);
             const unsigned grid = vec ? regs_grid<VT>(P) : (image ? image_grid<4>(n_size, m_size) : regs_grid<1>(P));
             const unsigned run = xcd_run_for(sizeof(T), m_size);
+            if (early_blocks && ev.kept) *early_blocks = grid;
             switch ((C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                   \
     case K:                                                                                                           \
         if (uni) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kUniform>), dim3(grid), dim3(kRegsBlock), 0, st,  \
-                                    x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                  \
+                                    x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none, ev);              \
         else if (vec) hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, VT, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, \
-                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);         \
+                                         st, x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none, ev);     \
         else if (image) {                                                                                             \
             if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                          \
                 hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st,   \
-                                   x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                   \
+                                   x, labels, scores, ce, P, m_size, C, ignore_index, run, tables, none, ev);               \
         } else hipLaunchKernelGGL((ohem_scores_regs<T, 4 * K, 1, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x,  \
-                                  labels, scores, ce, P, m_size, C, ignore_index, run, tables, none);                       \
+                                  labels, scores, ce, P, m_size, C, ignore_index, run, tables, none, ev);                   \
         break;
                 PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -632,6 +736,10 @@ static int launch_scores(const void *logits, int32_t dtype, const int64_t *label
     return check_launch();
 }
 
+// The score kernels that leave the threshold rule's sums give a block 256 pixels or more (a multiple of 64 slots keeps
+// the three arrays 256-byte aligned).
+static int64_t early_blocks_max(int64_t P) { return ceil_div(ceil_div(P > 0 ? P : 1, kRegsBlock), 64) * 64; }
+
 static int64_t select_workspace(int64_t P) {
     return align256(kOhemZeroWords * 4) + align256((ohem_tiles(P) + kTieRuns) * 4);
 }
@@ -646,7 +754,8 @@ static int check_workspace(const void *workspace, int64_t workspace_bytes, int64
 static int launch_select(const float *scores, const int64_t *labels, int64_t *out_labels, void *workspace,
                          int64_t P, int64_t ignore_index, float score_thresh, int64_t n_min, hipStream_t st,
                          const float *ce = nullptr, Partials part = Partials{nullptr, nullptr},
-                         bool tables_zeroed = false, uint8_t *kept_out = nullptr) {
+                         bool tables_zeroed = false, uint8_t *kept_out = nullptr, const int *below = nullptr,
+                         unsigned below_blocks = 0) {
     if (n_min >= P && part.sum) {                // nothing is relabelled, the loss is still wanted
         n_min = 0;
         score_thresh = INFINITY;
@@ -673,7 +782,8 @@ static int launch_select(const float *scores, const int64_t *labels, int64_t *ou
         // addresses: 512 blocks (two per compute unit) measured 30 us faster than 2048 on 8 M scores
         const unsigned hgrid = (unsigned)(ceil_div(P, 256 * 16) < 512 ? ceil_div(P, 256 * 16) : 512);
         for (int pass = 0; pass < 3; ++pass)
-            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, score_thresh, vec);
+            hipLaunchKernelGGL(ohem_hist, dim3(hgrid), dim3(256), 0, st, scores, tb, Pi, pass, k, score_thresh, vec,
+                               pass == 0 ? below : nullptr, below_blocks);
         hipLaunchKernelGGL(ohem_ties, dim3(kTieRuns / 4), dim3(256), 0, st, scores, tb, Pi, (int)tiles, k, score_thresh, vec);
     }
     hipLaunchKernelGGL(ohem_relabel, dim3((unsigned)tiles), dim3(256), 0, st, scores, labels, out_labels, tb, Pi, (int)tiles, k,
@@ -738,7 +848,8 @@ extern "C" int plh_ohem_score_label(const void *logits, int32_t dtype, const int
 
 extern "C" int64_t plh_ohem_ce_workspace_bytes(int64_t n_pixels) {
     if (n_pixels < 0 || n_pixels > kOhemMaxPixels) return PLH_ERR_BAD_SIZE;
-    return select_workspace(n_pixels) + align256(8 * ohem_tiles(n_pixels));
+    // the selection's tables, the relabelling pass's partial sums (8 bytes per tile), the score kernel's (12 bytes per block)
+    return select_workspace(n_pixels) + align256(8 * ohem_tiles(n_pixels)) + align256(12 * early_blocks_max(n_pixels));
 }
 
 // The one-call forwards: scores and per-pixel loss in one pass over the logits (cross entropy: the
@@ -774,17 +885,40 @@ static int ohem_loss_forward(bool large_margin, float lam, const void *logits, i
     part.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P));
     part.cnt = reinterpret_cast<int *>(part.sum + tiles);
     const float none = kept ? kNoTargetMark : 1.f;
+    if (n_min >= P) {                            // nothing is dropped (launch_select says the same), the loss is still wanted
+        n_min = 0;
+        score_thresh = INFINITY;
+    }
+    // cross entropy with the byte mask: the score kernel also leaves what the threshold rule gives (OhemEarly)
+    OhemEarly ev{nullptr, nullptr, nullptr, nullptr, score_thresh};
+    unsigned early_blocks = 0;
+    if (!large_margin && kept) {
+        const int64_t slots = early_blocks_max(P);
+        ev.kept = kept;
+        ev.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P) + align256(8 * tiles));
+        ev.cnt = reinterpret_cast<int *>(ev.sum + slots);
+        ev.below = ev.cnt + slots;
+    }
     if (large_margin)
         rc = lmargin_forward_with_scores(logits, dtype, labels, pixel_loss, scores, n_size, dimsize, m_size, ignore_index,
                                          lam, st, none);
     else
         rc = launch_scores(logits, dtype, labels, scores, pixel_loss, n_size, dimsize, m_size, ignore_index, st,
-                           static_cast<uint32_t *>(workspace), none);
+                           static_cast<uint32_t *>(workspace), none, &ev, &early_blocks);
     if (rc != PLH_OK) return rc;
+    if (early_blocks && n_min <= 0) {            // no position lies below n_min: the threshold rule is the selection
+        finish_partials(Partials{ev.sum, ev.cnt}, early_blocks, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
+        return check_launch();
+    }
     rc = launch_select(scores, labels, out_labels, workspace, P, ignore_index, score_thresh, n_min, st, pixel_loss, part,
-                       /*tables_zeroed=*/!large_margin, kept);
+                       /*tables_zeroed=*/!large_margin, kept, early_blocks ? ev.below : nullptr, early_blocks);
     if (rc != PLH_OK) return rc;
-    finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
+    if (early_blocks)
+        hipLaunchKernelGGL(ohem_finish, dim3(1), dim3(1024), 0, st,
+                           static_cast<const uint32_t *>(workspace) + 3 * kOhemBins, Partials{ev.sum, ev.cnt}, early_blocks,
+                           part, (unsigned)tiles, loss_out, n_valid_out);
+    else
+        finish_partials(part, (unsigned)tiles, loss_out, n_valid_out, kFinishMeanOverCount, 0, st);
     return check_launch();
 }
 
