@@ -21,6 +21,7 @@ arithmetic: the same bits on every box and under every torch version, so the pri
 compared between runs and with the CPU oracle.
 """
 import argparse
+import gc
 import json
 import os
 import statistics
@@ -643,6 +644,16 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
         dist["cold"] = step_distribution(crit, sets)
         del sets
     dist["graph"] = graph_step(crit, logits, labels)
+    if ms < 0.15:
+        # a step this short can be bound by the autograd engine's hand-over between the calling thread and its
+        # worker thread: the same steps with the backward run on the calling thread (a PyTorch switch, not the library's)
+        try:
+            with torch.autograd.set_multithreading_enabled(False):
+                st_ms, _ = time_steps(crit, logits, labels, steps, warmup)
+            dist["calling_thread"] = {"ms": round(st_ms, 4), "steps": steps,
+                                      "what": "eager steps under torch.autograd.set_multithreading_enabled(False)"}
+        except Exception as e:
+            dist["calling_thread"] = {"error": "%s: %s" % (type(e).__name__, e)}
     del crit
     logits.grad = None
     return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist, function_level=func)
@@ -670,6 +681,8 @@ def targets_block(headline, main_res, others, headline_cpu, with_cpu):
         e = {"ms": round(ms, 4), "graph_ms": (step_ms.get("graph") or {}).get("ms"), "bytes": nbytes,
              "frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
              "fwd_ms": (kern.get("forward") or {}).get("ms"), "bwd_ms": (kern.get("backward") or {}).get("ms")}
+        if "calling_thread" in step_ms:      # short steps: the eager step with the backward on the calling thread
+            e["calling_thread_ms"] = step_ms["calling_thread"].get("ms")
         if with_cpu:
             try:
                 c = headline_cpu if (t == headline and headline_cpu and "error" not in headline_cpu) else \
@@ -705,6 +718,11 @@ def main():
     _native.load()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    # Python's first full garbage collection of a process that has imported torch and numpy takes ~30 ms (measured:
+    # once, at about step 100 of a loop of 0.34 ms steps), which is 90 steps' worth inside 50 timed ones. Collect now
+    # and move what is alive out of the collector's sight; what the steps allocate is still collected.
+    gc.collect()
+    gc.freeze()
 
     name = args.workload
     main_res = run_workload(name, args.steps, args.warmup, device, args.dtype)
@@ -739,6 +757,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "python_gc": "collected and frozen before the first measurement",
         "ms_per_step": round(main_res["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
