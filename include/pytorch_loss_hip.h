@@ -292,10 +292,10 @@ int plh_ohem_lmargin_forward(const void *logits, int32_t dtype, const int64_t *l
  * plh_lsr_backward_kept (smooth = 0) and plh_lmargin_backward_kept are the matching gradients: plh_*_backward_scaled
  * on the ORIGINAL labels, with an upstream gradient of 0 for every pixel whose byte in `kept` is 0. Everything else
  * as for plh_ohem_ce_forward / plh_ohem_lmargin_forward; `scores` holds 2 instead of 1 for pixels without a target.
- * plh_ohem_ce_forward_kept on logits of up to 32 channels also has its score kernel leave mask, sum and count of
- * the rule "drop what scores above the threshold", which is the whole selection whenever n_min or more pixels score
- * within the threshold; the kernels of the selection then return at once. The loss then is a sum over other blocks
- * than the relabelling pass's: equal to plh_ohem_ce_forward's to rounding, not bit for bit.
+ * On logits of up to 32 channels both also have their score pass leave mask, sum and count of the rule "drop what
+ * scores above the threshold", which is the whole selection whenever n_min or more pixels score within the
+ * threshold; the kernels of the selection then return at once. The loss then is a sum over other blocks than the
+ * relabelling pass's: equal to plh_ohem_ce_forward's / plh_ohem_lmargin_forward's to rounding, not bit for bit.
  */
 int plh_ohem_ce_forward_kept(const void *logits, int32_t dtype, const int64_t *labels,
                              uint8_t *kept, float *scores, float *pixel_ce,

@@ -25,7 +25,7 @@ static unsigned lmargin_run_typed(int variant, const T *x, const int64_t *lab, c
 static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,
                   int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
                   int64_t m_size, int64_t ignore, float lam, void *stream, float *scores = nullptr,
-                  float no_target_score = 1.f) {
+                  float no_target_score = 1.f, const OhemEarly *early = nullptr) {
     const bool WantLoss = variant != kLmBackward, WantGrad = variant == kLmBackward || variant == kLmForwardBackwardCount;
     const bool WantCount = variant == kLmForwardBackwardCount, Reduce = variant == kLmForwardReduced;
     if (blocks_out) *blocks_out = 0;
@@ -54,6 +54,11 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     p.xcd_run = xcd_run_for(es, m_size);
     p.scores = scores;
     p.no_target_score = no_target_score;
+    if (early) {
+        p.early_kept = early->kept;
+        p.early_below = early->below;
+        p.early_thresh = early->thresh;
+    }
     unsigned blocks = 0;
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
@@ -68,10 +73,25 @@ static const Partials kNoPartials{nullptr, nullptr};
 
 // Declared in plh_common.hpp for the OHEM entry point: the per-pixel forward that also leaves each
 // pixel's score.
+// With `early` (see OhemEarly) the launch is a reduced forward whose partial sums run over the pixels of the threshold
+// rule; *early_blocks is the number of blocks that left them, 0 when the launch shape took none of it (the
+// per-pixel losses and scores are written either way).
 int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
                                 int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
-                                hipStream_t stream, float no_target_score) {
+                                hipStream_t stream, float no_target_score, const OhemEarly *early, unsigned *early_blocks) {
     const Upstream up{nullptr, 0, nullptr, 1.f};
+    if (early_blocks) *early_blocks = 0;
+    // up to kMaxRegsChannels channels every forward runs in the register-resident kernels (pick_shape), the ones that
+    // take LmParams::early_*; their partial sums come from at most one block per 256 pixels, which is what `early` holds
+    const bool regs = early && early->kept && early_blocks && dimsize <= kMaxRegsChannels;
+    if (regs) {
+        unsigned blocks = 0;
+        const int rc = launch(kLmForwardReduced, logits, dtype, labels, up, losses, nullptr, nullptr,
+                              Partials{early->sum, early->cnt}, &blocks, n_size, dimsize, m_size, ignore_index, lam, stream,
+                              scores, no_target_score, early);
+        if (rc == PLH_OK && (blocks & kLmTookEarly)) *early_blocks = blocks & ~kLmTookEarly;
+        return rc;
+    }
     return launch(kLmForward, logits, dtype, labels, up, losses, nullptr, nullptr, kNoPartials, nullptr, n_size, dimsize,
                   m_size, ignore_index, lam, stream, scores, no_target_score);
 }

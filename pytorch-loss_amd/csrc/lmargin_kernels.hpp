@@ -28,6 +28,12 @@ struct LmParams {
     float no_target_score;   // what `scores` gets where a pixel has no target (ignored, label out of range): 1, as the
                              // reference's score pass writes it, or a mark above 1 that the selection tells apart
                         // (1 for a pixel without a target), what the OHEM relabelling ranks
+    // lm_regs as the score pass of the OHEM loss (OhemEarly in plh_common.hpp): with `early_kept` the partial sums of a
+    // reduced forward run over the pixels that score within `early_thresh` and have a target, their byte mask goes
+    // to early_kept and per block the number of pixels whose score, capped at 1, lies within the threshold to early_below
+    uint8_t *early_kept = nullptr;
+    int *early_below = nullptr;
+    float early_thresh = 0.f;
 };
 
 // ---------------------------------------------------------------- regs ----
@@ -39,8 +45,11 @@ struct LmParams {
 // left out: it scales every e_j by 2^r, cancels in q_j = e_j / s_no and is taken back out of
 // log2(s_no), sum q_j u_j and the rebuilt full sum.
 constexpr float kLmMasked = -1e30f;
+constexpr unsigned kLmTookEarly = 0x80000000u;      // in launch_typed's block count: the kernel took LmParams::early_*
 
-template <class T, int CP, int V, int Form, bool WantLoss, bool WantGrad>
+// Early: the forward as the score pass of the OHEM loss (LmParams::early_*), instances of their own - tested at run time
+// inside the pixel loop, the by-products cost the plain forward 5 % ((8,19,1024,1024) fp32: 0.1132 -> 0.1185 ms).
+template <class T, int CP, int V, int Form, bool WantLoss, bool WantGrad, bool Early = false>
 __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                      const Upstream up,
                                                      float *__restrict__ loss, T *__restrict__ grad,
@@ -81,7 +90,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
     unsigned n_valid = 0;
     float mine = 0.f;
-    int cnt = 0;
+    int cnt = 0, below = 0;
+    static_assert(!Early || kMayReduce, "the OHEM by-products belong to the forward");
+    constexpr bool early = Early;
+    bool kp[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
@@ -137,8 +149,17 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
             // formed here: left to itself the compiler moves a pixel's whole reduction down to the guarded
             // stores at the end and keeps every pixel's exponentials alive until then
             asm volatile("" : "+v"(out[k]), "+v"(score[k]));
-            mine += out[k];
-            cnt += (ign || !live) ? 0 : 1;
+            if constexpr (kMayReduce) {
+                if (early) {
+                    kp[k] = live && tgt >= 0 && !(score[k] > p.early_thresh);
+                    mine += kp[k] ? out[k] : 0.f;
+                    cnt += kp[k] ? 1 : 0;
+                    below += (live && fminf(score[k], 1.f) <= p.early_thresh) ? 1 : 0;   // fminf: a NaN score counts as 1
+                } else {
+                    mine += out[k];
+                    cnt += (ign || !live) ? 0 : 1;
+                }
+            }
         }
         if constexpr (WantGrad) {
             // g_j = gk * (p_j + h * ((x_j + 1 - sum_qx) * q_j - coeff))
@@ -171,8 +192,14 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
         if constexpr (kInPlace) __builtin_amdgcn_sched_barrier(0);
     }
     if (live) {
-        if (WantLoss && loss) at.store_f32(loss, out);
+        if (WantLoss && loss) {
+            if (early) at.store_f32_cached(loss, out);      // the relabelling pass may read them again
+            else at.store_f32(loss, out);
+        }
         if (WantLoss && p.scores) at.store_f32_cached(p.scores, score);
+        if constexpr (kMayReduce) {
+            if (early) store_kept<V>(p.early_kept, at.pix, at.nv, kp);
+        }
         if constexpr (WantGrad) {
             // ignored pixels get exact zeros whatever their logits were (the bitwise AND also clears NaN)
             const typename Pack<T, V>::Raw mask = Pack<T, V>::mask(keep);
@@ -192,9 +219,11 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);
+        const float bb = early ? block_sum_256((float)below, red) : 0.f;
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = bs;
             part.cnt[blockIdx.x] = (int)bc;
+            if (early) p.early_below[blockIdx.x] = (int)bb;
         }
     }
 }
@@ -806,9 +835,21 @@ static unsigned launch_regs(const T *x, const int64_t *lab, const Upstream &up, 
                             unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = regs_grid<V>(p.P);
     const bool uni = tiles_are_uniform(p.m_size, V, sizeof(T));
+    const bool early = WantLoss && !WantGrad && p.early_kept && part.sum;
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
+        if constexpr (WantLoss && !WantGrad) {                                                                       \
+            if (early) {                                                                                             \
+                if (V * sizeof(T) == 8 && uni)                                                                       \
+                    hipLaunchKernelGGL((lm_regs<T, 4 * K, V, (V * sizeof(T) == 8 ? kUniform : kGeneral), true, false, true>), \
+                                       dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);    \
+                else                                                                                                 \
+                    hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kGeneral, true, false, true>), dim3(grid),              \
+                                       dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);               \
+                break;                                                                                               \
+            }                                                                                                        \
+        }                                                                                                            \
         if constexpr (V * sizeof(T) == 8) {                                                                          \
             if (uni) {                                                                                               \
                 hipLaunchKernelGGL((lm_regs<T, 4 * K, V, kUniform, WantLoss, WantGrad>), dim3(grid),  \
@@ -831,12 +872,21 @@ template <class T, bool WantLoss, bool WantGrad>
 static unsigned launch_image(const T *x, const int64_t *lab, const Upstream &up, float *loss, T *grad,
                              unsigned long long *cnt, Partials part, const LmParams &p, hipStream_t st) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
+    const bool early = WantLoss && !WantGrad && p.early_kept && part.sum;
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                                  \
     case K:                                                                                                          \
-        if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                             \
-            hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, WantLoss, WantGrad>), dim3(grid), \
+        if constexpr (4 * K <= kImageFormMaxChannels<T>) {                                                           \
+            if constexpr (WantLoss && !WantGrad) {                                                                   \
+                if (early) {                                                                                         \
+                    hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, true, false, true>), dim3(grid),             \
+                                       dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);               \
+                    break;                                                                                           \
+                }                                                                                                    \
+            }                                                                                                        \
+            hipLaunchKernelGGL((lm_regs<T, 4 * K, 4, kPerImage, WantLoss, WantGrad>), dim3(grid),                    \
                                dim3(kRegsBlock), 0, st, x, lab, up, loss, grad, cnt, part, p);                       \
+        }                                                                                                            \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
@@ -851,6 +901,7 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     const float *second_f32 = go_vec ? go_vec : p.scores;      // the score output belongs to forwards without upstream
     unsigned blocks = 0;
+    const unsigned early_bit = (WantLoss && !WantGrad && p.early_kept && part.sum) ? kLmTookEarly : 0u;
     // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
     constexpr bool kHasSplit = !(WantLoss && WantGrad);
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), x, WantGrad ? grad : nullptr, lab, WantLoss ? loss : nullptr,
@@ -908,15 +959,16 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
                 }
             }
             break;
+        // (the register-resident kernels are the ones that take LmParams::early_*: bit 31 of the result says so)
         case Shape::RegsVec:
-            blocks = launch_regs<T, V, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
+            blocks = launch_regs<T, V, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st) | early_bit;
             break;
         case Shape::RegsOne:
             if (image_form_pays<T>(p.C, p.m_size)) {
-                blocks = launch_image<T, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
+                blocks = launch_image<T, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st) | early_bit;
                 break;
             }
-            blocks = launch_regs<T, 1, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st);
+            blocks = launch_regs<T, 1, WantLoss, WantGrad>(x, lab, up, loss, grad, cnt, part, p, st) | early_bit;
             break;
         case Shape::Wave:
             if (p.C <= wrow_cap<T>(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C))) {

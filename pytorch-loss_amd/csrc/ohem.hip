@@ -41,37 +41,7 @@ __device__ __forceinline__ int key_digit(uint32_t key, int pass) { return (int)(
 // again. Both sort last (score_key clamps at 1) and tie with each other in pixel order.
 constexpr float kNoTargetMark = 2.f;
 
-// What the score kernel of the cross-entropy forward leaves besides scores and losses, for the case that the threshold
-// rule decides the selection (at least n_min pixels score within the threshold, so "beyond the n_min lowest" holds
-// for every pixel above it): the byte mask and the per-block sums of that rule, and per block the number of pixels
-// whose score, capped at 1 like the selection's keys, lies within the threshold. The first histogram kernel adds those
-// numbers up; when they reach n_min it raises kEarlyFlag in the selection's state and every later kernel of the
-// selection returns at once (the finish then adds up these sums instead of the relabelling pass's).
-struct OhemEarly {
-    uint8_t *kept;      // [P]; nullptr: nothing of this is produced
-    float *sum;         // [blocks of the score kernel]
-    int *cnt;           // [blocks]
-    int *below;         // [blocks]
-    float thresh;
-};
-constexpr int kEarlyFlag = 8;       // index into OhemTables::state
-
-// One byte per pixel for this thread's V pixels (nv of them exist).
-template <int V>
-__device__ __forceinline__ void store_kept(uint8_t *kept, int64_t pix, int nv, const bool (&kp)[V]) {
-    typedef unsigned short u16_a1 __attribute__((aligned(1)));
-    typedef unsigned u32_a1 __attribute__((aligned(1)));
-    if (nv == V && V == 2) {
-        *reinterpret_cast<u16_a1 *>(kept + pix) = (unsigned short)((unsigned)kp[0] | ((unsigned)kp[V - 1] << 8));
-    } else if (nv == V && V == 4) {
-        *reinterpret_cast<u32_a1 *>(kept + pix) =
-            (unsigned)kp[0] | ((unsigned)kp[1 % V] << 8) | ((unsigned)kp[2 % V] << 16) | ((unsigned)kp[3 % V] << 24);
-    } else {
-#pragma unroll
-        for (int k = 0; k < V; ++k)
-            if (k < nv) kept[pix + k] = kp[k] ? 1 : 0;
-    }
-}
+constexpr int kEarlyFlag = 8;       // index into OhemTables::state: raised when the threshold rule decided (OhemEarly)
 
 
 template <class T, int CP, int V, int Form>
@@ -889,10 +859,10 @@ static int ohem_loss_forward(bool large_margin, float lam, const void *logits, i
         n_min = 0;
         score_thresh = INFINITY;
     }
-    // cross entropy with the byte mask: the score kernel also leaves what the threshold rule gives (OhemEarly)
+    // with the byte mask the score pass also leaves what the threshold rule gives (OhemEarly)
     OhemEarly ev{nullptr, nullptr, nullptr, nullptr, score_thresh};
     unsigned early_blocks = 0;
-    if (!large_margin && kept) {
+    if (kept) {
         const int64_t slots = early_blocks_max(P);
         ev.kept = kept;
         ev.sum = reinterpret_cast<float *>(static_cast<char *>(workspace) + select_workspace(P) + align256(8 * tiles));
@@ -901,7 +871,7 @@ static int ohem_loss_forward(bool large_margin, float lam, const void *logits, i
     }
     if (large_margin)
         rc = lmargin_forward_with_scores(logits, dtype, labels, pixel_loss, scores, n_size, dimsize, m_size, ignore_index,
-                                         lam, st, none);
+                                         lam, st, none, &ev, &early_blocks);
     else
         rc = launch_scores(logits, dtype, labels, scores, pixel_loss, n_size, dimsize, m_size, ignore_index, st,
                            static_cast<uint32_t *>(workspace), none, &ev, &early_blocks);

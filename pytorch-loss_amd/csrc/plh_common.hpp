@@ -582,11 +582,44 @@ __device__ inline void finish_block(const float *__restrict__ sums, const int *_
 void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int64_t *count_out, FinishMode mode,
                      int64_t fixed_count, hipStream_t stream);
 
+// What the score pass of an OHEM loss forward (ohem.hip: the cross-entropy score kernel; the large-margin forward kernel
+// that also writes scores) leaves besides scores and losses, for the case that the threshold
+// rule decides the selection (at least n_min pixels score within the threshold, so "beyond the n_min lowest" holds
+// for every pixel above it): the byte mask and the per-block sums of that rule, and per block the number of pixels
+// whose score, capped at 1 like the selection's keys, lies within the threshold. The first histogram kernel adds those
+// numbers up; when they reach n_min it raises kEarlyFlag in the selection's state and every later kernel of the
+// selection returns at once (the finish then adds up these sums instead of the relabelling pass's).
+struct OhemEarly {
+    uint8_t *kept;      // [P]; nullptr: nothing of this is produced
+    float *sum;         // [blocks of the score kernel]
+    int *cnt;           // [blocks]
+    int *below;         // [blocks]
+    float thresh;
+};
+
+// One byte per pixel for this thread's V pixels (nv of them exist).
+template <int V>
+__device__ __forceinline__ void store_kept(uint8_t *kept, int64_t pix, int nv, const bool (&kp)[V]) {
+    typedef unsigned short u16_a1 __attribute__((aligned(1)));
+    typedef unsigned u32_a1 __attribute__((aligned(1)));
+    if (nv == V && V == 2) {
+        *reinterpret_cast<u16_a1 *>(kept + pix) = (unsigned short)((unsigned)kp[0] | ((unsigned)kp[V - 1] << 8));
+    } else if (nv == V && V == 4) {
+        *reinterpret_cast<u32_a1 *>(kept + pix) =
+            (unsigned)kp[0] | ((unsigned)kp[1 % V] << 8) | ((unsigned)kp[2 % V] << 16) | ((unsigned)kp[3 % V] << 24);
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k)
+            if (k < nv) kept[pix + k] = kp[k] ? 1 : 0;
+    }
+}
+
 // Defined in lmargin.hip: plh_lmargin_forward that also writes each pixel's softmax probability at
 // its label (1 where there is no target) into `scores`.
 int lmargin_forward_with_scores(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *scores,
                                 int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float lam,
-                                hipStream_t stream, float no_target_score = 1.f);
+                                hipStream_t stream, float no_target_score = 1.f, const OhemEarly *early = nullptr,
+                                unsigned *early_blocks = nullptr);
 
 // ---- the "regs" launch shape ---------------------------------------------------
 // 256 threads per block, V pixels per thread; block b of the grid owns the pixel tile

@@ -295,14 +295,14 @@ def test_kept_mask_is_the_relabelling(native, shape, scale, thresh, div, lam):
     assert torch.equal(got, want)               # -0.0 == 0.0: a dropped pixel's products may carry a sign
 
 
+@pytest.mark.parametrize("lam", [None, 0.3], ids=["ce", "lmargin"])
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("shape", [(2, 19, 32, 32), (2, 19, 40, 52), (2, 19, 65, 67), (3, 7, 9, 11), (500, 23), (2, 40, 24, 24)],
                          ids=["uniform", "general", "per_image", "one_pixel", "rows", "split"])
-def test_threshold_rule_from_the_score_kernel_switches_exactly_at_n_min(native, shape, dt):
-    """The cross-entropy forward with the byte mask takes mask, sum and count from its score kernel when at least
-    n_min pixels score within the threshold, and from the selection otherwise: n_min one below, at and one above
-    that number of pixels (and 0, and far above) give the relabelling of plh_ohem_score_label and the mean cross
-    entropy over it."""
+def test_threshold_rule_from_the_score_kernel_switches_exactly_at_n_min(native, shape, dt, lam):
+    """The forwards with the byte mask take mask, sum and count from their score pass when at least n_min pixels
+    score within the threshold, and from the selection otherwise: n_min one below, at and one above that number of
+    pixels (and 0, and far above) give the relabelling of plh_ohem_score_label and the mean loss over it."""
     x = synth.normal(137, 1, shape, 0.0, 2.5)
     y = synth.seg_labels(137, shape[:1] + shape[2:], shape[1], 255, 0.1)
     xt, yt = dev(x).to(dt), dev(y)
@@ -312,12 +312,16 @@ def test_threshold_rule_from_the_score_kernel_switches_exactly_at_n_min(native, 
     within = int((np.minimum(scores, 1.0) <= thresh).sum())
     assert 2 < within < y.size - 2
     for n_min in (0, within - 1, within, within + 1, within + (y.size - within) // 2, y.size - 1):
-        loss, n_valid, args, kept = native.ohem_ce_forward(xt, yt, 255, thresh, n_min)
+        loss, n_valid, args, kept = native.ohem_ce_forward(xt, yt, 255, thresh, n_min, lam)
         new_labels = native.ohem_score_label(xt, yt, 255, thresh, n_min)
         assert torch.equal(kept[:y.size].view(y.shape).bool(), new_labels != 255), n_min
         assert int(n_valid.item()) == int((new_labels != 255).sum().item()), n_min
-        want = torch.nn.functional.cross_entropy(torch.from_numpy(xw).double(), new_labels.cpu(), ignore_index=255,
-                                                 reduction="mean").item()
+        if lam is None:
+            want = torch.nn.functional.cross_entropy(torch.from_numpy(xw).double(), new_labels.cpu(), ignore_index=255,
+                                                     reduction="mean").item()
+        else:
+            nl = new_labels.cpu().numpy()
+            want = oracle.lmargin_forward(xw.astype(np.float64), nl, lam, 255).sum() / max(int((nl != 255).sum()), 1)
         tol = 1e-5 if dt == torch.float32 else 2.0 ** -8          # the loss comes back in the logits' type
         assert abs(loss.float().item() - want) <= tol * abs(want), (n_min, loss.item(), want)
         # with more than `within` positions below n_min, pixels above the threshold stay
