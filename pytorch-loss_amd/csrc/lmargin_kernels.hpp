@@ -323,40 +323,26 @@ __global__ __launch_bounds__(kSplitBlock) void lm_fwd_split(const T *__restrict_
         }
     }
     __syncthreads();
-    if (wave != 0) return;
+    if (wave >= V) return;                              // wavefront k finishes pixel k of every lane 
     const int used = (p.C + KW - 1) / KW;
-    float out[V], score[V];
-    float mine = 0.f;
-    int cnt = 0;
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        const LmSplitStats<V> st = lm_split_combine<V, true>(parts, lane * V + k, used);
-        const float m_all = fmaxf(st.m_no, st.x_y);
-        const float t_all = fast_exp(st.m_no - m_all);
-        const float e_y = fast_exp(st.x_y - m_all);
-        const float s_all = __builtin_fmaf(st.s_no, t_all, e_y);
-        const float lse_no = fast_log(st.s_no);
-        const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));
-        const float margin = st.sum_qt - lse_no - p.coeff * (st.sum_t - others * lse_no);
-        const float acc = p.half_lam * margin - (st.x_y - m_all) + fast_log(s_all);
-        const bool valid = at.live && !ign;
-        out[k] = valid ? acc : 0.f;
-        score[k] = (tgt < 0) ? p.no_target_score : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
-        mine += out[k];
-        cnt += valid ? 1 : 0;
-    }
-    if (at.live && loss) at.store_f32(loss, out);
-    if (at.live && p.scores) at.template store_f32<true>(p.scores, score);
-    if (Reduce) {
-        const float bs = group_reduce<64>(mine, OpSum());
-        const float bc = group_reduce<64>((float)cnt, OpSum());
-        if (lane == 0) {
-            part.sum[blockIdx.x] = bs;
-            part.cnt[blockIdx.x] = (int)bc;
-        }
-    }
+    bool ign;
+    PLH_SPLIT_MY_LABEL(my_lb, lb, wave, V)
+    const int tgt = narrow_label(my_lb, p.ignore, p.C, ign);
+    const LmSplitStats<V> st = lm_split_combine<V, true>(parts, lane * V + wave, used);
+    const float m_all = fmaxf(st.m_no, st.x_y);
+    const float t_all = fast_exp(st.m_no - m_all);
+    const float e_y = fast_exp(st.x_y - m_all);
+    const float s_all = __builtin_fmaf(st.s_no, t_all, e_y);
+    const float lse_no = fast_log(st.s_no);
+    const float others = (float)(p.C - 1 - ((tgt < 0) ? -1 : 0));
+    const float margin = st.sum_qt - lse_no - p.coeff * (st.sum_t - others * lse_no);
+    const float acc = p.half_lam * margin - (st.x_y - m_all) + fast_log(s_all);
+    const bool here = at.live && wave < at.nv;
+    const bool valid = here && !ign;
+    const float out = valid ? acc : 0.f;
+    if (here && loss) loss[at.pix + wave] = out;
+    if (here && p.scores) p.scores[at.pix + wave] = (tgt < 0) ? p.no_target_score : fminf(e_y * __builtin_amdgcn_rcpf(s_all), 1.f);
+    if (Reduce) split_block_partials<V>(out, valid, wave, lane, part);
 }
 
 template <class T, int KW, int V, bool PerImage = false>

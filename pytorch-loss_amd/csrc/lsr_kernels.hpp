@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 // wavefront reduces its part of a pixel's slice, the parts meet in LDS:
 //   forward   (m_w, s_w, d_w, y_w) = max, sum_j exp(x_j - m_w), sum_j (x_j - m_w), target logit if it is here;
 //             with M = max_w m_w:  S = sum_w s_w exp(m_w - M),  sum_j (x_j - M) = sum_w d_w + n_w (m_w - M),
-//             and wavefront 0 forms the loss as the regs kernel does;
+//             and wavefront k forms the loss of pixel k of every lane as the regs kernel does;
 //   backward  (c_w, s_w) in the base-2 domain, c_w = fl(m_w log2e), s_w = sum_j 2^(x_j log2e - c_w); every
 //             wavefront then evaluates 2^(x_j log2e - max_w c_w) / sum_w s_w 2^(c_w - max c) for its channels.
 
@@ -210,44 +210,31 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
         }
     }
     __syncthreads();
-    if (wave != 0) return;
     const int used = (p.C + KW - 1) / KW;               // wavefronts that hold channels
-    float out[V];
-    float mine = 0.f;
-    int cnt = 0;
     const float fc = (float)p.C;
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        const int q = lane * V + k;
-        float M = parts[0][0][q];
-        for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
-        float S = 0.f, D = 0.f, x_y = 0.f;
-        for (int w = 0; w < used; ++w) {
-            const float shift = parts[0][w][q] - M;
-            S = __builtin_fmaf(parts[1][w][q], fast_exp(shift), S);
-            D += __builtin_fmaf((float)split_count(w, KW, p.C), shift, parts[2][w][q]);
-            x_y += parts[3][w][q];
-        }
-        const float lse = fast_log(S);
-        const float all = D - fc * lse;
-        const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - M) - lse) : 0.f;
-        const float acc = -(p.w_neg * all + hot);
-        const bool valid = at.live && !ign;
-        out[k] = valid ? acc : 0.f;
-        mine += out[k];
-        cnt += valid ? 1 : 0;
+    if (wave >= V) return;                              // wavefront k finishes pixel k of every lane
+    bool ign;
+    PLH_SPLIT_MY_LABEL(my_lb, lb, wave, V)
+    const int tgt = narrow_label(my_lb, p.ignore, p.C, ign);
+    const int q = lane * V + wave;
+    float M = parts[0][0][q];
+    for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
+    float S = 0.f, D = 0.f, x_y = 0.f;
+    for (int w = 0; w < used; ++w) {
+        const float shift = parts[0][w][q] - M;
+        S = __builtin_fmaf(parts[1][w][q], fast_exp(shift), S);
+        D += __builtin_fmaf((float)split_count(w, KW, p.C), shift, parts[2][w][q]);
+        x_y += parts[3][w][q];
     }
-    if (at.live && loss) at.store_f32(loss, out);
-    if (Reduce) {
-        const float bs = group_reduce<64>(mine, OpSum());
-        const float bc = group_reduce<64>((float)cnt, OpSum());      // at most 256 per block: exact in fp32
-        if (lane == 0) {
-            part.sum[blockIdx.x] = bs;
-            part.cnt[blockIdx.x] = (int)bc;
-        }
-    }
+    const float lse = fast_log(S);
+    const float all = D - fc * lse;
+    const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - M) - lse) : 0.f;
+    const float acc = -(p.w_neg * all + hot);
+    const bool here = at.live && wave < at.nv;
+    const bool valid = here && !ign;
+    const float out = valid ? acc : 0.f;
+    if (here && loss) loss[at.pix + wave] = out;
+    if (Reduce) split_block_partials<V>(out, valid, wave, lane, part);
 }
 
 template <class T, int KW, int V, bool PerImage = false>

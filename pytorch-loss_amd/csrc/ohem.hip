@@ -153,26 +153,21 @@ __global__ __launch_bounds__(kSplitBlock) void ohem_scores_split(const T *__rest
         }
     }
     __syncthreads();
-    if (wave != 0 || !at.live) return;
+    if (wave >= V || !at.live || wave >= at.nv) return;     // wavefront k finishes pixel k of every lane
     const int used = (C + KW - 1) / KW;
-    float out[V], loss[V];
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], ignore, C, ign);
-        const int q = lane * V + k;
-        float M = parts[0][0][q];
-        for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
-        float S = 0.f, x_y = -INFINITY;
-        for (int w = 0; w < used; ++w) {
-            S = __builtin_fmaf(parts[1][w][q], fast_exp(parts[0][w][q] - M), S);
-            x_y = fmaxf(x_y, parts[2][w][q]);
-        }
-        out[k] = (tgt < 0) ? none : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
-        loss[k] = (tgt < 0) ? 0.f : fast_log(S) + (M - x_y);
+    bool ign;
+    PLH_SPLIT_MY_LABEL(my_lb, lb, wave, V)
+    const int tgt = narrow_label(my_lb, ignore, C, ign);
+    const int q = lane * V + wave;
+    float M = parts[0][0][q];
+    for (int w = 1; w < used; ++w) M = fmaxf(M, parts[0][w][q]);
+    float S = 0.f, x_y = -INFINITY;
+    for (int w = 0; w < used; ++w) {
+        S = __builtin_fmaf(parts[1][w][q], fast_exp(parts[0][w][q] - M), S);
+        x_y = fmaxf(x_y, parts[2][w][q]);
     }
-    at.template store_f32<true>(scores, out);
-    if (ce) at.template store_f32<true>(ce, loss);
+    scores[at.pix + wave] = (tgt < 0) ? none : fminf(fast_exp(x_y - M) * __builtin_amdgcn_rcpf(S), 1.f);
+    if (ce) ce[at.pix + wave] = (tgt < 0) ? 0.f : fast_log(S) + (M - x_y);
 }
 
 // Any channel count: a lane per pixel, two sweeps over the slice (the second one hits cache).

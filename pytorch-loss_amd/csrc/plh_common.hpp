@@ -1286,6 +1286,37 @@ __device__ __forceinline__ float block_sum_256(float v, float *lds4) {
     return r;
 }
 
+// The forwards of the split shape end with one wavefront's worth of work per pixel of a lane (combine the 8
+// wavefronts' statistics, a logarithm or two). Wavefront k of a block does that for pixel k of every lane, so the
+// tail of a block is one pixel long instead of V (16-bit elements, V = 4: LSR forward (8,150,512,512) 0.164 -> 0.138 ms).
+// PLH_SPLIT_MY_LABEL picks the label of that pixel (in the kernel's own body: handed to a function by reference, the
+// array of labels ends up in scratch memory); split_block_partials forms the block's sum and count from the V
+// finishing wavefronts (all of them call it, the others have left the kernel).
+#define PLH_SPLIT_MY_LABEL(my_lb, lb, wave, V)                                   \
+    int64_t my_lb = lb[0];                                                       \
+    _Pragma("unroll") for (int k_ = 1; k_ < V; ++k_) my_lb = ((wave) == k_) ? lb[k_] : my_lb;
+template <int V>
+__device__ __forceinline__ void split_block_partials(float out, bool counted, int wave, int lane, Partials part) {
+    __shared__ float fin[2][8];
+    const float bs = group_reduce<64>(out, OpSum());
+    const float bc = group_reduce<64>(counted ? 1.f : 0.f, OpSum());
+    if (lane == 0) {
+        fin[0][wave] = bs;
+        fin[1][wave] = bc;
+    }
+    __syncthreads();                                // the V wavefronts that are still here
+    if (threadIdx.x == 0) {
+        float ts = fin[0][0], tc = fin[1][0];
+#pragma unroll
+        for (int k = 1; k < V; ++k) {
+            ts += fin[0][k];
+            tc += fin[1][k];
+        }
+        part.sum[blockIdx.x] = ts;
+        part.cnt[blockIdx.x] = (int)tc;             // at most 256 per block: exact in fp32
+    }
+}
+
 __device__ __forceinline__ float block_max_256(float v, float *lds4) {
     v = group_reduce<64>(v, OpMax());
     const int wave = threadIdx.x >> 6;

@@ -349,34 +349,21 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
         }
     }
     __syncthreads();
-    if (wave != 0) return;
+    if (wave >= V) return;                              // wavefront k finishes pixel k of every lane 
     const int used = (p.C + KW - 1) / KW;
-    float out[V];
-    float mine = 0.f;
-    int cnt = 0;
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-        bool ign;
-        const int tgt = narrow_label(lb[k], p.ignore, p.C, ign);
-        float s = 0.f, f_y = 0.f;
-        for (int w = 0; w < used; ++w) {
-            s += parts[0][w][lane * V + k];
-            f_y += parts[1][w][lane * V + k];
-        }
-        const bool valid = at.live && !ign && tgt >= 0;
-        out[k] = valid ? logf(s) - logf(f_y) : 0.f;
-        mine += out[k];
-        cnt += (at.live && !ign) ? 1 : 0;
+    bool ign;
+    PLH_SPLIT_MY_LABEL(my_lb, lb, wave, V)
+    const int tgt = narrow_label(my_lb, p.ignore, p.C, ign);
+    float s = 0.f, f_y = 0.f;
+    for (int w = 0; w < used; ++w) {
+        s += parts[0][w][lane * V + wave];
+        f_y += parts[1][w][lane * V + wave];
     }
-    if (at.live && loss) at.store_f32(loss, out);
-    if (Reduce) {
-        const float bs = group_reduce<64>(mine, OpSum());
-        const float bc = group_reduce<64>((float)cnt, OpSum());
-        if (lane == 0) {
-            part.sum[blockIdx.x] = bs;
-            part.cnt[blockIdx.x] = (int)bc;
-        }
-    }
+    const bool here = at.live && wave < at.nv;
+    const bool valid = here && !ign && tgt >= 0;
+    const float out = valid ? logf(s) - logf(f_y) : 0.f;
+    if (here && loss) loss[at.pix + wave] = out;
+    if (Reduce) split_block_partials<V>(out, here && !ign, wave, lane, part);
     };
     if (p.order == 2) run(std::integral_constant<int, 2>());
     else run(std::integral_constant<int, 4>());
