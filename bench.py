@@ -435,6 +435,22 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         sb = lambda: lib.plh_taylor_softmax_backward(P(y_out), P(x), tag, P(grad), n, c, m, 4, 1, st())
         assert sf() == 0 and sb() == 0
         legs += [("log_softmax_forward", sf, 2 * eb), ("log_softmax_backward", sb, 3 * eb)]
+    if name == "lsr" and lib.plh_lsr_saves_lse(tag, n, c, m):
+        # channel planes of odd length: the module's own pair of entry points - the reduced forward that keeps every
+        # pixel's log-sum-exp and the backward that forms the gradient from it plane by plane (one scalar upstream)
+        E, Pn = n * c * m, n * m
+        lse = torch.empty(Pn, dtype=torch.float32, device=x.device)
+        one_loss = torch.empty((), dtype=torch.float32, device=x.device)
+        n_valid = torch.empty((), dtype=torch.int64, device=x.device)
+        rws_bytes = int(lib.plh_reduce_workspace_bytes(Pn))
+        rws = torch.empty(rws_bytes, dtype=torch.uint8, device=x.device)
+        up = torch.ones((), dtype=torch.float32, device=x.device)
+        fl = lambda: lib.plh_lsr_forward_reduced_lse(P(x), tag, P(labels), P(lse), P(one_loss), P(n_valid), 1, P(rws), rws_bytes,
+                                                     n, c, m, 255, 0.1, st())
+        bl = lambda: lib.plh_lsr_backward_scaled_lse(P(x), tag, P(labels), P(lse), None, P(up), 1.0, P(n_valid), P(grad),
+                                                     n, c, m, 255, 0.1, st())
+        assert fl() == 0 and bl() == 0
+        legs += [("forward_keeping_lse", fl, 4 * E + 8 * Pn + 4 * Pn), ("backward_from_lse", bl, 8 * E + 8 * Pn + 4 * Pn)]
     if name == "lovasz":
         # the same forward with its sort passes in the decoupled look-back form (an entry point of its own)
         lb_bytes = int(lib.plh_lovasz_lookback_workspace_bytes(n, c, m))

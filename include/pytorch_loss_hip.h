@@ -102,6 +102,30 @@ int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *la
                             int64_t n_size, int64_t dimsize, int64_t m_size,
                             int64_t ignore_index, float smooth, void *stream);
 
+/* The module step on channel planes of odd length (513 x 513, 769 x 769 crops; no counterpart in the reference, whose
+ * backward recomputes the softmax, csrc/lsr_kernel.cu:139-225). plh_lsr_saves_lse says (1 / 0) whether it applies to
+ * these sizes: fp32 logits, m_size odd and at least 4096, dimsize small enough for the register-resident forward on
+ * such planes (24). Then plh_lsr_forward_reduced_lse is plh_lsr_forward_reduced that also leaves every pixel's
+ * log-sum-exp in lse_out (n_size*m_size floats; it writes no per-pixel losses), and plh_lsr_backward_scaled_lse is
+ * plh_lsr_backward_scaled that forms the gradient from it, sumw*exp(x - lse) - w, plane by plane in each plane's own
+ * cache lines (`kept`: optional byte mask as in plh_lsr_backward_kept, else NULL). The gradient equals the
+ * recomputing kernels' to rounding (relative 1e-6). When logits and grad_logits do not sit at the same offset into a
+ * 128-byte line the recomputing kernel runs and `lse` is not read. PLH_ERR_BAD_SIZE for sizes that
+ * plh_lsr_saves_lse answers with 0. */
+int plh_lsr_saves_lse(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size);
+
+int plh_lsr_forward_reduced_lse(const void *logits, int32_t dtype, const int64_t *labels, float *lse_out,
+                                float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                void *workspace, int64_t workspace_bytes,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t ignore_index, float smooth, void *stream);
+
+int plh_lsr_backward_scaled_lse(const void *logits, int32_t dtype, const int64_t *labels, const float *lse,
+                                const uint8_t *kept, const float *grad_scalar, float scale, const int64_t *divide_by,
+                                void *grad_logits,
+                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                int64_t ignore_index, float smooth, void *stream);
+
 /* plh_lsr_forward_reduced for callers that cannot allocate device memory or bring a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
  * counterpart in the reference. Same arguments and results as plh_lsr_forward_reduced, without the

@@ -41,13 +41,15 @@ PLH_LSR_EXTERN(bf16)
 
 static int backward(const void *logits, int32_t dtype, const int64_t *labels, const Upstream &up, void *grad_logits,
                     int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float smooth,
-                    void *stream) {
+                    void *stream, const float *lse = nullptr) {
     if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
     const int rc = check_slice_args(logits, labels, grad_logits, n_size, dimsize, m_size, dtype_size(dtype),
                                     dtype_size(dtype));
     if (rc != PLH_OK) return rc;
     if (n_size * dimsize * m_size == 0) return PLH_OK;
-    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
+    if (lse && (misaligned(lse, 4) || !lsr_lse_applies(dtype_size(dtype), dimsize, m_size))) return PLH_ERR_BAD_SIZE;
+    LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
+    p.lse = const_cast<float *>(lse);           // read only in the backward
     dispatch_dtype(dtype, [&](auto tag) {
         using T = decltype(tag);
         lsr_backward_typed<T>(static_cast<const T *>(logits), labels, up, static_cast<T *>(grad_logits), p,
@@ -76,12 +78,12 @@ extern "C" int plh_lsr_forward(const void *logits, int32_t dtype, const int64_t 
     return check_launch();
 }
 
-extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
-                                       float *loss_out, int64_t *n_valid_out, int32_t mean,
-                                       void *workspace, int64_t workspace_bytes,
-                                       int64_t n_size, int64_t dimsize, int64_t m_size,
-                                       int64_t ignore_index, float smooth, void *stream) {
+static int forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses, float *lse_out,
+                           float *loss_out, int64_t *n_valid_out, int32_t mean, void *workspace, int64_t workspace_bytes,
+                           int64_t n_size, int64_t dimsize, int64_t m_size, int64_t ignore_index, float smooth,
+                           void *stream) {
     if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    if (lse_out && (misaligned(lse_out, 4) || !lsr_lse_applies(dtype_size(dtype), dimsize, m_size))) return PLH_ERR_BAD_SIZE;
     int rc = check_slice_args(logits, labels, loss_out, n_size, dimsize, m_size, dtype_size(dtype), 4);
     if (rc != PLH_OK) return rc;
     Partials part;
@@ -91,7 +93,8 @@ extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const 
     hipStream_t st = (hipStream_t)stream;
     unsigned blocks = 0;
     if (n_size * dimsize * m_size != 0) {
-        const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
+        LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, dtype_size(dtype));
+        p.lse = lse_out;
         dispatch_dtype(dtype, [&](auto tag) {
             using T = decltype(tag);
             blocks = lsr_forward_typed<T>(static_cast<const T *>(logits), labels, losses, part, true, p, st);
@@ -99,6 +102,30 @@ extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const 
     }
     finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
     return check_launch();
+}
+
+extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
+                                       float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                       void *workspace, int64_t workspace_bytes,
+                                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                                       int64_t ignore_index, float smooth, void *stream) {
+    return forward_reduced(logits, dtype, labels, losses, nullptr, loss_out, n_valid_out, mean, workspace, workspace_bytes,
+                           n_size, dimsize, m_size, ignore_index, smooth, stream);
+}
+
+extern "C" int plh_lsr_saves_lse(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size) {
+    return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 &&
+           lsr_lse_applies(dtype_size(dtype), dimsize, m_size) ? 1 : 0;
+}
+
+extern "C" int plh_lsr_forward_reduced_lse(const void *logits, int32_t dtype, const int64_t *labels, float *lse_out,
+                                           float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                           void *workspace, int64_t workspace_bytes,
+                                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                                           int64_t ignore_index, float smooth, void *stream) {
+    if (!lse_out && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
+    return forward_reduced(logits, dtype, labels, nullptr, lse_out, loss_out, n_valid_out, mean, workspace, workspace_bytes,
+                           n_size, dimsize, m_size, ignore_index, smooth, stream);
 }
 
 extern "C" int plh_lsr_forward_reduced_static(const void *logits, int32_t dtype, const int64_t *labels, float *losses,
@@ -150,4 +177,15 @@ extern "C" int plh_lsr_backward_kept(const void *logits, int32_t dtype, const in
     if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, divide_by, scale, kept};
     return backward(logits, dtype, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream);
+}
+
+extern "C" int plh_lsr_backward_scaled_lse(const void *logits, int32_t dtype, const int64_t *labels, const float *lse,
+                                           const uint8_t *kept, const float *grad_scalar, float scale,
+                                           const int64_t *divide_by, void *grad_logits,
+                                           int64_t n_size, int64_t dimsize, int64_t m_size,
+                                           int64_t ignore_index, float smooth, void *stream) {
+    if (n_size * dimsize * m_size != 0 && (!grad_scalar || !lse)) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale, kept};
+    return backward(logits, dtype, labels, up, grad_logits, n_size, dimsize, m_size, ignore_index, smooth, stream, lse);
 }

@@ -24,6 +24,9 @@ struct LsrParams {
     int64_t ignore;
     float w_pos, w_neg, sumw;
     unsigned xcd_run;   // tile permutation run length (xcd_run_for)
+    // Per-pixel log-sum-exp of the logits, fp32 [P]. Forward (the per-image form on fp32 logits): written when set.
+    // Backward: when set, lsr_bwd_planes forms the gradient from it plane by plane (see there).
+    float *lse = nullptr;
 };
 
 // ---------------------------------------------------------------- regs ----
@@ -54,6 +57,9 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     float mine = 0.f;
     int cnt = 0;
     const float fc = (float)p.C;
+    // the per-image form on fp32 logits also leaves each pixel's log-sum-exp where it is given a place (LsrParams::lse)
+    constexpr bool kMayLse = Form == kPerImage && sizeof(T) == 4;
+    float lse_abs[kMayLse ? V : 1];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
         bool ign;
@@ -71,6 +77,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
                 x_y = (tgt == j) ? xv[j] : x_y;
             }
         const float lse = (__builtin_amdgcn_logf(s) - r) * kLn2;
+        if constexpr (kMayLse) lse_abs[k] = mx + lse;
         const float all = (sx - fc * mx) - fc * lse;
         // no target channel (label outside [0, C)): every weight is w_neg
         const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - mx) - lse) : 0.f;
@@ -81,6 +88,9 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
         cnt += valid ? 1 : 0;
     }
     if (at.live && loss) at.store_f32(loss, out);
+    if constexpr (kMayLse) {
+        if (p.lse && at.live) at.store_f32_cached(p.lse, lse_abs);      // the backward reads it next
+    }
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);   // at most 1024 per block: exact in fp32
@@ -158,6 +168,103 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
     for (int j = 0; j < CP; ++j)
         if (chan_ok<CP>(j, p.C)) raw[j] = raw[j] & mask;
     at.store_slice(grad, p.C, p.m_size, raw);
+}
+
+// -------------------------------------------------------------- planes ----
+// Backward from the forward's per-pixel log-sum-exp, for channel planes that start on element boundaries only (odd
+// lengths: 513 x 513, 769 x 769 crops). With lse[p] at hand the gradient is elementwise,
+//   g[c][p] = gk (sumw exp(x[c][p] - lse[p]) - w(label[p] == c)),
+// so nothing ties the thread that writes an element to the other channels of its pixel, and every plane can be
+// walked in its OWN cache lines: a block takes 1024 pixels of an image, and in plane c its 256 threads move the
+// 32 whole lines that begin at the tile's first pixel shifted back by the plane's offset into its line (0..31
+// elements) - 16 aligned bytes per lane, loads and stores alike; lines are shared only where two planes meet. (The
+// register-resident kernel has one pixel set for all channels, and with it runs that begin and end inside lines in
+// every plane but one: 57 % of peak at (16,19,769,769) against 75 % here.) The pixels' (lse, label) pairs - the
+// tile's and the 32 before it - are staged in LDS once, transposed by pixel index mod 4, so that the four reads of
+// a lane's shifted window are conflict-free for every shift. One scalar upstream gradient (the module's 'mean' /
+// 'sum'), optionally the byte mask of an OHEM selection; fp32 logits whose gradient tensor sits at the same offset
+// into a 128-byte line.
+constexpr int kPlaneTile = 1024, kPlaneHalo = 32;
+struct PlanePixel {
+    float lse;
+    int lab;            // the label, -1 for a pixel that takes no part, C for one without a target channel
+};
+
+__device__ __forceinline__ float plane_grad(float x, PlanePixel px, int c, float scale, float n_pos, float n_neg) {
+    const float e = __builtin_amdgcn_exp2f((x - px.lse) * kLog2e);
+    const float g = __builtin_fmaf(e, scale, (px.lab == c) ? n_pos : n_neg);
+    return px.lab < 0 ? 0.f : g;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                      const Upstream up, T *__restrict__ grad, const LsrParams p,
+                                                      int tiles) {
+    static_assert(sizeof(T) == 4, "fp32 logits");
+    __shared__ PlanePixel pairs[4][(kPlaneTile + kPlaneHalo) / 4];
+    const int64_t M = p.m_size;
+    const int64_t n = blockIdx.x / tiles;
+    const int t = (int)(blockIdx.x - n * tiles);
+    const int l = threadIdx.x;
+    const int64_t p_first = (int64_t)t * kPlaneTile - kPlaneHalo;       // image-local pixel of staged entry 0
+    for (int i = l; i < kPlaneTile + kPlaneHalo; i += 256) {
+        const int64_t q = p_first + i;
+        PlanePixel px{0.f, -1};
+        if (q >= 0 && q < M) {
+            const int64_t at = n * M + q;
+            const int64_t lb = lab[at];
+            const bool dropped = lb == p.ignore || (up.keep && up.keep[at] == 0);
+            px.lse = p.lse[at];
+            px.lab = dropped ? -1 : ((lb < 0 || lb >= p.C) ? p.C : (int)lb);
+        }
+        pairs[i & 3][i >> 2] = px;
+    }
+    float gk = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk = gk / (float)(*up.divide_by);
+    const float scale = p.sumw * gk, n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+    __syncthreads();
+    constexpr int U = 4;                // planes in flight per thread
+    for (int c0 = 0; c0 < p.C; c0 += U) {
+        plh_f4 xv[U];
+        int64_t q[U], plane[U];
+        bool full[U];
+        int first[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u < p.C ? c0 + u : p.C - 1;
+            plane[u] = (n * p.C + c) * M;
+            const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) >> 2) & 31u);   // the plane's offset into its line
+            first[u] = kPlaneHalo + 4 * l - shift;                  // staged index of this lane's first pixel
+            q[u] = (int64_t)t * kPlaneTile - shift + 4 * l;
+            full[u] = q[u] >= 0 && q[u] + 3 < M;
+            xv[u] = __builtin_nontemporal_load(reinterpret_cast<const plh_f4 *>(x + plane[u] + (full[u] ? q[u] : 0)));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u;
+            if (c >= p.C) break;
+            const int i0 = first[u];
+            if (full[u]) {
+                plh_f4 g;
+                g.x = plane_grad(xv[u].x, pairs[(i0 + 0) & 3][(i0 + 0) >> 2], c, scale, n_pos, n_neg);
+                g.y = plane_grad(xv[u].y, pairs[(i0 + 1) & 3][(i0 + 1) >> 2], c, scale, n_pos, n_neg);
+                g.z = plane_grad(xv[u].z, pairs[(i0 + 2) & 3][(i0 + 2) >> 2], c, scale, n_pos, n_neg);
+                g.w = plane_grad(xv[u].w, pairs[(i0 + 3) & 3][(i0 + 3) >> 2], c, scale, n_pos, n_neg);
+                __builtin_nontemporal_store(g, reinterpret_cast<plh_f4 *>(grad + plane[u] + q[u]));
+            } else {                    // the two ends of a plane, element by element
+                for (int k = 0; k < 4; ++k)
+                    if (q[u] + k >= 0 && q[u] + k < M)
+                        grad[plane[u] + q[u] + k] = plane_grad(x[plane[u] + q[u] + k], pairs[(i0 + k) & 3][(i0 + k) >> 2], c,
+                                                               scale, n_pos, n_neg);
+            }
+        }
+    }
+}
+
+// Whether the forward leaves the log-sum-exp for these sizes (its per-image form on fp32 logits) and the backward
+// can run plane by plane: channel planes of odd length, long enough for that form, a slice that fits it.
+inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
+    return elem_bytes == 4 && (m_size & 1) && image_form_pays<float>((int)dimsize, m_size) && dimsize >= 1;
 }
 
 // --------------------------------------------------------------- split ----
@@ -935,6 +1042,18 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    if constexpr (sizeof(T) == 4) {
+        // from the forward's log-sum-exp, plane by plane: one scalar upstream gradient, logits and gradient at the same
+        // offset into a 128-byte line (whole lines of the one are whole lines of the other) and 16-byte aligned at that
+        if (p.lse && !go_vec && lsr_lse_applies(sizeof(T), p.C, p.m_size) &&
+            ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 127) == 0 &&
+            !misaligned(logits, 4) && p.P / p.m_size * ceil_div(p.m_size + kPlaneHalo - 1, (int64_t)kPlaneTile) < ((int64_t)1 << 31)) {
+            const int tiles = (int)ceil_div(p.m_size + kPlaneHalo - 1, (int64_t)kPlaneTile);
+            hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)(p.P / p.m_size * tiles)), dim3(256), 0, st, logits, labels,
+                               up, grad_logits, p, tiles);
+            return;
+        }
+    }
     switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, go_vec, nullptr, true, true, true,
                        kImageFormMaxChannels<T>)) {
         case Shape::RegsVec: launch_bwd_regs<T, V>(logits, labels, up, grad_logits, p, st); break;

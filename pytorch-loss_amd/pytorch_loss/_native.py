@@ -48,6 +48,9 @@ _SIGNATURES = {
     "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_lsr_saves_lse": (ctypes.c_int, [_i32, _i64, _i64, _i64]),
+    "plh_lsr_forward_reduced_lse": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lsr_backward_scaled_lse": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lovasz_lookback_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward_lookback": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_lovasz_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
@@ -329,6 +332,32 @@ def lsr_forward_reduced(logits, labels, ignore_index, smooth, mean, args=None):
 def lsr_backward_scaled(logits, labels, ignore_index, smooth, grad_scalar, divide_by=None, args=None):
     return _pixel_backward_scaled("plh_lsr_backward_scaled", args or lsr_args(logits, labels), ignore_index, smooth,
                                   grad_scalar, divide_by)
+
+
+def lsr_forward_reduced_lse(logits, labels, ignore_index, smooth, mean, args=None):
+    """lsr_forward_reduced that also keeps every pixel's log-sum-exp where the library's backward can use it (fp32
+    logits on channel planes of odd length, see plh_lsr_saves_lse). -> (loss, n_valid, lse or None)."""
+    a = args or lsr_args(logits, labels)
+    if a.x.numel() == 0 or not load().plh_lsr_saves_lse(a.tag, a.n, a.c, a.m):
+        return _pixel_forward_reduced("plh_lsr_forward_reduced", a, ignore_index, smooth, mean) + (None,)
+    dev = a.x.device
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    n_valid = torch.empty((), dtype=torch.int64, device=dev)
+    lse = torch.empty((a.n * a.m,), dtype=torch.float32, device=dev)
+    ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
+    _call(a.x, "plh_lsr_forward_reduced_lse", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(lse), _ptr(loss), _ptr(n_valid),
+          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(smooth))
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, lse
+
+
+def lsr_backward_scaled_lse(lse, ignore_index, smooth, grad_scalar, divide_by, args, kept=None):
+    """The gradient from the forward's log-sum-exp (lsr_forward_reduced_lse); `kept`: optional byte mask."""
+    a = args
+    grad = torch.empty_like(a.x)
+    go = _scalar_f32(grad_scalar)
+    _call(a.x, "plh_lsr_backward_scaled_lse", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(lse), _ptr(kept) if kept is not None else None,
+          _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), a.n, a.c, a.m, int(ignore_index), float(smooth))
+    return _back_to(grad, a.dtype)
 
 
 # -------------------------------------------------------------- lmargin ----

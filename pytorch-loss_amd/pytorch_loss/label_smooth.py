@@ -32,19 +32,29 @@ class _LSRReducedFunction(torch.autograd.Function):
     """'sum' / 'mean' of the per-pixel losses produced inside the forward kernel (per-block
     partials, then a fixed-order finishing kernel), so the module needs no ATen pass over the
     pixels for `losses.sum()` and `(labels != ignore).sum()`; backward folds the scalar
-    upstream gradient and the 1/n_valid of a mean into the gradient kernel."""
+    upstream gradient and the 1/n_valid of a mean into the gradient kernel. On fp32 logits whose channel
+    planes have an odd length (513 x 513, 769 x 769 crops) the forward also keeps every pixel's log-sum-exp
+    (4 bytes per pixel, only when a gradient will be asked for) and the backward forms the gradient from it
+    plane by plane instead of recomputing the softmax (see plh_lsr_backward_scaled_lse)."""
 
     @staticmethod
     def forward(ctx, logits, labels, lb_smooth, lb_ignore, mean):
         ctx.args = args = _native.lsr_args(logits, labels)
-        loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean, args=args)
-        ctx.variables = (logits, labels, lb_ignore, lb_smooth, n_valid if mean else None)
+        lse = None
+        if ctx.needs_input_grad[0]:
+            loss, n_valid, lse = _native.lsr_forward_reduced_lse(logits, labels, lb_ignore, lb_smooth, mean, args=args)
+        else:
+            loss, n_valid = _native.lsr_forward_reduced(logits, labels, lb_ignore, lb_smooth, mean, args=args)
+        ctx.variables = (logits, labels, lb_ignore, lb_smooth, n_valid if mean else None, lse)
         return loss
 
     @staticmethod
     def backward(ctx, grad_output):
-        logits, labels, lb_ignore, lb_smooth, n_valid = ctx.variables
-        grad = _native.lsr_backward_scaled(logits, labels, lb_ignore, lb_smooth, grad_output, n_valid, args=ctx.args)
+        logits, labels, lb_ignore, lb_smooth, n_valid, lse = ctx.variables
+        if lse is not None:
+            grad = _native.lsr_backward_scaled_lse(lse, lb_ignore, lb_smooth, grad_output, n_valid, ctx.args)
+        else:
+            grad = _native.lsr_backward_scaled(logits, labels, lb_ignore, lb_smooth, grad_output, n_valid, args=ctx.args)
         return grad, None, None, None, None
 
 

@@ -86,6 +86,15 @@ def test_arguments_are_rejected_before_any_launch(native):
         assert lib.plh_focal_forward_backward(p, bad, p, p, p, 4, 2.0, 0.25, None) == -7
         assert lib.plh_lovasz_forward(p, bad, lp, p, p, p, need, 2, 19, 64, 255, None) == -7
         assert lib.plh_lovasz_backward(p, p, bad, lp, p, p, 2, 19, 64, 255, None) == -7
+    # the forward that keeps the log-sum-exp and the backward that uses it: where they apply, and refusals elsewhere
+    assert lib.plh_lsr_saves_lse(0, 16, 19, 769 * 769) == 1 and lib.plh_lsr_saves_lse(0, 32, 24, 513 * 513) == 1
+    assert lib.plh_lsr_saves_lse(0, 8, 19, 1024 * 1024) == 0 and lib.plh_lsr_saves_lse(0, 8, 25, 769 * 769) == 0
+    assert lib.plh_lsr_saves_lse(1, 16, 19, 769 * 769) == 0 and lib.plh_lsr_saves_lse(2, 16, 19, 769 * 769) == 0
+    assert lib.plh_lsr_saves_lse(0, 16, 19, 63 * 65) == 0 and lib.plh_lsr_saves_lse(7, 16, 19, 769 * 769) == 0
+    assert lib.plh_lsr_forward_reduced_lse(p, 0, lp, p, p, None, 1, p, 1 << 20, 2, 19, 4096, 255, 0.1, None) == -2
+    assert lib.plh_lsr_forward_reduced_lse(p, 0, lp, None, p, None, 1, p, 1 << 20, 2, 19, 4097, 255, 0.1, None) == -1
+    assert lib.plh_lsr_backward_scaled_lse(p, 0, lp, p, None, p, 1.0, None, p, 2, 19, 4096, 255, 0.1, None) == -2
+    assert lib.plh_lsr_backward_scaled_lse(p, 0, lp, None, None, p, 1.0, None, p, 2, 19, 4097, 255, 0.1, None) == -1
     # online hard example mining
     assert lib.plh_ohem_workspace_bytes(-1) == -2 and lib.plh_ohem_workspace_bytes(1 << 31) == -2
     ohem_need = lib.plh_ohem_workspace_bytes(4096)

@@ -1,0 +1,138 @@
+"""LabelSmoothSoftmaxCEV3 on channel planes of odd length: the forward that keeps every pixel's log-sum-exp
+(plh_lsr_forward_reduced_lse) and the backward that forms the gradient from it plane by plane
+(plh_lsr_backward_scaled_lse), against the oracle and against the kernels that recompute the softmax."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+# (shape, logit scale): planes of 4225 .. 6499 pixels, so a plane spans several 1024-pixel tiles and has both a
+# partly filled first and last cache line; channel counts either side of a group of four planes; one image and several
+SHAPES = [((2, 19, 65, 67), 2.0), ((1, 24, 65, 65), 3.0), ((3, 5, 71, 73), 1.0), ((2, 1, 67, 97), 1.0), ((5, 7, 65, 65), 8.0)]
+
+
+@pytest.fixture(scope="module")
+def native():
+    from pytorch_loss import _native
+    _native.load()
+    return _native
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def inputs(seed, shape, scale, ignore_frac=0.1):
+    x = synth.normal(seed, 1, shape, 0.0, scale)
+    y = synth.seg_labels(seed, shape[:1] + shape[2:], shape[1], 255, ignore_frac)
+    return x, y
+
+
+@pytest.mark.parametrize("shape,scale", SHAPES)
+def test_the_library_says_where_it_applies(native, shape, scale):
+    lib = native.load()
+    n, c = shape[0], shape[1]
+    m = shape[2] * shape[3]
+    assert lib.plh_lsr_saves_lse(0, n, c, m) == 1
+    assert lib.plh_lsr_saves_lse(2, n, c, m) == 0           # 16-bit logits
+    assert lib.plh_lsr_saves_lse(0, n, c, m + 1) == 0       # planes of even length
+    assert lib.plh_lsr_saves_lse(0, n, 25, m) == 0          # more channels than the register-resident forward takes there
+    assert lib.plh_lsr_saves_lse(0, n, c, 4095) == 0        # short planes
+
+
+@pytest.mark.parametrize("mean", [True, False], ids=["mean", "sum"])
+@pytest.mark.parametrize("shape,scale", SHAPES)
+def test_forward_keeps_the_log_sum_exp_and_backward_uses_it(native, shape, scale, mean):
+    x, y = inputs(141, shape, scale)
+    y.reshape(-1)[::97] = shape[1] + 3                       # labels without a target channel, not ignored
+    xt, yt = dev(x), dev(y)
+    loss, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, mean)
+    assert lse is not None and lse.shape == (y.size,)
+    want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).reshape(-1).numpy()
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-6 * np.abs(want_lse).max()
+    loss2, n_valid2 = native.lsr_forward_reduced(xt, yt, 255, 0.1, mean)
+    assert loss.cpu().numpy().tobytes() == loss2.cpu().numpy().tobytes() and int(n_valid.item()) == int(n_valid2.item())
+    up = torch.full((), 0.7, device=xt.device)
+    div = n_valid if mean else None
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, up, div, native.lsr_args(xt, yt))
+    want = native.lsr_backward_scaled(xt, yt, 255, 0.1, up, div)
+    ref = want.abs().max().item()
+    assert (got - want).abs().max().item() <= 2e-6 * ref
+    flat = y.reshape(shape[0], -1)
+    g = got.cpu().numpy().reshape(shape[0], shape[1], -1)
+    assert not g.transpose(0, 2, 1)[flat == 255].any()      # exact zeros where ignored
+    # the oracle, under a unit upstream gradient
+    one = torch.ones((), device=xt.device)
+    got1 = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, None, native.lsr_args(xt, yt)).cpu().numpy()
+    want1 = oracle.lsr_backward(x, y, 255, 0.1, np.float32(1.0))
+    assert np.abs(got1 - want1).max() <= 2e-5 * np.abs(want1).max()
+
+
+def test_byte_mask_of_a_selection(native):
+    shape = (2, 19, 65, 67)
+    x, y = inputs(142, shape, 2.0)
+    xt, yt = dev(x), dev(y)
+    kept = (torch.rand(y.size, device=xt.device) < 0.6).to(torch.uint8)
+    _, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.0, True)
+    one = torch.ones((), device=xt.device)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.0, one, n_valid, native.lsr_args(xt, yt), kept=kept)
+    relabelled = yt.clone().reshape(-1)
+    relabelled[kept == 0] = 255
+    want = native.lsr_backward_scaled(xt, relabelled.reshape(yt.shape), 255, 0.0, one, n_valid)
+    assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("shape,scale", SHAPES[:3])
+def test_module_step_against_the_oracle(native, shape, scale, reduction):
+    import pytorch_loss as pl
+    x, y = inputs(143, shape, scale)
+    xt = dev(x).requires_grad_()
+    crit = pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=reduction, ignore_index=255)
+    loss = crit(xt, dev(y))
+    per = oracle.lsr_forward(x.astype(np.float64), y, 255, 0.1)
+    n_valid = int((y != 255).sum())
+    want = per.sum() / n_valid if reduction == "mean" else per.sum()
+    assert abs(loss.item() - want) <= 1e-5 * abs(want)
+    loss.backward()
+    want_g = oracle.lsr_backward(x, y, 255, 0.1, np.float32(1.0 / n_valid if reduction == "mean" else 1.0))
+    err = np.abs(xt.grad.cpu().numpy() - want_g).max()
+    assert err <= 2e-5 * np.abs(want_g).max()
+    # without a gradient asked for, nothing extra is kept
+    with torch.no_grad():
+        assert abs(crit(xt, dev(y)).item() - want) <= 1e-5 * abs(want)
+
+
+def test_views_whose_gradient_sits_elsewhere_in_a_line_take_the_recomputing_kernel(native):
+    """Logits that start one element into their storage: the fresh gradient tensor is 256-byte aligned, the logits are
+    not, so whole lines of the one are not whole lines of the other and the entry point recomputes."""
+    shape = (2, 19, 65, 67)
+    x, y = inputs(144, shape, 2.0)
+    store = torch.empty(x.size + 1, device="cuda")
+    xt = store[1:].view(shape)
+    xt.copy_(dev(x))
+    yt = dev(y)
+    _, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+    want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).reshape(-1).numpy()
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-6 * np.abs(want_lse).max()
+    one = torch.ones((), device=xt.device)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, n_valid, native.lsr_args(xt, yt))
+    want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, n_valid)
+    assert torch.equal(got, want)
+
+
+def test_sizes_outside_are_refused(native):
+    lib = native.load()
+    x = torch.zeros((2, 19, 64, 64), device="cuda")
+    y = torch.zeros((2, 64, 64), dtype=torch.int64, device="cuda")
+    lse = torch.zeros(2 * 64 * 64, device="cuda")
+    loss = torch.zeros((), device="cuda")
+    ws = torch.empty(int(lib.plh_reduce_workspace_bytes(2 * 64 * 64)), dtype=torch.uint8, device="cuda")
+    P = native._ptr
+    rc = lib.plh_lsr_forward_reduced_lse(P(x), 0, P(y), P(lse), P(loss), None, 1, P(ws), ws.numel(), 2, 19, 4096, 255, 0.1,
+                                         native._stream())
+    assert rc == -2                      # PLH_ERR_BAD_SIZE: planes of even length
