@@ -450,7 +450,8 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         bl = lambda: lib.plh_lsr_backward_scaled_lse(P(x), tag, P(labels), P(lse), None, P(up), 1.0, P(n_valid), P(grad),
                                                      n, c, m, 255, 0.1, st())
         assert fl() == 0 and bl() == 0
-        legs += [("forward_keeping_lse", fl, 4 * E + 8 * Pn + 4 * Pn), ("backward_from_lse", bl, 8 * E + 8 * Pn + 4 * Pn)]
+        eb = ELEM_BYTES[dtype]
+        legs += [("forward_keeping_lse", fl, eb * E + 8 * Pn + 4 * Pn), ("backward_from_lse", bl, 2 * eb * E + 8 * Pn + 4 * Pn)]
     if name == "lovasz":
         # the same forward with its sort passes in the decoupled look-back form (an entry point of its own)
         lb_bytes = int(lib.plh_lovasz_lookback_workspace_bytes(n, c, m))

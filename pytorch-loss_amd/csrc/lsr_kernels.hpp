@@ -172,19 +172,24 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 
 // -------------------------------------------------------------- planes ----
 // Backward from the forward's per-pixel log-sum-exp, for channel planes that start on element boundaries only (odd
-// lengths: 513 x 513, 769 x 769 crops). With lse[p] at hand the gradient is elementwise,
+// lengths: 513 x 513, 769 x 769 crops; any plane that does not start on a 128-byte line). With lse[p] at hand the
+// gradient is elementwise,
 //   g[c][p] = gk (sumw exp(x[c][p] - lse[p]) - w(label[p] == c)),
 // so nothing ties the thread that writes an element to the other channels of its pixel, and every plane can be
-// walked in its OWN cache lines: a block takes 1024 pixels of an image, and in plane c its 256 threads move the
-// 32 whole lines that begin at the tile's first pixel shifted back by the plane's offset into its line (0..31
-// elements) - 16 aligned bytes per lane, loads and stores alike; lines are shared only where two planes meet. (The
+// walked in its OWN cache lines: a block takes 1024 pixels of an image (2048 of 16-bit elements), and in plane c its
+// 256 threads move the 32 whole lines that begin at the tile's first pixel shifted back by the plane's offset into
+// its line - 16 aligned bytes per lane, loads and stores alike; lines are shared only where two planes meet. (The
 // register-resident kernel has one pixel set for all channels, and with it runs that begin and end inside lines in
 // every plane but one: 57 % of peak at (16,19,769,769) against 75 % here.) The pixels' (lse, label) pairs - the
-// tile's and the 32 before it - are staged in LDS once, transposed by pixel index mod 4, so that the four reads of
-// a lane's shifted window are conflict-free for every shift. One scalar upstream gradient (the module's 'mean' /
-// 'sum'), optionally the byte mask of an OHEM selection; fp32 logits whose gradient tensor sits at the same offset
-// into a 128-byte line.
-constexpr int kPlaneTile = 1024, kPlaneHalo = 32;
+// tile's and one line's worth before it - are staged in LDS once, transposed by pixel index mod the pixels of a
+// lane, so that the reads of a lane's shifted window are conflict-free for every shift. One scalar upstream gradient
+// (the module's 'mean' / 'sum'), optionally the byte mask of an OHEM selection; logits whose gradient tensor sits at
+// the same offset into a 128-byte line.
+// Per element type: a lane moves 16 bytes (4 fp32 or 8 16-bit elements), a line holds kLine elements, a block's tile
+// is 256 lanes' worth of pixels and the stage holds one line's worth of pixels before it.
+template <class T> struct PlaneGeom {
+    static constexpr int kPer = 16 / (int)sizeof(T), kLine = 128 / (int)sizeof(T), kTile = 256 * kPer, kHalo = kLine;
+};
 struct PlanePixel {
     float lse;
     int lab;            // the label, -1 for a pixel that takes no part, C for one without a target channel
@@ -200,14 +205,16 @@ template <class T>
 __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                       const Upstream up, T *__restrict__ grad, const LsrParams p,
                                                       int tiles) {
-    static_assert(sizeof(T) == 4, "fp32 logits");
-    __shared__ PlanePixel pairs[4][(kPlaneTile + kPlaneHalo) / 4];
+    static_assert(sizeof(T) == 4, "fp32 logits (see lsr_lse_applies)");
+    using G = PlaneGeom<T>;
+    constexpr int kPer = G::kPer, kTile = G::kTile, kHalo = G::kHalo;
+    __shared__ PlanePixel pairs[kPer][(kTile + kHalo) / kPer];          // entry i at [i % kPer][i / kPer]
     const int64_t M = p.m_size;
     const int64_t n = blockIdx.x / tiles;
     const int t = (int)(blockIdx.x - n * tiles);
     const int l = threadIdx.x;
-    const int64_t p_first = (int64_t)t * kPlaneTile - kPlaneHalo;       // image-local pixel of staged entry 0
-    for (int i = l; i < kPlaneTile + kPlaneHalo; i += 256) {
+    const int64_t p_first = (int64_t)t * kTile - kHalo;                 // image-local pixel of staged entry 0
+    for (int i = l; i < kTile + kHalo; i += 256) {
         const int64_t q = p_first + i;
         PlanePixel px{0.f, -1};
         if (q >= 0 && q < M) {
@@ -217,15 +224,15 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
             px.lse = p.lse[at];
             px.lab = dropped ? -1 : ((lb < 0 || lb >= p.C) ? p.C : (int)lb);
         }
-        pairs[i & 3][i >> 2] = px;
+        pairs[i % kPer][i / kPer] = px;
     }
     float gk = up.gout ? *up.gout * up.scale : up.scale;
     if (up.divide_by) gk = gk / (float)(*up.divide_by);
     const float scale = p.sumw * gk, n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
     __syncthreads();
-    constexpr int U = 4;                // planes in flight per thread
+    constexpr int U = 4;                            // planes in flight per thread
     for (int c0 = 0; c0 < p.C; c0 += U) {
-        plh_f4 xv[U];
+        plh_u4 xv[U];
         int64_t q[U], plane[U];
         bool full[U];
         int first[U];
@@ -233,11 +240,12 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
         for (int u = 0; u < U; ++u) {
             const int c = c0 + u < p.C ? c0 + u : p.C - 1;
             plane[u] = (n * p.C + c) * M;
-            const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) >> 2) & 31u);   // the plane's offset into its line
-            first[u] = kPlaneHalo + 4 * l - shift;                  // staged index of this lane's first pixel
-            q[u] = (int64_t)t * kPlaneTile - shift + 4 * l;
-            full[u] = q[u] >= 0 && q[u] + 3 < M;
-            xv[u] = __builtin_nontemporal_load(reinterpret_cast<const plh_f4 *>(x + plane[u] + (full[u] ? q[u] : 0)));
+            // the plane's offset into its line, in elements
+            const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) / sizeof(T)) & (unsigned)(G::kLine - 1));
+            first[u] = kHalo + kPer * l - shift;                     // staged index of this lane's first pixel
+            q[u] = (int64_t)t * kTile - shift + kPer * l;
+            full[u] = q[u] >= 0 && q[u] + (kPer - 1) < M;
+            xv[u] = __builtin_nontemporal_load(reinterpret_cast<const plh_u4 *>(x + plane[u] + (full[u] ? q[u] : 0)));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -245,26 +253,34 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
             if (c >= p.C) break;
             const int i0 = first[u];
             if (full[u]) {
-                plh_f4 g;
-                g.x = plane_grad(xv[u].x, pairs[(i0 + 0) & 3][(i0 + 0) >> 2], c, scale, n_pos, n_neg);
-                g.y = plane_grad(xv[u].y, pairs[(i0 + 1) & 3][(i0 + 1) >> 2], c, scale, n_pos, n_neg);
-                g.z = plane_grad(xv[u].z, pairs[(i0 + 2) & 3][(i0 + 2) >> 2], c, scale, n_pos, n_neg);
-                g.w = plane_grad(xv[u].w, pairs[(i0 + 3) & 3][(i0 + 3) >> 2], c, scale, n_pos, n_neg);
-                __builtin_nontemporal_store(g, reinterpret_cast<plh_f4 *>(grad + plane[u] + q[u]));
+                const unsigned in[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                unsigned out[4];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const int i = i0 + d;
+                    out[d] = f32_bits(plane_grad(bits_f32(in[d]), pairs[i % kPer][i / kPer], c, scale, n_pos, n_neg));
+                }
+                __builtin_nontemporal_store(plh_u4{out[0], out[1], out[2], out[3]},
+                                            reinterpret_cast<plh_u4 *>(grad + plane[u] + q[u]));
             } else {                    // the two ends of a plane, element by element
-                for (int k = 0; k < 4; ++k)
+                for (int k = 0; k < kPer; ++k)
                     if (q[u] + k >= 0 && q[u] + k < M)
-                        grad[plane[u] + q[u] + k] = plane_grad(x[plane[u] + q[u] + k], pairs[(i0 + k) & 3][(i0 + k) >> 2], c,
-                                                               scale, n_pos, n_neg);
+                        store_one(grad + plane[u] + q[u] + k,
+                                  plane_grad(load_one(x + plane[u] + q[u] + k), pairs[(i0 + k) % kPer][(i0 + k) / kPer], c,
+                                             scale, n_pos, n_neg));
             }
         }
     }
 }
 
-// Whether the forward leaves the log-sum-exp for these sizes (its per-image form on fp32 logits) and the backward
-// can run plane by plane: channel planes of odd length, long enough for that form, a slice that fits it.
+// Whether the forward leaves the log-sum-exp for these sizes (its per-image form) and the backward can run plane by
+// plane: channel planes that do not start on 128-byte lines, long enough for that form, a slice that fits it.
+// fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
+// (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
+// conversions.
 inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    return elem_bytes == 4 && (m_size & 1) && image_form_pays<float>((int)dimsize, m_size) && dimsize >= 1;
+    if (elem_bytes != 4 || dimsize < 1 || (m_size * (int64_t)elem_bytes) % 128 == 0) return false;
+    return image_form_pays<float>((int)dimsize, m_size);
 }
 
 // --------------------------------------------------------------- split ----
@@ -1044,13 +1060,13 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     if constexpr (sizeof(T) == 4) {
         // from the forward's log-sum-exp, plane by plane: one scalar upstream gradient, logits and gradient at the same
-        // offset into a 128-byte line (whole lines of the one are whole lines of the other) and 16-byte aligned at that
+        // offset into a 128-byte line (whole lines of the one are whole lines of the other)
+        const int64_t tiles = ceil_div(p.m_size + PlaneGeom<T>::kHalo - 1, (int64_t)PlaneGeom<T>::kTile);
         if (p.lse && !go_vec && lsr_lse_applies(sizeof(T), p.C, p.m_size) &&
             ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 127) == 0 &&
-            !misaligned(logits, 4) && p.P / p.m_size * ceil_div(p.m_size + kPlaneHalo - 1, (int64_t)kPlaneTile) < ((int64_t)1 << 31)) {
-            const int tiles = (int)ceil_div(p.m_size + kPlaneHalo - 1, (int64_t)kPlaneTile);
+            !misaligned(logits, sizeof(T)) && p.P / p.m_size * tiles < ((int64_t)1 << 31)) {
             hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)(p.P / p.m_size * tiles)), dim3(256), 0, st, logits, labels,
-                               up, grad_logits, p, tiles);
+                               up, grad_logits, p, (int)tiles);
             return;
         }
     }

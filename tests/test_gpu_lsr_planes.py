@@ -37,9 +37,8 @@ def test_the_library_says_where_it_applies(native, shape, scale):
     lib = native.load()
     n, c = shape[0], shape[1]
     m = shape[2] * shape[3]
-    assert lib.plh_lsr_saves_lse(0, n, c, m) == 1
-    assert lib.plh_lsr_saves_lse(2, n, c, m) == 0           # 16-bit logits
-    assert lib.plh_lsr_saves_lse(0, n, c, m + 1) == 0       # planes of even length
+    assert lib.plh_lsr_saves_lse(0, n, c, m) == 1 and lib.plh_lsr_saves_lse(2, n, c, m) == 0      # fp32 logits only
+    assert lib.plh_lsr_saves_lse(0, n, c, (m + 31) // 32 * 32) == 0     # planes that start on 128-byte lines
     assert lib.plh_lsr_saves_lse(0, n, 25, m) == 0          # more channels than the register-resident forward takes there
     assert lib.plh_lsr_saves_lse(0, n, c, 4095) == 0        # short planes
 
@@ -136,3 +135,16 @@ def test_sizes_outside_are_refused(native):
     rc = lib.plh_lsr_forward_reduced_lse(P(x), 0, P(y), P(lse), P(loss), None, 1, P(ws), ws.numel(), 2, 19, 4096, 255, 0.1,
                                          native._stream())
     assert rc == -2                      # PLH_ERR_BAD_SIZE: planes of even length
+
+
+def test_even_planes_off_the_lines(native):
+    """Planes of even length that do not start on 128-byte lines (1022 x 1022 style) take the same pair."""
+    shape = (2, 19, 66, 70)            # 4620 pixels: 18480 bytes, not a multiple of 128
+    x, y = inputs(146, shape, 2.0)
+    xt, yt = dev(x), dev(y)
+    _, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+    assert lse is not None
+    one = torch.ones((), device=xt.device)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, n_valid, native.lsr_args(xt, yt))
+    want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, n_valid)
+    assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
