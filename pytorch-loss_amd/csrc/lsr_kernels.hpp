@@ -24,7 +24,9 @@ struct LsrParams {
     int64_t ignore;
     float w_pos, w_neg, sumw;
     unsigned xcd_run;   // tile permutation run length (xcd_run_for)
-    // Per-pixel log-sum-exp of the logits, fp32 [P]. Forward (the per-image form on fp32 logits): written when set.
+    // Per-pixel log-sum-exp of the logits, fp32 [P]. Forward, fp32 logits in NCHW: written when set, by the per-image
+    // form of the register-resident kernel, the split kernels and the lane-per-pixel kernel (the shapes that
+    // lsr_lse_applies sends here).
     // Backward: when set, lsr_bwd_planes forms the gradient from it plane by plane (see there).
     float *lse = nullptr;
 };
@@ -204,7 +206,7 @@ __device__ __forceinline__ float plane_grad(float x, PlanePixel px, int c, float
 template <class T>
 __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                       const Upstream up, T *__restrict__ grad, const LsrParams p,
-                                                      int tiles) {
+                                                      int tiles, int planes_per_block) {
     static_assert(sizeof(T) == 4, "fp32 logits (see lsr_lse_applies)");
     using G = PlaneGeom<T>;
     constexpr int kPer = G::kPer, kTile = G::kTile, kHalo = G::kHalo;
@@ -231,14 +233,18 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
     const float scale = p.sumw * gk, n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
     __syncthreads();
     constexpr int U = 4;                            // planes in flight per thread
-    for (int c0 = 0; c0 < p.C; c0 += U) {
+    // blockIdx.y: which planes of the tile (many channels are shared out over several blocks, so that the grid fills
+    // the chip: (8,300,256,256) has 512 tiles)
+    const int c_begin = blockIdx.y * planes_per_block;
+    const int c_end = c_begin + planes_per_block < p.C ? c_begin + planes_per_block : p.C;
+    for (int c0 = c_begin; c0 < c_end; c0 += U) {
         plh_u4 xv[U];
         int64_t q[U], plane[U];
         bool full[U];
         int first[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int c = c0 + u < p.C ? c0 + u : p.C - 1;
+            const int c = c0 + u < c_end ? c0 + u : c_end - 1;
             plane[u] = (n * p.C + c) * M;
             // the plane's offset into its line, in elements
             const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) / sizeof(T)) & (unsigned)(G::kLine - 1));
@@ -250,7 +256,7 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int c = c0 + u;
-            if (c >= p.C) break;
+            if (c >= c_end) break;
             const int i0 = first[u];
             if (full[u]) {
                 const unsigned in[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
@@ -273,14 +279,21 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
     }
 }
 
-// Whether the forward leaves the log-sum-exp for these sizes (its per-image form) and the backward can run plane by
-// plane: channel planes that do not start on 128-byte lines, long enough for that form, a slice that fits it.
+// Whether the forward leaves the log-sum-exp for these sizes and the backward runs plane by plane: fp32 logits on
+// planes of 4096 pixels or more that do not start on 128-byte lines - up to 24 channels (the register-resident
+// forward's per-image form) or 33 and more (channels shared among wavefronts in tiles per image: fwd+bwd at
+// (8,150,513,513) 0.780 -> 0.680 ms) - and, whatever the planes' alignment, more than 512 channels, where the
+// recomputing kernels have a lane walk its pixel's channels ((4,600,256,256) 0.761 -> 0.527 ms). On aligned planes
+// with up to 512 channels the recomputing backward is as fast or faster (40 channels: 0.179 against 0.196 ms for the
+// pair, 150: 0.629 / 0.634, 300: 0.354 / 0.350).
 // fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
 // (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
 // conversions.
 inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    if (elem_bytes != 4 || dimsize < 1 || (m_size * (int64_t)elem_bytes) % 128 == 0) return false;
-    return image_form_pays<float>((int)dimsize, m_size);
+    if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
+    const bool off_lines = (m_size * (int64_t)elem_bytes) % 128 != 0;
+    if (dimsize <= kMaxRegsChannels) return off_lines && image_form_pays<float>((int)dimsize, m_size);
+    return off_lines || dimsize > kMaxDeepChannels;
 }
 
 // --------------------------------------------------------------- split ----
@@ -357,6 +370,9 @@ __global__ __launch_bounds__(kSplitBlock) void lsr_fwd_split(const T *__restrict
     const bool valid = here && !ign;
     const float out = valid ? acc : 0.f;
     if (here && loss) loss[at.pix + wave] = out;
+    if constexpr (sizeof(T) == 4) {
+        if (here && p.lse) __builtin_nontemporal_store(M + lse, p.lse + at.pix + wave);      // LsrParams::lse
+    }
     if (Reduce) split_block_partials<V>(out, valid, wave, lane, part);
 }
 
@@ -482,6 +498,9 @@ __global__ __launch_bounds__(256) void lsr_fwd_group(const T *__restrict__ x,
         const bool valid = live && (lb != p.ignore);
         if (live && sub == 0) {
             if (loss) loss[pix] = valid ? acc : 0.f;
+            if constexpr (sizeof(T) == 4) {
+                if (p.lse) p.lse[pix] = mx + lse;        // LsrParams::lse
+            }
             mine += valid ? acc : 0.f;
             cnt += valid ? 1.f : 0.f;
         }
@@ -1065,8 +1084,10 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         if (p.lse && !go_vec && lsr_lse_applies(sizeof(T), p.C, p.m_size) &&
             ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 127) == 0 &&
             !misaligned(logits, sizeof(T)) && p.P / p.m_size * tiles < ((int64_t)1 << 31)) {
-            hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)(p.P / p.m_size * tiles)), dim3(256), 0, st, logits, labels,
-                               up, grad_logits, p, (int)tiles);
+            // planes per block: all of them up to 32 channels, else 16 (a multiple of the four in flight)
+            const int per = p.C <= kMaxRegsChannels ? p.C : 16;
+            hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)(p.P / p.m_size * tiles), (unsigned)ceil_div(p.C, per)),
+                               dim3(256), 0, st, logits, labels, up, grad_logits, p, (int)tiles, per);
             return;
         }
     }

@@ -39,7 +39,10 @@ def test_the_library_says_where_it_applies(native, shape, scale):
     m = shape[2] * shape[3]
     assert lib.plh_lsr_saves_lse(0, n, c, m) == 1 and lib.plh_lsr_saves_lse(2, n, c, m) == 0      # fp32 logits only
     assert lib.plh_lsr_saves_lse(0, n, c, (m + 31) // 32 * 32) == 0     # planes that start on 128-byte lines
-    assert lib.plh_lsr_saves_lse(0, n, 25, m) == 0          # more channels than the register-resident forward takes there
+    assert lib.plh_lsr_saves_lse(0, n, 25, m) == 0 and lib.plh_lsr_saves_lse(0, n, 32, m) == 0   # the forward is not the per-image form there
+    assert lib.plh_lsr_saves_lse(0, n, 33, m) == 1 and lib.plh_lsr_saves_lse(0, n, 512, 4096) == 0   # 33 and more: planes off the lines
+    assert lib.plh_lsr_saves_lse(0, n, 513, 4096) == 1                                               # beyond 512: any plane
+    assert lib.plh_lsr_saves_lse(2, n, 150, m) == 0
     assert lib.plh_lsr_saves_lse(0, n, c, 4095) == 0        # short planes
 
 
@@ -148,3 +151,47 @@ def test_even_planes_off_the_lines(native):
     got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, n_valid, native.lsr_args(xt, yt))
     want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, n_valid)
     assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+
+
+# 33 channels and more, every forward shape that can take them: channels shared among wavefronts (aligned planes; planes
+# of odd length in tiles per image), the deep form (257..512), a lane per pixel (beyond 512, and planes whose tensors sit
+# on element boundaries only)
+WIDE = [((2, 40, 65, 65), 2.0), ((2, 150, 66, 70), 2.0), ((1, 60, 65, 67), 1.0), ((1, 300, 65, 65), 2.0),
+        ((1, 384, 65, 66), 3.0), ((1, 600, 64, 64), 1.0), ((2, 171, 65, 65), 2.0), ((1, 520, 65, 67), 1.0)]
+
+
+@pytest.mark.parametrize("shape,scale", WIDE)
+def test_many_channels(native, shape, scale):
+    x, y = inputs(147, shape, scale)
+    y.reshape(-1)[::101] = shape[1] + 1                      # labels without a target channel, not ignored
+    xt, yt = dev(x), dev(y)
+    loss, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+    assert lse is not None
+    want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).reshape(-1).numpy()
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-6 * np.abs(want_lse).max()
+    loss2, n_valid2 = native.lsr_forward_reduced(xt, yt, 255, 0.1, True)
+    assert loss.cpu().numpy().tobytes() == loss2.cpu().numpy().tobytes() and int(n_valid.item()) == int(n_valid2.item())
+    one = torch.ones((), device=xt.device)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, None, native.lsr_args(xt, yt))
+    want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, None)
+    assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+    want64 = oracle.lsr_backward(x, y, 255, 0.1, np.float32(1.0))
+    assert np.abs(got.cpu().numpy() - want64).max() <= 2e-5 * np.abs(want64).max()
+
+
+def test_many_channels_on_a_view_one_element_in(native):
+    """The forward then runs a lane per pixel, the backward recomputes (logits and gradient sit differently in
+    their lines): the pair still gives the module's results."""
+    shape = (1, 150, 65, 67)
+    x, y = inputs(148, shape, 2.0)
+    store = torch.empty(x.size + 1, device="cuda")
+    xt = store[1:].view(shape)
+    xt.copy_(dev(x))
+    yt = dev(y)
+    _, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+    want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).reshape(-1).numpy()
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-6 * np.abs(want_lse).max()
+    one = torch.ones((), device=xt.device)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, n_valid, native.lsr_args(xt, yt))
+    want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, n_valid)
+    assert torch.equal(got, want)
