@@ -282,10 +282,11 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
 // Whether the forward leaves the log-sum-exp for these sizes and the backward runs plane by plane: fp32 logits on
 // planes of 4096 pixels or more that do not start on 128-byte lines - up to 24 channels (the register-resident
 // forward's per-image form) or 33 and more (channels shared among wavefronts in tiles per image: fwd+bwd at
-// (8,150,513,513) 0.780 -> 0.680 ms) - and, whatever the planes' alignment, more than 512 channels, where the
-// recomputing kernels have a lane walk its pixel's channels ((4,600,256,256) 0.761 -> 0.527 ms). On aligned planes
-// with up to 512 channels the recomputing backward is as fast or faster (40 channels: 0.179 against 0.196 ms for the
-// pair, 150: 0.629 / 0.634, 300: 0.354 / 0.350).
+// (8,150,513,513) 0.780 -> 0.670 ms) - and, whatever the planes' alignment, more than 256 channels, where the
+// recomputing kernels keep a pixel's slice in two halves per wavefront ((8,300,256,256) 0.359 -> 0.334 ms,
+// (4,512,256,256) 0.343 -> 0.301 ms) or have a lane walk its pixel's channels ((4,600,256,256) 0.761 -> 0.523 ms).
+// On aligned planes with up to 256 channels the recomputing backward is as fast or faster (40 channels: 0.179 against
+// 0.196 ms for the pair, 150: 0.629 / 0.634).
 // fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
 // (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
 // conversions.
@@ -293,7 +294,7 @@ inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) 
     if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
     const bool off_lines = (m_size * (int64_t)elem_bytes) % 128 != 0;
     if (dimsize <= kMaxRegsChannels) return off_lines && image_form_pays<float>((int)dimsize, m_size);
-    return off_lines || dimsize > kMaxDeepChannels;
+    return off_lines || dimsize > kMaxSplitChannels;
 }
 
 // --------------------------------------------------------------- split ----
@@ -1084,9 +1085,17 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
         if (p.lse && !go_vec && lsr_lse_applies(sizeof(T), p.C, p.m_size) &&
             ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 127) == 0 &&
             !misaligned(logits, sizeof(T)) && p.P / p.m_size * tiles < ((int64_t)1 << 31)) {
-            // planes per block: all of them up to 32 channels, else 16 (a multiple of the four in flight)
-            const int per = p.C <= kMaxRegsChannels ? p.C : 16;
-            hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)(p.P / p.m_size * tiles), (unsigned)ceil_div(p.C, per)),
+            // planes per block (a multiple of the four in flight): all of them up to 32 channels; beyond, 16 on planes of
+            // 1 MiB and more and 4 on smaller ones, where short blocks measured better (backward at (8,300,256,256)
+            // 0.229 -> 0.213 ms, (8,300,384,384) 0.532 -> 0.491, (8,150,385,385) 0.251 -> 0.241; on 1 MiB planes
+            // (8,150,512,512) 0.439 -> 0.488) - 8 when the tiles alone outnumber the blocks the chip holds at once
+            // ((64,40,256,256) 4: 0.261, 8: 0.239 ms)
+            const int64_t tiles_all = p.P / p.m_size * tiles;
+            const int per = p.C <= kMaxRegsChannels                      ? p.C
+                            : p.m_size * (int64_t)sizeof(T) >= (1 << 20) ? 16
+                            : tiles_all <= 2048                          ? 4
+                                                                         : 8;
+            hipLaunchKernelGGL(lsr_bwd_planes<T>, dim3((unsigned)tiles_all, (unsigned)ceil_div(p.C, per)),
                                dim3(256), 0, st, logits, labels, up, grad_logits, p, (int)tiles, per);
             return;
         }

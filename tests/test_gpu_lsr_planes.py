@@ -40,8 +40,8 @@ def test_the_library_says_where_it_applies(native, shape, scale):
     assert lib.plh_lsr_saves_lse(0, n, c, m) == 1 and lib.plh_lsr_saves_lse(2, n, c, m) == 0      # fp32 logits only
     assert lib.plh_lsr_saves_lse(0, n, c, (m + 31) // 32 * 32) == 0     # planes that start on 128-byte lines
     assert lib.plh_lsr_saves_lse(0, n, 25, m) == 0 and lib.plh_lsr_saves_lse(0, n, 32, m) == 0   # the forward is not the per-image form there
-    assert lib.plh_lsr_saves_lse(0, n, 33, m) == 1 and lib.plh_lsr_saves_lse(0, n, 512, 4096) == 0   # 33 and more: planes off the lines
-    assert lib.plh_lsr_saves_lse(0, n, 513, 4096) == 1                                               # beyond 512: any plane
+    assert lib.plh_lsr_saves_lse(0, n, 33, m) == 1 and lib.plh_lsr_saves_lse(0, n, 256, 4096) == 0   # 33 and more: planes off the lines
+    assert lib.plh_lsr_saves_lse(0, n, 257, 4096) == 1                                               # beyond 256: any plane
     assert lib.plh_lsr_saves_lse(2, n, 150, m) == 0
     assert lib.plh_lsr_saves_lse(0, n, c, 4095) == 0        # short planes
 
@@ -157,7 +157,8 @@ def test_even_planes_off_the_lines(native):
 # of odd length in tiles per image), the deep form (257..512), a lane per pixel (beyond 512, and planes whose tensors sit
 # on element boundaries only)
 WIDE = [((2, 40, 65, 65), 2.0), ((2, 150, 66, 70), 2.0), ((1, 60, 65, 67), 1.0), ((1, 300, 65, 65), 2.0),
-        ((1, 384, 65, 66), 3.0), ((1, 600, 64, 64), 1.0), ((2, 171, 65, 65), 2.0), ((1, 520, 65, 67), 1.0)]
+        ((1, 384, 65, 66), 3.0), ((1, 600, 64, 64), 1.0), ((2, 171, 65, 65), 2.0), ((1, 520, 65, 67), 1.0),
+        ((2, 300, 64, 64), 2.0), ((420, 33, 65, 65), 2.0), ((1, 36, 513, 513), 2.0)]     # the last two: 8 and 16 planes per block
 
 
 @pytest.mark.parametrize("shape,scale", WIDE)
@@ -175,8 +176,9 @@ def test_many_channels(native, shape, scale):
     got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, None, native.lsr_args(xt, yt))
     want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, None)
     assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
-    want64 = oracle.lsr_backward(x, y, 255, 0.1, np.float32(1.0))
-    assert np.abs(got.cpu().numpy() - want64).max() <= 2e-5 * np.abs(want64).max()
+    if x.size <= 20_000_000:
+        want64 = oracle.lsr_backward(x, y, 255, 0.1, np.float32(1.0))
+        assert np.abs(got.cpu().numpy() - want64).max() <= 2e-5 * np.abs(want64).max()
 
 
 def test_many_channels_on_a_view_one_element_in(native):
