@@ -671,6 +671,25 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
                                       "what": "eager steps under torch.autograd.set_multithreading_enabled(False)"}
         except Exception as e:
             dist["calling_thread"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    if name in ("lmargin", "focal"):
+        # the same module with fb=True (what the reference's repository-root copies of these two modules do: gradient
+        # computed in the forward pass and kept): one pass over the inputs per step. Its bytes: large margin reads the
+        # logits and writes the gradient (2bE) and reads the labels twice (the count of valid pixels, then the pass
+        # itself: 16P); focal reads logits and labels and writes the gradient (3bE).
+        try:
+            import pytorch_loss as pl
+            fb = (pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255, fb=True) if name == "lmargin"
+                  else pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean", fb=True))
+            fb_ms, fb_loss = time_steps(fb, logits, labels, steps, warmup)
+            eb, E = ELEM_BYTES[dtype], numel(shape)
+            fb_bytes = 3 * eb * E if name == "focal" else 2 * eb * E + 16 * (E // shape[1])
+            dist["one_pass_fb"] = {"ms": round(fb_ms, 4), "bytes": fb_bytes,
+                                   "frac": round(fb_bytes / (fb_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                   "graph_ms": graph_step(fb, logits, labels).get("ms"),
+                                   "loss_rel_diff": float("%.2g" % (abs(fb_loss - loss) / max(abs(loss), 1e-30)))}
+            del fb
+        except Exception as e:
+            dist["one_pass_fb"] = {"error": "%s: %s" % (type(e).__name__, e)}
     del crit
     logits.grad = None
     return dict(ms_per_step=ms, gbps=gbps, loss=loss, roofline=roof, bytes=fwd + bwd, step_ms=dist, function_level=func)
@@ -700,6 +719,9 @@ def targets_block(headline, main_res, others, headline_cpu, with_cpu):
              "fwd_ms": (kern.get("forward") or {}).get("ms"), "bwd_ms": (kern.get("backward") or {}).get("ms")}
         if "calling_thread" in step_ms:      # short steps: the eager step with the backward on the calling thread
             e["calling_thread_ms"] = step_ms["calling_thread"].get("ms")
+        if "one_pass_fb" in step_ms:         # the module with fb=True: eager step, replayed step, fraction of peak on its own bytes
+            fb = step_ms["one_pass_fb"]
+            e["fb"] = {k: fb.get(k) for k in (("error",) if "error" in fb else ("ms", "graph_ms", "frac"))}
         if with_cpu:
             try:
                 c = headline_cpu if (t == headline and headline_cpu and "error" not in headline_cpu) else \

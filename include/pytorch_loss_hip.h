@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define PLH_ABI_VERSION 3
+#define PLH_ABI_VERSION 4
 
 #define PLH_OK 0
 #define PLH_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
@@ -174,6 +174,14 @@ int plh_focal_forward_backward(const void *logits, int32_t dtype, const void *la
                                float *losses, void *grad_logits,
                                int64_t numel, float gamma, float alpha, void *stream);
 
+/* The module step of the repository root's FocalLossV3 (focal_loss.py:196-200: FocalSigmoidLossFuncV3FB.apply, then
+ * loss.mean() / loss.sum()) in ONE pass: the kernel leaves the partial sums of the losses and writes grad_logits
+ * already divided by numel (mean) - the gradient under an upstream gradient of 1; plh_scale_unless_one is its backward.
+ * loss_out: the sum or the mean. Workspace as for plh_focal_forward_reduced. */
+int plh_focal_forward_backward_reduced(const void *logits, int32_t dtype, const void *labels, float *loss_out,
+                                       void *grad_logits, int32_t mean, void *workspace, int64_t workspace_bytes,
+                                       int64_t numel, float gamma, float alpha, void *stream);
+
 /* ---- large-margin softmax -------------------------------------------------------
  * Replaces large_margin_cpp.l_margin_forward / l_margin_backward /
  * l_margin_forward_backward (csrc/large_margin_kernel.cu:796-831; kernels :140-599).
@@ -208,6 +216,23 @@ int plh_lmargin_forward_backward(const void *logits, int32_t dtype, const int64_
                                  float *losses, void *grad_logits, int64_t *valid_cnt,
                                  int64_t n_size, int64_t dimsize, int64_t m_size,
                                  int64_t ignore_index, float lam, void *stream);
+
+/* The module step with fb=True and reduction 'mean' / 'sum' in ONE pass over the logits (replaces, in
+ * large_margin_softmax.py:198-229 of the repository root, l_margin_forward_backward followed by losses.sum() / valid_cnt,
+ * whose backward then multiplies the kept gradient by a per-pixel upstream tensor). The labels are counted first
+ * (n_valid_out: labels other than ignore_index; required), then one kernel reads the logits, leaves the partial sums of
+ * the losses and writes grad_logits already divided by that count (mean) - the gradient under an upstream gradient of 1.
+ * loss_out: the sum or the mean (0/0 = NaN when nothing is valid). Workspace as for plh_lmargin_forward_reduced. */
+int plh_lmargin_forward_backward_reduced(const void *logits, int32_t dtype, const int64_t *labels,
+                                         float *loss_out, int64_t *n_valid_out, void *grad_logits, int32_t mean,
+                                         void *workspace, int64_t workspace_bytes,
+                                         int64_t n_size, int64_t dimsize, int64_t m_size,
+                                         int64_t ignore_index, float lam, void *stream);
+
+/* data[i] *= *scalar in place for numel elements of `dtype`, except that nothing is read or written when *scalar is exactly
+ * 1: the backward of a kept gradient (replaces logits_grads.mul_(grad_output), large_margin_softmax.py:189 of the
+ * repository root, for a scalar upstream gradient, which loss.backward() makes 1). `data` on a 16-byte boundary. */
+int plh_scale_unless_one(void *data, int32_t dtype, int64_t numel, const float *scalar, void *stream);
 
 /* ---- Lovasz-softmax ---------------------------------------------------------------
  * Replaces lovasz_softmax_cpp.lovasz_softmax_forward / lovasz_softmax_backward

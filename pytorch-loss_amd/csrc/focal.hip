@@ -216,3 +216,22 @@ extern "C" int plh_focal_forward_backward(const void *logits, int32_t dtype, con
     return launch<true, true, false>(logits, labels, dtype, up, losses, grad_logits, nullptr, nullptr, numel, gamma,
                                      alpha, stream);
 }
+
+extern "C" int plh_focal_forward_backward_reduced(const void *logits, int32_t dtype, const void *labels, float *loss_out,
+                                                  void *grad_logits, int32_t mean, void *workspace,
+                                                  int64_t workspace_bytes, int64_t numel, float gamma, float alpha,
+                                                  void *stream) {
+    if (numel < 0 || numel > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    Partials part;
+    int rc = carve_partials(workspace, workspace_bytes, numel, loss_out, nullptr, part);
+    if (rc != PLH_OK) return rc;
+    // the mean's divisor is the element count, known here: the gradient is written already divided by it
+    const Upstream up{nullptr, 0, nullptr, (mean && numel > 0) ? 1.f / (float)numel : 1.f};
+    unsigned slots = 0;
+    rc = launch<true, true, true>(logits, labels, dtype, up, nullptr, grad_logits, part.sum, &slots, numel, gamma, alpha,
+                                  stream);
+    if (rc != PLH_OK) return rc;
+    part.cnt = nullptr;
+    finish_partials(part, slots, loss_out, nullptr, mean ? kFinishMeanOverFixed : kFinishSum, numel, (hipStream_t)stream);
+    return check_launch();
+}

@@ -55,9 +55,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                                                      float *__restrict__ loss, T *__restrict__ grad,
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
-    // only the plain forward leaves partial sums, so the other combinations carry no code for them
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
+    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
+    // backward carries no code for either
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
     const bool WantCount = kMayCount && valid_cnt != nullptr;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
@@ -420,9 +421,10 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
                                                 float *__restrict__ loss, T *__restrict__ grad,
                                                 unsigned long long *__restrict__ valid_cnt, Partials part,
                                                 const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
-    // only the plain forward leaves partial sums, so the other combinations carry no code for them
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
+    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
+    // backward carries no code for either
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
     const bool WantCount = kMayCount && valid_cnt != nullptr;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     constexpr int kPix = 256 / G;
@@ -520,9 +522,10 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
                                                const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
-    // only the plain forward leaves partial sums, so the other combinations carry no code for them
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
+    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
+    // backward carries no code for either
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
     const bool WantCount = kMayCount && valid_cnt != nullptr;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
@@ -739,9 +742,10 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                                                     const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
                                                     const LmParams p, int vec) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels and
-    // only the plain forward leaves partial sums, so the other combinations carry no code for them
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss && !WantGrad;
+    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
+    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
+    // backward carries no code for either
+    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
     const bool WantCount = kMayCount && valid_cnt != nullptr;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[kRowBlock / 64];
@@ -992,7 +996,7 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
 // forward (plain or with partial sums), backward, and the fused pair (with the count of valid pixels); each is
 // explicitly instantiated per element type in a translation unit of its own (lmargin_f32_fwd.hip, lmargin_f32_bwd.hip,
 // lmargin_f32_both.hip, ...) so that the nine parts compile in parallel.
-enum LmVariant { kLmForward = 0, kLmForwardReduced = 1, kLmBackward = 2, kLmForwardBackwardCount = 3 };
+enum LmVariant { kLmForward = 0, kLmForwardReduced = 1, kLmBackward = 2, kLmForwardBackwardCount = 3, kLmForwardBackwardReduced = 4 };
 
 #define PLH_LM_SIGNATURE(T, L, G)                                                                                    \
     unsigned launch_typed<T, L, G>(const T *, const int64_t *, const Upstream &, float *, T *, unsigned long long *, \

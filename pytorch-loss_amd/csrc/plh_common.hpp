@@ -582,6 +582,10 @@ __device__ inline void finish_block(const float *__restrict__ sums, const int *_
 void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int64_t *count_out, FinishMode mode,
                      int64_t fixed_count, hipStream_t stream);
 
+// Per block the number of labels other than `ignore`, as partials for finish_partials (the sums are zeros); returns the
+// number of blocks. For a pass that needs the mean's divisor before it runs. Defined in reduce.hip.
+unsigned count_valid_partials(const int64_t *labels, int64_t P, int64_t ignore, const Partials &part, hipStream_t stream);
+
 // What the score pass of an OHEM loss forward (ohem.hip: the cross-entropy score kernel; the large-margin forward kernel
 // that also writes scores) leaves besides scores and losses, for the case that the threshold
 // rule decides the selection (at least n_min pixels score within the threshold, so "beyond the n_min lowest" holds

@@ -18,7 +18,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpytorch_loss_hip.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 
@@ -41,11 +41,14 @@ _SIGNATURES = {
     "plh_focal_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i32, _p, _i64, _i64, _f32, _f32, _p]),
     "plh_focal_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _i64, _f32, _f32, _p]),
     "plh_focal_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_focal_forward_backward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i32, _p, _i64, _i64, _f32, _f32, _p]),
     "plh_lmargin_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_forward_backward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_scale_unless_one": (ctypes.c_int, [_p, _i32, _i64, _p, _p]),
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_lsr_saves_lse": (ctypes.c_int, [_i32, _i64, _i64, _i64]),
@@ -399,6 +402,29 @@ def lmargin_forward_backward(logits, labels, lam, ignore_index):
     return _back_to(losses, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), cnt
 
 
+def lmargin_forward_backward_reduced(logits, labels, lam, ignore_index, mean):
+    """One pass over the logits: -> (loss: the sum or the mean, gradient under an upstream gradient of 1)."""
+    a = lmargin_args(logits, labels)
+    dev = a.x.device
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    n_valid = torch.empty((), dtype=torch.int64, device=dev)
+    grad = torch.empty_like(a.x)
+    ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
+    _call(a.x, "plh_lmargin_forward_backward_reduced", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(loss), _ptr(n_valid), _ptr(grad),
+          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(lam))
+    return _back_to(loss, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), (a.tag if a.x.dtype == a.dtype else None)
+
+
+def scale_unless_one(data, tag, grad_scalar):
+    """data *= grad_scalar in place (a 0-dim tensor), without touching data when it is exactly 1; tag: the library's
+    dtype tag of `data`, or None for a tensor the library does not hold (then torch multiplies)."""
+    if tag is None or not data.is_contiguous() or data.data_ptr() % 16 != 0:
+        return data.mul_(grad_scalar)
+    if data.numel():
+        _call(data, "plh_scale_unless_one", _ptr(data), tag, data.numel(), _ptr(_scalar_f32(grad_scalar)))
+    return data
+
+
 # ---------------------------------------------------------------- focal ----
 
 class FocalArgs:
@@ -446,6 +472,17 @@ def focal_forward_backward(logits, labels, gamma, alpha):
         _call(a.x, "plh_focal_forward_backward", _ptr(a.x), a.tag, _ptr(a.y), _ptr(losses), _ptr(grad), a.x.numel(),
               float(gamma), float(alpha))
     return _back_to(losses, _loss_dtype(a.dtype)), _back_to(grad, a.dtype)
+
+
+def focal_forward_backward_reduced(logits, labels, gamma, alpha, mean):
+    """One pass: -> (loss: the sum or the mean, gradient under an upstream gradient of 1, dtype tag of the gradient or None)."""
+    a = focal_args(logits, labels, "focalloss_forward_backward")
+    loss = torch.empty((), dtype=torch.float32, device=a.x.device)
+    grad = torch.empty_like(a.x)
+    ws, ws_bytes = _reduce_workspace(a.x.numel(), a.x.device)
+    _call(a.x, "plh_focal_forward_backward_reduced", _ptr(a.x), a.tag, _ptr(a.y), _ptr(loss), _ptr(grad), 1 if mean else 0,
+          _ptr(ws), ws_bytes, a.x.numel(), float(gamma), float(alpha))
+    return _back_to(loss, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), (a.tag if a.x.dtype == a.dtype else None)
 
 
 def focal_forward_reduced(logits, labels, gamma, alpha, mean, args=None):

@@ -41,6 +41,7 @@ class FocalSigmoidLossFuncV3FB(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         grads = ctx.variables
+        ctx.variables = None        # handed over (see _FocalFusedReducedFunction.backward)
         grads.mul_(grad_output)
         return grads, None, None, None
 
@@ -63,21 +64,54 @@ class _FocalReducedFunction(torch.autograd.Function):
         return grads, None, None, None, None
 
 
-class FocalLossV3(nn.Module):
-    """Usage as nn.BCEWithLogitsLoss. reduction 'mean' averages over every element."""
+class _FocalFusedReducedFunction(torch.autograd.Function):
+    """fb=True with 'sum' / 'mean': loss and gradient from ONE pass over logits and labels (12 bytes per fp32 element
+    instead of the 20 of a forward and a backward). The kept gradient is the one under an upstream gradient of 1 (what
+    loss.backward() sends), already divided by the element count for 'mean'; backward multiplies it in place by the
+    upstream scalar, which costs a pass over it only when that scalar is not 1 - the reference's FB Function
+    multiplies every time (focal_loss.py:170 of the repository root)."""
 
-    def __init__(self, alpha=0.25, gamma=2, reduction="mean"):
+    @staticmethod
+    def forward(ctx, logits, labels, alpha, gamma, mean):
+        loss, grads, tag = _native.focal_forward_backward_reduced(logits, labels, gamma, alpha, mean)
+        ctx.variables = (grads, tag)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grads, tag = ctx.variables
+        # the kept gradient is handed over, not shared: while this context still referred to it autograd would copy it
+        # into logits.grad (a pass over it) instead of taking it
+        ctx.variables = None
+        return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
+
+
+class FocalLossV3(nn.Module):
+    """Usage as nn.BCEWithLogitsLoss. reduction 'mean' averages over every element.
+
+    fb=True computes the gradient in the forward pass, as the FocalLossV3 of the reference's repository root does
+    (focal_loss.py:196), and keeps it for backward: one pass over the inputs per step instead of two. The default keeps
+    nothing but the inputs (the packaged copy, pytorch_loss/focal_loss.py:173)."""
+
+    def __init__(self, alpha=0.25, gamma=2, reduction="mean", fb=False):
         super().__init__()
         self.alpha = alpha
         self.gamma = gamma
         self.reduction = reduction
+        self.fb = fb
 
     def forward(self, logits, label):
-        if self.reduction in ("mean", "sum") and logits.numel() > 0:
+        # fp16 logits keep the two passes: a gradient kept in fp16 at 1/numel of its size is subnormal before a loss
+        # scale could lift it, where the backward kernel multiplies in fp32 and rounds once
+        fused = self.fb and logits.dtype != torch.float16
+        if fused and self.reduction in ("mean", "sum") and logits.numel() > 0:
+            return _FocalFusedReducedFunction.apply(logits, label, self.alpha, self.gamma, self.reduction == "mean")
+        if not fused and self.reduction in ("mean", "sum") and logits.numel() > 0:
             return _FocalReducedFunction.apply(logits, label, self.alpha, self.gamma, self.reduction == "mean")
-        # the two-kernel Function moves the same bytes as the fused one once the upstream
-        # multiply is folded into the backward kernel, and keeps no gradient-sized tensor alive
-        loss = FocalSigmoidLossFuncV3.apply(logits, label, self.alpha, self.gamma)
+        # per-element losses: the two-kernel Function moves the same bytes as the fused one once the upstream multiply
+        # is folded into the backward kernel, and keeps no gradient-sized tensor alive
+        func = FocalSigmoidLossFuncV3FB if self.fb else FocalSigmoidLossFuncV3
+        loss = func.apply(logits, label, self.alpha, self.gamma)
         if self.reduction == "mean":
             return loss.mean()
         if self.reduction == "sum":

@@ -40,6 +40,7 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output, grad_cnt):
         grads = ctx.variables
+        ctx.variables = None        # handed over (see _LargeMarginFusedReducedFunction.backward)
         grads.mul_(grad_output.unsqueeze(1))
         return grads, None, None, None
 
@@ -61,12 +62,36 @@ class _LargeMarginReducedFunction(torch.autograd.Function):
         return grads, None, None, None, None
 
 
+class _LargeMarginFusedReducedFunction(torch.autograd.Function):
+    """fb=True with 'sum' / 'mean': loss and gradient from ONE pass over the logits. The kept gradient is the one under
+    an upstream gradient of 1 (what loss.backward() sends), already divided by the number of valid pixels for 'mean';
+    backward multiplies it in place by the upstream scalar, which costs a pass over it only when that scalar is not 1
+    (a weighted or scaled loss) - the reference's FB Function multiplies by a per-pixel tensor every time
+    (large_margin_softmax.py:189 of the repository root)."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, lam, ignore_index, mean):
+        loss, grads, tag = _native.lmargin_forward_backward_reduced(logits, labels, lam, ignore_index, mean)
+        ctx.variables = (grads, tag)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grads, tag = ctx.variables
+        # the kept gradient is handed over, not shared: while this context still referred to it autograd would copy it
+        # into logits.grad (a pass over it) instead of taking it
+        ctx.variables = None
+        return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
+
+
 class LargeMarginSoftmaxV3(nn.Module):
     """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
 
-    fb=True selects the fused forward+backward Function (one kernel, keeps a gradient-sized
-    tensor between forward and backward); the default recomputes in backward, which moves
-    fewer bytes in total.
+    fb=True selects the fused forward+backward (one kernel, keeps a gradient-sized tensor between
+    forward and backward): with 'mean' / 'sum' the reduction and the division are part of that one
+    pass, so a step reads the logits once and writes the gradient once; with 'none' it is the
+    reference's FB Function, whose backward multiplies the kept gradient by the per-pixel upstream
+    tensor. The default recomputes in backward and keeps nothing but the inputs.
     """
 
     def __init__(self, lam=0.3, reduction="mean", ignore_index=255, fb=False):
@@ -77,9 +102,12 @@ class LargeMarginSoftmaxV3(nn.Module):
         self.fb = fb
 
     def forward(self, logits, labels):
-        if not self.fb and self.reduction in ("sum", "mean") and logits.numel() > 0:
-            return _LargeMarginReducedFunction.apply(logits, labels, self.lam, self.ignore_index,
-                                                     self.reduction == "mean")
+        # fp16 logits keep the two passes: a gradient kept in fp16 at 1/n_valid of its size is subnormal before a loss
+        # scale could lift it, where the backward kernel multiplies in fp32 and rounds once
+        fused = self.fb and logits.dtype != torch.float16
+        if self.reduction in ("sum", "mean") and logits.numel() > 0:
+            func = _LargeMarginFusedReducedFunction if fused else _LargeMarginReducedFunction
+            return func.apply(logits, labels, self.lam, self.ignore_index, self.reduction == "mean")
         valid_cnt = None
         if self.fb:
             losses, valid_cnt = LargeMarginSoftmaxFuncV3FB.apply(logits, labels, self.lam, self.ignore_index)

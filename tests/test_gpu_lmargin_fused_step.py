@@ -1,0 +1,149 @@
+"""LargeMarginSoftmaxV3(fb=True) with 'mean' / 'sum': loss and gradient from one pass over the logits
+(plh_lmargin_forward_backward_reduced), the backward a multiplication that is skipped for an upstream gradient of 1
+(plh_scale_unless_one) - against the oracle and against the module that recomputes in backward."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+# one shape per launch form of the fused kernel: register-resident (two pixels per lane, one pixel per lane on odd
+# planes, the per-image form on long odd planes), rows (a wavefront per 64 rows, a wavefront per row, a block per row),
+# and 33 channels and more in NCHW, where the entry point runs the forward and the backward one after the other (a lane
+# per pixel on the short planes of 63 pixels)
+SHAPES = [(2, 19, 32, 40), (3, 7, 13, 11), (1, 12, 65, 67), (300, 10), (70, 200), (9, 3000), (2, 40, 16, 24), (1, 2, 8, 8),
+          (2, 150, 16, 24), (1, 300, 9, 7)]
+DTYPES = [(torch.float32, 2e-6), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)]
+
+
+@pytest.fixture(scope="module")
+def mod():
+    import pytorch_loss
+    from pytorch_loss import _native
+    _native.load()
+    return pytorch_loss
+
+
+def inputs(seed, shape, dtype, ignore_frac=0.1):
+    x = synth.normal(seed, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(seed, shape[:1] + shape[2:], shape[1], 255, ignore_frac)
+    xt = torch.from_numpy(x).cuda().to(dtype)
+    return xt.float().cpu().numpy(), y, xt, torch.from_numpy(y).cuda()
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("dtype,tol", DTYPES, ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=str)
+def test_one_pass_step_matches_the_oracle_and_the_recomputing_module(mod, shape, dtype, tol, reduction):
+    x, y, xt, yt = inputs(301, shape, dtype)
+    n_valid = int((y != 255).sum())
+    losses = oracle.lmargin_forward(x.astype(np.float64), y, 0.3, 255)
+    want_loss = losses.sum() / (n_valid if reduction == "mean" else 1)
+    up = np.full(y.shape, 1.0 / n_valid if reduction == "mean" else 1.0)
+    want_grad = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, up)
+
+    a = xt.clone().requires_grad_(True)
+    loss = mod.LargeMarginSoftmaxV3(lam=0.3, reduction=reduction, ignore_index=255, fb=True)(a, yt)
+    loss.backward()
+    b = xt.clone().requires_grad_(True)
+    loss_b = mod.LargeMarginSoftmaxV3(lam=0.3, reduction=reduction, ignore_index=255, fb=False)(b, yt)
+    loss_b.backward()
+
+    assert loss.dtype == loss_b.dtype and a.grad.dtype == dtype
+    assert abs(float(loss.detach()) - want_loss) <= max(tol, 2e-6) * abs(want_loss) * (4 if dtype != torch.float32 else 1)
+    scale = np.abs(want_grad).max()
+    assert np.abs(a.grad.float().cpu().numpy() - want_grad).max() <= tol * scale
+    # same arithmetic as the recomputing pair: equal to the last bits of fp32, to one rounding of the 16-bit types
+    assert abs(float(loss) - float(loss_b)) <= 1e-6 * abs(float(loss_b)) + (0 if dtype == torch.float32 else tol * abs(float(loss_b)))
+    assert (a.grad.float() - b.grad.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else tol) * scale
+    # ignored pixels: exact zeros
+    ign = torch.from_numpy(y == 255).cuda().unsqueeze(1).expand_as(a.grad)
+    assert a.grad[ign].abs().max().item() == 0 if ign.any() else True
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES, ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("factor", [0.4, 1024.0, -1.0, 1.0])
+def test_an_upstream_gradient_other_than_one_scales_the_kept_gradient(mod, dtype, tol, factor):
+    shape = (2, 19, 33, 31)                     # 19 * 1023 elements per image: the scaling kernel's ragged end
+    x, y, xt, yt = inputs(302, shape, dtype)
+    a = xt.clone().requires_grad_(True)
+    (mod.LargeMarginSoftmaxV3(fb=True)(a, yt) * factor).backward()
+    b = xt.clone().requires_grad_(True)
+    (mod.LargeMarginSoftmaxV3(fb=False)(b, yt) * factor).backward()
+    ref = b.grad.float()
+    assert (a.grad.float() - ref).abs().max().item() <= max(tol, 1e-6) * 2 * ref.abs().max().item()
+
+
+def test_scale_unless_one_leaves_the_data_alone_for_one(mod):
+    from pytorch_loss import _native
+    for dtype, tag in [(torch.float32, 0), (torch.float16, 1), (torch.bfloat16, 2)]:
+        for numel in [1, 7, 4096, 100003]:
+            data = torch.randn(numel, device="cuda").to(dtype)
+            data[0] = float("nan")                      # NaN * 1 would stay NaN anyway; -0.0 and denormals must not change either
+            if numel > 1:
+                data[1] = -0.0
+            before = data.clone()
+            _native.scale_unless_one(data, tag, torch.ones((), device="cuda"))
+            assert data.view(torch.int16 if dtype != torch.float32 else torch.int32).equal(
+                before.view(torch.int16 if dtype != torch.float32 else torch.int32))
+            data = torch.randn(numel, device="cuda").to(dtype)
+            want = (data.float() * 3.0).to(dtype)
+            _native.scale_unless_one(data, tag, torch.full((), 3.0, device="cuda", dtype=torch.float64))
+            assert data.equal(want)
+
+
+def test_nothing_valid(mod):
+    x = torch.randn(2, 5, 8, 8, device="cuda", requires_grad=True)
+    y = torch.full((2, 8, 8), 255, device="cuda", dtype=torch.int64)
+    loss = mod.LargeMarginSoftmaxV3(fb=True)(x, y)
+    loss.backward()
+    assert torch.isnan(loss) and x.grad.abs().max().item() == 0
+    x.grad = None
+    loss = mod.LargeMarginSoftmaxV3(fb=True, reduction="sum")(x, y)
+    loss.backward()
+    assert float(loss) == 0 and x.grad.abs().max().item() == 0
+
+
+def test_other_dtypes_and_empty_input(mod):
+    x = torch.randn(2, 6, 4, 4, device="cuda", dtype=torch.float64, requires_grad=True)
+    y = torch.randint(0, 6, (2, 4, 4), device="cuda")
+    (mod.LargeMarginSoftmaxV3(fb=True)(x, y) * 2.0).backward()
+    z = x.detach().clone().requires_grad_(True)
+    (mod.LargeMarginSoftmaxV3(fb=False)(z, y) * 2.0).backward()
+    assert x.grad.dtype == torch.float64 and (x.grad - z.grad).abs().max().item() <= 1e-6 * z.grad.abs().max().item()
+    e = torch.zeros(0, 5, 4, 4, device="cuda", requires_grad=True)
+    out = mod.LargeMarginSoftmaxV3(fb=True, reduction="sum")(e, torch.zeros(0, 4, 4, device="cuda", dtype=torch.int64))
+    assert float(out) == 0
+
+
+def test_full_size_step(mod):
+    """(8,19,1024,1024): loss against the recomputing module's, gradient against it on a strided sample."""
+    shape = (8, 19, 1024, 1024)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(shape, device="cuda", generator=g) * 2
+    y = torch.randint(0, 19, (8, 1024, 1024), device="cuda", generator=g)
+    y[torch.rand((8, 1024, 1024), device="cuda", generator=g) < 0.05] = 255
+    a = x.clone().requires_grad_(True)
+    la = mod.LargeMarginSoftmaxV3(fb=True)(a, y)
+    la.backward()
+    b = x.clone().requires_grad_(True)
+    lb = mod.LargeMarginSoftmaxV3(fb=False)(b, y)
+    lb.backward()
+    assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb))
+    assert (a.grad - b.grad).abs().max().item() <= 2e-6 * b.grad.abs().max().item()
+
+
+@pytest.mark.parametrize("shape", [(2, 19, 32, 40), (70, 200)], ids=str)
+def test_the_entry_point_on_fp16_logits(mod, shape):
+    """The module keeps fp16 logits on the two passes; the entry point itself takes them ('sum': nothing underflows)."""
+    from pytorch_loss import _native
+    x, y, xt, yt = inputs(303, shape, torch.float16)
+    loss, grad, tag = _native.lmargin_forward_backward_reduced(xt, yt, 0.3, 255, False)
+    want_grad = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, np.ones(y.shape))
+    want_loss = oracle.lmargin_forward(x.astype(np.float64), y, 0.3, 255).sum()
+    assert tag == 1 and grad.dtype == torch.float16
+    assert abs(float(loss) - want_loss) <= 4e-3 * abs(want_loss)
+    assert np.abs(grad.float().cpu().numpy() - want_grad).max() <= 2e-3 * np.abs(want_grad).max()
