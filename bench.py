@@ -671,15 +671,17 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
                                       "what": "eager steps under torch.autograd.set_multithreading_enabled(False)"}
         except Exception as e:
             dist["calling_thread"] = {"error": "%s: %s" % (type(e).__name__, e)}
-    if name in ("lmargin", "focal"):
-        # the same module with fb=True (what the reference's repository-root copies of these two modules do: gradient
-        # computed in the forward pass and kept): one pass over the inputs per step. Its bytes: large margin reads the
-        # logits and writes the gradient (2bE) and reads the labels twice (the count of valid pixels, then the pass
-        # itself: 16P); focal reads logits and labels and writes the gradient (3bE).
+    if name in ("lsr", "lmargin", "focal"):
+        # the same module with fb=True (what the reference's repository-root copies of the large-margin and focal
+        # modules do: gradient computed in the forward pass and kept; for LSR a keyword the reference does not have):
+        # one pass over the inputs per step. Its bytes: LSR and large margin read the logits and write the gradient
+        # (2bE) and read the labels twice (the count of valid pixels, then the pass itself: 16P); focal reads logits
+        # and labels and writes the gradient (3bE).
         try:
             import pytorch_loss as pl
-            fb = (pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255, fb=True) if name == "lmargin"
-                  else pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean", fb=True))
+            fb = {"lsr": lambda: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="mean", ignore_index=255, fb=True),
+                  "lmargin": lambda: pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255, fb=True),
+                  "focal": lambda: pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean", fb=True)}[name]()
             fb_ms, fb_loss = time_steps(fb, logits, labels, steps, warmup)
             eb, E = ELEM_BYTES[dtype], numel(shape)
             fb_bytes = 3 * eb * E if name == "focal" else 2 * eb * E + 16 * (E // shape[1])

@@ -102,6 +102,18 @@ int plh_lsr_backward_scaled(const void *logits, int32_t dtype, const int64_t *la
                             int64_t n_size, int64_t dimsize, int64_t m_size,
                             int64_t ignore_index, float smooth, void *stream);
 
+/* Loss ('mean' / 'sum') and its gradient under an upstream gradient of 1 from ONE pass over the logits, as
+ * plh_lmargin_forward_backward_reduced does for the large-margin loss (no counterpart in the reference, whose LSR
+ * module has no forward+backward Function; label_smooth.py:150-172 of the repository root runs lsr_forward, then
+ * lsr_backward). The labels are counted first (n_valid_out: required), the pass writes grad_logits already divided by
+ * the count (mean); plh_scale_unless_one is the backward. Up to 32 channels; beyond, and for (N, C) rows of more than
+ * 32 classes, the entry point runs the forward and the backward kernels one after the other (same outputs). */
+int plh_lsr_forward_backward_reduced(const void *logits, int32_t dtype, const int64_t *labels,
+                                     float *loss_out, int64_t *n_valid_out, void *grad_logits, int32_t mean,
+                                     void *workspace, int64_t workspace_bytes,
+                                     int64_t n_size, int64_t dimsize, int64_t m_size,
+                                     int64_t ignore_index, float smooth, void *stream);
+
 /* The module step on channel planes that do not start on 128-byte lines (513 x 513, 769 x 769 crops; no counterpart in the reference, whose
  * backward recomputes the softmax, csrc/lsr_kernel.cu:139-225). plh_lsr_saves_lse says (1 / 0) whether it applies to
  * these sizes: fp32 logits and channel planes of at least 4096 pixels, with either a plane byte length that is no

@@ -113,6 +113,59 @@ extern "C" int plh_lsr_forward_reduced(const void *logits, int32_t dtype, const 
                            n_size, dimsize, m_size, ignore_index, smooth, stream);
 }
 
+extern "C" int plh_lsr_forward_backward_reduced(const void *logits, int32_t dtype, const int64_t *labels,
+                                                float *loss_out, int64_t *n_valid_out, void *grad_logits, int32_t mean,
+                                                void *workspace, int64_t workspace_bytes,
+                                                int64_t n_size, int64_t dimsize, int64_t m_size,
+                                                int64_t ignore_index, float smooth, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    if (!n_valid_out) return PLH_ERR_NULL_POINTER;
+    const size_t es = dtype_size(dtype);
+    int rc = check_slice_args(logits, labels, grad_logits, n_size, dimsize, m_size, es, es);
+    if (rc != PLH_OK) return rc;
+    Partials part;
+    rc = carve_partials(workspace, workspace_bytes, n_size * m_size, loss_out, n_valid_out, part);
+    if (rc != PLH_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const FinishMode mode = mean ? kFinishMeanOverCount : kFinishSum;
+    if (n_size * dimsize * m_size == 0) {
+        finish_partials(part, 0, loss_out, n_valid_out, mode, 0, st);
+        return check_launch();
+    }
+    const LsrParams p = make_params(n_size, dimsize, m_size, ignore_index, smooth, es);
+    // One pass where the register-resident kernels run: the mean's divisor first (a count of the labels), so that the
+    // pass writes the gradient already divided by it. The partials of the count are gone before the pass leaves its own.
+    const bool one_pass = dimsize <= kMaxRegsChannels;
+    if (one_pass && mean) {
+        const unsigned counted = count_valid_partials(labels, n_size * m_size, ignore_index, part, st);
+        finish_partials(part, counted, loss_out, n_valid_out, kFinishSum, 0, st);
+    }
+    const Upstream up{nullptr, 0, mean ? n_valid_out : nullptr, 1.f};
+    unsigned blocks = 0;
+    if (one_pass)
+        dispatch_dtype(dtype, [&](auto tag) {
+            using T = decltype(tag);
+            blocks = lsr_fused_typed<T>(static_cast<const T *>(logits), labels, up, static_cast<T *>(grad_logits), part, p,
+                                        st);
+        });
+    if (blocks != 0) {
+        finish_partials(part, blocks, loss_out, n_valid_out, mode, 0, st);
+        return check_launch();
+    }
+    // every other shape: the forward and the backward one after the other (same outputs; the forward's own count
+    // divides the gradient - the count taken above, if any, is the same number)
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        blocks = lsr_forward_typed<T>(static_cast<const T *>(logits), labels, nullptr, part, true, p, st);
+    });
+    finish_partials(part, blocks, loss_out, n_valid_out, mode, 0, st);
+    dispatch_dtype(dtype, [&](auto tag) {
+        using T = decltype(tag);
+        lsr_backward_typed<T>(static_cast<const T *>(logits), labels, up, static_cast<T *>(grad_logits), p, st);
+    });
+    return check_launch();
+}
+
 extern "C" int plh_lsr_saves_lse(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size) {
     return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 &&
            lsr_lse_applies(dtype_size(dtype), dimsize, m_size) ? 1 : 0;

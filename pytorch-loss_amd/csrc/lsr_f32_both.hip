@@ -1,0 +1,6 @@
+// LSR kernels that leave loss partials and gradient in one pass, for float logits (one translation unit per element
+// type and direction).
+#include "lsr_kernels.hpp"
+namespace plh {
+PLH_LSR_INSTANTIATE_BOTH(float)
+}

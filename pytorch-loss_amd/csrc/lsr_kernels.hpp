@@ -103,13 +103,18 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_fwd_regs(const T *__restrict__
     }
 }
 
-template <class T, int CP, int V, int Form>
+// WithLoss: the same kernel also leaves the block's sum of losses and its count of valid pixels in `part`, with the
+// forward kernel's arithmetic (the module's 'mean' / 'sum' and its gradient from one pass over the logits).
+template <class T, int CP, int V, int Form, bool WithLoss = false>
 __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__ x,
                                                           const int64_t *__restrict__ lab,
                                                           const Upstream up, T *__restrict__ grad,
-                                                          const LsrParams p) {
+                                                          const LsrParams p, Partials part) {
+    __shared__ float red[WithLoss ? 4 : 1];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
-    if (!at.live) return;
+    if (!WithLoss && !at.live) return;
+    float mine = 0.f;
+    int cnt = 0;
 
     // Labels and the upstream gradient are asked for before the slice: in the rows form the slice arrives through
     // LDS behind a wait, and the block-uniform forms gain as well (fp32 (8,19,1024,1024) backward 0.2305 -> 0.227 ms,
@@ -145,13 +150,27 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
             float xv[CP];
             const float mx = widen_and_max<T, V, CP>(raw, k, p.C, xv);
             const float c = mx * kLog2e;
-            float s = 0.f;
+            float s = 0.f, sx = 0.f, x_y = 0.f;
 #pragma unroll
             for (int j = 0; j < CP; ++j)
                 if (chan_ok<CP>(j, p.C)) {
+                    if constexpr (WithLoss) {
+                        sx += xv[j];
+                        x_y = (tgt == j) ? xv[j] : x_y;
+                    }
                     xv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(xv[j], kLog2e, -c));
                     s += xv[j];
                 }
+            if constexpr (WithLoss) {           // as lsr_fwd_regs
+                const float fc = (float)p.C;
+                const float r = __builtin_fmaf(mx, kLog2e, -c);
+                const float lse = (__builtin_amdgcn_logf(s) - r) * kLn2;
+                const float all = (sx - fc * mx) - fc * lse;
+                const float hot = (tgt >= 0) ? (p.w_pos - p.w_neg) * ((x_y - mx) - lse) : 0.f;
+                const bool valid = at.live && !ign;
+                mine += valid ? -(p.w_neg * all + hot) : 0.f;
+                cnt += valid ? 1 : 0;
+            }
             const float gk = go[k];
             const float scale = p.sumw * gk * __builtin_amdgcn_rcpf(s);     // one reciprocal per pixel
             float n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
@@ -169,7 +188,15 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 #pragma unroll
     for (int j = 0; j < CP; ++j)
         if (chan_ok<CP>(j, p.C)) raw[j] = raw[j] & mask;
-    at.store_slice(grad, p.C, p.m_size, raw);
+    if (!WithLoss || at.live) at.store_slice(grad, p.C, p.m_size, raw);
+    if constexpr (WithLoss) {
+        const float bs = block_sum_256(mine, red);
+        const float bc = block_sum_256((float)cnt, red);   // at most 1024 per block: exact in fp32
+        if (threadIdx.x == 0) {
+            part.sum[blockIdx.x] = bs;
+            part.cnt[blockIdx.x] = (int)bc;
+        }
+    }
 }
 
 // -------------------------------------------------------------- planes ----
@@ -863,9 +890,9 @@ static unsigned launch_fwd_regs(const T *x, const int64_t *lab, float *loss, Par
     return grid;
 }
 
-template <class T, int V>
-static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
-                            hipStream_t st) {
+template <class T, int V, bool WithLoss = false>
+static unsigned launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
+                                hipStream_t st, Partials part = Partials{nullptr, nullptr}) {
     const unsigned grid = regs_grid<V>(p.P);
     const bool uni = tiles_are_uniform(p.m_size, V, sizeof(T));
     switch ((p.C + 3) / 4) {
@@ -873,17 +900,18 @@ static void launch_bwd_regs(const T *x, const int64_t *lab, const Upstream &up, 
     case K:                                                                                                      \
         if constexpr (V * sizeof(T) == 8) {                                                                      \
             if (uni) {                                                                                           \
-                hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kUniform>), dim3(grid), dim3(kRegsBlock), 0, st, x,    \
-                                   lab, up, grad, p);                                                            \
+                hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kUniform, WithLoss>), dim3(grid), dim3(kRegsBlock), 0, \
+                                   st, x, lab, up, grad, p, part);                                               \
                 break;                                                                                           \
             }                                                                                                    \
         }                                                                                                        \
-        hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kGeneral>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab, up,  \
-                           grad, p);                                                                             \
+        hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, V, kGeneral, WithLoss>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
+                           lab, up, grad, p, part);                                                              \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
+    return grid;
 }
 
 // `image`: tiles per image (channel planes that start on element boundaries only)
@@ -1015,20 +1043,21 @@ static unsigned launch_fwd_image(const T *x, const int64_t *lab, float *loss, Pa
     return grid;
 }
 
-template <class T>
-static void launch_bwd_image(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
-                             hipStream_t st) {
+template <class T, bool WithLoss = false>
+static unsigned launch_bwd_image(const T *x, const int64_t *lab, const Upstream &up, T *grad, const LsrParams &p,
+                                 hipStream_t st, Partials part = Partials{nullptr, nullptr}) {
     const unsigned grid = image_grid<4>(p.P / p.m_size, p.m_size);
     switch ((p.C + 3) / 4) {
 #define PLH_CASE(K)                                                                                              \
     case K:                                                                                                      \
         if constexpr (4 * K <= kImageFormMaxChannels<T>)                                                         \
-            hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, 4, kPerImage>), dim3(grid), dim3(kRegsBlock), 0, st, x,   \
-                               lab, up, grad, p);                                                                \
+            hipLaunchKernelGGL((lsr_bwd_regs<T, 4 * K, 4, kPerImage, WithLoss>), dim3(grid), dim3(kRegsBlock), 0, st, \
+                               x, lab, up, grad, p, part);                                                       \
         break;
         PLH_CASE(1) PLH_CASE(2) PLH_CASE(3) PLH_CASE(4) PLH_CASE(5) PLH_CASE(6) PLH_CASE(7) PLH_CASE(8)
 #undef PLH_CASE
     }
+    return grid;
 }
 
 // Launches the forward; returns the number of blocks that wrote partials.
@@ -1163,8 +1192,25 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
     }
 }
 
+// Loss partials and gradient from one pass, where the register-resident kernels run (up to kMaxRegsChannels channels in
+// NCHW); returns the number of blocks that left partials, 0 for every other shape (nothing launched: the caller runs
+// the forward and the backward one after the other).
+template <class T>
+unsigned lsr_fused_typed(const T *logits, const int64_t *labels, const Upstream &up, T *grad_logits, Partials part,
+                         const LsrParams &p, hipStream_t st) {
+    constexpr int V = ElemTraits<T>::kVec;
+    switch (pick_shape(p.C, p.m_size, V, sizeof(T), logits, grad_logits, labels, nullptr, nullptr, true, true, true,
+                       kImageFormMaxChannels<T>)) {
+        case Shape::RegsVec: return launch_bwd_regs<T, V, true>(logits, labels, up, grad_logits, p, st, part);
+        case Shape::RegsOne:
+            if (image_form_pays<T>(p.C, p.m_size)) return launch_bwd_image<T, true>(logits, labels, up, grad_logits, p, st, part);
+            return launch_bwd_regs<T, 1, true>(logits, labels, up, grad_logits, p, st, part);
+        default: return 0;
+    }
+}
+
 // Per-dtype entries into the kernels of this header; explicitly instantiated per element type and direction
-// (lsr_f32_fwd.hip, lsr_f32_bwd.hip, ...) so that the six parts compile in parallel.
+// (lsr_f32_fwd.hip, lsr_f32_bwd.hip, lsr_f32_both.hip, ...) so that the nine parts compile in parallel.
 template <class T>
 unsigned lsr_forward_typed(const T *logits, const int64_t *labels, float *losses, Partials part, bool reduce,
                            const LsrParams &p, hipStream_t st) {
@@ -1177,12 +1223,16 @@ unsigned lsr_forward_typed(const T *logits, const int64_t *labels, float *losses
 #define PLH_LSR_BWD_SIGNATURE(T)                                                                                    \
     void lsr_backward_typed<T>(const T *, const int64_t *, const Upstream &, T *, const LsrParams &, hipStream_t);
 
+#define PLH_LSR_BOTH_SIGNATURE(T)                                                                                   \
+    unsigned lsr_fused_typed<T>(const T *, const int64_t *, const Upstream &, T *, Partials, const LsrParams &, hipStream_t);
 #define PLH_LSR_EXTERN(T)                  \
     extern template PLH_LSR_FWD_SIGNATURE(T) \
-    extern template PLH_LSR_BWD_SIGNATURE(T)
+    extern template PLH_LSR_BWD_SIGNATURE(T) \
+    extern template PLH_LSR_BOTH_SIGNATURE(T)
 
 // one translation unit per element type and direction (lsr_<type>_fwd.hip, lsr_<type>_bwd.hip)
 #define PLH_LSR_INSTANTIATE_FWD(T) template PLH_LSR_FWD_SIGNATURE(T)
 #define PLH_LSR_INSTANTIATE_BWD(T) template PLH_LSR_BWD_SIGNATURE(T)
+#define PLH_LSR_INSTANTIATE_BOTH(T) template PLH_LSR_BOTH_SIGNATURE(T)
 
 }  // namespace plh

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "plh_focal_forward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i32, _p, _i64, _i64, _f32, _f32, _p]),
     "plh_focal_backward_scaled": (ctypes.c_int, [_p, _i32, _p, _p, _f32, _p, _i64, _f32, _f32, _p]),
     "plh_focal_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i64, _f32, _f32, _p]),
+    "plh_lsr_forward_backward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_focal_forward_backward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _i32, _p, _i64, _i64, _f32, _f32, _p]),
     "plh_lmargin_forward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _f32, _p]),
@@ -402,16 +403,26 @@ def lmargin_forward_backward(logits, labels, lam, ignore_index):
     return _back_to(losses, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), cnt
 
 
+def lsr_forward_backward_reduced(logits, labels, ignore_index, smooth, mean):
+    return _pixel_forward_backward_reduced("plh_lsr_forward_backward_reduced", lsr_args(logits, labels), ignore_index,
+                                           smooth, mean)
+
+
 def lmargin_forward_backward_reduced(logits, labels, lam, ignore_index, mean):
-    """One pass over the logits: -> (loss: the sum or the mean, gradient under an upstream gradient of 1)."""
-    a = lmargin_args(logits, labels)
+    return _pixel_forward_backward_reduced("plh_lmargin_forward_backward_reduced", lmargin_args(logits, labels),
+                                           ignore_index, lam, mean)
+
+
+def _pixel_forward_backward_reduced(entry, a, ignore_index, param, mean):
+    """One pass over the logits: -> (loss: the sum or the mean, gradient under an upstream gradient of 1, the
+    gradient's dtype tag or None)."""
     dev = a.x.device
     loss = torch.empty((), dtype=torch.float32, device=dev)
     n_valid = torch.empty((), dtype=torch.int64, device=dev)
     grad = torch.empty_like(a.x)
     ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
-    _call(a.x, "plh_lmargin_forward_backward_reduced", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(loss), _ptr(n_valid), _ptr(grad),
-          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(lam))
+    _call(a.x, entry, _ptr(a.x), a.tag, _ptr(a.lb), _ptr(loss), _ptr(n_valid), _ptr(grad),
+          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(param))
     return _back_to(loss, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), (a.tag if a.x.dtype == a.dtype else None)
 
 

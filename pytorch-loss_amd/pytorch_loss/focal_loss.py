@@ -103,7 +103,8 @@ class FocalLossV3(nn.Module):
     def forward(self, logits, label):
         # fp16 logits keep the two passes: a gradient kept in fp16 at 1/numel of its size is subnormal before a loss
         # scale could lift it, where the backward kernel multiplies in fp32 and rounds once
-        fused = self.fb and logits.dtype != torch.float16
+        # (and a forward that no backward will follow computes no gradient)
+        fused = self.fb and logits.dtype != torch.float16 and logits.requires_grad and torch.is_grad_enabled()
         if fused and self.reduction in ("mean", "sum") and logits.numel() > 0:
             return _FocalFusedReducedFunction.apply(logits, label, self.alpha, self.gamma, self.reduction == "mean")
         if not fused and self.reduction in ("mean", "sum") and logits.numel() > 0:

@@ -58,20 +58,50 @@ class _LSRReducedFunction(torch.autograd.Function):
         return grad, None, None, None, None
 
 
+class _LSRFusedReducedFunction(torch.autograd.Function):
+    """fb=True with 'sum' / 'mean': loss and gradient from ONE pass over the logits, as the large-margin module's
+    fb=True (large_margin_softmax._LargeMarginFusedReducedFunction). The kept gradient is the one under an upstream
+    gradient of 1, already divided by the number of valid pixels for 'mean'; backward multiplies it in place by the
+    upstream scalar, a pass over it only when that scalar is not 1."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, lb_smooth, lb_ignore, mean):
+        loss, grads, tag = _native.lsr_forward_backward_reduced(logits, labels, lb_ignore, lb_smooth, mean)
+        ctx.variables = (grads, tag)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grads, tag = ctx.variables
+        ctx.variables = None        # handed over: autograd takes the tensor instead of copying it
+        return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
+
+
 class LabelSmoothSoftmaxCEV3(nn.Module):
     """Usage as nn.CrossEntropyLoss: logits (N, C, *) float, labels (N, *) int64.
 
     reduction: 'mean' divides the summed loss by the number of non-ignored pixels,
     'sum' sums, anything else returns the per-pixel tensor.
+
+    fb (not in the reference, whose LSR module has no forward+backward Function; the keyword of its
+    LargeMarginSoftmaxV3): True computes the gradient in the forward pass of a 'mean' / 'sum' loss and keeps it for
+    backward - one pass over the logits per step instead of two, as long as the loss reaches backward() with an
+    upstream gradient of 1; a weighted or scaled loss costs a further pass over the kept gradient. fp16 logits and
+    reduction 'none' are not affected.
     """
 
-    def __init__(self, lb_smooth=0.1, reduction="mean", ignore_index=-100):
+    def __init__(self, lb_smooth=0.1, reduction="mean", ignore_index=-100, fb=False):
         super().__init__()
         self.lb_smooth = lb_smooth
         self.reduction = reduction
         self.lb_ignore = ignore_index
+        self.fb = fb
 
     def forward(self, logits, labels):
+        if (self.fb and self.reduction in ("sum", "mean") and logits.numel() > 0 and logits.dtype != torch.float16
+                and logits.requires_grad and torch.is_grad_enabled()):
+            return _LSRFusedReducedFunction.apply(logits, labels, self.lb_smooth, self.lb_ignore,
+                                                  self.reduction == "mean")
         if self.reduction in ("sum", "mean") and logits.numel() > 0:
             return _LSRReducedFunction.apply(logits, labels, self.lb_smooth, self.lb_ignore,
                                              self.reduction == "mean")

@@ -104,7 +104,8 @@ class LargeMarginSoftmaxV3(nn.Module):
     def forward(self, logits, labels):
         # fp16 logits keep the two passes: a gradient kept in fp16 at 1/n_valid of its size is subnormal before a loss
         # scale could lift it, where the backward kernel multiplies in fp32 and rounds once
-        fused = self.fb and logits.dtype != torch.float16
+        # (and a forward that no backward will follow computes no gradient)
+        fused = self.fb and logits.dtype != torch.float16 and logits.requires_grad and torch.is_grad_enabled()
         if self.reduction in ("sum", "mean") and logits.numel() > 0:
             func = _LargeMarginFusedReducedFunction if fused else _LargeMarginReducedFunction
             return func.apply(logits, labels, self.lam, self.ignore_index, self.reduction == "mean")
