@@ -42,6 +42,13 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     unsigned long long *cnt = reinterpret_cast<unsigned long long *>(valid_cnt);
     if (WantCount) hipLaunchKernelGGL(lm_zero_count, dim3(1), dim3(1), 0, st, cnt);
     if (n_size * dimsize * m_size == 0) return check_launch();
+    // the fused pair's count of valid pixels comes from a pass over the labels (256 atomics): with the fused kernel
+    // counting, one atomic per wavefront on the one address, the call took 0.81 ms at (8,19,1024,1024) fp32 and 0.76 ms
+    // at (65536,1000); now 0.26 and 0.085 ms
+    if (WantCount) {
+        count_valid_total(lab, n_size * m_size, ignore, cnt, st);
+        cnt = nullptr;
+    }
     if (WantLoss && WantGrad && (!grad || misaligned(grad, es))) return grad ? PLH_ERR_MISALIGNED : PLH_ERR_NULL_POINTER;
     if (loss && misaligned(loss, 4)) return PLH_ERR_MISALIGNED;
 

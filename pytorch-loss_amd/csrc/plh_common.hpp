@@ -586,6 +586,10 @@ void finish_partials(const Partials &part, unsigned blocks, float *loss_out, int
 // number of blocks. For a pass that needs the mean's divisor before it runs. Defined in reduce.hip.
 unsigned count_valid_partials(const int64_t *labels, int64_t P, int64_t ignore, const Partials &part, hipStream_t stream);
 
+// The number of labels other than `ignore`, added to *total (which an earlier launch on the stream has zeroed) by at
+// most 256 atomics. Defined in reduce.hip.
+void count_valid_total(const int64_t *labels, int64_t P, int64_t ignore, unsigned long long *total, hipStream_t stream);
+
 // What the score pass of an OHEM loss forward (ohem.hip: the cross-entropy score kernel; the large-margin forward kernel
 // that also writes scores) leaves besides scores and losses, for the case that the threshold
 // rule decides the selection (at least n_min pixels score within the threshold, so "beyond the n_min lowest" holds

@@ -119,3 +119,20 @@ def test_full_size_step(mod):
     lb.backward()
     assert float(la.detach()) == float(lb.detach())
     assert torch.equal(a.grad, b.grad)
+
+
+@pytest.mark.parametrize("shape", [(3, 7, 13, 11), (2, 19, 32, 40)], ids=str)
+def test_labels_that_start_on_an_8_byte_boundary_only(mod, shape):
+    """The count of valid labels reads 16-byte pairs where it can: a label view one element into its storage cannot."""
+    x, y, xt, yt = inputs(324, shape, torch.float32)
+    store = torch.empty(y.size + 1, dtype=torch.int64, device="cuda")
+    lab = store[1:].view(y.shape)
+    lab.copy_(yt)
+    assert lab.data_ptr() % 16 == 8
+    a = xt.clone().requires_grad_(True)
+    la = mod.LabelSmoothSoftmaxCEV3(ignore_index=255, fb=True)(a, lab)
+    la.backward()
+    b = xt.clone().requires_grad_(True)
+    lb = mod.LabelSmoothSoftmaxCEV3(ignore_index=255, fb=False)(b, yt)
+    lb.backward()
+    assert float(la.detach()) == float(lb.detach()) and torch.equal(a.grad, b.grad)
