@@ -55,11 +55,10 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                                                      float *__restrict__ loss, T *__restrict__ grad,
                                                      unsigned long long *__restrict__ valid_cnt, Partials part,
                                                      const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
-    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
-    // backward carries no code for either
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
-    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    // whether a launch wants the partial sums shows in their pointer: they come from the forward and from the fused
+    // pair (the module's 'mean' / 'sum' in one pass), so the backward carries no code for them. (valid_cnt: the fused
+    // pair's count of valid pixels comes from a pass over the labels, count_valid_total; the kernels do not touch it.)
+    constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
     const PixelRef<V, Form> at(p.P, p.m_size, p.C, p.xcd_run);
@@ -89,7 +88,6 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
     float out[V], score[V];
     float g[(WantGrad && !kInPlace) ? CP : 1][V];
     unsigned keep[V];      // all ones for a pixel that counts, 0 for an ignored one
-    unsigned n_valid = 0;
     float mine = 0.f;
     int cnt = 0, below = 0;
     static_assert(!Early || kMayReduce, "the OHEM by-products belong to the forward");
@@ -189,7 +187,6 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                     }
                 }
         }
-        if constexpr (kMayCount) n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && !ign));
         if constexpr (kInPlace) __builtin_amdgcn_sched_barrier(0);
     }
     if (live) {
@@ -212,10 +209,6 @@ __global__ __launch_bounds__(kRegsBlock) void lm_regs(const T *__restrict__ x, c
                 }
             at.store_slice(grad, p.C, p.m_size, raw);
         }
-    }
-    if (WantCount) {
-        // lanes leave only at the tail of the grid, so lane 0 of a wave with work is alive
-        if ((threadIdx.x & 63) == 0) atomicAdd(valid_cnt, (unsigned long long)n_valid);
     }
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
@@ -421,11 +414,10 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
                                                 float *__restrict__ loss, T *__restrict__ grad,
                                                 unsigned long long *__restrict__ valid_cnt, Partials part,
                                                 const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
-    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
-    // backward carries no code for either
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
-    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    // whether a launch wants the partial sums shows in their pointer: they come from the forward and from the fused
+    // pair (the module's 'mean' / 'sum' in one pass), so the backward carries no code for them. (valid_cnt: the fused
+    // pair's count of valid pixels comes from a pass over the labels, count_valid_total; the kernels do not touch it.)
+    constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     constexpr int kPix = 256 / G;
     __shared__ float red[4];
@@ -433,7 +425,6 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
     const int sub = threadIdx.x % G;
     const int grp = threadIdx.x / G;
 
-    unsigned long long n_valid = 0;
     const int64_t rounds = ceil_div_dev(p.P, (int64_t)gridDim.x * kPix);
     for (int64_t r = 0; r < rounds; ++r) {
         const int64_t pix = (r * gridDim.x + blockIdx.x) * kPix + grp;
@@ -497,11 +488,6 @@ __global__ __launch_bounds__(256) void lm_group(const T *__restrict__ x, const i
             }
         }
         // every lane of the wave is inside the loop, so the ballot sees the whole wave
-        if constexpr (kMayCount)
-            n_valid += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live && sub == 0 && !ign));
-    }
-    if (WantCount) {
-        if ((threadIdx.x & 63) == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
@@ -522,11 +508,10 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                                                const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                unsigned long long *__restrict__ valid_cnt, Partials part,
                                                const LmParams p) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
-    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
-    // backward carries no code for either
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
-    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    // whether a launch wants the partial sums shows in their pointer: they come from the forward and from the fused
+    // pair (the module's 'mean' / 'sum' in one pass), so the backward carries no code for them. (valid_cnt: the fused
+    // pair's count of valid pixels comes from a pass over the labels, count_valid_total; the kernels do not touch it.)
+    constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[4];
     constexpr int L = WaveRow<T, NI, LP, G>::L;
@@ -535,7 +520,6 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
     const WaveRowAt<G> at;
     const int lane = at.sub;
     float mine = 0.f, cnt = 0.f;
-    unsigned long long n_valid = 0;
     for (int64_t r0 = at.start; r0 < p.P; r0 += at.stride) {   // wave-uniform
         const bool live = r0 + at.grp < p.P;
         const int64_t row = live ? r0 + at.grp : p.P - 1;
@@ -649,10 +633,6 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
                 cnt += ign ? 0.f : 1.f;
             }
         }
-        if constexpr (kMayCount) n_valid += (lane == 0 && live && !ign) ? 1 : 0;
-    }
-    if (WantCount) {
-        if (lane == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
@@ -742,17 +722,15 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                                                     const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
                                                     const LmParams p, int vec) {
-    // which of the two by-products a launch wants shows in its pointers; only the fused pair counts valid pixels, and
-    // partial sums come from the forward and from the fused pair (the module's 'mean' / 'sum' in one pass), so the
-    // backward carries no code for either
-    constexpr bool kMayCount = WantLoss && WantGrad, kMayReduce = WantLoss;
-    const bool WantCount = kMayCount && valid_cnt != nullptr;
+    // whether a launch wants the partial sums shows in their pointer: they come from the forward and from the fused
+    // pair (the module's 'mean' / 'sum' in one pass), so the backward carries no code for them. (valid_cnt: the fused
+    // pair's count of valid pixels comes from a pass over the labels, count_valid_total; the kernels do not touch it.)
+    constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     __shared__ float red[kRowBlock / 64];
     constexpr int L = RowChunk<T>::kLen;
     float mine = 0.f;
     int cnt = 0;
-    unsigned long long n_valid = 0;
     for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {       // block-uniform
         const T *xs = x + row * p.C;
         const int64_t lb = lab[row];
@@ -779,7 +757,6 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                 cnt += ign ? 0 : 1;
             }
         }
-        if constexpr (kMayCount) n_valid += (threadIdx.x == 0 && !ign) ? 1 : 0;
         if constexpr (WantGrad) {
             float go[1];
             load_upstream<1>(up, row, go);
@@ -804,9 +781,6 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
             for (int j = threadIdx.x; j < sp.head; j += row_threads()) store_one(gs + j, one(load_one(xs + j), j));
             for (int j = sp.tail_from + threadIdx.x; j < p.C; j += row_threads()) store_one(gs + j, one(load_one(xs + j), j));
         }
-    }
-    if (WantCount) {
-        if (threadIdx.x == 0 && n_valid) atomicAdd(valid_cnt, n_valid);
     }
     if (Reduce) {
         if (threadIdx.x == 0) {
