@@ -39,6 +39,11 @@ CASES = {
     "ohem_lmargin": (lambda pl: pl.OhemLargeMarginLoss(score_thresh=0.7, n_min=500, ignore_index=255), _seg),
     "focal": (lambda pl: pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean"), _binary),
     "dice": (lambda pl: pl.SoftDiceLossV3(p=1, smooth=1.0), _binary),
+    # loss and gradient from one pass, the backward a multiplication that returns at once (count of the labels,
+    # finishing kernels and the scalar test are all kernels on the stream)
+    "lsr_fb": (lambda pl: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction="mean", ignore_index=255, fb=True), _seg),
+    "lmargin_fb": (lambda pl: pl.LargeMarginSoftmaxV3(lam=0.3, reduction="mean", ignore_index=255, fb=True), _seg),
+    "focal_fb": (lambda pl: pl.FocalLossV3(alpha=0.25, gamma=2, reduction="mean", fb=True), _binary),
 }
 
 
