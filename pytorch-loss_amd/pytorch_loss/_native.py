@@ -426,6 +426,18 @@ def _pixel_forward_backward_reduced(entry, a, ignore_index, param, mean):
     return _back_to(loss, _loss_dtype(a.dtype)), _back_to(grad, a.dtype), (a.tag if a.x.dtype == a.dtype else None)
 
 
+def take_kept(ctx):
+    """The gradient that a forward+backward Function kept in ctx.variables, handed over to the one backward that may use
+    it: while the context still referred to the tensor, autograd would copy it into logits.grad (a pass over it) instead
+    of taking it, and a second backward would multiply it a second time."""
+    kept = ctx.variables
+    if kept is None:
+        raise RuntimeError("pytorch_loss: the gradient kept by this forward+backward (fb) loss went to an earlier "
+                           "backward(); run the forward again, or use fb=False to call backward() twice")
+    ctx.variables = None
+    return kept
+
+
 def scale_unless_one(data, tag, grad_scalar):
     """data *= grad_scalar in place (a 0-dim tensor), without touching data when it is exactly 1; tag: the library's
     dtype tag of `data`, or None for a tensor the library does not hold (then torch multiplies)."""

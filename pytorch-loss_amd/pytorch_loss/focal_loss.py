@@ -40,8 +40,7 @@ class FocalSigmoidLossFuncV3FB(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        grads = ctx.variables
-        ctx.variables = None        # handed over (see _FocalFusedReducedFunction.backward)
+        grads = _native.take_kept(ctx)
         grads.mul_(grad_output)
         return grads, None, None, None
 
@@ -79,10 +78,7 @@ class _FocalFusedReducedFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        grads, tag = ctx.variables
-        # the kept gradient is handed over, not shared: while this context still referred to it autograd would copy it
-        # into logits.grad (a pass over it) instead of taking it
-        ctx.variables = None
+        grads, tag = _native.take_kept(ctx)
         return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
 
 

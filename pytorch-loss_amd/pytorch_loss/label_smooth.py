@@ -72,8 +72,7 @@ class _LSRFusedReducedFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        grads, tag = ctx.variables
-        ctx.variables = None        # handed over: autograd takes the tensor instead of copying it
+        grads, tag = _native.take_kept(ctx)
         return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
 
 

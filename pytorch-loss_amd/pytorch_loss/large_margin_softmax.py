@@ -39,8 +39,7 @@ class LargeMarginSoftmaxFuncV3FB(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output, grad_cnt):
-        grads = ctx.variables
-        ctx.variables = None        # handed over (see _LargeMarginFusedReducedFunction.backward)
+        grads = _native.take_kept(ctx)
         grads.mul_(grad_output.unsqueeze(1))
         return grads, None, None, None
 
@@ -77,10 +76,7 @@ class _LargeMarginFusedReducedFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        grads, tag = ctx.variables
-        # the kept gradient is handed over, not shared: while this context still referred to it autograd would copy it
-        # into logits.grad (a pass over it) instead of taking it
-        ctx.variables = None
+        grads, tag = _native.take_kept(ctx)
         return _native.scale_unless_one(grads, tag, grad_output), None, None, None, None
 
 

@@ -101,7 +101,7 @@ def test_nothing_valid_no_gradient_wanted_and_a_second_backward(mod):
     assert torch.equal(plain, mod.LabelSmoothSoftmaxCEV3(ignore_index=255, fb=False)(x.detach(), y))
     loss = mod.LabelSmoothSoftmaxCEV3(ignore_index=255, fb=True)(x, y)
     loss.backward(retain_graph=True)
-    with pytest.raises(Exception):          # the kept gradient went to the first backward
+    with pytest.raises(RuntimeError, match="went to an earlier backward"):
         loss.backward()
 
 
