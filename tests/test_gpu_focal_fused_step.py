@@ -92,7 +92,7 @@ def test_per_element_losses_and_other_dtypes(mod):
     assert la.shape == a.shape and torch.equal(la, lb)
     assert (a.grad - b.grad).abs().max().item() <= 2e-6 * b.grad.abs().max().item()
     e = torch.zeros(0, 5, device="cuda", requires_grad=True)
-    assert float(mod.FocalLossV3(fb=True, reduction="sum")(e, torch.zeros(0, 5, device="cuda"))) == 0
+    assert float(mod.FocalLossV3(fb=True, reduction="sum")(e, torch.zeros(0, 5, device="cuda")).detach()) == 0
 
 
 def test_full_size_step(mod):
