@@ -126,3 +126,34 @@ def test_elementwise_ops(pl, shape):
     want_g = oracle.soft_dice_backward(gr.astype(np.float64), rows.astype(np.float64),
                                        y.reshape(shape[0], -1).astype(np.float64), stats, 2)
     assert np.abs(xt.grad.cpu().numpy() - want_g).max() <= 1e-5 * np.abs(want_g).max() + 1e-12
+
+
+@pytest.mark.parametrize("shape", _shapes(7, 24, 48, 5000))
+def test_one_pass_fb_modules_match_the_two_pass_modules(pl, shape):
+    """LSR, large margin and focal with fb=True ('mean' and 'sum', an upstream scalar of 1 and another one) against
+    the same modules with fb=False, which the tests above hold to the oracle."""
+    n, c, m = shape
+    x, y = seg_inputs(300 + n * c * m, (n, c, m), 255, 0.1)
+    yt = dev(y)
+    soft = dev((synth.uniform01(301, 4, x.size).reshape(x.shape) < 0.2).astype(np.float32))
+    for name, make, labels in (
+            ("lsr", lambda fb, r: pl.LabelSmoothSoftmaxCEV3(lb_smooth=0.1, reduction=r, ignore_index=255, fb=fb), yt),
+            ("lmargin", lambda fb, r: pl.LargeMarginSoftmaxV3(lam=0.3, reduction=r, ignore_index=255, fb=fb), yt),
+            ("focal", lambda fb, r: pl.FocalLossV3(alpha=0.25, gamma=2, reduction=r, fb=fb), soft)):
+        if c == 1 and name == "lmargin":
+            continue
+        for reduction, factor in (("mean", 1.0), ("sum", 1.0), ("mean", 0.3)):
+            got = []
+            for fb in (True, False):
+                xt = dev(x).requires_grad_()
+                loss = make(fb, reduction)(xt, labels)
+                (loss * factor if factor != 1.0 else loss).backward()
+                got.append((float(loss.detach()), xt.grad))
+            (la, ga), (lb, gb) = got
+            what = "%s %s %s x%g" % (name, shape, reduction, factor)
+            if np.isnan(lb):
+                assert np.isnan(la), what          # nothing valid under 'mean'
+            else:
+                assert abs(la - lb) <= 1e-6 * abs(lb) + 1e-7, what
+            # (one class: every gradient is an exact 0 and what either side leaves is rounding)
+            assert (ga - gb).abs().max().item() <= 2e-6 * gb.abs().max().item() + (1e-7 if c == 1 else 1e-12), what
