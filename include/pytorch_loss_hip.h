@@ -122,7 +122,7 @@ int plh_lsr_forward_backward_reduced(const void *logits, int32_t dtype, const in
  * log-sum-exp in lse_out (n_size*m_size floats; it writes no per-pixel losses), and plh_lsr_backward_scaled_lse is
  * plh_lsr_backward_scaled that forms the gradient from it, sumw*exp(x - lse) - w, plane by plane in each plane's own
  * cache lines (`kept`: optional byte mask as in plh_lsr_backward_kept, else NULL). The gradient equals the
- * recomputing kernels' to rounding (relative 1e-6). When logits and grad_logits do not sit at the same offset into a
+ * recomputing kernels' to rounding (relative 1e-6; 1e-5 beyond 512 channels, whose sums are longer). When logits and grad_logits do not sit at the same offset into a
  * 128-byte line the recomputing kernel runs and `lse` is not read. PLH_ERR_BAD_SIZE for sizes that
  * plh_lsr_saves_lse answers with 0. */
 int plh_lsr_saves_lse(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size);

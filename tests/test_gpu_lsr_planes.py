@@ -197,3 +197,39 @@ def test_many_channels_on_a_view_one_element_in(native):
     got = native.lsr_backward_scaled_lse(lse, 255, 0.1, one, n_valid, native.lsr_args(xt, yt))
     want = native.lsr_backward_scaled(xt, yt, 255, 0.1, one, n_valid)
     assert torch.equal(got, want)
+
+
+# more than 512 channels in NCHW: the forward whose wavefronts stream the channels (planes of 256 pixels and more; tiles
+# that end inside a plane; channel counts that leave some wavefronts one channel short, and short last batches)
+STREAM = [((1, 600, 16, 16), 2.0), ((2, 513, 17, 19), 1.0), ((1, 1000, 20, 20), 3.0), ((3, 519, 16, 17), 2.0), ((1, 545, 65, 65), 2.0)]
+
+
+@pytest.mark.parametrize("shape,scale", STREAM)
+def test_forward_beyond_512_channels(native, shape, scale):
+    x, y = inputs(151, shape, scale)
+    y.reshape(-1)[::37] = shape[1] + 5                       # labels without a target channel, not ignored
+    x[0, 3, 0, :5] = -np.inf                                 # exp(-inf) = 0 inside a batch
+    x[0, ::8, 1, 2] = -np.inf                                # a wavefront whose channels are all -inf at one pixel
+    xt, yt = dev(x), dev(y)
+    want = oracle.lsr_forward(x.astype(np.float64), y, 255, 0.1)
+    got = native.lsr_forward(xt, yt, 255, 0.1).cpu().numpy()
+    finite = np.isfinite(want)
+    assert np.array_equal(np.isfinite(got), finite)
+    assert np.abs(got[finite] - want[finite]).max() <= 2e-6 * np.abs(want[finite]).max()
+    for mean in (True, False):
+        loss, n_valid = native.lsr_forward_reduced(xt, yt, 255, 0.1, mean)
+        assert int(n_valid.item()) == int((y != 255).sum())
+    y2 = y.copy()
+    y2[0, 0, :5] = 255
+    y2[0, 1, 2] = 255                                        # the pixels with infinite losses out of the sum
+    want2 = oracle.lsr_forward(x.astype(np.float64), y2, 255, 0.1)
+    loss, n_valid = native.lsr_forward_reduced(xt, dev(y2), 255, 0.1, True)
+    assert abs(float(loss) - want2.sum() / (y2 != 255).sum()) <= 2e-6 * abs(want2.sum() / (y2 != 255).sum())
+    if lib_saves(native, shape):
+        _, _, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+        want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).reshape(-1).numpy()
+        assert np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-6 * np.abs(want_lse).max()
+
+
+def lib_saves(native, shape):
+    return native.load().plh_lsr_saves_lse(0, shape[0], shape[1], shape[2] * shape[3]) == 1
