@@ -57,7 +57,8 @@ def test_one_pass_step_matches_the_oracle_and_the_recomputing_module(mod, shape,
     scale = np.abs(want_grad).max()
     assert np.abs(a.grad.float().cpu().numpy() - want_grad).max() <= tol * scale
     # same arithmetic as the recomputing pair: equal to the last bits of fp32, to one rounding of the 16-bit types
-    assert abs(float(loss) - float(loss_b)) <= 1e-6 * abs(float(loss_b)) + (0 if dtype == torch.float32 else tol * abs(float(loss_b)))
+    la, lb = float(loss.detach()), float(loss_b.detach())
+    assert abs(la - lb) <= 1e-6 * abs(lb) + (0 if dtype == torch.float32 else tol * abs(lb))
     assert (a.grad.float() - b.grad.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else tol) * scale
     # ignored pixels: exact zeros
     ign = torch.from_numpy(y == 255).cuda().unsqueeze(1).expand_as(a.grad)
@@ -132,7 +133,7 @@ def test_full_size_step(mod):
     b = x.clone().requires_grad_(True)
     lb = mod.LargeMarginSoftmaxV3(fb=False)(b, y)
     lb.backward()
-    assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb))
+    assert abs(float(la.detach()) - float(lb.detach())) <= 1e-6 * abs(float(lb.detach()))
     assert (a.grad - b.grad).abs().max().item() <= 2e-6 * b.grad.abs().max().item()
 
 
