@@ -671,7 +671,8 @@ def run_workload(name, steps, warmup, device, dtype="f32"):
                                       "what": "eager steps under torch.autograd.set_multithreading_enabled(False)"}
         except Exception as e:
             dist["calling_thread"] = {"error": "%s: %s" % (type(e).__name__, e)}
-    if name == "focal" or (name in ("lsr", "lmargin") and shape[1] <= 32):     # (beyond 32 channels fb=True runs two passes)
+    # (beyond 32 channels fb=True runs two passes, except for large margin on (N, C) rows)
+    if name == "focal" or (name in ("lsr", "lmargin") and shape[1] <= 32) or (name == "lmargin" and len(shape) == 2):
         # the same module with fb=True (what the reference's repository-root copies of the large-margin and focal
         # modules do: gradient computed in the forward pass and kept; for LSR a keyword the reference does not have):
         # one pass over the inputs per step. Its bytes: LSR and large margin read the logits and write the gradient
