@@ -117,7 +117,9 @@ int plh_lsr_forward_backward_reduced(const void *logits, int32_t dtype, const in
 /* The module step on channel planes that do not start on 128-byte lines (513 x 513, 769 x 769 crops; no counterpart in the reference, whose
  * backward recomputes the softmax, csrc/lsr_kernel.cu:139-225). plh_lsr_saves_lse says (1 / 0) whether it applies to
  * these sizes: fp32 logits and channel planes of at least 4096 pixels, with either a plane byte length that is no
- * multiple of 128 and dimsize up to 24 or from 33 (25..32 keep their kernels), or dimsize above 256 on any plane.
+ * multiple of 128 and dimsize up to 24 or from 33 (25..32 keep their kernels), or dimsize above 256 on any plane;
+ * and, for every dtype, (N, C) rows (m_size 1) of more than 4096 classes, where the backward becomes elementwise over
+ * the flattened tensor (bf16 (8192,32000): forward + backward 0.357 -> 0.286 ms).
  * Then plh_lsr_forward_reduced_lse is plh_lsr_forward_reduced that also leaves every pixel's
  * log-sum-exp in lse_out (n_size*m_size floats; it writes no per-pixel losses), and plh_lsr_backward_scaled_lse is
  * plh_lsr_backward_scaled that forms the gradient from it, sumw*exp(x - lse) - w, plane by plane in each plane's own

@@ -317,7 +317,11 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
 // fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
 // (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
 // conversions.
+// (N, C) rows, any element type: rows longer than kRowLseMin classes, where the forward is the block-per-row kernel
+// (lsr_fwd_row leaves one value per row) and the backward from it (lsr_bwd_row_lse) needs no reduction.
+constexpr int kRowLseMin = 2 * kWaveRowCap;
 inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
+    if (m_size == 1) return dimsize > kRowLseMin;
     if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
     const bool off_lines = (m_size * (int64_t)elem_bytes) % 128 != 0;
     if (dimsize <= kMaxRegsChannels) return off_lines && image_form_pays<float>((int)dimsize, m_size);
@@ -832,6 +836,10 @@ __global__ __launch_bounds__(256) void lsr_bwd_wrow(const T *__restrict__ x, con
 template <class T>
 __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                    float *__restrict__ loss, Partials part, const LsrParams p, int vec) {
+    // vec: bit 0 - rows can be walked in 16-byte chunks; bit 1 - `loss` takes every row's log-sum-exp instead of its loss
+    // (LsrParams::lse for rows: the reduced forward writes no per-row losses, so the one output slot serves; a second
+    // conditional store per row, through the struct or an argument of its own, cost the kernel 40 %: (8192,32000) fp32
+    // 0.167 -> 0.236 ms)
     const bool Reduce = part.sum != nullptr;
     __shared__ float red[kRowBlock / 64];
     float mine = 0.f;
@@ -839,7 +847,7 @@ __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x
     const float fc = (float)p.C;
     for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
         const T *xs = x + row * p.C;
-        const RowStats st = row_combine(row_sweep<T>(xs, p.C, vec != 0), red, true);
+        const RowStats st = row_combine(row_sweep<T>(xs, p.C, (vec & 1) != 0), red, true);
         if (threadIdx.x == 0) {
             const int64_t lb = lab[row];
             const bool ign = (lb == p.ignore);
@@ -849,7 +857,7 @@ __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x
             const float all = (st.sx - fc * st.m) - fc * lse;
             const float hot = has_y ? (p.w_pos - p.w_neg) * ((x_y - st.m) - lse) : 0.f;
             const float acc = ign ? 0.f : -(p.w_neg * all + hot);
-            if (loss) loss[row] = acc;
+            if (loss) loss[row] = (vec & 2) ? st.m + lse : acc;
             mine += acc;
             cnt += ign ? 0 : 1;
         }
@@ -858,6 +866,62 @@ __global__ __launch_bounds__(kRowBlock) void lsr_fwd_row(const T *__restrict__ x
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
+// Backward of a long row from the forward's log-sum-exp: elementwise, g[j] = gk (sumw exp(x[j] - lse) - w(label == j)),
+// so the row is read once and no reduction (two block-wide barriers per row) stands between the loads and the stores.
+// One scalar upstream gradient, optionally the byte mask of an OHEM selection. Blocks take rows in turn; a thread has four
+// 16-byte chunks in flight.
+template <class T>
+__global__ __launch_bounds__(kRowBlockShort) void lsr_bwd_row_lse(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                                  const Upstream up, T *__restrict__ grad, const LsrParams p,
+                                                                  int vec) {
+    constexpr int L = RowChunk<T>::kLen;
+    float gk0 = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk0 = gk0 / (float)(*up.divide_by);
+    const int threads = row_threads();
+    for (int64_t row = blockIdx.x; row < p.P; row += gridDim.x) {
+        const T *xs = x + row * p.C;
+        T *gs = grad + row * p.C;
+        const RowSplit<T> sp(xs, p.C, vec != 0);
+        const int64_t lb = lab[row];
+        const bool dropped = lb == p.ignore || (up.keep && up.keep[row] == 0);
+        const float gk = dropped ? 0.f : gk0;
+        const float shift = -p.lse[row] * kLog2e;
+        const float scale = p.sumw * gk, n_pos = -p.w_pos * gk, n_neg = -p.w_neg * gk;
+        const int tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        auto one = [&](float xv, int j) {
+            // ignored rows: exact zeros whatever the logits are (0 * inf would be NaN)
+            const float g = __builtin_fmaf(__builtin_amdgcn_exp2f(__builtin_fmaf(xv, kLog2e, shift)), scale, (j == tgt) ? n_pos : n_neg);
+            return dropped ? 0.f : g;
+        };
+        const T *body = xs + sp.head;
+        T *gbody = gs + sp.head;
+        // four chunks in flight per thread to the end of the row (the last trip's loads are masked, not serialised)
+        for (int i = threadIdx.x; i < sp.chunks; i += 4 * threads) {
+            float v[4][L];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int at = i + u * threads < sp.chunks ? i + u * threads : i;
+                RowChunk<T>::load(body + (int64_t)at * L, v[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int at = i + u * threads;
+                if (at < sp.chunks) {
+#pragma unroll
+                    for (int e = 0; e < L; ++e) v[u][e] = one(v[u][e], sp.head + at * L + e);
+                    RowChunk<T>::store(gbody + (int64_t)at * L, v[u]);
+                }
+            }
+        }
+        // the row's ends (and the whole row when it cannot be walked in chunks): element by element
+        const int n_edge = sp.head + (p.C - sp.tail_from);
+        for (int k = threadIdx.x; k < n_edge; k += threads) {
+            const int j = k < sp.head ? k : sp.tail_from + (k - sp.head);
+            store_one(gs + j, one(load_one(xs + j), j));
         }
     }
 }
@@ -973,6 +1037,90 @@ __global__ __launch_bounds__(kRowBlock) void lsr_bwd_rowregs(const T *__restrict
             }
         }
         if (has_edge) store_one(gs + edge_at, __builtin_fmaf(fast_exp(edge - m), scale, (edge_at == tgt) ? n_pos : n_neg));
+    }
+}
+
+// The same over the flattened (rows x classes) tensor, for logits and gradient on 16-byte boundaries: a block takes 1024
+// consecutive 16-byte chunks (four per thread, coalesced) wherever rows begin and end, so the accesses are those of a
+// copy; a chunk finds its row by one 32-bit division (the block's first element by a 64-bit one, block-uniform), and a
+// chunk that straddles two rows goes element by element. Rows longer than a chunk (kRowLseMin classes at least).
+template <class T>
+__global__ __launch_bounds__(256) void lsr_bwd_flat_lse(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                        const Upstream up, T *__restrict__ grad, const LsrParams p,
+                                                        int64_t chunks) {
+    constexpr int L = RowChunk<T>::kLen, U = 4;
+    float gk0 = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk0 = gk0 / (float)(*up.divide_by);
+    const int64_t first = (int64_t)blockIdx.x * (256 * U);             // the block's first chunk
+    const int64_t row0 = first * L / p.C;                               // block-uniform
+    const unsigned col0 = (unsigned)(first * L - row0 * p.C);
+    const unsigned C = (unsigned)p.C;
+    float v[U][L];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t ch = first + threadIdx.x + 256 * u;
+        live[u] = ch < chunks;
+        RowChunk<T>::load(x + (live[u] ? ch : first) * L, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (!live[u]) continue;
+        const unsigned off = col0 + (threadIdx.x + 256u * u) * L;       // from the start of row0: below 2^32 (C < 2^31)
+        const unsigned dr = off / C;
+        unsigned col = off - dr * C;
+        int64_t row = row0 + dr;
+        auto row_terms = [&](int64_t r, float &shift, float &scale, float &n_pos, float &n_neg, int &tgt, bool &dropped) {
+            const int64_t lb = lab[r];
+            dropped = lb == p.ignore || (up.keep && up.keep[r] == 0);
+            const float gk = dropped ? 0.f : gk0;
+            shift = -p.lse[r] * kLog2e;
+            scale = p.sumw * gk;
+            n_pos = -p.w_pos * gk;
+            n_neg = -p.w_neg * gk;
+            tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        };
+        float shift, scale, n_pos, n_neg;
+        int tgt;
+        bool dropped;
+        row_terms(row, shift, scale, n_pos, n_neg, tgt, dropped);
+        const int64_t ch = first + threadIdx.x + 256 * u;
+        if (col + L <= C) {
+#pragma unroll
+            for (int e = 0; e < L; ++e) {
+                const float g = __builtin_fmaf(__builtin_amdgcn_exp2f(__builtin_fmaf(v[u][e], kLog2e, shift)), scale,
+                                               ((int)(col + e) == tgt) ? n_pos : n_neg);
+                v[u][e] = dropped ? 0.f : g;            // ignored rows: exact zeros whatever the logits are
+            }
+        } else {                                        // the chunk crosses into the next row
+#pragma unroll
+            for (int e = 0; e < L; ++e) {
+                if (col + e == C) {
+                    row += 1;
+                    col -= C;                           // wraps: col + e becomes 0 for this element
+                    row_terms(row, shift, scale, n_pos, n_neg, tgt, dropped);
+                }
+                const float g = __builtin_fmaf(__builtin_amdgcn_exp2f(__builtin_fmaf(v[u][e], kLog2e, shift)), scale,
+                                               ((int)(col + e) == tgt) ? n_pos : n_neg);
+                v[u][e] = dropped ? 0.f : g;
+            }
+        }
+        RowChunk<T>::store(grad + ch * L, v[u]);
+    }
+    // what is left after the last whole chunk: at most L - 1 elements of the last row
+    if (blockIdx.x == gridDim.x - 1) {
+        const int64_t done = chunks * L, total = p.P * p.C;
+        const int64_t at = done + threadIdx.x;
+        if (at < total) {
+            const int64_t r = p.P - 1;
+            const int64_t lb = lab[r];
+            const bool dropped = lb == p.ignore || (up.keep && up.keep[r] == 0);
+            const float gk = dropped ? 0.f : gk0;
+            const int j = (int)(at - r * p.C);
+            const float g = __builtin_fmaf(__builtin_amdgcn_exp2f((load_one(x + at) - p.lse[r]) * kLog2e), p.sumw * gk,
+                                           (j == lb) ? -p.w_pos * gk : -p.w_neg * gk);
+            store_one(grad + at, dropped ? 0.f : g);
+        }
     }
 }
 
@@ -1204,8 +1352,11 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
             const int piece = wrow_piece<T>(logits, nullptr, p.C);
             if (p.C > wrow_cap<T>(piece)) {
                 const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-                hipLaunchKernelGGL((lsr_fwd_row<T>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels, losses, part, p,
-                                   row_chunks_ok<T>(logits, nullptr, p.C));
+                // (the forward that keeps the log-sum-exp has no per-row losses to write: lsr.hip)
+                const bool keep_lse = p.lse != nullptr && losses == nullptr;
+                hipLaunchKernelGGL((lsr_fwd_row<T>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, logits, labels,
+                                   keep_lse ? p.lse : losses, part, p,
+                                   (row_chunks_ok<T>(logits, nullptr, p.C) ? 1 : 0) | (keep_lse ? 2 : 0));
                 return grid;
             }
             unsigned grid = 0;
@@ -1243,6 +1394,20 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                            const LsrParams &p, hipStream_t st) {
     constexpr int V = ElemTraits<T>::kVec;
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
+    if (p.lse && p.m_size == 1 && !go_vec && lsr_lse_applies(sizeof(T), p.C, p.m_size)) {
+        // long rows, from the forward's log-sum-exp: elementwise - over the flattened tensor when both tensors sit on
+        // 16-byte boundaries, else row by row
+        constexpr int L = RowChunk<T>::kLen;
+        const int64_t chunks = p.P * p.C / L, blocks = ceil_div(chunks, (int64_t)1024);
+        if (!misaligned(logits, 16) && !misaligned(grad_logits, 16) && blocks >= 1 && blocks < ((int64_t)1 << 31)) {
+            hipLaunchKernelGGL((lsr_bwd_flat_lse<T>), dim3((unsigned)blocks), dim3(256), 0, st, logits, labels, up,
+                               grad_logits, p, chunks);
+            return;
+        }
+        const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+        hipLaunchKernelGGL((lsr_bwd_row_lse<T>), dim3(grid), dim3(kRowBlockShort), 0, st, logits, labels, up, grad_logits, p, 0);
+        return;
+    }
     if constexpr (sizeof(T) == 4) {
         // from the forward's log-sum-exp, plane by plane: one scalar upstream gradient, logits and gradient at the same
         // offset into a 128-byte line (whole lines of the one are whole lines of the other)

@@ -44,6 +44,7 @@ def test_the_library_says_where_it_applies(native, shape, scale):
     assert lib.plh_lsr_saves_lse(0, n, 257, 4096) == 1                                               # beyond 256: any plane
     assert lib.plh_lsr_saves_lse(2, n, 150, m) == 0
     assert lib.plh_lsr_saves_lse(0, n, c, 4095) == 0        # short planes
+    assert lib.plh_lsr_saves_lse(0, n, 4097, 1) == 1 and lib.plh_lsr_saves_lse(2, n, 4097, 1) == 1      # long rows: any element type
 
 
 @pytest.mark.parametrize("mean", [True, False], ids=["mean", "sum"])
@@ -233,3 +234,61 @@ def test_forward_beyond_512_channels(native, shape, scale):
 
 def lib_saves(native, shape):
     return native.load().plh_lsr_saves_lse(0, shape[0], shape[1], shape[2] * shape[3]) == 1
+
+
+# (N, C) rows longer than 4096 classes: the block-per-row forward leaves one log-sum-exp per row and the backward is
+# elementwise over the flattened tensor (row ends inside 16-byte chunks, a last chunk that is not whole, one row only)
+ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100)]
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", ROWS, ids=str)
+def test_long_rows(native, shape, dtype, tol):
+    lib = native.load()
+    tag = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    assert lib.plh_lsr_saves_lse(tag, shape[0], shape[1], 1) == 1 and lib.plh_lsr_saves_lse(tag, shape[0], 4096, 1) == 0
+    x = synth.normal(161, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(161, shape[:1], shape[1], 255, 0.2)
+    y[::3] = shape[1] + 7 if shape[0] > 2 else y[::3]           # rows without a target class, not ignored
+    xt = torch.from_numpy(x).cuda().to(dtype)
+    x = xt.float().cpu().numpy()
+    yt = dev(y)
+    loss, n_valid, lse = native.lsr_forward_reduced_lse(xt, yt, 255, 0.1, True)
+    assert lse is not None and lse.shape == (shape[0],)
+    want_lse = torch.logsumexp(torch.from_numpy(x).double(), 1).numpy()
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 4e-6 * np.abs(want_lse).max()
+    nv = int((y != 255).sum())
+    assert int(n_valid.item()) == nv
+    scalar = torch.full((), 0.7, device="cuda")
+    kept = torch.ones(shape[0], dtype=torch.uint8, device="cuda")
+    kept[1::2] = 0
+    up = np.full(shape[:1], 0.7 / max(nv, 1))
+    want = oracle.lsr_backward(x.astype(np.float64), y, 255, 0.1, up)
+    got = native.lsr_backward_scaled_lse(lse, 255, 0.1, scalar, n_valid, native.lsr_args(xt, yt))
+    assert got.dtype == dtype
+    assert np.abs(got.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
+    ign = torch.from_numpy(y == 255).cuda()
+    if ign.any():
+        assert got[ign].abs().max().item() == 0
+    got_kept = native.lsr_backward_scaled_lse(lse, 255, 0.1, scalar, n_valid, native.lsr_args(xt, yt), kept=kept)
+    want_kept = want.copy()
+    want_kept[1::2] = 0
+    assert np.abs(got_kept.float().cpu().numpy() - want_kept).max() <= tol * np.abs(want).max()
+    assert got_kept[1::2].abs().max().item() == 0 if shape[0] > 1 else True
+
+
+def test_long_rows_on_views_off_the_16_byte_boundaries(native):
+    """Logits one element into their storage: the backward goes row by row, element by element."""
+    shape = (3, 4099)
+    x = synth.normal(162, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(162, shape[:1], shape[1], 255, 0.0)
+    store = torch.empty(x.size + 1, device="cuda")
+    xt = store[1:].view(shape)
+    xt.copy_(torch.from_numpy(x))
+    yt = dev(y)
+    a = xt.requires_grad_(True)
+    from pytorch_loss import LabelSmoothSoftmaxCEV3
+    loss = LabelSmoothSoftmaxCEV3(ignore_index=255)(a, yt)
+    loss.backward()
+    want = oracle.lsr_backward(x.astype(np.float64), y, 255, 0.1, np.full(shape[:1], 1.0 / shape[0]))
+    assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
