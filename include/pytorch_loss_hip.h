@@ -243,6 +243,26 @@ int plh_lmargin_forward_backward_reduced(const void *logits, int32_t dtype, cons
                                          int64_t n_size, int64_t dimsize, int64_t m_size,
                                          int64_t ignore_index, float lam, void *stream);
 
+/* Long (N, C) rows (m_size 1, more than 4096 classes, every dtype): the forward leaves eight floats of statistics per row
+ * (stats_out: n_size * 8 floats on a 16-byte boundary) and the backward forms the gradient from them elementwise over the
+ * flattened tensor instead of sweeping every row for them again (no counterpart in the reference, whose backward
+ * recomputes: csrc/large_margin_kernel.cu:387-599). plh_lmargin_saves_stats says (1 / 0) whether the sizes qualify;
+ * the other two are plh_lmargin_forward_reduced and plh_lmargin_backward_scaled / _kept (`kept`: optional byte mask, else
+ * NULL) with that one more argument, and return PLH_ERR_BAD_SIZE for sizes that do not qualify. When logits or
+ * grad_logits do not sit on 16-byte boundaries the recomputing kernel runs and `stats` is not read. */
+int plh_lmargin_saves_stats(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size);
+int plh_lmargin_forward_reduced_stats(const void *logits, int32_t dtype, const int64_t *labels, float *stats_out,
+                                      float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                      void *workspace, int64_t workspace_bytes,
+                                      int64_t n_size, int64_t dimsize, int64_t m_size,
+                                      int64_t ignore_index, float lam, void *stream);
+int plh_lmargin_backward_scaled_stats(const void *logits, int32_t dtype, const int64_t *labels,
+                                      const float *stats, const uint8_t *kept,
+                                      const float *grad_scalar, float scale, const int64_t *divide_by,
+                                      void *grad_logits,
+                                      int64_t n_size, int64_t dimsize, int64_t m_size,
+                                      int64_t ignore_index, float lam, void *stream);
+
 /* data[i] *= *scalar in place for numel elements of `dtype`, except that nothing is read or written when *scalar is exactly
  * 1: the backward of a kept gradient (replaces logits_grads.mul_(grad_output), large_margin_softmax.py:189 of the
  * repository root, for a scalar upstream gradient, which loss.backward() makes 1). `data` on a 16-byte boundary. */

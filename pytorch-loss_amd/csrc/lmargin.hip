@@ -25,7 +25,7 @@ static unsigned lmargin_run_typed(int variant, const T *x, const int64_t *lab, c
 static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab, const Upstream &up, float *loss, void *grad,
                   int64_t *valid_cnt, Partials part, unsigned *blocks_out, int64_t n_size, int64_t dimsize,
                   int64_t m_size, int64_t ignore, float lam, void *stream, float *scores = nullptr,
-                  float no_target_score = 1.f, const OhemEarly *early = nullptr) {
+                  float no_target_score = 1.f, const OhemEarly *early = nullptr, float *saved = nullptr) {
     const bool WantLoss = variant != kLmBackward, WantGrad = variant >= kLmBackward;
     const bool WantCount = variant == kLmForwardBackwardCount;
     const bool Reduce = variant == kLmForwardReduced || variant == kLmForwardBackwardReduced;
@@ -62,6 +62,7 @@ static int launch(int variant, const void *x, int32_t dtype, const int64_t *lab,
     p.xcd_run = xcd_run_for(es, m_size);
     p.scores = scores;
     p.no_target_score = no_target_score;
+    p.saved = saved;
     if (early) {
         p.early_kept = early->kept;
         p.early_below = early->below;
@@ -220,4 +221,44 @@ extern "C" int plh_lmargin_forward_backward_reduced(const void *logits, int32_t 
     if (rc != PLH_OK) return rc;
     finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
     return check_launch();
+}
+
+extern "C" int plh_lmargin_saves_stats(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size) {
+    return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 && lm_saved_applies(dimsize, m_size) ? 1 : 0;
+}
+
+extern "C" int plh_lmargin_forward_reduced_stats(const void *logits, int32_t dtype, const int64_t *labels, float *stats_out,
+                                                 float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                                 void *workspace, int64_t workspace_bytes,
+                                                 int64_t n_size, int64_t dimsize, int64_t m_size,
+                                                 int64_t ignore_index, float lam, void *stream) {
+    if (n_size < 0 || m_size < 0 || n_size > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    if (!lm_saved_applies(dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (!stats_out && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
+    if (misaligned(stats_out, 16)) return PLH_ERR_MISALIGNED;
+    Partials part;
+    int rc = carve_partials(workspace, workspace_bytes, n_size * m_size, loss_out, n_valid_out, part);
+    if (rc != PLH_OK) return rc;
+    const Upstream up{nullptr, 0, nullptr, 1.f};
+    unsigned blocks = 0;
+    rc = launch(kLmForwardReduced, logits, dtype, labels, up, nullptr, nullptr, nullptr, part, &blocks, n_size, dimsize,
+                m_size, ignore_index, lam, stream, nullptr, 1.f, nullptr, stats_out);
+    if (rc != PLH_OK) return rc;
+    finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0,
+                    (hipStream_t)stream);
+    return check_launch();
+}
+
+extern "C" int plh_lmargin_backward_scaled_stats(const void *logits, int32_t dtype, const int64_t *labels,
+                                                 const float *stats, const uint8_t *kept,
+                                                 const float *grad_scalar, float scale, const int64_t *divide_by,
+                                                 void *grad_logits,
+                                                 int64_t n_size, int64_t dimsize, int64_t m_size,
+                                                 int64_t ignore_index, float lam, void *stream) {
+    if (!lm_saved_applies(dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (n_size * dimsize * m_size != 0 && (!grad_scalar || !stats)) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8) || misaligned(stats, 16)) return PLH_ERR_MISALIGNED;
+    const Upstream up{grad_scalar, 0, divide_by, scale, kept};
+    return launch(kLmBackward, logits, dtype, labels, up, nullptr, grad_logits, nullptr, kNoPartials, nullptr, n_size,
+                  dimsize, m_size, ignore_index, lam, stream, nullptr, 1.f, nullptr, const_cast<float *>(stats));
 }

@@ -34,7 +34,17 @@ struct LmParams {
     uint8_t *early_kept = nullptr;
     int *early_below = nullptr;
     float early_thresh = 0.f;
+    // (N, C) rows of more than kLmRowSavedMin classes: kLmSavedFloats floats per row that the forward leaves (lm_row)
+    // and the backward reads instead of sweeping the row for them (lm_bwd_flat_saved); see lm_saved_applies
+    float *saved = nullptr;
 };
+
+// What the block-per-row forward leaves per row for the elementwise backward: the maximum m over the classes other than
+// the target, 1 / sum exp(x - m) over them, t_all / s_all (which turns exp(x - m) into the full softmax), sum q x, and
+// the target's p_y - 1; padded to 32 bytes.
+constexpr int kLmSavedFloats = 8;
+constexpr int kLmRowSavedMin = 2 * kWaveRowCap;
+inline bool lm_saved_applies(int64_t dimsize, int64_t m_size) { return m_size == 1 && dimsize > kLmRowSavedMin; }
 
 // ---------------------------------------------------------------- regs ----
 
@@ -721,12 +731,15 @@ template <class T, bool WantLoss, bool WantGrad>
 __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                     const Upstream up, float *__restrict__ loss, T *__restrict__ grad,
                                                     unsigned long long *__restrict__ valid_cnt, Partials part,
-                                                    const LmParams p, int vec) {
+                                                    const LmParams p, int vec_flags) {
     // whether a launch wants the partial sums shows in their pointer: they come from the forward and from the fused
     // pair (the module's 'mean' / 'sum' in one pass), so the backward carries no code for them. (valid_cnt: the fused
     // pair's count of valid pixels comes from a pass over the labels, count_valid_total; the kernels do not touch it.)
+    // vec_flags: bit 0 - rows can be walked in 16-byte chunks; bit 1 - `loss` takes kLmSavedFloats statistics per row
+    // instead of the row's loss (LmParams::saved: the reduced forward writes no per-row losses, so the slot serves)
     constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
+    const int vec = vec_flags & 1;
     __shared__ float red[kRowBlock / 64];
     constexpr int L = RowChunk<T>::kLen;
     float mine = 0.f;
@@ -751,7 +764,15 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
                 const float off = st.m + lse_no;
                 const float margin = p.half_lam * ((sum_qx - off) - p.coeff * (st.sx - n_no * off));
                 const float acc = margin - (x_y - m_all) + logf(s_all);
-                if (loss) loss[row] = ign ? 0.f : acc;
+                if (loss) {
+                    if (vec_flags & 2) {
+                        plh_f4 *to = reinterpret_cast<plh_f4 *>(loss + row * kLmSavedFloats);
+                        to[0] = plh_f4{st.m, inv_no, t_all * inv_all, sum_qx};
+                        to[1] = plh_f4{e_y * inv_all - 1.f, 0.f, 0.f, 0.f};
+                    } else {
+                        loss[row] = ign ? 0.f : acc;
+                    }
+                }
                 if (p.scores) p.scores[row] = (ign || tgt < 0) ? p.no_target_score : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0 : 1;
@@ -786,6 +807,82 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
+// Backward of long rows from the statistics the forward left (LmParams::saved), elementwise over the flattened
+// (rows x classes) tensor like lsr_bwd_flat_lse: a block takes 1024 consecutive 16-byte chunks wherever rows begin and
+// end; the arithmetic per element is lm_row's. Logits and gradient on 16-byte boundaries, one scalar upstream
+// gradient, optionally the byte mask of an OHEM selection.
+template <class T>
+__global__ __launch_bounds__(256) void lm_bwd_flat_saved(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                         const Upstream up, T *__restrict__ grad, const LmParams p,
+                                                         int64_t chunks) {
+    constexpr int L = RowChunk<T>::kLen, U = 4;
+    float gk0 = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk0 = gk0 / (float)(*up.divide_by);
+    const int64_t first = (int64_t)blockIdx.x * (256 * U);
+    const int64_t row0 = first * L / p.C;                               // block-uniform
+    const unsigned col0 = (unsigned)(first * L - row0 * p.C);
+    const unsigned C = (unsigned)p.C;
+    struct RowTerms { float m, inv_no, k_all, sum_qx, g_hot, gk; int tgt; bool dropped; };
+    auto row_terms = [&](int64_t r) {
+        RowTerms t;
+        const int64_t lb = lab[r];
+        t.dropped = lb == p.ignore || (up.keep && up.keep[r] == 0);
+        t.gk = t.dropped ? 0.f : gk0;
+        const plh_f4 *from = reinterpret_cast<const plh_f4 *>(p.saved + r * kLmSavedFloats);
+        const plh_f4 a = from[0];
+        t.m = a.x; t.inv_no = a.y; t.k_all = a.z; t.sum_qx = a.w;
+        t.g_hot = p.saved[r * kLmSavedFloats + 4] * t.gk;
+        t.tgt = (lb >= 0 && lb < p.C) ? (int)lb : -1;
+        return t;
+    };
+    auto one = [&](float xv, int j, const RowTerms &t) {
+        const float e = fast_exp(xv - t.m);
+        const float q = e * t.inv_no;
+        const float g_cold = (e * t.k_all + p.half_lam * ((xv + 1.f - t.sum_qx) * q - p.coeff)) * t.gk;
+        return t.dropped ? 0.f : ((j == t.tgt) ? t.g_hot : g_cold);
+    };
+    float v[U][L];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t ch = first + threadIdx.x + 256 * u;
+        live[u] = ch < chunks;
+        RowChunk<T>::load(x + (live[u] ? ch : first) * L, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (!live[u]) continue;
+        const unsigned off = col0 + (threadIdx.x + 256u * u) * L;       // from the start of row0: below 2^32 (C < 2^31)
+        const unsigned dr = off / C;
+        unsigned col = off - dr * C;
+        int64_t row = row0 + dr;
+        RowTerms t = row_terms(row);
+        if (col + L <= C) {
+#pragma unroll
+            for (int e = 0; e < L; ++e) v[u][e] = one(v[u][e], (int)(col + e), t);
+        } else {                                        // the chunk crosses into the next row
+#pragma unroll
+            for (int e = 0; e < L; ++e) {
+                if (col + e == C) {
+                    row += 1;
+                    col -= C;                           // wraps: col + e becomes 0 for this element
+                    t = row_terms(row);
+                }
+                v[u][e] = one(v[u][e], (int)(col + e), t);
+            }
+        }
+        RowChunk<T>::store(grad + (first + threadIdx.x + 256 * u) * L, v[u]);
+    }
+    // what is left after the last whole chunk: at most L - 1 elements of the last row
+    if (blockIdx.x == gridDim.x - 1) {
+        const int64_t at = chunks * L + threadIdx.x;
+        if (at < p.P * p.C) {
+            const RowTerms t = row_terms(p.P - 1);
+            store_one(grad + at, one(load_one(x + at), (int)(at - (p.P - 1) * p.C), t));
         }
     }
 }
@@ -865,6 +962,17 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
     const float *go_vec = (up.gout && up.stride == 1) ? up.gout : nullptr;
     const float *second_f32 = go_vec ? go_vec : p.scores;      // the score output belongs to forwards without upstream
     unsigned blocks = 0;
+    if constexpr (WantGrad && !WantLoss) {
+        // long rows, from the statistics the forward left: elementwise over the flattened tensor
+        constexpr int L = RowChunk<T>::kLen;
+        const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)1024);
+        if (p.saved && !go_vec && lm_saved_applies(p.C, p.m_size) && !misaligned(x, 16) && !misaligned(grad, 16) &&
+            flat_blocks >= 1 && flat_blocks < ((int64_t)1 << 31)) {
+            hipLaunchKernelGGL((lm_bwd_flat_saved<T>), dim3((unsigned)flat_blocks), dim3(256), 0, st, x, lab, up, grad, p,
+                               chunks);
+            return (unsigned)flat_blocks;
+        }
+    }
     const unsigned early_bit = (WantLoss && !WantGrad && p.early_kept && part.sum) ? kLmTookEarly : 0u;
     // the split shape exists for the one-direction kernels (forward, reduced forward, backward)
     constexpr bool kHasSplit = !(WantLoss && WantGrad);
@@ -954,8 +1062,14 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
                 break;
             }
             blocks = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-            hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0, st,
-                               x, lab, up, loss, grad, cnt, part, p, row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C));
+            {
+                // (the forward that leaves the rows' statistics has no per-row losses to write: lmargin.hip)
+                const bool keep = WantLoss && !WantGrad && p.saved != nullptr && loss == nullptr &&
+                                  lm_saved_applies(p.C, p.m_size);
+                hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0,
+                                   st, x, lab, up, keep ? p.saved : loss, grad, cnt, part, p,
+                                   (row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C) ? 1 : 0) | (keep ? 2 : 0));
+            }
             break;
         case Shape::Lane:
             blocks = group_grid(p.P, 256);

@@ -50,6 +50,9 @@ _SIGNATURES = {
     "plh_lmargin_forward_backward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lmargin_forward_backward_reduced": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_scale_unless_one": (ctypes.c_int, [_p, _i32, _i64, _p, _p]),
+    "plh_lmargin_saves_stats": (ctypes.c_int, [_i32, _i64, _i64, _i64]),
+    "plh_lmargin_forward_reduced_stats": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _f32, _p]),
+    "plh_lmargin_backward_scaled_stats": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _f32, _p]),
     "plh_lovasz_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "plh_lovasz_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_lsr_saves_lse": (ctypes.c_int, [_i32, _i64, _i64, _i64]),
@@ -387,6 +390,33 @@ def lmargin_forward_reduced(logits, labels, lam, ignore_index, mean, args=None):
 def lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_scalar, divide_by=None, args=None):
     return _pixel_backward_scaled("plh_lmargin_backward_scaled", args or lmargin_args(logits, labels), ignore_index,
                                   lam, grad_scalar, divide_by)
+
+
+def lmargin_forward_reduced_stats(logits, labels, lam, ignore_index, mean, args=None):
+    """lmargin_forward_reduced that also keeps every row's statistics where the library's backward can use them (long
+    rows, see plh_lmargin_saves_stats). -> (loss, n_valid, stats or None)."""
+    a = args or lmargin_args(logits, labels)
+    if a.x.numel() == 0 or not load().plh_lmargin_saves_stats(a.tag, a.n, a.c, a.m):
+        return _pixel_forward_reduced("plh_lmargin_forward_reduced", a, ignore_index, lam, mean) + (None,)
+    dev = a.x.device
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    n_valid = torch.empty((), dtype=torch.int64, device=dev)
+    stats = torch.empty((a.n * a.m, 8), dtype=torch.float32, device=dev)
+    ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
+    _call(a.x, "plh_lmargin_forward_reduced_stats", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(stats), _ptr(loss), _ptr(n_valid),
+          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(ignore_index), float(lam))
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, stats
+
+
+def lmargin_backward_scaled_stats(stats, lam, ignore_index, grad_scalar, divide_by, args, kept=None):
+    """The gradient from the forward's row statistics (lmargin_forward_reduced_stats); `kept`: optional byte mask."""
+    a = args
+    grad = torch.empty_like(a.x)
+    go = _scalar_f32(grad_scalar)
+    _call(a.x, "plh_lmargin_backward_scaled_stats", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(stats),
+          _ptr(kept) if kept is not None else None, _ptr(go), 1.0, _ptr(divide_by), _ptr(grad), a.n, a.c, a.m,
+          int(ignore_index), float(lam))
+    return _back_to(grad, a.dtype)
 
 
 def lmargin_forward_backward(logits, labels, lam, ignore_index):

@@ -50,14 +50,22 @@ class _LargeMarginReducedFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels, lam, ignore_index, mean):
         ctx.args = args = _native.lmargin_args(logits, labels)
-        loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean, args=args)
-        ctx.variables = (logits, labels, lam, ignore_index, n_valid if mean else None)
+        stats = None
+        if ctx.needs_input_grad[0]:
+            # long rows: the forward also keeps eight floats per row, and the backward works elementwise from them
+            loss, n_valid, stats = _native.lmargin_forward_reduced_stats(logits, labels, lam, ignore_index, mean, args=args)
+        else:
+            loss, n_valid = _native.lmargin_forward_reduced(logits, labels, lam, ignore_index, mean, args=args)
+        ctx.variables = (logits, labels, lam, ignore_index, n_valid if mean else None, stats)
         return loss
 
     @staticmethod
     def backward(ctx, grad_output):
-        logits, labels, lam, ignore_index, n_valid = ctx.variables
-        grads = _native.lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_output, n_valid, args=ctx.args)
+        logits, labels, lam, ignore_index, n_valid, stats = ctx.variables
+        if stats is not None:
+            grads = _native.lmargin_backward_scaled_stats(stats, lam, ignore_index, grad_output, n_valid, ctx.args)
+        else:
+            grads = _native.lmargin_backward_scaled(logits, labels, lam, ignore_index, grad_output, n_valid, args=ctx.args)
         return grads, None, None, None, None
 
 

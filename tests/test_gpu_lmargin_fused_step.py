@@ -148,3 +148,67 @@ def test_the_entry_point_on_fp16_logits(mod, shape):
     assert tag == 1 and grad.dtype == torch.float16
     assert abs(float(loss) - want_loss) <= 4e-3 * abs(want_loss)
     assert np.abs(grad.float().cpu().numpy() - want_grad).max() <= 2e-3 * np.abs(want_grad).max()
+
+
+# (N, C) rows of more than 4096 classes: the forward leaves eight floats of statistics per row and the backward is
+# elementwise over the flattened tensor (row ends inside 16-byte chunks, a last chunk that is not whole, one row only)
+LONG_ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100)]
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES, ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", LONG_ROWS, ids=str)
+def test_long_rows_backward_from_the_forwards_statistics(mod, shape, dtype, tol):
+    from pytorch_loss import _native
+    lib = _native.load()
+    tag = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    assert lib.plh_lmargin_saves_stats(tag, shape[0], shape[1], 1) == 1
+    assert lib.plh_lmargin_saves_stats(tag, shape[0], 4096, 1) == 0 and lib.plh_lmargin_saves_stats(tag, 2, 5000, 4) == 0
+    x = synth.normal(331, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(331, shape[:1], shape[1], 255, 0.2)
+    if shape[0] > 2:
+        y[::3] = shape[1] + 7                           # rows without a target class, not ignored
+    xt = torch.from_numpy(x).cuda().to(dtype)
+    x = xt.float().cpu().numpy()
+    yt = torch.from_numpy(y).cuda()
+    args = _native.lmargin_args(xt, yt)
+    loss, n_valid, stats = _native.lmargin_forward_reduced_stats(xt, yt, 0.3, 255, True, args=args)
+    loss2, n_valid2 = _native.lmargin_forward_reduced(xt, yt, 0.3, 255, True)
+    assert stats is not None and stats.shape == (shape[0], 8)
+    assert torch.equal(loss, loss2) and int(n_valid) == int(n_valid2) == int((y != 255).sum())
+    nv = max(int((y != 255).sum()), 1)
+    scalar = torch.full((), 0.7, device="cuda")
+    want = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, np.full(shape[:1], 0.7 / nv))
+    got = _native.lmargin_backward_scaled_stats(stats, 0.3, 255, scalar, n_valid, args)
+    recomputed = _native.lmargin_backward_scaled(xt, yt, 0.3, 255, scalar, n_valid)
+    scale = np.abs(want).max()
+    assert got.dtype == dtype
+    assert np.abs(got.float().cpu().numpy() - want).max() <= tol * scale
+    assert (got.float() - recomputed.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else tol) * scale
+    ign = torch.from_numpy(y == 255).cuda()
+    if ign.any():
+        assert got[ign].abs().max().item() == 0
+    kept = torch.ones(shape[0], dtype=torch.uint8, device="cuda")
+    kept[1::2] = 0
+    got_kept = _native.lmargin_backward_scaled_stats(stats, 0.3, 255, scalar, n_valid, args, kept=kept)
+    want_kept = want.copy()
+    want_kept[1::2] = 0
+    assert np.abs(got_kept.float().cpu().numpy() - want_kept).max() <= tol * scale
+    if shape[0] > 1:
+        assert got_kept[1::2].abs().max().item() == 0
+
+
+def test_long_rows_module_step_and_views_off_the_16_byte_boundaries(mod):
+    shape = (3, 4099)
+    x = synth.normal(332, 1, shape, 0.0, 2.0)
+    y = synth.seg_labels(332, shape[:1], shape[1], 255, 0.0)
+    yt = torch.from_numpy(y).cuda()
+    want = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, np.full(shape[:1], 1.0 / shape[0]))
+    a = torch.from_numpy(x).cuda().requires_grad_(True)
+    mod.LargeMarginSoftmaxV3(ignore_index=255)(a, yt).backward()
+    assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+    store = torch.empty(x.size + 1, device="cuda")       # logits one element into their storage: the recomputing kernel
+    b = store[1:].view(shape)
+    b.copy_(torch.from_numpy(x))
+    b.requires_grad_(True)
+    mod.LargeMarginSoftmaxV3(ignore_index=255)(b, yt).backward()
+    assert np.abs(b.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
