@@ -224,7 +224,7 @@ extern "C" int plh_lmargin_forward_backward_reduced(const void *logits, int32_t 
 }
 
 extern "C" int plh_lmargin_saves_stats(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size) {
-    return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 && lm_saved_applies(dimsize, m_size) ? 1 : 0;
+    return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 && lm_saved_applies(dtype_size(dtype), dimsize, m_size) ? 1 : 0;
 }
 
 extern "C" int plh_lmargin_forward_reduced_stats(const void *logits, int32_t dtype, const int64_t *labels, float *stats_out,
@@ -233,7 +233,8 @@ extern "C" int plh_lmargin_forward_reduced_stats(const void *logits, int32_t dty
                                                  int64_t n_size, int64_t dimsize, int64_t m_size,
                                                  int64_t ignore_index, float lam, void *stream) {
     if (n_size < 0 || m_size < 0 || n_size > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
-    if (!lm_saved_applies(dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    if (!lm_saved_applies(dtype_size(dtype), dimsize, m_size)) return PLH_ERR_BAD_SIZE;
     if (!stats_out && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
     if (misaligned(stats_out, 16)) return PLH_ERR_MISALIGNED;
     Partials part;
@@ -255,7 +256,8 @@ extern "C" int plh_lmargin_backward_scaled_stats(const void *logits, int32_t dty
                                                  void *grad_logits,
                                                  int64_t n_size, int64_t dimsize, int64_t m_size,
                                                  int64_t ignore_index, float lam, void *stream) {
-    if (!lm_saved_applies(dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    if (!lm_saved_applies(dtype_size(dtype), dimsize, m_size)) return PLH_ERR_BAD_SIZE;
     if (n_size * dimsize * m_size != 0 && (!grad_scalar || !stats)) return PLH_ERR_NULL_POINTER;
     if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8) || misaligned(stats, 16)) return PLH_ERR_MISALIGNED;
     const Upstream up{grad_scalar, 0, divide_by, scale, kept};

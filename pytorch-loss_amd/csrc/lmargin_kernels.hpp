@@ -34,7 +34,7 @@ struct LmParams {
     uint8_t *early_kept = nullptr;
     int *early_below = nullptr;
     float early_thresh = 0.f;
-    // (N, C) rows of more than kLmRowSavedMin classes: kLmSavedFloats floats per row that the forward leaves (lm_row)
+    // (N, C) rows that the block-per-row kernels take (rows_take_block_kernels): kLmSavedFloats floats per row that the forward leaves (lm_row)
     // and the backward reads instead of sweeping the row for them (lm_bwd_flat_saved); see lm_saved_applies
     float *saved = nullptr;
 };
@@ -43,8 +43,9 @@ struct LmParams {
 // the target, 1 / sum exp(x - m) over them, t_all / s_all (which turns exp(x - m) into the full softmax), sum q x, and
 // the target's p_y - 1; padded to 32 bytes.
 constexpr int kLmSavedFloats = 8;
-constexpr int kLmRowSavedMin = 2 * kWaveRowCap;
-inline bool lm_saved_applies(int64_t dimsize, int64_t m_size) { return m_size == 1 && dimsize > kLmRowSavedMin; }
+inline bool lm_saved_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
+    return m_size == 1 && rows_take_block_kernels(elem_bytes, dimsize);
+}
 
 // ---------------------------------------------------------------- regs ----
 
@@ -966,7 +967,7 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
         // long rows, from the statistics the forward left: elementwise over the flattened tensor
         constexpr int L = RowChunk<T>::kLen;
         const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)1024);
-        if (p.saved && !go_vec && lm_saved_applies(p.C, p.m_size) && !misaligned(x, 16) && !misaligned(grad, 16) &&
+        if (p.saved && !go_vec && lm_saved_applies(sizeof(T), p.C, p.m_size) && !misaligned(x, 16) && !misaligned(grad, 16) &&
             flat_blocks >= 1 && flat_blocks < ((int64_t)1 << 31)) {
             hipLaunchKernelGGL((lm_bwd_flat_saved<T>), dim3((unsigned)flat_blocks), dim3(256), 0, st, x, lab, up, grad, p,
                                chunks);
@@ -1065,7 +1066,7 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
             {
                 // (the forward that leaves the rows' statistics has no per-row losses to write: lmargin.hip)
                 const bool keep = WantLoss && !WantGrad && p.saved != nullptr && loss == nullptr &&
-                                  lm_saved_applies(p.C, p.m_size);
+                                  lm_saved_applies(sizeof(T), p.C, p.m_size);
                 hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0,
                                    st, x, lab, up, keep ? p.saved : loss, grad, cnt, part, p,
                                    (row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C) ? 1 : 0) | (keep ? 2 : 0));

@@ -317,11 +317,12 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
 // fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
 // (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
 // conversions.
-// (N, C) rows, any element type: rows longer than kRowLseMin classes, where the forward is the block-per-row kernel
-// (lsr_fwd_row leaves one value per row) and the backward from it (lsr_bwd_row_lse) needs no reduction.
-constexpr int kRowLseMin = 2 * kWaveRowCap;
+// (N, C) rows, any element type: rows of more than 4096 classes, which the block-per-row forward takes whatever the
+// pointers' alignment (lsr_fwd_row leaves one value per row); the backward from it (lsr_bwd_flat_lse) needs no
+// reduction. (Rows of 2049 .. 4096 classes that the same forward takes gain nothing: fp32 (65536,4096) forward +
+// backward 0.511 ms recomputing - the row stays in the block's registers - against 0.555 ms, (65536,3000) 0.433 / 0.424.)
 inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    if (m_size == 1) return dimsize > kRowLseMin;
+    if (m_size == 1) return dimsize > 2 * kWaveRowCap;
     if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
     const bool off_lines = (m_size * (int64_t)elem_bytes) % 128 != 0;
     if (dimsize <= kMaxRegsChannels) return off_lines && image_form_pays<float>((int)dimsize, m_size);
@@ -1043,7 +1044,7 @@ __global__ __launch_bounds__(kRowBlock) void lsr_bwd_rowregs(const T *__restrict
 // The same over the flattened (rows x classes) tensor, for logits and gradient on 16-byte boundaries: a block takes 1024
 // consecutive 16-byte chunks (four per thread, coalesced) wherever rows begin and end, so the accesses are those of a
 // copy; a chunk finds its row by one 32-bit division (the block's first element by a 64-bit one, block-uniform), and a
-// chunk that straddles two rows goes element by element. Rows longer than a chunk (kRowLseMin classes at least).
+// chunk that straddles two rows goes element by element. Rows longer than a chunk (4097 classes at least).
 template <class T>
 __global__ __launch_bounds__(256) void lsr_bwd_flat_lse(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                         const Upstream up, T *__restrict__ grad, const LsrParams p,

@@ -162,7 +162,7 @@ def test_long_rows_backward_from_the_forwards_statistics(mod, shape, dtype, tol)
     lib = _native.load()
     tag = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
     assert lib.plh_lmargin_saves_stats(tag, shape[0], shape[1], 1) == 1
-    assert lib.plh_lmargin_saves_stats(tag, shape[0], 4096, 1) == 0 and lib.plh_lmargin_saves_stats(tag, 2, 5000, 4) == 0
+    assert lib.plh_lmargin_saves_stats(tag, shape[0], 2048, 1) == 0 and lib.plh_lmargin_saves_stats(tag, 2, 5000, 4) == 0
     x = synth.normal(331, 1, shape, 0.0, 2.0)
     y = synth.seg_labels(331, shape[:1], shape[1], 255, 0.2)
     if shape[0] > 2:
@@ -212,3 +212,28 @@ def test_long_rows_module_step_and_views_off_the_16_byte_boundaries(mod):
     b.requires_grad_(True)
     mod.LargeMarginSoftmaxV3(ignore_index=255)(b, yt).backward()
     assert np.abs(b.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+
+
+def test_rows_between_the_two_capacities_of_a_wavefront(mod):
+    """2049 .. 4096 classes: the block-per-row forward runs for fp32 rows and for 16-bit rows whose length is no multiple of
+    8, and only there the statistics are kept."""
+    from pytorch_loss import _native
+    lib = _native.load()
+    assert lib.plh_lmargin_saves_stats(0, 4, 2049, 1) == 1 and lib.plh_lmargin_saves_stats(0, 4, 4096, 1) == 1
+    assert lib.plh_lmargin_saves_stats(2, 4, 3000, 1) == 0 and lib.plh_lmargin_saves_stats(2, 4, 3001, 1) == 1
+    for shape, dtype, tol in [((3, 2049), torch.float32, 2e-6), ((4, 3000), torch.float32, 2e-6), ((2, 4096), torch.float32, 2e-6),
+                              ((4, 3001), torch.bfloat16, 1.6e-2), ((5, 2051), torch.float16, 2e-3)]:
+        x = synth.normal(341, 1, shape, 0.0, 2.0)
+        y = synth.seg_labels(341, shape[:1], shape[1], 255, 0.2)
+        xt = torch.from_numpy(x).cuda().to(dtype)
+        x = xt.float().cpu().numpy()
+        yt = torch.from_numpy(y).cuda()
+        args = _native.lmargin_args(xt, yt)
+        loss, n_valid, stats = _native.lmargin_forward_reduced_stats(xt, yt, 0.3, 255, True, args=args)
+        assert stats is not None
+        nv = max(int((y != 255).sum()), 1)
+        one = torch.ones((), device="cuda")
+        got = _native.lmargin_backward_scaled_stats(stats, 0.3, 255, one, n_valid, args)
+        want = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, np.full(shape[:1], 1.0 / nv))
+        assert np.abs(got.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
+        assert torch.equal(got, _native.lmargin_backward_scaled(xt, yt, 0.3, 255, one, n_valid))

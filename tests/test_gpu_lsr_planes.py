@@ -292,3 +292,4 @@ def test_long_rows_on_views_off_the_16_byte_boundaries(native):
     loss.backward()
     want = oracle.lsr_backward(x.astype(np.float64), y, 255, 0.1, np.full(shape[:1], 1.0 / shape[0]))
     assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+
