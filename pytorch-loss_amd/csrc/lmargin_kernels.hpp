@@ -719,12 +719,31 @@ __device__ __forceinline__ LmRowStats lm_row_sweep(const T *xs, int C, int tgt, 
         const float v[1] = {load_one(xs + j)};
         lm_row_absorb<1>(v, j, tgt, st);
     }
-    LmRowStats r;
-    r.m = row_block_reduce(st.m, lds, OpMax());
-    const float f = (st.m == -INFINITY) ? 0.f : fast_exp(st.m - r.m);
-    r.s = row_block_reduce(st.s * f, lds, OpSum());
-    r.ex = row_block_reduce(st.ex * f, lds, OpSum());
-    r.sx = row_block_reduce(st.sx, lds, OpSum());
+    // One exchange through LDS per row instead of four block-wide reductions (eight barriers): every wavefront brings
+    // its lanes to the wavefront's maximum and adds them up across lanes, leaves its four numbers in LDS, and every
+    // thread combines the wavefronts' sets itself, in a fixed order ((65536,3000) fp32 forward 0.267 -> 0.251 ms,
+    // (8192,32000) bf16 0.145 -> 0.132).
+    // lds: 4 floats per wavefront of the block.
+    const float mw = group_reduce<64>(st.m, OpMax());
+    const float f = (st.m == -INFINITY) ? 0.f : fast_exp(st.m - mw);
+    const float sw = group_reduce<64>(st.s * f, OpSum());
+    const float exw = group_reduce<64>(st.ex * f, OpSum());
+    const float sxw = group_reduce<64>(st.sx, OpSum());
+    if ((threadIdx.x & 63) == 0) {
+        float *mine = lds + 4 * (threadIdx.x >> 6);
+        mine[0] = mw; mine[1] = sw; mine[2] = exw; mine[3] = sxw;
+    }
+    __syncthreads();
+    const int waves = row_threads() / 64;
+    LmRowStats r{lds[0], 0.f, 0.f, 0.f};
+    for (int w = 1; w < waves; ++w) r.m = fmaxf(r.m, lds[4 * w]);
+    for (int w = 0; w < waves; ++w) {
+        const float fw = (lds[4 * w] == -INFINITY) ? 0.f : fast_exp(lds[4 * w] - r.m);
+        r.s = __builtin_fmaf(lds[4 * w + 1], fw, r.s);
+        r.ex = __builtin_fmaf(lds[4 * w + 2], fw, r.ex);
+        r.sx += lds[4 * w + 3];
+    }
+    __syncthreads();                    // before the next row's wavefronts write their numbers
     return r;
 }
 
@@ -741,7 +760,7 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
     constexpr bool kMayReduce = WantLoss;
     const bool Reduce = kMayReduce && part.sum != nullptr;
     const int vec = vec_flags & 1;
-    __shared__ float red[kRowBlock / 64];
+    __shared__ float red[4 * (kRowBlock / 64)];
     constexpr int L = RowChunk<T>::kLen;
     float mine = 0.f;
     int cnt = 0;
@@ -1067,7 +1086,13 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
                 // (the forward that leaves the rows' statistics has no per-row losses to write: lmargin.hip)
                 const bool keep = WantLoss && !WantGrad && p.saved != nullptr && loss == nullptr &&
                                   lm_saved_applies(sizeof(T), p.C, p.m_size);
-                hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(row_threads_for(p.C, kLmRowShortMax)), 0,
+                // short rows get small blocks (more rows in flight per CU, no idle lanes behind the barriers): forward
+                // fp32 (65536,3000) 0.249 -> 0.181 ms with 64 threads, (65536,2049) 0.214 -> 0.127, bf16 (65536,3001) 0.251 ->
+                // 0.145; the backward sweeps (65536,3000) 0.398 -> 0.349 with 128. Rows of 32000 fp32 classes and more keep 256.
+                const int64_t row_bytes = (int64_t)p.C * (int64_t)sizeof(T);
+                const int threads = WantGrad ? (row_bytes <= 12 * 1024 ? 128 : kRowBlockShort)
+                                             : (row_bytes <= 32 * 1024 ? 64 : kRowBlockShort);
+                hipLaunchKernelGGL((lm_row<T, WantLoss, WantGrad>), dim3(blocks), dim3(threads), 0,
                                    st, x, lab, up, keep ? p.saved : loss, grad, cnt, part, p,
                                    (row_chunks_ok<T>(x, WantGrad ? grad : nullptr, p.C) ? 1 : 0) | (keep ? 2 : 0));
             }

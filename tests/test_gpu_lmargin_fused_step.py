@@ -236,4 +236,5 @@ def test_rows_between_the_two_capacities_of_a_wavefront(mod):
         got = _native.lmargin_backward_scaled_stats(stats, 0.3, 255, one, n_valid, args)
         want = oracle.lmargin_backward(x.astype(np.float64), y, 0.3, 255, np.full(shape[:1], 1.0 / nv))
         assert np.abs(got.float().cpu().numpy() - want).max() <= tol * np.abs(want).max()
-        assert torch.equal(got, _native.lmargin_backward_scaled(xt, yt, 0.3, 255, one, n_valid))
+        recomputed = _native.lmargin_backward_scaled(xt, yt, 0.3, 255, one, n_valid)      # other block size, other summation order
+        assert (got.float() - recomputed.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else tol) * np.abs(want).max()
