@@ -1522,12 +1522,7 @@ constexpr int kWaveRowShort = 256;
 // barriers (bf16 LSR forward at (65536, 4096): 45 % of peak).
 template <class T>
 inline int wrow_cap(int piece) { return piece == 8 ? 2 * kWaveRowCap : kWaveRowCap; }
-// Rows that the block-per-row kernels take whatever the pointers' alignment: longer than the larger capacity, or longer
-// than the smaller one when pieces of 8 elements are out of the question (fp32, or a 16-bit row length that is no
-// multiple of 8). Where the forwards leave per-row values for an elementwise backward.
-inline bool rows_take_block_kernels(size_t elem_bytes, int64_t dimsize) {
-    return dimsize > 2 * kWaveRowCap || (dimsize > kWaveRowCap && (elem_bytes == 4 || dimsize % 8 != 0));
-}
+
 
 template <class T>
 static int wrow_piece(const T *x, const T *second, int C, const T *third = nullptr) {

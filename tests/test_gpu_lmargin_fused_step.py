@@ -215,14 +215,15 @@ def test_long_rows_module_step_and_views_off_the_16_byte_boundaries(mod):
 
 
 def test_rows_between_the_two_capacities_of_a_wavefront(mod):
-    """2049 .. 4096 classes: the block-per-row forward runs for fp32 rows and for 16-bit rows whose length is no multiple of
-    8, and only there the statistics are kept."""
+    """2049 .. 4096 classes: the forward that keeps the statistics is the block-per-row kernel for every element type (also
+    where a wavefront could hold a 16-bit row in pieces of 8)."""
     from pytorch_loss import _native
     lib = _native.load()
     assert lib.plh_lmargin_saves_stats(0, 4, 2049, 1) == 1 and lib.plh_lmargin_saves_stats(0, 4, 4096, 1) == 1
-    assert lib.plh_lmargin_saves_stats(2, 4, 3000, 1) == 0 and lib.plh_lmargin_saves_stats(2, 4, 3001, 1) == 1
+    assert lib.plh_lmargin_saves_stats(2, 4, 3000, 1) == 1 and lib.plh_lmargin_saves_stats(2, 4, 2048, 1) == 0
     for shape, dtype, tol in [((3, 2049), torch.float32, 2e-6), ((4, 3000), torch.float32, 2e-6), ((2, 4096), torch.float32, 2e-6),
-                              ((4, 3001), torch.bfloat16, 1.6e-2), ((5, 2051), torch.float16, 2e-3)]:
+                              ((4, 3001), torch.bfloat16, 1.6e-2), ((5, 2051), torch.float16, 2e-3), ((4, 3000), torch.bfloat16, 1.6e-2),
+                              ((3, 4096), torch.float16, 2e-3)]:
         x = synth.normal(341, 1, shape, 0.0, 2.0)
         y = synth.seg_labels(341, shape[:1], shape[1], 255, 0.2)
         xt = torch.from_numpy(x).cuda().to(dtype)
