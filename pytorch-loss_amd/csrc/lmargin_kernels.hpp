@@ -833,14 +833,14 @@ __global__ __launch_bounds__(kRowBlock) void lm_row(const T *__restrict__ x, con
 }
 
 // Backward of long rows from the statistics the forward left (LmParams::saved), elementwise over the flattened
-// (rows x classes) tensor like lsr_bwd_flat_lse: a block takes 1024 consecutive 16-byte chunks wherever rows begin and
+// (rows x classes) tensor like lsr_bwd_flat_lse: a block takes 512 consecutive 16-byte chunks wherever rows begin and
 // end; the arithmetic per element is lm_row's. Logits and gradient on 16-byte boundaries, one scalar upstream
 // gradient, optionally the byte mask of an OHEM selection.
 template <class T>
 __global__ __launch_bounds__(256) void lm_bwd_flat_saved(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                          const Upstream up, T *__restrict__ grad, const LmParams p,
                                                          int64_t chunks) {
-    constexpr int L = RowChunk<T>::kLen, U = 4;
+    constexpr int L = RowChunk<T>::kLen, U = kFlatChunks;
     float gk0 = up.gout ? *up.gout * up.scale : up.scale;
     if (up.divide_by) gk0 = gk0 / (float)(*up.divide_by);
     const int64_t first = (int64_t)blockIdx.x * (256 * U);
@@ -986,7 +986,7 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
     if constexpr (WantGrad && !WantLoss) {
         // long rows, from the statistics the forward left: elementwise over the flattened tensor
         constexpr int L = RowChunk<T>::kLen;
-        const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)1024);
+        const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)(256 * kFlatChunks));
         if (p.saved && !go_vec && lm_saved_applies(sizeof(T), p.C, p.m_size) && !misaligned(x, 16) && !misaligned(grad, 16) &&
             flat_blocks >= 1 && flat_blocks < ((int64_t)1 << 31)) {
             hipLaunchKernelGGL((lm_bwd_flat_saved<T>), dim3((unsigned)flat_blocks), dim3(256), 0, st, x, lab, up, grad, p,

@@ -1520,6 +1520,9 @@ constexpr int kWaveRowShort = 256;
 // 16-bit rows that move in 16-byte pieces go up to 4096 elements (8 steps of 64 lanes, 8 elements each: the
 // same 64 registers as an fp32 row of 2048); a block per row spends most of such a short row's time in its
 // barriers (bf16 LSR forward at (65536, 4096): 45 % of peak).
+// 16-byte chunks per thread of the elementwise backwards over flattened rows (lsr_bwd_flat_lse, lm_bwd_flat_saved)
+constexpr int kFlatChunks = 2;
+
 template <class T>
 inline int wrow_cap(int piece) { return piece == 8 ? 2 * kWaveRowCap : kWaveRowCap; }
 
