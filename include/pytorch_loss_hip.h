@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define PLH_ABI_VERSION 4
+#define PLH_ABI_VERSION 5
 
 #define PLH_OK 0
 #define PLH_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
@@ -457,6 +457,26 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
                            const int64_t *divide_by, void *grad_logits,
                            int64_t n_size, int64_t dimsize, int64_t m_size,
                            int64_t order, int64_t ignore_index, void *stream);
+
+/* Long (N, C) rows (m_size 1, more than 2048 classes, every dtype): the reduced forward leaves each row's S = sum_j f(x_j)
+ * (sums_out: n_size floats) and the backward forms the gradient from it elementwise over the flattened tensor instead of
+ * summing every row again (no counterpart in the reference, where autograd keeps the log-softmax output between
+ * TaylorSoftmaxFunc and F.nll_loss: pytorch_loss/taylor_softmax.py:175-198). plh_taylor_ce_saves_sums says (1 / 0)
+ * whether the sizes qualify; the other two are plh_taylor_ce_forward with loss_out (no per-row losses) and
+ * plh_taylor_ce_backward with one scalar upstream gradient, each with that one more argument, and return
+ * PLH_ERR_BAD_SIZE for sizes that do not qualify. When logits or grad_logits do not sit on 16-byte boundaries the
+ * recomputing kernel runs and `sums` is not read. */
+int plh_taylor_ce_saves_sums(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size);
+int plh_taylor_ce_forward_reduced_sums(const void *logits, int32_t dtype, const int64_t *labels,
+                                       float *sums_out, float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                       void *workspace, int64_t workspace_bytes,
+                                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                                       int64_t order, int64_t ignore_index, void *stream);
+int plh_taylor_ce_backward_scaled_sums(const void *logits, int32_t dtype, const int64_t *labels,
+                                       const float *sums, const float *grad_scalar, float scale,
+                                       const int64_t *divide_by, void *grad_logits,
+                                       int64_t n_size, int64_t dimsize, int64_t m_size,
+                                       int64_t order, int64_t ignore_index, void *stream);
 
 /* ---- soft dice loss ---------------------------------------------------------------------
  * Replaces soft_dice_cpp.soft_dice_forward / soft_dice_backward (csrc/soft_dice_kernel_v2.cu:258-436).

@@ -140,3 +140,60 @@ extern "C" int plh_taylor_ce_backward(const void *logits, int32_t dtype, const i
         make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es), (hipStream_t)stream);
     return check_launch();
 }
+
+extern "C" int plh_taylor_ce_saves_sums(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size) {
+    return dtype_ok(dtype) && n_size > 0 && dimsize > 0 && m_size > 0 &&
+                   taylor_sums_apply(dtype_size(dtype), dimsize, m_size) ? 1 : 0;
+}
+
+extern "C" int plh_taylor_ce_forward_reduced_sums(const void *logits, int32_t dtype, const int64_t *labels,
+                                                  float *sums_out, float *loss_out, int64_t *n_valid_out, int32_t mean,
+                                                  void *workspace, int64_t workspace_bytes,
+                                                  int64_t n_size, int64_t dimsize, int64_t m_size,
+                                                  int64_t order, int64_t ignore_index, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    int rc = check_order(order);
+    if (rc != PLH_OK) return rc;
+    if (n_size < 0 || m_size < 0 || n_size > kMaxNumel || m_size > kMaxNumel) return PLH_ERR_BAD_SIZE;
+    if (!taylor_sums_apply(dtype_size(dtype), dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (!loss_out) return PLH_ERR_NULL_POINTER;
+    if (!sums_out && n_size * dimsize * m_size != 0) return PLH_ERR_NULL_POINTER;
+    if (misaligned(sums_out, 4)) return PLH_ERR_MISALIGNED;
+    const size_t es = dtype_size(dtype);
+    rc = check_slice_args(logits, labels, loss_out, n_size, dimsize, m_size, es, 4);
+    if (rc != PLH_OK) return rc;
+    Partials part = kNone;
+    rc = carve_partials(workspace, workspace_bytes, n_size * m_size, loss_out, n_valid_out, part);
+    if (rc != PLH_OK) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    unsigned blocks = 0;
+    if (n_size * dimsize * m_size != 0) {
+        TaylorParams p = make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es);
+        p.sums = sums_out;
+        blocks = run(kTaylorCeFwd, dtype, logits, nullptr, labels, kUnit, nullptr, nullptr, part, p, st);
+    }
+    finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
+    return check_launch();
+}
+
+extern "C" int plh_taylor_ce_backward_scaled_sums(const void *logits, int32_t dtype, const int64_t *labels,
+                                                  const float *sums, const float *grad_scalar, float scale,
+                                                  const int64_t *divide_by, void *grad_logits,
+                                                  int64_t n_size, int64_t dimsize, int64_t m_size,
+                                                  int64_t order, int64_t ignore_index, void *stream) {
+    if (!dtype_ok(dtype)) return PLH_ERR_BAD_DTYPE;
+    int rc = check_order(order);
+    if (rc != PLH_OK) return rc;
+    if (!taylor_sums_apply(dtype_size(dtype), dimsize, m_size)) return PLH_ERR_BAD_SIZE;
+    if (n_size * dimsize * m_size != 0 && (!grad_scalar || !sums)) return PLH_ERR_NULL_POINTER;
+    if (misaligned(grad_scalar, 4) || misaligned(divide_by, 8) || misaligned(sums, 4)) return PLH_ERR_MISALIGNED;
+    const size_t es = dtype_size(dtype);
+    rc = check_slice_args(logits, labels, grad_logits, n_size, dimsize, m_size, es, es);
+    if (rc != PLH_OK) return rc;
+    if (n_size * dimsize * m_size == 0) return PLH_OK;
+    const Upstream up{grad_scalar, 0, divide_by, scale};
+    TaylorParams p = make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es);
+    p.sums = const_cast<float *>(sums);
+    run(kTaylorCeBwd, dtype, logits, nullptr, labels, up, grad_logits, nullptr, kNone, p, (hipStream_t)stream);
+    return check_launch();
+}

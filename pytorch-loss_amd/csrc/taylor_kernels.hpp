@@ -23,7 +23,16 @@ struct TaylorParams {
     int use_log;
     int64_t ignore;     // cross entropy only
     unsigned xcd_run;
+    // cross entropy of long rows: one float per row, the row's S. The reduced forward writes it beside its partial sums
+    // and the backward reads it instead of sweeping the row for it (taylor_ce_bwd_flat_sums); see taylor_sums_apply
+    float *sums = nullptr;
 };
+
+// Rows (m_size 1) beyond what a wavefront's registers hold in the backward: there the backward would read its row
+// twice (S, then the gradient), and with S kept it is one elementwise pass over the flattened tensor.
+inline bool taylor_sums_apply(size_t /*elem_bytes*/, int64_t dimsize, int64_t m_size) {
+    return m_size == 1 && dimsize > kWaveRowCap;
+}
 
 // 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and
 // its terms vanish, which the zero past the end of the table reproduces).
@@ -728,7 +737,7 @@ __global__ __launch_bounds__(256) void taylor_wrow(const T *__restrict__ x, cons
                 float f_y = 1.f, df;
                 if (has_y) taylor_pair24<ORD>(load_one(xs + lb), f_y, df);
                 const float v = has_y ? logf(s) - logf(f_y) : 0.f;
-                if (loss) loss[row] = v;
+                if (loss) loss[row] = (loss == p.sums) ? s : v;     // the slot takes the rows' S (TaylorParams::sums)
                 mine += v;
                 cnt += (lb != p.ignore) ? 1.f : 0.f;
             }
@@ -877,7 +886,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
         const int64_t lb = lab[row];
         const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
         float s = 0.f;
-        row_visit<T>(xs, p.C, vec != 0, [&](float v, int) {
+        row_visit<T>(xs, p.C, (vec & 1) != 0, [&](float v, int) {
             float f, df;
             taylor_pair(v, p.order, f, df);
             s += f;
@@ -888,7 +897,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
                 float f_y = 1.f, df;
                 if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df);
                 const float v = has_y ? logf(s) - logf(f_y) : 0.f;
-                if (loss) loss[row] = v;
+                if (loss) loss[row] = (vec & 2) ? s : v;       // bit 1: the slot takes the rows' S (TaylorParams::sums)
                 mine += v;
                 cnt += (lb != p.ignore) ? 1 : 0;
             }
@@ -901,7 +910,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
             float f_y = 1.f, df_y;
             if (has_y) taylor_pair(load_one(xs + lb), p.order, f_y, df_y);
             const float cold = inv * gk, hot = cold - gk / f_y;          // see taylor_group
-            row_map<T>(xs, out + row * p.C, p.C, vec != 0, [&](float v, int j) {
+            row_map<T>(xs, out + row * p.C, p.C, (vec & 1) != 0, [&](float v, int j) {
                 float f, df;
                 taylor_pair(v, p.order, f, df);
                 return has_y ? df * ((j == tgt) ? hot : cold) : 0.f;
@@ -912,6 +921,92 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
         if (threadIdx.x == 0) {
             part.sum[blockIdx.x] = mine;
             part.cnt[blockIdx.x] = cnt;
+        }
+    }
+}
+
+// Cross-entropy backward of long rows from the sums the forward left (TaylorParams::sums), elementwise over the
+// flattened (rows x classes) tensor: a block takes 256 * kFlatChunks consecutive 16-byte chunks wherever rows begin and
+// end, so the accesses are those of a copy; a chunk finds its row by one 32-bit division (the block's first element by
+// a 64-bit one, block-uniform), and a chunk that straddles two rows goes element by element. The target's own term
+// needs f(x_y), which the target element computes from itself. Logits and gradient on 16-byte boundaries, one scalar
+// upstream gradient, rows longer than a chunk.
+template <class T>
+__global__ __launch_bounds__(256) void taylor_ce_bwd_flat_sums(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                               const Upstream up, T *__restrict__ grad,
+                                                               const TaylorParams p, int64_t chunks) {
+    constexpr int L = RowChunk<T>::kLen, U = kFlatChunks;
+    float gk0 = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk0 = gk0 / (float)(*up.divide_by);
+    const int64_t first = (int64_t)blockIdx.x * (256 * U);
+    const int64_t row0 = first * L / p.C;                               // block-uniform
+    const unsigned col0 = (unsigned)(first * L - row0 * p.C);
+    const unsigned C = (unsigned)p.C;
+    struct RowTerms { float gk, cold; int tgt; };
+    auto row_terms = [&](int64_t r) {
+        RowTerms t;
+        const int64_t lb = lab[r];
+        const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
+        t.gk = has_y ? gk0 : 0.f;
+        t.cold = t.gk / p.sums[r];
+        t.tgt = has_y ? (int)lb : -1;
+        return t;
+    };
+    // rows without a target: exact zeros whatever the logits are (taylor_ce_row)
+    auto one = [&](float xv, int j, const RowTerms &t) {
+        float f, df;
+        taylor_pair(xv, p.order, f, df);
+        const float k = (j == t.tgt) ? t.cold - t.gk / f : t.cold;
+        return t.tgt >= 0 ? df * k : 0.f;
+    };
+    auto cold_only = [&](float xv, const RowTerms &t) {
+        float f, df;
+        taylor_pair(xv, p.order, f, df);
+        return t.tgt >= 0 ? df * t.cold : 0.f;
+    };
+    float v[U][L];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t ch = first + threadIdx.x + 256 * u;
+        live[u] = ch < chunks;
+        RowChunk<T>::load(x + (live[u] ? ch : first) * L, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (!live[u]) continue;
+        const unsigned off = col0 + (threadIdx.x + 256u * u) * L;       // from the start of row0: below 2^32 (C < 2^31)
+        const unsigned dr = off / C;
+        unsigned col = off - dr * C;
+        int64_t row = row0 + dr;
+        RowTerms t = row_terms(row);
+        if (col + L <= C) {
+            if (t.tgt >= (int)col && t.tgt < (int)(col + L)) {          // the one chunk of its row that holds the target
+#pragma unroll
+                for (int e = 0; e < L; ++e) v[u][e] = one(v[u][e], (int)(col + e), t);
+            } else {
+#pragma unroll
+                for (int e = 0; e < L; ++e) v[u][e] = cold_only(v[u][e], t);
+            }
+        } else {                                        // the chunk crosses into the next row
+#pragma unroll
+            for (int e = 0; e < L; ++e) {
+                if (col + e == C) {
+                    row += 1;
+                    col -= C;                           // wraps: col + e becomes 0 for this element
+                    t = row_terms(row);
+                }
+                v[u][e] = one(v[u][e], (int)(col + e), t);
+            }
+        }
+        RowChunk<T>::store(grad + (first + threadIdx.x + 256 * u) * L, v[u]);
+    }
+    // what is left after the last whole chunk: at most L - 1 elements of the last row
+    if (blockIdx.x == gridDim.x - 1) {
+        const int64_t at = chunks * L + threadIdx.x;
+        if (at < p.P * p.C) {
+            const RowTerms t = row_terms(p.P - 1);
+            store_one(grad + at, one(load_one(x + at), (int)(at - (p.P - 1) * p.C), t));
         }
     }
 }
@@ -929,6 +1024,17 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                                    lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true,
                                    kImageFormMaxChannels<T, (Kind == kTaylorBwd) ? 2 : 1>);
     const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
+    if constexpr (Kind == kTaylorCeBwd) {
+        // long rows, from the sums the forward left: elementwise over the flattened tensor
+        constexpr int L = RowChunk<T>::kLen;
+        const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)(256 * kFlatChunks));
+        if (p.sums && !go_vec && taylor_sums_apply(sizeof(T), p.C, p.m_size) && !misaligned(x, 16) && !misaligned(out, 16) &&
+            flat_blocks >= 1 && flat_blocks < ((int64_t)1 << 31)) {
+            hipLaunchKernelGGL((taylor_ce_bwd_flat_sums<T>), dim3((unsigned)flat_blocks), dim3(256), 0, st, x, lab, up, out,
+                               p, chunks);
+            return (unsigned)flat_blocks;
+        }
+    }
     if constexpr (kIsCe) {
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
@@ -1023,6 +1129,10 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         // cross-entropy backward with 64 registers of row ran at a third of its two-sweep form (bf16 (65536, 4096):
         // 0.782 against 0.304 ms)
         constexpr bool kForward = (Kind == kTaylorFwd || Kind == kTaylorCeFwd);
+        // (the forward that leaves the rows' sums has no per-row losses to write, so their slot serves)
+        const bool keep = Kind == kTaylorCeFwd && p.sums != nullptr && loss == nullptr &&
+                          taylor_sums_apply(sizeof(T), p.C, p.m_size);
+        float *const loss_slot = keep ? p.sums : loss;
         if (!walk && p.C <= (kForward ? wrow_cap<T>(piece) : kWaveRowCap)) {
             unsigned grid = 0;
 #define PLH_GO(NI, W, G)                                                                                          \
@@ -1031,12 +1141,12 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         if constexpr (Kind != kTaylorCeFwd && wrow_cached_form<T>(W, G)) {                                        \
             if (wrow_rows_end_inside_lines<T>(p.C)) {                                                             \
                 hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, G, true>), dim3(grid), dim3(256), 0, st, x, g, \
-                                   lab, up, out, loss, part, p);                                                  \
+                                   lab, up, out, loss_slot, part, p);                                             \
                 break;                                                                                            \
             }                                                                                                     \
         }                                                                                                         \
         hipLaunchKernelGGL((taylor_wrow<T, NI, W, Kind, G>), dim3(grid), dim3(256), 0, st, x, g, lab, up, out, \
-                           loss, part, p);                                                                        \
+                           loss_slot, part, p);                                                                   \
     } while (0)
             PLH_WROW_DISPATCH_IF(piece, p.C, PLH_GO, (kForward ? 2 : 0));
 #undef PLH_GO
@@ -1044,8 +1154,14 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         }
         const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
         if constexpr (Kind == kTaylorCeFwd || Kind == kTaylorCeBwd) {
-            hipLaunchKernelGGL((taylor_ce_row<T, Kind>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, lab, up, out, loss,
-                               part, p, row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C));
+            // short rows get small blocks in the forward (more rows in flight per CU, no idle lanes behind the barrier):
+            // fp32 (65536,3000) 0.173 -> 0.152 ms with 64 threads, (65536,2049) 0.146 -> 0.110, bf16 (65536,3001) 0.164 ->
+            // 0.104; rows of 16 KiB lose with them (fp32 (32768,4096) 0.096 -> 0.105)
+            const int threads = (Kind == kTaylorCeFwd && (int64_t)p.C * (int64_t)sizeof(T) <= 12 * 1024) ? 64 : row_threads_for_sweep<T>(p.C);
+            hipLaunchKernelGGL((taylor_ce_row<T, Kind>), dim3(grid), dim3(threads), 0, st, x, lab, up, out,
+                               loss_slot, part, p,
+                               (row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C) ? 1 : 0) |
+                                   (keep ? 2 : 0));
         } else {
             const int vec = row_chunks_ok<T>(x, out, p.C) && !(Kind == kTaylorBwd && misaligned(g, 16));
             hipLaunchKernelGGL((taylor_sm_row<T, Kind>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, g, out, p, vec);

@@ -18,7 +18,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpytorch_loss_hip.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 
@@ -80,6 +80,9 @@ _SIGNATURES = {
     "plh_taylor_softmax_backward": (ctypes.c_int, [_p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "plh_taylor_ce_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_taylor_ce_backward": (ctypes.c_int, [_p, _i32, _p, _p, _i64, _f32, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_taylor_ce_saves_sums": (ctypes.c_int, [_i32, _i64, _i64, _i64]),
+    "plh_taylor_ce_forward_reduced_sums": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p]),
+    "plh_taylor_ce_backward_scaled_sums": (ctypes.c_int, [_p, _i32, _p, _p, _p, _f32, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "plh_soft_dice_workspace_bytes": (_i64, [_i64, _i64]),
     "plh_soft_dice_forward": (ctypes.c_int, [_p, _i32, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _f32, _p]),
     "plh_soft_dice_backward": (ctypes.c_int, [_p, _p, _i32, _p, _p, _p, _i64, _i64, _f32, _p]),
@@ -761,6 +764,34 @@ def taylor_ce_forward(logits, labels, n, ignore_index, reduction, args=None):
     else:
         losses.zero_()
     return _back_to(losses, _loss_dtype(a.dtype)), None
+
+
+def taylor_ce_forward_reduced_sums(logits, labels, n, ignore_index, mean, args=None):
+    """The reduced forward that also leaves each row's sum of f for the backward, where the shape has a backward that
+    uses it (long (N, C) rows, see plh_taylor_ce_saves_sums). -> (loss, n_valid, sums or None)."""
+    _check_order(n)
+    a = args or taylor_args(logits, labels)
+    if a.x.numel() == 0 or not load().plh_taylor_ce_saves_sums(a.tag, a.n, a.c, a.m):
+        loss, n_valid = taylor_ce_forward(logits, labels, n, ignore_index, "mean" if mean else "sum", args=a)
+        return loss, n_valid, None
+    dev = a.x.device
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    n_valid = torch.empty((), dtype=torch.int64, device=dev)
+    sums = torch.empty((a.n * a.m,), dtype=torch.float32, device=dev)
+    ws, ws_bytes = _reduce_workspace(a.n * a.m, dev)
+    _call(a.x, "plh_taylor_ce_forward_reduced_sums", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(sums), _ptr(loss), _ptr(n_valid),
+          1 if mean else 0, _ptr(ws), ws_bytes, a.n, a.c, a.m, int(n), int(ignore_index))
+    return _back_to(loss, _loss_dtype(a.dtype)), n_valid, sums
+
+
+def taylor_ce_backward_scaled_sums(sums, n, ignore_index, grad_scalar, divide_by, args):
+    """The gradient from the forward's row sums (taylor_ce_forward_reduced_sums), for one scalar upstream gradient."""
+    a = args
+    grad = torch.empty_like(a.x)
+    go = _scalar_f32(grad_scalar)
+    _call(a.x, "plh_taylor_ce_backward_scaled_sums", _ptr(a.x), a.tag, _ptr(a.lb), _ptr(sums), _ptr(go), 1.0,
+          _ptr(divide_by), _ptr(grad), a.n, a.c, a.m, int(n), int(ignore_index))
+    return _back_to(grad, a.dtype)
 
 
 def taylor_ce_backward(logits, labels, n, ignore_index, grad_output, divide_by=None, args=None):

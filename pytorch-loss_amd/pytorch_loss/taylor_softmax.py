@@ -78,14 +78,23 @@ class TaylorCrossEntropyFunctionV3(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels, n, ignore_index, reduction):
         ctx.args = args = _native.taylor_args(logits, labels)
-        loss, n_valid = _native.taylor_ce_forward(logits, labels, n, ignore_index, reduction, args=args)
-        ctx.vars = (n, ignore_index, n_valid if reduction == "mean" else None)
+        sums = None
+        if reduction in ("mean", "sum") and ctx.needs_input_grad[0]:
+            # long rows: the forward leaves each row's sum for an elementwise backward
+            loss, n_valid, sums = _native.taylor_ce_forward_reduced_sums(logits, labels, n, ignore_index,
+                                                                         reduction == "mean", args=args)
+        else:
+            loss, n_valid = _native.taylor_ce_forward(logits, labels, n, ignore_index, reduction, args=args)
+        ctx.vars = (n, ignore_index, n_valid if reduction == "mean" else None, sums)
         return loss
 
     @staticmethod
     def backward(ctx, grad_output):
-        n, ignore_index, n_valid = ctx.vars
-        grad = _native.taylor_ce_backward(None, None, n, ignore_index, grad_output, n_valid, args=ctx.args)
+        n, ignore_index, n_valid, sums = ctx.vars
+        if sums is not None:
+            grad = _native.taylor_ce_backward_scaled_sums(sums, n, ignore_index, grad_output, n_valid, ctx.args)
+        else:
+            grad = _native.taylor_ce_backward(None, None, n, ignore_index, grad_output, n_valid, args=ctx.args)
         return grad, None, None, None, None
 
 

@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol(native):
         assert name in native._SIGNATURES, "binding lacks " + name
         assert len(native._SIGNATURES[name][1]) == n_args, name
     assert set(native._SIGNATURES) == set(decl)
-    assert lib.plh_abi_version() == native.ABI_VERSION == 4
+    assert lib.plh_abi_version() == native.ABI_VERSION == 5
 
 
 def test_error_strings(native):

@@ -1,0 +1,105 @@
+"""Taylor cross entropy on long (N, C) rows: the reduced forward leaves each row's sum of f
+(plh_taylor_ce_forward_reduced_sums) and the backward forms the gradient from it elementwise over the flattened tensor
+(plh_taylor_ce_backward_scaled_sums) - against the oracle and against the pair that recomputes the sum in backward."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import synth
+
+pytestmark = pytest.mark.gpu
+
+# rows whose lengths leave the 16-byte chunks of the flattened tensor straddling rows (2049, 3001, 4099), rows that do not
+# (4096), a single row, and a tensor that ends in a partial chunk (3 x 2051 elements)
+SHAPES = [(7, 2049), (5, 3001), (33, 4096), (3, 4099), (1, 5000), (3, 2051), (130, 2304)]
+DTYPES = [(torch.float32, 2e-6), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)]
+
+
+@pytest.fixture(scope="module")
+def mod():
+    import pytorch_loss
+    from pytorch_loss import _native
+    _native.load()
+    return pytorch_loss
+
+
+def inputs(seed, shape, dtype, ignore_frac=0.2):
+    x = synth.normal(seed, 1, shape, 0.0, 0.75)
+    y = synth.seg_labels(seed, shape[:1], shape[1], 255, ignore_frac)
+    xt = torch.from_numpy(x).cuda().to(dtype)
+    return xt.float().cpu().numpy().astype(np.float64), y, xt, torch.from_numpy(y).cuda()
+
+
+def test_the_predicate_names_long_rows_only(mod):
+    from pytorch_loss import _native
+    lib = _native.load()
+    for tag in (0, 1, 2):
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 2049, 1) == 1
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 2048, 1) == 0
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 4000, 2) == 0
+    assert lib.plh_taylor_ce_saves_sums(7, 8, 4000, 1) == 0
+
+
+@pytest.mark.parametrize("order", [2, 4, 6])
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("dtype,tol", DTYPES, ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=str)
+def test_step_from_row_sums_matches_the_oracle(mod, shape, dtype, tol, reduction, order):
+    from pytorch_loss import _native
+    x, y, xt, yt = inputs(401, shape, dtype)
+    n_valid = int((y != 255).sum())
+    want_loss = oracle.taylor_ce(x, y, order, 255).sum() / (n_valid if reduction == "mean" else 1)
+    factor = 3.0
+    want_grad = oracle.taylor_ce_backward(x, y, order, 255, factor / (n_valid if reduction == "mean" else 1))
+
+    # the module takes this path for a scalar loss
+    a = xt.clone().requires_grad_(True)
+    loss = mod.TaylorCrossEntropyLossV3(n=order, ignore_index=255, reduction=reduction)(a, yt)
+    (loss * factor).backward()
+    assert abs(float(loss.detach()) - want_loss) <= max(tol, 1e-5) * abs(want_loss)
+    scale = np.abs(want_grad).max()
+    assert np.abs(a.grad.float().cpu().numpy() - want_grad).max() <= tol * scale
+    ign = torch.from_numpy(y == 255).cuda().unsqueeze(1).expand_as(a.grad)
+    assert a.grad[ign].abs().max().item() == 0 if ign.any() else True
+
+    # the entry points themselves: sums are the rows' S, and the gradient equals the recomputing backward's
+    args = _native.taylor_args(xt, yt)
+    loss2, nv, sums = _native.taylor_ce_forward_reduced_sums(xt, yt, order, 255, reduction == "mean", args=args)
+    assert sums is not None and sums.shape == (shape[0],)
+    f = sum(x ** i / float(math.factorial(i)) for i in range(order + 1))
+    assert np.abs(sums.cpu().numpy() - f.sum(1)).max() <= 1e-5 * np.abs(f.sum(1)).max()
+    assert int(nv) == n_valid and torch.equal(loss2, loss.detach())
+    up = torch.full((), factor, device="cuda")
+    divide = nv if reduction == "mean" else None
+    g_sums = _native.taylor_ce_backward_scaled_sums(sums, order, 255, up, divide, args)
+    g_again = _native.taylor_ce_backward(None, None, order, 255, up, divide, args=args)
+    assert g_sums.dtype == dtype
+    assert (g_sums.float() - g_again.float()).abs().max().item() <= (2e-6 if dtype == torch.float32 else tol) * scale
+
+
+def test_views_off_the_16_byte_grid_take_the_recomputing_backward(mod):
+    """Logits that start 4 bytes into a 16-byte chunk: the sums are written but the backward sweeps its rows again."""
+    shape = (6, 2500)
+    x, y, xt, yt = inputs(402, shape, torch.float32)
+    base = torch.zeros(shape[0] * shape[1] + 1, device="cuda")
+    view = base[1:].view(shape)
+    view.copy_(xt)
+    a = view.detach().requires_grad_(True)
+    assert a.data_ptr() % 16 == 4
+    loss = mod.TaylorCrossEntropyLossV3(n=4, ignore_index=255)(a, yt)
+    loss.backward()
+    n_valid = int((y != 255).sum())
+    want = oracle.taylor_ce_backward(x, y, 4, 255, 1.0 / n_valid)
+    assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+
+
+def test_rows_without_any_valid_label(mod):
+    shape = (4, 3000)
+    x, y, xt, yt = inputs(403, shape, torch.float32, ignore_frac=1.0)
+    a = xt.clone().requires_grad_(True)
+    loss = mod.TaylorCrossEntropyLossV3(n=2, ignore_index=255, reduction="sum")(a, yt)
+    loss.backward()
+    assert float(loss.detach()) == 0.0 and a.grad.abs().max().item() == 0.0
