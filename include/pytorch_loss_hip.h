@@ -243,7 +243,9 @@ int plh_lmargin_forward_backward_reduced(const void *logits, int32_t dtype, cons
                                          int64_t n_size, int64_t dimsize, int64_t m_size,
                                          int64_t ignore_index, float lam, void *stream);
 
-/* Long (N, C) rows (m_size 1, more than 2048 classes, every dtype): the forward leaves eight floats of statistics per row
+/* (N, C) rows (m_size 1) of more than 2048 classes, and shorter ones of more than 32 wherever the elementwise backward is
+ * the faster one (16-bit logits: all of them; fp32: a class count that is no multiple of 32, or below 96, or above 1536):
+ * the forward leaves eight floats of statistics per row
  * (stats_out: n_size * 8 floats on a 16-byte boundary) and the backward forms the gradient from them elementwise over the
  * flattened tensor instead of sweeping every row for them again (no counterpart in the reference, whose backward
  * recomputes: csrc/large_margin_kernel.cu:387-599). plh_lmargin_saves_stats says (1 / 0) whether the sizes qualify;

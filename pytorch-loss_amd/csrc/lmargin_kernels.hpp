@@ -34,18 +34,23 @@ struct LmParams {
     uint8_t *early_kept = nullptr;
     int *early_below = nullptr;
     float early_thresh = 0.f;
-    // (N, C) rows of more than kWaveRowCap classes (the block-per-row forward's): kLmSavedFloats floats per row that the forward leaves (lm_row)
+    // (N, C) rows of more than 32 classes: kLmSavedFloats floats per row that the forward leaves (lm_wrow, lm_row)
     // and the backward reads instead of sweeping the row for them (lm_bwd_flat_saved); see lm_saved_applies
     float *saved = nullptr;
 };
 
-// What the block-per-row forward leaves per row for the elementwise backward: the maximum m over the classes other than
+// What the forward of (N, C) rows leaves per row for the elementwise backward: the maximum m over the classes other than
 // the target, 1 / sum exp(x - m) over them, t_all / s_all (which turns exp(x - m) into the full softmax), sum q x, and
 // the target's p_y - 1; padded to 32 bytes.
 constexpr int kLmSavedFloats = 8;
 inline bool lm_saved_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    (void)elem_bytes;       // every element type: the large-margin forward of such rows is the block-per-row kernel
-    return m_size == 1 && dimsize > kWaveRowCap;
+    if (m_size != 1 || dimsize <= kMaxRegsChannels) return false;
+    if (dimsize > kWaveRowCap) return true;     // the block-per-row forward's rows: every element type
+    // Rows that a wavefront holds in registers: the elementwise backward runs at 67-82 % of the HBM peak whatever the row
+    // length; the backward that recomputes reaches 74-87 % on fp32 rows of a multiple of 32 classes between 96 and 1536
+    // and 17-70 % elsewhere (fp32 (262144,300) 0.125 against 0.105 ms), on 16-bit rows 73-75 % at 256, 512 and 1024
+    // classes (against 68-70 %) and 17-69 % elsewhere (bf16 (65536,1100) 0.128 against 0.052 ms)
+    return elem_bytes != 4 || dimsize % 32 != 0 || dimsize < 96 || dimsize > 1536;
 }
 
 // ---------------------------------------------------------------- regs ----
@@ -604,7 +609,19 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             acc = p.half_lam * (sum_ex * inv_no - lse_no - p.coeff * (sum_d - n_no * lse_no));
             if (!closed) acc = 0.f;
         }
-        if (!closed) {
+        if constexpr (kClosed) {
+            // (read again from memory, one element per lane and step: with the registers' values the compiler keeps the
+            // exponentials of the sweep above alive for this path, and the registers that costs the common path up to half
+            // its speed - fp32 (65536,1100) forward 0.086 -> 0.055 ms without it)
+            if (!closed) {
+#pragma nounroll
+                for (int j = lane; j < p.C; j += G) {
+                    const float xv = load_one(xs + j);
+                    const float q = fast_exp(xv - m_no) * inv_no;
+                    acc += (j == tgt) ? 0.f : p.half_lam * (q - p.coeff) * ((xv - m_no) - lse_no);
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int e0 = (lane + G * i) * L;
@@ -639,7 +656,15 @@ __global__ __launch_bounds__(256) void lm_wrow(const T *__restrict__ x, const in
             if (!closed) acc = group_reduce<G>(acc, OpSum());
             acc += -(x_y - m_all) + logf(s_all);
             if (lane == 0 && live) {
-                if (loss) loss[row] = ign ? 0.f : acc;
+                if (loss) {
+                    if (kClosed && loss == p.saved) {       // the slot takes the row's statistics (LmParams::saved)
+                        plh_f4 *to = reinterpret_cast<plh_f4 *>(loss + row * kLmSavedFloats);
+                        to[0] = plh_f4{m_no, inv_no, t_all * inv_all, sum_qx + m_no};     // here sum_qx is sum q (x - m_no)
+                        to[1] = plh_f4{e_y * inv_all - 1.f, 0.f, 0.f, 0.f};
+                    } else {
+                        loss[row] = ign ? 0.f : acc;
+                    }
+                }
                 if (p.scores) p.scores[row] = (ign || tgt < 0) ? p.no_target_score : fminf(e_y * inv_all, 1.f);
                 mine += ign ? 0.f : acc;
                 cnt += ign ? 0.f : 1.f;
@@ -1076,6 +1101,9 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
             // (16-bit rows of 2049 .. 4096 classes: the forward goes to the block-per-row kernel even where a wavefront
             // could hold the row in pieces of 8 - bf16 (65536,3000) forward 0.169 -> 0.145 ms - and leaves the row
             // statistics for the elementwise backward, 0.211 -> 0.144 ms)
+            float *loss_w;
+            loss_w = (WantLoss && !WantGrad && p.saved != nullptr && loss == nullptr &&
+                      lm_saved_applies(sizeof(T), p.C, p.m_size)) ? p.saved : loss;
             if (p.C <= wrow_cap<T>(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C)) &&
                 !(WantLoss && !WantGrad && sizeof(T) == 2 && p.C > kWaveRowCap)) {
 #define PLH_GO(NI, W, G)                                                                                           \
@@ -1084,12 +1112,12 @@ unsigned launch_typed(const T *x, const int64_t *lab, const Upstream &up, float 
         if constexpr (WantGrad && wrow_cached_form<T>(W, G)) {                                                     \
             if (wrow_rows_end_inside_lines<T>(p.C)) {                                                              \
                 hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, G, true>), dim3(blocks), \
-                                   dim3(256), 0, st, x, lab, up, loss, grad, cnt, part, p);                        \
+                                   dim3(256), 0, st, x, lab, up, loss_w, grad, cnt, part, p);                        \
                 break;                                                                                             \
             }                                                                                                      \
         }                                                                                                          \
         hipLaunchKernelGGL((lm_wrow<T, NI, W, WantLoss, WantGrad, G>), dim3(blocks), dim3(256), 0, \
-                           st, x, lab, up, loss, grad, cnt, part, p);                                              \
+                           st, x, lab, up, loss_w, grad, cnt, part, p);                                              \
     } while (0)
                 PLH_WROW_DISPATCH_IF(wrow_piece<T>(x, WantGrad ? grad : nullptr, p.C), p.C, PLH_GO, (WantGrad ? 1 : 2));
 #undef PLH_GO

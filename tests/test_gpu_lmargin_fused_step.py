@@ -150,19 +150,33 @@ def test_the_entry_point_on_fp16_logits(mod, shape):
     assert np.abs(grad.float().cpu().numpy() - want_grad).max() <= 2e-3 * np.abs(want_grad).max()
 
 
-# (N, C) rows of more than 4096 classes: the forward leaves eight floats of statistics per row and the backward is
-# elementwise over the flattened tensor (row ends inside 16-byte chunks, a last chunk that is not whole, one row only)
-LONG_ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100)]
+# (N, C) rows: the forward leaves eight floats of statistics per row and the backward is elementwise over the flattened
+# tensor (row ends inside 16-byte chunks, a last chunk that is not whole, one row only); the rows of up to 2048 classes are
+# the ones that a wavefront holds in registers in the forward (several rows per wavefront up to 512 classes)
+LONG_ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100),
+             (300, 33), (130, 48), (40, 64), (70, 200), (260, 300), (17, 1000), (9, 1100), (6, 2040), (1, 77)]
+ROWS_16BIT_ONLY = [(20, 256), (9, 1024), (5, 2048)]
 
 
 @pytest.mark.parametrize("dtype,tol", DTYPES, ids=["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape", LONG_ROWS, ids=str)
 def test_long_rows_backward_from_the_forwards_statistics(mod, shape, dtype, tol):
+    check_backward_from_statistics(shape, dtype, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", DTYPES[1:], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", ROWS_16BIT_ONLY, ids=str)
+def test_16_bit_rows_of_a_power_of_two_take_the_statistics_too(mod, shape, dtype, tol):
+    check_backward_from_statistics(shape, dtype, tol)
+
+
+def check_backward_from_statistics(shape, dtype, tol):
     from pytorch_loss import _native
     lib = _native.load()
     tag = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
     assert lib.plh_lmargin_saves_stats(tag, shape[0], shape[1], 1) == 1
-    assert lib.plh_lmargin_saves_stats(tag, shape[0], 2048, 1) == 0 and lib.plh_lmargin_saves_stats(tag, 2, 5000, 4) == 0
+    assert lib.plh_lmargin_saves_stats(tag, shape[0], 512, 1) == (0 if tag == 0 else 1) and lib.plh_lmargin_saves_stats(tag, 2, 5000, 4) == 0
+    assert lib.plh_lmargin_saves_stats(tag, shape[0], 32, 1) == 0
     x = synth.normal(331, 1, shape, 0.0, 2.0)
     y = synth.seg_labels(331, shape[:1], shape[1], 255, 0.2)
     if shape[0] > 2:
@@ -220,7 +234,7 @@ def test_rows_between_the_two_capacities_of_a_wavefront(mod):
     from pytorch_loss import _native
     lib = _native.load()
     assert lib.plh_lmargin_saves_stats(0, 4, 2049, 1) == 1 and lib.plh_lmargin_saves_stats(0, 4, 4096, 1) == 1
-    assert lib.plh_lmargin_saves_stats(2, 4, 3000, 1) == 1 and lib.plh_lmargin_saves_stats(2, 4, 2048, 1) == 0
+    assert lib.plh_lmargin_saves_stats(2, 4, 3000, 1) == 1 and lib.plh_lmargin_saves_stats(2, 4, 2048, 1) == 1
     for shape, dtype, tol in [((3, 2049), torch.float32, 2e-6), ((4, 3000), torch.float32, 2e-6), ((2, 4096), torch.float32, 2e-6),
                               ((4, 3001), torch.bfloat16, 1.6e-2), ((5, 2051), torch.float16, 2e-3), ((4, 3000), torch.bfloat16, 1.6e-2),
                               ((3, 4096), torch.float16, 2e-3)]:
