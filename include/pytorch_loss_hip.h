@@ -118,8 +118,10 @@ int plh_lsr_forward_backward_reduced(const void *logits, int32_t dtype, const in
  * backward recomputes the softmax, csrc/lsr_kernel.cu:139-225). plh_lsr_saves_lse says (1 / 0) whether it applies to
  * these sizes: fp32 logits and channel planes of at least 4096 pixels, with either a plane byte length that is no
  * multiple of 128 and dimsize up to 24 or from 33 (25..32 keep their kernels), or dimsize above 256 on any plane;
- * and, for every dtype, (N, C) rows (m_size 1) of more than 4096 classes, where the backward becomes elementwise over
- * the flattened tensor (bf16 (8192,32000): forward + backward 0.357 -> 0.286 ms).
+ * and (N, C) rows (m_size 1) of more than 32 classes, where the backward becomes elementwise over the flattened tensor
+ * (bf16 (8192,32000): forward + backward 0.357 -> 0.275 ms), wherever that is the faster one: fp32 rows except those of a
+ * multiple of 32 classes from 96 to 768 and those of 2049..4096 classes; 16-bit rows of more than 1024 classes, and of a
+ * multiple of 8 classes up to 96.
  * Then plh_lsr_forward_reduced_lse is plh_lsr_forward_reduced that also leaves every pixel's
  * log-sum-exp in lse_out (n_size*m_size floats; it writes no per-pixel losses), and plh_lsr_backward_scaled_lse is
  * plh_lsr_backward_scaled that forms the gradient from it, sumw*exp(x - lse) - w, plane by plane in each plane's own
@@ -460,7 +462,9 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
                            int64_t n_size, int64_t dimsize, int64_t m_size,
                            int64_t order, int64_t ignore_index, void *stream);
 
-/* Long (N, C) rows (m_size 1, more than 2048 classes, every dtype): the reduced forward leaves each row's S = sum_j f(x_j)
+/* (N, C) rows (m_size 1) of more than 32 classes wherever the elementwise backward is the faster one (fp32 rows except
+ * those of a multiple of 32 classes from 96 to 768; 16-bit rows of more than 2048 classes, and of a multiple of 8 classes
+ * up to 96): the reduced forward leaves each row's S = sum_j f(x_j)
  * (sums_out: n_size floats) and the backward forms the gradient from it elementwise over the flattened tensor instead of
  * summing every row again (no counterpart in the reference, where autograd keeps the log-softmax output between
  * TaylorSoftmaxFunc and F.nll_loss: pytorch_loss/taylor_softmax.py:175-198). plh_taylor_ce_saves_sums says (1 / 0)

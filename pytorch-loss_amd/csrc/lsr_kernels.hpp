@@ -317,12 +317,16 @@ __global__ __launch_bounds__(256) void lsr_bwd_planes(const T *__restrict__ x, c
 // fp32 logits only: with 16-bit logits (8 elements per lane, 64 per line) the pair measured no gain - bf16
 // (16,19,769,769): forward 0.0815 -> 0.0963 ms with the extra output, backward 0.180 -> 0.160 ms, bound by its
 // conversions.
-// (N, C) rows, any element type: rows of more than 4096 classes, which the block-per-row forward takes whatever the
-// pointers' alignment (lsr_fwd_row leaves one value per row); the backward from it (lsr_bwd_flat_lse) needs no
-// reduction. (Rows of 2049 .. 4096 classes that the same forward takes gain nothing: fp32 (65536,4096) forward +
-// backward 0.511 ms recomputing - the row stays in the block's registers - against 0.555 ms, (65536,3000) 0.433 / 0.424.)
+// (N, C) rows of more than 32 classes, any element type: the forward leaves one value per row (lsr_fwd_wrow, lsr_fwd_row)
+// and the backward from it (lsr_bwd_flat_lse) needs no reduction and no row in registers; which rows take it:
+// row_backward_is_elementwise.
 inline bool lsr_lse_applies(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    if (m_size == 1) return dimsize > 2 * kWaveRowCap;
+    if (m_size == 1) {
+        // (fp32 rows of 2049 .. 4096 classes stay with the backward that keeps the row in the block's registers:
+        // (32768,4096) forward + backward 0.255 ms against 0.272)
+        if (elem_bytes == 4 && dimsize > kWaveRowCap && dimsize <= 2 * kWaveRowCap) return false;
+        return row_backward_is_elementwise(elem_bytes, dimsize, 1024);
+    }
     if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
     const bool off_lines = (m_size * (int64_t)elem_bytes) % 128 != 0;
     if (dimsize <= kMaxRegsChannels) return off_lines && image_form_pays<float>((int)dimsize, m_size);
@@ -764,7 +768,7 @@ __global__ __launch_bounds__(256) void lsr_fwd_wrow(const T *__restrict__ x, con
             const float all = d - fc * lse;
             const float hot = has_y ? (p.w_pos - p.w_neg) * ((x_y - mx) - lse) : 0.f;
             const float acc = ign ? 0.f : -(p.w_neg * all + hot);
-            if (loss) loss[row] = acc;
+            if (loss) loss[row] = (loss == p.lse) ? mx + lse : acc;       // the slot takes the row's log-sum-exp (LsrParams::lse)
             mine += acc;
             cnt += ign ? 0.f : 1.f;
         }
@@ -1093,17 +1097,20 @@ __global__ __launch_bounds__(256) void lsr_bwd_flat_lse(const T *__restrict__ x,
                                                ((int)(col + e) == tgt) ? n_pos : n_neg);
                 v[u][e] = dropped ? 0.f : g;            // ignored rows: exact zeros whatever the logits are
             }
-        } else {                                        // the chunk crosses into the next row
+        } else {                                        // the chunk crosses into the next row: both rows' terms, chosen per element
+            float shift2, scale2, n_pos2, n_neg2;
+            int tgt2;
+            bool dropped2;
+            row_terms(row + 1, shift2, scale2, n_pos2, n_neg2, tgt2, dropped2);
+            tgt2 = tgt2 < 0 ? -1 : tgt2 + (int)C;       // in the first row's column numbers
 #pragma unroll
             for (int e = 0; e < L; ++e) {
-                if (col + e == C) {
-                    row += 1;
-                    col -= C;                           // wraps: col + e becomes 0 for this element
-                    row_terms(row, shift, scale, n_pos, n_neg, tgt, dropped);
-                }
-                const float g = __builtin_fmaf(__builtin_amdgcn_exp2f(__builtin_fmaf(v[u][e], kLog2e, shift)), scale,
-                                               ((int)(col + e) == tgt) ? n_pos : n_neg);
-                v[u][e] = dropped ? 0.f : g;
+                const bool next = col + e >= C;
+                const int t = next ? tgt2 : tgt;
+                const float g = __builtin_fmaf(__builtin_amdgcn_exp2f(__builtin_fmaf(v[u][e], kLog2e, next ? shift2 : shift)),
+                                               next ? scale2 : scale,
+                                               ((int)(col + e) == t) ? (next ? n_pos2 : n_pos) : (next ? n_neg2 : n_neg));
+                v[u][e] = (next ? dropped2 : dropped) ? 0.f : g;
             }
         }
         RowChunk<T>::store(grad + ch * L, v[u]);
@@ -1367,9 +1374,11 @@ static unsigned forward_shape(const T *logits, const int64_t *labels, float *los
 #define PLH_GO(NI, W, G)                                                                                            \
     do {                                                                                                            \
         grid = group_grid(p.P, WaveRowAt<G>::kRowsPerBlock);                                                        \
-        hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, G>), dim3(grid), dim3(256), 0, st, logits, labels, losses, \
+        hipLaunchKernelGGL((lsr_fwd_wrow<T, NI, W, G>), dim3(grid), dim3(256), 0, st, logits, labels, slot_w, \
                            part, p);                                                                                \
     } while (0)
+            float *slot_w;
+            slot_w = (p.lse != nullptr && losses == nullptr && lsr_lse_applies(sizeof(T), p.C, p.m_size)) ? p.lse : losses;
             PLH_WROW_DISPATCH(piece, p.C, PLH_GO);
 #undef PLH_GO
             return grid;
@@ -1408,9 +1417,12 @@ void lsr_backward_typed(const T *logits, const int64_t *labels, const Upstream &
                                grad_logits, p, chunks);
             return;
         }
-        const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
-        hipLaunchKernelGGL((lsr_bwd_row_lse<T>), dim3(grid), dim3(kRowBlockShort), 0, st, logits, labels, up, grad_logits, p, 0);
-        return;
+        if (p.C > 2 * kWaveRowCap) {
+            const unsigned grid = (unsigned)(p.P < kMinPartialSlots ? p.P : kMinPartialSlots);
+            hipLaunchKernelGGL((lsr_bwd_row_lse<T>), dim3(grid), dim3(kRowBlockShort), 0, st, logits, labels, up, grad_logits, p, 0);
+            return;
+        }
+        // (shorter rows off the 16-byte boundaries: the kernels below, which recompute)
     }
     if constexpr (sizeof(T) == 4) {
         // from the forward's log-sum-exp, plane by plane: one scalar upstream gradient, logits and gradient at the same

@@ -28,10 +28,10 @@ struct TaylorParams {
     float *sums = nullptr;
 };
 
-// Rows (m_size 1) beyond what a wavefront's registers hold in the backward: there the backward would read its row
-// twice (S, then the gradient), and with S kept it is one elementwise pass over the flattened tensor.
-inline bool taylor_sums_apply(size_t /*elem_bytes*/, int64_t dimsize, int64_t m_size) {
-    return m_size == 1 && dimsize > kWaveRowCap;
+// Rows (m_size 1) whose backward is one elementwise pass over the flattened tensor with S kept (beyond what a wavefront's
+// registers hold the other backward reads its row twice, S and then the gradient): row_backward_is_elementwise.
+inline bool taylor_sums_apply(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
+    return m_size == 1 && row_backward_is_elementwise(elem_bytes, dimsize, kWaveRowCap);
 }
 
 // 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and
@@ -988,15 +988,17 @@ __global__ __launch_bounds__(256) void taylor_ce_bwd_flat_sums(const T *__restri
 #pragma unroll
                 for (int e = 0; e < L; ++e) v[u][e] = cold_only(v[u][e], t);
             }
-        } else {                                        // the chunk crosses into the next row
+        } else {                                        // the chunk crosses into the next row: both rows' terms, chosen per element
+            RowTerms t2 = row_terms(row + 1);
+            t2.tgt = t2.tgt < 0 ? -1 : t2.tgt + (int)C;     // in the first row's column numbers
 #pragma unroll
             for (int e = 0; e < L; ++e) {
-                if (col + e == C) {
-                    row += 1;
-                    col -= C;                           // wraps: col + e becomes 0 for this element
-                    t = row_terms(row);
-                }
-                v[u][e] = one(v[u][e], (int)(col + e), t);
+                const bool next = col + e >= C;
+                RowTerms te;
+                te.gk = next ? t2.gk : t.gk;
+                te.cold = next ? t2.cold : t.cold;
+                te.tgt = next ? t2.tgt : t.tgt;
+                v[u][e] = one(v[u][e], (int)(col + e), te);
             }
         }
         RowChunk<T>::store(grad + (first + threadIdx.x + 256 * u) * L, v[u]);

@@ -236,17 +236,41 @@ def lib_saves(native, shape):
     return native.load().plh_lsr_saves_lse(0, shape[0], shape[1], shape[2] * shape[3]) == 1
 
 
-# (N, C) rows longer than 4096 classes: the block-per-row forward leaves one log-sum-exp per row and the backward is
-# elementwise over the flattened tensor (row ends inside 16-byte chunks, a last chunk that is not whole, one row only)
-ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100)]
+# (N, C) rows: the forward leaves one log-sum-exp per row and the backward is elementwise over the flattened tensor (row
+# ends inside 16-byte chunks, a last chunk that is not whole, one row only); the first six are the block-per-row forward's,
+# the next ones rows that a wavefront holds in registers (several rows per wavefront among them), the last ones those of
+# them that qualify only with fp32 logits
+ROWS = [(5, 5000), (3, 4099), (7, 6001), (1, 4097), (2, 8192), (33, 4100),
+        (300, 40), (130, 48), (40, 64), (9, 1100), (6, 2040), (5, 2048), (17, 1032)]
+ROWS_16BIT_ONLY = [(4, 3000), (3, 4096), (5, 2051)]
+ROWS_FP32_ONLY = [(70, 200), (260, 300), (17, 1000), (1, 77), (9, 1024), (300, 33), (50, 100)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)], ids=["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape", ROWS, ids=str)
 def test_long_rows(native, shape, dtype, tol):
+    check_rows_from_lse(native, shape, dtype, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)], ids=["f16", "bf16"])
+@pytest.mark.parametrize("shape", ROWS_16BIT_ONLY, ids=str)
+def test_rows_that_qualify_with_16_bit_logits_only(native, shape, dtype, tol):
+    assert native.load().plh_lsr_saves_lse(0, shape[0], shape[1], 1) == 0
+    check_rows_from_lse(native, shape, dtype, tol)
+
+
+@pytest.mark.parametrize("shape", ROWS_FP32_ONLY, ids=str)
+def test_rows_that_qualify_with_fp32_logits_only(native, shape):
+    lib = native.load()
+    assert lib.plh_lsr_saves_lse(1, shape[0], shape[1], 1) == 0 and lib.plh_lsr_saves_lse(2, shape[0], shape[1], 1) == 0
+    check_rows_from_lse(native, shape, torch.float32, 2e-6)
+
+
+def check_rows_from_lse(native, shape, dtype, tol):
     lib = native.load()
     tag = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
-    assert lib.plh_lsr_saves_lse(tag, shape[0], shape[1], 1) == 1 and lib.plh_lsr_saves_lse(tag, shape[0], 4096, 1) == 0
+    assert lib.plh_lsr_saves_lse(tag, shape[0], shape[1], 1) == 1 and lib.plh_lsr_saves_lse(tag, shape[0], 512, 1) == 0
+    assert lib.plh_lsr_saves_lse(tag, shape[0], 32, 1) == 0
     x = synth.normal(161, 1, shape, 0.0, 2.0)
     y = synth.seg_labels(161, shape[:1], shape[1], 255, 0.2)
     y[::3] = shape[1] + 7 if shape[0] > 2 else y[::3]           # rows without a target class, not ignored
