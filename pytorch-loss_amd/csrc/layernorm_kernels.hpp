@@ -12,6 +12,7 @@
 // runs one pixel per lane; anything larger, and m_size == 1 (rows contiguous), takes a two-sweep
 // kernel whose second sweep is served by cache.
 #pragma once
+#include <type_traits>
 #include "plh_common.hpp"
 
 namespace plh {
@@ -277,14 +278,29 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
     // planes that start on element boundaries only (odd lengths, misaligned tensors) and are long enough that
     // the partly filled last group of every image is a small share: the same pixels per lane in groups per image
     const bool image = !vec && dimsize <= 768 && m_size >= 4096;
-    const int64_t groups = image ? n_size * ceil_div(m_size, 64 * VT) : ceil_div(p.P, 64 * (vec ? VT : 1));
-    const unsigned grid = (unsigned)(ws > 1 ? groups : ceil_div(groups, 4));
     const int slots = p.per_wave;
+    // 16-bit elements, more than 48 slots per wave: 64 and 96 slots of four pixels are 256 and 384 values per lane, and
+    // where the kernel spills them (up to 1168 bytes per lane: the per-image form, and fp16 with 96 slots) two pixels per
+    // lane are faster: fp16 (32,768,4098) forward 0.565 -> 0.174 ms, backward 0.739 -> 0.271; (32,768,4096) 0.109 -> 0.092
+    // and 0.180 -> 0.172. (bf16 on aligned planes keeps four: 0.129 against 0.192 ms backward at (32,768,4096).)
+    constexpr int VN = (sizeof(T) == 2) ? 2 : VT;
+    const bool narrow = sizeof(T) == 2 && ws == 8 && slots > 48 && slots <= 96 &&
+                        (image || (vec && std::is_same<T, f16>::value && slots > 64));
+    const int vv = narrow ? VN : VT;
+    const int64_t groups = image ? n_size * ceil_div(m_size, 64 * vv) : ceil_div(p.P, 64 * (vec ? vv : 1));
+    const unsigned grid = (unsigned)(ws > 1 ? groups : ceil_div(groups, 4));
 #define PLH_LN(KW, VV, WS) \
     hipLaunchKernelGGL((ln_regs<T, KW, VV, WS, Bwd>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
 #define PLH_LN_IMAGE(KW, WS) \
     hipLaunchKernelGGL((ln_regs<T, KW, VT, WS, Bwd, true>), dim3(grid), dim3(WS > 4 ? 64 * WS : kLnBlock), 0, st, x, g, out, p)
 #define PLH_LN_V(KW, WS) do { if (vec) PLH_LN(KW, VT, WS); else if (image) PLH_LN_IMAGE(KW, WS); else PLH_LN(KW, 1, WS); } while (0)
+#define PLH_LN_NARROW(KW, WS)                                                                                              \
+    do {                                                                                                                   \
+        if (vec) PLH_LN(KW, VN, WS);                                                                                       \
+        else if (image)                                                                                                    \
+            hipLaunchKernelGGL((ln_regs<T, KW, VN, WS, Bwd, true>), dim3(grid), dim3(64 * WS), 0, st, x, g, out, p);       \
+        else PLH_LN(KW, 1, WS);                                                                                            \
+    } while (0)
     // Slot counts in steps of about 1.5x: a wave whose channels fall short of its slots re-reads its last
     // channel for the rest, and at 12 channels in 16 slots that cost a third of the bandwidth.
     if (ws == 1) {
@@ -301,9 +317,10 @@ void ln_launch(const T *x, const T *g, T *out, int64_t n_size, int64_t dimsize, 
     else if (slots <= 24) PLH_LN_V(24, 8);
     else if (slots <= 32) PLH_LN_V(32, 8);
     else if (slots <= 48) PLH_LN_V(48, 8);
-    else if (slots <= 64) PLH_LN_V(64, 8);
-    else if (slots <= 96) PLH_LN_V(96, 8);             // C <= 768
+    else if (slots <= 64) { if (narrow) PLH_LN_NARROW(64, 8); else PLH_LN_V(64, 8); }
+    else if (slots <= 96) { if (narrow) PLH_LN_NARROW(96, 8); else PLH_LN_V(96, 8); }      // C <= 768
     else PLH_LN(128, 1, 8);                            // 768 < C <= 1024: one pixel per lane
+#undef PLH_LN_NARROW
 #undef PLH_LN_V
 #undef PLH_LN_IMAGE
 #undef PLH_LN

@@ -981,8 +981,10 @@ template <class T> __device__ __forceinline__ void chunk_widen(const plh_u4 &t, 
     }
 }
 
+// (16 chunks per thread are launched with 256 threads only: bounds of 1024 would cap the kernel at 128 registers, and it
+// spilled 64 of its row's values to scratch memory under them)
 template <class T, int NCH>
-__global__ __launch_bounds__(kRowBlock) void lsr_bwd_rowregs(const T *__restrict__ x, const int64_t *__restrict__ lab,
+__global__ __launch_bounds__(NCH == 16 ? kRowBlockShort : kRowBlock) void lsr_bwd_rowregs(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                             const Upstream up, T *__restrict__ grad, const LsrParams p) {
     __shared__ float red[kRowBlock / 64];
     constexpr int L = RowChunk<T>::kLen;

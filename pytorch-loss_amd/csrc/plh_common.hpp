@@ -365,6 +365,7 @@ __device__ __forceinline__ float widen_hi(unsigned d, f16) {
 }
 
 typedef unsigned plh_u2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+typedef unsigned plh_u1_a2 __attribute__((aligned(2)));
 template <class T> struct Pack<T, 4> {          // T = f16 or bf16
     typedef plh_u2 Raw;
     static __device__ __forceinline__ Raw load(const T *p) {
@@ -407,6 +408,13 @@ template <class T> struct Pack<T, 2> {          // T = f16 or bf16: one dword, t
     }
     static __device__ __forceinline__ void store(T *p, Raw r) {
         __builtin_nontemporal_store(r, reinterpret_cast<unsigned *>(p));
+    }
+    // the same 4 bytes from any element boundary (the per-image form on channel planes of odd length)
+    static __device__ __forceinline__ Raw load_unaligned(const T *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const plh_u1_a2 *>(p));
+    }
+    static __device__ __forceinline__ void store_unaligned(T *p, Raw r) {
+        __builtin_nontemporal_store((plh_u1_a2)r, reinterpret_cast<plh_u1_a2 *>(p));
     }
     static __device__ __forceinline__ float get(Raw r, int k) { return (k & 1) ? widen_hi(r, T{}) : widen_lo(r, T{}); }
     static __device__ __forceinline__ Raw put(const float (&g)[2]) { return narrow2(g[0], g[1], T{}); }

@@ -102,7 +102,10 @@ def test_module_on_nchw(pl, affine):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(2, 19, 64), (1, 96, 260), (1, 256, 128), (1, 600, 66), (4, 80, 1), (2, 30, 7)])
+# (the last four: 385..768 channels in the forms that hold two pixels per lane - planes of 4096 pixels and more that are
+# not whole groups of four pixels, in groups per image, and fp16 with more than 512 channels on aligned planes)
+@pytest.mark.parametrize("shape", [(2, 19, 64), (1, 96, 260), (1, 256, 128), (1, 600, 66), (4, 80, 1), (2, 30, 7),
+                                   (1, 600, 4098), (2, 448, 4102), (1, 768, 4097), (1, 640, 256)])
 def test_16bit(pl, dt, shape):
     ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dt]
     x = synth.normal(124, 1, shape, 0.3, 1.5)
