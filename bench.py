@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|focal_seg|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|lsr_vocab|lmargin_vocab|lmargin_rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|focal_seg|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|lsr_vocab|lmargin_vocab|taylor_vocab|lmargin_rows]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -86,6 +86,8 @@ WORKLOADS = {
                       "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lmargin_vocab": dict(base="lmargin", shape=(8192, 32000), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (8192,32000), "
                           "int64 labels 5% ignore=255, lam=0.3, mean"),
+    "taylor_vocab": dict(base="taylor", shape=(8192, 32000), desc="TaylorCrossEntropyLossV3 fwd+bwd, fp32 logits (8192,32000), "
+                         "int64 labels 5% ignore=255, n=4, mean"),
     # classifier-sized rows: a wavefront holds a row in its registers
     "lmargin_rows": dict(base="lmargin", shape=(65536, 1000), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (65536,1000), "
                          "int64 labels 5% ignore=255, lam=0.3, mean"),
@@ -470,6 +472,22 @@ def kernel_rooflines(name, logits, labels, dtype="f32"):
         assert fs() == 0 and bs() == 0
         eb = ELEM_BYTES[dtype]
         legs += [("forward_keeping_stats", fs, eb * E + 8 * Pn + 32 * Pn), ("backward_from_stats", bs, 2 * eb * E + 8 * Pn + 32 * Pn)]
+    if name == "taylor" and lib.plh_taylor_ce_saves_sums(tag, n, c, m):
+        # rows: the module's forward leaves each row's sum of f and its backward works from it, elementwise
+        E, Pn = n * c * m, n * m
+        sums = torch.empty((Pn,), dtype=torch.float32, device=x.device)
+        one_loss = torch.empty((), dtype=torch.float32, device=x.device)
+        n_valid = torch.empty((), dtype=torch.int64, device=x.device)
+        rws_bytes = int(lib.plh_reduce_workspace_bytes(Pn))
+        rws = torch.empty(rws_bytes, dtype=torch.uint8, device=x.device)
+        up = torch.ones((), dtype=torch.float32, device=x.device)
+        fs = lambda: lib.plh_taylor_ce_forward_reduced_sums(P(x), tag, P(labels), P(sums), P(one_loss), P(n_valid), 1, P(rws),
+                                                            rws_bytes, n, c, m, 4, 255, st())
+        bs = lambda: lib.plh_taylor_ce_backward_scaled_sums(P(x), tag, P(labels), P(sums), P(up), 1.0, P(n_valid), P(grad),
+                                                            n, c, m, 4, 255, st())
+        assert fs() == 0 and bs() == 0
+        eb = ELEM_BYTES[dtype]
+        legs += [("forward_keeping_sums", fs, eb * E + 8 * Pn + 4 * Pn), ("backward_from_sums", bs, 2 * eb * E + 8 * Pn + 4 * Pn)]
     if name == "lovasz":
         # the same forward with its sort passes in the decoupled look-back form (an entry point of its own)
         lb_bytes = int(lib.plh_lovasz_lookback_workspace_bytes(n, c, m))
