@@ -463,7 +463,7 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
                            int64_t order, int64_t ignore_index, void *stream);
 
 /* (N, C) rows (m_size 1) of more than 32 classes wherever the elementwise backward is the faster one (fp32 rows except
- * those of a multiple of 32 classes from 96 to 768; 16-bit rows of more than 2048 classes, and of a multiple of 8 classes
+ * those of a multiple of 32 classes from 96 to 768; 16-bit rows of more than 1024 classes, and of a multiple of 8 classes
  * up to 96): the reduced forward leaves each row's S = sum_j f(x_j)
  * (sums_out: n_size floats) and the backward forms the gradient from it elementwise over the flattened tensor instead of
  * summing every row again (no counterpart in the reference, where autograd keeps the log-softmax output between

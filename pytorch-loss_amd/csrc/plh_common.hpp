@@ -1531,8 +1531,9 @@ constexpr int kWaveRowShort = 256;
 // elementwise backward runs at 75-79 % of the HBM peak on fp32 rows of any length (1 GiB of logits; 80-90 % on 256 MiB),
 // the recomputing one at 55-72 % (70-88 %), best on rows of a multiple of 32 classes from 96 to 768, which stay with it.
 // 16-bit rows: the elementwise backward pays up to 96 classes (bf16 (1048576,64) 0.085 -> 0.043 ms) and beyond
-// `long_16bit` classes (LSR 1024: bf16 (244032,1100) 0.264 -> 0.196 ms; Taylor 2048), and only on rows of whole 16-byte
-// chunks among the short ones; between, the recomputing kernels are as fast or faster (bf16 (1048576,256) 0.187 / 0.191).
+// `long_16bit` classes (1024 for both: LSR bf16 (244032,1100) 0.264 -> 0.196 ms, Taylor (209715,1280) 0.205 -> 0.173), and
+// only on rows of whole 16-byte chunks among the short ones; between, the recomputing kernels are as fast or faster
+// (bf16 (1048576,256) 0.187 / 0.191).
 inline bool row_backward_is_elementwise(size_t elem_bytes, int64_t dimsize, int64_t long_16bit) {
     if (dimsize <= 32) return false;            // the register-resident kernels' rows
     if (elem_bytes == 4) return !(dimsize % 32 == 0 && dimsize >= 96 && dimsize <= 768);

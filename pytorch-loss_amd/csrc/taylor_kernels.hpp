@@ -31,7 +31,7 @@ struct TaylorParams {
 // Rows (m_size 1) whose backward is one elementwise pass over the flattened tensor with S kept (beyond what a wavefront's
 // registers hold the other backward reads its row twice, S and then the gradient): row_backward_is_elementwise.
 inline bool taylor_sums_apply(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    return m_size == 1 && row_backward_is_elementwise(elem_bytes, dimsize, kWaveRowCap);
+    return m_size == 1 && row_backward_is_elementwise(elem_bytes, dimsize, 1024);
 }
 
 // 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and

@@ -98,7 +98,7 @@ def test_arguments_are_rejected_before_any_launch(native):
     assert lib.plh_lsr_saves_lse(0, 8192, 512, 1) == 0 and lib.plh_lsr_saves_lse(0, 8192, 1000, 1) == 1 and lib.plh_lsr_saves_lse(0, 8192, 32, 1) == 0
     assert lib.plh_lsr_saves_lse(2, 8192, 1000, 1) == 0 and lib.plh_lsr_saves_lse(2, 8192, 1100, 1) == 1 and lib.plh_lsr_saves_lse(1, 8192, 64, 1) == 1
     assert lib.plh_taylor_ce_saves_sums(0, 8192, 1000, 1) == 1 and lib.plh_taylor_ce_saves_sums(0, 8192, 256, 1) == 0
-    assert lib.plh_taylor_ce_saves_sums(2, 8192, 1100, 1) == 0 and lib.plh_taylor_ce_saves_sums(2, 8192, 2049, 1) == 1 and lib.plh_taylor_ce_saves_sums(2, 8192, 48, 1) == 1
+    assert lib.plh_taylor_ce_saves_sums(2, 8192, 1100, 1) == 1 and lib.plh_taylor_ce_saves_sums(2, 8192, 1000, 1) == 0 and lib.plh_taylor_ce_saves_sums(2, 8192, 2049, 1) == 1 and lib.plh_taylor_ce_saves_sums(2, 8192, 48, 1) == 1
     assert lib.plh_lmargin_saves_stats(1, 8192, 32000, 1) == 1 and lib.plh_lmargin_saves_stats(0, 8192, 1024, 1) == 0 and lib.plh_lmargin_saves_stats(0, 8192, 1000, 1) == 1 and lib.plh_lmargin_saves_stats(2, 8192, 1024, 1) == 1 and lib.plh_lmargin_saves_stats(2, 8192, 1100, 1) == 1 and lib.plh_lmargin_saves_stats(2, 8192, 4096, 1) == 1
     assert lib.plh_lmargin_saves_stats(0, 8, 5000, 64) == 0 and lib.plh_lmargin_saves_stats(9, 8192, 32000, 1) == 0
     assert lib.plh_lsr_saves_lse(0, 16, 19, 63 * 65) == 0 and lib.plh_lsr_saves_lse(7, 16, 19, 769 * 769) == 0

@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 # rows whose lengths leave the 16-byte chunks of the flattened tensor straddling rows (2049, 3001, 4099), rows that do not
 # (4096), a single row, and a tensor that ends in a partial chunk (3 x 2051 elements)
 SHAPES = [(7, 2049), (5, 3001), (33, 4096), (3, 4099), (1, 5000), (3, 2051), (130, 2304),
-          (300, 40), (130, 48), (40, 64), (90, 88)]           # the last ones: rows that a wavefront holds in registers
-SHAPES_FP32_ONLY = [(70, 200), (260, 300), (17, 1000), (1, 77), (9, 1024), (300, 33), (6, 2040), (9, 1100)]
+          (300, 40), (130, 48), (40, 64), (90, 88), (6, 2040), (9, 1100), (5, 2048)]           # the last ones: rows that a wavefront holds in registers
+SHAPES_FP32_ONLY = [(70, 200), (260, 300), (17, 1000), (1, 77), (9, 1024), (300, 33)]
 DTYPES = [(torch.float32, 2e-6), (torch.float16, 2e-3), (torch.bfloat16, 1.6e-2)]
 
 
@@ -40,7 +40,8 @@ def test_the_predicate_names_long_rows_only(mod):
     lib = _native.load()
     for tag in (0, 1, 2):
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 2049, 1) == 1
-        assert lib.plh_taylor_ce_saves_sums(tag, 8, 2048, 1) == (1 if tag == 0 else 0)
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 2048, 1) == 1 and lib.plh_taylor_ce_saves_sums(tag, 8, 1100, 1) == 1
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 1000, 1) == (1 if tag == 0 else 0)
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 512, 1) == 0 and lib.plh_taylor_ce_saves_sums(tag, 8, 32, 1) == 0
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 64, 1) == 1
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 4000, 2) == 0
