@@ -88,6 +88,13 @@ __device__ __forceinline__ void taylor_pair(float x, int order, float &f, float 
     df = prev;
 }
 
+// ORD = 2 or 4: that order inlined; 0: the order at run time.
+template <int ORD>
+__device__ __forceinline__ void taylor_pair_as(float x, int order, float &f, float &df) {
+    if constexpr (ORD == 0) taylor_pair(x, order, f, df);
+    else taylor_pair24<ORD>(x, f, df);
+}
+
 // ---------------------------------------------------------------- regs ----
 
 template <class T, int CP, int V, int Form>
@@ -871,7 +878,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_sm_row(const T *__restrict__
     }
 }
 
-template <class T, int Kind>
+template <class T, int Kind, int ORD = 0>
 __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                            const Upstream up, T *__restrict__ out,
                                                            float *__restrict__ loss, Partials part,
@@ -888,7 +895,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
         float s = 0.f;
         row_visit<T>(xs, p.C, (vec & 1) != 0, [&](float v, int) {
             float f, df;
-            taylor_pair(v, p.order, f, df);
+            taylor_pair_as<ORD>(v, p.order, f, df);
             s += f;
         });
         s = row_block_reduce(s, red, OpSum());
@@ -912,7 +919,7 @@ __global__ __launch_bounds__(kRowBlock) void taylor_ce_row(const T *__restrict__
             const float cold = inv * gk, hot = cold - gk / f_y;          // see taylor_group
             row_map<T>(xs, out + row * p.C, p.C, (vec & 1) != 0, [&](float v, int j) {
                 float f, df;
-                taylor_pair(v, p.order, f, df);
+                taylor_pair_as<ORD>(v, p.order, f, df);
                 return has_y ? df * ((j == tgt) ? hot : cold) : 0.f;
             });
         }
@@ -1173,10 +1180,18 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
             // fp32 (65536,3000) 0.173 -> 0.152 ms with 64 threads, (65536,2049) 0.146 -> 0.110, bf16 (65536,3001) 0.164 ->
             // 0.104; rows of 16 KiB lose with them (fp32 (32768,4096) 0.096 -> 0.105)
             const int threads = (Kind == kTaylorCeFwd && (int64_t)p.C * (int64_t)sizeof(T) <= 12 * 1024) ? 64 : row_threads_for_sweep<T>(p.C);
-            hipLaunchKernelGGL((taylor_ce_row<T, Kind>), dim3(grid), dim3(threads), 0, st, x, lab, up, out,
-                               loss_slot, part, p,
-                               (row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C) ? 1 : 0) |
-                                   (keep ? 2 : 0));
+            const int row_flags = (row_chunks_ok<T>(x, (Kind == kTaylorCeBwd) ? (const T *)out : (const T *)nullptr, p.C) ? 1 : 0) |
+                                  (keep ? 2 : 0);
+            // (16-bit forwards: the order a compile-time constant of the sweep, as in the elementwise backward)
+            if (Kind == kTaylorCeFwd && sizeof(T) == 2 && p.order == 2)
+                hipLaunchKernelGGL((taylor_ce_row<T, Kind, (Kind == kTaylorCeFwd && sizeof(T) == 2) ? 2 : 0>), dim3(grid),
+                                   dim3(threads), 0, st, x, lab, up, out, loss_slot, part, p, row_flags);
+            else if (Kind == kTaylorCeFwd && sizeof(T) == 2 && p.order == 4)
+                hipLaunchKernelGGL((taylor_ce_row<T, Kind, (Kind == kTaylorCeFwd && sizeof(T) == 2) ? 4 : 0>), dim3(grid),
+                                   dim3(threads), 0, st, x, lab, up, out, loss_slot, part, p, row_flags);
+            else
+                hipLaunchKernelGGL((taylor_ce_row<T, Kind>), dim3(grid), dim3(threads), 0, st, x, lab, up, out, loss_slot,
+                                   part, p, row_flags);
         } else {
             const int vec = row_chunks_ok<T>(x, out, p.C) && !(Kind == kTaylorBwd && misaligned(g, 16));
             hipLaunchKernelGGL((taylor_sm_row<T, Kind>), dim3(grid), dim3(row_threads_for_sweep<T>(p.C)), 0, st, x, g, out, p, vec);
