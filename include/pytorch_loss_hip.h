@@ -464,14 +464,16 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
 
 /* (N, C) rows (m_size 1) of more than 32 classes wherever the elementwise backward is the faster one (fp32 rows except
  * those of a multiple of 32 classes from 96 to 768; 16-bit rows of more than 1024 classes, and of a multiple of 8 classes
- * up to 96): the reduced forward leaves each row's S = sum_j f(x_j)
+ * up to 96), and fp32 channel planes (NCHW) of 4096 pixels or more that do not start on 128-byte lines, with up to 24
+ * channels (513 x 513, 769 x 769 crops; orders 2 and 4, other orders leave sums_out unwritten and recompute): the reduced
+ * forward leaves each row's (pixel's) S = sum_j f(x_j)
  * (sums_out: n_size floats) and the backward forms the gradient from it elementwise over the flattened tensor instead of
  * summing every row again (no counterpart in the reference, where autograd keeps the log-softmax output between
  * TaylorSoftmaxFunc and F.nll_loss: pytorch_loss/taylor_softmax.py:175-198). plh_taylor_ce_saves_sums says (1 / 0)
  * whether the sizes qualify; the other two are plh_taylor_ce_forward with loss_out (no per-row losses) and
  * plh_taylor_ce_backward with one scalar upstream gradient, each with that one more argument, and return
- * PLH_ERR_BAD_SIZE for sizes that do not qualify. When logits or grad_logits do not sit on 16-byte boundaries the
- * recomputing kernel runs and `sums` is not read. */
+ * PLH_ERR_BAD_SIZE for sizes that do not qualify. When logits or grad_logits do not sit on 16-byte boundaries (rows), or
+ * not at the same offset into a 128-byte line (planes), the recomputing kernel runs and `sums` is not read. */
 int plh_taylor_ce_saves_sums(int32_t dtype, int64_t n_size, int64_t dimsize, int64_t m_size);
 int plh_taylor_ce_forward_reduced_sums(const void *logits, int32_t dtype, const int64_t *labels,
                                        float *sums_out, float *loss_out, int64_t *n_valid_out, int32_t mean,

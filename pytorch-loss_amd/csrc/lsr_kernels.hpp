@@ -216,13 +216,7 @@ __global__ __launch_bounds__(kRegsBlock) void lsr_bwd_regs(const T *__restrict__
 // the same offset into a 128-byte line.
 // Per element type: a lane moves 16 bytes (4 fp32 or 8 16-bit elements), a line holds kLine elements, a block's tile
 // is 256 lanes' worth of pixels and the stage holds one line's worth of pixels before it.
-template <class T> struct PlaneGeom {
-    static constexpr int kPer = 16 / (int)sizeof(T), kLine = 128 / (int)sizeof(T), kTile = 256 * kPer, kHalo = kLine;
-};
-struct PlanePixel {
-    float lse;
-    int lab;            // the label, -1 for a pixel that takes no part, C for one without a target channel
-};
+// (PlaneGeom and PlanePixel: plh_common.hpp, shared with the Taylor cross entropy's backward of the same form.)
 
 __device__ __forceinline__ float plane_grad(float x, PlanePixel px, int c, float scale, float n_pos, float n_neg) {
     const float e = __builtin_amdgcn_exp2f((x - px.lse) * kLog2e);

@@ -1526,6 +1526,17 @@ struct WaveRowSpan {
 constexpr int kWaveRowCap = 2048;       // 32 steps of 64 lanes, one element each
 constexpr int kWaveRowShort = 256;
 
+// Geometry of the backwards that walk every channel plane in its own cache lines (lsr_bwd_planes, taylor_ce_bwd_planes):
+// a lane moves 16 bytes (4 fp32 or 8 16-bit elements), a line holds kLine elements, a block's tile is 256 lanes' worth
+// of pixels and the stage holds one line's worth of pixels before it. PlanePixel: what is staged per pixel.
+template <class T> struct PlaneGeom {
+    static constexpr int kPer = 16 / (int)sizeof(T), kLine = 128 / (int)sizeof(T), kTile = 256 * kPer, kHalo = kLine;
+};
+struct PlanePixel {
+    float lse;          // LSR: the pixel's log-sum-exp; Taylor cross entropy: the upstream gradient over the pixel's S
+    int lab;            // the label, -1 for a pixel that takes no part, C for one without a target channel
+};
+
 // Which (N, C) rows of LSR and Taylor cross entropy take the backward that is elementwise over the flattened tensor, from
 // one value per row that the forward leaves, instead of the one that holds the row in registers and recomputes. The
 // elementwise backward runs at 75-79 % of the HBM peak on fp32 rows of any length (1 GiB of logits; 80-90 % on 256 MiB),

@@ -169,7 +169,9 @@ extern "C" int plh_taylor_ce_forward_reduced_sums(const void *logits, int32_t dt
     unsigned blocks = 0;
     if (n_size * dimsize * m_size != 0) {
         TaylorParams p = make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es);
-        p.sums = sums_out;
+        // (channel planes: the kernels that leave and use S per pixel are compiled for orders 2 and 4; other orders
+        // leave sums_out unwritten and the backward recomputes)
+        p.sums = (m_size > 1 && order > 4) ? nullptr : sums_out;
         blocks = run(kTaylorCeFwd, dtype, logits, nullptr, labels, kUnit, nullptr, nullptr, part, p, st);
     }
     finish_partials(part, blocks, loss_out, n_valid_out, mean ? kFinishMeanOverCount : kFinishSum, 0, st);
@@ -193,7 +195,7 @@ extern "C" int plh_taylor_ce_backward_scaled_sums(const void *logits, int32_t dt
     if (n_size * dimsize * m_size == 0) return PLH_OK;
     const Upstream up{grad_scalar, 0, divide_by, scale};
     TaylorParams p = make_taylor(n_size, dimsize, m_size, order, 1, ignore_index, es);
-    p.sums = const_cast<float *>(sums);
+    p.sums = (m_size > 1 && order > 4) ? nullptr : const_cast<float *>(sums);
     run(kTaylorCeBwd, dtype, logits, nullptr, labels, up, grad_logits, nullptr, kNone, p, (hipStream_t)stream);
     return check_launch();
 }

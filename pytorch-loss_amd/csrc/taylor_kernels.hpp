@@ -30,8 +30,12 @@ struct TaylorParams {
 
 // Rows (m_size 1) whose backward is one elementwise pass over the flattened tensor with S kept (beyond what a wavefront's
 // registers hold the other backward reads its row twice, S and then the gradient): row_backward_is_elementwise.
+// Channel planes (NCHW) that do not start on 128-byte lines, fp32, up to 24 channels and 4096 pixels or more (odd crops:
+// the forward is the per-image form of the register-resident kernel and leaves S per pixel, the backward walks every
+// plane in its own lines, taylor_ce_bwd_planes): orders 2 and 4, which those kernels are compiled for.
 inline bool taylor_sums_apply(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
-    return m_size == 1 && row_backward_is_elementwise(elem_bytes, dimsize, 1024);
+    if (m_size == 1) return row_backward_is_elementwise(elem_bytes, dimsize, 1024);
+    return elem_bytes == 4 && dimsize >= 1 && (m_size * 4) % 128 != 0 && image_form_pays<float>((int)dimsize, m_size);
 }
 
 // 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
     at.labels(lab, p.ignore, lb);
     typename Pack<T, V>::Raw raw[CP];
     at.load_slice(x, p.C, p.m_size, raw);
-    float out[V];
+    float out[V], sums[V];
     float mine = 0.f;
     int cnt = 0;
 #pragma unroll
@@ -239,10 +243,14 @@ __global__ __launch_bounds__(kRegsBlock) void taylor_ce_fwd_regs(const T *__rest
             }
         const bool valid = at.live && !ign && tgt >= 0;
         out[k] = valid ? logf(s) - logf(f_y) : 0.f;
+        sums[k] = s;
         mine += out[k];
         cnt += (at.live && !ign) ? 1 : 0;
     }
-    if (at.live && loss) at.store_f32(loss, out);
+    if (at.live && loss) {
+        if (loss == p.sums) at.store_f32(loss, sums);      // the slot takes the pixels' S (TaylorParams::sums)
+        else at.store_f32(loss, out);
+    }
     if (Reduce) {
         const float bs = block_sum_256(mine, red);
         const float bc = block_sum_256((float)cnt, red);
@@ -1023,6 +1031,88 @@ __global__ __launch_bounds__(256) void taylor_ce_bwd_flat_sums(const T *__restri
     }
 }
 
+// Cross-entropy backward from the forward's per-pixel S, for channel planes that start on element boundaries only (odd
+// crops): the walk of lsr_bwd_planes - a block takes 1024 pixels of an image and in plane c its 256 threads move the
+// 32 whole lines that begin at the tile's first pixel shifted back by the plane's offset into its line, so loads and
+// stores are aligned 16-byte accesses in every plane; the pixels' (gout / S, label) pairs, the tile's and one line's
+// worth before it, are staged in LDS once, transposed by pixel index mod 4. With k = gout / S the gradient is
+// f'(x) k, and f'(x) (k - gout / f(x)) in the target's plane. One scalar upstream gradient, fp32, orders 2 and 4.
+template <class T, int ORD>
+__global__ __launch_bounds__(256) void taylor_ce_bwd_planes(const T *__restrict__ x, const int64_t *__restrict__ lab,
+                                                            const Upstream up, T *__restrict__ grad, const TaylorParams p,
+                                                            int tiles) {
+    static_assert(sizeof(T) == 4, "fp32 logits (see taylor_sums_apply)");
+    using G = PlaneGeom<T>;
+    constexpr int kPer = G::kPer, kTile = G::kTile, kHalo = G::kHalo;
+    __shared__ PlanePixel pairs[kPer][(kTile + kHalo) / kPer];          // entry i at [i % kPer][i / kPer]
+    const int64_t M = p.m_size;
+    const int64_t n = blockIdx.x / tiles;
+    const int t = (int)(blockIdx.x - n * tiles);
+    const int l = threadIdx.x;
+    float gk = up.gout ? *up.gout * up.scale : up.scale;
+    if (up.divide_by) gk = gk / (float)(*up.divide_by);
+    const int64_t p_first = (int64_t)t * kTile - kHalo;                 // image-local pixel of staged entry 0
+    for (int i = l; i < kTile + kHalo; i += 256) {
+        const int64_t q = p_first + i;
+        PlanePixel px{0.f, -1};
+        if (q >= 0 && q < M) {
+            const int64_t at = n * M + q;
+            const int64_t lb = lab[at];
+            const bool has_y = lb != p.ignore && lb >= 0 && lb < p.C;
+            px.lse = gk / p.sums[at];
+            px.lab = has_y ? (int)lb : -1;              // pixels without a target: exact zeros (taylor_ce_bwd_regs)
+        }
+        pairs[i % kPer][i / kPer] = px;
+    }
+    __syncthreads();
+    auto one = [&](float xv, PlanePixel px, int c) {
+        float f, df;
+        taylor_pair24<ORD>(xv, f, df);
+        const float k = (px.lab == c) ? px.lse - gk / f : px.lse;
+        return px.lab < 0 ? 0.f : df * k;
+    };
+    constexpr int U = 4;                            // planes in flight per thread
+    for (int c0 = 0; c0 < p.C; c0 += U) {
+        plh_u4 xv[U];
+        int64_t q[U], plane[U];
+        bool full[U];
+        int first[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u < p.C ? c0 + u : p.C - 1;
+            plane[u] = (n * p.C + c) * M;
+            // the plane's offset into its line, in elements
+            const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) / sizeof(T)) & (unsigned)(G::kLine - 1));
+            first[u] = kHalo + kPer * l - shift;                     // staged index of this lane's first pixel
+            q[u] = (int64_t)t * kTile - shift + kPer * l;
+            full[u] = q[u] >= 0 && q[u] + (kPer - 1) < M;
+            xv[u] = __builtin_nontemporal_load(reinterpret_cast<const plh_u4 *>(x + plane[u] + (full[u] ? q[u] : 0)));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u;
+            if (c >= p.C) break;
+            const int i0 = first[u];
+            if (full[u]) {
+                const unsigned in[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
+                unsigned out[4];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const int i = i0 + d;
+                    out[d] = f32_bits(one(bits_f32(in[d]), pairs[i % kPer][i / kPer], c));
+                }
+                __builtin_nontemporal_store(plh_u4{out[0], out[1], out[2], out[3]},
+                                            reinterpret_cast<plh_u4 *>(grad + plane[u] + q[u]));
+            } else {                    // the two ends of a plane, element by element
+                for (int k = 0; k < kPer; ++k)
+                    if (q[u] + k >= 0 && q[u] + k < M)
+                        store_one(grad + plane[u] + q[u] + k,
+                                  one(load_one(x + plane[u] + q[u] + k), pairs[(i0 + k) % kPer][(i0 + k) / kPer], c));
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------ dispatch ----
 
 template <class T, int Kind>
@@ -1036,11 +1126,26 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
                                    lab, (Kind == kTaylorCeFwd) ? (const void *)loss : nullptr, go_vec, true, kIsCe, true,
                                    kImageFormMaxChannels<T, (Kind == kTaylorBwd) ? 2 : 1>);
     const bool g_ok = (Kind != kTaylorBwd) || !misaligned(g, VT * sizeof(T));
+    if constexpr (Kind == kTaylorCeBwd && sizeof(T) == 4) {
+        // odd crops, from the forward's per-pixel S, plane by plane: one scalar upstream gradient, logits and gradient at
+        // the same offset into a 128-byte line (whole lines of the one are whole lines of the other)
+        const int64_t tiles = ceil_div(p.m_size + PlaneGeom<T>::kHalo - 1, (int64_t)PlaneGeom<T>::kTile);
+        if (p.sums && !go_vec && p.m_size > 1 && !walk && taylor_sums_apply(sizeof(T), p.C, p.m_size) &&
+            ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(out)) & 127) == 0 && !misaligned(x, sizeof(T)) &&
+            p.P / p.m_size * tiles < ((int64_t)1 << 31)) {
+            const unsigned grid = (unsigned)(p.P / p.m_size * tiles);
+            if (p.order == 2)
+                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 2>), dim3(grid), dim3(256), 0, st, x, lab, up, out, p, (int)tiles);
+            else
+                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 4>), dim3(grid), dim3(256), 0, st, x, lab, up, out, p, (int)tiles);
+            return grid;
+        }
+    }
     if constexpr (Kind == kTaylorCeBwd) {
         // long rows, from the sums the forward left: elementwise over the flattened tensor
         constexpr int L = RowChunk<T>::kLen;
         const int64_t chunks = p.P * p.C / L, flat_blocks = ceil_div(chunks, (int64_t)(256 * kFlatChunks));
-        if (p.sums && !go_vec && taylor_sums_apply(sizeof(T), p.C, p.m_size) && !misaligned(x, 16) && !misaligned(out, 16) &&
+        if (p.sums && !go_vec && p.m_size == 1 && taylor_sums_apply(sizeof(T), p.C, p.m_size) && !misaligned(x, 16) && !misaligned(out, 16) &&
             flat_blocks >= 1 && flat_blocks < ((int64_t)1 << 31)) {
             // (the order as a compile-time constant pays on 16-bit logits, bf16 (4194304,64) 0.238 -> 0.215 ms, and costs fp32
             // ones 3 %, (4194304,64) 0.357 -> 0.372: those keep the test per evaluation)
@@ -1115,6 +1220,9 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         constexpr int kSlices = (Kind == kTaylorBwd) ? 2 : 1;
         const bool image = !vec && image_form_pays<T, kSlices>(p.C, p.m_size);
         const unsigned grid = vec ? regs_grid<VT>(p.P) : (image ? image_grid<4>(p.P / p.m_size, p.m_size) : regs_grid<1>(p.P));
+        // (the per-image forward that leaves the pixels' S has no per-pixel losses to write, so their slot serves)
+        float *const loss_px = (Kind == kTaylorCeFwd && image && p.sums != nullptr && loss == nullptr && p.m_size > 1 &&
+                                taylor_sums_apply(sizeof(T), p.C, p.m_size)) ? p.sums : loss;
 #define PLH_GO(CPV, VV, UU)                                                                                          \
     do {                                                                                                             \
         if constexpr (Kind == kTaylorFwd)                                                                            \
@@ -1123,7 +1231,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
             hipLaunchKernelGGL((taylor_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, g, x, out, p); \
         else if constexpr (Kind == kTaylorCeFwd)                                                                     \
             hipLaunchKernelGGL((taylor_ce_fwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, \
-                               lab, loss, part, p);                                                                  \
+                               lab, loss_px, part, p);                                                               \
         else                                                                                                         \
             hipLaunchKernelGGL((taylor_ce_bwd_regs<T, CPV, VV, UU>), dim3(grid), dim3(kRegsBlock), 0, st, x, lab,    \
                                up, out, p);                                                                          \

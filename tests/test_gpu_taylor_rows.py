@@ -44,7 +44,7 @@ def test_the_predicate_names_long_rows_only(mod):
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 1000, 1) == (1 if tag == 0 else 0)
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 512, 1) == 0 and lib.plh_taylor_ce_saves_sums(tag, 8, 32, 1) == 0
         assert lib.plh_taylor_ce_saves_sums(tag, 8, 64, 1) == 1
-        assert lib.plh_taylor_ce_saves_sums(tag, 8, 4000, 2) == 0
+        assert lib.plh_taylor_ce_saves_sums(tag, 8, 4000, 2) == 0 and lib.plh_taylor_ce_saves_sums(tag, 8, 19, 1024 * 1024) == 0
     assert lib.plh_taylor_ce_saves_sums(7, 8, 4000, 1) == 0
 
 
@@ -118,3 +118,64 @@ def test_rows_without_any_valid_label(mod):
     loss = mod.TaylorCrossEntropyLossV3(n=2, ignore_index=255, reduction="sum")(a, yt)
     loss.backward()
     assert float(loss.detach()) == 0.0 and a.grad.abs().max().item() == 0.0
+
+
+# Channel planes of odd length (crops), fp32, up to 24 channels: the per-image forward leaves S per pixel and the
+# backward walks every plane in its own cache lines (taylor_ce_bwd_planes). The last shape has planes that end inside a
+# tile's first line; (1, 24, 67, 67) the most channels the form takes.
+CROPS = [(2, 19, 65, 67), (1, 24, 67, 67), (3, 5, 63, 66), (1, 1, 4097, 1), (2, 7, 1, 5001)]
+
+
+@pytest.mark.parametrize("order", [2, 4, 6])
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("shape", CROPS, ids=str)
+def test_odd_crops_backward_from_the_pixels_sums(mod, shape, reduction, order):
+    from pytorch_loss import _native
+    lib = _native.load()
+    n, c, m = shape[0], shape[1], shape[2] * shape[3]
+    assert lib.plh_taylor_ce_saves_sums(0, n, c, m) == 1 and lib.plh_taylor_ce_saves_sums(2, n, c, m) == 0
+    assert lib.plh_taylor_ce_saves_sums(0, n, c, (m + 31) // 32 * 32) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 25, m) == 0
+    x = synth.normal(411, 1, shape, 0.0, 0.75).astype(np.float32)
+    y = synth.seg_labels(411, shape[:1] + shape[2:], c, 255, 0.15)
+    y[0, 0, :3] = c + 3                                  # labels out of range: no target, zero loss and gradient
+    xt, yt = torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()
+    n_valid = int((y != 255).sum())
+    x64 = x.astype(np.float64)
+    factor = 0.5
+    a = xt.clone().requires_grad_(True)
+    loss = mod.TaylorCrossEntropyLossV3(n=order, ignore_index=255, reduction=reduction)(a, yt)
+    (loss * factor).backward()
+    b = xt.clone().requires_grad_(True)
+    per = mod.TaylorCrossEntropyLossV3(n=order, ignore_index=255, reduction="none")(b, yt)
+    want = per.sum() / (n_valid if reduction == "mean" else 1)
+    (want * factor).backward()                          # the per-pixel path: the recomputing backward kernel
+    assert abs(float(loss.detach()) - float(want.detach())) <= 1e-5 * abs(float(want.detach()))
+    scale = b.grad.abs().max().item()
+    up = factor / (n_valid if reduction == "mean" else 1)
+    assert (a.grad - b.grad).abs().max().item() <= 2e-6 * scale + 1e-6 * up   # (one channel: the exact gradient is 0)
+    ign = torch.from_numpy(y == 255).cuda().unsqueeze(1).expand_as(a.grad)
+    assert a.grad[ign].abs().max().item() == 0
+    # and against the oracle where every label is a class or ignored
+    y2 = np.where(y >= c, 255, y)
+    y2t = torch.from_numpy(y2).cuda()
+    a2 = xt.clone().requires_grad_(True)
+    loss2 = mod.TaylorCrossEntropyLossV3(n=order, ignore_index=255, reduction="sum")(a2, y2t)
+    loss2.backward()
+    want_g = oracle.taylor_ce_backward(x64, y2, order, 255, 1.0)
+    assert abs(float(loss2.detach()) - oracle.taylor_ce(x64, y2, order, 255).sum()) <= 1e-5 * abs(float(loss2.detach()))
+    assert np.abs(a2.grad.cpu().numpy() - want_g).max() <= 2e-6 * np.abs(want_g).max() + 1e-6
+
+
+def test_odd_crops_on_views_at_another_offset_into_their_lines(mod):
+    """Logits one element into their storage: logits and gradient sit at different offsets into a 128-byte line, and the
+    recomputing backward runs (the forward's sums are not read)."""
+    shape = (2, 19, 65, 67)
+    x = synth.normal(412, 1, shape, 0.0, 0.75).astype(np.float32)
+    y = synth.seg_labels(412, shape[:1] + shape[2:], shape[1], 255, 0.1)
+    store = torch.empty(x.size + 1, device="cuda")
+    xt = store[1:].view(shape)
+    xt.copy_(torch.from_numpy(x))
+    a = xt.requires_grad_(True)
+    mod.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="sum")(a, torch.from_numpy(y).cuda()).backward()
+    want = oracle.taylor_ce_backward(x.astype(np.float64), y, 4, 255, 1.0)
+    assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
