@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|focal_seg|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|lsr_vocab|lmargin_vocab|taylor_vocab|lmargin_rows]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lsr|lmargin|focal|lovasz|taylor|onehot|ohem|dice|layernorm|focal_seg|lsr_c150|lsr_c300|lsr_crop769|lmargin_crop513|taylor_crop769|lsr_vocab|lmargin_vocab|taylor_vocab|lmargin_rows]
                     [--no-cpu-baseline] [--no-others]
 
 A step is one fwd+bwd pass of the loss module over one batch of synthetic input that is
@@ -82,6 +82,8 @@ WORKLOADS = {
                         "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lmargin_crop513": dict(base="lmargin", shape=(32, 19, 513, 513), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (32,19,513,513), "
                             "int64 labels 5% ignore=255, lam=0.3, mean"),
+    "taylor_crop769": dict(base="taylor", shape=(16, 19, 769, 769), desc="TaylorCrossEntropyLossV3 fwd+bwd, fp32 logits (16,19,769,769), "
+                           "int64 labels 5% ignore=255, n=4, mean"),
     "lsr_vocab": dict(base="lsr", shape=(8192, 32000), desc="LabelSmoothSoftmaxCEV3 fwd+bwd, fp32 logits (8192,32000), "
                       "int64 labels 5% ignore=255, lb_smooth=0.1, mean"),
     "lmargin_vocab": dict(base="lmargin", shape=(8192, 32000), desc="LargeMarginSoftmaxV3 fwd+bwd, fp32 logits (8192,32000), "
