@@ -30,12 +30,14 @@ struct TaylorParams {
 
 // Rows (m_size 1) whose backward is one elementwise pass over the flattened tensor with S kept (beyond what a wavefront's
 // registers hold the other backward reads its row twice, S and then the gradient): row_backward_is_elementwise.
-// Channel planes (NCHW) that do not start on 128-byte lines, fp32, up to 24 channels and 4096 pixels or more (odd crops:
-// the forward is the per-image form of the register-resident kernel and leaves S per pixel, the backward walks every
-// plane in its own lines, taylor_ce_bwd_planes): orders 2 and 4, which those kernels are compiled for.
+// Channel planes (NCHW) that do not start on 128-byte lines, fp32, 4096 pixels or more, up to 24 channels or 33 .. 256
+// (odd crops: the forward is the per-image form of the register-resident kernel, or the split kernel in tiles per image,
+// and leaves S per pixel; the backward walks every plane in its own lines, taylor_ce_bwd_planes): orders 2 and 4, which
+// those kernels are compiled for.
 inline bool taylor_sums_apply(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
     if (m_size == 1) return row_backward_is_elementwise(elem_bytes, dimsize, 1024);
-    return elem_bytes == 4 && dimsize >= 1 && (m_size * 4) % 128 != 0 && image_form_pays<float>((int)dimsize, m_size);
+    if (elem_bytes != 4 || dimsize < 1 || m_size < 4096 || (m_size * 4) % 128 == 0) return false;
+    return image_form_pays<float>((int)dimsize, m_size) || (dimsize > kMaxRegsChannels && dimsize <= kMaxSplitChannels);
 }
 
 // 1 / i! for i = 0..33; 34! does not fit fp32 (the reference's running factorial becomes inf there and
@@ -386,7 +388,7 @@ __global__ __launch_bounds__(kSplitBlock) void taylor_ce_fwd_split(const T *__re
     const bool here = at.live && wave < at.nv;
     const bool valid = here && !ign && tgt >= 0;
     const float out = valid ? logf(s) - logf(f_y) : 0.f;
-    if (here && loss) loss[at.pix + wave] = out;
+    if (here && loss) loss[at.pix + wave] = (loss == p.sums) ? s : out;       // the slot takes the pixels' S (TaylorParams::sums)
     if (Reduce) split_block_partials<V>(out, here && !ign, wave, lane, part);
     };
     if (p.order == 2) run(std::integral_constant<int, 2>());
@@ -1040,7 +1042,7 @@ __global__ __launch_bounds__(256) void taylor_ce_bwd_flat_sums(const T *__restri
 template <class T, int ORD>
 __global__ __launch_bounds__(256) void taylor_ce_bwd_planes(const T *__restrict__ x, const int64_t *__restrict__ lab,
                                                             const Upstream up, T *__restrict__ grad, const TaylorParams p,
-                                                            int tiles) {
+                                                            int tiles, int planes_per_block) {
     static_assert(sizeof(T) == 4, "fp32 logits (see taylor_sums_apply)");
     using G = PlaneGeom<T>;
     constexpr int kPer = G::kPer, kTile = G::kTile, kHalo = G::kHalo;
@@ -1072,14 +1074,17 @@ __global__ __launch_bounds__(256) void taylor_ce_bwd_planes(const T *__restrict_
         return px.lab < 0 ? 0.f : df * k;
     };
     constexpr int U = 4;                            // planes in flight per thread
-    for (int c0 = 0; c0 < p.C; c0 += U) {
+    // blockIdx.y: which planes of the tile (many channels are shared out over several blocks, so that the grid fills the chip)
+    const int c_begin = blockIdx.y * planes_per_block;
+    const int c_end = c_begin + planes_per_block < p.C ? c_begin + planes_per_block : p.C;
+    for (int c0 = c_begin; c0 < c_end; c0 += U) {
         plh_u4 xv[U];
         int64_t q[U], plane[U];
         bool full[U];
         int first[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int c = c0 + u < p.C ? c0 + u : p.C - 1;
+            const int c = c0 + u < c_end ? c0 + u : c_end - 1;
             plane[u] = (n * p.C + c) * M;
             // the plane's offset into its line, in elements
             const int shift = (int)((reinterpret_cast<uintptr_t>(x + plane[u]) / sizeof(T)) & (unsigned)(G::kLine - 1));
@@ -1091,7 +1096,7 @@ __global__ __launch_bounds__(256) void taylor_ce_bwd_planes(const T *__restrict_
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int c = c0 + u;
-            if (c >= p.C) break;
+            if (c >= c_end) break;
             const int i0 = first[u];
             if (full[u]) {
                 const unsigned in[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
@@ -1133,12 +1138,19 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         if (p.sums && !go_vec && p.m_size > 1 && !walk && taylor_sums_apply(sizeof(T), p.C, p.m_size) &&
             ((reinterpret_cast<uintptr_t>(x) ^ reinterpret_cast<uintptr_t>(out)) & 127) == 0 && !misaligned(x, sizeof(T)) &&
             p.P / p.m_size * tiles < ((int64_t)1 << 31)) {
-            const unsigned grid = (unsigned)(p.P / p.m_size * tiles);
+            // planes per block as for lsr_bwd_planes: all of them up to 32 channels; beyond, 16 on planes of 1 MiB and
+            // more, else 4 (8 when the tiles alone outnumber the blocks the chip holds at once)
+            const int64_t tiles_all = p.P / p.m_size * tiles;
+            const int per = p.C <= kMaxRegsChannels                      ? p.C
+                            : p.m_size * (int64_t)sizeof(T) >= (1 << 20) ? 16
+                            : tiles_all <= 2048                          ? 4
+                                                                         : 8;
+            const dim3 grid((unsigned)tiles_all, (unsigned)ceil_div(p.C, per));
             if (p.order == 2)
-                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 2>), dim3(grid), dim3(256), 0, st, x, lab, up, out, p, (int)tiles);
+                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 2>), grid, dim3(256), 0, st, x, lab, up, out, p, (int)tiles, per);
             else
-                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 4>), dim3(grid), dim3(256), 0, st, x, lab, up, out, p, (int)tiles);
-            return grid;
+                hipLaunchKernelGGL((taylor_ce_bwd_planes<T, 4>), grid, dim3(256), 0, st, x, lab, up, out, p, (int)tiles, per);
+            return (unsigned)tiles_all;
         }
     }
     if constexpr (Kind == kTaylorCeBwd) {
@@ -1187,6 +1199,9 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
     const bool image = shape == Shape::SplitImage || (shape == Shape::Split && !g_ok && p.m_size >= 4096);
     if (image || (shape == Shape::Split && g_ok)) {
         const unsigned grid = image ? split_image_grid<VT>(p.P / p.m_size, p.m_size) : split_grid<VT>(p.P);
+        // (the tiles-per-image forward that leaves the pixels' S has no per-pixel losses to write, so their slot serves)
+        float *const loss_sp = (Kind == kTaylorCeFwd && shape == Shape::SplitImage && p.sums != nullptr && loss == nullptr &&
+                                taylor_sums_apply(sizeof(T), p.C, p.m_size)) ? p.sums : loss;
 #define PLH_GO(KW, IMG)                                                                                               \
     do {                                                                                                              \
         if constexpr (Kind == kTaylorFwd)                                                                             \
@@ -1195,7 +1210,7 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
             hipLaunchKernelGGL((taylor_sm_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, g, x, out, p); \
         else if constexpr (Kind == kTaylorCeFwd)                                                                      \
             hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, \
-                               lab, loss, part, p);                                                                   \
+                               lab, loss_sp, part, p);                                                                \
         else                                                                                                          \
             hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VT, IMG>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, \
                                out, p);                                                                               \

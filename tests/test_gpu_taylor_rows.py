@@ -123,7 +123,8 @@ def test_rows_without_any_valid_label(mod):
 # Channel planes of odd length (crops), fp32, up to 24 channels: the per-image forward leaves S per pixel and the
 # backward walks every plane in its own cache lines (taylor_ce_bwd_planes). The last shape has planes that end inside a
 # tile's first line; (1, 24, 67, 67) the most channels the form takes.
-CROPS = [(2, 19, 65, 67), (1, 24, 67, 67), (3, 5, 63, 66), (1, 1, 4097, 1), (2, 7, 1, 5001)]
+CROPS = [(2, 19, 65, 67), (1, 24, 67, 67), (3, 5, 63, 66), (1, 1, 4097, 1), (2, 7, 1, 5001),
+         (1, 33, 65, 67), (2, 150, 65, 65), (1, 256, 63, 67), (1, 40, 1, 9001)]      # 33 .. 256 channels: the forward in tiles per image
 
 
 @pytest.mark.parametrize("order", [2, 4, 6])
@@ -135,6 +136,7 @@ def test_odd_crops_backward_from_the_pixels_sums(mod, shape, reduction, order):
     n, c, m = shape[0], shape[1], shape[2] * shape[3]
     assert lib.plh_taylor_ce_saves_sums(0, n, c, m) == 1 and lib.plh_taylor_ce_saves_sums(2, n, c, m) == 0
     assert lib.plh_taylor_ce_saves_sums(0, n, c, (m + 31) // 32 * 32) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 25, m) == 0
+    assert lib.plh_taylor_ce_saves_sums(0, n, 32, m) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 33, m) == 1 and lib.plh_taylor_ce_saves_sums(0, n, 257, m) == 0
     x = synth.normal(411, 1, shape, 0.0, 0.75).astype(np.float32)
     y = synth.seg_labels(411, shape[:1] + shape[2:], c, 255, 0.15)
     y[0, 0, :3] = c + 3                                  # labels out of range: no target, zero loss and gradient
