@@ -465,7 +465,8 @@ int plh_taylor_ce_backward(const void *logits, int32_t dtype, const int64_t *lab
 /* (N, C) rows (m_size 1) of more than 32 classes wherever the elementwise backward is the faster one (fp32 rows except
  * those of a multiple of 32 classes from 96 to 768; 16-bit rows of more than 1024 classes, and of a multiple of 8 classes
  * up to 96), and fp32 channel planes (NCHW) of 4096 pixels or more that do not start on 128-byte lines, with up to 24
- * channels or 33..256 (513 x 513, 769 x 769 crops; orders 2 and 4, other orders leave sums_out unwritten and recompute): the reduced
+ * channels or 33..256 (513 x 513, 769 x 769 crops), and 257..512 channels on any plane of that size (orders 2 and 4, other
+ * orders leave sums_out unwritten and recompute): the reduced
  * forward leaves each row's (pixel's) S = sum_j f(x_j)
  * (sums_out: n_size floats) and the backward forms the gradient from it elementwise over the flattened tensor instead of
  * summing every row again (no counterpart in the reference, where autograd keeps the log-softmax output between

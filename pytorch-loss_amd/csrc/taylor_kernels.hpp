@@ -36,7 +36,10 @@ struct TaylorParams {
 // those kernels are compiled for.
 inline bool taylor_sums_apply(size_t elem_bytes, int64_t dimsize, int64_t m_size) {
     if (m_size == 1) return row_backward_is_elementwise(elem_bytes, dimsize, 1024);
-    if (elem_bytes != 4 || dimsize < 1 || m_size < 4096 || (m_size * 4) % 128 == 0) return false;
+    if (elem_bytes != 4 || dimsize < 1 || m_size < 4096) return false;
+    // 257 .. 512 channels on any plane: the recomputing kernels keep a pixel's slice in two halves per wavefront there
+    if (dimsize > kMaxSplitChannels && dimsize <= kMaxDeepChannels) return true;
+    if ((m_size * 4) % 128 == 0) return false;
     return image_form_pays<float>((int)dimsize, m_size) || (dimsize > kMaxRegsChannels && dimsize <= kMaxSplitChannels);
 }
 
@@ -1178,12 +1181,15 @@ unsigned taylor_launch(const T *x, const T *g, const int64_t *lab, const Upstrea
         if (shape == Shape::SplitDeep) {            // 257..512 channels: up to 64 slots per wavefront, half the pixels per lane
             constexpr int VD = VT / 2;
             const unsigned grid = split_grid<VD>(p.P);
+            // (the forward that leaves the pixels' S has no per-pixel losses to write, so their slot serves)
+            float *const loss_dp = (Kind == kTaylorCeFwd && p.sums != nullptr && loss == nullptr &&
+                                    taylor_sums_apply(sizeof(T), p.C, p.m_size)) ? p.sums : loss;
             switch (split_slots_deep(p.C)) {
 #define PLH_CASE(KW)                                                                                                  \
     case KW:                                                                                                          \
         if constexpr (Kind == kTaylorCeFwd)                                                                           \
             hipLaunchKernelGGL((taylor_ce_fwd_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, \
-                               loss, part, p);                                                                        \
+                               loss_dp, part, p);                                                                     \
         else                                                                                                          \
             hipLaunchKernelGGL((taylor_ce_bwd_split<T, KW, VD>), dim3(grid), dim3(kSplitBlock), 0, st, x, lab, up, out, \
                                p);                                                                                    \

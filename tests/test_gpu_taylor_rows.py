@@ -124,7 +124,8 @@ def test_rows_without_any_valid_label(mod):
 # backward walks every plane in its own cache lines (taylor_ce_bwd_planes). The last shape has planes that end inside a
 # tile's first line; (1, 24, 67, 67) the most channels the form takes.
 CROPS = [(2, 19, 65, 67), (1, 24, 67, 67), (3, 5, 63, 66), (1, 1, 4097, 1), (2, 7, 1, 5001),
-         (1, 33, 65, 67), (2, 150, 65, 65), (1, 256, 63, 67), (1, 40, 1, 9001)]      # 33 .. 256 channels: the forward in tiles per image
+         (1, 33, 65, 67), (2, 150, 65, 65), (1, 256, 63, 67), (1, 40, 1, 9001),      # 33 .. 256 channels: the forward in tiles per image
+         (1, 300, 65, 65), (1, 512, 63, 67)]                                       # 257 .. 512
 
 
 @pytest.mark.parametrize("order", [2, 4, 6])
@@ -135,8 +136,8 @@ def test_odd_crops_backward_from_the_pixels_sums(mod, shape, reduction, order):
     lib = _native.load()
     n, c, m = shape[0], shape[1], shape[2] * shape[3]
     assert lib.plh_taylor_ce_saves_sums(0, n, c, m) == 1 and lib.plh_taylor_ce_saves_sums(2, n, c, m) == 0
-    assert lib.plh_taylor_ce_saves_sums(0, n, c, (m + 31) // 32 * 32) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 25, m) == 0
-    assert lib.plh_taylor_ce_saves_sums(0, n, 32, m) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 33, m) == 1 and lib.plh_taylor_ce_saves_sums(0, n, 257, m) == 0
+    assert lib.plh_taylor_ce_saves_sums(0, n, c, (m + 31) // 32 * 32) == (1 if c > 256 else 0) and lib.plh_taylor_ce_saves_sums(0, n, 25, m) == 0
+    assert lib.plh_taylor_ce_saves_sums(0, n, 32, m) == 0 and lib.plh_taylor_ce_saves_sums(0, n, 33, m) == 1 and lib.plh_taylor_ce_saves_sums(0, n, 513, m) == 0
     x = synth.normal(411, 1, shape, 0.0, 0.75).astype(np.float32)
     y = synth.seg_labels(411, shape[:1] + shape[2:], c, 255, 0.15)
     y[0, 0, :3] = c + 3                                  # labels out of range: no target, zero loss and gradient
@@ -180,4 +181,20 @@ def test_odd_crops_on_views_at_another_offset_into_their_lines(mod):
     a = xt.requires_grad_(True)
     mod.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="sum")(a, torch.from_numpy(y).cuda()).backward()
     want = oracle.taylor_ce_backward(x.astype(np.float64), y, 4, 255, 1.0)
+    assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+
+
+def test_more_than_256_channels_on_aligned_planes(mod):
+    """257 .. 512 channels take the pair whatever the planes' alignment (here 64 x 64: whole lines)."""
+    from pytorch_loss import _native
+    shape = (1, 300, 64, 64)
+    assert _native.load().plh_taylor_ce_saves_sums(0, 1, 300, 4096) == 1
+    x = synth.normal(413, 1, shape, 0.0, 0.75).astype(np.float32)
+    y = synth.seg_labels(413, shape[:1] + shape[2:], shape[1], 255, 0.1)
+    a = torch.from_numpy(x).cuda().requires_grad_(True)
+    loss = mod.TaylorCrossEntropyLossV3(n=4, ignore_index=255, reduction="sum")(a, torch.from_numpy(y).cuda())
+    loss.backward()
+    x64 = x.astype(np.float64)
+    assert abs(float(loss.detach()) - oracle.taylor_ce(x64, y, 4, 255).sum()) <= 1e-5 * abs(float(loss.detach()))
+    want = oracle.taylor_ce_backward(x64, y, 4, 255, 1.0)
     assert np.abs(a.grad.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
